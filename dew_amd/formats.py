@@ -1,0 +1,195 @@
+"""The quantized expert banks the MoE layer holds, in the reference's own storage layouts, so a checkpoint
+packed for it is read here unchanged.
+
+`NvFp4` mirrors the reference's bank (src/dew/nn/kernels/formats.py:27-137): K-major uint32 `words
+[E, N, K/8]`, each the GF(2)-encoded word (src/dew/algebra/bits.py:696-705) of eight E2M1 codes taken in
+the staged depth order (word w of a 128-deep group holds depths 128g + 16j + w, j = 0..7;
+src/dew/nn/kernels/templates/gemm/packed.py:27-33); `scales [E, N, K/16]` float8_e4m3fn bytes in natural
+depth order; `scale [E]` fp32; `form` the 8-byte digest of the encoder that packed the words. MXFP4
+checkpoints enter through `NvFp4.of(*codecs.mxfp4_as_nvfp4(...))`, as the reference loads them
+(src/dew/interop/quantized_loads.py:106-143).
+
+`Fp8Blocks` / `Fp8Channels` hold e4m3 codes `[E, K, N]` with 128x128-block or per-output-channel fp32
+scales (a DeepSeek-style checkpoint's `weight` / `weight_scale_inv`, src/dew/interop/codecs.py:670-703).
+
+The HIP kernels read a one-time device re-layout of these banks (`prepared.py`); the encoder is an
+invertible GF(2) map, so that re-layout is exact.
+"""
+
+import dataclasses
+import hashlib
+
+import torch
+
+NVFP4_ENCODER = (
+    0x4000100, 0x8000202, 0x4040401, 0x2800080, 0x1000000, 0x2000000, 0x4000000, 0x8000002,
+    0x4040001, 0x20000808, 0x4010000, 0x8020002, 0x4000001, 0x8000000, 0x4040005, 0x20000008,
+    0x40001000, 0x80002020, 0x40404010, 0x20080008, 0x10000000, 0x20000000, 0x40000000, 0x80000020,
+    0x40400010, 0x2008080, 0x40100000, 0x80200020, 0x40000010, 0x80000000, 0x40400050, 0x2000080)
+"""Stored bit i = parity(natural word & NVFP4_ENCODER[i]) (src/dew/algebra/bits.py:702-705)."""
+
+FORM_HEX = hashlib.sha256(",".join(map(str, NVFP4_ENCODER)).encode()).hexdigest()[:16]
+"""Version of the stored word layout (src/dew/algebra/bits.py:306-311): 7fb7f1b609cea47a."""
+
+NVFP4_OWED = 256.0
+NVFP4_GROUP = 128
+NVFP4_STAGE = 256
+"""An NVFP4 matrix's depth is whole 256s (src/dew/nn/kernels/formats.py:139)."""
+
+
+def form_bytes(device=None) -> torch.Tensor:
+    return torch.tensor(list(bytes.fromhex(FORM_HEX)), dtype=torch.uint8, device=device)
+
+
+def staged_rows(depth: int, device=None) -> torch.Tensor:
+    """The depth each packed row holds: row `8w + j` of group g holds depth `128g + 16j + w`
+    (src/dew/nn/kernels/formats.py:144-155)."""
+    if depth % NVFP4_GROUP:
+        raise ValueError(f"an NVFP4 matrix's depth is whole {NVFP4_GROUP}-deep groups, not {depth}")
+    index = torch.arange(depth, device=device)
+    group, within = index // NVFP4_GROUP, index % NVFP4_GROUP
+    return NVFP4_GROUP * group + 16 * (within % 8) + within // 8
+
+
+def _encoder_tables(device):
+    """The encoder as four 256-entry tables, one a byte of the natural word: it is GF(2)-linear, so a
+    word's image is the xor of its bytes' images."""
+    tables = []
+    for byte in range(4):
+        column = []
+        for value in range(256):
+            natural = value << (8 * byte)
+            column.append(sum((bin(natural & mask).count("1") & 1) << bit for bit, mask in enumerate(NVFP4_ENCODER)))
+        tables.append(torch.tensor(column, dtype=torch.int64, device=device))
+    return tables
+
+
+def encoded_words(nibbles: torch.Tensor) -> torch.Tensor:
+    """Eight nibbles `[..., 8]` (code j at natural bits 4j..4j+3) as the stored word, int32 bits
+    `[...]` (`bits.packed`, src/dew/algebra/bits.py:921-931)."""
+    pairs = nibbles.to(torch.int64).reshape(*nibbles.shape[:-1], 4, 2)
+    natural_bytes = pairs[..., 0] | (pairs[..., 1] << 4)
+    tables = _encoder_tables(nibbles.device)
+    stored = tables[0][natural_bytes[..., 0]]
+    for byte in range(1, 4):
+        stored = stored ^ tables[byte][natural_bytes[..., byte]]
+    return torch.where(stored >= 2 ** 31, stored - 2 ** 32, stored).to(torch.int32)
+
+
+@dataclasses.dataclass(frozen=True)
+class NvFp4:
+    """A bank of NVFP4 expert matrices standing for `W [E, K, N]`; fields as the module docstring lays them
+    out. `words` is held as int32 (torch has no uint32 arithmetic); the bits are the reference's uint32."""
+
+    words: torch.Tensor
+    scales: torch.Tensor
+    scale: torch.Tensor
+    form: torch.Tensor = None
+
+    def __post_init__(self):
+        if self.form is None:
+            object.__setattr__(self, "form", form_bytes(self.words.device))
+
+    @classmethod
+    def of(cls, codes: torch.Tensor, scales: torch.Tensor, scale: torch.Tensor) -> "NvFp4":
+        """The bank of `codes [E, K, N]` (uint8 nibbles, sign bit 3, natural depth order), block scales
+        `[E, K/16, N]` (e4m3 bytes) and tensor scales `[E]`: packed in the staged order, K-major
+        (src/dew/nn/kernels/formats.py:82-96)."""
+        if codes.ndim == 2:
+            codes, scales, scale = codes[None], scales[None], scale.reshape(1)
+        experts, depth, width = codes.shape
+        if depth % NVFP4_STAGE:
+            raise ValueError(f"an NVFP4 matrix's depth is whole {NVFP4_STAGE}s, not {depth}")
+        ordered = codes[:, staged_rows(depth, codes.device), :]                       # [E, K (staged), N]
+        words = encoded_words(ordered.transpose(1, 2).reshape(experts, width, depth // 8, 8))
+        return cls(words.contiguous(), scales.transpose(1, 2).contiguous().view(torch.uint8),
+                   scale.to(torch.float32).reshape(experts).contiguous())
+
+    @classmethod
+    def quantized(cls, weight: torch.Tensor) -> "NvFp4":
+        """`weight [E, K, N]` quantized to NVFP4, each expert's matrix on its own
+        (src/dew/nn/kernels/formats.py:71-80)."""
+        from . import codecs
+
+        parts = [codecs.nvfp4_coded(matrix) for matrix in weight]
+        return cls.of(*(torch.stack(field) for field in zip(*parts, strict=True)))
+
+    def checked(self) -> "NvFp4":
+        """Itself where its words are this form's; refused otherwise (src/dew/nn/kernels/formats.py:49-69)."""
+        held = self.form.reshape(-1, 8).cpu()
+        found = {bytes(row.tolist()).hex() for row in held}
+        if found != {FORM_HEX}:
+            raise ValueError(f"NVFP4 words packed by form version {', '.join(sorted(found))}, where this "
+                             f"library decodes form version {FORM_HEX}: repack them from the source weights")
+        return self
+
+    @property
+    def shape(self):
+        experts, width, words = self.words.shape
+        return (experts, 8 * words, width)
+
+    @property
+    def dtype(self):
+        """The dtype its decode yields and it is multiplied as (src/dew/nn/kernels/formats.py:115-118)."""
+        return torch.bfloat16
+
+    @property
+    def factor(self) -> torch.Tensor:
+        """2^8 times each expert's tensor scale, owed to the accumulator
+        (src/dew/nn/kernels/formats.py:132-137)."""
+        return self.scale.to(torch.float32) * NVFP4_OWED
+
+    def to(self, device) -> "NvFp4":
+        return NvFp4(self.words.to(device), self.scales.to(device), self.scale.to(device), self.form.to(device))
+
+
+@dataclasses.dataclass(frozen=True)
+class Fp8Blocks:
+    """FP8 e4m3 codes `[E, K, N]` (uint8) with fp32 `scale_inv [E, ceil(K/128), ceil(N/128)]`: value
+    `f32(code) * scale_inv[k // 128, n // 128]`, rounded to the compute dtype before the product, as the
+    reference dequantizes such a checkpoint at load (src/dew/interop/codecs.py:638-648,670-703)."""
+
+    codes: torch.Tensor
+    scale_inv: torch.Tensor
+
+    @classmethod
+    def quantized(cls, weight: torch.Tensor) -> "Fp8Blocks":
+        from . import codecs
+
+        return cls(*codecs.fp8_block_cast(weight, (128, 128)))
+
+    @property
+    def shape(self):
+        return tuple(self.codes.shape)
+
+    @property
+    def dtype(self):
+        return torch.bfloat16
+
+    def to(self, device) -> "Fp8Blocks":
+        return Fp8Blocks(self.codes.to(device), self.scale_inv.to(device))
+
+
+@dataclasses.dataclass(frozen=True)
+class Fp8Channels:
+    """FP8 e4m3 codes `[E, K, N]` (uint8) with one fp32 scale per output channel `[E, N]`."""
+
+    codes: torch.Tensor
+    scales: torch.Tensor
+
+    @classmethod
+    def quantized(cls, weight: torch.Tensor) -> "Fp8Channels":
+        from . import codecs
+
+        return cls(*codecs.fp8_channel_cast(weight))
+
+    @property
+    def shape(self):
+        return tuple(self.codes.shape)
+
+    @property
+    def dtype(self):
+        return torch.bfloat16
+
+    def to(self, device) -> "Fp8Channels":
+        return Fp8Channels(self.codes.to(device), self.scales.to(device))

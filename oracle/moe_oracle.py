@@ -1,0 +1,449 @@
+"""CPU oracle for the quantized Mixture-of-Experts expert path. TEST INFRASTRUCTURE ONLY.
+
+This module is the checker the HIP kernels are compared with. Nothing in the product package imports it;
+only the tests, the smoke check and the benchmark's cpu-baseline leg do. It restates, in NumPy alone, the
+arithmetic of the reference's own JAX path on a device that has no grouped kernel: dequantize the expert
+weights, multiply each expert's sorted rows by its matrix with fp32 sums, SwiGLU with the reference's two
+roundings, down projection, fp32-weighted combine. Citations are `file:line` into the reference tree.
+
+What pins each function (see tests/test_oracle_*.py):
+
+* `route`: router_indices (exact) / router_weights (1e-6) of tests/fixtures/moe/{mixtral,deepseek,
+  deepseek_v2,deepseek_v4}.npz.
+* `sparse_mlp` (fp32 mode): block_output / experts_output of the same files (2e-5).
+* `sorted_by_expert`: brute force on tiny inputs + invariants (a stable counting sort is a closed form).
+* `dequantize_fp8_blocks`: tests/fixtures/codecs/deepseek_kernels.npz `v3/*/dequantized`, bit for bit.
+* `decode_mxfp4`: tests/fixtures/gpt_oss/mxfp4.npz `output`, bit for bit.
+* `nvfp4_words_to_codes` / `nvfp4_bank_decoded`: the 32 literal encoder masks and the 8-step decode form of
+  src/dew/algebra/bits.py:696-705 checked against each other on every basis word and random words; staged
+  order known answers of tests/test_gemm_nvfp4.py:37-38; form digest 7fb7f1b609cea47a.
+* `combine`: known answer of tests/test_moe_precision.py:652-674 (weights 1/2 +- 2^-11 give 2^-10).
+* `swiglu`: closed form, the two bf16 roundings checked on hand-computed cases.
+* `grouped_matmul`: tools/grouped_oracle.py:20-27 semantics (float64 per-group product) on integer inputs,
+  where fp32 sums are exact.
+
+Parity unpinned (no byte fixture in the reference, closed form only): the exact bits of the softmax
+denominator's compensated sum (src/dew/nn/precision.py:1832); it moves router weights by at most one fp32
+ulp and no index.
+"""
+
+import numpy as np
+
+F32 = np.float32
+
+# --------------------------------------------------------------------------------------------------
+# Number formats
+# --------------------------------------------------------------------------------------------------
+
+
+def bf16_round(x):
+    """fp32 values rounded to bfloat16 (ties to even) and held in fp32: the cast pair the reference's
+    `cast_rounded` writes (src/dew/nn/activations.py:281-286). NaN stays NaN."""
+    x = np.ascontiguousarray(x, dtype=F32)
+    bits = x.view(np.uint32)
+    rounded = (bits + (np.uint32(0x7FFF) + ((bits >> np.uint32(16)) & np.uint32(1)))) & np.uint32(0xFFFF0000)
+    out = rounded.view(F32)
+    nan = np.isnan(x)
+    if nan.any():
+        out = np.where(nan, x, out)
+    return out
+
+
+def bf16_bits(x):
+    """The uint16 bit patterns of fp32 values rounded to bfloat16."""
+    return (bf16_round(x).view(np.uint32) >> np.uint32(16)).astype(np.uint16)
+
+
+def bf16_from_bits(bits):
+    """fp32 values of bfloat16 bit patterns (uint16)."""
+    return (np.ascontiguousarray(bits, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(F32)
+
+
+def _e4m3_table():
+    """float8_e4m3fn's value for every byte (OCP 8-bit float v1.0: bias 7, no infinities, 0x7f/0xff NaN)."""
+    codes = np.arange(256, dtype=np.uint32)
+    sign = np.where(codes & 0x80, -1.0, 1.0)
+    exponent = ((codes >> 3) & 0xF).astype(np.int32)
+    mantissa = (codes & 7).astype(np.float64)
+    normal = (1.0 + mantissa / 8.0) * np.exp2(exponent - 7.0)
+    subnormal = (mantissa / 8.0) * 2.0 ** -6
+    value = np.where(exponent == 0, subnormal, normal) * sign
+    value[(codes & 0x7F) == 0x7F] = np.nan
+    return value.astype(F32)
+
+
+E4M3 = _e4m3_table()
+"""Value of every float8_e4m3fn byte."""
+
+E2M1 = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0], F32)
+"""Value of every E2M1 nibble, sign in bit 3 (src/dew/nn/fake_quant.py:21)."""
+
+
+# --------------------------------------------------------------------------------------------------
+# Dequantizers (the reference dequantizes, then multiplies in the compute dtype)
+# --------------------------------------------------------------------------------------------------
+
+
+def dequantize_fp8_blocks(codes, scale_inv, block=(128, 128)):
+    """`f32(code) * scale_inv[i // br, j // bc]` for e4m3 `codes` `[..., rows, cols]` (uint8) and fp32
+    `scale_inv` `[..., ceil(rows/br), ceil(cols/bc)]`: src/dew/interop/codecs.py:670-703 (DeepSeek's
+    weight-only reading of 128x128 block scales, contract stated at :638-648)."""
+    codes = np.asarray(codes, np.uint8)
+    rows, cols = codes.shape[-2:]
+    br, bc = block
+    each = np.repeat(np.repeat(np.asarray(scale_inv, F32), br, axis=-2), bc, axis=-1)[..., :rows, :cols]
+    return (E4M3[codes] * each).astype(F32)
+
+
+def dequantize_fp8_channels(codes, scales):
+    """Per-output-channel FP8: `codes [..., depth, width]` e4m3 bytes, `scales [..., width]` fp32, value
+    `f32(code) * scale[n]`: the frozen row-scaled rule of src/dew/quantization.py:505-525 (a `(1, K)` block
+    on the `[N, K]` view), read back in `[depth, width]` orientation."""
+    return (E4M3[np.asarray(codes, np.uint8)] * np.asarray(scales, F32)[..., None, :]).astype(F32)
+
+
+def decode_mxfp4(blocks, scales):
+    """Packed MXFP4 `[expert, out, group, 16]` bytes + E8M0 `[expert, out, group]` bytes to fp32
+    `[expert, in, out]`: low nibble first, 32 elements a scale `2^(b-127)`
+    (src/dew/interop/codecs.py:115-128,193-224)."""
+    blocks = np.asarray(blocks, np.uint8)
+    scales = np.asarray(scales, np.uint8)
+    experts, outs, groups, _ = blocks.shape
+    nibbles = np.stack([blocks & 15, blocks >> 4], axis=-1).reshape(experts, outs, groups, 32)
+    power = np.ldexp(F32(1), scales.astype(np.int32) - 127).astype(F32)
+    values = E2M1[nibbles] * power[..., None]
+    return np.ascontiguousarray(values.reshape(experts, outs, groups * 32).swapaxes(1, 2))
+
+
+# ---- NVFP4 bank: GF(2)-encoded words in staged depth order ----------------------------------------
+
+NVFP4_ENCODER = (
+    0x4000100, 0x8000202, 0x4040401, 0x2800080, 0x1000000, 0x2000000, 0x4000000, 0x8000002,
+    0x4040001, 0x20000808, 0x4010000, 0x8020002, 0x4000001, 0x8000000, 0x4040005, 0x20000008,
+    0x40001000, 0x80002020, 0x40404010, 0x20080008, 0x10000000, 0x20000000, 0x40000000, 0x80000020,
+    0x40400010, 0x2008080, 0x40100000, 0x80200020, 0x40000010, 0x80000000, 0x40400050, 0x2000080)
+"""Stored bit i of a word = parity(natural word & NVFP4_ENCODER[i]); the natural word holds code j at bits
+4j..4j+3 (src/dew/algebra/bits.py:702-705, `bits.packed` :921-931)."""
+
+NVFP4_MASK = np.uint32(0x81C081C0)
+NVFP4_OWED = 256.0
+"""The 2^8 the bf16 decode owes the accumulator (src/dew/nn/kernels/formats.py:132-137)."""
+
+
+def nvfp4_form_digest():
+    """The 8-byte version a bank stores beside its words: sha256 of the encoder masks joined by commas,
+    first 16 hex digits (src/dew/algebra/bits.py:306-311; src/dew/nn/kernels/formats.py:21)."""
+    import hashlib
+
+    return hashlib.sha256(",".join(map(str, NVFP4_ENCODER)).encode()).hexdigest()[:16]
+
+
+def _rotr32(x, n):
+    return (x >> np.uint32(n)) | (x << np.uint32(32 - n))
+
+
+def nvfp4_words_to_halves(words):
+    """The decode form of src/dew/algebra/bits.py:696-700 on stored uint32 words: a rotation by 6, three
+    left shifts, four masked xors. Returns uint16 `[..., 8]`: code j's bfloat16 bit pattern, equal to
+    `E2M1[code] * 2^-126` (code 2i the low half of register i, 2i+1 the high half)."""
+    s = np.asarray(words, np.uint32)
+    v1 = _rotr32(s, 6)
+    r0 = (s ^ v1) & NVFP4_MASK
+    r1 = (s ^ (s << np.uint32(6))) & NVFP4_MASK
+    r2 = (s ^ (v1 << np.uint32(2))) & NVFP4_MASK
+    r3 = (s << np.uint32(2)) & NVFP4_MASK
+    regs = np.stack([r0, r1, r2, r3], axis=-1)
+    halves = np.stack([regs & np.uint32(0xFFFF), regs >> np.uint32(16)], axis=-1)
+    return halves.reshape(*s.shape, 8).astype(np.uint16)
+
+
+def nvfp4_words_to_codes(words):
+    """Stored words to their eight E2M1 nibbles `[..., 8]` uint8 (sign bit 3), through the decode form: the
+    bfloat16 half has the mantissa bit at 6, exponent bits at 7-8 and sign at 15
+    (src/dew/algebra/bits.py:683-686)."""
+    halves = nvfp4_words_to_halves(words).astype(np.uint32)
+    return (((halves >> 6) & 7) | ((halves >> 15) << 3)).astype(np.uint8)
+
+
+def nvfp4_staged_depths(depth):
+    """Depth held by packed row `8w + j` of each 128-deep group: `128 g + 16 j + w`
+    (src/dew/nn/kernels/templates/gemm/packed.py:27-33; src/dew/nn/kernels/formats.py:144-155)."""
+    if depth % 128:
+        raise ValueError(f"an NVFP4 matrix's depth is whole 128-deep groups, not {depth}")
+    index = np.arange(depth)
+    group, within = np.divmod(index, 128)
+    word, code = np.divmod(within, 8)
+    return 128 * group + 16 * code + word
+
+
+def nvfp4_bank_codes(words):
+    """A bank's nibbles in natural depth order: `words [E, N, K/8]` uint32 to uint8 `[E, K, N]`."""
+    words = np.asarray(words, np.uint32)
+    experts, width, nwords = words.shape
+    staged = nvfp4_words_to_codes(words).reshape(experts, width, nwords * 8)   # staged position p = 8w + j
+    natural = np.empty_like(staged)
+    natural[..., nvfp4_staged_depths(nwords * 8)] = staged
+    return np.ascontiguousarray(natural.swapaxes(1, 2))
+
+
+def nvfp4_bank_decoded(words, scales):
+    """`NvFp4.decoded()` (src/dew/nn/kernels/formats.py:108-113): each code times its 16-block's e4m3 scale
+    over 2^8, exactly representable in bfloat16, `[E, K, N]` fp32. `scales [E, N, K/16]` are e4m3 bytes."""
+    codes = nvfp4_bank_codes(words)
+    owed = (E4M3[np.asarray(scales, np.uint8)] * F32(1.0 / NVFP4_OWED)).swapaxes(1, 2)      # [E, K/16, N]
+    values = E2M1[codes] * np.repeat(owed, 16, axis=1)
+    rounded = bf16_round(values)
+    assert np.array_equal(rounded, values), "an NVFP4 value over 2^8 is exact in bfloat16"
+    return rounded
+
+
+def nvfp4_bank_factor(scale):
+    """`NvFp4.factor`: 2^8 times each expert's tensor scale (src/dew/nn/kernels/formats.py:132-137)."""
+    return (F32(NVFP4_OWED) * np.asarray(scale, F32)).astype(F32)
+
+
+# --------------------------------------------------------------------------------------------------
+# Router (src/dew/nn/moe.py:466-565)
+# --------------------------------------------------------------------------------------------------
+
+_LN2_HI, _LN2_LO = F32(0.693145751953125), F32(1.428606765330187e-06)
+_EXP_TERMS = tuple(F32(t) for t in (1.0 / 5040.0, 1.0 / 720.0, 1.0 / 120.0, 1.0 / 24.0, 1.0 / 6.0, 0.5, 1.0, 1.0))
+_INV_LN2 = F32(1.0 / np.log(2.0))
+
+
+def exp_f32(x):
+    """`e^x` in fp32 by one fixed sequence of IEEE fp32 operations, no fused multiply-add: Cody-Waite
+    reduction `x = n ln2 + r`, Taylor sum to r^7 by Horner, times 2^n in two exact steps. The algorithm is
+    the reference's own portable exp (src/dew/nn/precision.py:470-488); the HIP router runs the same
+    sequence, so scores and hence top-k choices agree bit for bit between the two."""
+    x = np.clip(np.asarray(x, F32), F32(-104.0), F32(90.0))
+    n = np.rint(x * _INV_LN2).astype(F32)
+    r = ((x - n * _LN2_HI).astype(F32) - (n * _LN2_LO).astype(F32)).astype(F32)
+    p = np.full_like(r, _EXP_TERMS[0])
+    for term in _EXP_TERMS[1:]:
+        p = ((p * r).astype(F32) + term).astype(F32)
+    n = n.astype(np.int32)
+    half = n // 2                                  # floor division: both halves stay normal exponents
+    first = np.ldexp(F32(1), half).astype(F32)
+    second = np.ldexp(F32(1), n - half).astype(F32)
+    return ((p * first).astype(F32) * second).astype(F32)
+
+
+def _sum_rounded_once(values):
+    """Sum over the last axis, rounded once to fp32: the role of `compensated_sum`
+    (src/dew/nn/precision.py:1832-1844). Realised as a float64 sum in one fixed order (64 interleaved
+    partial sums, then a halving tree), the order the HIP router's wave reduction uses."""
+    v = np.asarray(values, np.float64)
+    count = v.shape[-1]
+    lanes = np.zeros((*v.shape[:-1], 64), np.float64)
+    for start in range(0, count, 64):
+        chunk = v[..., start:start + 64]
+        lanes[..., :chunk.shape[-1]] += chunk
+    width = 32
+    while width >= 1:
+        lanes = lanes[..., :width] + lanes[..., width:2 * width]
+        width //= 2
+    return lanes[..., 0].astype(F32)
+
+
+def expert_softmax(logits):
+    """src/dew/nn/moe.py:184-191: exp(x - max) over their once-rounded sum, IEEE division."""
+    logits = np.asarray(logits, F32)
+    shifted = exp_f32(logits - logits.max(axis=-1, keepdims=True))
+    return (shifted / _sum_rounded_once(shifted)[..., None]).astype(F32)
+
+
+def logistic(x, exp=exp_f32):
+    """`1 / (1 + e^-x)` in fp32 with a true division (src/dew/nn/precision.py:568-575)."""
+    x = np.asarray(x, F32)
+    return (F32(1) / (F32(1) + exp(-x)).astype(F32)).astype(F32)
+
+
+def sqrt_softplus(x):
+    """DeepSeek V4's score `sqrt(softplus(x))` (src/dew/nn/moe.py:539-540); float64 inside, for the
+    fixture's sake only (no BASELINE config uses it)."""
+    x = np.asarray(x, np.float64)
+    return np.sqrt(np.logaddexp(0.0, x)).astype(F32)
+
+
+def top_k(values, k):
+    """`jax.lax.top_k`: the k largest along the last axis in descending order, ties to the lower index.
+    Returns (values, indices int32)."""
+    values = np.asarray(values)
+    order = np.argsort(-values, axis=-1, kind="stable")[..., :k]
+    return np.take_along_axis(values, order, axis=-1), order.astype(np.int32)
+
+
+def route(logits, top_k_count, *, score_function="softmax", normalize_weights=True, bias=None,
+          routed_scaling_factor=1.0, expert_groups=1, groups_per_token=1, group_score="top2",
+          weight_sum_epsilon=1e-20):
+    """`Router.__call__` from its logits on (src/dew/nn/moe.py:466-494): scores, selection (bias,
+    group-limited mask :496-565), top-k, weights. Returns (weights fp32 [T, k], indices int32 [T, k])."""
+    logits = np.asarray(logits, F32)
+    experts = logits.shape[-1]
+    if score_function == "softmax":
+        scores = expert_softmax(logits)
+    elif score_function == "sigmoid":
+        scores = logistic(logits)
+    elif score_function == "sqrtsoftplus":
+        scores = sqrt_softplus(logits)
+    else:
+        raise ValueError(score_function)
+    selection = scores if bias is None else (scores + np.asarray(bias, F32)).astype(F32)
+    if expert_groups > 1:
+        per_group = experts // expert_groups
+        grouped = selection.reshape(*selection.shape[:-1], expert_groups, per_group)
+        if group_score == "max":
+            group_scores = grouped.max(axis=-1)
+        else:
+            best_two, _ = top_k(grouped, 2)
+            group_scores = (best_two[..., 0] + best_two[..., 1]).astype(F32)
+        _, groups = top_k(group_scores, groups_per_token)
+        kept = np.zeros(group_scores.shape, bool)
+        np.put_along_axis(kept, groups, True, axis=-1)
+        selection = np.where(np.repeat(kept, per_group, axis=-1), selection, F32(-np.inf))
+    _, indices = top_k(selection, top_k_count)
+    if normalize_weights and score_function == "softmax":
+        weights = expert_softmax(np.take_along_axis(logits, indices, axis=-1))        # moe.py:194-199,485
+    else:
+        weights = np.take_along_axis(scores, indices, axis=-1)
+        if normalize_weights:
+            total = weights[..., 0].copy()
+            for j in range(1, top_k_count):
+                total = (total + weights[..., j]).astype(F32)
+            total = (total + F32(weight_sum_epsilon)).astype(F32)
+            weights = (weights / total[..., None]).astype(F32)
+    return (weights * F32(routed_scaling_factor)).astype(F32), indices
+
+
+def router_logits(x, kernel):
+    """`Router.logits` (src/dew/nn/moe.py:526-534): IEEE fp32 product of the tokens (widened to fp32) and
+    the `[D, E]` fp32 kernel."""
+    return (np.asarray(x, F32) @ np.asarray(kernel, F32)).astype(F32)
+
+
+# --------------------------------------------------------------------------------------------------
+# Dispatch (src/dew/nn/moe.py:1101-1128)
+# --------------------------------------------------------------------------------------------------
+
+
+def sorted_by_expert(indices, num_experts):
+    """`_sorted_locally`'s bookkeeping: stable argsort of the flattened expert ids, group sizes, offsets,
+    and the token row each sorted slot reads. Returns dict(order, rows, sizes, offsets), all int32."""
+    indices = np.asarray(indices)
+    k = indices.shape[-1]
+    experts = indices.reshape(-1)
+    order = np.argsort(experts, kind="stable").astype(np.int32)
+    sizes = np.bincount(experts, minlength=num_experts)[:num_experts].astype(np.int32)
+    offsets = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    return {"order": order, "rows": (order // k).astype(np.int32), "sizes": sizes, "offsets": offsets}
+
+
+# --------------------------------------------------------------------------------------------------
+# Grouped products, SwiGLU, combine
+# --------------------------------------------------------------------------------------------------
+
+
+def grouped_matmul(x, w, sizes, *, dtype="bfloat16", factor=None, accumulate=F32):
+    """Each group's leading rows of `x [rows, depth]` times its matrix `w [groups, depth, width]`
+    (`jax.lax.ragged_dot` semantics, src/dew/nn/kernels/xla_products.py:86-115): operands rounded to the
+    compute dtype, products summed in fp32 (`accumulate`), one rounding to the compute dtype; rows past
+    `sum(sizes)` are zero. `factor [groups]` multiplies the fp32 sums before the rounding (the NVFP4
+    bank's deferred factor, src/dew/nn/kernels/gemm.py:660-662)."""
+    x = np.asarray(x, F32)
+    w = np.asarray(w, F32)
+    if dtype == "bfloat16":
+        x = bf16_round(x)
+    out = np.zeros((x.shape[0], w.shape[2]), F32)
+    start = 0
+    for group, size in enumerate(np.asarray(sizes).tolist()):
+        if size:
+            matrix = bf16_round(w[group]) if dtype == "bfloat16" else w[group]
+            summed = (x[start:start + size].astype(accumulate) @ matrix.astype(accumulate))
+            if factor is not None:
+                summed = summed.astype(F32) * F32(factor[group])
+            out[start:start + size] = summed.astype(F32)
+        start += size
+    return bf16_round(out) if dtype == "bfloat16" else out
+
+
+def swiglu(gate, up, *, dtype="bfloat16", limit=None, exp=np.exp):
+    """`gated_product('swiglu')` after `swiglu_clamped` (src/dew/nn/activations.py:267-278,327-356):
+    bf16 rounds the activation `g * logistic(g)` and then the product with `u`; fp32 rounds nowhere.
+    The reference's exp here is the backend's own accurate one, so NumPy's stands for it."""
+    gate, up = np.asarray(gate, F32), np.asarray(up, F32)
+    if limit is not None:
+        gate, up = np.minimum(gate, F32(limit)), np.clip(up, F32(-limit), F32(limit))
+    sig = (F32(1) / (F32(1) + exp(-gate).astype(F32)).astype(F32)).astype(F32)
+    if dtype != "bfloat16":
+        return ((gate * sig).astype(F32) * up).astype(F32)
+    gate, up = bf16_round(gate), bf16_round(up)
+    sig = (F32(1) / (F32(1) + exp(-gate).astype(F32)).astype(F32)).astype(F32)
+    activated = bf16_round((gate * sig).astype(F32))
+    return bf16_round((activated * up).astype(F32))
+
+
+def combine(slots, weights, *, dtype="bfloat16"):
+    """`ExpertMLP._combine` (src/dew/nn/moe.py:1328-1333): `out[t] = round(sum_j f32(y[t, j]) * w[t, j])`,
+    fp32 weights, fp32 sum in slot order, one rounding."""
+    slots = np.asarray(slots, F32)
+    weights = np.asarray(weights, F32)
+    total = np.zeros((slots.shape[0], slots.shape[2]), F32)
+    for j in range(slots.shape[1]):
+        total = (total + (slots[:, j, :] * weights[:, j, None]).astype(F32)).astype(F32)
+    return bf16_round(total) if dtype == "bfloat16" else total
+
+
+def expert_mlp(x, weights, indices, gate_w, up_w, down_w, *, dtype="bfloat16", factors=(None, None, None),
+               limit=None):
+    """`ExpertMLP.__call__` (src/dew/nn/moe.py:1335-1353) on one device: sort, gather, paired gate/up
+    products, SwiGLU, down product scattered to slot order, combine. The matrices are the dequantized
+    `[E, depth, width]` values. Returns (out [T, D], trace dict of the intermediates)."""
+    x = np.asarray(x, F32)
+    experts = gate_w.shape[0]
+    plan = sorted_by_expert(indices, experts)
+    rows = x[plan["rows"]]
+    gate = grouped_matmul(rows, gate_w, plan["sizes"], dtype=dtype, factor=factors[0])
+    up = grouped_matmul(rows, up_w, plan["sizes"], dtype=dtype, factor=factors[1])
+    hidden = swiglu(gate, up, dtype=dtype, limit=limit)
+    projected = grouped_matmul(hidden, down_w, plan["sizes"], dtype=dtype, factor=factors[2])
+    slots = np.zeros_like(projected)
+    slots[plan["order"]] = projected
+    tokens, k = np.asarray(indices).shape
+    slots = slots.reshape(tokens, k, -1)
+    out = combine(slots, weights, dtype=dtype)
+    return out, {**plan, "gate": gate, "up": up, "hidden": hidden, "slots": slots}
+
+
+def gated_mlp(x, gate_w, up_w, down_w, *, dtype="bfloat16"):
+    """The dense shared expert (`GatedMLP`, src/dew/nn/mlp.py:106,239): SwiGLU MLP on every token, the same
+    rounding points as one expert holding all rows."""
+    sizes = [np.asarray(x).shape[0]]
+    gate = grouped_matmul(x, np.asarray(gate_w)[None], sizes, dtype=dtype)
+    up = grouped_matmul(x, np.asarray(up_w)[None], sizes, dtype=dtype)
+    return grouped_matmul(swiglu(gate, up, dtype=dtype), np.asarray(down_w)[None], sizes, dtype=dtype)
+
+
+def sparse_mlp(x, logits, gate_w, up_w, down_w, *, top_k_count, dtype="bfloat16", shared=None,
+               factors=(None, None, None), limit=None, **router):
+    """`SparseMLP.__call__` (src/dew/nn/moe.py:1488-1503) from the router logits on: route, routed
+    experts, plus the shared expert's output (`shared` = its three dense matrices)."""
+    weights, indices = route(logits, top_k_count, **router)
+    routed, trace = expert_mlp(x, weights, indices, gate_w, up_w, down_w, dtype=dtype, factors=factors,
+                               limit=limit)
+    trace.update(weights=weights, indices=indices)
+    if shared is not None:
+        both = routed + gated_mlp(x, *shared, dtype=dtype)
+        routed = bf16_round(both) if dtype == "bfloat16" else both.astype(F32)
+    return routed, trace
+
+
+def relative_errors(got, want, floor=None):
+    """The two error figures reported per config: the reference's own `max|d| / max|want|`
+    (tools/benchmark_kernels.py:143-144) and the element-wise max relative error with an absolute floor
+    (by default 1% of max|want|) under the denominator."""
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    scale = np.abs(want).max()
+    floor = 1e-2 * scale if floor is None else floor
+    delta = np.abs(got - want)
+    return float(delta.max() / scale), float((delta / np.maximum(np.abs(want), floor)).max())

@@ -1,0 +1,255 @@
+"""Pins the CPU oracle against the golden vectors the reference's own tests hold, and against what the
+mathematics fixes, so that a dropped term, a wrong sign or a transposed operand fails here."""
+
+import numpy as np
+import pytest
+from conftest import golden
+
+from oracle import moe_oracle as oracle
+
+ROUTER_TOLERANCE = 1e-6      # tests/test_moe.py:37 of the reference
+OUTPUT_TOLERANCE = 2e-5      # tests/test_moe.py:40
+
+
+def by_expert(indices, weights):
+    order = np.argsort(indices, axis=-1, kind="stable")
+    return np.take_along_axis(indices, order, -1), np.take_along_axis(weights, order, -1)
+
+
+def stacked(tensors, projection, experts):
+    return np.stack([tensors[f"mlp.experts.{e}.{projection}.weight"].T for e in range(experts)])
+
+
+ROUTERS = {
+    "mixtral": dict(score_function="softmax", normalize_weights=True),
+    "deepseek": dict(score_function="sigmoid", normalize_weights=True, routed_scaling_factor=2.5,
+                     expert_groups=4, groups_per_token=2, biased=True),
+    "deepseek_v2": dict(score_function="softmax", normalize_weights=False, routed_scaling_factor=2.5,
+                        expert_groups=4, groups_per_token=2, group_score="max"),
+    "deepseek_v4": dict(score_function="sqrtsoftplus", normalize_weights=True, routed_scaling_factor=2.5,
+                        biased=True),
+}
+
+
+def routed(name):
+    tensors = golden(f"moe/{name}.npz")
+    settings = dict(ROUTERS[name])
+    bias = tensors["mlp.gate.e_score_correction_bias"] if settings.pop("biased", False) else None
+    hidden = tensors["hidden"].reshape(-1, tensors["hidden"].shape[-1])
+    logits = oracle.router_logits(hidden, tensors["mlp.gate.weight"].T)
+    k = tensors["router_indices"].shape[-1]
+    return tensors, hidden, logits, k, dict(settings, bias=bias)
+
+
+@pytest.mark.parametrize("name", list(ROUTERS))
+def test_router_reproduces_the_recorded_choice_and_gate_values(name):
+    tensors, _, logits, k, settings = routed(name)
+    weights, indices = oracle.route(logits, k, **settings)
+    theirs_i, theirs_w = by_expert(tensors["router_indices"], tensors["router_weights"])
+    ours_i, ours_w = by_expert(indices, weights)
+    assert np.array_equal(ours_i, theirs_i)
+    assert np.abs(ours_w - theirs_w).max() < ROUTER_TOLERANCE
+
+
+def test_fp32_block_reproduces_the_mixtral_block_output():
+    tensors, hidden, logits, k, settings = routed("mixtral")
+    mats = [stacked(tensors, p, 8) for p in ("gate_proj", "up_proj", "down_proj")]
+    out, _ = oracle.sparse_mlp(hidden, logits, *mats, top_k_count=k, dtype="float32", **settings)
+    assert np.abs(out - tensors["block_output"].reshape(out.shape)).max() < OUTPUT_TOLERANCE
+
+
+def test_fp32_block_reproduces_the_deepseek_block_output_with_its_shared_expert():
+    tensors, hidden, logits, k, settings = routed("deepseek")
+    mats = [stacked(tensors, p, 8) for p in ("gate_proj", "up_proj", "down_proj")]
+    shared = [tensors[f"mlp.shared_experts.{p}.weight"].T for p in ("gate_proj", "up_proj", "down_proj")]
+    out, _ = oracle.sparse_mlp(hidden, logits, *mats, top_k_count=k, dtype="float32", shared=shared,
+                               **settings)
+    assert np.abs(out - tensors["block_output"].reshape(out.shape)).max() < OUTPUT_TOLERANCE
+    without, _ = oracle.sparse_mlp(hidden, logits, *mats, top_k_count=k, dtype="float32", **settings)
+    assert np.abs(without - tensors["block_output"].reshape(out.shape)).max() > 1e-2
+
+
+def test_fp32_experts_reproduce_the_deepseek_v4_clamped_output():
+    tensors = golden("moe/deepseek_v4.npz")
+    hidden = tensors["hidden"].reshape(-1, 16)
+    mats = [stacked(tensors, p, 8) for p in ("gate_proj", "up_proj", "down_proj")]
+    out, _ = oracle.expert_mlp(hidden, tensors["router_weights"], tensors["router_indices"], *mats,
+                               dtype="float32", limit=1.0)
+    assert np.abs(out - tensors["experts_output"]).max() < OUTPUT_TOLERANCE
+    unclamped, _ = oracle.expert_mlp(hidden, tensors["router_weights"], tensors["router_indices"], *mats,
+                                     dtype="float32")
+    assert np.abs(unclamped - tensors["experts_output"]).max() > 1.0
+
+
+def test_top_k_takes_the_lower_index_on_ties_in_descending_order():
+    values = np.array([[1.0, 3.0, 3.0, -np.inf, 2.0, 3.0]], np.float32)
+    got_values, got = oracle.top_k(values, 4)
+    assert got.tolist() == [[1, 2, 5, 4]] and got_values.tolist() == [[3.0, 3.0, 3.0, 2.0]]
+
+
+def test_exp_matches_float64_to_two_ulp_and_is_exact_at_zero():
+    x = np.linspace(-87, 88, 200001).astype(np.float32)
+    got = oracle.exp_f32(x).astype(np.float64)
+    want = np.exp(x.astype(np.float64))
+    assert np.max(np.abs(got - want) / want) < 2.5e-7
+    assert oracle.exp_f32(np.float32(0.0)) == 1.0
+    assert oracle.exp_f32(np.float32(-104.0)) < 1e-44 and np.isfinite(oracle.exp_f32(np.float32(88.0)))
+
+
+def test_softmax_sums_to_one_and_orders_as_its_logits():
+    rng = np.random.default_rng(0)
+    logits = rng.standard_normal((512, 128)).astype(np.float32)
+    scores = oracle.expert_softmax(logits)
+    assert np.abs(scores.astype(np.float64).sum(-1) - 1).max() < 1e-6
+    want = np.exp(logits.astype(np.float64))
+    want /= want.sum(-1, keepdims=True)
+    assert np.abs(scores - want).max() < 2e-8
+    assert np.array_equal(np.argsort(-scores, -1, kind="stable")[:, :8], np.argsort(-logits, -1, kind="stable")[:, :8])
+
+
+# ---- dispatch ------------------------------------------------------------------------------------
+
+
+def test_sort_by_expert_is_the_stable_counting_sort():
+    rng = np.random.default_rng(1)
+    for tokens, k, experts in ((1, 1, 1), (7, 2, 4), (64, 8, 128), (300, 3, 5)):
+        indices = rng.integers(0, experts, size=(tokens, k)).astype(np.int32)
+        plan = oracle.sorted_by_expert(indices, experts)
+        flat = indices.reshape(-1)
+        brute = sorted(range(flat.size), key=lambda slot: (flat[slot], slot))       # brute force
+        assert plan["order"].tolist() == brute
+        assert plan["sizes"].tolist() == [int((flat == e).sum()) for e in range(experts)]
+        assert plan["offsets"][0] == 0 and np.array_equal(np.diff(plan["offsets"]), plan["sizes"])
+        assert np.array_equal(plan["rows"], plan["order"] // k)
+        assert (np.diff(flat[plan["order"]]) >= 0).all()
+
+
+# ---- formats --------------------------------------------------------------------------------------
+
+
+def test_bf16_rounding_ties_to_even():
+    x = np.array([1.0, 1.0 + 2 ** -8, 1.0 + 3 * 2 ** -8, 1.0 + 2 ** -8 + 2 ** -20, -3.3895e38], np.float32)
+    want = np.array([1.0, 1.0, 1.0 + 2 ** -6, 1.0 + 2 ** -7, -3.3895314e38], np.float32)
+    got = oracle.bf16_round(x)
+    assert np.array_equal(got[:4], want[:4]) and np.isfinite(got[4])
+    assert np.array_equal(oracle.bf16_from_bits(oracle.bf16_bits(x)), got)
+
+
+def test_e4m3_table_known_values():
+    table = oracle.E4M3
+    assert table[0x00] == 0 and table[0x01] == 2.0 ** -9 and table[0x08] == 2.0 ** -6
+    assert table[0x38] == 1.0 and table[0x7E] == 448.0 and np.isnan(table[0x7F]) and table[0xFE] == -448.0
+    import torch
+    theirs = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).float().numpy()
+    assert np.array_equal(np.nan_to_num(table, nan=7.0), np.nan_to_num(theirs, nan=7.0))
+
+
+@pytest.mark.parametrize("shape", ["256x384", "130x259", "5x7"])
+def test_fp8_block_dequantize_reproduces_the_deepseek_kernels_bytes(shape):
+    held = golden("codecs/deepseek_kernels.npz")
+    got = oracle.dequantize_fp8_blocks(held[f"v3/{shape}/codes"], held[f"v3/{shape}/scales"])
+    assert np.array_equal(got.view(np.uint32), held[f"v3/{shape}/dequantized"].view(np.uint32))
+
+
+def test_fp8_channel_dequantize_is_the_block_rule_with_one_column_blocks():
+    rng = np.random.default_rng(2)
+    codes = rng.integers(0, 0x7E, size=(3, 8, 5)).astype(np.uint8)
+    scales = rng.uniform(0.5, 2, size=(3, 5)).astype(np.float32)
+    got = oracle.dequantize_fp8_channels(codes, scales)
+    want = oracle.dequantize_fp8_blocks(codes, scales[:, None, :], block=(8, 1))
+    assert np.array_equal(got, want)
+
+
+def test_mxfp4_decode_reproduces_the_gpt_oss_fixture():
+    held = golden("gpt_oss/mxfp4.npz")
+    got = oracle.decode_mxfp4(held["blocks"], held["scales"])
+    assert np.array_equal(got.view(np.uint32), held["output"].view(np.uint32))
+
+
+def natural_word(codes):
+    return sum(int(c) << (4 * j) for j, c in enumerate(codes))
+
+
+def encode_word(natural):
+    return sum((bin(natural & mask).count("1") & 1) << i for i, mask in enumerate(oracle.NVFP4_ENCODER))
+
+
+def test_nvfp4_decode_form_inverts_the_encoder_masks_on_every_basis_word_and_every_code():
+    assert oracle.nvfp4_form_digest() == "7fb7f1b609cea47a"
+    # GF(2)-linear: the 32 basis words and zero fix the map; every code in every position besides.
+    naturals = [0] + [1 << bit for bit in range(32)] + [natural_word([c] * 8) for c in range(16)]
+    rng = np.random.default_rng(3)
+    naturals += [int(v) for v in rng.integers(0, 2 ** 32, size=4000, dtype=np.uint64)]
+    stored = np.array([encode_word(n) for n in naturals], np.uint32)
+    codes = oracle.nvfp4_words_to_codes(stored)
+    want = np.array([[(n >> (4 * j)) & 15 for j in range(8)] for n in naturals], np.uint8)
+    assert np.array_equal(codes, want)
+    halves = oracle.nvfp4_words_to_halves(stored)
+    values = oracle.bf16_from_bits(halves).astype(np.float64) * 2.0 ** 126
+    assert np.array_equal(values, oracle.E2M1[want].astype(np.float64))
+
+
+def test_nvfp4_staged_order_known_answers():
+    order = oracle.nvfp4_staged_depths(256)          # tests/test_gemm_nvfp4.py:37-38
+    assert sorted(order.tolist()) == list(range(256))
+    assert order[8 * 3 + 5] == 16 * 5 + 3 and order[128] == 128
+
+
+def test_nvfp4_bank_decodes_to_code_times_scale_over_256():
+    rng = np.random.default_rng(4)
+    experts, depth, width = 2, 256, 3
+    codes = rng.integers(0, 16, size=(experts, depth, width)).astype(np.uint8)
+    scales = rng.integers(0x20, 0x50, size=(experts, width, depth // 16)).astype(np.uint8)
+    staged = codes[:, oracle.nvfp4_staged_depths(depth), :].swapaxes(1, 2).reshape(experts, width, depth // 8, 8)
+    words = np.array([[[encode_word(natural_word(w)) for w in column] for column in bank] for bank in staged],
+                     np.uint32)
+    assert np.array_equal(oracle.nvfp4_bank_codes(words), codes)
+    decoded = oracle.nvfp4_bank_decoded(words, scales)
+    want = oracle.E2M1[codes] * np.repeat(oracle.E4M3[scales].swapaxes(1, 2), 16, axis=1) / 256
+    assert np.array_equal(decoded, want.astype(np.float32))
+    assert oracle.nvfp4_bank_factor(np.float32(0.25)) == 64.0
+
+
+# ---- products --------------------------------------------------------------------------------------
+
+
+def test_grouped_matmul_is_the_float64_per_group_product_on_small_integers():
+    rng = np.random.default_rng(5)
+    sizes = [3, 0, 5, 1]
+    x = rng.integers(-3, 4, size=(12, 16)).astype(np.float32)       # 3 rows past the routed ones
+    w = rng.integers(-2, 3, size=(4, 16, 8)).astype(np.float32)
+    got = oracle.grouped_matmul(x, w, sizes)
+    want = np.zeros((12, 8))
+    start = 0
+    for group, size in enumerate(sizes):                             # tools/grouped_oracle.py:20-27
+        want[start:start + size] = x[start:start + size].astype(np.float64) @ w[group].astype(np.float64)
+        start += size
+    assert np.array_equal(got.astype(np.float64), want) and not got[9:].any()
+    scaled = oracle.grouped_matmul(x, w, sizes, factor=np.array([2, 2, .5, 4], np.float32))
+    assert np.array_equal(scaled[:3], got[:3] * 2) and np.array_equal(scaled[3:8], got[3:8] * .5)
+
+
+def test_grouped_matmul_rounds_operands_to_bf16_and_the_sum_once():
+    x = np.array([[1 + 2 ** -9, 1.0]], np.float32)                    # first rounds to 1 in bf16
+    w = np.array([[[1.0], [2 ** -9]]], np.float32)
+    assert oracle.grouped_matmul(x, w, [1])[0, 0] == 1.0              # 1 + 2^-9 rounds once to 1
+    assert oracle.grouped_matmul(x, w, [1], dtype="float32")[0, 0] == np.float32(1 + 2 ** -9 + 2 ** -9)
+
+
+def test_swiglu_rounds_after_the_activation_and_again_after_the_product():
+    gate = np.array([1.0, -2.0, 0.0, 20.0], np.float32)
+    up = np.array([3.0, 1.5, 5.0, 1.0 + 2 ** -7], np.float32)
+    got = oracle.swiglu(gate, up)
+    for g, u, h in zip(gate.tolist(), up.tolist(), got.tolist(), strict=True):
+        silu = np.float32(g / (1 + np.exp(-np.float64(g))))
+        activated = oracle.bf16_round(np.array([silu], np.float32))[0]
+        assert h == oracle.bf16_round(np.array([activated * np.float32(u)], np.float32))[0]
+    # Two roundings differ from one: silu(1)=0.7310586 -> bf16 0.73046875; times 3 = 2.19140625 -> 2.1875
+    assert got[0] == 2.1875 and oracle.bf16_round(np.array([0.7310586 * 3], np.float32))[0] == 2.1875
+    assert oracle.swiglu(gate, up, dtype="float32")[0] == np.float32(np.float32(0.7310586) * 3)
+
+
+def test_bf16_combine_weighs_in_fp32_and_rounds_once():
+    slots = np.array([[[1.0], [-1.0]]], np.float32)                   # tests/test_moe_precision.py:652-674
+    weights = np.array([[0.5 + 2 ** -11, 0.5 - 2 ** -11]], np.float32)
+    assert oracle.combine(slots, weights)[0, 0] == 2.0 ** -10
