@@ -1,0 +1,80 @@
+"""Loader of libdew_moe_hip.so and its C ABI (include/dew_moe_hip.h) through ctypes.
+
+The library is the only compute path: nothing here falls back to PyTorch or the CPU. A missing library
+raises on first use, naming the build command."""
+
+import ctypes
+import os
+from pathlib import Path
+
+LIBRARY = Path(__file__).resolve().parent / "libdew_moe_hip.so"
+
+W_FP8_BLOCK, W_FP8_CHANNEL, W_NVFP4 = 1, 2, 3
+LAYOUT_REFERENCE, LAYOUT_PREPARED = 0, 1
+SCORE_SOFTMAX, SCORE_SIGMOID = 0, 1
+
+EXPORTS = (
+    "dew_moe_last_error", "dew_moe_architecture", "dew_moe_kernels", "dew_moe_kernel_fields",
+    "dew_moe_device_check", "dew_moe_route", "dew_moe_permute_workspace_bytes", "dew_moe_permute",
+    "dew_moe_prepared_bytes", "dew_moe_prepare_bank", "dew_moe_grouped_gemm", "dew_moe_gateup_swiglu",
+    "dew_moe_swiglu", "dew_moe_combine",
+)
+"""Every symbol include/dew_moe_hip.h declares."""
+
+
+class Bank(ctypes.Structure):
+    """`dew_moe_bank` of include/dew_moe_hip.h."""
+
+    _fields_ = [("format", ctypes.c_int32), ("layout", ctypes.c_int32), ("experts", ctypes.c_int32),
+                ("depth", ctypes.c_int32), ("width", ctypes.c_int32), ("codes", ctypes.c_void_p),
+                ("scales", ctypes.c_void_p), ("tensor_scale", ctypes.c_void_p)]
+
+
+class KernelError(RuntimeError):
+    """An entry point refused its arguments or a launch failed; the message is the library's own."""
+
+
+_handle = None
+
+
+def library() -> ctypes.CDLL:
+    """The loaded library, its prototypes declared. Raises if it has not been built."""
+    global _handle
+    if _handle is not None:
+        return _handle
+    path = Path(os.environ.get("DEW_MOE_HIP_LIBRARY", LIBRARY))
+    if not path.exists():
+        raise KernelError(f"{path} is not built: run `make -C {LIBRARY.parent / 'csrc'}` (or "
+                          f"`python -c 'import __graft_entry__ as g; g.build()'` at the repository root). "
+                          f"There is no CPU or PyTorch fallback for the MoE kernels.")
+    lib = ctypes.CDLL(str(path))
+    c = ctypes
+    ptr, i32, i64, f32, size = c.c_void_p, c.c_int32, c.c_int64, c.c_float, c.c_size_t
+    bank = c.POINTER(Bank)
+    prototypes = {
+        "dew_moe_last_error": (c.c_char_p, []),
+        "dew_moe_architecture": (c.c_char_p, []),
+        "dew_moe_kernels": (c.c_char_p, []),
+        "dew_moe_kernel_fields": (c.c_char_p, []),
+        "dew_moe_device_check": (i32, []),
+        "dew_moe_route": (i32, [ptr, ptr, i32, i32, i32, i32, i32, f32, i32, i32, ptr, ptr, ptr]),
+        "dew_moe_permute_workspace_bytes": (size, [i32, i32]),
+        "dew_moe_permute": (i32, [ptr, i32, i32, i32, ptr, ptr, ptr, ptr, ptr, size, ptr]),
+        "dew_moe_prepared_bytes": (size, [i32, i32, i32, i32]),
+        "dew_moe_prepare_bank": (i32, [bank, ptr, bank, ptr]),
+        "dew_moe_grouped_gemm": (i32, [ptr, ptr, ptr, bank, ptr, ptr, i32, ptr]),
+        "dew_moe_gateup_swiglu": (i32, [ptr, ptr, ptr, bank, bank, ptr, i32, ptr]),
+        "dew_moe_swiglu": (i32, [ptr, ptr, ptr, i64, ptr]),
+        "dew_moe_combine": (i32, [ptr, ptr, ptr, ptr, i32, i32, i32, ptr]),
+    }
+    for name, (restype, argtypes) in prototypes.items():
+        function = getattr(lib, name)
+        function.restype, function.argtypes = restype, argtypes
+    _handle = lib
+    return lib
+
+
+def check(code: int, what: str) -> None:
+    """Raise `KernelError` with the library's message unless `code` is 0."""
+    if code != 0:
+        raise KernelError(f"{what}: {library().dew_moe_last_error().decode()} (code {code})")

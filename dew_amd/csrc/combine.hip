@@ -1,0 +1,105 @@
+// Weighted combine of a token's k expert outputs, and the stand-alone SwiGLU product.
+// Both are HBM-bound elementwise kernels: 16-byte loads and stores, fp32 arithmetic, explicit roundings.
+#include "common.h"
+
+#pragma clang fp contract(off)
+
+namespace dew {
+
+struct alignas(16) Bf16x8 {
+  bf16_t v[8];
+};
+
+// out[t, :] = bf16( sum_j f32(slots[t, j, :]) * weights[t, j] ): the products and the running sum each
+// round to fp32 in slot order, then one rounding to bf16 (reference src/dew/nn/moe.py:1328-1333). With an
+// addend, out = bf16(f32(out) + f32(addend)), the shared expert's bf16 add (src/dew/nn/moe.py:1503).
+__global__ __launch_bounds__(256) void combine_kernel(const bf16_t* __restrict__ slots,
+                                                      const float* __restrict__ weights,
+                                                      const bf16_t* __restrict__ addend, bf16_t* __restrict__ out,
+                                                      int tokens, int top_k, int width) {
+  const int chunks = width / 8;
+  const long long total = static_cast<long long>(tokens) * chunks;
+  for (long long item = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; item < total;
+       item += static_cast<long long>(gridDim.x) * blockDim.x) {
+    const int token = static_cast<int>(item / chunks);
+    const int chunk = static_cast<int>(item % chunks);
+    float sum[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sum[i] = 0.0f;
+    const bf16_t* base = slots + (static_cast<size_t>(token) * top_k) * width + static_cast<size_t>(chunk) * 8;
+    for (int j = 0; j < top_k; ++j) {
+      const float w = weights[static_cast<size_t>(token) * top_k + j];
+      const Bf16x8 y = *reinterpret_cast<const Bf16x8*>(base + static_cast<size_t>(j) * width);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float product = bf16_to_f32(y.v[i]) * w;
+        sum[i] = sum[i] + product;
+      }
+    }
+    Bf16x8 result;
+    if (addend != nullptr) {
+      const Bf16x8 a = *reinterpret_cast<const Bf16x8*>(addend + static_cast<size_t>(token) * width +
+                                                       static_cast<size_t>(chunk) * 8);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) result.v[i] = f32_to_bf16(bf16_round(sum[i]) + bf16_to_f32(a.v[i]));
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) result.v[i] = f32_to_bf16(sum[i]);
+    }
+    *reinterpret_cast<Bf16x8*>(out + static_cast<size_t>(token) * width + static_cast<size_t>(chunk) * 8) = result;
+  }
+}
+
+// a = bf16(g * logistic(g)); h = bf16(a * u), on bf16 gate and up
+// (reference src/dew/nn/activations.py:267-278; logistic = 1 / (1 + e^-x) with a true division).
+__device__ __forceinline__ bf16_t swiglu_one(float g, float u) {
+  const float sig = 1.0f / (1.0f + expf(-g));
+  const float activated = bf16_round(g * sig);
+  return f32_to_bf16(activated * u);
+}
+
+__global__ __launch_bounds__(256) void swiglu_kernel(const bf16_t* __restrict__ gate, const bf16_t* __restrict__ up,
+                                                     bf16_t* __restrict__ hidden, long long chunks) {
+  for (long long item = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; item < chunks;
+       item += static_cast<long long>(gridDim.x) * blockDim.x) {
+    const Bf16x8 g = reinterpret_cast<const Bf16x8*>(gate)[item];
+    const Bf16x8 u = reinterpret_cast<const Bf16x8*>(up)[item];
+    Bf16x8 h;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) h.v[i] = swiglu_one(bf16_to_f32(g.v[i]), bf16_to_f32(u.v[i]));
+    reinterpret_cast<Bf16x8*>(hidden)[item] = h;
+  }
+}
+
+}  // namespace dew
+
+extern "C" int dew_moe_combine(const void* slots, const float* weights, const void* addend, void* out,
+                               int32_t tokens, int32_t top_k, int32_t width, void* stream) {
+  using namespace dew;
+  DEW_REQUIRE(tokens >= 0 && top_k >= 1 && width >= 8, "dew_moe_combine: tokens %d top_k %d width %d", tokens, top_k,
+              width);
+  DEW_REQUIRE(width % 8 == 0, "dew_moe_combine: width %d is not a multiple of 8 (16-byte rows)", width);
+  if (tokens == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(slots && weights && out, "dew_moe_combine: slots, weights and out must not be null");
+  DEW_REQUIRE(aligned16(slots) && aligned16(out) && aligned16(addend), "dew_moe_combine: buffers must be 16-byte aligned");
+  const long long total = static_cast<long long>(tokens) * (width / 8);
+  const int blocks = static_cast<int>(min((total + 255) / 256, 256ll * 64));
+  hipLaunchKernelGGL(combine_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const bf16_t*>(slots), weights, static_cast<const bf16_t*>(addend),
+                     static_cast<bf16_t*>(out), tokens, top_k, width);
+  return launched("combine_kernel");
+}
+
+extern "C" int dew_moe_swiglu(const void* gate, const void* up, void* hidden, int64_t count, void* stream) {
+  using namespace dew;
+  DEW_REQUIRE(count >= 0 && count % 8 == 0, "dew_moe_swiglu: count %lld is not a multiple of 8", static_cast<long long>(count));
+  if (count == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(gate && up && hidden, "dew_moe_swiglu: gate, up and hidden must not be null");
+  DEW_REQUIRE(aligned16(gate) && aligned16(up) && aligned16(hidden), "dew_moe_swiglu: buffers must be 16-byte aligned");
+  const long long chunks = count / 8;
+  const int blocks = static_cast<int>(min((chunks + 255) / 256, 256ll * 64));
+  hipLaunchKernelGGL(swiglu_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const bf16_t*>(gate), static_cast<const bf16_t*>(up), static_cast<bf16_t*>(hidden),
+                     chunks);
+  return launched("swiglu_kernel");
+}

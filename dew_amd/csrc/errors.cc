@@ -1,0 +1,62 @@
+// Error string plumbing and introspection strings.
+#include <stdarg.h>
+#include <string.h>
+
+#include "common.h"
+
+namespace dew {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list args;
+  va_start(args, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, args);
+  va_end(args);
+}
+
+int fail(int code, const char* fmt, ...) {
+  va_list args;
+  va_start(args, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, args);
+  va_end(args);
+  return code;
+}
+
+int launched(const char* kernel) {
+  hipError_t status = hipGetLastError();
+  if (status == hipSuccess) return DEW_MOE_OK;
+  return fail(DEW_MOE_ELAUNCH, "%s: %s", kernel, hipGetErrorString(status));
+}
+
+}  // namespace dew
+
+extern "C" {
+
+const char* dew_moe_last_error(void) { return dew::g_error; }
+
+const char* dew_moe_architecture(void) { return "gfx950"; }
+
+const char* dew_moe_kernel_fields(void) { return "name,tile_m,tile_n,tile_k,waves,mfma,operands"; }
+
+const char* dew_moe_kernels(void) {
+  return "route,1 token/wave,-,-,4,-,f32 logits\n"
+         "permute_count|permute_scan|permute_scatter,2048 slots/block,-,-,4,-,i32 ballot+LDS histogram\n"
+         "grouped_gemm,128,128,64,4,v_mfma_f32_32x32x16_bf16,bf16 x {fp8 block|fp8 channel|nvfp4} dequantized in registers\n"
+         "gateup_swiglu,128,2x128,64,4,v_mfma_f32_32x32x16_bf16,paired gate/up + SwiGLU epilogue\n"
+         "combine,1 token/block,-,-,4,-,bf16 slots x f32 weights\n";
+}
+
+int dew_moe_device_check(void) {
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return dew::fail(DEW_MOE_EDEVICE, "no HIP device is current");
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, device) != hipSuccess)
+    return dew::fail(DEW_MOE_EDEVICE, "hipGetDeviceProperties failed for device %d", device);
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return dew::fail(DEW_MOE_EDEVICE, "device %d is %s; these kernels are built for gfx950 only", device,
+                     prop.gcnArchName);
+  return DEW_MOE_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,395 @@
+// Grouped GEMM over expert-sorted rows on the gfx950 matrix cores: bf16 activations times quantized expert
+// weights dequantized to bf16 in registers (exactly the values the reference's load produces), fp32
+// accumulation in v_mfma_f32_32x32x16_bf16, one rounding to bf16.
+//
+//   out[scatter[i], :] = bf16( sum_k x[gather[i], k] * W[e(i)][k, :] )       (expert_projection)
+//   hidden[i, :] = swiglu(x[gather[i]] @ Wg[e], x[gather[i]] @ Wu[e])        (paired gate/up + epilogue)
+//
+// Work decomposition: a 256-thread block (4 wavefronts, 2 x 2) owns a 128-row x 128-column tile of one
+// expert's group (two such tiles, gate and up, when paired) and walks the depth in 64-deep steps. Tiles are
+// enumerated on the device from `offsets` (no host read of the routing): block (x, y) takes m-tile x of
+// column strip y; experts with no rows own no tiles. Global loads of step t+1 are in flight while step t
+// multiplies out of LDS. LDS rows are 128 bytes (64 bf16) with the 16-byte chunk index xor-swizzled by
+// (row >> 1) & 7, which makes both the ds_write_b128 of the loaders and the ds_read_b128 of the MFMA
+// operand fetch conflict-free.
+#include "common.h"
+
+namespace dew {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;  // a 16-byte register quad (native vector: stays in VGPRs)
+
+constexpr int BM = 128, BN = 128, BK = 64;
+constexpr int kThreads = 256;
+constexpr int kChunksPerRow = BK / 8;  // 16-byte chunks in an LDS row
+
+struct BankView {
+  const uint8_t* codes;
+  const void* scales;
+  const float* tensor_scale;
+};
+
+struct GemmParams {
+  const bf16_t* x;
+  const int32_t* gather;
+  const int32_t* offsets;
+  const int32_t* scatter;
+  BankView w0, w1;
+  bf16_t* out;
+  int experts, depth, width, rows;
+};
+
+__device__ __forceinline__ int swizzled(int row, int chunk) { return row * kChunksPerRow + (chunk ^ ((row >> 1) & 7)); }
+
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  bf16x2_t pair = {static_cast<__bf16>(a), static_cast<__bf16>(b)};
+  return __builtin_bit_cast(uint32_t, pair);
+}
+
+// 16 e4m3 codes times one fp32 scale -> 16 bf16 (two LDS chunks): bf16(f32(code) * scale), the value the
+// reference's dequantize-then-cast produces (src/dew/interop/codecs.py:670-703; gemm.py:1067-1071).
+__device__ __forceinline__ void dequant_fp8(const u32x4_t& raw, float scale, u32x4_t (&out)[2]) {
+  const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+  uint32_t packed[8];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const f32x2_t lo = __builtin_amdgcn_cvt_pk_f32_fp8(words[q], false);
+    const f32x2_t hi = __builtin_amdgcn_cvt_pk_f32_fp8(words[q], true);
+    packed[2 * q] = pack_bf16(lo.x * scale, lo.y * scale);
+    packed[2 * q + 1] = pack_bf16(hi.x * scale, hi.y * scale);
+  }
+  out[0] = u32x4_t{packed[0], packed[1], packed[2], packed[3]};
+  out[1] = u32x4_t{packed[4], packed[5], packed[6], packed[7]};
+}
+
+// 32 E2M1 nibbles under two e4m3 block scales (each already over 2^8) -> 32 bf16 (four LDS chunks): each
+// product code * scale / 2^8 is exact in bf16 (src/dew/nn/kernels/formats.py:108-113).
+__device__ __forceinline__ void dequant_fp4(const u32x4_t& raw, float scale0, float scale1, u32x4_t (&out)[4]) {
+  const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+  uint32_t packed[16];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const float scale = q < 2 ? scale0 : scale1;
+    const f32x2_t b0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(words[q], 1.0f, 0);
+    const f32x2_t b1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(words[q], 1.0f, 1);
+    const f32x2_t b2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(words[q], 1.0f, 2);
+    const f32x2_t b3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(words[q], 1.0f, 3);
+    packed[4 * q] = pack_bf16(b0.x * scale, b0.y * scale);
+    packed[4 * q + 1] = pack_bf16(b1.x * scale, b1.y * scale);
+    packed[4 * q + 2] = pack_bf16(b2.x * scale, b2.y * scale);
+    packed[4 * q + 3] = pack_bf16(b3.x * scale, b3.y * scale);
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c) out[c] = u32x4_t{packed[4 * c], packed[4 * c + 1], packed[4 * c + 2], packed[4 * c + 3]};
+}
+
+// a = bf16(g * logistic(g)); h = bf16(a * u) on the bf16-rounded products (src/dew/nn/activations.py:267-278).
+__device__ __forceinline__ bf16_t swiglu_rounded(float gate_sum, float up_sum) {
+  const float g = bf16_round(gate_sum), u = bf16_round(up_sum);
+  const float sig = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf(-g)));
+  const float activated = bf16_round(__fmul_rn(g, sig));
+  return f32_to_bf16(__fmul_rn(activated, u));
+}
+
+template <int FORMAT, bool PAIRED>
+__global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
+  constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4;
+  constexpr int kMatrices = PAIRED ? 2 : 1;
+  constexpr int kAtomK = kFp4 ? 64 : 32;                       // depth an atom covers
+  constexpr int kAtomsPerStep = (BN / 32) * (BK / kAtomK);     // per matrix
+  constexpr int kLoads = kAtomsPerStep * kMatrices / 4;        // 16-byte loads a lane issues per step
+  constexpr int kChunksPerLoad = kFp4 ? 4 : 2;
+
+  __shared__ u32x4_t lds_a[BM * kChunksPerRow];
+  __shared__ u32x4_t lds_b[kMatrices * BN * kChunksPerRow];
+  __shared__ int wave_tiles[4];
+  __shared__ int found[3];  // expert, first sorted row of the tile, total m-tiles
+
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int m_tile = blockIdx.x, n0 = blockIdx.y * BN;
+
+  // ---- which expert owns m-tile `m_tile`? inclusive scan of ceil(size / BM) over the experts ----
+  if (tid == 0) found[0] = -1;
+  int carried = 0;
+  for (int base = 0; base < p.experts; base += kThreads) {
+    const int e = base + tid;
+    int start = 0, tiles = 0;
+    if (e < p.experts) {
+      start = p.offsets[e];
+      tiles = (p.offsets[e + 1] - start + BM - 1) / BM;
+    }
+    int inclusive = tiles;
+#pragma unroll
+    for (int offset = 1; offset < 64; offset <<= 1) {
+      const int other = __shfl_up(inclusive, offset, 64);
+      if (lane >= offset) inclusive += other;
+    }
+    __syncthreads();
+    if (lane == 63) wave_tiles[wave] = inclusive;
+    __syncthreads();
+    int before = carried;
+    for (int w = 0; w < wave; ++w) before += wave_tiles[w];
+    const int first = before + inclusive - tiles;
+    if (tiles > 0 && m_tile >= first && m_tile < first + tiles) {
+      found[0] = e;
+      found[1] = start + (m_tile - first) * BM;
+    }
+    carried += wave_tiles[0] + wave_tiles[1] + wave_tiles[2] + wave_tiles[3];
+  }
+  if (tid == 0) found[2] = carried;
+  __syncthreads();
+  const int expert = found[0];
+
+  if (expert < 0) {
+    // Past the last real tile: zero the rows no expert owns (sorted positions offsets[E] .. rows).
+    const int tail_begin = p.offsets[p.experts] + (m_tile - found[2]) * BM;
+    const int tail_end = min(tail_begin + BM, p.rows);
+    for (int item = tid; item < (tail_end - tail_begin) * (BN / 8); item += kThreads) {
+      const int sorted = tail_begin + item / (BN / 8);
+      const int row = p.scatter ? p.scatter[sorted] : sorted;
+      *reinterpret_cast<u32x4_t*>(p.out + static_cast<size_t>(row) * p.width + n0 + (item % (BN / 8)) * 8) = u32x4_t{0, 0, 0, 0};
+    }
+    return;
+  }
+
+  const int row0 = found[1];
+  const int valid_rows = min(BM, p.offsets[expert + 1] - row0);
+  const int steps = p.depth / BK;
+
+  // ---- A loader: 16-byte chunk `a_chunk` of rows a_row + 32 i ----
+  const int a_chunk = tid % kChunksPerRow, a_row = tid / kChunksPerRow;
+  const u32x4_t* a_src[BM / 32];
+#pragma unroll
+  for (int i = 0; i < BM / 32; ++i) {
+    const int sorted = row0 + min(a_row + 32 * i, valid_rows - 1);
+    const int source = p.gather ? p.gather[sorted] : sorted;
+    a_src[i] = reinterpret_cast<const u32x4_t*>(p.x + static_cast<size_t>(source) * p.depth) + a_chunk;
+  }
+
+  // ---- B loader: atom `wave + 4 j` of the step: (matrix, n-atom, k-atom) ----
+  const uint8_t* b_src[kLoads];
+  const uint16_t* b_scale_src[kLoads];
+  float b_scale[kLoads];
+  int b_row[kLoads], b_chunk[kLoads], b_matrix[kLoads];
+  const int n_atoms = p.width / 32, k_atoms = p.depth / kAtomK;
+#pragma unroll
+  for (int j = 0; j < kLoads; ++j) {
+    const int atom = wave + 4 * j;
+    const int matrix = atom / kAtomsPerStep;
+    const int within = atom % kAtomsPerStep;
+    const int na = within / (BK / kAtomK), ka = within % (BK / kAtomK);
+    const uint8_t* codes = matrix == 0 ? p.w0.codes : p.w1.codes;
+    const void* scales = matrix == 0 ? p.w0.scales : p.w1.scales;
+    const size_t first_atom = (static_cast<size_t>(expert) * n_atoms + n0 / 32 + na) * k_atoms + ka;
+    b_src[j] = codes + first_atom * kAtomBytes + lane * 16;
+    b_matrix[j] = matrix;
+    b_row[j] = na * 32 + lane % 32;
+    b_chunk[j] = ka * (kAtomK / 8) + (lane / 32) * kChunksPerLoad;
+    b_scale[j] = 1.0f;
+    b_scale_src[j] = nullptr;
+    if (kFp4) {
+      b_scale_src[j] = static_cast<const uint16_t*>(scales) + first_atom * 64 + lane;
+    } else if (FORMAT == DEW_MOE_W_FP8_CHANNEL) {
+      b_scale[j] = static_cast<const float*>(scales)[static_cast<size_t>(expert) * p.width + n0 + b_row[j]];
+    }
+  }
+
+  u32x4_t a_regs[BM / 32], b_regs[kLoads];
+  uint32_t s_regs[kLoads];
+  auto load_step = [&](int step) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < BM / 32; ++i) a_regs[i] = a_src[i][static_cast<size_t>(step) * kChunksPerRow];
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) {
+      b_regs[j] = *reinterpret_cast<const u32x4_t*>(b_src[j] + static_cast<size_t>(step) * (BK / kAtomK) * kAtomBytes);
+      if (kFp4) {
+        s_regs[j] = b_scale_src[j][static_cast<size_t>(step) * (BK / kAtomK) * 64];
+      } else if (FORMAT == DEW_MOE_W_FP8_BLOCK) {
+        const void* scales = b_matrix[j] == 0 ? p.w0.scales : p.w1.scales;
+        const int k_blocks = p.depth / 128, n_blocks = p.width / 128;
+        const size_t at = (static_cast<size_t>(expert) * k_blocks + (step * BK) / 128) * n_blocks + n0 / 128;
+        s_regs[j] = __float_as_uint(static_cast<const float*>(scales)[at]);
+      }
+    }
+  };
+
+  auto store_step = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < BM / 32; ++i) lds_a[swizzled(a_row + 32 * i, a_chunk)] = a_regs[i];
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) {
+      u32x4_t* dst = lds_b + b_matrix[j] * BN * kChunksPerRow;
+      if (kFp4) {
+        const float scale0 = __builtin_amdgcn_cvt_f32_fp8(s_regs[j], 0) * 0.00390625f;
+        const float scale1 = __builtin_amdgcn_cvt_f32_fp8(s_regs[j], 1) * 0.00390625f;
+        u32x4_t chunks[4];
+        dequant_fp4(b_regs[j], scale0, scale1, chunks);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) dst[swizzled(b_row[j], b_chunk[j] + c)] = chunks[c];
+      } else {
+        const float scale = FORMAT == DEW_MOE_W_FP8_BLOCK ? __uint_as_float(s_regs[j]) : b_scale[j];
+        u32x4_t chunks[2];
+        dequant_fp8(b_regs[j], scale, chunks);
+#pragma unroll
+        for (int c = 0; c < 2; ++c) dst[swizzled(b_row[j], b_chunk[j] + c)] = chunks[c];
+      }
+    }
+  };
+
+  // ---- accumulators: wave (wm, wn) owns rows wm*64.., columns wn*64.. as 2 x 2 MFMA tiles ----
+  const int wm0 = (wave / 2) * 64, wn0 = (wave % 2) * 64;
+  f32x16_t acc[kMatrices][2][2];
+#pragma unroll
+  for (int m = 0; m < kMatrices; ++m)
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int q = 0; q < 16; ++q) acc[m][i][j][q] = 0.0f;
+
+  load_step(0);
+  for (int step = 0; step < steps; ++step) {
+    store_step();
+    __syncthreads();
+    if (step + 1 < steps) load_step(step + 1);
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      const int chunk = 2 * kk + lane / 32;
+      bf16x8_t a_frag[2], b_frag[kMatrices][2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) a_frag[i] = __builtin_bit_cast(bf16x8_t, lds_a[swizzled(wm0 + 32 * i + lane % 32, chunk)]);
+#pragma unroll
+      for (int m = 0; m < kMatrices; ++m)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          b_frag[m][j] = __builtin_bit_cast(bf16x8_t, lds_b[m * BN * kChunksPerRow + swizzled(wn0 + 32 * j + lane % 32, chunk)]);
+#pragma unroll
+      for (int m = 0; m < kMatrices; ++m)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            acc[m][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_frag[i], b_frag[m][j], acc[m][i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: acc[..][q] is row 8 (q / 4) + 4 (lane / 32) + q % 4, column lane % 32 of its 32 x 32 tile ----
+  float factor0 = 1.0f, factor1 = 1.0f;
+  if (kFp4) {  // the 2^8 the decode owes times the expert's tensor scale (src/dew/nn/kernels/gemm.py:660-662)
+    factor0 = 256.0f * p.w0.tensor_scale[expert];
+    if (PAIRED) factor1 = 256.0f * p.w1.tensor_scale[expert];
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      const int row = wm0 + 32 * i + 8 * (q / 4) + 4 * (lane / 32) + q % 4;
+      if (row >= valid_rows) continue;
+      const int sorted = row0 + row;
+      const int out_row = p.scatter ? p.scatter[sorted] : sorted;
+      bf16_t* dst = p.out + static_cast<size_t>(out_row) * p.width + n0 + wn0 + lane % 32;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if (PAIRED) {
+          dst[32 * j] = swiglu_rounded(acc[0][i][j][q] * factor0, acc[kMatrices - 1][i][j][q] * factor1);
+        } else {
+          dst[32 * j] = f32_to_bf16(acc[0][i][j][q] * factor0);
+        }
+      }
+    }
+  }
+}
+
+static int check_bank(const char* who, const dew_moe_bank* bank, const char* name) {
+  DEW_REQUIRE(bank, "%s: %s bank must not be null", who, name);
+  DEW_REQUIRE(bank->layout == DEW_MOE_LAYOUT_PREPARED, "%s: %s bank is in the reference layout; call dew_moe_prepare_bank once at load", who, name);
+  DEW_REQUIRE(bank->format == DEW_MOE_W_FP8_BLOCK || bank->format == DEW_MOE_W_FP8_CHANNEL || bank->format == DEW_MOE_W_NVFP4,
+              "%s: %s bank has unknown format %d", who, name, bank->format);
+  DEW_REQUIRE(bank->experts >= 1 && bank->experts <= 4096, "%s: %s bank has %d experts", who, name, bank->experts);
+  DEW_REQUIRE(bank->depth >= BK && bank->depth % 128 == 0, "%s: %s bank depth %d is not a multiple of 128", who, name, bank->depth);
+  DEW_REQUIRE(bank->width % BN == 0 && bank->width >= BN, "%s: %s bank width %d is not a multiple of %d", who, name, bank->width, BN);
+  DEW_REQUIRE(bank->codes && bank->scales, "%s: %s bank codes and scales must not be null", who, name);
+  DEW_REQUIRE(bank->format != DEW_MOE_W_NVFP4 || bank->tensor_scale, "%s: %s NVFP4 bank needs tensor scales", who, name);
+  DEW_REQUIRE(aligned16(bank->codes), "%s: %s bank codes must be 16-byte aligned", who, name);
+  return DEW_MOE_OK;
+}
+
+template <bool PAIRED>
+static int launch(const char* who, const GemmParams& p, int format, hipStream_t stream) {
+  // every expert may end in a partial tile, and the zeroed tail may add one more
+  const int m_tiles = (p.rows + BM - 1) / BM + p.experts + 1;
+  const dim3 grid(m_tiles, p.width / BN), block(kThreads);
+  switch (format) {
+    case DEW_MOE_W_FP8_BLOCK:
+      hipLaunchKernelGGL((grouped_gemm_kernel<DEW_MOE_W_FP8_BLOCK, PAIRED>), grid, block, 0, stream, p);
+      break;
+    case DEW_MOE_W_FP8_CHANNEL:
+      hipLaunchKernelGGL((grouped_gemm_kernel<DEW_MOE_W_FP8_CHANNEL, PAIRED>), grid, block, 0, stream, p);
+      break;
+    default:
+      hipLaunchKernelGGL((grouped_gemm_kernel<DEW_MOE_W_NVFP4, PAIRED>), grid, block, 0, stream, p);
+      break;
+  }
+  return launched(who);
+}
+
+}  // namespace dew
+
+extern "C" int dew_moe_grouped_gemm(const void* x, const int32_t* gather, const int32_t* offsets,
+                                    const dew_moe_bank* w, const int32_t* scatter, void* out, int32_t rows,
+                                    void* stream) {
+  using namespace dew;
+  const char* who = "dew_moe_grouped_gemm";
+  if (int rc = check_bank(who, w, "weight")) return rc;
+  DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
+  if (rows == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(x && offsets && out, "%s: x, offsets and out must not be null", who);
+  DEW_REQUIRE(aligned16(x) && aligned16(out), "%s: x and out must be 16-byte aligned", who);
+  GemmParams p{};
+  p.x = static_cast<const bf16_t*>(x);
+  p.gather = gather;
+  p.offsets = offsets;
+  p.scatter = scatter;
+  p.w0 = BankView{static_cast<const uint8_t*>(w->codes), w->scales, w->tensor_scale};
+  p.w1 = p.w0;
+  p.out = static_cast<bf16_t*>(out);
+  p.experts = w->experts;
+  p.depth = w->depth;
+  p.width = w->width;
+  p.rows = rows;
+  return launch<false>(who, p, w->format, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int dew_moe_gateup_swiglu(const void* x, const int32_t* gather, const int32_t* offsets,
+                                     const dew_moe_bank* gate, const dew_moe_bank* up, void* hidden, int32_t rows,
+                                     void* stream) {
+  using namespace dew;
+  const char* who = "dew_moe_gateup_swiglu";
+  if (int rc = check_bank(who, gate, "gate")) return rc;
+  if (int rc = check_bank(who, up, "up")) return rc;
+  DEW_REQUIRE(gate->format == up->format && gate->experts == up->experts && gate->depth == up->depth && gate->width == up->width,
+              "%s: gate [%d, %d, %d] format %d and up [%d, %d, %d] format %d differ", who, gate->experts, gate->depth,
+              gate->width, gate->format, up->experts, up->depth, up->width, up->format);
+  DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
+  if (rows == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(x && offsets && hidden, "%s: x, offsets and hidden must not be null", who);
+  DEW_REQUIRE(aligned16(x) && aligned16(hidden), "%s: x and hidden must be 16-byte aligned", who);
+  GemmParams p{};
+  p.x = static_cast<const bf16_t*>(x);
+  p.gather = gather;
+  p.offsets = offsets;
+  p.scatter = nullptr;
+  p.w0 = BankView{static_cast<const uint8_t*>(gate->codes), gate->scales, gate->tensor_scale};
+  p.w1 = BankView{static_cast<const uint8_t*>(up->codes), up->scales, up->tensor_scale};
+  p.out = static_cast<bf16_t*>(hidden);
+  p.experts = gate->experts;
+  p.depth = gate->depth;
+  p.width = gate->width;
+  p.rows = rows;
+  return launch<true>(who, p, gate->format, static_cast<hipStream_t>(stream));
+}

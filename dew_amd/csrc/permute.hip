@@ -1,0 +1,188 @@
+// Dispatch bookkeeping: the stable counting sort of routed slots by expert id
+// (reference src/dew/nn/moe.py:1101-1128 `_sorted_locally`: argsort(experts), bincount, order // k).
+//
+// Three stream-ordered launches, no global atomics, so the result is deterministic:
+//   count   each 2048-slot block builds an LDS histogram of its slots (one sub-histogram per wavefront)
+//   scan    one block turns the per-block counts into sizes, offsets and each block's base per expert
+//   scatter each wavefront ranks its 64 slots among themselves with ballots (match-any over the id's bits),
+//           adds the running count of earlier slots, and writes order[] / rows[]
+// Slots whose id is >= experts (a dropped slot's sentinel) sort last, in slot order, outside every group.
+#include "common.h"
+
+namespace dew {
+
+constexpr int kPermuteThreads = 256;
+constexpr int kPermuteWaves = kPermuteThreads / 64;
+constexpr int kSlotsPerBlock = 2048;
+constexpr int kSlotsPerWave = kSlotsPerBlock / kPermuteWaves;
+constexpr int kMaxExperts = 1024;  // buckets = experts + 1 (the sentinel's) <= 1025 handled by loops
+
+struct PermuteParams {
+  const int32_t* ids;  // [slots]
+  int32_t* sizes;      // [experts]
+  int32_t* offsets;    // [experts + 1]
+  int32_t* order;      // [slots]
+  int32_t* rows;       // [slots]
+  int32_t* counts;     // workspace [blocks][buckets]
+  int32_t* bases;      // workspace [blocks][buckets]
+  int slots, experts, top_k, blocks, buckets;
+};
+
+__device__ __forceinline__ int bucket_of(int id, int experts) {
+  return (id < 0 || id >= experts) ? experts : id;
+}
+
+__global__ __launch_bounds__(kPermuteThreads) void permute_count_kernel(PermuteParams p) {
+  extern __shared__ int32_t hist[];  // [buckets]
+  for (int b = threadIdx.x; b < p.buckets; b += kPermuteThreads) hist[b] = 0;
+  __syncthreads();
+  const int begin = blockIdx.x * kSlotsPerBlock;
+  const int end = min(begin + kSlotsPerBlock, p.slots);
+  for (int slot = begin + threadIdx.x; slot < end; slot += kPermuteThreads)
+    atomicAdd(&hist[bucket_of(p.ids[slot], p.experts)], 1);
+  __syncthreads();
+  for (int b = threadIdx.x; b < p.buckets; b += kPermuteThreads)
+    p.counts[static_cast<size_t>(blockIdx.x) * p.buckets + b] = hist[b];
+}
+
+// One block: totals per bucket, exclusive scan over buckets, then each block's base per bucket.
+__global__ __launch_bounds__(kPermuteThreads) void permute_scan_kernel(PermuteParams p) {
+  extern __shared__ int32_t totals[];  // [buckets + 1]
+  for (int b = threadIdx.x; b < p.buckets; b += kPermuteThreads) {
+    int sum = 0;
+    for (int blk = 0; blk < p.blocks; ++blk) sum += p.counts[static_cast<size_t>(blk) * p.buckets + b];
+    totals[b] = sum;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {  // buckets <= 1025: a serial scan is a few microseconds and exact
+    int running = 0;
+    for (int b = 0; b < p.buckets; ++b) {
+      const int size = totals[b];
+      totals[b] = running;
+      running += size;
+    }
+    totals[p.buckets] = running;
+  }
+  __syncthreads();
+  for (int b = threadIdx.x; b < p.buckets; b += kPermuteThreads) {
+    const int start = totals[b];
+    if (b < p.experts) {
+      p.sizes[b] = totals[b + 1] - start;
+      p.offsets[b] = start;
+    } else {
+      p.offsets[p.experts] = start;  // slots routed to a real expert
+    }
+    int running = start;
+    for (int blk = 0; blk < p.blocks; ++blk) {
+      const size_t at = static_cast<size_t>(blk) * p.buckets + b;
+      const int count = p.counts[at];
+      p.bases[at] = running;
+      running += count;
+    }
+  }
+}
+
+__global__ __launch_bounds__(kPermuteThreads) void permute_scatter_kernel(PermuteParams p) {
+  extern __shared__ int32_t running[];  // [kPermuteWaves][buckets]: next free position per wave and bucket
+  const int lane = threadIdx.x % 64;
+  const int wave = threadIdx.x / 64;
+  const int block_begin = blockIdx.x * kSlotsPerBlock;
+  // pass 1: each wave counts its own contiguous 512 slots
+  for (int i = threadIdx.x; i < kPermuteWaves * p.buckets; i += kPermuteThreads) running[i] = 0;
+  __syncthreads();
+  int32_t* mine = running + wave * p.buckets;
+  const int wave_begin = block_begin + wave * kSlotsPerWave;
+  for (int round = 0; round < kSlotsPerWave / 64; ++round) {
+    const int slot = wave_begin + round * 64 + lane;
+    if (slot < p.slots) atomicAdd(&mine[bucket_of(p.ids[slot], p.experts)], 1);
+  }
+  __syncthreads();
+  // turn the per-wave counts into each wave's first position: block base + earlier waves' counts
+  for (int b = threadIdx.x; b < p.buckets; b += kPermuteThreads) {
+    int next = p.bases[static_cast<size_t>(blockIdx.x) * p.buckets + b];
+    for (int w = 0; w < kPermuteWaves; ++w) {
+      const int count = running[w * p.buckets + b];
+      running[w * p.buckets + b] = next;
+      next += count;
+    }
+  }
+  __syncthreads();
+  // pass 2: rank within the round by ballots, then advance the wave's running positions
+  int bits = 1;
+  while ((1 << bits) < p.buckets) ++bits;
+  for (int round = 0; round < kSlotsPerWave / 64; ++round) {
+    const int slot = wave_begin + round * 64 + lane;
+    const bool valid = slot < p.slots;
+    const int bucket = valid ? bucket_of(p.ids[slot], p.experts) : p.buckets;  // invalid lanes match nobody real
+    unsigned long long same = __ballot(valid);
+    for (int bit = 0; bit < bits; ++bit) {
+      const bool set = (bucket >> bit) & 1;
+      const unsigned long long vote = __ballot(set);
+      same &= set ? vote : ~vote;
+    }
+    const unsigned long long below = same & ((1ull << lane) - 1ull);
+    const int rank = __popcll(below);
+    const int count = __popcll(same);
+    int position = 0;
+    if (valid) position = mine[bucket] + rank;
+    __syncthreads();
+    if (valid && rank == count - 1) mine[bucket] = position + 1;
+    __syncthreads();
+    if (valid) {
+      p.order[position] = slot;
+      p.rows[position] = slot / p.top_k;
+    }
+  }
+}
+
+}  // namespace dew
+
+extern "C" size_t dew_moe_permute_workspace_bytes(int32_t slots, int32_t experts) {
+  if (slots <= 0 || experts <= 0) return 256;
+  const size_t blocks = (static_cast<size_t>(slots) + dew::kSlotsPerBlock - 1) / dew::kSlotsPerBlock;
+  return 2 * blocks * (static_cast<size_t>(experts) + 1) * sizeof(int32_t) + 256;
+}
+
+extern "C" int dew_moe_permute(const int32_t* indices, int32_t tokens, int32_t top_k, int32_t experts,
+                               int32_t* sizes, int32_t* offsets, int32_t* order, int32_t* rows,
+                               void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace dew;
+  DEW_REQUIRE(tokens >= 0 && top_k >= 1, "dew_moe_permute: tokens %d top_k %d", tokens, top_k);
+  DEW_REQUIRE(experts >= 1 && experts <= kMaxExperts, "dew_moe_permute: experts %d (at most %d)", experts,
+              kMaxExperts);
+  DEW_REQUIRE(static_cast<int64_t>(tokens) * top_k < (1ll << 30), "dew_moe_permute: %d x %d slots overflow int32",
+              tokens, top_k);
+  DEW_REQUIRE(sizes && offsets, "dew_moe_permute: sizes and offsets must not be null");
+  const int slots = tokens * top_k;
+  DEW_REQUIRE(slots == 0 || (indices && order && rows), "dew_moe_permute: indices, order and rows must not be null");
+  DEW_REQUIRE(workspace && workspace_bytes >= dew_moe_permute_workspace_bytes(slots, experts),
+              "dew_moe_permute: workspace of %zu bytes, need %zu", workspace_bytes,
+              dew_moe_permute_workspace_bytes(slots, experts));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  PermuteParams p;
+  p.ids = indices;
+  p.sizes = sizes;
+  p.offsets = offsets;
+  p.order = order;
+  p.rows = rows;
+  p.slots = slots;
+  p.experts = experts;
+  p.top_k = top_k;
+  p.buckets = experts + 1;
+  p.blocks = (slots + kSlotsPerBlock - 1) / kSlotsPerBlock;
+  uintptr_t base = (reinterpret_cast<uintptr_t>(workspace) + 255) & ~static_cast<uintptr_t>(255);
+  p.counts = reinterpret_cast<int32_t*>(base);
+  p.bases = p.counts + static_cast<size_t>(p.blocks) * p.buckets;
+  if (p.blocks > 0) {
+    hipLaunchKernelGGL(permute_count_kernel, dim3(p.blocks), dim3(kPermuteThreads), sizeof(int32_t) * p.buckets, s, p);
+    if (int rc = launched("permute_count_kernel")) return rc;
+  }
+  hipLaunchKernelGGL(permute_scan_kernel, dim3(1), dim3(kPermuteThreads), sizeof(int32_t) * (p.buckets + 1), s, p);
+  if (int rc = launched("permute_scan_kernel")) return rc;
+  if (p.blocks > 0) {
+    hipLaunchKernelGGL(permute_scatter_kernel, dim3(p.blocks), dim3(kPermuteThreads),
+                       sizeof(int32_t) * kPermuteWaves * p.buckets, s, p);
+    if (int rc = launched("permute_scatter_kernel")) return rc;
+  }
+  return DEW_MOE_OK;
+}

@@ -1,0 +1,253 @@
+// Router: scores, (group-limited) selection, top-k and gate weights, one wavefront per token.
+// Follows Router.__call__ from the logits on (reference src/dew/nn/moe.py:466-565). Every floating-point
+// step is a fixed sequence of IEEE fp32/fp64 operations with contraction off, the same sequence the CPU
+// oracle runs, so the chosen experts agree bit for bit.
+#include "common.h"
+
+#pragma clang fp contract(off)
+
+namespace dew {
+
+constexpr int kWave = 64;
+constexpr int kMaxPerLane = 8;   // experts <= 512
+constexpr int kRouteWaves = 4;   // tokens per 256-thread block
+
+// e^x by Cody-Waite reduction and a degree-7 Taylor sum in Horner form, times 2^n in two exact steps
+// (the reference's portable exp, src/dew/nn/precision.py:470-488).
+__device__ __forceinline__ float exp_f32(float x) {
+  x = fminf(fmaxf(x, -104.0f), 90.0f);
+  const float n = rintf(x * 0x1.715476p+0f);
+  const float r = (x - n * 0x1.62e4p-1f) - n * 0x1.7f7d1cp-20f;
+  float p = 0x1.a01a02p-13f;               // 1/5040 ... 1/6 rounded to fp32
+  p = p * r + 0x1.6c16c2p-10f;
+  p = p * r + 0x1.111112p-7f;
+  p = p * r + 0x1.555556p-5f;
+  p = p * r + 0x1.555556p-3f;
+  p = p * r + 0.5f;
+  p = p * r + 1.0f;
+  p = p * r + 1.0f;
+  const int ni = static_cast<int>(n);
+  const int half = ni >> 1;  // floor(n / 2)
+  const float first = __uint_as_float(static_cast<uint32_t>(half + 127) << 23);
+  const float second = __uint_as_float(static_cast<uint32_t>(ni - half + 127) << 23);
+  return (p * first) * second;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int offset = 32; offset >= 1; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, kWave));
+  return v;
+}
+
+// Sum rounded once: fp64 partials per lane, then a butterfly; every lane ends with the same value.
+__device__ __forceinline__ float wave_sum_once(double v) {
+#pragma unroll
+  for (int offset = 32; offset >= 1; offset >>= 1) v = v + __shfl_xor(v, offset, kWave);
+  return static_cast<float>(v);
+}
+
+struct Best {
+  float value;
+  int index;
+};
+
+__device__ __forceinline__ bool better(float v, int i, const Best& than) {
+  return v > than.value || (v == than.value && i < than.index);
+}
+
+__device__ __forceinline__ Best wave_best(Best b) {
+#pragma unroll
+  for (int offset = 32; offset >= 1; offset >>= 1) {
+    const float v = __shfl_xor(b.value, offset, kWave);
+    const int i = __shfl_xor(b.index, offset, kWave);
+    if (better(v, i, b)) {
+      b.value = v;
+      b.index = i;
+    }
+  }
+  return b;
+}
+
+struct RouteParams {
+  const float* logits;
+  const float* bias;
+  float* weights;
+  int32_t* indices;
+  int tokens, experts, top_k, score_function, normalize, expert_groups, groups_per_token;
+  float scaling;
+};
+
+__global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p) {
+  extern __shared__ float shared[];  // [kRouteWaves][experts] selections, for the group scores
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  const int token_raw = blockIdx.x * kRouteWaves + wave;
+  const bool active = token_raw < p.tokens;
+  const int token = active ? token_raw : p.tokens - 1;
+  const float* row = p.logits + static_cast<size_t>(token) * p.experts;
+  const float ninf = -__builtin_inff();
+
+  float logit[kMaxPerLane], score[kMaxPerLane], select[kMaxPerLane];
+#pragma unroll
+  for (int i = 0; i < kMaxPerLane; ++i) {
+    const int e = lane + kWave * i;
+    logit[i] = e < p.experts ? row[e] : ninf;
+  }
+
+  float top = ninf, denom = 1.0f;
+  if (p.score_function == DEW_MOE_SCORE_SOFTMAX) {
+    float m = ninf;
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) m = fmaxf(m, logit[i]);
+    top = wave_max(m);
+    double partial = 0.0;
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) {
+      const int e = lane + kWave * i;
+      score[i] = e < p.experts ? exp_f32(logit[i] - top) : 0.0f;
+      partial = partial + static_cast<double>(score[i]);
+    }
+    denom = wave_sum_once(partial);
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) score[i] = score[i] / denom;
+  } else {
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) score[i] = 1.0f / (1.0f + exp_f32(-logit[i]));
+  }
+
+#pragma unroll
+  for (int i = 0; i < kMaxPerLane; ++i) {
+    const int e = lane + kWave * i;
+    float s = score[i];
+    if (p.bias != nullptr && e < p.experts) s = s + p.bias[e];
+    select[i] = e < p.experts ? s : ninf;
+  }
+
+  if (p.expert_groups > 1) {
+    float* mine = shared + wave * p.experts;
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) {
+      const int e = lane + kWave * i;
+      if (e < p.experts) mine[e] = select[i];
+    }
+    __syncthreads();
+    const int per_group = p.experts / p.expert_groups;
+    // lane g scores group g: the sum of its two best selections
+    float group_score = ninf;
+    if (lane < p.expert_groups) {
+      float first = ninf, second = ninf;
+      for (int j = 0; j < per_group; ++j) {
+        const float v = mine[lane * per_group + j];
+        if (v > first) {
+          second = first;
+          first = v;
+        } else if (v > second) {
+          second = v;
+        }
+      }
+      group_score = first + second;
+    }
+    unsigned long long kept = 0ull;
+    bool taken = false;
+    for (int round = 0; round < p.groups_per_token; ++round) {
+      Best b;
+      b.value = ninf;
+      b.index = 0x7fffffff;
+      if (lane < p.expert_groups && !taken) {
+        b.value = group_score;
+        b.index = lane;
+      }
+      b = wave_best(b);
+      kept |= 1ull << b.index;
+      if (b.index == lane) taken = true;
+    }
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) {
+      const int e = lane + kWave * i;
+      if (e < p.experts && !((kept >> (e / per_group)) & 1ull)) select[i] = ninf;
+    }
+  }
+
+  // top-k: k rounds of a wave-wide argmax, ties to the lower index
+  unsigned taken_mask = 0u;
+  int my_choice = 0;
+  for (int round = 0; round < p.top_k; ++round) {
+    Best b;
+    b.value = ninf;
+    b.index = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) {
+      const int e = lane + kWave * i;
+      if (e < p.experts && !((taken_mask >> i) & 1u) && better(select[i], e, b)) {
+        b.value = select[i];
+        b.index = e;
+      }
+    }
+    b = wave_best(b);
+    if ((b.index % kWave) == lane) taken_mask |= 1u << (b.index / kWave);
+    if (lane == round) my_choice = b.index;
+  }
+
+  // gate weights: lane j < k owns the j-th choice
+  const bool owner = lane < p.top_k;
+  const float chosen_logit = owner ? row[my_choice] : ninf;
+  float weight = 0.0f;
+  if (p.score_function == DEW_MOE_SCORE_SOFTMAX && p.normalize) {
+    const float m = wave_max(chosen_logit);
+    const float shifted = owner ? exp_f32(chosen_logit - m) : 0.0f;
+    const float total = wave_sum_once(static_cast<double>(shifted));
+    weight = shifted / total;
+  } else {
+    if (owner) {
+      weight = p.score_function == DEW_MOE_SCORE_SOFTMAX ? exp_f32(chosen_logit - top) / denom
+                                                         : 1.0f / (1.0f + exp_f32(-chosen_logit));
+    }
+    if (p.normalize) {
+      float total = __shfl(weight, 0, kWave);
+      for (int j = 1; j < p.top_k; ++j) total = total + __shfl(weight, j, kWave);
+      total = total + 1e-20f;
+      weight = weight / total;
+    }
+  }
+  weight = weight * p.scaling;
+  if (active && owner) {
+    p.weights[static_cast<size_t>(token) * p.top_k + lane] = weight;
+    p.indices[static_cast<size_t>(token) * p.top_k + lane] = my_choice;
+  }
+}
+
+}  // namespace dew
+
+extern "C" int dew_moe_route(const float* logits, const float* bias, int32_t tokens, int32_t experts,
+                             int32_t top_k, int32_t score_function, int32_t normalize, float scaling,
+                             int32_t expert_groups, int32_t groups_per_token, float* weights,
+                             int32_t* indices, void* stream) {
+  using namespace dew;
+  DEW_REQUIRE(logits && weights && indices, "dew_moe_route: logits, weights and indices must not be null");
+  DEW_REQUIRE(tokens >= 0 && experts >= 1, "dew_moe_route: tokens %d experts %d", tokens, experts);
+  DEW_REQUIRE(experts <= kWave * kMaxPerLane, "dew_moe_route: at most %d experts, got %d", kWave * kMaxPerLane,
+              experts);
+  DEW_REQUIRE(top_k >= 1 && top_k <= experts && top_k <= kWave, "dew_moe_route: top_k %d of %d experts (at most %d)",
+              top_k, experts, kWave);
+  DEW_REQUIRE(score_function == DEW_MOE_SCORE_SOFTMAX || score_function == DEW_MOE_SCORE_SIGMOID,
+              "dew_moe_route: score_function %d is neither softmax (0) nor sigmoid (1)", score_function);
+  DEW_REQUIRE(expert_groups >= 1 && expert_groups <= kWave && experts % expert_groups == 0,
+              "dew_moe_route: %d experts do not split into %d groups (at most %d)", experts, expert_groups, kWave);
+  if (expert_groups > 1) {
+    DEW_REQUIRE(groups_per_token >= 1 && groups_per_token <= expert_groups,
+                "dew_moe_route: groups_per_token %d of %d groups", groups_per_token, expert_groups);
+    DEW_REQUIRE(experts / expert_groups >= 2, "dew_moe_route: a group's score sums its two best experts, got %d a group",
+                experts / expert_groups);
+    DEW_REQUIRE(top_k <= groups_per_token * (experts / expert_groups),
+                "dew_moe_route: top_k %d exceeds the %d experts of the kept groups", top_k,
+                groups_per_token * (experts / expert_groups));
+  }
+  if (tokens == 0) return DEW_MOE_OK;
+  RouteParams p{logits, bias, weights, indices, tokens, experts, top_k, score_function, normalize ? 1 : 0,
+                expert_groups, groups_per_token, scaling};
+  const int blocks = (tokens + kRouteWaves - 1) / kRouteWaves;
+  const size_t shared = expert_groups > 1 ? sizeof(float) * kRouteWaves * experts : 0;
+  hipLaunchKernelGGL(route_kernel, dim3(blocks), dim3(kWave * kRouteWaves), shared,
+                     static_cast<hipStream_t>(stream), p);
+  return launched("route_kernel");
+}

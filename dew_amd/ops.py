@@ -1,0 +1,203 @@
+"""The kernels as functions of torch tensors: each checks what only the host can (devices, dtypes,
+contiguity), allocates its outputs with torch (device memory and streams are torch's here; the arithmetic is
+the library's) and calls the C ABI on torch's current stream. No function reads a device value on the host."""
+
+import dataclasses
+
+import torch
+
+from . import _lib, formats
+from ._lib import KernelError
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _device(tensor: torch.Tensor, name: str, dtype=None) -> torch.Tensor:
+    if not tensor.is_cuda:
+        raise KernelError(f"{name} must be on the GPU: the MoE kernels have no CPU path")
+    if dtype is not None and tensor.dtype != dtype:
+        raise KernelError(f"{name} must be {dtype}, got {tensor.dtype}")
+    if not tensor.is_contiguous():
+        raise KernelError(f"{name} must be contiguous")
+    return tensor
+
+
+def _ptr(tensor):
+    return None if tensor is None else tensor.data_ptr()
+
+
+def device_check() -> None:
+    """Refuse a device the kernels were not built for, by name."""
+    _lib.check(_lib.library().dew_moe_device_check(), "dew_moe_device_check")
+
+
+# ---- router -------------------------------------------------------------------------------------------
+
+
+def route(logits: torch.Tensor, top_k: int, *, score_function: str = "softmax", normalize_weights: bool = True,
+          bias: torch.Tensor | None = None, routed_scaling_factor: float = 1.0, expert_groups: int = 1,
+          groups_per_token: int = 1):
+    """(weights fp32 `[..., k]`, indices int32 `[..., k]`) of router `logits [..., E]` (fp32)."""
+    scores = {"softmax": _lib.SCORE_SOFTMAX, "sigmoid": _lib.SCORE_SIGMOID}
+    if score_function not in scores:
+        raise KernelError(f"score_function must be one of {list(scores)}, got {score_function!r}")
+    _device(logits, "logits", torch.float32)
+    if bias is not None:
+        _device(bias, "bias", torch.float32)
+        if bias.shape != logits.shape[-1:]:
+            raise KernelError(f"bias {tuple(bias.shape)} does not match {logits.shape[-1]} experts")
+    experts = logits.shape[-1]
+    tokens = logits.numel() // experts
+    weights = torch.empty((*logits.shape[:-1], top_k), dtype=torch.float32, device=logits.device)
+    indices = torch.empty((*logits.shape[:-1], top_k), dtype=torch.int32, device=logits.device)
+    _lib.check(_lib.library().dew_moe_route(
+        _ptr(logits), _ptr(bias), tokens, experts, top_k, scores[score_function], int(bool(normalize_weights)),
+        float(routed_scaling_factor), expert_groups, groups_per_token, _ptr(weights), _ptr(indices), _stream()),
+        "dew_moe_route")
+    return weights, indices
+
+
+# ---- dispatch -----------------------------------------------------------------------------------------
+
+
+@dataclasses.dataclass(frozen=True)
+class Plan:
+    """The sort of routed slots by expert: `order [R]` (slot of each sorted position), `rows [R]` (its
+    token), `sizes [E]`, `offsets [E + 1]`, all int32 on the device."""
+
+    order: torch.Tensor
+    rows: torch.Tensor
+    sizes: torch.Tensor
+    offsets: torch.Tensor
+
+
+def sort_by_expert(indices: torch.Tensor, num_experts: int) -> Plan:
+    _device(indices, "indices", torch.int32)
+    top_k = indices.shape[-1]
+    tokens = indices.numel() // top_k
+    slots = tokens * top_k
+    device = indices.device
+    lib = _lib.library()
+    workspace = torch.empty(lib.dew_moe_permute_workspace_bytes(slots, num_experts), dtype=torch.uint8, device=device)
+    sizes = torch.empty(num_experts, dtype=torch.int32, device=device)
+    offsets = torch.empty(num_experts + 1, dtype=torch.int32, device=device)
+    order = torch.empty(slots, dtype=torch.int32, device=device)
+    rows = torch.empty(slots, dtype=torch.int32, device=device)
+    _lib.check(lib.dew_moe_permute(_ptr(indices), tokens, top_k, num_experts, _ptr(sizes), _ptr(offsets), _ptr(order),
+                                   _ptr(rows), _ptr(workspace), workspace.numel(), _stream()), "dew_moe_permute")
+    return Plan(order, rows, sizes, offsets)
+
+
+# ---- banks ----------------------------------------------------------------------------------------------
+
+
+@dataclasses.dataclass(frozen=True)
+class PreparedBank:
+    """A bank re-laid for the matrix cores (`dew_moe_prepare_bank`); holds the buffers it points into."""
+
+    descriptor: _lib.Bank
+    shape: tuple
+    keep: tuple
+
+    @property
+    def experts(self):
+        return self.shape[0]
+
+
+def prepare(bank) -> PreparedBank:
+    """The one-time re-layout of a `formats.NvFp4`, `formats.Fp8Blocks` or `formats.Fp8Channels` bank."""
+    if isinstance(bank, PreparedBank):
+        return bank
+    if isinstance(bank, formats.NvFp4):
+        bank.checked()
+        fmt, codes, scales, tensor = _lib.W_NVFP4, bank.words, bank.scales, bank.scale
+        _device(codes, "NvFp4.words", torch.int32), _device(scales, "NvFp4.scales", torch.uint8)
+        _device(tensor, "NvFp4.scale", torch.float32)
+    elif isinstance(bank, formats.Fp8Blocks):
+        fmt, codes, scales, tensor = _lib.W_FP8_BLOCK, bank.codes, bank.scale_inv, None
+        _device(codes, "Fp8Blocks.codes", torch.uint8), _device(scales, "Fp8Blocks.scale_inv", torch.float32)
+    elif isinstance(bank, formats.Fp8Channels):
+        fmt, codes, scales, tensor = _lib.W_FP8_CHANNEL, bank.codes, bank.scales, None
+        _device(codes, "Fp8Channels.codes", torch.uint8), _device(scales, "Fp8Channels.scales", torch.float32)
+    else:
+        raise KernelError(f"no HIP kernel multiplies a {type(bank).__name__} bank")
+    experts, depth, width = bank.shape
+    lib = _lib.library()
+    reference = _lib.Bank(fmt, _lib.LAYOUT_REFERENCE, experts, depth, width, _ptr(codes), _ptr(scales), _ptr(tensor))
+    buffer = torch.empty(lib.dew_moe_prepared_bytes(fmt, experts, depth, width), dtype=torch.uint8, device=codes.device)
+    out = _lib.Bank()
+    _lib.check(lib.dew_moe_prepare_bank(reference, _ptr(buffer), out, _stream()), "dew_moe_prepare_bank")
+    return PreparedBank(out, (experts, depth, width), (buffer, scales, tensor))
+
+
+# ---- products -----------------------------------------------------------------------------------------
+
+
+def grouped_gemm(x: torch.Tensor, bank: PreparedBank, offsets: torch.Tensor, *, gather: torch.Tensor | None = None,
+                 scatter: torch.Tensor | None = None, rows: int | None = None) -> torch.Tensor:
+    """`out[scatter[i]] = x[gather[i]] @ W[expert of sorted position i]`, bf16 `[rows, N]`."""
+    _device(x, "x", torch.bfloat16), _device(offsets, "offsets", torch.int32)
+    experts, depth, width = bank.shape
+    if x.shape[-1] != depth:
+        raise KernelError(f"x rows are {x.shape[-1]} deep, the bank {depth}")
+    if offsets.numel() != experts + 1:
+        raise KernelError(f"offsets has {offsets.numel()} entries, the bank {experts} experts")
+    for name, index in (("gather", gather), ("scatter", scatter)):
+        if index is not None:
+            _device(index, name, torch.int32)
+    rows = (gather.numel() if gather is not None else x.shape[0]) if rows is None else rows
+    if gather is None and rows > x.shape[0]:
+        raise KernelError(f"{rows} rows asked of an x of {x.shape[0]}")
+    if (gather is not None and gather.numel() < rows) or (scatter is not None and scatter.numel() < rows):
+        raise KernelError("gather and scatter must cover every row")
+    out = torch.empty((rows, width), dtype=torch.bfloat16, device=x.device)
+    _lib.check(_lib.library().dew_moe_grouped_gemm(_ptr(x), _ptr(gather), _ptr(offsets), bank.descriptor, _ptr(scatter),
+                                                   _ptr(out), rows, _stream()), "dew_moe_grouped_gemm")
+    return out
+
+
+def gateup_swiglu(x: torch.Tensor, gate: PreparedBank, up: PreparedBank, offsets: torch.Tensor, *,
+                  gather: torch.Tensor | None = None, rows: int | None = None) -> torch.Tensor:
+    """`hidden[i] = swiglu(x[gather[i]] @ Wg[e], x[gather[i]] @ Wu[e])`, bf16 `[rows, F]`, one launch."""
+    _device(x, "x", torch.bfloat16), _device(offsets, "offsets", torch.int32)
+    experts, depth, width = gate.shape
+    if x.shape[-1] != depth:
+        raise KernelError(f"x rows are {x.shape[-1]} deep, the banks {depth}")
+    if offsets.numel() != experts + 1:
+        raise KernelError(f"offsets has {offsets.numel()} entries, the banks {experts} experts")
+    if gather is not None:
+        _device(gather, "gather", torch.int32)
+    rows = (gather.numel() if gather is not None else x.shape[0]) if rows is None else rows
+    if gather is None and rows > x.shape[0]:
+        raise KernelError(f"{rows} rows asked of an x of {x.shape[0]}")
+    hidden = torch.empty((rows, width), dtype=torch.bfloat16, device=x.device)
+    _lib.check(_lib.library().dew_moe_gateup_swiglu(_ptr(x), _ptr(gather), _ptr(offsets), gate.descriptor, up.descriptor,
+                                                    _ptr(hidden), rows, _stream()), "dew_moe_gateup_swiglu")
+    return hidden
+
+
+def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    _device(gate, "gate", torch.bfloat16), _device(up, "up", torch.bfloat16)
+    if gate.shape != up.shape:
+        raise KernelError(f"gate {tuple(gate.shape)} and up {tuple(up.shape)} differ")
+    hidden = torch.empty_like(gate)
+    _lib.check(_lib.library().dew_moe_swiglu(_ptr(gate), _ptr(up), _ptr(hidden), gate.numel(), _stream()), "dew_moe_swiglu")
+    return hidden
+
+
+def combine(slots: torch.Tensor, weights: torch.Tensor, addend: torch.Tensor | None = None) -> torch.Tensor:
+    """`out[t] = bf16(sum_j f32(slots[t, j]) * weights[t, j])` (+ the shared expert's `addend`)."""
+    _device(slots, "slots", torch.bfloat16), _device(weights, "weights", torch.float32)
+    tokens, top_k, width = slots.shape
+    if weights.shape != (tokens, top_k):
+        raise KernelError(f"routing {tuple(weights.shape)} does not describe slots {tuple(slots.shape)}")
+    if addend is not None:
+        _device(addend, "addend", torch.bfloat16)
+        if addend.shape != (tokens, width):
+            raise KernelError(f"addend {tuple(addend.shape)} is not [{tokens}, {width}]")
+    out = torch.empty((tokens, width), dtype=torch.bfloat16, device=slots.device)
+    _lib.check(_lib.library().dew_moe_combine(_ptr(slots), _ptr(weights), _ptr(addend), _ptr(out), tokens, top_k, width,
+                                              _stream()), "dew_moe_combine")
+    return out

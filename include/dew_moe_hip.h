@@ -1,0 +1,119 @@
+/* C ABI of libdew_moe_hip.so: the MI355X (gfx950) kernels of the quantized Mixture-of-Experts expert path.
+ *
+ * Plain pointers and sizes only: every pointer is DEVICE memory on the current HIP device unless said
+ * otherwise, `stream` is a hipStream_t passed as void*. No entry point allocates, frees or synchronizes:
+ * group bookkeeping is read on the device from `offsets`, so calls are stream-ordered and graph-safe, as
+ * the reference's CUTLASS FFI library is (kernels/cutlass/ffi.cu:1-6, groups.cuh:19-30). Every entry point
+ * returns 0 on success and a nonzero DEW_MOE_E* code otherwise; dew_moe_last_error() then names the refused
+ * argument, as the reference's `const char* why` does (kernels/cutlass/grouped.h:56-65, ffi.cu:93-95).
+ *
+ * Notation: T tokens, D model width, F expert hidden width, E experts, k choices a token, R = T*k routed
+ * slots. bf16 tensors are row-major uint16 bit patterns.
+ */
+#ifndef DEW_MOE_HIP_H
+#define DEW_MOE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  DEW_MOE_OK = 0,
+  DEW_MOE_EINVAL = 1,   /* a shape, alignment or null-pointer contract is not met            */
+  DEW_MOE_EDEVICE = 2,  /* the current device is not gfx950 (ffi.cu:102-106 refuses by name)  */
+  DEW_MOE_ELAUNCH = 3   /* hipGetLastError() after a launch                                   */
+};
+
+/* Weight formats (reference layouts; src/dew/nn/kernels/formats.py:27-47, src/dew/interop/codecs.py:670-703).
+ * K = depth (inputs), N = width (outputs) of each expert's matrix W[e] : [K, N].                       */
+enum {
+  DEW_MOE_W_FP8_BLOCK = 1,   /* codes u8 e4m3 [E,K,N]; scales f32 [E,ceil(K/128),ceil(N/128)]           */
+  DEW_MOE_W_FP8_CHANNEL = 2, /* codes u8 e4m3 [E,K,N]; scales f32 [E,N]                                 */
+  DEW_MOE_W_NVFP4 = 3        /* codes = NvFp4.words u32 [E,N,K/8] (staged order, GF(2)-encoded);        */
+                             /* scales = NvFp4.scales e4m3 bytes [E,N,K/16]; tensor_scale f32 [E].      */
+                             /* MXFP4 banks arrive in this form (codecs.mxfp4_as_nvfp4).                */
+};
+
+enum { DEW_MOE_LAYOUT_REFERENCE = 0, DEW_MOE_LAYOUT_PREPARED = 1 };
+
+typedef struct dew_moe_bank {
+  int32_t format;            /* DEW_MOE_W_*                                                             */
+  int32_t layout;            /* DEW_MOE_LAYOUT_*                                                        */
+  int32_t experts, depth, width;
+  const void* codes;
+  const void* scales;
+  const float* tensor_scale; /* NVFP4 only, else NULL                                                   */
+} dew_moe_bank;
+
+enum { DEW_MOE_SCORE_SOFTMAX = 0, DEW_MOE_SCORE_SIGMOID = 1 };
+
+/* ---- introspection (kernels/cutlass/ffi.cu:133-176: dew_cutlass_kernels/kernel_fields/architecture) ---- */
+const char* dew_moe_last_error(void);   /* thread-local, valid until the thread's next failing call      */
+const char* dew_moe_architecture(void); /* "gfx950"                                                      */
+const char* dew_moe_kernels(void);      /* one line per kernel: name, tile, waves, MFMA instruction      */
+const char* dew_moe_kernel_fields(void);
+int dew_moe_device_check(void);         /* DEW_MOE_OK iff the current device is gfx950                    */
+
+/* ---- Router (src/dew/nn/moe.py:466-565, from the logits on) ----------------------------------------
+ * scores = softmax | sigmoid of logits[T,E]; selection = scores (+ bias[E]); with expert_groups > 1 only the
+ * experts of the groups_per_token best groups (a group's score = sum of its two best selections) stay,
+ * the rest -inf; indices = the k largest selections in descending order, ties to the lower index;
+ * weights = softmax of the chosen logits (softmax and normalize), else the chosen scores, divided by
+ * (their sum + 1e-20) when normalize; times `scaling`. Bit-exact with the CPU oracle.                   */
+int dew_moe_route(const float* logits, const float* bias /* nullable */, int32_t tokens, int32_t experts,
+                  int32_t top_k, int32_t score_function, int32_t normalize, float scaling,
+                  int32_t expert_groups, int32_t groups_per_token, float* weights /* [T,k] */,
+                  int32_t* indices /* [T,k] */, void* stream);
+
+/* ---- Dispatch bookkeeping (src/dew/nn/moe.py:1101-1128 `_sorted_locally`) --------------------------
+ * Stable counting sort of the R = tokens*top_k flattened expert ids: sizes[E] = bincount,
+ * offsets[E+1] = exclusive prefix (offsets[E] = number of slots whose id is < E), order[R] = argsort
+ * (slot index of each sorted position; ids >= E sort last in slot order), rows[R] = order / top_k.       */
+size_t dew_moe_permute_workspace_bytes(int32_t slots, int32_t experts);
+int dew_moe_permute(const int32_t* indices /* [T,k] */, int32_t tokens, int32_t top_k, int32_t experts,
+                    int32_t* sizes, int32_t* offsets, int32_t* order, int32_t* rows, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
+/* ---- One-time weight re-layout -----------------------------------------------------------------------
+ * The GEMM kernels read a bank re-laid into MFMA-fragment order (exact: a permutation of the codes; the
+ * NVFP4 word encoder is an invertible GF(2) map, src/dew/algebra/bits.py:208-223,240-250). Call once per
+ * bank at load; `prepared` must hold dew_moe_prepared_bytes() bytes, 256-byte aligned. `out` describes
+ * the prepared bank and is what the GEMM entry points take.                                             */
+size_t dew_moe_prepared_bytes(int32_t format, int32_t experts, int32_t depth, int32_t width);
+int dew_moe_prepare_bank(const dew_moe_bank* reference, void* prepared, dew_moe_bank* out /* host */,
+                         void* stream);
+
+/* ---- Grouped products (src/dew/nn/moe.py:666-770 expert_projection / paired_projections; replaces the
+ *      launches of kernels/cutlass/ffi.cu:180-220 behind src/dew/nn/kernels/grouped_matmul.py:1826-1831) --
+ * Sorted position i in [offsets[e], offsets[e+1]) belongs to expert e and reads row gather[i] of x (row i
+ * when gather is NULL). out row = scatter[i] (i when NULL). Operands bf16, weights dequantized to bf16
+ * exactly as the reference's load does, fp32 accumulation, one rounding to bf16. Sorted positions in
+ * [offsets[E], rows) are written as zeros (kernels/cutlass/ffi.cu:117-123).                             */
+int dew_moe_grouped_gemm(const void* x /* bf16 [*,K] */, const int32_t* gather, const int32_t* offsets,
+                         const dew_moe_bank* w /* prepared, [E,K,N] */, const int32_t* scatter,
+                         void* out /* bf16 [rows,N] */, int32_t rows, void* stream);
+
+/* gate and up in one launch with the SwiGLU epilogue: hidden[i] = swiglu(x[gather[i]] @ Wg[e], .. @ Wu[e])
+ * with the reference's rounding sequence (src/dew/nn/activations.py:267-278): both products rounded to
+ * bf16, a = bf16(g * logistic(g)), hidden = bf16(a * u).                                                */
+int dew_moe_gateup_swiglu(const void* x, const int32_t* gather, const int32_t* offsets,
+                          const dew_moe_bank* gate, const dew_moe_bank* up, void* hidden /* bf16 [rows,F] */,
+                          int32_t rows, void* stream);
+
+/* The unfused epilogue alone (src/dew/nn/activations.py:336-356 gated_product('swiglu')).               */
+int dew_moe_swiglu(const void* gate, const void* up, void* hidden, int64_t count, void* stream);
+
+/* ---- Combine (src/dew/nn/moe.py:1328-1333 `_combine`, :1503 shared add) ----------------------------
+ * out[t,:] = bf16( sum_j f32(slots[t,j,:]) * weights[t,j] ), fp32 sum in slot order; with `addend`
+ * (the shared expert's output, bf16 [T,D]) out = bf16(f32(out) + f32(addend)).                          */
+int dew_moe_combine(const void* slots /* bf16 [T,k,D] */, const float* weights /* [T,k] */,
+                    const void* addend /* nullable */, void* out /* bf16 [T,D] */, int32_t tokens,
+                    int32_t top_k, int32_t width, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DEW_MOE_HIP_H */

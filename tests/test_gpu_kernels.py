@@ -1,0 +1,228 @@
+"""Parity of each HIP kernel, called through the C ABI, with the CPU oracle on the same seeded inputs.
+Integer outputs (indices, sizes, offsets, order, rows) and router weights must match bit for bit; products
+are compared with the tolerance stated beside each check."""
+
+import numpy as np
+import pytest
+import torch
+from moe_cases import CONFIGS, dequantized, inputs, quantize
+
+from oracle import moe_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from dew_amd import ops
+
+    ops.device_check()
+    return ops
+
+
+def dev(t):
+    return None if t is None else t.cuda()
+
+
+def bf16_np(t):
+    return t.float().cpu().numpy()
+
+
+ROUTERS = [
+    ("softmax-8-top2", 8, 2, dict(score_function="softmax", normalize_weights=True), False, 1000),
+    ("softmax-128-top8", 128, 8, dict(score_function="softmax", normalize_weights=True), False, 777),
+    ("softmax-128-top8-raw", 128, 8, dict(score_function="softmax", normalize_weights=False), False, 130),
+    ("softmax-5-top5", 5, 5, dict(score_function="softmax", normalize_weights=True), False, 9),
+    ("sigmoid-256-top8-groups", 256, 8, dict(score_function="sigmoid", normalize_weights=True, routed_scaling_factor=2.5,
+                                             expert_groups=8, groups_per_token=4), True, 1111),
+    ("sigmoid-64-top6-raw", 64, 6, dict(score_function="sigmoid", normalize_weights=False, routed_scaling_factor=1.5), True, 65),
+    ("softmax-320-top4-groups", 320, 4, dict(score_function="softmax", normalize_weights=True, expert_groups=5,
+                                             groups_per_token=2), False, 33),
+]
+
+
+@pytest.mark.parametrize("name,experts,k,settings,biased,tokens", ROUTERS, ids=[r[0] for r in ROUTERS])
+def test_router_matches_the_oracle_bit_for_bit(ops, name, experts, k, settings, biased, tokens):
+    import zlib
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    logits = (rng.standard_normal((tokens, experts)) * 2).astype(np.float32)
+    logits[0, :] = 0.25                                   # an all-ties row: the lower indices win
+    logits[1, : experts // 2] = logits[1, experts // 2: 2 * (experts // 2)]   # pairwise ties
+    bias = (rng.standard_normal(experts) * 0.1).astype(np.float32) if biased else None
+    want_w, want_i = oracle.route(logits, k, bias=bias, **settings)
+    got_w, got_i = ops.route(torch.from_numpy(logits).cuda(), k, bias=None if bias is None else torch.from_numpy(bias).cuda(),
+                             **settings)
+    assert np.array_equal(got_i.cpu().numpy(), want_i)
+    assert np.array_equal(got_w.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
+
+
+def test_router_reproduces_the_reference_fixtures_on_the_device(ops):
+    from conftest import golden
+    for name, settings in (("mixtral", dict(score_function="softmax", normalize_weights=True)),
+                           ("deepseek", dict(score_function="sigmoid", normalize_weights=True, routed_scaling_factor=2.5,
+                                             expert_groups=4, groups_per_token=2))):
+        held = golden(f"moe/{name}.npz")
+        hidden = held["hidden"].reshape(-1, 16)
+        logits = oracle.router_logits(hidden, held["mlp.gate.weight"].T)
+        bias = held.get("mlp.gate.e_score_correction_bias") if name == "deepseek" else None
+        k = held["router_indices"].shape[-1]
+        weights, indices = ops.route(torch.from_numpy(logits).cuda(), k,
+                                     bias=None if bias is None else torch.from_numpy(bias).cuda(), **settings)
+        order_theirs = np.argsort(held["router_indices"], -1, kind="stable")
+        order_ours = np.argsort(indices.cpu().numpy(), -1, kind="stable")
+        assert np.array_equal(np.take_along_axis(indices.cpu().numpy(), order_ours, -1),
+                              np.take_along_axis(held["router_indices"], order_theirs, -1))
+        assert np.abs(np.take_along_axis(weights.cpu().numpy(), order_ours, -1)
+                      - np.take_along_axis(held["router_weights"], order_theirs, -1)).max() < 1e-6
+
+
+@pytest.mark.parametrize("tokens,k,experts", [(1, 1, 1), (7, 2, 4), (64, 8, 128), (300, 3, 5), (2048, 2, 8),
+                                               (1025, 2, 8), (16384, 2, 8), (8192, 8, 256), (3000, 6, 512)])
+def test_permute_is_the_stable_sort_by_expert(ops, tokens, k, experts):
+    rng = np.random.default_rng(tokens * 31 + experts)
+    indices = rng.integers(0, experts, size=(tokens, k)).astype(np.int32)
+    if experts > 2:
+        indices[indices == 1] = 2                          # an empty expert
+    want = oracle.sorted_by_expert(indices, experts)
+    got = ops.sort_by_expert(torch.from_numpy(indices).cuda(), experts)
+    for field in ("sizes", "offsets", "order", "rows"):
+        assert np.array_equal(getattr(got, field).cpu().numpy(), want[field]), field
+
+
+def test_permute_sorts_dropped_slots_last_and_outside_every_group(ops):
+    indices = np.array([[0, 3], [3, 1], [2, 3], [0, 0]], np.int32)      # id 3 = the sentinel of 3 experts
+    got = ops.sort_by_expert(torch.from_numpy(indices).cuda(), 3)
+    assert got.sizes.tolist() == [3, 1, 1] and got.offsets.tolist() == [0, 3, 4, 5]
+    assert got.order.tolist() == [0, 6, 7, 3, 4, 1, 2, 5]
+
+
+def grouped_case(quant, experts, depth, width, sizes, seed):
+    rng = np.random.default_rng(seed)
+    weight = torch.from_numpy((rng.standard_normal((experts, depth, width)) * 0.02).astype(np.float32))
+    bank = quantize(weight, quant)
+    rows = int(np.sum(sizes))
+    x = torch.from_numpy(rng.standard_normal((rows, depth)).astype(np.float32)).to(torch.bfloat16)
+    offsets = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    return bank, x, offsets
+
+
+SIZES = [("ragged", [130, 0, 1, 257, 64, 0, 127, 5]), ("single", [3]), ("even", [128, 128, 128, 128])]
+
+
+@pytest.mark.parametrize("quant", ["fp8_channel", "fp8_block", "mxfp4", "nvfp4"])
+@pytest.mark.parametrize("label,sizes", SIZES, ids=[s[0] for s in SIZES])
+def test_grouped_gemm_matches_the_dequantized_fp32_sum(ops, quant, label, sizes):
+    """bf16 x decoded-weight products are exact in fp32, so kernel and oracle differ by summation order
+    alone before the one bf16 rounding: allow one bf16 ulp (2^-8 relative) plus an fp32-sum floor."""
+    bank, x, offsets = grouped_case(quant, len(sizes), 512, 256, sizes, seed=len(sizes) * 7 + len(quant))
+    values, factor = dequantized(bank)
+    want = oracle.grouped_matmul(bf16_np(x), values, sizes, factor=factor)
+    got = bf16_np(ops.grouped_gemm(x.cuda(), ops.prepare(bank.to("cuda")), torch.from_numpy(offsets).cuda()))
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= 2 ** -8 * scale
+    assert (np.abs(got - want) <= 2 ** -7 * np.abs(want) + 1e-5 * scale).all()
+    assert (got == want).mean() > 0.97                     # nearly every element rounds identically
+
+
+def test_grouped_gemm_is_exact_on_small_integers(ops):
+    """Known answer: integer rows times an MXFP4 bank of small powers of two sum exactly in fp32
+    (the reference's tests/test_gemm_nvfp4.py:41-52 states the same for its product)."""
+    rng = np.random.default_rng(11)
+    sizes = [40, 0, 100, 3]
+    weight = torch.from_numpy(rng.choice([-1.0, -0.5, 0.0, 0.5, 1.0, 2.0], size=(4, 256, 128)).astype(np.float32))
+    bank = quantize(weight, "mxfp4")
+    x = torch.from_numpy(rng.integers(-3, 4, size=(143, 256)).astype(np.float32)).to(torch.bfloat16)
+    offsets = torch.tensor(np.concatenate([[0], np.cumsum(sizes)]), dtype=torch.int32)
+    got = bf16_np(ops.grouped_gemm(x.cuda(), ops.prepare(bank.to("cuda")), offsets.cuda()))
+    want = np.zeros((143, 128))
+    start = 0
+    for e, size in enumerate(sizes):
+        want[start:start + size] = bf16_np(x)[start:start + size].astype(np.float64) @ weight[e].numpy().astype(np.float64)
+        start += size
+    assert np.array_equal(got.astype(np.float64), oracle.bf16_round(want.astype(np.float32)).astype(np.float64))
+
+
+def test_grouped_gemm_gathers_scatters_and_zeroes_unrouted_rows(ops):
+    rng = np.random.default_rng(5)
+    sizes = [70, 0, 130]
+    bank, _, offsets = grouped_case("fp8_block", 3, 256, 128, sizes, seed=3)
+    tokens = torch.from_numpy(rng.standard_normal((50, 256)).astype(np.float32)).to(torch.bfloat16)
+    rows = 210                                              # 10 sorted positions past sum(sizes)
+    gather = rng.integers(0, 50, size=rows).astype(np.int32)
+    scatter = rng.permutation(rows).astype(np.int32)
+    values, _ = dequantized(bank)
+    want_sorted = oracle.grouped_matmul(bf16_np(tokens)[gather], values, sizes)
+    want = np.zeros_like(want_sorted)
+    want[scatter] = want_sorted
+    got = bf16_np(ops.grouped_gemm(tokens.cuda(), ops.prepare(bank.to("cuda")), torch.from_numpy(offsets).cuda(),
+                                   gather=torch.from_numpy(gather).cuda(), scatter=torch.from_numpy(scatter).cuda(), rows=rows))
+    assert not got[scatter[200:]].any()
+    assert np.abs(got - want).max() <= 2 ** -8 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("quant", ["fp8_channel", "fp8_block", "mxfp4", "nvfp4"])
+def test_gateup_swiglu_matches_the_two_products_and_the_rounded_epilogue(ops, quant):
+    sizes = [100, 0, 37, 200]
+    rng = np.random.default_rng(21)
+    gate, x, offsets = grouped_case(quant, 4, 512, 256, sizes, seed=1)
+    up, _, _ = grouped_case(quant, 4, 512, 256, sizes, seed=2)
+    gather = rng.integers(0, x.shape[0], size=x.shape[0]).astype(np.int32)
+    gate_values, gate_factor = dequantized(gate)
+    up_values, up_factor = dequantized(up)
+    rows = bf16_np(x)[gather]
+    want_gate = oracle.grouped_matmul(rows, gate_values, sizes, factor=gate_factor)
+    want_up = oracle.grouped_matmul(rows, up_values, sizes, factor=up_factor)
+    want = oracle.swiglu(want_gate, want_up)
+    xd, od, gd = x.cuda(), torch.from_numpy(offsets).cuda(), torch.from_numpy(gather).cuda()
+    pg, pu = ops.prepare(gate.to("cuda")), ops.prepare(up.to("cuda"))
+    fused = bf16_np(ops.gateup_swiglu(xd, pg, pu, od, gather=gd))
+    apart = ops.swiglu(ops.grouped_gemm(xd, pg, od, gather=gd), ops.grouped_gemm(xd, pu, od, gather=gd))
+    assert np.array_equal(fused, bf16_np(apart))           # the fused epilogue is the unfused arithmetic
+    scale = np.abs(want).max()
+    # a one-ulp difference in gate or up moves the product by up to ~3 ulp of the result
+    assert np.abs(fused - want).max() <= 2 ** -6 * scale
+    assert (fused == want).mean() > 0.9
+
+
+def test_swiglu_kernel_matches_the_oracle_on_every_bf16_gate(ops):
+    gate_bits = np.arange(65536, dtype=np.uint16)
+    gate = oracle.bf16_from_bits(gate_bits)
+    keep = np.isfinite(gate)
+    gate = gate[keep]
+    gate = np.concatenate([gate, np.zeros(-gate.size % 8, np.float32)])
+    up = np.resize(np.array([1.0, -0.75, 3.140625, 1e-3, 100.0, 2 ** -20, -7.0, 0.5], np.float32), gate.shape)
+    want = oracle.swiglu(gate, up)
+    got = bf16_np(ops.swiglu(torch.from_numpy(gate).to(torch.bfloat16).cuda(), torch.from_numpy(up).to(torch.bfloat16).cuda()))
+    mismatched = (got != want) & ~(np.isnan(got) & np.isnan(want))
+    # exp differs in the last fp32 place between libraries; after two bf16 roundings that flips at most a
+    # handful of results by one ulp
+    assert mismatched.mean() < 2e-3
+    assert np.abs(got - want)[mismatched].max(initial=0) <= 2 ** -7 * np.abs(want)[mismatched].max(initial=1)
+
+
+def test_combine_weighs_in_fp32_and_rounds_once(ops):
+    slots = torch.tensor([[[1.0] * 8, [-1.0] * 8]], dtype=torch.bfloat16)     # tests/test_moe_precision.py:652-674
+    weights = torch.tensor([[0.5 + 2 ** -11, 0.5 - 2 ** -11]], dtype=torch.float32)
+    assert (ops.combine(slots.cuda(), weights.cuda()).float().cpu() == 2.0 ** -10).all()
+    rng = np.random.default_rng(8)
+    slots = torch.from_numpy(rng.standard_normal((333, 8, 512)).astype(np.float32)).to(torch.bfloat16)
+    weights = torch.from_numpy(rng.uniform(0, 1, size=(333, 8)).astype(np.float32))
+    addend = torch.from_numpy(rng.standard_normal((333, 512)).astype(np.float32)).to(torch.bfloat16)
+    want = oracle.combine(bf16_np(slots), weights.numpy())
+    assert np.array_equal(bf16_np(ops.combine(slots.cuda(), weights.cuda())), want)
+    with_shared = oracle.bf16_round(want + bf16_np(addend))
+    assert np.array_equal(bf16_np(ops.combine(slots.cuda(), weights.cuda(), addend.cuda())), with_shared)
+
+
+def test_entry_points_refuse_what_they_cannot_run(ops):
+    from dew_amd._lib import KernelError
+    with pytest.raises(KernelError, match="top_k"):
+        ops.route(torch.zeros((4, 8), device="cuda"), 9)
+    with pytest.raises(KernelError, match="multiple of 128"):
+        ops.prepare(quantize(torch.zeros((1, 128, 64)), "fp8_block").to("cuda"))
+    with pytest.raises(KernelError, match="GPU"):
+        ops.route(torch.zeros((4, 8)), 2)
+    bank = ops.prepare(quantize(torch.zeros((2, 128, 128)), "fp8_block").to("cuda"))
+    with pytest.raises(KernelError, match="deep"):
+        ops.grouped_gemm(torch.zeros((4, 256), dtype=torch.bfloat16, device="cuda"), bank,
+                         torch.zeros(3, dtype=torch.int32, device="cuda"))
