@@ -1,0 +1,239 @@
+"""Benchmark of the quantized MoE expert path on one MI355X.
+
+A step is one pass of the hot path over one batch of synthetic input already resident in HBM: route ->
+sort by expert -> gate/up grouped GEMM with the SwiGLU epilogue -> down grouped GEMM scattered to slot
+order -> weighted combine (+ shared expert where the config has one). Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--no-cpu-baseline]
+
+`value` is algorithmic TFLOP/s of the whole step: 6 * R * D * F (+ 6 * T * D * F_shared), the reference's
+own convention of three projections per dispatched row (src/dew/nn/moe.py:1275-1281), over the measured step
+time. `roofline` is the dominant kernel alone (the paired gate/up launch: two thirds of the FLOPs), timed
+with HIP events recorded on the launch stream around every one of its launches in the timed region.
+`cpu_baseline` is the CPU oracle on a bounded sample of the same workload, on this box's host cores.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+sys.path.insert(0, str(ROOT / "tests"))
+
+PEAKS = {"bf16_mfma": 2500.0, "fp8_mfma": 5000.0, "fp4_mfma": 10100.0, "hbm_gbs": 8000.0}
+"""MI355X published dense peaks, TFLOP/s and GB/s."""
+
+
+def build_workload(case, device, seed=0):
+    """Synthetic tensors of `case` on the device: bf16 activations ~N(0,1), fp32 router logits ~N(0,1) (+ a
+    per-expert bias), banks ~N(0,0.02) quantized on the device one expert matrix at a time."""
+    import torch
+    from moe_cases import quantize
+
+    from dew_amd import formats, gemm
+
+    generator = torch.Generator(device=device)
+    generator.manual_seed(seed)
+    x = torch.randn((case.tokens, case.d_model), generator=generator, device=device, dtype=torch.float32).to(torch.bfloat16)
+    logits = torch.randn((case.tokens, case.experts), generator=generator, device=device, dtype=torch.float32)
+    if case.logit_bias_std:
+        logits = logits + case.logit_bias_std * torch.randn(case.experts, generator=generator, device=device)
+    bias = None
+    if case.router.get("score_function") == "sigmoid":
+        bias = 0.05 * torch.randn(case.experts, generator=generator, device=device)
+
+    def bank(depth, width, experts):
+        parts = []
+        for _ in range(experts):
+            weight = 0.02 * torch.randn((1, depth, width), generator=generator, device=device, dtype=torch.float32)
+            parts.append(quantize(weight, case.quant))
+        first = parts[0]
+        if isinstance(first, formats.NvFp4):
+            held = formats.NvFp4(torch.cat([p.words for p in parts]), torch.cat([p.scales for p in parts]),
+                                 torch.cat([p.scale for p in parts]))
+        elif isinstance(first, formats.Fp8Blocks):
+            held = formats.Fp8Blocks(torch.cat([p.codes for p in parts]), torch.cat([p.scale_inv for p in parts]))
+        else:
+            held = formats.Fp8Channels(torch.cat([p.codes for p in parts]), torch.cat([p.scales for p in parts]))
+        gemm.prepared(held)      # the one-time re-layout, outside the timed region (done at load)
+        return held
+
+    banks = {"gate": bank(case.d_model, case.d_ff, case.experts), "up": bank(case.d_model, case.d_ff, case.experts),
+             "down": bank(case.d_ff, case.d_model, case.experts)}
+    shared = None
+    if case.shared:
+        shared = {"gate": bank(case.d_model, case.d_ff, 1), "up": bank(case.d_model, case.d_ff, 1),
+                  "down": bank(case.d_ff, case.d_model, 1)}
+    torch.cuda.synchronize()
+    return dict(x=x, logits=logits.contiguous(), bias=bias, banks=banks, shared=shared)
+
+
+class Stepper:
+    """One step of the hot path, launch by launch, with optional HIP events around the gate/up launch."""
+
+    def __init__(self, case, data):
+        import torch
+
+        from dew_amd import gemm, ops
+
+        self.torch, self.ops, self.case, self.data = torch, ops, case, data
+        self.gate, self.up, self.down = (gemm.prepared(data["banks"][n]) for n in ("gate", "up", "down"))
+        self.shared = None if data["shared"] is None else tuple(gemm.prepared(data["shared"][n]) for n in ("gate", "up", "down"))
+        tokens = case.tokens
+        self.dense_offsets = torch.tensor([0, tokens], dtype=torch.int32, device=data["x"].device)
+        self.events = []
+
+    def __call__(self, timed: bool = False):
+        torch, ops, case, data = self.torch, self.ops, self.case, self.data
+        weights, indices = ops.route(data["logits"], case.top_k, bias=data["bias"], **case.router)
+        plan = ops.sort_by_expert(indices, case.experts)
+        if timed:
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+        hidden = ops.gateup_swiglu(data["x"], self.gate, self.up, plan.offsets, gather=plan.rows)
+        if timed:
+            stop.record()
+            self.events.append((start, stop))
+        slots = ops.grouped_gemm(hidden, self.down, plan.offsets, scatter=plan.order)
+        addend = None
+        if self.shared is not None:
+            shared_hidden = ops.gateup_swiglu(data["x"], self.shared[0], self.shared[1], self.dense_offsets)
+            addend = ops.grouped_gemm(shared_hidden, self.shared[2], self.dense_offsets)
+        return ops.combine(slots.view(case.tokens, case.top_k, case.d_model), weights, addend), plan
+
+    def gateup_ms(self):
+        return sum(start.elapsed_time(stop) for start, stop in self.events) / max(1, len(self.events))
+
+
+def cpu_baseline(case, data, out, plan, budget_rows=192):
+    """The CPU oracle (dequantize -> bf16-exact fp32 GEMMs -> SwiGLU -> down) on a bounded sample: the
+    busiest expert's first `budget_rows` sorted rows, all three projections at full width. Also checks the
+    GPU's hidden-to-output path for those rows against it."""
+    import numpy as np
+    import torch
+    from moe_cases import dequantized
+
+    from dew_amd import formats
+    from oracle import moe_oracle as oracle
+
+    sizes = plan.sizes.cpu().numpy()
+    offsets = plan.offsets.cpu().numpy()
+    expert = int(sizes.argmax())
+    rows = int(min(budget_rows, sizes[expert]))
+    sorted_rows = plan.rows.cpu().numpy()[offsets[expert]:offsets[expert] + rows]
+    slots = plan.order.cpu().numpy()[offsets[expert]:offsets[expert] + rows]
+
+    def one(bank):
+        if isinstance(bank, formats.NvFp4):
+            return formats.NvFp4(bank.words[expert:expert + 1].cpu(), bank.scales[expert:expert + 1].cpu(), bank.scale[expert:expert + 1].cpu())
+        if isinstance(bank, formats.Fp8Blocks):
+            return formats.Fp8Blocks(bank.codes[expert:expert + 1].cpu(), bank.scale_inv[expert:expert + 1].cpu())
+        return formats.Fp8Channels(bank.codes[expert:expert + 1].cpu(), bank.scales[expert:expert + 1].cpu())
+
+    held = [one(data["banks"][n]) for n in ("gate", "up", "down")]
+    x = data["x"][torch.from_numpy(sorted_rows).to(data["x"].device).long()].float().cpu().numpy()
+    threads = os.cpu_count() or 1
+    began = time.perf_counter()
+    mats, factors = zip(*(dequantized(bank) for bank in held), strict=True)
+    dequant_s = time.perf_counter() - began
+    began = time.perf_counter()
+    gate = oracle.grouped_matmul(x, mats[0], [rows], factor=factors[0])
+    up = oracle.grouped_matmul(x, mats[1], [rows], factor=factors[1])
+    hidden = oracle.swiglu(gate, up)
+    down = oracle.grouped_matmul(hidden, mats[2], [rows], factor=factors[2])
+    gemm_s = time.perf_counter() - began
+    flops = 6.0 * rows * case.d_model * case.d_ff
+    return {"value": round(flops / (dequant_s + gemm_s) / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"{rows} sorted rows of expert {expert} (the busiest), 3 projections at full width: dequantize "
+                      f"{dequant_s:.2f} s + fp32 GEMMs/SwiGLU {gemm_s:.2f} s (NumPy/OpenBLAS on bf16-exact fp32 operands)",
+            "gemm_only_tflops": round(flops / gemm_s / 1e12, 5)}, (slots, down)
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=20)
+    parser.add_argument("--warmup", type=int, default=3)
+    parser.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    parser.add_argument("--no-cpu-baseline", action="store_true")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (expert-parallel sharding is described "
+                 "in DESIGN.md, not built). Run with --gpus 1.")
+
+    import numpy as np
+    import torch
+    from moe_cases import CONFIGS
+
+    from dew_amd import ops
+
+    ops.device_check()
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    case = CONFIGS[args.config]
+    data = build_workload(case, device)
+    stepper = Stepper(case, data)
+
+    for _ in range(args.warmup):
+        stepper()
+    torch.cuda.synchronize()
+    began = time.perf_counter()
+    for _ in range(args.steps):
+        out, plan = stepper(timed=True)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - began
+    ms_per_step = 1e3 * elapsed / args.steps
+
+    routed_rows = case.tokens * case.top_k
+    flops = 6.0 * routed_rows * case.d_model * case.d_ff + (6.0 * case.tokens * case.d_model * case.d_ff if case.shared else 0.0)
+    gateup_flops = 4.0 * routed_rows * case.d_model * case.d_ff
+    gateup_ms = stepper.gateup_ms()
+    achieved = gateup_flops / (gateup_ms * 1e-3) / 1e12
+    decode = args.config == "c3"
+    bytes_per_weight = 0.5 if case.quant in ("mxfp4", "nvfp4") else 1.0
+    touched = int((plan.sizes > 0).sum().item())
+    if decode:
+        # bandwidth view: the touched experts' gate and up codes read once + activations in, hidden out
+        gateup_bytes = touched * 2 * case.d_model * case.d_ff * bytes_per_weight + case.tokens * case.d_model * 2 + routed_rows * case.d_ff * 2
+        roofline = {"bound": "hbm", "achieved": round(gateup_bytes / (gateup_ms * 1e-3) / 1e9, 1), "peak": PEAKS["hbm_gbs"],
+                    "unit": "GB/s", "traffic": None}
+    else:
+        roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAKS["bf16_mfma"], "unit": "TFLOP/s", "traffic": None,
+                    "peak_note": "dense bf16 MFMA: the kernel multiplies bf16 activations by weights dequantized exactly to "
+                                 "bf16 (v_mfma_f32_32x32x16_bf16)",
+                    "frac_of_fp8_peak": round(achieved / PEAKS["fp8_mfma"], 4), "frac_of_fp4_peak": round(achieved / PEAKS["fp4_mfma"], 4)}
+    roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
+    roofline["kernel"] = "grouped_gemm_kernel<paired gate/up + SwiGLU>"
+    roofline["kernel_ms"] = round(gateup_ms, 4)
+
+    result = {
+        "metric": "grouped-GEMM TFLOP/s & % MFMA peak (prefill); HBM GB/s & % peak (decode)",
+        "value": round(flops / (ms_per_step * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{args.config}: T={case.tokens} D={case.d_model} F={case.d_ff} E={case.experts} k={case.top_k} "
+                               f"{case.quant} weights, {case.router['score_function']} router"
+                               + (" + shared expert" if case.shared else ""),
+                   "routed_rows": routed_rows, "experts_touched": touched,
+                   "algorithmic_flops": flops},
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        baseline, (slots, want) = cpu_baseline(case, data, out, plan)
+        result["cpu_baseline"] = baseline
+        # parity on the sample at full size: the device's down-projection rows for those slots
+        hidden = ops.gateup_swiglu(data["x"], stepper.gate, stepper.up, plan.offsets, gather=plan.rows)
+        projected = ops.grouped_gemm(hidden, stepper.down, plan.offsets, scatter=plan.order).float().cpu().numpy()
+        got = projected[slots]
+        scale = float(np.abs(want).max())
+        result["sample_parity"] = {"max_abs_over_max_ref": round(float(np.abs(got - want).max() / scale), 6),
+                                   "rows": int(len(slots))}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,115 @@
+"""The grouped-product front the MoE layer calls, shaped as the reference's GEMM template front
+(`gemm.gemm(lhs, rhs, group_sizes, *, paired, gather, scatter, epilogue, out_dtype, compute, ...)`,
+src/dew/nn/kernels/gemm.py:84-198), forward semantics only: every call is decided by the `GROUPED`
+selector (src/dew/nn/kernels/grouped_matmul.py:2206; selection.py) and runs the gfx950 HIP launch.
+
+A product's law (src/dew/nn/moe.py:675-677; docs/design/kernel-templates.md:876 of the reference): operands
+in the compute dtype (bf16), fp32 sums, one rounding; rows past `sum(group_sizes)` are zero; empty groups
+are allowed; an NVFP4 bank's deferred factor multiplies the sums before the rounding
+(src/dew/nn/kernels/gemm.py:655-662).
+"""
+
+import dataclasses
+
+import torch
+
+from . import formats, ops, selection
+from .selection import INHERENT, Kernel, Op, Requirement
+
+GROUPED_MATMUL = "grouped_matmul"
+"""The selector's choice name (`generation.Choice.GROUPED_MATMUL` in the reference)."""
+
+
+@dataclasses.dataclass(frozen=True)
+class GroupSizes:
+    """Group sizes `[E]` with their exclusive prefix `[E + 1]`, both int32 on the device: what the dispatch
+    sort produces, so no product recomputes the prefix. A plain int32 sizes tensor is accepted wherever this
+    is, at the price of one tiny prefix launch."""
+
+    sizes: torch.Tensor
+    offsets: torch.Tensor
+
+    @classmethod
+    def of(cls, group_sizes) -> "GroupSizes":
+        if isinstance(group_sizes, GroupSizes):
+            return group_sizes
+        sizes = group_sizes.to(torch.int32).contiguous()
+        return cls(sizes, ops.group_offsets(sizes))
+
+
+@dataclasses.dataclass(frozen=True)
+class GroupedCase:
+    """The facts of one grouped call the selector's requirements read."""
+
+    lhs: torch.Tensor
+    rhs: object
+    paired: object = None
+    epilogue: object = None
+    out_dtype: torch.dtype = torch.bfloat16
+    compute: torch.dtype = torch.bfloat16
+
+
+_BANKS = (formats.NvFp4, formats.Fp8Blocks, formats.Fp8Channels, ops.PreparedBank)
+
+
+def _shape(bank):
+    return bank.shape
+
+
+HIP = Kernel("hip", (
+    Requirement("device", lambda c: c.lhs.is_cuda, "the rows are not on the GPU; the HIP kernels have no CPU path"),
+    Requirement("quantized-bank", lambda c: isinstance(c.rhs, _BANKS) and (c.paired is None or isinstance(c.paired, _BANKS)),
+                lambda c: f"the matrices are {type(c.rhs).__name__}; the kernels multiply NvFp4, Fp8Blocks and "
+                          f"Fp8Channels banks", row="dense bf16 banks"),
+    Requirement("bf16", lambda c: c.lhs.dtype == torch.bfloat16 and c.compute == torch.bfloat16 and c.out_dtype == torch.bfloat16,
+                lambda c: f"rows {c.lhs.dtype}, compute {c.compute}, out {c.out_dtype}; the kernels compute and write bfloat16",
+                row="fp32 outputs"),
+    Requirement("depth", lambda c: _shape(c.rhs)[1] % 128 == 0 and c.lhs.shape[-1] == _shape(c.rhs)[1],
+                lambda c: f"depth {_shape(c.rhs)[1]} against rows {c.lhs.shape[-1]} deep; depths are whole 128s",
+                row="ragged depth"),
+    Requirement("width", lambda c: _shape(c.rhs)[2] % 128 == 0,
+                lambda c: f"width {_shape(c.rhs)[2]} is not a multiple of the 128-column tile", row="ragged width"),
+    Requirement("pair", lambda c: c.paired is None or (_shape(c.paired) == _shape(c.rhs) and type(c.paired) is type(c.rhs)),
+                "a paired product's matrices share one shape and format"),
+    Requirement("epilogue", lambda c: c.epilogue in (None, "swiglu") and (c.epilogue is None or c.paired is not None),
+                lambda c: f"epilogue {c.epilogue!r}; the kernels fuse 'swiglu' over a pair and nothing else",
+                row="bias and clamp epilogues"),
+))
+
+GROUPED = Op(GROUPED_MATMUL, (HIP,), preferred=lambda case: "hip",
+             foreign=("xla", "pallas", "mosaic", "triton", "cutlass"))
+"""The grouped product's selector. `chosen(grouped_matmul='hip')` names the HIP launch; the reference's other
+names are refused as unlowerable."""
+
+
+def prepared(bank) -> ops.PreparedBank:
+    """The bank's one-time device re-layout, cached on the bank object."""
+    if isinstance(bank, ops.PreparedBank):
+        return bank
+    held = getattr(bank, "_prepared", None)
+    if held is None:
+        held = ops.prepare(bank)
+        object.__setattr__(bank, "_prepared", held)
+    return held
+
+
+def gemm(lhs: torch.Tensor, rhs, group_sizes, *, paired=None, gather: torch.Tensor | None = None,
+         scatter: torch.Tensor | None = None, epilogue: str | None = None, out_dtype=torch.bfloat16,
+         compute=torch.bfloat16, implementation: str | None = None):
+    """Each group's rows of `lhs` (read at `gather` where given) times its matrix of the bank `rhs`, written
+    at `scatter` where given. With `paired`, a second bank multiplied by the same rows in the same launch:
+    returns both products, or, with `epilogue='swiglu'`, their gated product alone."""
+    case = GroupedCase(lhs, rhs, paired, epilogue, out_dtype, compute)
+    named = None if implementation in (None, "auto") else implementation
+    selection.select(GROUPED, case, named)
+    groups = GroupSizes.of(group_sizes)
+    first = prepared(rhs)
+    if paired is None:
+        return ops.grouped_gemm(lhs, first, groups.offsets, gather=gather, scatter=scatter)
+    second = prepared(paired)
+    if scatter is not None:
+        raise selection.KernelRefused(GROUPED_MATMUL, "hip", selection.Refusal("pair-scatter", "a paired product writes sorted rows"), iter(()))
+    if epilogue == "swiglu":
+        return ops.gateup_swiglu(lhs, first, second, groups.offsets, gather=gather)
+    return (ops.grouped_gemm(lhs, first, groups.offsets, gather=gather),
+            ops.grouped_gemm(lhs, second, groups.offsets, gather=gather))

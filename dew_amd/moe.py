@@ -1,0 +1,306 @@
+"""The sparse mixture-of-experts layer behind the reference's own names and signatures
+(src/dew/nn/moe.py): `Router`, `ExpertMLP`, `SparseMLP`, `expert_projection`, `paired_projections`,
+`Gathered`. Constructor fields, call signatures and the parameter tree paths are the reference's:
+
+    variables = {
+      'params': {'gate': {'kernel': fp32 [D, E]},
+                 'experts': {'gate_proj': {'kernel': bank}, 'up_proj': {...}, 'down_proj': {...}},
+                 'shared_experts': {'gate_proj': {'kernel': bank [1, D, F]}, ...}},
+      'moe': {'gate': {'e_score_correction_bias': fp32 [E]}},           # src/dew/nn/moe.py:445-451
+      'quantization': {'experts': {'gate_proj': {'kernel': bank}, ...}} # src/dew/quantization.py:483,555-561
+    }
+
+A quantized bank found in the 'quantization' collection takes the place of the parameter at the same path,
+as `quantization.expert_matrix` does. Modules are plain classes applied functionally:
+`SparseMLP(...).apply(variables, x)`. Every product runs the gfx950 HIP kernels through the C ABI; there is
+no other compute path here.
+"""
+
+import dataclasses
+from typing import NamedTuple
+
+import torch
+
+from . import gemm, ops, selection
+from .gemm import GroupSizes
+
+GROUPED_MATMULS = ("auto", "hip", "xla", "pallas")
+"""`implementation` names (src/dew/nn/moe.py:76): 'auto' and 'hip' run the HIP launches; the reference's
+'xla' and 'pallas' are known and refused as unlowerable on this host."""
+
+EXPERT_AXES = {"gate_proj": ("exp", "embed", "mlp"), "up_proj": ("exp", "embed", "mlp"),
+               "down_proj": ("exp", "mlp", "embed")}
+"""Logical axes of the three expert banks `[E, in, out]` (src/dew/nn/moe.py:1231-1235)."""
+
+WEIGHT_SUM_EPSILON = 1e-20
+"""src/dew/nn/moe.py:181; the router kernel adds this to a normalized weight sum."""
+
+
+class Gathered(NamedTuple):
+    """Expert-sorted rows read where they lie: row i is `tokens[rows[i]]`, landing at slot `slots[i]`
+    (src/dew/nn/moe.py:648-663)."""
+
+    tokens: torch.Tensor
+    rows: torch.Tensor
+    slots: torch.Tensor
+
+
+def _implementation(implementation: str) -> str | None:
+    if implementation not in GROUPED_MATMULS:
+        raise ValueError(f"implementation must be one of {list(GROUPED_MATMULS)}, got {implementation!r}")
+    return None if implementation == "auto" else implementation
+
+
+def expert_projection(x, kernel, group_sizes, dtype=None, implementation: str = "auto", precision=None,
+                      bias=None, scatter: torch.Tensor | None = None) -> torch.Tensor:
+    """The grouped matmul of `x`'s expert-sorted rows through each expert's matrix in `kernel`
+    (src/dew/nn/moe.py:666-726): operands bf16, fp32 sums, one rounding; `Gathered` rows are read where
+    they lie; with `scatter` each output row lands at its entry's row."""
+    if bias is not None:
+        raise selection.KernelRefused(gemm.GROUPED_MATMUL, "hip", selection.Refusal(
+            "bias", "a per-expert bias epilogue is not built"), iter(()))
+    tokens, rows = (x.tokens, x.rows) if isinstance(x, Gathered) else (x, None)
+    compute = torch.bfloat16 if dtype is None else dtype
+    return gemm.gemm(tokens, kernel, group_sizes, gather=rows, scatter=scatter, compute=compute, out_dtype=compute,
+                     implementation=_implementation(implementation))
+
+
+def paired_projections(x, first, second, group_sizes, dtype=None, implementation: str = "auto", precision=None):
+    """`expert_projection` of the same rows through a gate's and an up projection's banks as one paired
+    product (src/dew/nn/moe.py:745-770). Returns (gate, up)."""
+    tokens, rows = (x.tokens, x.rows) if isinstance(x, Gathered) else (x, None)
+    compute = torch.bfloat16 if dtype is None else dtype
+    return gemm.gemm(tokens, first, group_sizes, paired=second, gather=rows, compute=compute, out_dtype=compute,
+                     implementation=_implementation(implementation))
+
+
+def gated_projections(x, gate, up, group_sizes, dtype=None, implementation: str = "auto", precision=None) -> torch.Tensor:
+    """The paired product with the SwiGLU product as the launch's epilogue: `gated_product('swiglu')` of
+    `paired_projections`' outputs (src/dew/nn/moe.py:1319-1325) in one kernel, bit for bit the unfused
+    arithmetic (both sums round to bf16 first)."""
+    tokens, rows = (x.tokens, x.rows) if isinstance(x, Gathered) else (x, None)
+    compute = torch.bfloat16 if dtype is None else dtype
+    return gemm.gemm(tokens, gate, group_sizes, paired=up, gather=rows, epilogue="swiglu", compute=compute,
+                     out_dtype=compute, implementation=_implementation(implementation))
+
+
+def _at(tree, path):
+    for key in path:
+        if tree is None or key not in tree:
+            return None
+        tree = tree[key]
+    return tree
+
+
+def expert_matrix(variables: dict, path: tuple, name: str = "kernel"):
+    """The matrix a site multiplies: its bank in the 'quantization' collection where one is held, else its
+    parameter (src/dew/quantization.py:555-561)."""
+    held = _at(variables.get("quantization"), (*path, name))
+    if held is not None:
+        return held
+    found = _at(variables.get("params"), (*path, name))
+    if found is None:
+        raise KeyError(f"no {'/'.join(path)}/{name} in 'quantization' or 'params'")
+    return found
+
+
+class _Module:
+    path: tuple = ()
+
+    def apply(self, variables: dict, *args, **kwargs):
+        return self._bound(variables, ())(*args, **kwargs)
+
+    def _bound(self, variables, path):
+        bound = dataclasses.replace(self)
+        object.__setattr__(bound, "variables", variables)
+        object.__setattr__(bound, "path", tuple(path))
+        return bound
+
+
+@dataclasses.dataclass(frozen=True)
+class Router(_Module):
+    """The gate: logits, scores, (group-limited, bias-corrected) top-k choice and gate weights
+    (src/dew/nn/moe.py:316-565). Parameters: `kernel [in_features, num_experts]` fp32; with `expert_bias`
+    the selection bias at `moe/<path>/e_score_correction_bias`."""
+
+    num_experts: int
+    in_features: int
+    top_k: int
+    score_function: str = "softmax"
+    normalize_weights: bool = True
+    routed_scaling_factor: float = 1.0
+    expert_groups: int = 1
+    groups_per_token: int = 1
+    group_score: str = "top2"
+    expert_bias: bool = False
+
+    def __post_init__(self):
+        if self.score_function not in ("softmax", "sigmoid"):
+            raise ValueError(f"score_function {self.score_function!r}: the HIP router scores by 'softmax' or 'sigmoid'")
+        if self.group_score != "top2":
+            raise ValueError("the HIP router scores a group by its two best experts ('top2')")
+        if self.num_experts % self.expert_groups:
+            raise ValueError(f"{self.num_experts} experts do not split into {self.expert_groups} groups")
+
+    def logits(self, x: torch.Tensor) -> torch.Tensor:
+        """Each token's gate logit for every expert, fp32 (src/dew/nn/moe.py:526-534)."""
+        kernel = _at(self.variables["params"], (*self.path, "kernel"))
+        return ops.router_logits(x.reshape(-1, x.shape[-1]).contiguous(), kernel).reshape(*x.shape[:-1], self.num_experts)
+
+    def routed(self, logits: torch.Tensor):
+        """(weights, indices) from the logits on (src/dew/nn/moe.py:466-494)."""
+        bias = _at(self.variables.get("moe"), (*self.path, "e_score_correction_bias")) if self.expert_bias else None
+        if self.expert_bias and bias is None:
+            raise KeyError(f"no moe/{'/'.join(self.path)}/e_score_correction_bias")
+        return ops.route(logits, self.top_k, score_function=self.score_function,
+                         normalize_weights=self.normalize_weights, bias=bias,
+                         routed_scaling_factor=self.routed_scaling_factor, expert_groups=self.expert_groups,
+                         groups_per_token=self.groups_per_token)
+
+    def __call__(self, x, tokens=None, media=None, routes=None, blocks=None):
+        if tokens is not None or media is not None or routes is not None or blocks is not None:
+            raise ValueError("hash, media, replayed and block routing are not part of the HIP router")
+        return self.routed(self.logits(x))
+
+
+def _sorted_locally(indices: torch.Tensor, num_experts: int):
+    """`_sorted_locally`'s bookkeeping (src/dew/nn/moe.py:1101-1128): the stable sort of the slots by
+    expert. Returns (plan, group sizes with their offsets)."""
+    plan = ops.sort_by_expert(indices.reshape(-1, indices.shape[-1]), num_experts)
+    return plan, GroupSizes(plan.sizes, plan.offsets)
+
+
+@dataclasses.dataclass(frozen=True)
+class ExpertMLP(_Module):
+    """The routed experts of one layer (src/dew/nn/moe.py:1239-1353): sort the slots by expert, gate/up
+    products with SwiGLU, down product scattered to slot order, fp32-weighted combine. Banks at
+    `<path>/{gate_proj,up_proj,down_proj}/kernel`, `[E, in, out]`."""
+
+    num_experts: int
+    hidden_features: int
+    out_features: int
+    activation: str = "swiglu"
+    implementation: str = "auto"
+    dispatch: str = "auto"
+    capacity_factor: float | None = None
+    swiglu_limit: float | None = None
+    scale_inputs: bool = False
+    dtype: torch.dtype | None = None
+    precision: object = None
+    fused: bool = True
+    """Whether SwiGLU runs as the paired launch's epilogue (ours) or as its own kernel after the paired
+    product (the reference's arrangement); the results are bit-identical."""
+
+    def __post_init__(self):
+        if self.activation != "swiglu":
+            raise ValueError(f"activation {self.activation!r}: the HIP experts are SwiGLU experts")
+        if self.dispatch not in ("auto", "global"):
+            raise ValueError(f"dispatch {self.dispatch!r}: one device sorts its slots locally ('global')")
+        if self.capacity_factor is not None or self.swiglu_limit is not None or self.scale_inputs:
+            raise ValueError("capacity dropping, the SwiGLU clamp and input scaling are not part of the HIP experts")
+
+    def model_flops(self, rows: int) -> float:
+        """Three projections per dispatched row (src/dew/nn/moe.py:1275-1281)."""
+        return 3 * 2.0 * rows * self.out_features * self.hidden_features
+
+    def kernels(self):
+        return tuple(expert_matrix(self.variables, (*self.path, name)) for name in EXPERT_AXES)
+
+    def _project(self, tokens: Gathered, sizes: GroupSizes, kernels) -> torch.Tensor:
+        """src/dew/nn/moe.py:1305-1326."""
+        gate_w, up_w, down_w = kernels
+        if self.fused:
+            hidden = gated_projections(tokens, gate_w, up_w, sizes, self.dtype, self.implementation, self.precision)
+        else:
+            gate, up = paired_projections(tokens, gate_w, up_w, sizes, self.dtype, self.implementation, self.precision)
+            hidden = ops.swiglu(gate, up)
+        return expert_projection(hidden, down_w, sizes, self.dtype, self.implementation, self.precision,
+                                 scatter=tokens.slots)
+
+    def _combine(self, slots: torch.Tensor, weights: torch.Tensor, addend=None) -> torch.Tensor:
+        """src/dew/nn/moe.py:1328-1333."""
+        return ops.combine(slots, weights, addend)
+
+    def __call__(self, x: torch.Tensor, weights: torch.Tensor, indices: torch.Tensor, addend=None) -> torch.Tensor:
+        if weights.shape != indices.shape:
+            raise ValueError(f"routing {tuple(indices.shape)} does not describe weights {tuple(weights.shape)}")
+        tokens = x.reshape(-1, x.shape[-1]).contiguous()
+        top_k = indices.shape[-1]
+        plan, sizes = _sorted_locally(indices, self.num_experts)
+        projected = self._project(Gathered(tokens, plan.rows, plan.order), sizes, self.kernels())
+        slots = projected.reshape(tokens.shape[0], top_k, self.out_features)
+        out = self._combine(slots, weights.reshape(-1, top_k).contiguous(),
+                            None if addend is None else addend.reshape(-1, self.out_features))
+        return out.reshape(*x.shape[:-1], self.out_features)
+
+
+@dataclasses.dataclass(frozen=True)
+class GatedMLP(_Module):
+    """The dense SwiGLU MLP every token takes (the shared expert; src/dew/nn/mlp.py:106,239): the routed
+    kernels with one group holding every row. Banks `[1, in, out]` at `<path>/{gate,up,down}_proj/kernel`."""
+
+    hidden_features: int
+    out_features: int
+    implementation: str = "auto"
+
+    def __call__(self, x: torch.Tensor) -> torch.Tensor:
+        tokens = x.reshape(-1, x.shape[-1]).contiguous()
+        gate_w, up_w, down_w = (expert_matrix(self.variables, (*self.path, name)) for name in EXPERT_AXES)
+        sizes = GroupSizes(torch.tensor([tokens.shape[0]], dtype=torch.int32, device=x.device),
+                           torch.tensor([0, tokens.shape[0]], dtype=torch.int32, device=x.device))
+        hidden = gated_projections(tokens, gate_w, up_w, sizes, None, self.implementation)
+        return expert_projection(hidden, down_w, sizes, None, self.implementation).reshape(*x.shape[:-1], self.out_features)
+
+
+@dataclasses.dataclass(frozen=True)
+class SparseMLP(_Module):
+    """Router plus routed experts plus the optional shared expert (src/dew/nn/moe.py:1356-1503).
+    `shared` is the shared expert's hidden width (the reference passes a `GatedMLP` factory; its width is
+    what the factory fixes), None for no shared branch."""
+
+    num_experts: int
+    top_k: int
+    hidden_features: int
+    out_features: int
+    activation: str = "swiglu"
+    implementation: str = "auto"
+    dispatch: str = "auto"
+    score_function: str = "softmax"
+    normalize_weights: bool = True
+    routed_scaling_factor: float = 1.0
+    expert_groups: int = 1
+    groups_per_token: int = 1
+    group_score: str = "top2"
+    expert_bias: bool = False
+    shared: int | None = None
+    dtype: torch.dtype | None = None
+    fused: bool = True
+
+    @property
+    def gate(self) -> Router:
+        return Router(self.num_experts, self.out_features, self.top_k, self.score_function, self.normalize_weights,
+                      self.routed_scaling_factor, self.expert_groups, self.groups_per_token, self.group_score,
+                      self.expert_bias)._bound(self.variables, (*self.path, "gate"))
+
+    @property
+    def experts(self) -> ExpertMLP:
+        return ExpertMLP(self.num_experts, self.hidden_features, self.out_features, self.activation,
+                         self.implementation, self.dispatch, dtype=self.dtype,
+                         fused=self.fused)._bound(self.variables, (*self.path, "experts"))
+
+    @property
+    def shared_experts(self) -> GatedMLP:
+        return GatedMLP(self.shared, self.out_features, self.implementation)._bound(
+            self.variables, (*self.path, "shared_experts"))
+
+    def __call__(self, x, tokens=None, media=None, routes=None, blocks=None, *, logits: torch.Tensor | None = None):
+        """`logits`, where given, are the gate's (a benchmark's synthetic router logits); else the gate
+        kernel multiplies the tokens."""
+        gate = self.gate
+        if logits is None:
+            weights, indices = gate(x, tokens, media, routes, blocks)
+        else:
+            weights, indices = gate.routed(logits)
+        # routed + shared (src/dew/nn/moe.py:1497-1503): the bf16 add runs in the combine kernel's epilogue
+        shared = None if self.shared is None else self.shared_experts(x)
+        return self.experts(x, weights, indices, addend=shared)

@@ -59,6 +59,26 @@ def route(logits: torch.Tensor, top_k: int, *, score_function: str = "softmax", 
     return weights, indices
 
 
+def router_logits(x: torch.Tensor, kernel: torch.Tensor) -> torch.Tensor:
+    """fp32 gate logits `[..., E]` of bf16 tokens `[..., D]` and the fp32 gate kernel `[D, E]`."""
+    _device(x, "x", torch.bfloat16), _device(kernel, "kernel", torch.float32)
+    depth, experts = kernel.shape
+    if x.shape[-1] != depth:
+        raise KernelError(f"tokens are {x.shape[-1]} wide, the gate kernel {depth}")
+    logits = torch.empty((*x.shape[:-1], experts), dtype=torch.float32, device=x.device)
+    _lib.check(_lib.library().dew_moe_router_logits(_ptr(x), _ptr(kernel), _ptr(logits), x.numel() // depth, depth, experts,
+                                                    _stream()), "dew_moe_router_logits")
+    return logits
+
+
+def group_offsets(sizes: torch.Tensor) -> torch.Tensor:
+    """`[0, cumsum(sizes)]` int32 `[E + 1]`."""
+    _device(sizes, "group_sizes", torch.int32)
+    offsets = torch.empty(sizes.numel() + 1, dtype=torch.int32, device=sizes.device)
+    _lib.check(_lib.library().dew_moe_group_offsets(_ptr(sizes), sizes.numel(), _ptr(offsets), _stream()), "dew_moe_group_offsets")
+    return offsets
+
+
 # ---- dispatch -----------------------------------------------------------------------------------------
 
 

@@ -68,6 +68,11 @@ int dew_moe_route(const float* logits, const float* bias /* nullable */, int32_t
                   int32_t expert_groups, int32_t groups_per_token, float* weights /* [T,k] */,
                   int32_t* indices /* [T,k] */, void* stream);
 
+/* Gate logits (src/dew/nn/moe.py:526-534): logits[T,E] = f32(x[T,D] bf16) @ kernel[D,E] f32, IEEE fp32.      */
+int dew_moe_router_logits(const void* x /* bf16 [T,D] */, const float* kernel /* [D,E] */,
+                          float* logits /* [T,E] */, int32_t tokens, int32_t depth, int32_t experts,
+                          void* stream);
+
 /* ---- Dispatch bookkeeping (src/dew/nn/moe.py:1101-1128 `_sorted_locally`) --------------------------
  * Stable counting sort of the R = tokens*top_k flattened expert ids: sizes[E] = bincount,
  * offsets[E+1] = exclusive prefix (offsets[E] = number of slots whose id is < E), order[R] = argsort
@@ -76,6 +81,10 @@ size_t dew_moe_permute_workspace_bytes(int32_t slots, int32_t experts);
 int dew_moe_permute(const int32_t* indices /* [T,k] */, int32_t tokens, int32_t top_k, int32_t experts,
                     int32_t* sizes, int32_t* offsets, int32_t* order, int32_t* rows, void* workspace,
                     size_t workspace_bytes, void* stream);
+
+/* offsets[E+1] = exclusive prefix of group sizes[E] (implicit in jax.lax.ragged_dot's group_sizes,
+ * src/dew/nn/kernels/xla_products.py:86-115; explicit at src/dew/nn/moe.py:1172).                        */
+int dew_moe_group_offsets(const int32_t* sizes, int32_t experts, int32_t* offsets, void* stream);
 
 /* ---- One-time weight re-layout -----------------------------------------------------------------------
  * The GEMM kernels read a bank re-laid into MFMA-fragment order (exact: a permutation of the codes; the

@@ -1,0 +1,138 @@
+"""The whole layer (SparseMLP: route, sort, gate/up + SwiGLU, down, combine, shared expert) on the device,
+through the reference-shaped API, against the CPU oracle on the same seeded inputs.
+
+Bars: routing indices, group sizes/offsets and the permutation bit-exact; router weights bit-exact; outputs
+within max relative error 2e-2 (measured both as max|d| / max|ref| and element-wise as |d| / max(|ref|,
+rms(ref))). The bf16-exact kernels land near 2^-8, far inside the bar; the observed figures are printed."""
+
+import numpy as np
+import pytest
+import torch
+from moe_cases import CONFIGS, dequantized, inputs
+
+from oracle import moe_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+TOLERANCE = 2e-2
+
+CASES = {
+    "c1-full": CONFIGS["c1"],
+    "c2-reduced": CONFIGS["c2"].scaled(tokens=640, d_model=1024, d_ff=1792),
+    "c3-reduced": CONFIGS["c3"].scaled(d_model=1024, d_ff=384 + 128),
+    "c3-one-token": CONFIGS["c3"].scaled(tokens=1, d_model=512, d_ff=256, experts=16, top_k=4),
+    "c4-reduced": CONFIGS["c4"].scaled(tokens=384, d_model=1024, d_ff=512),
+    "c5-reduced": CONFIGS["c5"].scaled(tokens=300, d_model=1024, d_ff=1792),
+}
+
+
+def layer_and_variables(case, data):
+    from dew_amd import moe
+
+    router = dict(case.router)
+    layer = moe.SparseMLP(num_experts=case.experts, top_k=case.top_k, hidden_features=case.d_ff,
+                          out_features=case.d_model, expert_bias=data["bias"] is not None,
+                          shared=case.d_ff if case.shared else None, **router)
+    banks = {name: {"kernel": bank.to("cuda")} for name, bank in data["banks"].items()}
+    variables = {"params": {}, "quantization": {"experts": {f"{n}_proj": v for n, v in banks.items()}}}
+    if data["bias"] is not None:
+        variables["moe"] = {"gate": {"e_score_correction_bias": data["bias"].cuda()}}
+    if case.shared:
+        variables["quantization"]["shared_experts"] = {f"{n}_proj": {"kernel": b.to("cuda")} for n, b in data["shared"].items()}
+    return layer, variables
+
+
+def oracle_output(case, data):
+    mats, factors = zip(*(dequantized(data["banks"][name]) for name in ("gate", "up", "down")), strict=True)
+    shared = None
+    if case.shared:
+        shared = [dequantized(data["shared"][name])[0][0] for name in ("gate", "up", "down")]
+    return oracle.sparse_mlp(data["x"].float().numpy(), data["logits"].numpy(), *mats, top_k_count=case.top_k,
+                             shared=shared, factors=factors, bias=None if data["bias"] is None else data["bias"].numpy(),
+                             **case.router)
+
+
+@pytest.mark.parametrize("name", list(CASES))
+def test_layer_matches_the_oracle(name):
+    from dew_amd import ops
+
+    case = CASES[name]
+    data = inputs(case, seed=0)
+    layer, variables = layer_and_variables(case, data)
+    x, logits = data["x"].cuda(), data["logits"].cuda()
+    got = layer.apply(variables, x, logits=logits).float().cpu().numpy()
+    want, trace = oracle_output(case, data)
+
+    # routing: bit-exact
+    weights, indices = layer._bound(variables, ()).gate.routed(logits)
+    assert np.array_equal(indices.cpu().numpy(), trace["indices"])
+    assert np.array_equal(weights.cpu().numpy().view(np.uint32), trace["weights"].view(np.uint32))
+    plan = ops.sort_by_expert(indices, case.experts)
+    for field in ("order", "rows", "sizes", "offsets"):
+        assert np.array_equal(getattr(plan, field).cpu().numpy(), trace[field]), field
+
+    by_max, by_element = oracle.relative_errors(got, want)
+    print(f"\n{name}: max|d|/max|ref| = {by_max:.3e}, element-wise max rel = {by_element:.3e}, "
+          f"identical = {(got == want).mean():.4f}")
+    assert by_max <= TOLERANCE and by_element <= TOLERANCE
+
+    # the unfused arrangement (paired product, then the SwiGLU kernel) is the fused one bit for bit
+    import dataclasses
+    unfused = dataclasses.replace(layer, fused=False).apply(variables, x, logits=logits).float().cpu().numpy()
+    assert np.array_equal(unfused, got)
+
+
+def test_layer_multiplies_its_own_gate_kernel_when_no_logits_are_given():
+    from dew_amd import moe
+
+    case = CASES["c3-one-token"].scaled(tokens=37)
+    data = inputs(case, seed=3)
+    rng = np.random.default_rng(4)
+    kernel = torch.from_numpy((rng.standard_normal((case.d_model, case.experts)) * 0.05).astype(np.float32))
+    layer, variables = layer_and_variables(case, data)
+    variables["params"]["gate"] = {"kernel": kernel.cuda()}
+    x = data["x"].cuda()
+    logits = layer._bound(variables, ()).gate.logits(x).cpu().numpy()
+    want_logits = oracle.router_logits(data["x"].float().numpy(), kernel.numpy())
+    assert np.abs(logits - want_logits).max() <= 1e-5 * np.abs(want_logits).max()
+    got = layer.apply(variables, x)
+    again = layer.apply(variables, x, logits=torch.from_numpy(logits).cuda())
+    assert torch.equal(got, again)
+
+
+def test_idle_experts_change_nothing():
+    """Adding experts no token is routed to leaves the output unchanged (the reference's
+    tests/test_moe.py:356-368)."""
+    from dew_amd import formats, moe, ops
+
+    case = CASES["c3-one-token"].scaled(tokens=50, experts=4, top_k=2)
+    data = inputs(case, seed=5)
+    x, logits = data["x"].cuda(), data["logits"].cuda()
+    layer, variables = layer_and_variables(case, data)
+    got = layer.apply(variables, x, logits=logits)
+    wide = case.scaled(experts=8)
+
+    def widened(bank):
+        return formats.Fp8Blocks(torch.cat([bank.codes, torch.full_like(bank.codes, 0x55)]),
+                                 torch.cat([bank.scale_inv, bank.scale_inv]))
+
+    wide_data = dict(data, banks={n: widened(b) for n, b in data["banks"].items()})
+    wide_logits = torch.cat([logits, torch.full_like(logits, -1e4)], dim=-1)
+    wide_layer, wide_variables = layer_and_variables(wide, wide_data)
+    assert torch.equal(wide_layer.apply(wide_variables, x, logits=wide_logits), got)
+
+
+def test_a_named_kernel_that_cannot_run_is_refused_by_name():
+    from dew_amd import moe, selection
+
+    case = CASES["c3-one-token"]
+    data = inputs(case, seed=1)
+    layer, variables = layer_and_variables(case, data)
+    x, logits = data["x"].cuda(), data["logits"].cuda()
+    with selection.chosen(grouped_matmul="hip"):
+        layer.apply(variables, x, logits=logits)
+    assert any(route.kernel == "hip" and route.forced == "hip" for route in selection.routes())
+    with pytest.raises(selection.Unlowerable, match="xla"), selection.chosen(grouped_matmul="xla"):
+        layer.apply(variables, x, logits=logits)
+    with pytest.raises(selection.KernelRefused, match="bf16"), selection.chosen(grouped_matmul="hip"):
+        layer.apply(variables, x.float(), logits=logits)
