@@ -50,14 +50,6 @@ __global__ __launch_bounds__(256) void combine_kernel(const bf16_t* __restrict__
   }
 }
 
-// a = bf16(g * logistic(g)); h = bf16(a * u), on bf16 gate and up
-// (reference src/dew/nn/activations.py:267-278; logistic = 1 / (1 + e^-x) with a true division).
-__device__ __forceinline__ bf16_t swiglu_one(float g, float u) {
-  const float sig = 1.0f / (1.0f + expf(-g));
-  const float activated = bf16_round(g * sig);
-  return f32_to_bf16(activated * u);
-}
-
 __global__ __launch_bounds__(256) void swiglu_kernel(const bf16_t* __restrict__ gate, const bf16_t* __restrict__ up,
                                                      bf16_t* __restrict__ hidden, long long chunks) {
   for (long long item = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; item < chunks;
@@ -66,7 +58,7 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const bf16_t* __restrict__ 
     const Bf16x8 u = reinterpret_cast<const Bf16x8*>(up)[item];
     Bf16x8 h;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) h.v[i] = swiglu_one(bf16_to_f32(g.v[i]), bf16_to_f32(u.v[i]));
+    for (int i = 0; i < 8; ++i) h.v[i] = swiglu_rounded(bf16_to_f32(g.v[i]), bf16_to_f32(u.v[i]));
     reinterpret_cast<Bf16x8*>(hidden)[item] = h;
   }
 }

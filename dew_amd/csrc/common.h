@@ -36,6 +36,19 @@ __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
 
 __device__ __forceinline__ float bf16_round(float f) { return bf16_to_f32(f32_to_bf16(f)); }
 
+// SwiGLU on the fp32 sums of the gate and up products with the reference's roundings
+// (src/dew/nn/activations.py:267-278): g = bf16(gate), u = bf16(up), a = bf16(g * logistic(g)), h = bf16(a * u).
+// logistic(g) = 1 / (1 + e^-g) uses the hardware exp2 and reciprocal (each within 1 ulp of fp32): the
+// activation is rounded to 8 significant bits right after, so about one result in 2^12 differs by one bf16
+// ulp from a correctly rounded logistic, the same order as the spread between two libraries' expf.
+__device__ __forceinline__ bf16_t swiglu_rounded(float gate_sum, float up_sum) {
+  const float g = bf16_round(gate_sum), u = bf16_round(up_sum);
+  const float e = __builtin_amdgcn_exp2f(g * -1.44269504088896340736f);
+  const float sig = __builtin_amdgcn_rcpf(1.0f + e);
+  const float activated = bf16_round(g * sig);
+  return f32_to_bf16(activated * u);
+}
+
 // ---- prepared bank geometry (fragment-native atoms) ----
 // FP8 atom: 32 n x 32 k bytes = 1 KiB; lane l = (g = l / 32, n = l % 32) holds k = 16 g .. 16 g + 15.
 // FP4 atom: 32 n x 64 k nibbles = 1 KiB; lane l holds k = 32 g .. 32 g + 31 (byte j: low nibble k = 32 g + 2 j).

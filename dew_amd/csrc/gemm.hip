@@ -22,7 +22,7 @@ typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;  // a 16-byte register quad (native vector: stays in VGPRs)
 
-constexpr int BM = 128, BN = 128, BK = 64;
+constexpr int BK = 64;
 constexpr int kThreads = 256;
 constexpr int kChunksPerRow = BK / 8;  // 16-byte chunks in an LDS row
 
@@ -39,7 +39,7 @@ struct GemmParams {
   const int32_t* scatter;
   BankView w0, w1;
   bf16_t* out;
-  int experts, depth, width, rows;
+  int experts, depth, width, rows, m_tile_bound;
 };
 
 __device__ __forceinline__ int swizzled(int row, int chunk) { return row * kChunksPerRow + (chunk ^ ((row >> 1) & 7)); }
@@ -86,30 +86,56 @@ __device__ __forceinline__ void dequant_fp4(const u32x4_t& raw, float scale0, fl
   for (int c = 0; c < 4; ++c) out[c] = u32x4_t{packed[4 * c], packed[4 * c + 1], packed[4 * c + 2], packed[4 * c + 3]};
 }
 
-// a = bf16(g * logistic(g)); h = bf16(a * u) on the bf16-rounded products (src/dew/nn/activations.py:267-278).
-__device__ __forceinline__ bf16_t swiglu_rounded(float gate_sum, float up_sum) {
-  const float g = bf16_round(gate_sum), u = bf16_round(up_sum);
-  const float sig = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf(-g)));
-  const float activated = bf16_round(__fmul_rn(g, sig));
-  return f32_to_bf16(__fmul_rn(activated, u));
+// The same for a bank whose block scales are all powers of two (an MXFP4 checkpoint's): the hardware
+// conversion applies the scale's exponent itself, one instruction for two codes, exactly.
+__device__ __forceinline__ void dequant_fp4_pow2(const u32x4_t& raw, float scale0, float scale1, u32x4_t (&out)[4]) {
+  const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const float scale = q < 2 ? scale0 : scale1;
+    out[q] = u32x4_t{__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(words[q], scale, 0)),
+                     __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(words[q], scale, 1)),
+                     __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(words[q], scale, 2)),
+                     __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(words[q], scale, 3))};
+  }
 }
 
-template <int FORMAT, bool PAIRED>
+// One grouped-GEMM kernel, templated on the weight format, on whether two banks (gate, up) are multiplied in
+// the same launch with the SwiGLU epilogue, and on the block tile: BM rows x BN columns of each matrix. The
+// four wavefronts sit 2 x 2; each owns (BM/2) x (BN/2) of every matrix as 32 x 32 MFMA tiles.
+template <int FORMAT, bool PAIRED, int BM, int BN>
 __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
-  constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4;
+  constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4;
+  constexpr bool kPow2 = FORMAT == DEW_MOE_W_MXFP4;
   constexpr int kMatrices = PAIRED ? 2 : 1;
   constexpr int kAtomK = kFp4 ? 64 : 32;                       // depth an atom covers
   constexpr int kAtomsPerStep = (BN / 32) * (BK / kAtomK);     // per matrix
   constexpr int kLoads = kAtomsPerStep * kMatrices / 4;        // 16-byte loads a lane issues per step
   constexpr int kChunksPerLoad = kFp4 ? 4 : 2;
+  constexpr int kRowLoads = BM / 32;                           // A rows a lane loads per step
+  constexpr int TI = BM / 64, TJ = BN / 64;                    // MFMA tiles per wavefront: rows, columns
+  constexpr int kStageChunks = (BM + kMatrices * BN) * kChunksPerRow;
 
-  __shared__ u32x4_t lds_a[BM * kChunksPerRow];
-  __shared__ u32x4_t lds_b[kMatrices * BN * kChunksPerRow];
+  extern __shared__ u32x4_t lds[];  // two stages of [A: BM rows][B: kMatrices x BN rows], 128-byte rows
   __shared__ int wave_tiles[4];
   __shared__ int found[3];  // expert, first sorted row of the tile, total m-tiles
 
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
-  const int m_tile = blockIdx.x, n0 = blockIdx.y * BN;
+
+  // ---- block -> (m-tile, column strip). Workgroup ids are dealt round-robin to the 8 XCDs, each with its
+  // own L2: give every XCD a contiguous run of the tile order, and order tiles so that a run of 32 blocks
+  // (one XCD's residents) covers kGroupM m-tiles x 4 strips, sharing A rows and B strips through that L2.
+  constexpr int kGroupM = 8;
+  const int n_strips = p.width / BN;
+  const int total = p.m_tile_bound * n_strips;
+  const int per_xcd = (total + 7) / 8;
+  const int order = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (order >= total) return;
+  const int group = order / (kGroupM * n_strips);
+  const int group_m = min(kGroupM, p.m_tile_bound - group * kGroupM);
+  const int within = order % (kGroupM * n_strips);
+  const int m_tile = group * kGroupM + within % group_m;
+  const int n0 = (within / group_m) * BN;
 
   // ---- which expert owns m-tile `m_tile`? inclusive scan of ceil(size / BM) over the experts ----
   if (tid == 0) found[0] = -1;
@@ -161,9 +187,9 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
 
   // ---- A loader: 16-byte chunk `a_chunk` of rows a_row + 32 i ----
   const int a_chunk = tid % kChunksPerRow, a_row = tid / kChunksPerRow;
-  const u32x4_t* a_src[BM / 32];
+  const u32x4_t* a_src[kRowLoads];
 #pragma unroll
-  for (int i = 0; i < BM / 32; ++i) {
+  for (int i = 0; i < kRowLoads; ++i) {
     const int sorted = row0 + min(a_row + 32 * i, valid_rows - 1);
     const int source = p.gather ? p.gather[sorted] : sorted;
     a_src[i] = reinterpret_cast<const u32x4_t*>(p.x + static_cast<size_t>(source) * p.depth) + a_chunk;
@@ -173,109 +199,136 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   const uint8_t* b_src[kLoads];
   const uint16_t* b_scale_src[kLoads];
   float b_scale[kLoads];
-  int b_row[kLoads], b_chunk[kLoads], b_matrix[kLoads];
+  int b_row[kLoads], b_first[kLoads];  // stage row and first 16-byte chunk the lane's dequantized values fill
+  const float* block_scales[kLoads];
   const int n_atoms = p.width / 32, k_atoms = p.depth / kAtomK;
 #pragma unroll
   for (int j = 0; j < kLoads; ++j) {
     const int atom = wave + 4 * j;
     const int matrix = atom / kAtomsPerStep;
-    const int within = atom % kAtomsPerStep;
-    const int na = within / (BK / kAtomK), ka = within % (BK / kAtomK);
+    const int slot = atom % kAtomsPerStep;
+    const int na = slot / (BK / kAtomK), ka = slot % (BK / kAtomK);
     const uint8_t* codes = matrix == 0 ? p.w0.codes : p.w1.codes;
     const void* scales = matrix == 0 ? p.w0.scales : p.w1.scales;
     const size_t first_atom = (static_cast<size_t>(expert) * n_atoms + n0 / 32 + na) * k_atoms + ka;
     b_src[j] = codes + first_atom * kAtomBytes + lane * 16;
-    b_matrix[j] = matrix;
-    b_row[j] = na * 32 + lane % 32;
-    b_chunk[j] = ka * (kAtomK / 8) + (lane / 32) * kChunksPerLoad;
+    b_row[j] = BM + matrix * BN + na * 32 + lane % 32;  // rows of a stage: A first, then each matrix
+    b_first[j] = ka * (kAtomK / 8) + (lane / 32) * kChunksPerLoad;
     b_scale[j] = 1.0f;
     b_scale_src[j] = nullptr;
+    block_scales[j] = nullptr;
     if (kFp4) {
       b_scale_src[j] = static_cast<const uint16_t*>(scales) + first_atom * 64 + lane;
     } else if (FORMAT == DEW_MOE_W_FP8_CHANNEL) {
-      b_scale[j] = static_cast<const float*>(scales)[static_cast<size_t>(expert) * p.width + n0 + b_row[j]];
+      b_scale[j] = static_cast<const float*>(scales)[static_cast<size_t>(expert) * p.width + n0 + na * 32 + lane % 32];
+    } else {
+      block_scales[j] = static_cast<const float*>(scales) +
+                        static_cast<size_t>(expert) * (p.depth / 128) * (p.width / 128) + (n0 + na * 32) / 128;
     }
   }
-
-  u32x4_t a_regs[BM / 32], b_regs[kLoads];
+  u32x4_t a_regs[kRowLoads], b_regs[kLoads];
   uint32_t s_regs[kLoads];
   auto load_step = [&](int step) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < BM / 32; ++i) a_regs[i] = a_src[i][static_cast<size_t>(step) * kChunksPerRow];
+    for (int i = 0; i < kRowLoads; ++i) a_regs[i] = a_src[i][static_cast<size_t>(step) * kChunksPerRow];
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
       b_regs[j] = *reinterpret_cast<const u32x4_t*>(b_src[j] + static_cast<size_t>(step) * (BK / kAtomK) * kAtomBytes);
       if (kFp4) {
         s_regs[j] = b_scale_src[j][static_cast<size_t>(step) * (BK / kAtomK) * 64];
       } else if (FORMAT == DEW_MOE_W_FP8_BLOCK) {
-        const void* scales = b_matrix[j] == 0 ? p.w0.scales : p.w1.scales;
-        const int k_blocks = p.depth / 128, n_blocks = p.width / 128;
-        const size_t at = (static_cast<size_t>(expert) * k_blocks + (step * BK) / 128) * n_blocks + n0 / 128;
-        s_regs[j] = __float_as_uint(static_cast<const float*>(scales)[at]);
+        s_regs[j] = __float_as_uint(block_scales[j][static_cast<size_t>((step * BK) / 128) * (p.width / 128)]);
       }
     }
   };
 
-  auto store_step = [&]() __attribute__((always_inline)) {
+  auto store_a = [&](u32x4_t* stage) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < BM / 32; ++i) lds_a[swizzled(a_row + 32 * i, a_chunk)] = a_regs[i];
+    for (int i = 0; i < kRowLoads; ++i) stage[swizzled(a_row + 32 * i, a_chunk)] = a_regs[i];
+  };
+  auto store_b = [&](u32x4_t* stage) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
-      u32x4_t* dst = lds_b + b_matrix[j] * BN * kChunksPerRow;
       if (kFp4) {
         const float scale0 = __builtin_amdgcn_cvt_f32_fp8(s_regs[j], 0) * 0.00390625f;
         const float scale1 = __builtin_amdgcn_cvt_f32_fp8(s_regs[j], 1) * 0.00390625f;
         u32x4_t chunks[4];
-        dequant_fp4(b_regs[j], scale0, scale1, chunks);
+        if (kPow2) {
+          dequant_fp4_pow2(b_regs[j], scale0, scale1, chunks);
+        } else {
+          dequant_fp4(b_regs[j], scale0, scale1, chunks);
+        }
 #pragma unroll
-        for (int c = 0; c < 4; ++c) dst[swizzled(b_row[j], b_chunk[j] + c)] = chunks[c];
+        for (int c = 0; c < 4; ++c) stage[swizzled(b_row[j], b_first[j] + c)] = chunks[c];
       } else {
         const float scale = FORMAT == DEW_MOE_W_FP8_BLOCK ? __uint_as_float(s_regs[j]) : b_scale[j];
         u32x4_t chunks[2];
         dequant_fp8(b_regs[j], scale, chunks);
 #pragma unroll
-        for (int c = 0; c < 2; ++c) dst[swizzled(b_row[j], b_chunk[j] + c)] = chunks[c];
+        for (int c = 0; c < 2; ++c) stage[swizzled(b_row[j], b_first[j] + c)] = chunks[c];
       }
     }
   };
 
-  // ---- accumulators: wave (wm, wn) owns rows wm*64.., columns wn*64.. as 2 x 2 MFMA tiles ----
-  const int wm0 = (wave / 2) * 64, wn0 = (wave % 2) * 64;
-  f32x16_t acc[kMatrices][2][2];
+  // ---- accumulators ----
+  const int wm0 = (wave / 2) * (BM / 2), wn0 = (wave % 2) * (BN / 2);
+  f32x16_t acc[kMatrices][TI][TJ];
 #pragma unroll
   for (int m = 0; m < kMatrices; ++m)
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TI; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < TJ; ++j)
 #pragma unroll
         for (int q = 0; q < 16; ++q) acc[m][i][j][q] = 0.0f;
 
+  // Operand fragments are double-buffered in registers: while the matrix cores work on one 16-deep slice,
+  // the next slice's ds_read_b128s are in flight.
+  bf16x8_t a_frag[2][TI], b_frag[2][kMatrices][TJ];
+  auto fetch = [&](const u32x4_t* stage, int kk, int set) __attribute__((always_inline)) {
+    const int chunk = 2 * kk + lane / 32;
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+      a_frag[set][i] = __builtin_bit_cast(bf16x8_t, stage[swizzled(wm0 + 32 * i + lane % 32, chunk)]);
+#pragma unroll
+    for (int m = 0; m < kMatrices; ++m)
+#pragma unroll
+      for (int j = 0; j < TJ; ++j)
+        b_frag[set][m][j] = __builtin_bit_cast(bf16x8_t, stage[swizzled(BM + m * BN + wn0 + 32 * j + lane % 32, chunk)]);
+  };
+  auto multiply = [&](int set) __attribute__((always_inline)) {
+#pragma unroll
+    for (int m = 0; m < kMatrices; ++m)
+#pragma unroll
+      for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+          acc[m][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_frag[set][i], b_frag[set][m][j], acc[m][i][j], 0, 0, 0);
+  };
+
+  // ---- pipeline: LDS stage s holds step s; registers hold step s + 1; global loads of step s + 2 fly.
+  // One barrier a step: the stage written during step s was last read before the barrier of step s - 1.
   load_step(0);
+  store_a(lds);
+  store_b(lds);
+  load_step(min(1, steps - 1));
+  __syncthreads();
+  fetch(lds, 0, 0);
   for (int step = 0; step < steps; ++step) {
-    store_step();
+    u32x4_t* current = lds + (step & 1) * kStageChunks;
+    u32x4_t* next = lds + ((step + 1) & 1) * kStageChunks;
+    fetch(current, 1, 1);
+    multiply(0);
+    store_a(next);
+    fetch(current, 2, 0);
+    multiply(1);
+    store_b(next);
+    fetch(current, 3, 1);
+    multiply(0);
+    load_step(min(step + 2, steps - 1));
     __syncthreads();
-    if (step + 1 < steps) load_step(step + 1);
-#pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      const int chunk = 2 * kk + lane / 32;
-      bf16x8_t a_frag[2], b_frag[kMatrices][2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) a_frag[i] = __builtin_bit_cast(bf16x8_t, lds_a[swizzled(wm0 + 32 * i + lane % 32, chunk)]);
-#pragma unroll
-      for (int m = 0; m < kMatrices; ++m)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-          b_frag[m][j] = __builtin_bit_cast(bf16x8_t, lds_b[m * BN * kChunksPerRow + swizzled(wn0 + 32 * j + lane % 32, chunk)]);
-#pragma unroll
-      for (int m = 0; m < kMatrices; ++m)
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int j = 0; j < 2; ++j)
-            acc[m][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_frag[i], b_frag[m][j], acc[m][i][j], 0, 0, 0);
-    }
-    __syncthreads();
+    fetch(next, 0, 0);
+    multiply(1);
   }
 
   // ---- epilogue: acc[..][q] is row 8 (q / 4) + 4 (lane / 32) + q % 4, column lane % 32 of its 32 x 32 tile ----
@@ -285,7 +338,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
     if (PAIRED) factor1 = 256.0f * p.w1.tensor_scale[expert];
   }
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < TI; ++i) {
 #pragma unroll
     for (int q = 0; q < 16; ++q) {
       const int row = wm0 + 32 * i + 8 * (q / 4) + 4 * (lane / 32) + q % 4;
@@ -294,7 +347,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
       const int out_row = p.scatter ? p.scatter[sorted] : sorted;
       bf16_t* dst = p.out + static_cast<size_t>(out_row) * p.width + n0 + wn0 + lane % 32;
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < TJ; ++j) {
         if (PAIRED) {
           dst[32 * j] = swiglu_rounded(acc[0][i][j][q] * factor0, acc[kMatrices - 1][i][j][q] * factor1);
         } else {
@@ -308,34 +361,63 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
 static int check_bank(const char* who, const dew_moe_bank* bank, const char* name) {
   DEW_REQUIRE(bank, "%s: %s bank must not be null", who, name);
   DEW_REQUIRE(bank->layout == DEW_MOE_LAYOUT_PREPARED, "%s: %s bank is in the reference layout; call dew_moe_prepare_bank once at load", who, name);
-  DEW_REQUIRE(bank->format == DEW_MOE_W_FP8_BLOCK || bank->format == DEW_MOE_W_FP8_CHANNEL || bank->format == DEW_MOE_W_NVFP4,
+  DEW_REQUIRE(bank->format == DEW_MOE_W_FP8_BLOCK || bank->format == DEW_MOE_W_FP8_CHANNEL || bank->format == DEW_MOE_W_NVFP4 ||
+                  bank->format == DEW_MOE_W_MXFP4,
               "%s: %s bank has unknown format %d", who, name, bank->format);
   DEW_REQUIRE(bank->experts >= 1 && bank->experts <= 4096, "%s: %s bank has %d experts", who, name, bank->experts);
-  DEW_REQUIRE(bank->depth >= BK && bank->depth % 128 == 0, "%s: %s bank depth %d is not a multiple of 128", who, name, bank->depth);
-  DEW_REQUIRE(bank->width % BN == 0 && bank->width >= BN, "%s: %s bank width %d is not a multiple of %d", who, name, bank->width, BN);
+  DEW_REQUIRE(bank->depth >= 128 && bank->depth % 128 == 0, "%s: %s bank depth %d is not a multiple of 128", who, name, bank->depth);
+  DEW_REQUIRE(bank->width % 128 == 0 && bank->width >= 128, "%s: %s bank width %d is not a multiple of 128", who, name, bank->width);
   DEW_REQUIRE(bank->codes && bank->scales, "%s: %s bank codes and scales must not be null", who, name);
-  DEW_REQUIRE(bank->format != DEW_MOE_W_NVFP4 || bank->tensor_scale, "%s: %s NVFP4 bank needs tensor scales", who, name);
+  DEW_REQUIRE((bank->format != DEW_MOE_W_NVFP4 && bank->format != DEW_MOE_W_MXFP4) || bank->tensor_scale, "%s: %s NVFP4 bank needs tensor scales", who, name);
   DEW_REQUIRE(aligned16(bank->codes), "%s: %s bank codes must be 16-byte aligned", who, name);
   return DEW_MOE_OK;
 }
 
+template <int FORMAT, bool PAIRED, int BM, int BN>
+static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
+  constexpr int kMatrices = PAIRED ? 2 : 1;
+  constexpr size_t kShared = 2 * static_cast<size_t>(BM + kMatrices * BN) * BK * sizeof(bf16_t);
+  auto kernel = grouped_gemm_kernel<FORMAT, PAIRED, BM, BN>;
+  static bool configured = false;  // dynamic LDS above 64 KiB must be opted into once per kernel
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(kShared)) != hipSuccess)
+      return fail(DEW_MOE_ELAUNCH, "%s: cannot reserve %zu bytes of LDS", who, kShared);
+    configured = true;
+  }
+  // every expert may end in a partial tile, and the zeroed tail may add one more
+  p.m_tile_bound = (p.rows + BM - 1) / BM + p.experts + 1;
+  const int total = p.m_tile_bound * (p.width / BN);
+  const int blocks = ((total + 7) / 8) * 8;
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreads), kShared, stream, p);
+  return launched(who);
+}
+
+// Tile choice from what the host knows (rows and experts; the routing itself stays on the device): large
+// tiles when the average group fills them, the 128 x 128 tile otherwise.
+template <int FORMAT, bool PAIRED>
+static int launch_format(const char* who, const GemmParams& p, hipStream_t stream) {
+  const bool large = p.rows / p.experts >= 768 && p.width % 256 == 0;
+  if (PAIRED) {
+    if (large) return launch_tile<FORMAT, true, 256, 128>(who, p, stream);
+    return launch_tile<FORMAT, true, 128, 128>(who, p, stream);
+  }
+  if (large) return launch_tile<FORMAT, false, 256, 256>(who, p, stream);
+  return launch_tile<FORMAT, false, 128, 128>(who, p, stream);
+}
+
 template <bool PAIRED>
 static int launch(const char* who, const GemmParams& p, int format, hipStream_t stream) {
-  // every expert may end in a partial tile, and the zeroed tail may add one more
-  const int m_tiles = (p.rows + BM - 1) / BM + p.experts + 1;
-  const dim3 grid(m_tiles, p.width / BN), block(kThreads);
   switch (format) {
     case DEW_MOE_W_FP8_BLOCK:
-      hipLaunchKernelGGL((grouped_gemm_kernel<DEW_MOE_W_FP8_BLOCK, PAIRED>), grid, block, 0, stream, p);
-      break;
+      return launch_format<DEW_MOE_W_FP8_BLOCK, PAIRED>(who, p, stream);
     case DEW_MOE_W_FP8_CHANNEL:
-      hipLaunchKernelGGL((grouped_gemm_kernel<DEW_MOE_W_FP8_CHANNEL, PAIRED>), grid, block, 0, stream, p);
-      break;
+      return launch_format<DEW_MOE_W_FP8_CHANNEL, PAIRED>(who, p, stream);
+    case DEW_MOE_W_MXFP4:
+      return launch_format<DEW_MOE_W_MXFP4, PAIRED>(who, p, stream);
     default:
-      hipLaunchKernelGGL((grouped_gemm_kernel<DEW_MOE_W_NVFP4, PAIRED>), grid, block, 0, stream, p);
-      break;
+      return launch_format<DEW_MOE_W_NVFP4, PAIRED>(who, p, stream);
   }
-  return launched(who);
 }
 
 }  // namespace dew

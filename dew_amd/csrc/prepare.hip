@@ -90,9 +90,11 @@ __global__ __launch_bounds__(256) void prepare_nvfp4_codes_kernel(const uint32_t
   }
 }
 
+// Also notes in *general whether any scale is not a normal power of two (mantissa bits set, or a zero or
+// subnormal exponent).
 __global__ __launch_bounds__(256) void prepare_nvfp4_scales_kernel(const uint8_t* __restrict__ scales,
                                                                    uint16_t* __restrict__ out, int experts, int depth,
-                                                                   int width) {
+                                                                   int width, uint32_t* __restrict__ general) {
   const int n_atoms = width / 32, k_atoms = depth / 64;
   const long long total = static_cast<long long>(experts) * n_atoms * k_atoms * 64;
   for (long long item = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; item < total;
@@ -105,6 +107,7 @@ __global__ __launch_bounds__(256) void prepare_nvfp4_scales_kernel(const uint8_t
     const int n = na * 32 + lane % 32;
     const uint8_t* src = scales + (static_cast<size_t>(e) * width + n) * (depth / 16) + ka * 4 + 2 * (lane / 32);
     out[item] = static_cast<uint16_t>(src[0]) | (static_cast<uint16_t>(src[1]) << 8);
+    if ((src[0] & 7) || (src[1] & 7) || !(src[0] & 0x78) || !(src[1] & 0x78)) atomicOr(general, 1u);
   }
 }
 
@@ -118,7 +121,7 @@ static size_t codes_bytes(int format, int experts, int depth, int width) {
 extern "C" size_t dew_moe_prepared_bytes(int32_t format, int32_t experts, int32_t depth, int32_t width) {
   if (experts <= 0 || depth <= 0 || width <= 0) return 0;
   size_t bytes = dew::codes_bytes(format, experts, depth, width);
-  if (format == DEW_MOE_W_NVFP4) bytes += static_cast<size_t>(experts) * width * (depth / 16);
+  if (format == DEW_MOE_W_NVFP4) bytes += static_cast<size_t>(experts) * width * (depth / 16) + 256;  // + a flag word
   return bytes;
 }
 
@@ -147,10 +150,16 @@ extern "C" int dew_moe_prepare_bank(const dew_moe_bank* ref, void* prepared, dew
     hipLaunchKernelGGL(prepare_nvfp4_codes_kernel, dim3(grid), dim3(256), 0, s, static_cast<const uint32_t*>(ref->codes),
                        codes_out, ref->experts, ref->depth, ref->width);
     if (int rc = launched("prepare_nvfp4_codes_kernel")) return rc;
+    uint32_t* general = reinterpret_cast<uint32_t*>(scales_out + static_cast<size_t>(ref->experts) * ref->width * (ref->depth / 16));
+    if (hipMemsetAsync(general, 0, sizeof(uint32_t), s) != hipSuccess) return fail(DEW_MOE_ELAUNCH, "dew_moe_prepare_bank: memset failed");
     hipLaunchKernelGGL(prepare_nvfp4_scales_kernel, dim3(grid), dim3(256), 0, s, static_cast<const uint8_t*>(ref->scales),
-                       reinterpret_cast<uint16_t*>(scales_out), ref->experts, ref->depth, ref->width);
+                       reinterpret_cast<uint16_t*>(scales_out), ref->experts, ref->depth, ref->width, general);
     if (int rc = launched("prepare_nvfp4_scales_kernel")) return rc;
     out->scales = scales_out;
+    uint32_t found = 1;
+    if (hipMemcpyAsync(&found, general, sizeof(found), hipMemcpyDeviceToHost, s) != hipSuccess || hipStreamSynchronize(s) != hipSuccess)
+      return fail(DEW_MOE_ELAUNCH, "dew_moe_prepare_bank: reading the scale summary back failed: %s", hipGetErrorString(hipGetLastError()));
+    if (!found) out->format = DEW_MOE_W_MXFP4;
   } else {
     DEW_REQUIRE(ref->depth % 128 == 0, "dew_moe_prepare_bank: an FP8 bank's depth is whole 128s, not %d", ref->depth);
     hipLaunchKernelGGL(prepare_fp8_kernel, dim3(grid), dim3(256), 0, s, static_cast<const uint8_t*>(ref->codes),

@@ -1,7 +1,8 @@
 /* C ABI of libdew_moe_hip.so: the MI355X (gfx950) kernels of the quantized Mixture-of-Experts expert path.
  *
  * Plain pointers and sizes only: every pointer is DEVICE memory on the current HIP device unless said
- * otherwise, `stream` is a hipStream_t passed as void*. No entry point allocates, frees or synchronizes:
+ * otherwise, `stream` is a hipStream_t passed as void*. No entry point allocates or frees, and none but the
+ * load-time dew_moe_prepare_bank synchronizes:
  * group bookkeeping is read on the device from `offsets`, so calls are stream-ordered and graph-safe, as
  * the reference's CUTLASS FFI library is (kernels/cutlass/ffi.cu:1-6, groups.cuh:19-30). Every entry point
  * returns 0 on success and a nonzero DEW_MOE_E* code otherwise; dew_moe_last_error() then names the refused
@@ -32,9 +33,11 @@ enum {
 enum {
   DEW_MOE_W_FP8_BLOCK = 1,   /* codes u8 e4m3 [E,K,N]; scales f32 [E,ceil(K/128),ceil(N/128)]           */
   DEW_MOE_W_FP8_CHANNEL = 2, /* codes u8 e4m3 [E,K,N]; scales f32 [E,N]                                 */
-  DEW_MOE_W_NVFP4 = 3        /* codes = NvFp4.words u32 [E,N,K/8] (staged order, GF(2)-encoded);        */
+  DEW_MOE_W_NVFP4 = 3,       /* codes = NvFp4.words u32 [E,N,K/8] (staged order, GF(2)-encoded);        */
                              /* scales = NvFp4.scales e4m3 bytes [E,N,K/16]; tensor_scale f32 [E].      */
                              /* MXFP4 banks arrive in this form (codecs.mxfp4_as_nvfp4).                */
+  DEW_MOE_W_MXFP4 = 4        /* prepared banks only: an NVFP4 bank whose block scales are all powers of */
+                             /* two, as an MXFP4 checkpoint's are; dew_moe_prepare_bank finds it so.    */
 };
 
 enum { DEW_MOE_LAYOUT_REFERENCE = 0, DEW_MOE_LAYOUT_PREPARED = 1 };
@@ -90,7 +93,9 @@ int dew_moe_group_offsets(const int32_t* sizes, int32_t experts, int32_t* offset
  * The GEMM kernels read a bank re-laid into MFMA-fragment order (exact: a permutation of the codes; the
  * NVFP4 word encoder is an invertible GF(2) map, src/dew/algebra/bits.py:208-223,240-250). Call once per
  * bank at load; `prepared` must hold dew_moe_prepared_bytes() bytes, 256-byte aligned. `out` describes
- * the prepared bank and is what the GEMM entry points take.                                             */
+ * the prepared bank and is what the GEMM entry points take. For an NVFP4 bank the call waits for the
+ * stream once, to read back whether every block scale is a power of two (then out->format is
+ * DEW_MOE_W_MXFP4 and the kernels convert codes and scale in one hardware instruction).                 */
 size_t dew_moe_prepared_bytes(int32_t format, int32_t experts, int32_t depth, int32_t width);
 int dew_moe_prepare_bank(const dew_moe_bank* reference, void* prepared, dew_moe_bank* out /* host */,
                          void* stream);

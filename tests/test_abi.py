@@ -28,7 +28,7 @@ def test_introspection_strings_and_size_queries():
     for line in lib.dew_moe_kernels().decode().strip().splitlines():
         assert len(line.split(",")) == len(fields)
     assert lib.dew_moe_prepared_bytes(_lib.W_FP8_BLOCK, 2, 256, 128) == 2 * 256 * 128
-    assert lib.dew_moe_prepared_bytes(_lib.W_NVFP4, 2, 256, 128) == 2 * 256 * 128 // 2 + 2 * 128 * 16
+    assert lib.dew_moe_prepared_bytes(_lib.W_NVFP4, 2, 256, 128) == 2 * 256 * 128 // 2 + 2 * 128 * 16 + 256
     assert lib.dew_moe_permute_workspace_bytes(4096, 8) >= 2 * 2 * 9 * 4
 
 
