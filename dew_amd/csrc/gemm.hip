@@ -9,9 +9,9 @@
 // expert's group (two such tiles, gate and up, when paired) and walks the depth in 64-deep steps. Tiles are
 // enumerated on the device from `offsets` (no host read of the routing): block (x, y) takes m-tile x of
 // column strip y; experts with no rows own no tiles. Global loads of step t+1 are in flight while step t
-// multiplies out of LDS. LDS rows are 128 bytes (64 bf16) with the 16-byte chunk index xor-swizzled by
-// (row >> 1) & 7, which makes both the ds_write_b128 of the loaders and the ds_read_b128 of the MFMA
-// operand fetch conflict-free.
+// multiplies out of LDS. LDS rows are 128 bytes (64 bf16) with the 16-byte chunk index xor-swizzled by a
+// function of the row (`swizzled`), which makes both the ds_write_b128 of the loaders and the ds_read_b128
+// of the MFMA operand fetch conflict-free.
 #include "common.h"
 
 namespace dew {
@@ -42,7 +42,15 @@ struct GemmParams {
   int experts, depth, width, rows, m_tile_bound;
 };
 
-__device__ __forceinline__ int swizzled(int row, int chunk) { return row * kChunksPerRow + (chunk ^ ((row >> 1) & 7)); }
+// LDS index of 16-byte chunk `chunk` of row `row` (128-byte rows). The chunk is xor-swizzled by
+// f(row) = ((row >> 1) & 7) ^ ((row & 1) << 2), chosen against the measured service order of gfx950's LDS:
+// ds_read_b128 serves 16 lanes a pass over 64 banks, the passes being lanes {0-3,12-15,20-23,24-27},
+// {4-7,8-11,16-19,28-31} and the same + 32; ds_write_b128 serves 8 consecutive lanes a pass over 128 bytes.
+// With lane = row (mod 32) on the read side and on the weight-store side, f is injective on every read pass's
+// rows of one parity and on every aligned run of 8 rows, so fragment reads and both stores are conflict-free.
+__device__ __forceinline__ int swizzled(int row, int chunk) {
+  return row * kChunksPerRow + (chunk ^ (((row >> 1) & 7) ^ ((row & 1) << 2)));
+}
 
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
   bf16x2_t pair = {static_cast<__bf16>(a), static_cast<__bf16>(b)};
@@ -97,6 +105,23 @@ __device__ __forceinline__ void dequant_fp4_pow2(const u32x4_t& raw, float scale
                      __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(words[q], scale, 1)),
                      __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(words[q], scale, 2)),
                      __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(words[q], scale, 3))};
+  }
+}
+
+// Instruction order of one phase of the main loop, stated to the scheduler: `MFMAS` matrix instructions in a
+// row, the phase's `DSR` operand reads issued one behind each of the first of them (so they are long done
+// when the next phase multiplies them), and the phase's other work (vector ALU, LDS stores, global loads)
+// dealt evenly into the shadows of all of them. Masks: 0x8 MFMA, 0x100 DS read, 0x200 DS write, 0x2 VALU,
+// 0x20 VMEM read.
+template <int M, int MFMAS, int DSR, int DSW, int VALU, int VMEM>
+__device__ __forceinline__ void schedule_phase() {
+  if constexpr (M < MFMAS) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    if constexpr (M < DSR) __builtin_amdgcn_sched_group_barrier(0x100, 1 + (M == 0 ? (DSR > MFMAS ? DSR - MFMAS : 0) : 0), 0);
+    if constexpr (VALU > 0) __builtin_amdgcn_sched_group_barrier(0x002, (VALU + MFMAS - 1) / MFMAS, 0);
+    if constexpr (DSW > 0) __builtin_amdgcn_sched_group_barrier(0x200, (DSW + MFMAS - 1) / MFMAS, 0);
+    if constexpr (VMEM > 0) __builtin_amdgcn_sched_group_barrier(0x020, (VMEM + MFMAS - 1) / MFMAS, 0);
+    schedule_phase<M + 1, MFMAS, DSR, DSW, VALU, VMEM>();
   }
 }
 
@@ -228,9 +253,11 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   }
   u32x4_t a_regs[kRowLoads], b_regs[kLoads];
   uint32_t s_regs[kLoads];
-  auto load_step = [&](int step) __attribute__((always_inline)) {
+  auto load_a = [&](int step) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < kRowLoads; ++i) a_regs[i] = a_src[i][static_cast<size_t>(step) * kChunksPerRow];
+  };
+  auto load_b = [&](int step) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
       b_regs[j] = *reinterpret_cast<const u32x4_t*>(b_src[j] + static_cast<size_t>(step) * (BK / kAtomK) * kAtomBytes);
@@ -306,29 +333,51 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
           acc[m][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_frag[set][i], b_frag[set][m][j], acc[m][i][j], 0, 0, 0);
   };
 
-  // ---- pipeline: LDS stage s holds step s; registers hold step s + 1; global loads of step s + 2 fly.
+  // ---- pipeline: LDS stage s holds step s; registers hold step s + 1; the global loads of step s + 2 are
+  // issued right behind the LDS stores that free their registers, a whole step ahead of their use.
   // One barrier a step: the stage written during step s was last read before the barrier of step s - 1.
-  load_step(0);
+  load_a(0);
+  load_b(0);
   store_a(lds);
   store_b(lds);
-  load_step(min(1, steps - 1));
+  load_a(min(1, steps - 1));
+  load_b(min(1, steps - 1));
   __syncthreads();
   fetch(lds, 0, 0);
+  constexpr int kMfmas = kMatrices * TI * TJ, kReads = TI + kMatrices * TJ;
+  constexpr int kStoresB = kLoads * kChunksPerLoad;
+  constexpr int kDequantOps = kPow2 ? kLoads * 22 : (kFp4 ? kLoads * 70 : kLoads * 34);
+  constexpr int kLoadsB = kLoads * (kFp4 || FORMAT == DEW_MOE_W_FP8_BLOCK ? 2 : 1);
   for (int step = 0; step < steps; ++step) {
     u32x4_t* current = lds + (step & 1) * kStageChunks;
     u32x4_t* next = lds + ((step + 1) & 1) * kStageChunks;
+    const int ahead = min(step + 2, steps - 1);
+    // phase 1: slice 0 multiplies; slice 1's operands are read; the A rows of step + 1 go to the other
+    // stage and the A rows of step + 2 are requested
     fetch(current, 1, 1);
     multiply(0);
     store_a(next);
+    load_a(ahead);
+    schedule_phase<0, kMfmas, kReads, kRowLoads, 2 * kRowLoads, kRowLoads>();
+    __builtin_amdgcn_sched_barrier(0);
+    // phase 2: slice 1 multiplies; the weights of step + 1 are dequantized and stored, those of step + 2 requested
     fetch(current, 2, 0);
     multiply(1);
     store_b(next);
+    load_b(ahead);
+    schedule_phase<0, kMfmas, kReads, kStoresB, kDequantOps + kLoadsB, kLoadsB>();
+    __builtin_amdgcn_sched_barrier(0);
+    // phase 3: slice 2 multiplies
     fetch(current, 3, 1);
     multiply(0);
-    load_step(min(step + 2, steps - 1));
+    schedule_phase<0, kMfmas, kReads, 0, 0, 0>();
+    __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
+    // phase 4: slice 3 multiplies; the first operands of the next stage are read
     fetch(next, 0, 0);
     multiply(1);
+    schedule_phase<0, kMfmas, kReads, 0, 0, 0>();
+    __builtin_amdgcn_sched_barrier(0);
   }
 
   // ---- epilogue: acc[..][q] is row 8 (q / 4) + 4 (lane / 32) + q % 4, column lane % 32 of its 32 x 32 tile ----
