@@ -149,8 +149,8 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
 
   // ---- block -> (m-tile, column strip). Workgroup ids are dealt round-robin to the 8 XCDs, each with its
   // own L2: give every XCD a contiguous run of the tile order, and order tiles so that a run of 32 blocks
-  // (one XCD's residents) covers kGroupM m-tiles x 4 strips, sharing A rows and B strips through that L2.
-  constexpr int kGroupM = 8;
+  // (one XCD's residents) covers kGroupM m-tiles x 8 strips, sharing A rows and B strips through that L2.
+  constexpr int kGroupM = 4;
   const int n_strips = p.width / BN;
   const int total = p.m_tile_bound * n_strips;
   const int per_xcd = (total + 7) / 8;
@@ -252,7 +252,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
     }
   }
   u32x4_t a_regs[kRowLoads], b_regs[kLoads];
-  uint32_t s_regs[kLoads];
+  uint32_t s_regs[kLoads];  // FP4: the lane's two e4m3 scale bytes in the low half (the high half is the next lane's)
   auto load_a = [&](int step) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < kRowLoads; ++i) a_regs[i] = a_src[i][static_cast<size_t>(step) * kChunksPerRow];
@@ -262,7 +262,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
     for (int j = 0; j < kLoads; ++j) {
       b_regs[j] = *reinterpret_cast<const u32x4_t*>(b_src[j] + static_cast<size_t>(step) * (BK / kAtomK) * kAtomBytes);
       if (kFp4) {
-        s_regs[j] = b_scale_src[j][static_cast<size_t>(step) * (BK / kAtomK) * 64];
+        __builtin_memcpy(&s_regs[j], b_scale_src[j] + static_cast<size_t>(step) * (BK / kAtomK) * 64, sizeof(uint32_t));
       } else if (FORMAT == DEW_MOE_W_FP8_BLOCK) {
         s_regs[j] = __float_as_uint(block_scales[j][static_cast<size_t>((step * BK) / 128) * (p.width / 128)]);
       }
