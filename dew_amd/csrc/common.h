@@ -26,12 +26,9 @@ typedef uint16_t bf16_t;
 
 __device__ __forceinline__ float bf16_to_f32(bf16_t v) { return __uint_as_float(static_cast<uint32_t>(v) << 16); }
 
-// Round to nearest, ties to even (finite inputs and infinities; NaN stays NaN by the quiet bit).
+// Round to nearest, ties to even: the hardware conversion (v_cvt_pk_bf16_f32), one instruction, no branch.
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<bf16_t>((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<bf16_t>(u >> 16);
+  return __builtin_bit_cast(bf16_t, static_cast<__bf16>(f));
 }
 
 __device__ __forceinline__ float bf16_round(float f) { return bf16_to_f32(f32_to_bf16(f)); }

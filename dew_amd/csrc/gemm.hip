@@ -12,6 +12,8 @@
 // multiplies out of LDS. LDS rows are 128 bytes (64 bf16) with the 16-byte chunk index xor-swizzled by a
 // function of the row (`swizzled`), which makes both the ds_write_b128 of the loaders and the ds_read_b128
 // of the MFMA operand fetch conflict-free.
+#include <type_traits>
+
 #include "common.h"
 
 namespace dew {
@@ -251,46 +253,47 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
                         static_cast<size_t>(expert) * (p.depth / 128) * (p.width / 128) + (n0 + na * 32) / 128;
     }
   }
-  u32x4_t a_regs[kRowLoads], b_regs[kLoads];
-  uint32_t s_regs[kLoads];  // FP4: the lane's two e4m3 scale bytes in the low half (the high half is the next lane's)
-  auto load_a = [&](int step) __attribute__((always_inline)) {
+  // Two register sets hold the raw global data of two steps, so every load has two steps to land.
+  u32x4_t a_regs[2][kRowLoads], b_regs[2][kLoads];
+  uint32_t s_regs[2][kLoads];  // FP4: the lane's two e4m3 scale bytes in the low half (the high half is the next lane's)
+  auto load_a = [&](auto set, int step) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < kRowLoads; ++i) a_regs[i] = a_src[i][static_cast<size_t>(step) * kChunksPerRow];
+    for (int i = 0; i < kRowLoads; ++i) a_regs[set.value][i] = a_src[i][static_cast<size_t>(step) * kChunksPerRow];
   };
-  auto load_b = [&](int step) __attribute__((always_inline)) {
+  auto load_b = [&](auto set, int step) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
-      b_regs[j] = *reinterpret_cast<const u32x4_t*>(b_src[j] + static_cast<size_t>(step) * (BK / kAtomK) * kAtomBytes);
+      b_regs[set.value][j] = *reinterpret_cast<const u32x4_t*>(b_src[j] + static_cast<size_t>(step) * (BK / kAtomK) * kAtomBytes);
       if (kFp4) {
-        __builtin_memcpy(&s_regs[j], b_scale_src[j] + static_cast<size_t>(step) * (BK / kAtomK) * 64, sizeof(uint32_t));
+        __builtin_memcpy(&s_regs[set.value][j], b_scale_src[j] + static_cast<size_t>(step) * (BK / kAtomK) * 64, sizeof(uint32_t));
       } else if (FORMAT == DEW_MOE_W_FP8_BLOCK) {
-        s_regs[j] = __float_as_uint(block_scales[j][static_cast<size_t>((step * BK) / 128) * (p.width / 128)]);
+        s_regs[set.value][j] = __float_as_uint(block_scales[j][static_cast<size_t>((step * BK) / 128) * (p.width / 128)]);
       }
     }
   };
 
-  auto store_a = [&](u32x4_t* stage) __attribute__((always_inline)) {
+  auto store_a = [&](auto set, u32x4_t* stage) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < kRowLoads; ++i) stage[swizzled(a_row + 32 * i, a_chunk)] = a_regs[i];
+    for (int i = 0; i < kRowLoads; ++i) stage[swizzled(a_row + 32 * i, a_chunk)] = a_regs[set.value][i];
   };
-  auto store_b = [&](u32x4_t* stage) __attribute__((always_inline)) {
+  auto store_b = [&](auto set, u32x4_t* stage) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
       if (kFp4) {
-        const float scale0 = __builtin_amdgcn_cvt_f32_fp8(s_regs[j], 0) * 0.00390625f;
-        const float scale1 = __builtin_amdgcn_cvt_f32_fp8(s_regs[j], 1) * 0.00390625f;
+        const float scale0 = __builtin_amdgcn_cvt_f32_fp8(s_regs[set.value][j], 0) * 0.00390625f;
+        const float scale1 = __builtin_amdgcn_cvt_f32_fp8(s_regs[set.value][j], 1) * 0.00390625f;
         u32x4_t chunks[4];
         if (kPow2) {
-          dequant_fp4_pow2(b_regs[j], scale0, scale1, chunks);
+          dequant_fp4_pow2(b_regs[set.value][j], scale0, scale1, chunks);
         } else {
-          dequant_fp4(b_regs[j], scale0, scale1, chunks);
+          dequant_fp4(b_regs[set.value][j], scale0, scale1, chunks);
         }
 #pragma unroll
         for (int c = 0; c < 4; ++c) stage[swizzled(b_row[j], b_first[j] + c)] = chunks[c];
       } else {
-        const float scale = FORMAT == DEW_MOE_W_FP8_BLOCK ? __uint_as_float(s_regs[j]) : b_scale[j];
+        const float scale = FORMAT == DEW_MOE_W_FP8_BLOCK ? __uint_as_float(s_regs[set.value][j]) : b_scale[j];
         u32x4_t chunks[2];
-        dequant_fp8(b_regs[j], scale, chunks);
+        dequant_fp8(b_regs[set.value][j], scale, chunks);
 #pragma unroll
         for (int c = 0; c < 2; ++c) stage[swizzled(b_row[j], b_first[j] + c)] = chunks[c];
       }
@@ -333,38 +336,35 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
           acc[m][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_frag[set][i], b_frag[set][m][j], acc[m][i][j], 0, 0, 0);
   };
 
-  // ---- pipeline: LDS stage s holds step s; registers hold step s + 1; the global loads of step s + 2 are
-  // issued right behind the LDS stores that free their registers, a whole step ahead of their use.
-  // One barrier a step: the stage written during step s was last read before the barrier of step s - 1.
-  load_a(0);
-  load_b(0);
-  store_a(lds);
-  store_b(lds);
-  load_a(min(1, steps - 1));
-  load_b(min(1, steps - 1));
-  __syncthreads();
-  fetch(lds, 0, 0);
+  // ---- pipeline. At the top of step s: LDS stage s & 1 holds step s; register set (s + 1) & 1 holds the raw
+  // data of step s + 1 and set s & 1 that of step s + 2. During step s the set (s + 1) & 1 is stored to the
+  // other stage (weights dequantized on the way) and at once reloaded with step s + 3, two steps ahead of
+  // its use. One barrier a step: the stage written during step s was last read before the barrier of step
+  // s - 1. The loop is unrolled by two so that stages and register sets are compile-time constants.
+  constexpr std::integral_constant<int, 0> even{};
+  constexpr std::integral_constant<int, 1> odd{};
   constexpr int kMfmas = kMatrices * TI * TJ, kReads = TI + kMatrices * TJ;
   constexpr int kStoresB = kLoads * kChunksPerLoad;
   constexpr int kDequantOps = kPow2 ? kLoads * 22 : (kFp4 ? kLoads * 70 : kLoads * 34);
   constexpr int kLoadsB = kLoads * (kFp4 || FORMAT == DEW_MOE_W_FP8_BLOCK ? 2 : 1);
-  for (int step = 0; step < steps; ++step) {
-    u32x4_t* current = lds + (step & 1) * kStageChunks;
-    u32x4_t* next = lds + ((step + 1) & 1) * kStageChunks;
-    const int ahead = min(step + 2, steps - 1);
+  auto iterate = [&](auto parity, int step) __attribute__((always_inline)) {
+    constexpr std::integral_constant<int, 1 - parity.value> other{};
+    u32x4_t* current = lds + parity.value * kStageChunks;
+    u32x4_t* next = lds + other.value * kStageChunks;
+    const int ahead = min(step + 3, steps - 1);
     // phase 1: slice 0 multiplies; slice 1's operands are read; the A rows of step + 1 go to the other
-    // stage and the A rows of step + 2 are requested
+    // stage and their registers are reloaded
     fetch(current, 1, 1);
     multiply(0);
-    store_a(next);
-    load_a(ahead);
+    store_a(other, next);
+    load_a(other, ahead);
     schedule_phase<0, kMfmas, kReads, kRowLoads, 2 * kRowLoads, kRowLoads>();
     __builtin_amdgcn_sched_barrier(0);
-    // phase 2: slice 1 multiplies; the weights of step + 1 are dequantized and stored, those of step + 2 requested
+    // phase 2: slice 1 multiplies; the weights of step + 1 are dequantized and stored, their registers reloaded
     fetch(current, 2, 0);
     multiply(1);
-    store_b(next);
-    load_b(ahead);
+    store_b(other, next);
+    load_b(other, ahead);
     schedule_phase<0, kMfmas, kReads, kStoresB, kDequantOps + kLoadsB, kLoadsB>();
     __builtin_amdgcn_sched_barrier(0);
     // phase 3: slice 2 multiplies
@@ -378,30 +378,54 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
     multiply(1);
     schedule_phase<0, kMfmas, kReads, 0, 0, 0>();
     __builtin_amdgcn_sched_barrier(0);
+  };
+  load_a(even, 0);
+  load_b(even, 0);
+  store_a(even, lds);
+  store_b(even, lds);
+  load_a(odd, min(1, steps - 1));
+  load_b(odd, min(1, steps - 1));
+  load_a(even, min(2, steps - 1));
+  load_b(even, min(2, steps - 1));
+  __syncthreads();
+  fetch(lds, 0, 0);
+  for (int step = 0; step < steps; step += 2) {  // depth is whole 128s, so steps is even
+    iterate(even, step);
+    iterate(odd, step + 1);
   }
 
-  // ---- epilogue: acc[..][q] is row 8 (q / 4) + 4 (lane / 32) + q % 4, column lane % 32 of its 32 x 32 tile ----
+  // ---- epilogue: acc[..][q] is row 8 (q / 4) + 4 (lane / 32) + q % 4, column lane % 32 of its 32 x 32 tile.
+  // Neighbouring lanes hold neighbouring columns: each pair of lanes swaps one value so that the even lane
+  // holds both columns of row q and the odd lane both of row q + 1, and every lane stores 4 bytes a row pair.
   float factor0 = 1.0f, factor1 = 1.0f;
   if (kFp4) {  // the 2^8 the decode owes times the expert's tensor scale (src/dew/nn/kernels/gemm.py:660-662)
     factor0 = 256.0f * p.w0.tensor_scale[expert];
     if (PAIRED) factor1 = 256.0f * p.w1.tensor_scale[expert];
   }
+  const bool odd_lane = lane & 1;
+  const int column = n0 + wn0 + (lane % 32 & ~1);  // first of the lane pair's two columns
 #pragma unroll
   for (int i = 0; i < TI; ++i) {
 #pragma unroll
-    for (int q = 0; q < 16; ++q) {
-      const int row = wm0 + 32 * i + 8 * (q / 4) + 4 * (lane / 32) + q % 4;
-      if (row >= valid_rows) continue;
-      const int sorted = row0 + row;
-      const int out_row = p.scatter ? p.scatter[sorted] : sorted;
-      bf16_t* dst = p.out + static_cast<size_t>(out_row) * p.width + n0 + wn0 + lane % 32;
+    for (int q = 0; q < 16; q += 2) {
+      const int row = wm0 + 32 * i + 8 * (q / 4) + 4 * (lane / 32) + q % 4 + (odd_lane ? 1 : 0);
+      const bool valid = row < valid_rows;
+      int out_row = row0 + min(row, valid_rows - 1);
+      if (p.scatter) out_row = p.scatter[out_row];
+      uint32_t* dst = reinterpret_cast<uint32_t*>(p.out + static_cast<size_t>(out_row) * p.width + column);
 #pragma unroll
       for (int j = 0; j < TJ; ++j) {
-        if (PAIRED) {
-          dst[32 * j] = swiglu_rounded(acc[0][i][j][q] * factor0, acc[kMatrices - 1][i][j][q] * factor1);
-        } else {
-          dst[32 * j] = f32_to_bf16(acc[0][i][j][q] * factor0);
+        uint32_t mine[2];
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+          mine[r] = PAIRED ? swiglu_rounded(acc[0][i][j][q + r] * factor0, acc[kMatrices - 1][i][j][q + r] * factor1)
+                           : f32_to_bf16(acc[0][i][j][q + r] * factor0);
         }
+        // even lane keeps row q and sends its row q + 1; odd lane keeps row q + 1 and sends its row q
+        const uint32_t sent = odd_lane ? mine[0] : mine[1];
+        const uint32_t got = __builtin_amdgcn_mov_dpp(sent, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+        const uint32_t packed = odd_lane ? (got | (mine[1] << 16)) : (mine[0] | (got << 16));
+        if (valid) dst[16 * j] = packed;
       }
     }
   }
