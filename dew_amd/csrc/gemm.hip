@@ -5,13 +5,19 @@
 //   out[scatter[i], :] = bf16( sum_k x[gather[i], k] * W[e(i)][k, :] )       (expert_projection)
 //   hidden[i, :] = swiglu(x[gather[i]] @ Wg[e], x[gather[i]] @ Wu[e])        (paired gate/up + epilogue)
 //
-// Work decomposition: a 256-thread block (4 wavefronts, 2 x 2) owns a 128-row x 128-column tile of one
-// expert's group (two such tiles, gate and up, when paired) and walks the depth in 64-deep steps. Tiles are
-// enumerated on the device from `offsets` (no host read of the routing): block (x, y) takes m-tile x of
-// column strip y; experts with no rows own no tiles. Global loads of step t+1 are in flight while step t
-// multiplies out of LDS. LDS rows are 128 bytes (64 bf16) with the 16-byte chunk index xor-swizzled by a
-// function of the row (`swizzled`), which makes both the ds_write_b128 of the loaders and the ds_read_b128
-// of the MFMA operand fetch conflict-free.
+// Work decomposition: a 256-thread block (4 wavefronts, 2 x 2) owns a BM-row x BN-column tile of one expert's
+// group (two such tiles, gate and up, when paired) and walks the depth in 64-deep steps. Tiles are enumerated
+// on the device from `offsets` (no host read of the routing); experts with no rows own no tiles.
+//
+// Operand paths, shaped by what the LDS of this chip costs (measured: ds_read_b128 ~230 B/clk a CU,
+// ds_write_b128 ~70 B/clk):
+//   A (activation rows, gathered by index): global -> registers (two steps ahead) -> LDS (two stages, 128-byte
+//     rows, chunk index xor-swizzled so stores and fragment reads are conflict-free) -> ds_read_b128 fragments.
+//   B (weights): never touch the LDS. The prepared bank is in MFMA-fragment order, so each wavefront loads the
+//     16-byte pieces of its own 32-column tiles straight from global memory (1 KiB coalesced per load) and
+//     dequantizes one 16-deep slice at a time in the shadow of the previous slice's matrix instructions.
+//     A lane's 16 bytes hold a run of consecutive depths, so the depth order inside a 64-deep step is permuted
+//     (the same permutation on the A side: only the LDS chunk a lane reads changes).
 #include <type_traits>
 
 #include "common.h"
@@ -48,8 +54,8 @@ struct GemmParams {
 // f(row) = ((row >> 1) & 7) ^ ((row & 1) << 2), chosen against the measured service order of gfx950's LDS:
 // ds_read_b128 serves 16 lanes a pass over 64 banks, the passes being lanes {0-3,12-15,20-23,24-27},
 // {4-7,8-11,16-19,28-31} and the same + 32; ds_write_b128 serves 8 consecutive lanes a pass over 128 bytes.
-// With lane = row (mod 32) on the read side and on the weight-store side, f is injective on every read pass's
-// rows of one parity and on every aligned run of 8 rows, so fragment reads and both stores are conflict-free.
+// With lane = row (mod 32) on the read side, f is injective on every read pass's rows of one parity, and a
+// store pass writes the 8 chunks of one row, so fragment reads and stores are conflict-free.
 __device__ __forceinline__ int swizzled(int row, int chunk) {
   return row * kChunksPerRow + (chunk ^ (((row >> 1) & 7) ^ ((row & 1) << 2)));
 }
@@ -59,55 +65,32 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
   return __builtin_bit_cast(uint32_t, pair);
 }
 
-// 16 e4m3 codes times one fp32 scale -> 16 bf16 (two LDS chunks): bf16(f32(code) * scale), the value the
-// reference's dequantize-then-cast produces (src/dew/interop/codecs.py:670-703; gemm.py:1067-1071).
-__device__ __forceinline__ void dequant_fp8(const u32x4_t& raw, float scale, u32x4_t (&out)[2]) {
-  const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
-  uint32_t packed[8];
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    const f32x2_t lo = __builtin_amdgcn_cvt_pk_f32_fp8(words[q], false);
-    const f32x2_t hi = __builtin_amdgcn_cvt_pk_f32_fp8(words[q], true);
-    packed[2 * q] = pack_bf16(lo.x * scale, lo.y * scale);
-    packed[2 * q + 1] = pack_bf16(hi.x * scale, hi.y * scale);
-  }
-  out[0] = u32x4_t{packed[0], packed[1], packed[2], packed[3]};
-  out[1] = u32x4_t{packed[4], packed[5], packed[6], packed[7]};
+// Eight e4m3 codes (two dwords) times one fp32 scale -> one bf16x8 fragment: bf16(f32(code) * scale), the
+// value the reference's dequantize-then-cast produces (src/dew/interop/codecs.py:670-703; gemm.py:1067-1071).
+__device__ __forceinline__ bf16x8_t fragment_fp8(uint32_t w0, uint32_t w1, float scale) {
+  const f32x2_t a = __builtin_amdgcn_cvt_pk_f32_fp8(w0, false), b = __builtin_amdgcn_cvt_pk_f32_fp8(w0, true);
+  const f32x2_t c = __builtin_amdgcn_cvt_pk_f32_fp8(w1, false), d = __builtin_amdgcn_cvt_pk_f32_fp8(w1, true);
+  return __builtin_bit_cast(bf16x8_t, u32x4_t{pack_bf16(a.x * scale, a.y * scale), pack_bf16(b.x * scale, b.y * scale),
+                                              pack_bf16(c.x * scale, c.y * scale), pack_bf16(d.x * scale, d.y * scale)});
 }
 
-// 32 E2M1 nibbles under two e4m3 block scales (each already over 2^8) -> 32 bf16 (four LDS chunks): each
+// Eight E2M1 nibbles (one dword) under one e4m3 block scale already over 2^8 -> one bf16x8 fragment; each
 // product code * scale / 2^8 is exact in bf16 (src/dew/nn/kernels/formats.py:108-113).
-__device__ __forceinline__ void dequant_fp4(const u32x4_t& raw, float scale0, float scale1, u32x4_t (&out)[4]) {
-  const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
-  uint32_t packed[16];
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    const float scale = q < 2 ? scale0 : scale1;
-    const f32x2_t b0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(words[q], 1.0f, 0);
-    const f32x2_t b1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(words[q], 1.0f, 1);
-    const f32x2_t b2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(words[q], 1.0f, 2);
-    const f32x2_t b3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(words[q], 1.0f, 3);
-    packed[4 * q] = pack_bf16(b0.x * scale, b0.y * scale);
-    packed[4 * q + 1] = pack_bf16(b1.x * scale, b1.y * scale);
-    packed[4 * q + 2] = pack_bf16(b2.x * scale, b2.y * scale);
-    packed[4 * q + 3] = pack_bf16(b3.x * scale, b3.y * scale);
-  }
-#pragma unroll
-  for (int c = 0; c < 4; ++c) out[c] = u32x4_t{packed[4 * c], packed[4 * c + 1], packed[4 * c + 2], packed[4 * c + 3]};
+__device__ __forceinline__ bf16x8_t fragment_fp4(uint32_t word, float scale) {
+  const f32x2_t a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 0), b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 1);
+  const f32x2_t c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 3);
+  return __builtin_bit_cast(bf16x8_t, u32x4_t{pack_bf16(a.x * scale, a.y * scale), pack_bf16(b.x * scale, b.y * scale),
+                                              pack_bf16(c.x * scale, c.y * scale), pack_bf16(d.x * scale, d.y * scale)});
 }
 
 // The same for a bank whose block scales are all powers of two (an MXFP4 checkpoint's): the hardware
 // conversion applies the scale's exponent itself, one instruction for two codes, exactly.
-__device__ __forceinline__ void dequant_fp4_pow2(const u32x4_t& raw, float scale0, float scale1, u32x4_t (&out)[4]) {
-  const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    const float scale = q < 2 ? scale0 : scale1;
-    out[q] = u32x4_t{__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(words[q], scale, 0)),
-                     __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(words[q], scale, 1)),
-                     __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(words[q], scale, 2)),
-                     __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(words[q], scale, 3))};
-  }
+__device__ __forceinline__ bf16x8_t fragment_fp4_pow2(uint32_t word, float scale) {
+  return __builtin_bit_cast(bf16x8_t, u32x4_t{
+      __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 0)),
+      __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 1)),
+      __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 2)),
+      __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 3))});
 }
 
 // Instruction order of one phase of the main loop, stated to the scheduler: `MFMAS` matrix instructions in a
@@ -135,15 +118,14 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4;
   constexpr bool kPow2 = FORMAT == DEW_MOE_W_MXFP4;
   constexpr int kMatrices = PAIRED ? 2 : 1;
-  constexpr int kAtomK = kFp4 ? 64 : 32;                       // depth an atom covers
-  constexpr int kAtomsPerStep = (BN / 32) * (BK / kAtomK);     // per matrix
-  constexpr int kLoads = kAtomsPerStep * kMatrices / 4;        // 16-byte loads a lane issues per step
-  constexpr int kChunksPerLoad = kFp4 ? 4 : 2;
-  constexpr int kRowLoads = BM / 32;                           // A rows a lane loads per step
-  constexpr int TI = BM / 64, TJ = BN / 64;                    // MFMA tiles per wavefront: rows, columns
-  constexpr int kStageChunks = (BM + kMatrices * BN) * kChunksPerRow;
+  constexpr int kAtomK = kFp4 ? 64 : 32;       // depth an atom covers
+  constexpr int kAtoms = BK / kAtomK;          // 16-byte loads a lane makes per 32-column tile per step
+  constexpr int kRowLoads = BM / 32;           // A rows a lane loads per step
+  constexpr int TI = BM / 64, TJ = BN / 64;    // MFMA tiles per wavefront: rows, columns of each matrix
+  constexpr int kTiles = kMatrices * TJ;       // weight tiles a wavefront multiplies
+  constexpr int kStageChunks = BM * kChunksPerRow;
 
-  extern __shared__ u32x4_t lds[];  // two stages of [A: BM rows][B: kMatrices x BN rows], 128-byte rows
+  extern __shared__ u32x4_t lds[];  // two stages of A: BM rows of 128 bytes each
   __shared__ int wave_tiles[4];
   __shared__ int found[3];  // expert, first sorted row of the tile, total m-tiles
 
@@ -211,6 +193,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   const int row0 = found[1];
   const int valid_rows = min(BM, p.offsets[expert + 1] - row0);
   const int steps = p.depth / BK;
+  const int wm0 = (wave / 2) * (BM / 2), wn0 = (wave % 2) * (BN / 2);
 
   // ---- A loader: 16-byte chunk `a_chunk` of rows a_row + 32 i ----
   const int a_chunk = tid % kChunksPerRow, a_row = tid / kChunksPerRow;
@@ -222,86 +205,82 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
     a_src[i] = reinterpret_cast<const u32x4_t*>(p.x + static_cast<size_t>(source) * p.depth) + a_chunk;
   }
 
-  // ---- B loader: atom `wave + 4 j` of the step: (matrix, n-atom, k-atom) ----
-  const uint8_t* b_src[kLoads];
-  const uint16_t* b_scale_src[kLoads];
-  float b_scale[kLoads];
-  int b_row[kLoads], b_first[kLoads];  // stage row and first 16-byte chunk the lane's dequantized values fill
-  const float* block_scales[kLoads];
+  // ---- B loader: tile t = (matrix, 32-column tile j of the wavefront); the lane's piece of each atom ----
+  const uint8_t* b_src[kTiles];
+  const uint16_t* b_scale_src[kTiles];  // FP4: the lane's two e4m3 block scales of each atom
+  const float* block_scales[kTiles];    // FP8 block: the tile's column of 128 x 128 scales
+  float channel_scale[kTiles];          // FP8 channel: the lane's column scale
   const int n_atoms = p.width / 32, k_atoms = p.depth / kAtomK;
 #pragma unroll
-  for (int j = 0; j < kLoads; ++j) {
-    const int atom = wave + 4 * j;
-    const int matrix = atom / kAtomsPerStep;
-    const int slot = atom % kAtomsPerStep;
-    const int na = slot / (BK / kAtomK), ka = slot % (BK / kAtomK);
+  for (int t = 0; t < kTiles; ++t) {
+    const int matrix = t / TJ, column = n0 + wn0 + 32 * (t % TJ);
     const uint8_t* codes = matrix == 0 ? p.w0.codes : p.w1.codes;
     const void* scales = matrix == 0 ? p.w0.scales : p.w1.scales;
-    const size_t first_atom = (static_cast<size_t>(expert) * n_atoms + n0 / 32 + na) * k_atoms + ka;
-    b_src[j] = codes + first_atom * kAtomBytes + lane * 16;
-    b_row[j] = BM + matrix * BN + na * 32 + lane % 32;  // rows of a stage: A first, then each matrix
-    b_first[j] = ka * (kAtomK / 8) + (lane / 32) * kChunksPerLoad;
-    b_scale[j] = 1.0f;
-    b_scale_src[j] = nullptr;
-    block_scales[j] = nullptr;
+    const size_t first_atom = (static_cast<size_t>(expert) * n_atoms + column / 32) * k_atoms;
+    b_src[t] = codes + first_atom * kAtomBytes + lane * 16;
+    b_scale_src[t] = nullptr;
+    block_scales[t] = nullptr;
+    channel_scale[t] = 1.0f;
     if (kFp4) {
-      b_scale_src[j] = static_cast<const uint16_t*>(scales) + first_atom * 64 + lane;
+      b_scale_src[t] = static_cast<const uint16_t*>(scales) + first_atom * 64 + lane;
     } else if (FORMAT == DEW_MOE_W_FP8_CHANNEL) {
-      b_scale[j] = static_cast<const float*>(scales)[static_cast<size_t>(expert) * p.width + n0 + na * 32 + lane % 32];
+      channel_scale[t] = static_cast<const float*>(scales)[static_cast<size_t>(expert) * p.width + column + lane % 32];
     } else {
-      block_scales[j] = static_cast<const float*>(scales) +
-                        static_cast<size_t>(expert) * (p.depth / 128) * (p.width / 128) + (n0 + na * 32) / 128;
+      block_scales[t] = static_cast<const float*>(scales) + static_cast<size_t>(expert) * (p.depth / 128) * (p.width / 128) + column / 128;
     }
   }
-  // Two register sets hold the raw global data of two steps, so every load has two steps to land.
-  u32x4_t a_regs[2][kRowLoads], b_regs[2][kLoads];
-  uint32_t s_regs[2][kLoads];  // FP4: the lane's two e4m3 scale bytes in the low half (the high half is the next lane's)
-  auto load_a = [&](auto set, int step) __attribute__((always_inline)) {
+
+  // Raw global data in flight: two register sets each for A (steps s + 1, s + 2) and B (steps s, s + 1).
+  u32x4_t a_regs[2][kRowLoads], b_regs[2][kTiles][kAtoms];
+  uint32_t s_regs[2][kTiles];  // FP4: two e4m3 scale bytes in the low half; FP8 block: the fp32 scale's bits
+  auto load_a = [&](auto set, int step, auto begin, auto end) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < kRowLoads; ++i) a_regs[set.value][i] = a_src[i][static_cast<size_t>(step) * kChunksPerRow];
+    for (int i = begin.value; i < end.value; ++i) a_regs[set.value][i] = a_src[i][static_cast<size_t>(step) * kChunksPerRow];
+  };
+  auto store_a = [&](auto set, u32x4_t* stage, auto begin, auto end) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = begin.value; i < end.value; ++i) stage[swizzled(a_row + 32 * i, a_chunk)] = a_regs[set.value][i];
   };
   auto load_b = [&](auto set, int step) __attribute__((always_inline)) {
 #pragma unroll
-    for (int j = 0; j < kLoads; ++j) {
-      b_regs[set.value][j] = *reinterpret_cast<const u32x4_t*>(b_src[j] + static_cast<size_t>(step) * (BK / kAtomK) * kAtomBytes);
+    for (int t = 0; t < kTiles; ++t) {
+#pragma unroll
+      for (int a = 0; a < kAtoms; ++a)
+        b_regs[set.value][t][a] = *reinterpret_cast<const u32x4_t*>(b_src[t] + (static_cast<size_t>(step) * kAtoms + a) * kAtomBytes);
       if (kFp4) {
-        __builtin_memcpy(&s_regs[set.value][j], b_scale_src[j] + static_cast<size_t>(step) * (BK / kAtomK) * 64, sizeof(uint32_t));
+        __builtin_memcpy(&s_regs[set.value][t], b_scale_src[t] + static_cast<size_t>(step) * 64, sizeof(uint32_t));
       } else if (FORMAT == DEW_MOE_W_FP8_BLOCK) {
-        s_regs[set.value][j] = __float_as_uint(block_scales[j][static_cast<size_t>((step * BK) / 128) * (p.width / 128)]);
+        s_regs[set.value][t] = __float_as_uint(block_scales[t][static_cast<size_t>((step * BK) / 128) * (p.width / 128)]);
       }
     }
   };
 
-  auto store_a = [&](auto set, u32x4_t* stage) __attribute__((always_inline)) {
+  // ---- fragments: slice kk of a step is 16 depths; a lane's are the 8 its weight bytes cover ----
+  bf16x8_t a_frag[2][TI], b_frag[2][kTiles];
+  float fp4_scale[kTiles];
+  auto fetch = [&](const u32x4_t* stage, auto kk, auto into) __attribute__((always_inline)) {
+    const int chunk = kFp4 ? 4 * (lane / 32) + kk.value : 4 * (kk.value / 2) + 2 * (lane / 32) + kk.value % 2;
 #pragma unroll
-    for (int i = 0; i < kRowLoads; ++i) stage[swizzled(a_row + 32 * i, a_chunk)] = a_regs[set.value][i];
+    for (int i = 0; i < TI; ++i)
+      a_frag[into.value][i] = __builtin_bit_cast(bf16x8_t, stage[swizzled(wm0 + 32 * i + lane % 32, chunk)]);
   };
-  auto store_b = [&](auto set, u32x4_t* stage) __attribute__((always_inline)) {
+  auto dequantize = [&](auto set, auto kk, auto into) __attribute__((always_inline)) {
 #pragma unroll
-    for (int j = 0; j < kLoads; ++j) {
-      if (kFp4) {
-        const float scale0 = __builtin_amdgcn_cvt_f32_fp8(s_regs[set.value][j], 0) * 0.00390625f;
-        const float scale1 = __builtin_amdgcn_cvt_f32_fp8(s_regs[set.value][j], 1) * 0.00390625f;
-        u32x4_t chunks[4];
-        if (kPow2) {
-          dequant_fp4_pow2(b_regs[set.value][j], scale0, scale1, chunks);
-        } else {
-          dequant_fp4(b_regs[set.value][j], scale0, scale1, chunks);
-        }
-#pragma unroll
-        for (int c = 0; c < 4; ++c) stage[swizzled(b_row[j], b_first[j] + c)] = chunks[c];
+    for (int t = 0; t < kTiles; ++t) {
+      if constexpr (kFp4) {
+        if constexpr (kk.value % 2 == 0)  // slices 0, 1 lie in the lane's first 16-deep block, 2, 3 in its second
+          fp4_scale[t] = (kk.value == 0 ? __builtin_amdgcn_cvt_f32_fp8(s_regs[set.value][t], 0)
+                                        : __builtin_amdgcn_cvt_f32_fp8(s_regs[set.value][t], 1)) * 0.00390625f;
+        const uint32_t word = b_regs[set.value][t][0][kk.value];
+        b_frag[into.value][t] = kPow2 ? fragment_fp4_pow2(word, fp4_scale[t]) : fragment_fp4(word, fp4_scale[t]);
       } else {
-        const float scale = FORMAT == DEW_MOE_W_FP8_BLOCK ? __uint_as_float(s_regs[set.value][j]) : b_scale[j];
-        u32x4_t chunks[2];
-        dequant_fp8(b_regs[set.value][j], scale, chunks);
-#pragma unroll
-        for (int c = 0; c < 2; ++c) stage[swizzled(b_row[j], b_first[j] + c)] = chunks[c];
+        const float scale = FORMAT == DEW_MOE_W_FP8_BLOCK ? __uint_as_float(s_regs[set.value][t]) : channel_scale[t];
+        const u32x4_t& raw = b_regs[set.value][t][kk.value / 2 % kAtoms];
+        b_frag[into.value][t] = fragment_fp8(raw[2 * (kk.value % 2)], raw[2 * (kk.value % 2) + 1], scale);
       }
     }
   };
 
-  // ---- accumulators ----
-  const int wm0 = (wave / 2) * (BM / 2), wn0 = (wave % 2) * (BN / 2);
   f32x16_t acc[kMatrices][TI][TJ];
 #pragma unroll
   for (int m = 0; m < kMatrices; ++m)
@@ -311,87 +290,83 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
       for (int j = 0; j < TJ; ++j)
 #pragma unroll
         for (int q = 0; q < 16; ++q) acc[m][i][j][q] = 0.0f;
-
-  // Operand fragments are double-buffered in registers: while the matrix cores work on one 16-deep slice,
-  // the next slice's ds_read_b128s are in flight.
-  bf16x8_t a_frag[2][TI], b_frag[2][kMatrices][TJ];
-  auto fetch = [&](const u32x4_t* stage, int kk, int set) __attribute__((always_inline)) {
-    const int chunk = 2 * kk + lane / 32;
-#pragma unroll
-    for (int i = 0; i < TI; ++i)
-      a_frag[set][i] = __builtin_bit_cast(bf16x8_t, stage[swizzled(wm0 + 32 * i + lane % 32, chunk)]);
-#pragma unroll
-    for (int m = 0; m < kMatrices; ++m)
-#pragma unroll
-      for (int j = 0; j < TJ; ++j)
-        b_frag[set][m][j] = __builtin_bit_cast(bf16x8_t, stage[swizzled(BM + m * BN + wn0 + 32 * j + lane % 32, chunk)]);
-  };
-  auto multiply = [&](int set) __attribute__((always_inline)) {
+  auto multiply = [&](auto from) __attribute__((always_inline)) {
 #pragma unroll
     for (int m = 0; m < kMatrices; ++m)
 #pragma unroll
       for (int i = 0; i < TI; ++i)
 #pragma unroll
         for (int j = 0; j < TJ; ++j)
-          acc[m][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_frag[set][i], b_frag[set][m][j], acc[m][i][j], 0, 0, 0);
+          acc[m][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_frag[from.value][i], b_frag[from.value][m * TJ + j], acc[m][i][j], 0, 0, 0);
   };
 
-  // ---- pipeline. At the top of step s: LDS stage s & 1 holds step s; register set (s + 1) & 1 holds the raw
-  // data of step s + 1 and set s & 1 that of step s + 2. During step s the set (s + 1) & 1 is stored to the
-  // other stage (weights dequantized on the way) and at once reloaded with step s + 3, two steps ahead of
-  // its use. One barrier a step: the stage written during step s was last read before the barrier of step
-  // s - 1. The loop is unrolled by two so that stages and register sets are compile-time constants.
-  constexpr std::integral_constant<int, 0> even{};
-  constexpr std::integral_constant<int, 1> odd{};
-  constexpr int kMfmas = kMatrices * TI * TJ, kReads = TI + kMatrices * TJ;
-  constexpr int kStoresB = kLoads * kChunksPerLoad;
-  constexpr int kDequantOps = kPow2 ? kLoads * 22 : (kFp4 ? kLoads * 70 : kLoads * 34);
-  constexpr int kLoadsB = kLoads * (kFp4 || FORMAT == DEW_MOE_W_FP8_BLOCK ? 2 : 1);
+  // ---- pipeline. At the top of step s: LDS stage s & 1 holds the A rows of step s; A register set (s + 1) & 1
+  // holds step s + 1 and set s & 1 step s + 2; B register set s & 1 holds step s and set (s + 1) & 1 step s + 1.
+  // A step is four phases, one 16-deep slice each: the slice multiplies while the next slice's A fragments are
+  // read from LDS and its B fragments dequantized; phases 1-3 also move the A rows of step s + 1 to the other
+  // stage and reload their registers with step s + 3; phase 4 reloads the B set of step s with step s + 2.
+  // One barrier a step: the stage written during step s was last read before the barrier of step s - 1.
+  // The loop is unrolled by two so that stages and register sets are compile-time constants.
+  constexpr std::integral_constant<int, 0> c0{};
+  constexpr std::integral_constant<int, 1> c1{};
+  constexpr std::integral_constant<int, 2> c2{};
+  constexpr std::integral_constant<int, 3> c3{};
+  constexpr std::integral_constant<int, (kRowLoads + 2) / 3> a_first{};
+  constexpr std::integral_constant<int, (2 * kRowLoads + 2) / 3> a_second{};
+  constexpr std::integral_constant<int, kRowLoads> a_end{};
+  constexpr int kMfmas = kMatrices * TI * TJ;
+  constexpr int kDequantOps = kTiles * (kPow2 ? 5 : 17);  // vector instructions to dequantize one slice
+  constexpr int kA1 = a_first.value, kA2 = a_second.value - a_first.value, kA3 = kRowLoads - a_second.value;
+  constexpr int kLoadsB = kTiles * (kAtoms + (kFp4 || FORMAT == DEW_MOE_W_FP8_BLOCK ? 1 : 0));
   auto iterate = [&](auto parity, int step) __attribute__((always_inline)) {
     constexpr std::integral_constant<int, 1 - parity.value> other{};
     u32x4_t* current = lds + parity.value * kStageChunks;
     u32x4_t* next = lds + other.value * kStageChunks;
-    const int ahead = min(step + 3, steps - 1);
-    // phase 1: slice 0 multiplies; slice 1's operands are read; the A rows of step + 1 go to the other
-    // stage and their registers are reloaded
-    fetch(current, 1, 1);
-    multiply(0);
-    store_a(other, next);
-    load_a(other, ahead);
-    schedule_phase<0, kMfmas, kReads, kRowLoads, 2 * kRowLoads, kRowLoads>();
+    const int ahead_a = min(step + 3, steps - 1), ahead_b = min(step + 2, steps - 1);
+    fetch(current, c1, c1);
+    dequantize(parity, c1, c1);
+    multiply(c0);
+    store_a(other, next, c0, a_first);
+    load_a(other, ahead_a, c0, a_first);
+    schedule_phase<0, kMfmas, TI, kA1, kDequantOps + 2 * kA1, kA1>();
     __builtin_amdgcn_sched_barrier(0);
-    // phase 2: slice 1 multiplies; the weights of step + 1 are dequantized and stored, their registers reloaded
-    fetch(current, 2, 0);
-    multiply(1);
-    store_b(other, next);
-    load_b(other, ahead);
-    schedule_phase<0, kMfmas, kReads, kStoresB, kDequantOps + kLoadsB, kLoadsB>();
+
+    fetch(current, c2, c0);
+    dequantize(parity, c2, c0);
+    multiply(c1);
+    store_a(other, next, a_first, a_second);
+    load_a(other, ahead_a, a_first, a_second);
+    schedule_phase<0, kMfmas, TI, kA2, kDequantOps + 2 * kA2, kA2>();
     __builtin_amdgcn_sched_barrier(0);
-    // phase 3: slice 2 multiplies
-    fetch(current, 3, 1);
-    multiply(0);
-    schedule_phase<0, kMfmas, kReads, 0, 0, 0>();
+
+    fetch(current, c3, c1);
+    dequantize(parity, c3, c1);
+    multiply(c0);
+    store_a(other, next, a_second, a_end);
+    load_a(other, ahead_a, a_second, a_end);
+    schedule_phase<0, kMfmas, TI, kA3, kDequantOps + 2 * kA3, kA3>();
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
-    // phase 4: slice 3 multiplies; the first operands of the next stage are read
-    fetch(next, 0, 0);
-    multiply(1);
-    schedule_phase<0, kMfmas, kReads, 0, 0, 0>();
+
+    fetch(next, c0, c0);
+    dequantize(other, c0, c0);
+    multiply(c1);
+    load_b(parity, ahead_b);
+    schedule_phase<0, kMfmas, TI, 0, kDequantOps + kLoadsB, kLoadsB>();
     __builtin_amdgcn_sched_barrier(0);
   };
-  load_a(even, 0);
-  load_b(even, 0);
-  store_a(even, lds);
-  store_b(even, lds);
-  load_a(odd, min(1, steps - 1));
-  load_b(odd, min(1, steps - 1));
-  load_a(even, min(2, steps - 1));
-  load_b(even, min(2, steps - 1));
+  load_a(c0, 0, c0, a_end);
+  load_b(c0, 0);
+  load_b(c1, min(1, steps - 1));
+  store_a(c0, lds, c0, a_end);
+  load_a(c1, min(1, steps - 1), c0, a_end);
+  load_a(c0, min(2, steps - 1), c0, a_end);
   __syncthreads();
-  fetch(lds, 0, 0);
+  fetch(lds, c0, c0);
+  dequantize(c0, c0, c0);
   for (int step = 0; step < steps; step += 2) {  // depth is whole 128s, so steps is even
-    iterate(even, step);
-    iterate(odd, step + 1);
+    iterate(c0, step);
+    iterate(c1, step + 1);
   }
 
   // ---- epilogue: acc[..][q] is row 8 (q / 4) + 4 (lane / 32) + q % 4, column lane % 32 of its 32 x 32 tile.
@@ -448,8 +423,7 @@ static int check_bank(const char* who, const dew_moe_bank* bank, const char* nam
 
 template <int FORMAT, bool PAIRED, int BM, int BN>
 static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
-  constexpr int kMatrices = PAIRED ? 2 : 1;
-  constexpr size_t kShared = 2 * static_cast<size_t>(BM + kMatrices * BN) * BK * sizeof(bf16_t);
+  constexpr size_t kShared = 2 * static_cast<size_t>(BM) * BK * sizeof(bf16_t);
   auto kernel = grouped_gemm_kernel<FORMAT, PAIRED, BM, BN>;
   static bool configured = false;  // dynamic LDS above 64 KiB must be opted into once per kernel
   if (!configured) {
@@ -470,7 +444,8 @@ static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
 // tiles when the average group fills them, the 128 x 128 tile otherwise.
 template <int FORMAT, bool PAIRED>
 static int launch_format(const char* who, const GemmParams& p, hipStream_t stream) {
-  const bool large = p.rows / p.experts >= 768 && p.width % 256 == 0;
+  constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4;  // FP8's raw registers do not fit the large tile
+  const bool large = kFp4 && p.rows / p.experts >= 768 && p.width % 256 == 0;
   if (PAIRED) {
     if (large) return launch_tile<FORMAT, true, 256, 128>(who, p, stream);
     return launch_tile<FORMAT, true, 128, 128>(who, p, stream);
