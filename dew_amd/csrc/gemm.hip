@@ -11,8 +11,9 @@
 //
 // Operand paths, shaped by what the LDS of this chip costs (measured: ds_read_b128 ~230 B/clk a CU,
 // ds_write_b128 ~70 B/clk):
-//   A (activation rows, gathered by index): global -> registers (two steps ahead) -> LDS (two stages, 128-byte
-//     rows, chunk index xor-swizzled so stores and fragment reads are conflict-free) -> ds_read_b128 fragments.
+//   A (activation rows, gathered by index): global -> LDS directly (global_load_lds_dwordx4, no registers and
+//     no ds_write, two steps ahead into a ring of three stages; 128-byte rows, chunk index xor-swizzled so
+//     the fragment reads are conflict-free) -> ds_read_b128 fragments.
 //   B (weights): never touch the LDS. The prepared bank is in MFMA-fragment order, so each wavefront loads the
 //     16-byte pieces of its own 32-column tiles straight from global memory (1 KiB coalesced per load) and
 //     dequantizes one 16-deep slice at a time in the shadow of the previous slice's matrix instructions.
@@ -124,8 +125,9 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   constexpr int TI = BM / 64, TJ = BN / 64;    // MFMA tiles per wavefront: rows, columns of each matrix
   constexpr int kTiles = kMatrices * TJ;       // weight tiles a wavefront multiplies
   constexpr int kStageChunks = BM * kChunksPerRow;
+  constexpr int kStages = 3;
 
-  extern __shared__ u32x4_t lds[];  // two stages of A: BM rows of 128 bytes each
+  extern __shared__ u32x4_t lds[];  // a ring of three stages of A: BM rows of 128 bytes each
   __shared__ int wave_tiles[4];
   __shared__ int found[3];  // expert, first sorted row of the tile, total m-tiles
 
@@ -195,15 +197,26 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   const int steps = p.depth / BK;
   const int wm0 = (wave / 2) * (BM / 2), wn0 = (wave % 2) * (BN / 2);
 
-  // ---- A loader: 16-byte chunk `a_chunk` of rows a_row + 32 i ----
-  const int a_chunk = tid % kChunksPerRow, a_row = tid / kChunksPerRow;
-  const u32x4_t* a_src[kRowLoads];
+  // ---- A loader. One global_load_lds_dwordx4 of a wavefront fills 1 KiB of LDS, lane l landing at byte 16 l:
+  // 8 rows of a stage, lane l = row l / 8, stored chunk l % 8. The lane therefore fetches the logical chunk
+  // that the swizzle keeps at that place. Wavefront w issues the loads of rows 8 (w kRowLoads + i) .. + 7.
+  const bf16_t* a_src[kRowLoads];
 #pragma unroll
   for (int i = 0; i < kRowLoads; ++i) {
-    const int sorted = row0 + min(a_row + 32 * i, valid_rows - 1);
+    const int row = (wave * kRowLoads + i) * 8 + lane / 8;
+    const int chunk = (lane % 8) ^ (((row >> 1) & 7) ^ ((row & 1) << 2));
+    const int sorted = row0 + min(row, valid_rows - 1);
     const int source = p.gather ? p.gather[sorted] : sorted;
-    a_src[i] = reinterpret_cast<const u32x4_t*>(p.x + static_cast<size_t>(source) * p.depth) + a_chunk;
+    a_src[i] = p.x + static_cast<size_t>(source) * p.depth + chunk * 8;
   }
+  auto load_a = [&](u32x4_t* stage, int step, auto begin, auto end) __attribute__((always_inline)) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass, which only needs the kernel's stub, does not know the builtin
+#pragma unroll
+    for (int i = begin.value; i < end.value; ++i)
+      __builtin_amdgcn_global_load_lds(a_src[i] + static_cast<size_t>(step) * BK,
+                                       (__attribute__((address_space(3))) void*)(stage + (wave * kRowLoads + i) * 64), 16, 0, 0);
+#endif
+  };
 
   // ---- B loader: tile t = (matrix, 32-column tile j of the wavefront); the lane's piece of each atom ----
   const uint8_t* b_src[kTiles];
@@ -230,20 +243,12 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
     }
   }
 
-  // Raw global data in flight: two register sets each for A (steps s + 1, s + 2) and B (steps s, s + 1).
-  u32x4_t a_regs[2][kRowLoads], b_regs[2][kTiles][kAtoms];
-  uint32_t s_regs[2][kTiles];  // FP4: two e4m3 scale bytes in the low half; FP8 block: the fp32 scale's bits
-  auto load_a = [&](auto set, int step, auto begin, auto end) __attribute__((always_inline)) {
+  // Raw weight data in flight: four register sets (steps s .. s + 3), so a load has two to three steps to land.
+  u32x4_t b_regs[4][kTiles][kAtoms];
+  uint32_t s_regs[4][kTiles];  // FP4: two e4m3 scale bytes in the low half; FP8 block: the fp32 scale's bits
+  auto load_b = [&](auto set, int step, auto begin, auto end) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = begin.value; i < end.value; ++i) a_regs[set.value][i] = a_src[i][static_cast<size_t>(step) * kChunksPerRow];
-  };
-  auto store_a = [&](auto set, u32x4_t* stage, auto begin, auto end) __attribute__((always_inline)) {
-#pragma unroll
-    for (int i = begin.value; i < end.value; ++i) stage[swizzled(a_row + 32 * i, a_chunk)] = a_regs[set.value][i];
-  };
-  auto load_b = [&](auto set, int step) __attribute__((always_inline)) {
-#pragma unroll
-    for (int t = 0; t < kTiles; ++t) {
+    for (int t = begin.value; t < end.value; ++t) {
 #pragma unroll
       for (int a = 0; a < kAtoms; ++a)
         b_regs[set.value][t][a] = *reinterpret_cast<const u32x4_t*>(b_src[t] + (static_cast<size_t>(step) * kAtoms + a) * kAtomBytes);
@@ -300,74 +305,111 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
           acc[m][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_frag[from.value][i], b_frag[from.value][m * TJ + j], acc[m][i][j], 0, 0, 0);
   };
 
-  // ---- pipeline. At the top of step s: LDS stage s & 1 holds the A rows of step s; A register set (s + 1) & 1
-  // holds step s + 1 and set s & 1 step s + 2; B register set s & 1 holds step s and set (s + 1) & 1 step s + 1.
-  // A step is four phases, one 16-deep slice each: the slice multiplies while the next slice's A fragments are
-  // read from LDS and its B fragments dequantized; phases 1-3 also move the A rows of step s + 1 to the other
-  // stage and reload their registers with step s + 3; phase 4 reloads the B set of step s with step s + 2.
-  // One barrier a step: the stage written during step s was last read before the barrier of step s - 1.
-  // The loop is unrolled by two so that stages and register sets are compile-time constants.
+  // ---- pipeline. At the top of step s: LDS stage s % 3 holds the A rows of step s and the loads of step s + 1
+  // into stage (s + 1) % 3 are in flight; B register sets s % 4 .. (s + 2) % 4 hold (or are receiving) steps
+  // s .. s + 2. A step is four phases, one 16-deep slice each: the slice multiplies while the next slice's A
+  // fragments are read from LDS and its B fragments dequantized. Each phase also issues a quarter of the step's
+  // global loads, so the memory pipeline sees an even stream: A rows of step s + 2 into stage (s + 2) % 3 (last
+  // read during step s - 1) and weights of step s + 3 into set (s + 3) % 4 (last read during step s - 1).
+  // One barrier a step, after phase 3: by then this wavefront's A loads of step s + 1 have landed (a vmcnt wait
+  // that leaves the younger loads in flight) and its own fragment reads are done, so after the barrier stage
+  // (s + 1) % 3 may be read and stage s % 3 overwritten. The loop is unrolled by four so that the B register
+  // sets are compile-time constants.
   constexpr std::integral_constant<int, 0> c0{};
   constexpr std::integral_constant<int, 1> c1{};
   constexpr std::integral_constant<int, 2> c2{};
   constexpr std::integral_constant<int, 3> c3{};
-  constexpr std::integral_constant<int, (kRowLoads + 2) / 3> a_first{};
-  constexpr std::integral_constant<int, (2 * kRowLoads + 2) / 3> a_second{};
-  constexpr std::integral_constant<int, kRowLoads> a_end{};
+  constexpr std::integral_constant<int, kRowLoads / 4> a1{};
+  constexpr std::integral_constant<int, 2 * kRowLoads / 4> a2{};
+  constexpr std::integral_constant<int, 3 * kRowLoads / 4> a3{};
+  constexpr std::integral_constant<int, kRowLoads> a4{};
+  constexpr std::integral_constant<int, kTiles / 4> b1{};
+  constexpr std::integral_constant<int, 2 * kTiles / 4> b2{};
+  constexpr std::integral_constant<int, 3 * kTiles / 4> b3{};
+  constexpr std::integral_constant<int, kTiles> b4{};
+  constexpr std::integral_constant<int, kTiles> all_tiles{};
   constexpr int kMfmas = kMatrices * TI * TJ;
   constexpr int kDequantOps = kTiles * (kPow2 ? 5 : 17);  // vector instructions to dequantize one slice
-  constexpr int kA1 = a_first.value, kA2 = a_second.value - a_first.value, kA3 = kRowLoads - a_second.value;
-  constexpr int kLoadsB = kTiles * (kAtoms + (kFp4 || FORMAT == DEW_MOE_W_FP8_BLOCK ? 1 : 0));
-  auto iterate = [&](auto parity, int step) __attribute__((always_inline)) {
-    constexpr std::integral_constant<int, 1 - parity.value> other{};
-    u32x4_t* current = lds + parity.value * kStageChunks;
-    u32x4_t* next = lds + other.value * kStageChunks;
-    const int ahead_a = min(step + 3, steps - 1), ahead_b = min(step + 2, steps - 1);
+  constexpr int kLoadsPerTile = kAtoms + (kFp4 || FORMAT == DEW_MOE_W_FP8_BLOCK ? 1 : 0);
+  constexpr int kLoadsPerPhase = (kRowLoads + 3) / 4 + ((kTiles + 3) / 4) * kLoadsPerTile;
+  // s_waitcnt vmcnt(kYounger) lgkmcnt(0): everything but the kYounger youngest vector-memory operations is done.
+  // Younger than the A loads of step s + 1 (the last of them issued in phase 4 of step s - 1) are at least the
+  // loads of phases 1-3 of step s.
+  constexpr int kYounger = a3.value + b3.value * kLoadsPerTile;
+  static_assert(kYounger < 64, "vmcnt is a 6-bit counter");
+  constexpr int kWaitLanded = (kYounger & 0xF) | (7 << 4) | (0 << 8) | ((kYounger >> 4) << 14);
+  constexpr int kWaitAll = (0 & 0xF) | (7 << 4) | (0 << 8) | (0 << 14);  // vmcnt(0) lgkmcnt(0)
+  int stage_index = 0;  // s % 3
+  auto iterate = [&](auto set, int step) __attribute__((always_inline)) {
+    constexpr std::integral_constant<int, (set.value + 1) % 4> following{};
+    constexpr std::integral_constant<int, (set.value + 3) % 4> filling{};
+    const int next_index = stage_index == kStages - 1 ? 0 : stage_index + 1;
+    const int fill_index = next_index == kStages - 1 ? 0 : next_index + 1;
+    u32x4_t* current = lds + stage_index * kStageChunks;
+    u32x4_t* next = lds + next_index * kStageChunks;
+    u32x4_t* fill = lds + fill_index * kStageChunks;
+    const int ahead_a = min(step + 2, steps - 1), ahead_b = min(step + 3, steps - 1);
     fetch(current, c1, c1);
-    dequantize(parity, c1, c1);
+    dequantize(set, c1, c1);
     multiply(c0);
-    store_a(other, next, c0, a_first);
-    load_a(other, ahead_a, c0, a_first);
-    schedule_phase<0, kMfmas, TI, kA1, kDequantOps + 2 * kA1, kA1>();
+    load_a(fill, ahead_a, c0, a1);
+    load_b(filling, ahead_b, c0, b1);
+    schedule_phase<0, kMfmas, TI, 0, kDequantOps + 2 * kLoadsPerPhase, kLoadsPerPhase>();
     __builtin_amdgcn_sched_barrier(0);
 
     fetch(current, c2, c0);
-    dequantize(parity, c2, c0);
+    dequantize(set, c2, c0);
     multiply(c1);
-    store_a(other, next, a_first, a_second);
-    load_a(other, ahead_a, a_first, a_second);
-    schedule_phase<0, kMfmas, TI, kA2, kDequantOps + 2 * kA2, kA2>();
+    load_a(fill, ahead_a, a1, a2);
+    load_b(filling, ahead_b, b1, b2);
+    schedule_phase<0, kMfmas, TI, 0, kDequantOps + 2 * kLoadsPerPhase, kLoadsPerPhase>();
     __builtin_amdgcn_sched_barrier(0);
 
     fetch(current, c3, c1);
-    dequantize(parity, c3, c1);
+    dequantize(set, c3, c1);
     multiply(c0);
-    store_a(other, next, a_second, a_end);
-    load_a(other, ahead_a, a_second, a_end);
-    schedule_phase<0, kMfmas, TI, kA3, kDequantOps + 2 * kA3, kA3>();
+    load_a(fill, ahead_a, a2, a3);
+    load_b(filling, ahead_b, b2, b3);
+    schedule_phase<0, kMfmas, TI, 0, kDequantOps + 2 * kLoadsPerPhase, kLoadsPerPhase>();
     __builtin_amdgcn_sched_barrier(0);
-    __syncthreads();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(kWaitLanded);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
 
     fetch(next, c0, c0);
-    dequantize(other, c0, c0);
+    dequantize(following, c0, c0);
     multiply(c1);
-    load_b(parity, ahead_b);
-    schedule_phase<0, kMfmas, TI, 0, kDequantOps + kLoadsB, kLoadsB>();
+    load_a(fill, ahead_a, a3, a4);
+    load_b(filling, ahead_b, b3, b4);
+    schedule_phase<0, kMfmas, TI, 0, kDequantOps + 2 * kLoadsPerPhase, kLoadsPerPhase>();
     __builtin_amdgcn_sched_barrier(0);
+    stage_index = next_index;
   };
-  load_a(c0, 0, c0, a_end);
-  load_b(c0, 0);
-  load_b(c1, min(1, steps - 1));
-  store_a(c0, lds, c0, a_end);
-  load_a(c1, min(1, steps - 1), c0, a_end);
-  load_a(c0, min(2, steps - 1), c0, a_end);
-  __syncthreads();
+  load_b(c0, 0, c0, all_tiles);
+  load_b(c1, min(1, steps - 1), c0, all_tiles);
+  load_b(c2, min(2, steps - 1), c0, all_tiles);
+  load_a(lds, 0, c0, a4);
+  load_a(lds + kStageChunks, min(1, steps - 1), c0, a4);
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(kWaitAll);
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
   fetch(lds, c0, c0);
   dequantize(c0, c0, c0);
-  for (int step = 0; step < steps; step += 2) {  // depth is whole 128s, so steps is even
+  int step = 0;
+  for (; step + 3 < steps; step += 4) {
+    iterate(c0, step);
+    iterate(c1, step + 1);
+    iterate(c2, step + 2);
+    iterate(c3, step + 3);
+  }
+  if (step < steps) {  // depth is whole 128s: an even number of steps, so the tail is two steps or none
     iterate(c0, step);
     iterate(c1, step + 1);
   }
+  __builtin_amdgcn_s_waitcnt(kWaitAll);  // the clamped tail loads still target the LDS
 
   // ---- epilogue: acc[..][q] is row 8 (q / 4) + 4 (lane / 32) + q % 4, column lane % 32 of its 32 x 32 tile.
   // Neighbouring lanes hold neighbouring columns: each pair of lanes swaps one value so that the even lane
@@ -423,7 +465,7 @@ static int check_bank(const char* who, const dew_moe_bank* bank, const char* nam
 
 template <int FORMAT, bool PAIRED, int BM, int BN>
 static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
-  constexpr size_t kShared = 2 * static_cast<size_t>(BM) * BK * sizeof(bf16_t);
+  constexpr size_t kShared = 3 * static_cast<size_t>(BM) * BK * sizeof(bf16_t);
   auto kernel = grouped_gemm_kernel<FORMAT, PAIRED, BM, BN>;
   static bool configured = false;  // dynamic LDS above 64 KiB must be opted into once per kernel
   if (!configured) {
