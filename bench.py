@@ -160,6 +160,8 @@ def main():
     parser.add_argument("--warmup", type=int, default=3)
     parser.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--graph", choices=["auto", "on", "off"], default="auto",
+                        help="replay the step as one captured HIP graph (auto: for the launch-bound configs c1 and c3)")
     args = parser.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (expert-parallel sharding is described "
@@ -178,14 +180,37 @@ def main():
     data = build_workload(case, device)
     stepper = Stepper(case, data)
 
+    graphed = args.graph == "on" or (args.graph == "auto" and args.config in ("c1", "c3"))
     for _ in range(args.warmup):
         stepper()
     torch.cuda.synchronize()
-    began = time.perf_counter()
-    for _ in range(args.steps):
-        out, plan = stepper(timed=True)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - began
+    if graphed:
+        # The step makes seven short launches; captured once, it replays as one graph with no host work between
+        # kernels. The launches themselves are the same C-ABI calls on the capture stream.
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out, plan = stepper()
+        graph.replay()
+        torch.cuda.synchronize()
+        began = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - began
+        # the dominant kernel's duration, by HIP events around eager launches of it on the same inputs
+        for _ in range(args.steps):
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            ops.gateup_swiglu(data["x"], stepper.gate, stepper.up, plan.offsets, gather=plan.rows)
+            stop.record()
+            stepper.events.append((start, stop))
+        torch.cuda.synchronize()
+    else:
+        began = time.perf_counter()
+        for _ in range(args.steps):
+            out, plan = stepper(timed=True)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - began
     ms_per_step = 1e3 * elapsed / args.steps
 
     routed_rows = case.tokens * case.top_k
@@ -218,7 +243,7 @@ def main():
         "config": {"workload": f"{args.config}: T={case.tokens} D={case.d_model} F={case.d_ff} E={case.experts} k={case.top_k} "
                                f"{case.quant} weights, {case.router['score_function']} router"
                                + (" + shared expert" if case.shared else ""),
-                   "routed_rows": routed_rows, "experts_touched": touched,
+                   "routed_rows": routed_rows, "experts_touched": touched, "launch": "hip graph replay" if graphed else "eager",
                    "algorithmic_flops": flops},
         "roofline": roofline,
     }

@@ -113,16 +113,18 @@ __device__ __forceinline__ void schedule_phase() {
 
 // One grouped-GEMM kernel, templated on the weight format, on whether two banks (gate, up) are multiplied in
 // the same launch with the SwiGLU epilogue, and on the block tile: BM rows x BN columns of each matrix. The
-// four wavefronts sit 2 x 2; each owns (BM/2) x (BN/2) of every matrix as 32 x 32 MFMA tiles.
-template <int FORMAT, bool PAIRED, int BM, int BN>
+// four wavefronts sit WM x WN (2 x 2, or 1 x 4 for the 32-row decode tile); each owns (BM/WM) x (BN/WN) of
+// every matrix as 32 x 32 MFMA tiles.
+template <int FORMAT, bool PAIRED, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
+  static_assert(WM * WN == 4 && BM % (32 * WM) == 0 && BN % (32 * WN) == 0 && BM % 32 == 0, "tile shape");
   constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4;
   constexpr bool kPow2 = FORMAT == DEW_MOE_W_MXFP4;
   constexpr int kMatrices = PAIRED ? 2 : 1;
   constexpr int kAtomK = kFp4 ? 64 : 32;       // depth an atom covers
   constexpr int kAtoms = BK / kAtomK;          // 16-byte loads a lane makes per 32-column tile per step
   constexpr int kRowLoads = BM / 32;           // A rows a lane loads per step
-  constexpr int TI = BM / 64, TJ = BN / 64;    // MFMA tiles per wavefront: rows, columns of each matrix
+  constexpr int TI = BM / (32 * WM), TJ = BN / (32 * WN);  // MFMA tiles per wavefront: rows, columns of each matrix
   constexpr int kTiles = kMatrices * TJ;       // weight tiles a wavefront multiplies
   constexpr int kStageChunks = BM * kChunksPerRow;
   constexpr int kStages = 3;
@@ -195,7 +197,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   const int row0 = found[1];
   const int valid_rows = min(BM, p.offsets[expert + 1] - row0);
   const int steps = p.depth / BK;
-  const int wm0 = (wave / 2) * (BM / 2), wn0 = (wave % 2) * (BN / 2);
+  const int wm0 = (wave / WN) * (BM / WM), wn0 = (wave % WN) * (BN / WN);
 
   // ---- A loader. One global_load_lds_dwordx4 of a wavefront fills 1 KiB of LDS, lane l landing at byte 16 l:
   // 8 rows of a stage, lane l = row l / 8, stored chunk l % 8. The lane therefore fetches the logical chunk
@@ -319,9 +321,9 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   constexpr std::integral_constant<int, 1> c1{};
   constexpr std::integral_constant<int, 2> c2{};
   constexpr std::integral_constant<int, 3> c3{};
-  constexpr std::integral_constant<int, kRowLoads / 4> a1{};
-  constexpr std::integral_constant<int, 2 * kRowLoads / 4> a2{};
-  constexpr std::integral_constant<int, 3 * kRowLoads / 4> a3{};
+  constexpr std::integral_constant<int, (kRowLoads + 3) / 4> a1{};  // A loads early in the step, weights late
+  constexpr std::integral_constant<int, (2 * kRowLoads + 3) / 4> a2{};
+  constexpr std::integral_constant<int, (3 * kRowLoads + 3) / 4> a3{};
   constexpr std::integral_constant<int, kRowLoads> a4{};
   constexpr std::integral_constant<int, kTiles / 4> b1{};
   constexpr std::integral_constant<int, 2 * kTiles / 4> b2{};
@@ -333,9 +335,11 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   constexpr int kLoadsPerTile = kAtoms + (kFp4 || FORMAT == DEW_MOE_W_FP8_BLOCK ? 1 : 0);
   constexpr int kLoadsPerPhase = (kRowLoads + 3) / 4 + ((kTiles + 3) / 4) * kLoadsPerTile;
   // s_waitcnt vmcnt(kYounger) lgkmcnt(0): everything but the kYounger youngest vector-memory operations is done.
-  // Younger than the A loads of step s + 1 (the last of them issued in phase 4 of step s - 1) are at least the
-  // loads of phases 1-3 of step s.
-  constexpr int kYounger = a3.value + b3.value * kLoadsPerTile;
+  // Younger than the last A load of step s + 1 (issued during step s - 1, in the last phase that has one) are
+  // the weight loads of the later phases of step s - 1 and all loads of phases 1-3 of step s.
+  constexpr int kWeightsAfterLastA = a4.value > a3.value ? 0 : a3.value > a2.value ? kTiles - b3.value
+                                     : a2.value > a1.value ? kTiles - b2.value : kTiles - b1.value;
+  constexpr int kYounger = kWeightsAfterLastA * kLoadsPerTile + a3.value + b3.value * kLoadsPerTile;
   static_assert(kYounger < 64, "vmcnt is a 6-bit counter");
   constexpr int kWaitLanded = (kYounger & 0xF) | (7 << 4) | (0 << 8) | ((kYounger >> 4) << 14);
   constexpr int kWaitAll = (0 & 0xF) | (7 << 4) | (0 << 8) | (0 << 14);  // vmcnt(0) lgkmcnt(0)
@@ -463,10 +467,10 @@ static int check_bank(const char* who, const dew_moe_bank* bank, const char* nam
   return DEW_MOE_OK;
 }
 
-template <int FORMAT, bool PAIRED, int BM, int BN>
+template <int FORMAT, bool PAIRED, int BM, int BN, int WM, int WN>
 static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
   constexpr size_t kShared = 3 * static_cast<size_t>(BM) * BK * sizeof(bf16_t);
-  auto kernel = grouped_gemm_kernel<FORMAT, PAIRED, BM, BN>;
+  auto kernel = grouped_gemm_kernel<FORMAT, PAIRED, BM, BN, WM, WN>;
   static bool configured = false;  // dynamic LDS above 64 KiB must be opted into once per kernel
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -482,18 +486,19 @@ static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
   return launched(who);
 }
 
-// Tile choice from what the host knows (rows and experts; the routing itself stays on the device): large
-// tiles when the average group fills them, the 128 x 128 tile otherwise.
+// Tile choice from what the host knows (rows and experts; the routing itself stays on the device): 256-row
+// tiles when the average group fills them, 128-row tiles otherwise, and for decode-sized groups a 32-row tile
+// whose four wavefronts split the columns, so that thousands of wavefronts stream the weights at once.
 template <int FORMAT, bool PAIRED>
 static int launch_format(const char* who, const GemmParams& p, hipStream_t stream) {
   constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4;  // FP8's raw registers do not fit the large tile
-  const bool large = kFp4 && p.rows / p.experts >= 768 && p.width % 256 == 0;
-  if (PAIRED) {
-    if (large) return launch_tile<FORMAT, true, 256, 128>(who, p, stream);
-    return launch_tile<FORMAT, true, 128, 128>(who, p, stream);
+  const int average = p.rows / p.experts;
+  if (average < 24) return launch_tile<FORMAT, PAIRED, 32, 128, 1, 4>(who, p, stream);
+  if (kFp4 && average >= 768 && p.width % 256 == 0) {
+    if (PAIRED) return launch_tile<FORMAT, true, 256, 128, 2, 2>(who, p, stream);
+    return launch_tile<FORMAT, false, 256, 256, 2, 2>(who, p, stream);
   }
-  if (large) return launch_tile<FORMAT, false, 256, 256>(who, p, stream);
-  return launch_tile<FORMAT, false, 128, 128>(who, p, stream);
+  return launch_tile<FORMAT, PAIRED, 128, 128, 2, 2>(who, p, stream);
 }
 
 template <bool PAIRED>
