@@ -495,10 +495,10 @@ static int launch_format(const char* who, const GemmParams& p, hipStream_t strea
   const int average = p.rows / p.experts;
   if (average < 24) return launch_tile<FORMAT, PAIRED, 32, 128, 1, 4>(who, p, stream);
   if (kFp4 && average >= 768 && p.width % 256 == 0) {
-    if (PAIRED) return launch_tile<FORMAT, true, 256, 128, 2, 2>(who, p, stream);
-    return launch_tile<FORMAT, false, 256, 256, 2, 2>(who, p, stream);
+    if (PAIRED) return launch_tile<FORMAT, true, 256, 128, 1, 4>(who, p, stream);
+    return launch_tile<FORMAT, false, 256, 256, 1, 4>(who, p, stream);
   }
-  return launch_tile<FORMAT, PAIRED, 128, 128, 2, 2>(who, p, stream);
+  return launch_tile<FORMAT, PAIRED, 128, 128, 1, 4>(who, p, stream);
 }
 
 template <bool PAIRED>

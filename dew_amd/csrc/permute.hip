@@ -135,6 +135,89 @@ __global__ __launch_bounds__(kPermuteThreads) void permute_scatter_kernel(Permut
   }
 }
 
+// All of the above in one launch for at most kSlotsPerBlock slots (a decode step): one block counts, scans
+// and scatters, with the LDS histogram as the only intermediate.
+__global__ __launch_bounds__(kPermuteThreads) void permute_small_kernel(PermuteParams p) {
+  extern __shared__ int32_t running[];  // [kPermuteWaves][buckets] then [buckets + 1] totals
+  int32_t* totals = running + kPermuteWaves * p.buckets;
+  const int lane = threadIdx.x % 64;
+  const int wave = threadIdx.x / 64;
+  for (int i = threadIdx.x; i < kPermuteWaves * p.buckets; i += kPermuteThreads) running[i] = 0;
+  __syncthreads();
+  int32_t* mine = running + wave * p.buckets;
+  const int segment = ((p.slots + kPermuteThreads - 1) / kPermuteThreads) * 64;  // contiguous slots per wavefront
+  const int rounds = segment / 64;
+  const int wave_begin = wave * segment;
+  for (int round = 0; round < rounds; ++round) {
+    const int slot = wave_begin + round * 64 + lane;
+    if (slot < p.slots) atomicAdd(&mine[bucket_of(p.ids[slot], p.experts)], 1);
+  }
+  __syncthreads();
+  for (int b = threadIdx.x; b < p.buckets; b += kPermuteThreads) {
+    int sum = 0;
+    for (int w = 0; w < kPermuteWaves; ++w) sum += running[w * p.buckets + b];
+    totals[b] = sum;
+  }
+  __syncthreads();
+  if (threadIdx.x < 64) {  // exclusive scan of the bucket totals by one wavefront, 64 buckets a round
+    int carried = 0;
+    for (int base = 0; base < p.buckets; base += 64) {
+      const int b = base + lane;
+      const int size = b < p.buckets ? totals[b] : 0;
+      int inclusive = size;
+#pragma unroll
+      for (int offset = 1; offset < 64; offset <<= 1) {
+        const int other = __shfl_up(inclusive, offset, 64);
+        if (lane >= offset) inclusive += other;
+      }
+      if (b < p.buckets) totals[b] = carried + inclusive - size;
+      carried += __shfl(inclusive, 63, 64);
+    }
+    if (lane == 0) totals[p.buckets] = carried;
+  }
+  __syncthreads();
+  for (int b = threadIdx.x; b < p.buckets; b += kPermuteThreads) {
+    const int start = totals[b];
+    if (b < p.experts) {
+      p.sizes[b] = totals[b + 1] - start;
+      p.offsets[b] = start;
+    } else {
+      p.offsets[p.experts] = start;
+    }
+    int next = start;
+    for (int w = 0; w < kPermuteWaves; ++w) {
+      const int count = running[w * p.buckets + b];
+      running[w * p.buckets + b] = next;
+      next += count;
+    }
+  }
+  __syncthreads();
+  int bits = 1;
+  while ((1 << bits) < p.buckets) ++bits;
+  for (int round = 0; round < rounds; ++round) {
+    const int slot = wave_begin + round * 64 + lane;
+    const bool valid = slot < p.slots;
+    const int bucket = valid ? bucket_of(p.ids[slot], p.experts) : p.buckets;
+    unsigned long long same = __ballot(valid);
+    for (int bit = 0; bit < bits; ++bit) {
+      const bool set = (bucket >> bit) & 1;
+      const unsigned long long vote = __ballot(set);
+      same &= set ? vote : ~vote;
+    }
+    const int rank = __popcll(same & ((1ull << lane) - 1ull));
+    const int count = __popcll(same);
+    int position = 0;
+    if (valid) position = mine[bucket] + rank;
+    __syncthreads();
+    if (valid && rank == count - 1) mine[bucket] = position + 1;
+    __syncthreads();
+    if (valid) {
+      p.order[position] = slot;
+      p.rows[position] = slot / p.top_k;
+    }
+  }
+}
+
 }  // namespace dew
 
 extern "C" size_t dew_moe_permute_workspace_bytes(int32_t slots, int32_t experts) {
@@ -173,6 +256,11 @@ extern "C" int dew_moe_permute(const int32_t* indices, int32_t tokens, int32_t t
   uintptr_t base = (reinterpret_cast<uintptr_t>(workspace) + 255) & ~static_cast<uintptr_t>(255);
   p.counts = reinterpret_cast<int32_t*>(base);
   p.bases = p.counts + static_cast<size_t>(p.blocks) * p.buckets;
+  if (p.blocks <= 1) {
+    hipLaunchKernelGGL(permute_small_kernel, dim3(1), dim3(kPermuteThreads),
+                       sizeof(int32_t) * ((kPermuteWaves + 1) * p.buckets + 1), s, p);
+    return launched("permute_small_kernel");
+  }
   if (p.blocks > 0) {
     hipLaunchKernelGGL(permute_count_kernel, dim3(p.blocks), dim3(kPermuteThreads), sizeof(int32_t) * p.buckets, s, p);
     if (int rc = launched("permute_count_kernel")) return rc;

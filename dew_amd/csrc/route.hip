@@ -77,6 +77,7 @@ struct RouteParams {
   float scaling;
 };
 
+template <int kPerLane>  // experts <= 64 * kPerLane
 __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p) {
   extern __shared__ float shared[];  // [kRouteWaves][experts] selections, for the group scores
   const int lane = threadIdx.x % kWave;
@@ -87,9 +88,9 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
   const float* row = p.logits + static_cast<size_t>(token) * p.experts;
   const float ninf = -__builtin_inff();
 
-  float logit[kMaxPerLane], score[kMaxPerLane], select[kMaxPerLane];
+  float logit[kPerLane], score[kPerLane], select[kPerLane];
 #pragma unroll
-  for (int i = 0; i < kMaxPerLane; ++i) {
+  for (int i = 0; i < kPerLane; ++i) {
     const int e = lane + kWave * i;
     logit[i] = e < p.experts ? row[e] : ninf;
   }
@@ -98,25 +99,25 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
   if (p.score_function == DEW_MOE_SCORE_SOFTMAX) {
     float m = ninf;
 #pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i) m = fmaxf(m, logit[i]);
+    for (int i = 0; i < kPerLane; ++i) m = fmaxf(m, logit[i]);
     top = wave_max(m);
     double partial = 0.0;
 #pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i) {
+    for (int i = 0; i < kPerLane; ++i) {
       const int e = lane + kWave * i;
       score[i] = e < p.experts ? exp_f32(logit[i] - top) : 0.0f;
       partial = partial + static_cast<double>(score[i]);
     }
     denom = wave_sum_once(partial);
 #pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i) score[i] = score[i] / denom;
+    for (int i = 0; i < kPerLane; ++i) score[i] = score[i] / denom;
   } else {
 #pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i) score[i] = 1.0f / (1.0f + exp_f32(-logit[i]));
+    for (int i = 0; i < kPerLane; ++i) score[i] = 1.0f / (1.0f + exp_f32(-logit[i]));
   }
 
 #pragma unroll
-  for (int i = 0; i < kMaxPerLane; ++i) {
+  for (int i = 0; i < kPerLane; ++i) {
     const int e = lane + kWave * i;
     float s = score[i];
     if (p.bias != nullptr && e < p.experts) s = s + p.bias[e];
@@ -126,7 +127,7 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
   if (p.expert_groups > 1) {
     float* mine = shared + wave * p.experts;
 #pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i) {
+    for (int i = 0; i < kPerLane; ++i) {
       const int e = lane + kWave * i;
       if (e < p.experts) mine[e] = select[i];
     }
@@ -162,7 +163,7 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
       if (b.index == lane) taken = true;
     }
 #pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i) {
+    for (int i = 0; i < kPerLane; ++i) {
       const int e = lane + kWave * i;
       if (e < p.experts && !((kept >> (e / per_group)) & 1ull)) select[i] = ninf;
     }
@@ -176,7 +177,7 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
     b.value = ninf;
     b.index = 0x7fffffff;
 #pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i) {
+    for (int i = 0; i < kPerLane; ++i) {
       const int e = lane + kWave * i;
       if (e < p.experts && !((taken_mask >> i) & 1u) && better(select[i], e, b)) {
         b.value = select[i];
@@ -247,7 +248,16 @@ extern "C" int dew_moe_route(const float* logits, const float* bias, int32_t tok
                 expert_groups, groups_per_token, scaling};
   const int blocks = (tokens + kRouteWaves - 1) / kRouteWaves;
   const size_t shared = expert_groups > 1 ? sizeof(float) * kRouteWaves * experts : 0;
-  hipLaunchKernelGGL(route_kernel, dim3(blocks), dim3(kWave * kRouteWaves), shared,
-                     static_cast<hipStream_t>(stream), p);
+  const dim3 grid(blocks), block(kWave * kRouteWaves);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (experts <= 64) {
+    hipLaunchKernelGGL(route_kernel<1>, grid, block, shared, s, p);
+  } else if (experts <= 128) {
+    hipLaunchKernelGGL(route_kernel<2>, grid, block, shared, s, p);
+  } else if (experts <= 256) {
+    hipLaunchKernelGGL(route_kernel<4>, grid, block, shared, s, p);
+  } else {
+    hipLaunchKernelGGL(route_kernel<kMaxPerLane>, grid, block, shared, s, p);
+  }
   return launched("route_kernel");
 }
