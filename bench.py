@@ -153,6 +153,31 @@ def cpu_baseline(case, data, out, plan, budget_rows=192):
             "gemm_only_tflops": round(flops / gemm_s / 1e12, 5)}, (slots, down)
 
 
+def sustained_rates(device):
+    """What the chip sustains in this run: bf16 MFMA on random operands (TFLOP/s) and a plain copy (GB/s of
+    bytes read plus bytes written), each timed with HIP events over several launches after a warm-up."""
+    import torch
+
+    from dew_amd import ops
+
+    operands = torch.randn(16384, device=device).to(torch.bfloat16)
+    ops.probe_mfma(operands, 2000)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    flops = sum(ops.probe_mfma(operands, 20000) for _ in range(3))
+    stop.record()
+    torch.cuda.synchronize()
+    mfma = flops / (start.elapsed_time(stop) * 1e-3) / 1e12
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=device).random_()
+    dst = torch.empty_like(src)
+    ops.probe_copy(src, dst)
+    start.record()
+    moved = sum(2 * ops.probe_copy(src, dst) for _ in range(5))
+    stop.record()
+    torch.cuda.synchronize()
+    return round(mfma, 1), round(moved / (start.elapsed_time(stop) * 1e-3) / 1e9, 1)
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -160,6 +185,9 @@ def main():
     parser.add_argument("--warmup", type=int, default=3)
     parser.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--calibrate-copy", action="store_true",
+                        help="only run the plain copy probe (1 GiB read + 1 GiB written, 5 launches): the known traffic "
+                             "that rocprofv3's FETCH_SIZE / WRITE_SIZE are scaled by")
     parser.add_argument("--graph", choices=["auto", "on", "off"], default="auto",
                         help="replay the step as one captured HIP graph (auto: for the launch-bound configs c1 and c3)")
     args = parser.parse_args()
@@ -176,6 +204,11 @@ def main():
     ops.device_check()
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.calibrate_copy:
+        mfma, copy = sustained_rates(device)
+        print(json.dumps({"probe_copy_bytes_read_per_launch": 1 << 30, "probe_copy_bytes_written_per_launch": 1 << 30,
+                          "sustained_copy_gbs": copy, "sustained_bf16_mfma_tflops": mfma}))
+        return
     case = CONFIGS[args.config]
     data = build_workload(case, device)
     stepper = Stepper(case, data)
@@ -232,6 +265,11 @@ def main():
                                  "bf16 (v_mfma_f32_32x32x16_bf16)",
                     "frac_of_fp8_peak": round(achieved / PEAKS["fp8_mfma"], 4), "frac_of_fp4_peak": round(achieved / PEAKS["fp4_mfma"], 4)}
     roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
+    sustained_mfma, sustained_copy = sustained_rates(device)
+    roofline["sustained"] = {"bf16_mfma_random_operands_tflops": sustained_mfma, "plain_copy_gbs": sustained_copy,
+                             "frac_of_sustained": round(roofline["achieved"] / (sustained_copy if decode else sustained_mfma), 4),
+                             "note": "measured in this run by dew_moe_probe_mfma / dew_moe_probe_copy: the rate the chip holds on "
+                                     "random data at its power limit, below the published peak"}
     roofline["kernel"] = "grouped_gemm_kernel<paired gate/up + SwiGLU>"
     roofline["kernel_ms"] = round(gateup_ms, 4)
 

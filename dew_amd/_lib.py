@@ -9,7 +9,7 @@ from pathlib import Path
 
 LIBRARY = Path(__file__).resolve().parent / "libdew_moe_hip.so"
 
-W_FP8_BLOCK, W_FP8_CHANNEL, W_NVFP4 = 1, 2, 3
+W_FP8_BLOCK, W_FP8_CHANNEL, W_NVFP4, W_MXFP4 = 1, 2, 3, 4
 LAYOUT_REFERENCE, LAYOUT_PREPARED = 0, 1
 SCORE_SOFTMAX, SCORE_SIGMOID = 0, 1
 
@@ -17,7 +17,7 @@ EXPORTS = (
     "dew_moe_last_error", "dew_moe_architecture", "dew_moe_kernels", "dew_moe_kernel_fields",
     "dew_moe_device_check", "dew_moe_route", "dew_moe_router_logits", "dew_moe_group_offsets", "dew_moe_permute_workspace_bytes", "dew_moe_permute",
     "dew_moe_prepared_bytes", "dew_moe_prepare_bank", "dew_moe_grouped_gemm", "dew_moe_gateup_swiglu",
-    "dew_moe_swiglu", "dew_moe_combine",
+    "dew_moe_swiglu", "dew_moe_combine", "dew_moe_probe_mfma", "dew_moe_probe_copy",
 )
 """Every symbol include/dew_moe_hip.h declares."""
 
@@ -68,6 +68,8 @@ def library() -> ctypes.CDLL:
         "dew_moe_gateup_swiglu": (i32, [ptr, ptr, ptr, bank, bank, ptr, i32, ptr]),
         "dew_moe_swiglu": (i32, [ptr, ptr, ptr, i64, ptr]),
         "dew_moe_combine": (i32, [ptr, ptr, ptr, ptr, i32, i32, i32, ptr]),
+        "dew_moe_probe_mfma": (i32, [ptr, i32, ptr, c.POINTER(c.c_double), ptr]),
+        "dew_moe_probe_copy": (i32, [ptr, ptr, size, ptr]),
     }
     for name, (restype, argtypes) in prototypes.items():
         function = getattr(lib, name)

@@ -221,3 +221,29 @@ def combine(slots: torch.Tensor, weights: torch.Tensor, addend: torch.Tensor | N
     _lib.check(_lib.library().dew_moe_combine(_ptr(slots), _ptr(weights), _ptr(addend), _ptr(out), tokens, top_k, width,
                                               _stream()), "dew_moe_combine")
     return out
+
+
+# ---- measurement aids ---------------------------------------------------------------------------------
+
+
+def probe_mfma(operands: torch.Tensor, iters: int) -> float:
+    """Launch the back-to-back MFMA probe on `operands` (bf16, 16384 values); returns its FLOP count."""
+    import ctypes
+
+    _device(operands, "operands", torch.bfloat16)
+    if operands.numel() < 16384:
+        raise KernelError("the MFMA probe reads 16384 bf16 operands")
+    sink = torch.empty(1024 * 256, dtype=torch.float32, device=operands.device)
+    flops = ctypes.c_double(0.0)
+    _lib.check(_lib.library().dew_moe_probe_mfma(_ptr(operands), iters, _ptr(sink), ctypes.byref(flops), _stream()), "dew_moe_probe_mfma")
+    return flops.value
+
+
+def probe_copy(src: torch.Tensor, dst: torch.Tensor) -> int:
+    """Launch the plain copy probe; returns the bytes copied (read once, written once)."""
+    _device(src, "src"), _device(dst, "dst")
+    size = src.numel() * src.element_size()
+    if size != dst.numel() * dst.element_size() or size % 16:
+        raise KernelError("the copy probe takes two buffers of one size, a multiple of 16 bytes")
+    _lib.check(_lib.library().dew_moe_probe_copy(_ptr(src), _ptr(dst), size, _stream()), "dew_moe_probe_copy")
+    return size

@@ -226,3 +226,36 @@ def test_entry_points_refuse_what_they_cannot_run(ops):
     with pytest.raises(KernelError, match="deep"):
         ops.grouped_gemm(torch.zeros((4, 256), dtype=torch.bfloat16, device="cuda"), bank,
                          torch.zeros(3, dtype=torch.int32, device="cuda"))
+
+
+@pytest.mark.parametrize("quant", ["mxfp4", "nvfp4"])
+def test_large_tile_kernels_match_the_oracle(ops, quant):
+    """Groups averaging 768 rows or more take the 256-row tile (paired 256 x 2 x 128, unpaired 256 x 256)."""
+    sizes = [1100, 700]
+    gate, x, offsets = grouped_case(quant, 2, 256, 256, sizes, seed=31)
+    up, _, _ = grouped_case(quant, 2, 256, 256, sizes, seed=32)
+    gate_values, gate_factor = dequantized(gate)
+    up_values, up_factor = dequantized(up)
+    rows = bf16_np(x)
+    want_gate = oracle.grouped_matmul(rows, gate_values, sizes, factor=gate_factor)
+    want = oracle.swiglu(want_gate, oracle.grouped_matmul(rows, up_values, sizes, factor=up_factor))
+    xd, od = x.cuda(), torch.from_numpy(offsets).cuda()
+    pg, pu = ops.prepare(gate.to("cuda")), ops.prepare(up.to("cuda"))
+    got_gate = bf16_np(ops.grouped_gemm(xd, pg, od))
+    assert np.abs(got_gate - want_gate).max() <= 2 ** -8 * np.abs(want_gate).max() and (got_gate == want_gate).mean() > 0.97
+    fused = bf16_np(ops.gateup_swiglu(xd, pg, pu, od))
+    assert np.abs(fused - want).max() <= 2 ** -6 * np.abs(want).max() and (fused == want).mean() > 0.9
+
+
+def test_an_mxfp4_bank_is_recognized_at_preparation_and_a_general_bank_is_not(ops):
+    from dew_amd import _lib
+    weight = torch.from_numpy((np.random.default_rng(3).standard_normal((2, 256, 128)) * 0.02).astype(np.float32))
+    assert ops.prepare(quantize(weight, "mxfp4").to("cuda")).descriptor.format == _lib.W_MXFP4
+    assert ops.prepare(quantize(weight, "nvfp4").to("cuda")).descriptor.format == _lib.W_NVFP4
+
+
+def test_probes_run_and_the_copy_probe_copies(ops):
+    src = torch.arange(1 << 20, dtype=torch.int32, device="cuda")
+    dst = torch.zeros_like(src)
+    assert ops.probe_copy(src, dst) == 4 << 20 and torch.equal(src, dst)
+    assert ops.probe_mfma(torch.randn(16384, device="cuda").to(torch.bfloat16), 10) == 1024 * 4 * 10 * 16 * 32768.0
