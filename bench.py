@@ -153,6 +153,21 @@ def cpu_baseline(case, data, out, plan, budget_rows=192):
             "gemm_only_tflops": round(flops / gemm_s / 1e12, 5)}, (slots, down)
 
 
+# HBM bytes one launch of the dominant (gate/up) kernel moved, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (KiB per
+# dispatch, two runs of this file per workload), each scaled by what the same counter reads for the plain copy probe of known
+# size (--calibrate-copy: FETCH_SIZE reads half of the bytes fetched, WRITE_SIZE all of the bytes written). The counters
+# cannot be read from inside this process, so the figures sit here and are refreshed with the summaries kept beside the
+# kernel traces; a workload without an entry reports null.
+COUNTER_SCALE = {"FETCH_SIZE": 2.0, "WRITE_SIZE": 1.0}
+COUNTED_KIB = {"c2": {"FETCH_SIZE": 3272720.5, "WRITE_SIZE": 917504.0},
+               "c3": {"FETCH_SIZE": 195104.3, "WRITE_SIZE": 768.0}}
+
+
+def measured_traffic(config):
+    counted = COUNTED_KIB.get(config)
+    return None if counted is None else round(sum(counted[name] * COUNTER_SCALE[name] for name in counted) * 1024.0)
+
+
 def sustained_rates(device):
     """What the chip sustains in this run: bf16 MFMA on random operands (TFLOP/s) and a plain copy (GB/s of
     bytes read plus bytes written), each timed with HIP events over several launches after a warm-up."""
@@ -265,6 +280,8 @@ def main():
                                  "bf16 (v_mfma_f32_32x32x16_bf16)",
                     "frac_of_fp8_peak": round(achieved / PEAKS["fp8_mfma"], 4), "frac_of_fp4_peak": round(achieved / PEAKS["fp4_mfma"], 4)}
     roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
+    roofline["traffic"] = measured_traffic(args.config)
+    roofline["algorithmic"] = {"per_launch": gateup_bytes if decode else gateup_flops, "unit": "bytes" if decode else "flop"}
     sustained_mfma, sustained_copy = sustained_rates(device)
     roofline["sustained"] = {"bf16_mfma_random_operands_tflops": sustained_mfma, "plain_copy_gbs": sustained_copy,
                              "frac_of_sustained": round(roofline["achieved"] / (sustained_copy if decode else sustained_mfma), 4),
