@@ -113,8 +113,8 @@ __device__ __forceinline__ void schedule_phase() {
 
 // One grouped-GEMM kernel, templated on the weight format, on whether two banks (gate, up) are multiplied in
 // the same launch with the SwiGLU epilogue, and on the block tile: BM rows x BN columns of each matrix. The
-// four wavefronts sit WM x WN (2 x 2, or 1 x 4 for the 32-row decode tile); each owns (BM/WM) x (BN/WN) of
-// every matrix as 32 x 32 MFMA tiles.
+// four wavefronts sit WM x WN (1 x 4: side by side along the columns, so no two of them need the same weight
+// bytes); each owns (BM/WM) x (BN/WN) of every matrix as 32 x 32 MFMA tiles.
 template <int FORMAT, bool PAIRED, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   static_assert(WM * WN == 4 && BM % (32 * WM) == 0 && BN % (32 * WN) == 0 && BM % 32 == 0, "tile shape");
@@ -136,13 +136,15 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
 
   // ---- block -> (m-tile, column strip). Workgroup ids are dealt round-robin to the 8 XCDs, each with its
-  // own L2: give every XCD a contiguous run of the tile order, and order tiles so that a run of 32 blocks
-  // (one XCD's residents) covers kGroupM m-tiles x 8 strips, sharing A rows and B strips through that L2.
-  constexpr int kGroupM = 4;
+  // own L2. Tiles are ordered so that 32 consecutive ones (one XCD's residents) cover kGroupM m-tiles x 8
+  // strips, sharing A rows and B strips through that L2, and such chunks of 32 are dealt round-robin to the
+  // XCDs: the m-tile bound overshoots the real tile count by up to one tile per expert, and the empty tiles
+  // at the end of the order then spread over all XCDs instead of idling the last ones.
+  constexpr int kGroupM = 4, kChunk = 32;
   const int n_strips = p.width / BN;
   const int total = p.m_tile_bound * n_strips;
-  const int per_xcd = (total + 7) / 8;
-  const int order = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  const int local = blockIdx.x / 8;
+  const int order = ((local / kChunk) * 8 + blockIdx.x % 8) * kChunk + local % kChunk;
   if (order >= total) return;
   const int group = order / (kGroupM * n_strips);
   const int group_m = min(kGroupM, p.m_tile_bound - group * kGroupM);
@@ -481,7 +483,7 @@ static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
   // every expert may end in a partial tile, and the zeroed tail may add one more
   p.m_tile_bound = (p.rows + BM - 1) / BM + p.experts + 1;
   const int total = p.m_tile_bound * (p.width / BN);
-  const int blocks = ((total + 7) / 8) * 8;
+  const int blocks = ((total + 255) / 256) * 256;  // whole chunks of 32 tiles for each of the 8 XCDs
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreads), kShared, stream, p);
   return launched(who);
 }
