@@ -34,6 +34,7 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;  // a 16-byte regi
 constexpr int BK = 64;
 constexpr int kThreads = 256;
 constexpr int kChunksPerRow = BK / 8;  // 16-byte chunks in an LDS row
+constexpr int kMaxDepthBlocks = 256;   // FP8 128 x 128 blocks: depth up to 32768
 
 struct BankView {
   const uint8_t* codes;
@@ -116,7 +117,7 @@ __device__ __forceinline__ void schedule_phase() {
 // four wavefronts sit WM x WN (1 x 4: side by side along the columns, so no two of them need the same weight
 // bytes); each owns (BM/WM) x (BN/WN) of every matrix as 32 x 32 MFMA tiles.
 template <int FORMAT, bool PAIRED, int BM, int BN, int WM, int WN>
-__global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
+__global__ __launch_bounds__(kThreads, (PAIRED && BM == 128) ? 2 : 1) void grouped_gemm_kernel(GemmParams p) {
   static_assert(WM * WN == 4 && BM % (32 * WM) == 0 && BN % (32 * WN) == 0 && BM % 32 == 0, "tile shape");
   constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4;
   constexpr bool kPow2 = FORMAT == DEW_MOE_W_MXFP4;
@@ -128,10 +129,17 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   constexpr int kTiles = kMatrices * TJ;       // weight tiles a wavefront multiplies
   constexpr int kStageChunks = BM * kChunksPerRow;
   constexpr int kStages = 3;
+  // Weight register sets in flight. The 128-row paired tile runs two blocks a CU (256 registers a lane each),
+  // which FP8's 32 raw bytes a lane a tile a step only fit with three sets; two resident blocks cover the
+  // shorter lookahead.
+  constexpr int kSets = (!kFp4 && PAIRED && BM == 128) ? 3 : 4;
 
   extern __shared__ u32x4_t lds[];  // a ring of three stages of A: BM rows of 128 bytes each
   __shared__ int wave_tiles[4];
   __shared__ int found[3];  // expert, first sorted row of the tile, total m-tiles
+  // FP8 128 x 128 blocks: the scales of the block's column blocks down the whole depth, read once
+  constexpr int kScaleColumns = FORMAT == DEW_MOE_W_FP8_BLOCK ? kMatrices * (BN / 128) : 1;
+  __shared__ float depth_scales[kScaleColumns][FORMAT == DEW_MOE_W_FP8_BLOCK ? kMaxDepthBlocks : 1];
 
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
 
@@ -225,7 +233,6 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   // ---- B loader: tile t = (matrix, 32-column tile j of the wavefront); the lane's piece of each atom ----
   const uint8_t* b_src[kTiles];
   const uint16_t* b_scale_src[kTiles];  // FP4: the lane's two e4m3 block scales of each atom
-  const float* block_scales[kTiles];    // FP8 block: the tile's column of 128 x 128 scales
   float channel_scale[kTiles];          // FP8 channel: the lane's column scale
   const int n_atoms = p.width / 32, k_atoms = p.depth / kAtomK;
 #pragma unroll
@@ -236,31 +243,34 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
     const size_t first_atom = (static_cast<size_t>(expert) * n_atoms + column / 32) * k_atoms;
     b_src[t] = codes + first_atom * kAtomBytes + lane * 16;
     b_scale_src[t] = nullptr;
-    block_scales[t] = nullptr;
     channel_scale[t] = 1.0f;
     if (kFp4) {
       b_scale_src[t] = static_cast<const uint16_t*>(scales) + first_atom * 64 + lane;
     } else if (FORMAT == DEW_MOE_W_FP8_CHANNEL) {
       channel_scale[t] = static_cast<const float*>(scales)[static_cast<size_t>(expert) * p.width + column + lane % 32];
-    } else {
-      block_scales[t] = static_cast<const float*>(scales) + static_cast<size_t>(expert) * (p.depth / 128) * (p.width / 128) + column / 128;
+    }
+  }
+  if constexpr (FORMAT == DEW_MOE_W_FP8_BLOCK) {
+    const int depth_blocks = p.depth / 128, width_blocks = p.width / 128;
+    for (int item = tid; item < kScaleColumns * depth_blocks; item += kThreads) {
+      const int which = item / depth_blocks, block = item % depth_blocks;
+      const float* scales = static_cast<const float*>(which / (BN / 128) == 0 ? p.w0.scales : p.w1.scales);
+      depth_scales[which][block] =
+          scales[(static_cast<size_t>(expert) * depth_blocks + block) * width_blocks + n0 / 128 + which % (BN / 128)];
     }
   }
 
-  // Raw weight data in flight: four register sets (steps s .. s + 3), so a load has two to three steps to land.
-  u32x4_t b_regs[4][kTiles][kAtoms];
-  uint32_t s_regs[4][kTiles];  // FP4: two e4m3 scale bytes in the low half; FP8 block: the fp32 scale's bits
+  // Raw weight data in flight: kSets register sets (steps s .. s + kSets - 1), so a load has kSets - 2 to
+  // kSets - 1 steps to land.
+  u32x4_t b_regs[kSets][kTiles][kAtoms];
+  uint32_t s_regs[kSets][kTiles];  // FP4: two e4m3 scale bytes in the low half
   auto load_b = [&](auto set, int step, auto begin, auto end) __attribute__((always_inline)) {
 #pragma unroll
     for (int t = begin.value; t < end.value; ++t) {
 #pragma unroll
       for (int a = 0; a < kAtoms; ++a)
         b_regs[set.value][t][a] = *reinterpret_cast<const u32x4_t*>(b_src[t] + (static_cast<size_t>(step) * kAtoms + a) * kAtomBytes);
-      if (kFp4) {
-        __builtin_memcpy(&s_regs[set.value][t], b_scale_src[t] + static_cast<size_t>(step) * 64, sizeof(uint32_t));
-      } else if (FORMAT == DEW_MOE_W_FP8_BLOCK) {
-        s_regs[set.value][t] = __float_as_uint(block_scales[t][static_cast<size_t>((step * BK) / 128) * (p.width / 128)]);
-      }
+      if (kFp4) __builtin_memcpy(&s_regs[set.value][t], b_scale_src[t] + static_cast<size_t>(step) * 64, sizeof(uint32_t));
     }
   };
 
@@ -273,7 +283,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
     for (int i = 0; i < TI; ++i)
       a_frag[into.value][i] = __builtin_bit_cast(bf16x8_t, stage[swizzled(wm0 + 32 * i + lane % 32, chunk)]);
   };
-  auto dequantize = [&](auto set, auto kk, auto into) __attribute__((always_inline)) {
+  auto dequantize = [&](auto set, auto kk, auto into, int step) __attribute__((always_inline)) {
 #pragma unroll
     for (int t = 0; t < kTiles; ++t) {
       if constexpr (kFp4) {
@@ -283,7 +293,9 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
         const uint32_t word = b_regs[set.value][t][0][kk.value];
         b_frag[into.value][t] = kPow2 ? fragment_fp4_pow2(word, fp4_scale[t]) : fragment_fp4(word, fp4_scale[t]);
       } else {
-        const float scale = FORMAT == DEW_MOE_W_FP8_BLOCK ? __uint_as_float(s_regs[set.value][t]) : channel_scale[t];
+        const float scale = FORMAT == DEW_MOE_W_FP8_BLOCK
+                                ? depth_scales[(t / TJ) * (BN / 128) + (wn0 + 32 * (t % TJ)) / 128][step / (128 / BK)]
+                                : channel_scale[t];
         const u32x4_t& raw = b_regs[set.value][t][kk.value / 2 % kAtoms];
         b_frag[into.value][t] = fragment_fp8(raw[2 * (kk.value % 2)], raw[2 * (kk.value % 2) + 1], scale);
       }
@@ -314,10 +326,10 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   // s .. s + 2. A step is four phases, one 16-deep slice each: the slice multiplies while the next slice's A
   // fragments are read from LDS and its B fragments dequantized. Each phase also issues a quarter of the step's
   // global loads, so the memory pipeline sees an even stream: A rows of step s + 2 into stage (s + 2) % 3 (last
-  // read during step s - 1) and weights of step s + 3 into set (s + 3) % 4 (last read during step s - 1).
+  // read during step s - 1) and weights of step s + kSets - 1 into the set last read during step s - 1.
   // One barrier a step, after phase 3: by then this wavefront's A loads of step s + 1 have landed (a vmcnt wait
   // that leaves the younger loads in flight) and its own fragment reads are done, so after the barrier stage
-  // (s + 1) % 3 may be read and stage s % 3 overwritten. The loop is unrolled by four so that the B register
+  // (s + 1) % 3 may be read and stage s % 3 overwritten. The loop is unrolled by kSets so that the B register
   // sets are compile-time constants.
   constexpr std::integral_constant<int, 0> c0{};
   constexpr std::integral_constant<int, 1> c1{};
@@ -334,7 +346,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   constexpr std::integral_constant<int, kTiles> all_tiles{};
   constexpr int kMfmas = kMatrices * TI * TJ;
   constexpr int kDequantOps = kTiles * (kPow2 ? 5 : 17);  // vector instructions to dequantize one slice
-  constexpr int kLoadsPerTile = kAtoms + (kFp4 || FORMAT == DEW_MOE_W_FP8_BLOCK ? 1 : 0);
+  constexpr int kLoadsPerTile = kAtoms + (kFp4 ? 1 : 0);
   constexpr int kLoadsPerPhase = (kRowLoads + 3) / 4 + ((kTiles + 3) / 4) * kLoadsPerTile;
   // s_waitcnt vmcnt(kYounger) lgkmcnt(0): everything but the kYounger youngest vector-memory operations is done.
   // Younger than the last A load of step s + 1 (issued during step s - 1, in the last phase that has one) are
@@ -346,17 +358,17 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   constexpr int kWaitLanded = (kYounger & 0xF) | (7 << 4) | (0 << 8) | ((kYounger >> 4) << 14);
   constexpr int kWaitAll = (0 & 0xF) | (7 << 4) | (0 << 8) | (0 << 14);  // vmcnt(0) lgkmcnt(0)
   int stage_index = 0;  // s % 3
-  auto iterate = [&](auto set, int step) __attribute__((always_inline)) {
-    constexpr std::integral_constant<int, (set.value + 1) % 4> following{};
-    constexpr std::integral_constant<int, (set.value + 3) % 4> filling{};
+  auto iterate = [&](auto set, int step, auto last_steps) __attribute__((always_inline)) {
+    constexpr std::integral_constant<int, (set.value + 1) % kSets> following{};
+    constexpr std::integral_constant<int, (set.value + kSets - 1) % kSets> filling{};
     const int next_index = stage_index == kStages - 1 ? 0 : stage_index + 1;
     const int fill_index = next_index == kStages - 1 ? 0 : next_index + 1;
     u32x4_t* current = lds + stage_index * kStageChunks;
     u32x4_t* next = lds + next_index * kStageChunks;
     u32x4_t* fill = lds + fill_index * kStageChunks;
-    const int ahead_a = min(step + 2, steps - 1), ahead_b = min(step + 3, steps - 1);
+    const int ahead_a = min(step + 2, steps - 1), ahead_b = min(step + kSets - 1, steps - 1);
     fetch(current, c1, c1);
-    dequantize(set, c1, c1);
+    dequantize(set, c1, c1, step);
     multiply(c0);
     load_a(fill, ahead_a, c0, a1);
     load_b(filling, ahead_b, c0, b1);
@@ -364,7 +376,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
     __builtin_amdgcn_sched_barrier(0);
 
     fetch(current, c2, c0);
-    dequantize(set, c2, c0);
+    dequantize(set, c2, c0, step);
     multiply(c1);
     load_a(fill, ahead_a, a1, a2);
     load_b(filling, ahead_b, b1, b2);
@@ -372,20 +384,22 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
     __builtin_amdgcn_sched_barrier(0);
 
     fetch(current, c3, c1);
-    dequantize(set, c3, c1);
+    dequantize(set, c3, c1, step);
     multiply(c0);
     load_a(fill, ahead_a, a2, a3);
     load_b(filling, ahead_b, b2, b3);
     schedule_phase<0, kMfmas, TI, 0, kDequantOps + 2 * kLoadsPerPhase, kLoadsPerPhase>();
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_waitcnt(kWaitLanded);
+    // In the steps after the unrolled loop the compiler drops weight loads nobody consumes, so the count of
+    // younger operations no longer holds there: wait for everything (nothing useful is in flight by then).
+    __builtin_amdgcn_s_waitcnt(last_steps.value ? kWaitAll : kWaitLanded);
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
 
     fetch(next, c0, c0);
-    dequantize(following, c0, c0);
+    dequantize(following, c0, c0, step + 1);
     multiply(c1);
     load_a(fill, ahead_a, a3, a4);
     load_b(filling, ahead_b, b3, b4);
@@ -395,7 +409,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   };
   load_b(c0, 0, c0, all_tiles);
   load_b(c1, min(1, steps - 1), c0, all_tiles);
-  load_b(c2, min(2, steps - 1), c0, all_tiles);
+  if constexpr (kSets == 4) load_b(c2, min(2, steps - 1), c0, all_tiles);
   load_a(lds, 0, c0, a4);
   load_a(lds + kStageChunks, min(1, steps - 1), c0, a4);
   asm volatile("" ::: "memory");
@@ -403,17 +417,18 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
   fetch(lds, c0, c0);
-  dequantize(c0, c0, c0);
+  dequantize(c0, c0, c0, 0);
   int step = 0;
-  for (; step + 3 < steps; step += 4) {
-    iterate(c0, step);
-    iterate(c1, step + 1);
-    iterate(c2, step + 2);
-    iterate(c3, step + 3);
+  for (; step + kSets <= steps; step += kSets) {
+    iterate(c0, step, std::false_type{});
+    iterate(c1, step + 1, std::false_type{});
+    iterate(c2, step + 2, std::false_type{});
+    if constexpr (kSets == 4) iterate(c3, step + 3, std::false_type{});
   }
-  if (step < steps) {  // depth is whole 128s: an even number of steps, so the tail is two steps or none
-    iterate(c0, step);
-    iterate(c1, step + 1);
+  if (step < steps) iterate(c0, step++, std::true_type{});  // the last steps % kSets steps
+  if (step < steps) iterate(c1, step++, std::true_type{});
+  if constexpr (kSets == 4) {
+    if (step < steps) iterate(c2, step++, std::true_type{});
   }
   __builtin_amdgcn_s_waitcnt(kWaitAll);  // the clamped tail loads still target the LDS
 
@@ -462,6 +477,7 @@ static int check_bank(const char* who, const dew_moe_bank* bank, const char* nam
               "%s: %s bank has unknown format %d", who, name, bank->format);
   DEW_REQUIRE(bank->experts >= 1 && bank->experts <= 4096, "%s: %s bank has %d experts", who, name, bank->experts);
   DEW_REQUIRE(bank->depth >= 128 && bank->depth % 128 == 0, "%s: %s bank depth %d is not a multiple of 128", who, name, bank->depth);
+  DEW_REQUIRE(bank->depth <= 128 * kMaxDepthBlocks, "%s: %s bank depth %d is above %d", who, name, bank->depth, 128 * kMaxDepthBlocks);
   DEW_REQUIRE(bank->width % 128 == 0 && bank->width >= 128, "%s: %s bank width %d is not a multiple of 128", who, name, bank->width);
   DEW_REQUIRE(bank->codes && bank->scales, "%s: %s bank codes and scales must not be null", who, name);
   DEW_REQUIRE((bank->format != DEW_MOE_W_NVFP4 && bank->format != DEW_MOE_W_MXFP4) || bank->tensor_scale, "%s: %s NVFP4 bank needs tensor scales", who, name);

@@ -259,3 +259,27 @@ def test_probes_run_and_the_copy_probe_copies(ops):
     dst = torch.zeros_like(src)
     assert ops.probe_copy(src, dst) == 4 << 20 and torch.equal(src, dst)
     assert ops.probe_mfma(torch.randn(16384, device="cuda").to(torch.bfloat16), 10) == 1024 * 4 * 10 * 16 * 32768.0
+
+
+@pytest.mark.parametrize("quant", ["fp8_channel", "fp8_block", "mxfp4", "nvfp4"])
+@pytest.mark.parametrize("depth", [128, 384, 640, 896])
+@pytest.mark.parametrize("label,sizes", [("decode", [3, 0, 9]), ("medium", [150, 70, 1]), ("large", [800])])
+def test_depths_that_leave_steps_after_the_unrolled_loop(ops, quant, depth, label, sizes):
+    """Depth / 64 steps that are not a multiple of the main loop's unroll (3 or 4) end in separately compiled
+    steps; both launches must still agree with the oracle and with each other."""
+    if quant in ("mxfp4", "nvfp4"):
+        depth = 2 * depth  # an NvFp4 bank's depth is whole 256s
+    gate, x, offsets = grouped_case(quant, len(sizes), depth, 256, sizes, seed=depth + len(quant))
+    up, _, _ = grouped_case(quant, len(sizes), depth, 256, sizes, seed=depth + 50)
+    gate_values, gate_factor = dequantized(gate)
+    rows = bf16_np(x)
+    want_gate = oracle.grouped_matmul(rows, gate_values, sizes, factor=gate_factor)
+    xd, od = x.cuda(), torch.from_numpy(offsets).cuda()
+    pg, pu = ops.prepare(gate.to("cuda")), ops.prepare(up.to("cuda"))
+    fused = bf16_np(ops.gateup_swiglu(xd, pg, pu, od))
+    got_gate = ops.grouped_gemm(xd, pg, od)
+    apart = bf16_np(ops.swiglu(got_gate, ops.grouped_gemm(xd, pu, od)))
+    assert np.array_equal(fused, apart)
+    got_gate = bf16_np(got_gate)
+    assert np.abs(got_gate - want_gate).max() <= 2 ** -8 * np.abs(want_gate).max() + 1e-6
+    assert (got_gate == want_gate).mean() > 0.97
