@@ -117,7 +117,7 @@ __device__ __forceinline__ void schedule_phase() {
 // four wavefronts sit WM x WN (1 x 4: side by side along the columns, so no two of them need the same weight
 // bytes); each owns (BM/WM) x (BN/WN) of every matrix as 32 x 32 MFMA tiles.
 template <int FORMAT, bool PAIRED, int BM, int BN, int WM, int WN>
-__global__ __launch_bounds__(kThreads, (PAIRED && BM == 128) ? 2 : 1) void grouped_gemm_kernel(GemmParams p) {
+__global__ __launch_bounds__(kThreads, (BM == 128 && (PAIRED ? 2 : 1) * BN == 256) ? 2 : 1) void grouped_gemm_kernel(GemmParams p) {
   static_assert(WM * WN == 4 && BM % (32 * WM) == 0 && BN % (32 * WN) == 0 && BM % 32 == 0, "tile shape");
   constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4;
   constexpr bool kPow2 = FORMAT == DEW_MOE_W_MXFP4;
@@ -129,10 +129,11 @@ __global__ __launch_bounds__(kThreads, (PAIRED && BM == 128) ? 2 : 1) void group
   constexpr int kTiles = kMatrices * TJ;       // weight tiles a wavefront multiplies
   constexpr int kStageChunks = BM * kChunksPerRow;
   constexpr int kStages = 3;
-  // Weight register sets in flight. The 128-row paired tile runs two blocks a CU (256 registers a lane each),
+  // Weight register sets in flight. The 128-row tile of 256 columns in all (paired 2 x 128, or unpaired 256: two
+  // MFMAs for each A fragment read from LDS) runs two blocks a CU (256 registers a lane each),
   // which FP8's 32 raw bytes a lane a tile a step only fit with three sets; two resident blocks cover the
   // shorter lookahead.
-  constexpr int kSets = (!kFp4 && PAIRED && BM == 128) ? 3 : 4;
+  constexpr int kSets = (!kFp4 && BM == 128 && kMatrices * BN == 256) ? 3 : 4;
 
   extern __shared__ u32x4_t lds[];  // a ring of three stages of A: BM rows of 128 bytes each
   __shared__ int wave_tiles[4];
@@ -516,6 +517,8 @@ static int launch_format(const char* who, const GemmParams& p, hipStream_t strea
     if (PAIRED) return launch_tile<FORMAT, true, 256, 128, 1, 4>(who, p, stream);
     return launch_tile<FORMAT, false, 256, 256, 1, 4>(who, p, stream);
   }
+  if (!PAIRED && p.width % 256 == 0 && static_cast<long long>(p.rows / 128 + 1) * (p.width / 256) >= 512)
+    return launch_tile<FORMAT, false, 128, 256, 1, 4>(who, p, stream);  // enough tiles to fill the chip twice over
   return launch_tile<FORMAT, PAIRED, 128, 128, 1, 4>(who, p, stream);
 }
 
