@@ -435,37 +435,65 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (PAIRED ? 2 : 1) * BN == 25
 
   // ---- epilogue: acc[..][q] is row 8 (q / 4) + 4 (lane / 32) + q % 4, column lane % 32 of its 32 x 32 tile.
   // Neighbouring lanes hold neighbouring columns: each pair of lanes swaps one value so that the even lane
-  // holds both columns of row q and the odd lane both of row q + 1, and every lane stores 4 bytes a row pair.
+  // holds both columns of row q and the odd lane both of row q + 1. The packed pairs are staged in the LDS the
+  // A ring no longer needs, row-major, and the block then writes whole output rows, 16 bytes a lane, so that
+  // the tile leaves as full cache lines (direct 4-byte stores of 64-byte row pieces took a quarter of the
+  // kernel's time). Tiles of 256 columns are staged in two passes of BM / 2 rows.
   float factor0 = 1.0f, factor1 = 1.0f;
   if (kFp4) {  // the 2^8 the decode owes times the expert's tensor scale (src/dew/nn/kernels/gemm.py:660-662)
     factor0 = 256.0f * p.w0.tensor_scale[expert];
     if (PAIRED) factor1 = 256.0f * p.w1.tensor_scale[expert];
   }
+  constexpr int kPasses = BN == 256 ? 2 : 1;
+  constexpr int kPassTiles = TI / kPasses, kPassRows = BM / kPasses;
+  constexpr int kRowDwords = BN / 2 + 4;  // a staged row: BN bf16 and 16 bytes of padding
+  constexpr int kRowChunks = BN / 8;      // 16-byte pieces of an output row
+  constexpr int kStoreIters = kPassRows * kRowChunks / kThreads;
+  static_assert(kPassRows * kRowChunks % kThreads == 0, "whole store rounds");
+  static_assert(TI % kPasses == 0 && kPassRows * kRowDwords * 4 <= kStages * kStageChunks * 16, "staged tile fits the A ring");
+  uint32_t* staged = reinterpret_cast<uint32_t*>(lds);
   const bool odd_lane = lane & 1;
-  const int column = n0 + wn0 + (lane % 32 & ~1);  // first of the lane pair's two columns
+  __builtin_amdgcn_s_barrier();  // every wavefront has read its last A fragments: the ring is free
 #pragma unroll
-  for (int i = 0; i < TI; ++i) {
+  for (int pass = 0; pass < kPasses; ++pass) {
+    if (pass > 0) __syncthreads();  // the previous pass has left the LDS
+    // where this thread's rows of the pass go: the scatter indices are fetched before the arithmetic below
+    int out_rows[kStoreIters];
 #pragma unroll
-    for (int q = 0; q < 16; q += 2) {
-      const int row = wm0 + 32 * i + 8 * (q / 4) + 4 * (lane / 32) + q % 4 + (odd_lane ? 1 : 0);
-      const bool valid = row < valid_rows;
-      int out_row = row0 + min(row, valid_rows - 1);
-      if (p.scatter) out_row = p.scatter[out_row];
-      uint32_t* dst = reinterpret_cast<uint32_t*>(p.out + static_cast<size_t>(out_row) * p.width + column);
+    for (int it = 0; it < kStoreIters; ++it) {
+      const int sorted = row0 + min(pass * kPassRows + (tid + it * kThreads) / kRowChunks, valid_rows - 1);
+      out_rows[it] = p.scatter ? p.scatter[sorted] : sorted;
+    }
 #pragma unroll
-      for (int j = 0; j < TJ; ++j) {
-        uint32_t mine[2];
+    for (int ii = 0; ii < kPassTiles; ++ii) {
+      const int i = pass * kPassTiles + ii;
 #pragma unroll
-        for (int r = 0; r < 2; ++r) {
-          mine[r] = PAIRED ? swiglu_rounded(acc[0][i][j][q + r] * factor0, acc[kMatrices - 1][i][j][q + r] * factor1)
-                           : f32_to_bf16(acc[0][i][j][q + r] * factor0);
+      for (int q = 0; q < 16; q += 2) {
+        const int row = 32 * ii + 8 * (q / 4) + 4 * (lane / 32) + q % 4 + (odd_lane ? 1 : 0);  // within the pass
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+          uint32_t mine[2];
+#pragma unroll
+          for (int r = 0; r < 2; ++r) {
+            mine[r] = PAIRED ? swiglu_rounded(acc[0][i][j][q + r] * factor0, acc[kMatrices - 1][i][j][q + r] * factor1)
+                             : f32_to_bf16(acc[0][i][j][q + r] * factor0);
+          }
+          // even lane keeps row q and sends its row q + 1; odd lane keeps row q + 1 and sends its row q
+          const uint32_t sent = odd_lane ? mine[0] : mine[1];
+          const uint32_t got = __builtin_amdgcn_mov_dpp(sent, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+          const uint32_t packed = odd_lane ? (got | (mine[1] << 16)) : (mine[0] | (got << 16));
+          staged[row * kRowDwords + (wn0 + 32 * j + (lane % 32 & ~1)) / 2] = packed;
         }
-        // even lane keeps row q and sends its row q + 1; odd lane keeps row q + 1 and sends its row q
-        const uint32_t sent = odd_lane ? mine[0] : mine[1];
-        const uint32_t got = __builtin_amdgcn_mov_dpp(sent, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
-        const uint32_t packed = odd_lane ? (got | (mine[1] << 16)) : (mine[0] | (got << 16));
-        if (valid) dst[16 * j] = packed;
       }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < kStoreIters; ++it) {
+      const int item = tid + it * kThreads;
+      const int staged_row = item / kRowChunks, chunk = item % kRowChunks;
+      if (pass * kPassRows + staged_row < valid_rows)
+        *reinterpret_cast<u32x4_t*>(p.out + static_cast<size_t>(out_rows[it]) * p.width + n0 + chunk * 8) =
+            *reinterpret_cast<const u32x4_t*>(staged + staged_row * kRowDwords + chunk * 4);
     }
   }
 }
