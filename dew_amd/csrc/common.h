@@ -46,6 +46,19 @@ __device__ __forceinline__ bf16_t swiglu_rounded(float gate_sum, float up_sum) {
   return f32_to_bf16(activated * u);
 }
 
+// GPT-OSS's gating of one (gate, up) pair already rounded to bf16 (src/dew/nn/gpt_oss.py:120-121 over
+// src/dew/nn/activations.py:72-74,327-333): gate clamped from above and up both ways by `limit`, then
+// (up + 1) * gate * logistic(1.702 gate) with every operation rounded to bf16 as an array of that dtype
+// rounds it; 1.702 enters as the bf16 it is multiplied in, 1.703125.
+__device__ __forceinline__ bf16_t gated_pair_rounded(float gate, float up, float limit) {
+  const float g = fminf(gate, limit), u = fminf(fmaxf(up, -limit), limit);
+  const float t = bf16_round(g * 1.703125f);
+  const float sig = bf16_round(__builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(t * -1.44269504088896340736f)));
+  const float q = bf16_round(g * sig);
+  const float u1 = bf16_round(u + 1.0f);
+  return f32_to_bf16(u1 * q);
+}
+
 // ---- prepared bank geometry (fragment-native atoms) ----
 // FP8 atom: 32 n x 32 k bytes = 1 KiB; lane l = (g = l / 32, n = l % 32) holds k = 16 g .. 16 g + 15.
 // FP4 atom: 32 n x 64 k nibbles = 1 KiB; lane l holds k = 32 g .. 32 g + 31 (byte j: low nibble k = 32 g + 2 j).

@@ -49,8 +49,14 @@ struct GemmParams {
   const int32_t* scatter;
   BankView w0, w1;
   bf16_t* out;
+  const float* bias;  // [experts, width] values of the compute dtype held in fp32, or null
+  float limit;        // the interleaved gated epilogue's clamp
   int experts, depth, width, rows, m_tile_bound;
 };
+
+// What the epilogue writes: the rounded product (plus bias); SwiGLU of two banks' products; or, for one bank
+// whose columns interleave gate (even) and up (odd), the clamped quick-GELU gating of each column pair.
+enum Epilogue { kPlain = 0, kSwigluOfTwo = 1, kInterleavedGated = 2 };
 
 // LDS index of 16-byte chunk `chunk` of row `row` (128-byte rows). The chunk is xor-swizzled by
 // f(row) = ((row >> 1) & 7) ^ ((row & 1) << 2), chosen against the measured service order of gfx950's LDS:
@@ -116,8 +122,11 @@ __device__ __forceinline__ void schedule_phase() {
 // the same launch with the SwiGLU epilogue, and on the block tile: BM rows x BN columns of each matrix. The
 // four wavefronts sit WM x WN (1 x 4: side by side along the columns, so no two of them need the same weight
 // bytes); each owns (BM/WM) x (BN/WN) of every matrix as 32 x 32 MFMA tiles.
-template <int FORMAT, bool PAIRED, int BM, int BN, int WM, int WN>
-__global__ __launch_bounds__(kThreads, (BM == 128 && (PAIRED ? 2 : 1) * BN == 256) ? 2 : 1) void grouped_gemm_kernel(GemmParams p) {
+template <int FORMAT, int MODE, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 : 1) * BN == 256) ? 2 : 1) void grouped_gemm_kernel(GemmParams p) {
+  constexpr bool PAIRED = MODE == kSwigluOfTwo;
+  constexpr bool kGated = MODE == kInterleavedGated;
+  constexpr int kOutBN = kGated ? BN / 2 : BN;  // output columns of the tile
   static_assert(WM * WN == 4 && BM % (32 * WM) == 0 && BN % (32 * WN) == 0 && BM % 32 == 0, "tile shape");
   constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4;
   constexpr bool kPow2 = FORMAT == DEW_MOE_W_MXFP4;
@@ -197,10 +206,11 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (PAIRED ? 2 : 1) * BN == 25
     // Past the last real tile: zero the rows no expert owns (sorted positions offsets[E] .. rows).
     const int tail_begin = p.offsets[p.experts] + (m_tile - found[2]) * BM;
     const int tail_end = min(tail_begin + BM, p.rows);
-    for (int item = tid; item < (tail_end - tail_begin) * (BN / 8); item += kThreads) {
-      const int sorted = tail_begin + item / (BN / 8);
+    const int out_width = kGated ? p.width / 2 : p.width, out_n0 = kGated ? n0 / 2 : n0;
+    for (int item = tid; item < (tail_end - tail_begin) * (kOutBN / 8); item += kThreads) {
+      const int sorted = tail_begin + item / (kOutBN / 8);
       const int row = p.scatter ? p.scatter[sorted] : sorted;
-      *reinterpret_cast<u32x4_t*>(p.out + static_cast<size_t>(row) * p.width + n0 + (item % (BN / 8)) * 8) = u32x4_t{0, 0, 0, 0};
+      *reinterpret_cast<u32x4_t*>(p.out + static_cast<size_t>(row) * out_width + out_n0 + (item % (kOutBN / 8)) * 8) = u32x4_t{0, 0, 0, 0};
     }
     return;
   }
@@ -446,13 +456,19 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (PAIRED ? 2 : 1) * BN == 25
   }
   constexpr int kPasses = BN == 256 ? 2 : 1;
   constexpr int kPassTiles = TI / kPasses, kPassRows = BM / kPasses;
-  constexpr int kRowDwords = BN / 2 + 4;  // a staged row: BN bf16 and 16 bytes of padding
-  constexpr int kRowChunks = BN / 8;      // 16-byte pieces of an output row
+  constexpr int kRowDwords = kOutBN / 2 + 4;  // a staged row: the tile's output columns in bf16 and 16 bytes of padding
+  constexpr int kRowChunks = kOutBN / 8;      // 16-byte pieces of an output row
   constexpr int kStoreIters = kPassRows * kRowChunks / kThreads;
   static_assert(kPassRows * kRowChunks % kThreads == 0, "whole store rounds");
   static_assert(TI % kPasses == 0 && kPassRows * kRowDwords * 4 <= kStages * kStageChunks * 16, "staged tile fits the A ring");
   uint32_t* staged = reinterpret_cast<uint32_t*>(lds);
   const bool odd_lane = lane & 1;
+  const int out_width = kGated ? p.width / 2 : p.width, out_n0 = kGated ? n0 / 2 : n0;
+  // Each expert's bias meets its rows' fp32 sums before their one rounding (src/dew/nn/moe.py:729-742).
+  float bias[TJ];
+#pragma unroll
+  for (int j = 0; j < TJ; ++j)
+    bias[j] = (!PAIRED && p.bias) ? p.bias[static_cast<size_t>(expert) * p.width + n0 + wn0 + 32 * j + lane % 32] : 0.0f;
   __builtin_amdgcn_s_barrier();  // every wavefront has read its last A fragments: the ring is free
 #pragma unroll
   for (int pass = 0; pass < kPasses; ++pass) {
@@ -472,17 +488,29 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (PAIRED ? 2 : 1) * BN == 25
         const int row = 32 * ii + 8 * (q / 4) + 4 * (lane / 32) + q % 4 + (odd_lane ? 1 : 0);  // within the pass
 #pragma unroll
         for (int j = 0; j < TJ; ++j) {
-          uint32_t mine[2];
+          if constexpr (kGated) {
+            // The even lane holds a gate column and the odd lane the up column beside it, rows q and q + 1 each:
+            // the even lane takes the pair of row q, the odd lane the pair of row q + 1, and each writes one value.
+            float mine[2];
 #pragma unroll
-          for (int r = 0; r < 2; ++r) {
-            mine[r] = PAIRED ? swiglu_rounded(acc[0][i][j][q + r] * factor0, acc[kMatrices - 1][i][j][q + r] * factor1)
-                             : f32_to_bf16(acc[0][i][j][q + r] * factor0);
+            for (int r = 0; r < 2; ++r) mine[r] = bf16_round(acc[0][i][j][q + r] * factor0 + bias[j]);
+            const float sent = odd_lane ? mine[0] : mine[1];
+            const float got = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(uint32_t, sent), 0xB1, 0xF, 0xF, true));
+            const bf16_t value = odd_lane ? gated_pair_rounded(got, mine[1], p.limit) : gated_pair_rounded(mine[0], got, p.limit);
+            reinterpret_cast<bf16_t*>(staged)[row * (2 * kRowDwords) + (wn0 + 32 * j + lane % 32) / 2] = value;
+          } else {
+            uint32_t mine[2];
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+              mine[r] = PAIRED ? swiglu_rounded(acc[0][i][j][q + r] * factor0, acc[kMatrices - 1][i][j][q + r] * factor1)
+                               : f32_to_bf16(acc[0][i][j][q + r] * factor0 + bias[j]);
+            }
+            // even lane keeps row q and sends its row q + 1; odd lane keeps row q + 1 and sends its row q
+            const uint32_t sent = odd_lane ? mine[0] : mine[1];
+            const uint32_t got = __builtin_amdgcn_mov_dpp(sent, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+            const uint32_t packed = odd_lane ? (got | (mine[1] << 16)) : (mine[0] | (got << 16));
+            staged[row * kRowDwords + (wn0 + 32 * j + (lane % 32 & ~1)) / 2] = packed;
           }
-          // even lane keeps row q and sends its row q + 1; odd lane keeps row q + 1 and sends its row q
-          const uint32_t sent = odd_lane ? mine[0] : mine[1];
-          const uint32_t got = __builtin_amdgcn_mov_dpp(sent, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
-          const uint32_t packed = odd_lane ? (got | (mine[1] << 16)) : (mine[0] | (got << 16));
-          staged[row * kRowDwords + (wn0 + 32 * j + (lane % 32 & ~1)) / 2] = packed;
         }
       }
     }
@@ -492,7 +520,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (PAIRED ? 2 : 1) * BN == 25
       const int item = tid + it * kThreads;
       const int staged_row = item / kRowChunks, chunk = item % kRowChunks;
       if (pass * kPassRows + staged_row < valid_rows)
-        *reinterpret_cast<u32x4_t*>(p.out + static_cast<size_t>(out_rows[it]) * p.width + n0 + chunk * 8) =
+        *reinterpret_cast<u32x4_t*>(p.out + static_cast<size_t>(out_rows[it]) * out_width + out_n0 + chunk * 8) =
             *reinterpret_cast<const u32x4_t*>(staged + staged_row * kRowDwords + chunk * 4);
     }
   }
@@ -514,10 +542,10 @@ static int check_bank(const char* who, const dew_moe_bank* bank, const char* nam
   return DEW_MOE_OK;
 }
 
-template <int FORMAT, bool PAIRED, int BM, int BN, int WM, int WN>
+template <int FORMAT, int MODE, int BM, int BN, int WM, int WN>
 static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
   constexpr size_t kShared = 3 * static_cast<size_t>(BM) * BK * sizeof(bf16_t);
-  auto kernel = grouped_gemm_kernel<FORMAT, PAIRED, BM, BN, WM, WN>;
+  auto kernel = grouped_gemm_kernel<FORMAT, MODE, BM, BN, WM, WN>;
   static bool configured = false;  // dynamic LDS above 64 KiB must be opted into once per kernel
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -536,47 +564,40 @@ static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
 // Tile choice from what the host knows (rows and experts; the routing itself stays on the device): 256-row
 // tiles when the average group fills them, 128-row tiles otherwise, and for decode-sized groups a 32-row tile
 // whose four wavefronts split the columns, so that thousands of wavefronts stream the weights at once.
-template <int FORMAT, bool PAIRED>
+template <int FORMAT, int MODE>
 static int launch_format(const char* who, const GemmParams& p, hipStream_t stream) {
-  constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4;  // FP8's raw registers do not fit the large tile
+  constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4;  // the 256-row tiles are kept to the FP4 banks
   const int average = p.rows / p.experts;
-  if (average < 24) return launch_tile<FORMAT, PAIRED, 32, 128, 1, 4>(who, p, stream);
-  if (kFp4 && average >= 768 && p.width % 256 == 0) {
-    if (PAIRED) return launch_tile<FORMAT, true, 256, 128, 1, 4>(who, p, stream);
-    return launch_tile<FORMAT, false, 256, 256, 1, 4>(who, p, stream);
+  if (average < 24) return launch_tile<FORMAT, MODE, 32, 128, 1, 4>(who, p, stream);
+  if constexpr (MODE == kSwigluOfTwo) {
+    if (kFp4 && average >= 768 && p.width % 256 == 0) return launch_tile<FORMAT, MODE, 256, 128, 1, 4>(who, p, stream);
+    return launch_tile<FORMAT, MODE, 128, 128, 1, 4>(who, p, stream);
+  } else {
+    if (kFp4 && average >= 768 && p.width % 256 == 0) return launch_tile<FORMAT, MODE, 256, 256, 1, 4>(who, p, stream);
+    if (p.width % 256 == 0 && static_cast<long long>(p.rows / 128 + 1) * (p.width / 256) >= 512)
+      return launch_tile<FORMAT, MODE, 128, 256, 1, 4>(who, p, stream);  // enough tiles to fill the chip twice over
+    return launch_tile<FORMAT, MODE, 128, 128, 1, 4>(who, p, stream);
   }
-  if (!PAIRED && p.width % 256 == 0 && static_cast<long long>(p.rows / 128 + 1) * (p.width / 256) >= 512)
-    return launch_tile<FORMAT, false, 128, 256, 1, 4>(who, p, stream);  // enough tiles to fill the chip twice over
-  return launch_tile<FORMAT, PAIRED, 128, 128, 1, 4>(who, p, stream);
 }
 
-template <bool PAIRED>
+template <int MODE>
 static int launch(const char* who, const GemmParams& p, int format, hipStream_t stream) {
   switch (format) {
     case DEW_MOE_W_FP8_BLOCK:
-      return launch_format<DEW_MOE_W_FP8_BLOCK, PAIRED>(who, p, stream);
+      return launch_format<DEW_MOE_W_FP8_BLOCK, MODE>(who, p, stream);
     case DEW_MOE_W_FP8_CHANNEL:
-      return launch_format<DEW_MOE_W_FP8_CHANNEL, PAIRED>(who, p, stream);
+      return launch_format<DEW_MOE_W_FP8_CHANNEL, MODE>(who, p, stream);
     case DEW_MOE_W_MXFP4:
-      return launch_format<DEW_MOE_W_MXFP4, PAIRED>(who, p, stream);
+      return launch_format<DEW_MOE_W_MXFP4, MODE>(who, p, stream);
     default:
-      return launch_format<DEW_MOE_W_NVFP4, PAIRED>(who, p, stream);
+      return launch_format<DEW_MOE_W_NVFP4, MODE>(who, p, stream);
   }
 }
 
-}  // namespace dew
-
-extern "C" int dew_moe_grouped_gemm(const void* x, const int32_t* gather, const int32_t* offsets,
-                                    const dew_moe_bank* w, const int32_t* scatter, void* out, int32_t rows,
-                                    void* stream) {
-  using namespace dew;
-  const char* who = "dew_moe_grouped_gemm";
-  if (int rc = check_bank(who, w, "weight")) return rc;
-  DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
-  if (rows == 0) return DEW_MOE_OK;
+static int fill_single(const char* who, GemmParams& p, const void* x, const int32_t* gather, const int32_t* offsets,
+                       const dew_moe_bank* w, const float* bias, const int32_t* scatter, void* out, int32_t rows) {
   DEW_REQUIRE(x && offsets && out, "%s: x, offsets and out must not be null", who);
   DEW_REQUIRE(aligned16(x) && aligned16(out), "%s: x and out must be 16-byte aligned", who);
-  GemmParams p{};
   p.x = static_cast<const bf16_t*>(x);
   p.gather = gather;
   p.offsets = offsets;
@@ -584,11 +605,48 @@ extern "C" int dew_moe_grouped_gemm(const void* x, const int32_t* gather, const 
   p.w0 = BankView{static_cast<const uint8_t*>(w->codes), w->scales, w->tensor_scale};
   p.w1 = p.w0;
   p.out = static_cast<bf16_t*>(out);
+  p.bias = bias;
   p.experts = w->experts;
   p.depth = w->depth;
   p.width = w->width;
   p.rows = rows;
-  return launch<false>(who, p, w->format, static_cast<hipStream_t>(stream));
+  return DEW_MOE_OK;
+}
+
+}  // namespace dew
+
+extern "C" int dew_moe_grouped_gemm_bias(const void* x, const int32_t* gather, const int32_t* offsets,
+                                         const dew_moe_bank* w, const float* bias, const int32_t* scatter, void* out,
+                                         int32_t rows, void* stream) {
+  using namespace dew;
+  const char* who = "dew_moe_grouped_gemm";
+  if (int rc = check_bank(who, w, "weight")) return rc;
+  DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
+  if (rows == 0) return DEW_MOE_OK;
+  GemmParams p{};
+  if (int rc = fill_single(who, p, x, gather, offsets, w, bias, scatter, out, rows)) return rc;
+  return launch<kPlain>(who, p, w->format, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int dew_moe_grouped_gemm(const void* x, const int32_t* gather, const int32_t* offsets,
+                                    const dew_moe_bank* w, const int32_t* scatter, void* out, int32_t rows,
+                                    void* stream) {
+  return dew_moe_grouped_gemm_bias(x, gather, offsets, w, nullptr, scatter, out, rows, stream);
+}
+
+extern "C" int dew_moe_gateup_interleaved(const void* x, const int32_t* gather, const int32_t* offsets,
+                                          const dew_moe_bank* gate_up, const float* bias, float limit, void* hidden,
+                                          int32_t rows, void* stream) {
+  using namespace dew;
+  const char* who = "dew_moe_gateup_interleaved";
+  if (int rc = check_bank(who, gate_up, "gate_up")) return rc;
+  DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
+  DEW_REQUIRE(limit > 0.0f, "%s: the clamp limit %g must be positive", who, static_cast<double>(limit));
+  if (rows == 0) return DEW_MOE_OK;
+  GemmParams p{};
+  if (int rc = fill_single(who, p, x, gather, offsets, gate_up, bias, nullptr, hidden, rows)) return rc;
+  p.limit = limit;
+  return launch<kInterleavedGated>(who, p, gate_up->format, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int dew_moe_gateup_swiglu(const void* x, const int32_t* gather, const int32_t* offsets,
@@ -617,5 +675,5 @@ extern "C" int dew_moe_gateup_swiglu(const void* x, const int32_t* gather, const
   p.depth = gate->depth;
   p.width = gate->width;
   p.rows = rows;
-  return launch<true>(who, p, gate->format, static_cast<hipStream_t>(stream));
+  return launch<kSwigluOfTwo>(who, p, gate->format, static_cast<hipStream_t>(stream));
 }

@@ -8,7 +8,8 @@ namespace dew {
 constexpr int LT = 64, LE = 64, LK = 16;
 
 __global__ __launch_bounds__(256) void router_logits_kernel(const bf16_t* __restrict__ x, const float* __restrict__ kernel,
-                                                            float* __restrict__ logits, int tokens, int depth, int experts) {
+                                                            const float* __restrict__ bias, float* __restrict__ logits,
+                                                            int tokens, int depth, int experts) {
   __shared__ float xs[LK][LT + 1];
   __shared__ float ks[LK][LE + 1];
   const int t0 = blockIdx.x * LT, e0 = blockIdx.y * LE;
@@ -47,7 +48,8 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const bf16_t* __rest
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int t = t0 + ty * 4 + i, e = e0 + tx * 4 + j;
-      if (t < tokens && e < experts) logits[static_cast<size_t>(t) * experts + e] = acc[i][j];
+      // a biased router (GPT-OSS's, src/dew/nn/gpt_oss.py:163-165) adds its fp32 bias to the finished sum
+      if (t < tokens && e < experts) logits[static_cast<size_t>(t) * experts + e] = bias ? acc[i][j] + bias[e] : acc[i][j];
     }
 }
 
@@ -65,15 +67,15 @@ __global__ void group_offsets_kernel(const int32_t* __restrict__ sizes, int32_t*
 
 }  // namespace dew
 
-extern "C" int dew_moe_router_logits(const void* x, const float* kernel, float* logits, int32_t tokens, int32_t depth,
-                                     int32_t experts, void* stream) {
+extern "C" int dew_moe_router_logits(const void* x, const float* kernel, const float* bias, float* logits, int32_t tokens,
+                                     int32_t depth, int32_t experts, void* stream) {
   using namespace dew;
   DEW_REQUIRE(tokens >= 0 && depth >= 1 && experts >= 1, "dew_moe_router_logits: tokens %d depth %d experts %d", tokens, depth, experts);
   if (tokens == 0) return DEW_MOE_OK;
   DEW_REQUIRE(x && kernel && logits, "dew_moe_router_logits: x, kernel and logits must not be null");
   const dim3 grid((tokens + LT - 1) / LT, (experts + LE - 1) / LE);
   hipLaunchKernelGGL(router_logits_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<const bf16_t*>(x),
-                     kernel, logits, tokens, depth, experts);
+                     kernel, bias, logits, tokens, depth, experts);
   return launched("router_logits_kernel");
 }
 

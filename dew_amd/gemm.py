@@ -47,6 +47,7 @@ class GroupedCase:
     epilogue: object = None
     out_dtype: torch.dtype = torch.bfloat16
     compute: torch.dtype = torch.bfloat16
+    epilogue_operands: tuple = ()
 
 
 _BANKS = (formats.NvFp4, formats.Fp8Blocks, formats.Fp8Channels, ops.PreparedBank)
@@ -54,6 +55,23 @@ _BANKS = (formats.NvFp4, formats.Fp8Blocks, formats.Fp8Channels, ops.PreparedBan
 
 def _shape(bank):
     return bank.shape
+
+
+def _bias_fits(case, bias) -> bool:
+    return bias is None or (torch.is_tensor(bias) and bias.dtype == torch.float32
+                            and tuple(bias.shape) == (_shape(case.rhs)[0], _shape(case.rhs)[2]))
+
+
+_EPILOGUES = {
+    None: lambda c: not c.epilogue_operands,
+    "swiglu": lambda c: c.paired is not None and not c.epilogue_operands,
+    # the reference's `_plus_bias` (src/dew/nn/moe.py:729-747): each expert's bias on its rows' fp32 sums
+    "plus_bias": lambda c: c.paired is None and len(c.epilogue_operands) == 1 and c.epilogue_operands[0] is not None
+                           and _bias_fits(c, c.epilogue_operands[0]),
+    # GPT-OSS's interleaved gate/up with its clamped gating (src/dew/nn/gpt_oss.py:111-121)
+    "gpt_oss_gated": lambda c: c.paired is None and len(c.epilogue_operands) == 2 and _bias_fits(c, c.epilogue_operands[0])
+                               and float(c.epilogue_operands[1]) > 0 and _shape(c.rhs)[2] % 256 == 0,
+}
 
 
 HIP = Kernel("hip", (
@@ -71,9 +89,11 @@ HIP = Kernel("hip", (
                 lambda c: f"width {_shape(c.rhs)[2]} is not a multiple of the 128-column tile", row="ragged width"),
     Requirement("pair", lambda c: c.paired is None or (_shape(c.paired) == _shape(c.rhs) and type(c.paired) is type(c.rhs)),
                 "a paired product's matrices share one shape and format"),
-    Requirement("epilogue", lambda c: c.epilogue in (None, "swiglu") and (c.epilogue is None or c.paired is not None),
-                lambda c: f"epilogue {c.epilogue!r}; the kernels fuse 'swiglu' over a pair and nothing else",
-                row="bias and clamp epilogues"),
+    Requirement("epilogue", lambda c: _EPILOGUES.get(c.epilogue, lambda c: False)(c),
+                lambda c: f"epilogue {c.epilogue!r} with {len(c.epilogue_operands)} operands"
+                          f"{' over a pair' if c.paired is not None else ''}; the kernels fuse 'swiglu' over a pair, "
+                          f"'plus_bias' [E, N] on one bank and 'gpt_oss_gated' (bias [E, N] or None, limit) on one "
+                          f"interleaved bank", row="other epilogues"),
 ))
 
 GROUPED = Op(GROUPED_MATMUL, (HIP,), preferred=lambda case: "hip",
@@ -94,18 +114,26 @@ def prepared(bank) -> ops.PreparedBank:
 
 
 def gemm(lhs: torch.Tensor, rhs, group_sizes, *, paired=None, gather: torch.Tensor | None = None,
-         scatter: torch.Tensor | None = None, epilogue: str | None = None, out_dtype=torch.bfloat16,
-         compute=torch.bfloat16, implementation: str | None = None):
+         scatter: torch.Tensor | None = None, epilogue: str | None = None, epilogue_operands: tuple = (),
+         out_dtype=torch.bfloat16, compute=torch.bfloat16, implementation: str | None = None):
     """Each group's rows of `lhs` (read at `gather` where given) times its matrix of the bank `rhs`, written
     at `scatter` where given. With `paired`, a second bank multiplied by the same rows in the same launch:
-    returns both products, or, with `epilogue='swiglu'`, their gated product alone."""
-    case = GroupedCase(lhs, rhs, paired, epilogue, out_dtype, compute)
+    returns both products, or, with `epilogue='swiglu'`, their gated product alone. On one bank,
+    `epilogue='plus_bias'` adds `epilogue_operands = (bias [E, N],)` to the fp32 sums before the rounding, and
+    `epilogue='gpt_oss_gated'` with `(bias or None, limit)` returns GPT-OSS's gated `[rows, N / 2]`."""
+    case = GroupedCase(lhs, rhs, paired, epilogue, out_dtype, compute, tuple(epilogue_operands))
     named = None if implementation in (None, "auto") else implementation
     selection.select(GROUPED, case, named)
     groups = GroupSizes.of(group_sizes)
     first = prepared(rhs)
+    if epilogue == "gpt_oss_gated":
+        if scatter is not None:
+            raise selection.KernelRefused(GROUPED_MATMUL, "hip", selection.Refusal("gated-scatter", "the gated product writes sorted rows"), iter(()))
+        return ops.gateup_interleaved(lhs, first, groups.offsets, bias=epilogue_operands[0], limit=float(epilogue_operands[1]),
+                                      gather=gather)
     if paired is None:
-        return ops.grouped_gemm(lhs, first, groups.offsets, gather=gather, scatter=scatter)
+        return ops.grouped_gemm(lhs, first, groups.offsets, gather=gather, scatter=scatter,
+                                bias=epilogue_operands[0] if epilogue == "plus_bias" else None)
     second = prepared(paired)
     if scatter is not None:
         raise selection.KernelRefused(GROUPED_MATMUL, "hip", selection.Refusal("pair-scatter", "a paired product writes sorted rows"), iter(()))

@@ -55,14 +55,25 @@ def expert_projection(x, kernel, group_sizes, dtype=None, implementation: str = 
                       bias=None, scatter: torch.Tensor | None = None) -> torch.Tensor:
     """The grouped matmul of `x`'s expert-sorted rows through each expert's matrix in `kernel`
     (src/dew/nn/moe.py:666-726): operands bf16, fp32 sums, one rounding; `Gathered` rows are read where
-    they lie; with `scatter` each output row lands at its entry's row."""
-    if bias is not None:
-        raise selection.KernelRefused(gemm.GROUPED_MATMUL, "hip", selection.Refusal(
-            "bias", "a per-expert bias epilogue is not built"), iter(()))
+    they lie; with `scatter` each output row lands at its entry's row; `bias [E, out]` is added to each
+    expert's rows' fp32 sums before the rounding."""
     tokens, rows = (x.tokens, x.rows) if isinstance(x, Gathered) else (x, None)
     compute = torch.bfloat16 if dtype is None else dtype
     return gemm.gemm(tokens, kernel, group_sizes, gather=rows, scatter=scatter, compute=compute, out_dtype=compute,
-                     implementation=_implementation(implementation))
+                     implementation=_implementation(implementation), **_biased(bias, compute))
+
+
+def _biased(bias, compute) -> dict:
+    """The epilogue adding each expert's bias to its rows' sums (src/dew/nn/moe.py:729-742): the bias rounded
+    to the compute dtype as an operand is, held in fp32."""
+    if bias is None:
+        return {}
+    return {"epilogue": "plus_bias", "epilogue_operands": (rounded_operand(bias, compute),)}
+
+
+def rounded_operand(value: torch.Tensor, compute) -> torch.Tensor:
+    """`value` rounded to `compute` and held in fp32 (the reference's `rounded_operand(...).astype(work)`)."""
+    return value.to(compute).to(torch.float32).contiguous()
 
 
 def paired_projections(x, first, second, group_sizes, dtype=None, implementation: str = "auto", precision=None):

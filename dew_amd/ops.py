@@ -59,15 +59,20 @@ def route(logits: torch.Tensor, top_k: int, *, score_function: str = "softmax", 
     return weights, indices
 
 
-def router_logits(x: torch.Tensor, kernel: torch.Tensor) -> torch.Tensor:
-    """fp32 gate logits `[..., E]` of bf16 tokens `[..., D]` and the fp32 gate kernel `[D, E]`."""
+def router_logits(x: torch.Tensor, kernel: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """fp32 gate logits `[..., E]` of bf16 tokens `[..., D]` and the fp32 gate kernel `[D, E]`, plus the
+    router's fp32 `bias [E]` where it has one."""
     _device(x, "x", torch.bfloat16), _device(kernel, "kernel", torch.float32)
     depth, experts = kernel.shape
     if x.shape[-1] != depth:
         raise KernelError(f"tokens are {x.shape[-1]} wide, the gate kernel {depth}")
+    if bias is not None:
+        _device(bias, "bias", torch.float32)
+        if bias.numel() != experts:
+            raise KernelError(f"the router bias holds {bias.numel()} values for {experts} experts")
     logits = torch.empty((*x.shape[:-1], experts), dtype=torch.float32, device=x.device)
-    _lib.check(_lib.library().dew_moe_router_logits(_ptr(x), _ptr(kernel), _ptr(logits), x.numel() // depth, depth, experts,
-                                                    _stream()), "dew_moe_router_logits")
+    _lib.check(_lib.library().dew_moe_router_logits(_ptr(x), _ptr(kernel), _ptr(bias), _ptr(logits), x.numel() // depth, depth,
+                                                    experts, _stream()), "dew_moe_router_logits")
     return logits
 
 
@@ -155,9 +160,20 @@ def prepare(bank) -> PreparedBank:
 # ---- products -----------------------------------------------------------------------------------------
 
 
+def _expert_bias(bias: torch.Tensor | None, experts: int, width: int) -> torch.Tensor | None:
+    """An epilogue bias `[E, N]`: values of the compute dtype (bf16) held in fp32, as the reference's `_biased`."""
+    if bias is None:
+        return None
+    _device(bias, "bias", torch.float32)
+    if tuple(bias.shape) != (experts, width):
+        raise KernelError(f"the bias is {tuple(bias.shape)}, the bank's outputs ({experts}, {width})")
+    return bias
+
+
 def grouped_gemm(x: torch.Tensor, bank: PreparedBank, offsets: torch.Tensor, *, gather: torch.Tensor | None = None,
-                 scatter: torch.Tensor | None = None, rows: int | None = None) -> torch.Tensor:
-    """`out[scatter[i]] = x[gather[i]] @ W[expert of sorted position i]`, bf16 `[rows, N]`."""
+                 scatter: torch.Tensor | None = None, rows: int | None = None,
+                 bias: torch.Tensor | None = None) -> torch.Tensor:
+    """`out[scatter[i]] = x[gather[i]] @ W[expert of sorted position i] (+ bias[expert])`, bf16 `[rows, N]`."""
     _device(x, "x", torch.bfloat16), _device(offsets, "offsets", torch.int32)
     experts, depth, width = bank.shape
     if x.shape[-1] != depth:
@@ -172,10 +188,36 @@ def grouped_gemm(x: torch.Tensor, bank: PreparedBank, offsets: torch.Tensor, *, 
         raise KernelError(f"{rows} rows asked of an x of {x.shape[0]}")
     if (gather is not None and gather.numel() < rows) or (scatter is not None and scatter.numel() < rows):
         raise KernelError("gather and scatter must cover every row")
+    bias = _expert_bias(bias, experts, width)
     out = torch.empty((rows, width), dtype=torch.bfloat16, device=x.device)
-    _lib.check(_lib.library().dew_moe_grouped_gemm(_ptr(x), _ptr(gather), _ptr(offsets), bank.descriptor, _ptr(scatter),
-                                                   _ptr(out), rows, _stream()), "dew_moe_grouped_gemm")
+    _lib.check(_lib.library().dew_moe_grouped_gemm_bias(_ptr(x), _ptr(gather), _ptr(offsets), bank.descriptor, _ptr(bias),
+                                                        _ptr(scatter), _ptr(out), rows, _stream()), "dew_moe_grouped_gemm")
     return out
+
+
+def gateup_interleaved(x: torch.Tensor, gate_up: PreparedBank, offsets: torch.Tensor, *, limit: float = 7.0,
+                       bias: torch.Tensor | None = None, gather: torch.Tensor | None = None,
+                       rows: int | None = None) -> torch.Tensor:
+    """GPT-OSS's fused projection and gating, one launch: `p = x[gather[i]] @ W[e] + bias[e]` with gate in the even
+    columns and up in the odd ones, `hidden = (clip(up) + 1) * min(gate, limit) * logistic(1.702 min(gate, limit))`,
+    bf16 `[rows, N / 2]`."""
+    _device(x, "x", torch.bfloat16), _device(offsets, "offsets", torch.int32)
+    experts, depth, width = gate_up.shape
+    if x.shape[-1] != depth:
+        raise KernelError(f"x rows are {x.shape[-1]} deep, the bank {depth}")
+    if offsets.numel() != experts + 1:
+        raise KernelError(f"offsets has {offsets.numel()} entries, the bank {experts} experts")
+    if gather is not None:
+        _device(gather, "gather", torch.int32)
+    rows = (gather.numel() if gather is not None else x.shape[0]) if rows is None else rows
+    if gather is None and rows > x.shape[0]:
+        raise KernelError(f"{rows} rows asked of an x of {x.shape[0]}")
+    bias = _expert_bias(bias, experts, width)
+    hidden = torch.empty((rows, width // 2), dtype=torch.bfloat16, device=x.device)
+    _lib.check(_lib.library().dew_moe_gateup_interleaved(_ptr(x), _ptr(gather), _ptr(offsets), gate_up.descriptor, _ptr(bias),
+                                                         float(limit), _ptr(hidden), rows, _stream()),
+               "dew_moe_gateup_interleaved")
+    return hidden
 
 
 def gateup_swiglu(x: torch.Tensor, gate: PreparedBank, up: PreparedBank, offsets: torch.Tensor, *,

@@ -71,10 +71,11 @@ int dew_moe_route(const float* logits, const float* bias /* nullable */, int32_t
                   int32_t expert_groups, int32_t groups_per_token, float* weights /* [T,k] */,
                   int32_t* indices /* [T,k] */, void* stream);
 
-/* Gate logits (src/dew/nn/moe.py:526-534): logits[T,E] = f32(x[T,D] bf16) @ kernel[D,E] f32, IEEE fp32.      */
+/* Gate logits (src/dew/nn/moe.py:526-534): logits[T,E] = f32(x[T,D] bf16) @ kernel[D,E] f32, IEEE fp32, plus
+ * bias[E] where the router has one (GPT-OSS's, src/dew/nn/gpt_oss.py:163-165).                              */
 int dew_moe_router_logits(const void* x /* bf16 [T,D] */, const float* kernel /* [D,E] */,
-                          float* logits /* [T,E] */, int32_t tokens, int32_t depth, int32_t experts,
-                          void* stream);
+                          const float* bias /* nullable [E] */, float* logits /* [T,E] */, int32_t tokens,
+                          int32_t depth, int32_t experts, void* stream);
 
 /* ---- Dispatch bookkeeping (src/dew/nn/moe.py:1101-1128 `_sorted_locally`) --------------------------
  * Stable counting sort of the R = tokens*top_k flattened expert ids: sizes[E] = bincount,
@@ -109,6 +110,20 @@ int dew_moe_prepare_bank(const dew_moe_bank* reference, void* prepared, dew_moe_
 int dew_moe_grouped_gemm(const void* x /* bf16 [*,K] */, const int32_t* gather, const int32_t* offsets,
                          const dew_moe_bank* w /* prepared, [E,K,N] */, const int32_t* scatter,
                          void* out /* bf16 [rows,N] */, int32_t rows, void* stream);
+
+/* The same with each expert's bias[E,N] (values of the compute dtype held in fp32) added to its rows' fp32
+ * sums before their one rounding (src/dew/nn/moe.py:729-742 _biased / _plus_bias; NULL = none).          */
+int dew_moe_grouped_gemm_bias(const void* x, const int32_t* gather, const int32_t* offsets,
+                              const dew_moe_bank* w, const float* bias, const int32_t* scatter, void* out,
+                              int32_t rows, void* stream);
+
+/* GPT-OSS's fused gate_up bank, gate in the even columns and up in the odd ones, with its epilogue
+ * (src/dew/nn/gpt_oss.py:111-121): projected = bf16(sum + bias), gate = min(even, limit), up = clip(odd,
+ * +-limit), hidden[rows, N/2] = (up + 1) * gate * logistic(1.702 gate), every operation rounded to bf16 as
+ * the reference's bf16 arrays round it.                                                                  */
+int dew_moe_gateup_interleaved(const void* x, const int32_t* gather, const int32_t* offsets,
+                               const dew_moe_bank* gate_up /* prepared, [E,K,2F] */, const float* bias /* nullable [E,2F] */,
+                               float limit, void* hidden /* bf16 [rows,F] */, int32_t rows, void* stream);
 
 /* gate and up in one launch with the SwiGLU epilogue: hidden[i] = swiglu(x[gather[i]] @ Wg[e], .. @ Wu[e])
  * with the reference's rounding sequence (src/dew/nn/activations.py:267-278): both products rounded to

@@ -19,12 +19,18 @@ What pins each function (tests/test_oracle_golden.py):
   order known answers of tests/test_gemm_nvfp4.py:37-38; form digest 7fb7f1b609cea47a.
 * `combine`: known answer of tests/test_moe_precision.py:652-674 (weights 1/2 +- 2^-11 give 2^-10).
 * `swiglu`: closed form, the two bf16 roundings checked on hand-computed cases.
+* `gpt_oss_mlp` (fp32 mode): `output` of tests/fixtures/gpt_oss/moe.npz at the reference's own tolerance (1.6e-4,
+  tests/test_gpt_oss.py:45-66): biased router, top-k on the logits, softmax of the chosen, interleaved gate/up
+  with both biases, clamp 7, (up + 1) * gate * logistic(1.702 gate). Dropping the down bias must move it by > 0.5.
 * `grouped_matmul`: tools/grouped_oracle.py:20-27 semantics (float64 per-group product) on integer inputs,
   where fp32 sums are exact.
 
 Parity unpinned (no byte fixture in the reference, closed form only): the exact bits of the softmax
 denominator's compensated sum (src/dew/nn/precision.py:1832); it moves router weights by at most one fp32
-ulp and no index.
+ulp and no index. `gpt_oss_gating`'s bf16 mode: where each bf16 rounding falls follows JAX's arithmetic on
+bf16 arrays (every elementwise operation rounds its result; the logistic is formed in fp32 and rounded once,
+src/dew/nn/activations.py:85-98), which no fixture of the reference records in bf16; GPT-OSS's final
+`sum(slots * weights)` is restated with fp32 weights and one rounding (`combine`).
 """
 
 import numpy as np
@@ -413,6 +419,78 @@ def expert_mlp(x, weights, indices, gate_w, up_w, down_w, *, dtype="bfloat16", f
     slots = slots.reshape(tokens, k, -1)
     out = combine(slots, weights, dtype=dtype)
     return out, {**plan, "gate": gate, "up": up, "hidden": hidden, "slots": slots}
+
+
+def gpt_oss_gating(projected, *, limit=7.0, dtype="bfloat16", exp=np.exp):
+    """GPT-OSS's activation of one interleaved projection `[..., 2F]` (src/dew/nn/gpt_oss.py:120-121):
+    gate = even columns clamped from above, up = odd columns clamped both ways
+    (src/dew/nn/activations.py:327-333), `(up + 1) * quick_gelu(gate)` with `quick_gelu(x) = x * logistic(1.702 x)`
+    (src/dew/nn/activations.py:72-74). In bf16 every operation rounds, the Python scalar 1.702 entering as a bf16."""
+    projected = np.asarray(projected, F32)
+    gate = np.minimum(projected[..., 0::2], F32(limit))
+    up = np.clip(projected[..., 1::2], F32(-limit), F32(limit))
+    rounded = bf16_round if dtype == "bfloat16" else (lambda v: np.asarray(v, F32))
+    slope = rounded(np.asarray(1.702, F32))
+    scaled = rounded(gate * slope)
+    sig = rounded((F32(1) / (F32(1) + exp(-scaled).astype(F32)).astype(F32)).astype(F32))
+    gelu = rounded(gate * sig)
+    return rounded(rounded(up + F32(1)) * gelu)
+
+
+def _biased_matmul(x, w, sizes, bias, *, dtype, factor=None):
+    """`grouped_matmul` with each expert's bias added to its rows' fp32 sums before the one rounding
+    (src/dew/nn/moe.py:729-742: the bias rounded to the compute dtype, held in fp32)."""
+    x = np.asarray(x, F32)
+    w = np.asarray(w, F32)
+    if dtype == "bfloat16":
+        x = bf16_round(x)
+    out = np.zeros((x.shape[0], w.shape[2]), F32)
+    start = 0
+    for group, size in enumerate(np.asarray(sizes).tolist()):
+        if size:
+            matrix = bf16_round(w[group]) if dtype == "bfloat16" else w[group]
+            summed = x[start:start + size] @ matrix
+            if factor is not None:
+                summed = summed.astype(F32) * F32(factor[group])
+            held = np.asarray(bias[group], F32)
+            summed = (summed.astype(F32) + (bf16_round(held) if dtype == "bfloat16" else held)).astype(F32)
+            out[start:start + size] = summed
+        start += size
+    return bf16_round(out) if dtype == "bfloat16" else out
+
+
+def gpt_oss_experts(x, weights, indices, gate_up, gate_up_bias, down, down_bias, *, dtype="bfloat16", limit=7.0,
+                    factors=(None, None)):
+    """`GptOssExperts.__call__` (src/dew/nn/gpt_oss.py:70-126) on one device: sort the slots by expert, the
+    fused biased projection, the clamped gating, the biased down projection back in slot order, and the
+    weighted sum over each token's slots. `gate_up [E, D, 2F]` and `down [E, F, D]` are the dequantized values."""
+    x = np.asarray(x, F32)
+    experts = gate_up.shape[0]
+    plan = sorted_by_expert(indices, experts)
+    rows = x[plan["rows"]]
+    projected = _biased_matmul(rows, gate_up, plan["sizes"], gate_up_bias, dtype=dtype, factor=factors[0])
+    hidden = gpt_oss_gating(projected, limit=limit, dtype=dtype)
+    output = _biased_matmul(hidden, down, plan["sizes"], down_bias, dtype=dtype, factor=factors[1])
+    slots = np.zeros_like(output)
+    slots[plan["order"]] = output
+    tokens, k = np.asarray(indices).shape
+    slots = slots.reshape(tokens, k, -1)
+    return combine(slots, weights, dtype=dtype), {**plan, "projected": projected, "hidden": hidden, "slots": slots}
+
+
+def gpt_oss_mlp(x, router_kernel, router_bias, gate_up, gate_up_bias, down, down_bias, *, top_k_count,
+                dtype="bfloat16", limit=7.0, factors=(None, None)):
+    """`GptOssMLP.__call__` (src/dew/nn/gpt_oss.py:155-171): logits = x @ kernel + bias in fp32, the k largest
+    logits, the softmax of the chosen logits (`renormalized_softmax`, src/dew/nn/moe.py:194-199), the experts."""
+    x = np.asarray(x, F32)
+    flat = x.reshape(-1, x.shape[-1])
+    logits = (router_logits(bf16_round(flat) if dtype == "bfloat16" else flat, router_kernel)
+              + np.asarray(router_bias, F32)).astype(F32)
+    weights, indices = route(logits, top_k_count, score_function="softmax", normalize_weights=True)
+    out, trace = gpt_oss_experts(flat, weights, indices, gate_up, gate_up_bias, down, down_bias, dtype=dtype,
+                                 limit=limit, factors=factors)
+    trace.update(logits=logits, weights=weights, indices=indices)
+    return out.reshape(*x.shape[:-1], -1), trace
 
 
 def gated_mlp(x, gate_w, up_w, down_w, *, dtype="bfloat16"):

@@ -1,0 +1,135 @@
+"""GPT-OSS's experts on the HIP kernels against the oracle: the bias epilogue, the interleaved clamped gating,
+and the whole layer (biased router, top-k of the logits, softmax of the chosen, experts, weighted sum)."""
+
+import numpy as np
+import pytest
+import torch
+
+from moe_cases import dequantized, quantize
+from oracle import moe_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from dew_amd import ops
+    ops.device_check()
+    return ops
+
+
+def bf16_np(tensor):
+    return tensor.detach().float().cpu().numpy()
+
+
+def bank_case(quant, experts, depth, width, sizes, seed, scale=0.02):
+    rng = np.random.default_rng(seed)
+    weight = torch.from_numpy((rng.standard_normal((experts, depth, width)) * scale).astype(np.float32))
+    bank = quantize(weight, quant)
+    x = torch.from_numpy(rng.standard_normal((int(np.sum(sizes)), depth)).astype(np.float32)).to(torch.bfloat16)
+    bias = torch.from_numpy(rng.standard_normal((experts, width)).astype(np.float32))
+    offsets = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    return bank, x, bias, offsets
+
+
+SIZES = [("decode", [3, 0, 9, 1]), ("medium", [150, 70, 0, 1]), ("wide", [700, 4, 20, 300]), ("large", [900, 800])]
+
+
+@pytest.mark.parametrize("quant", ["fp8_channel", "fp8_block", "mxfp4", "nvfp4"])
+@pytest.mark.parametrize("label,sizes", SIZES, ids=[s[0] for s in SIZES])
+def test_the_bias_meets_the_fp32_sums_before_their_one_rounding(ops, quant, label, sizes):
+    bank, x, bias, offsets = bank_case(quant, len(sizes), 256, 512, sizes, seed=len(label) + len(quant))
+    held = bias.to(torch.bfloat16).float()          # rounded to the compute dtype, held in fp32
+    values, factor = dequantized(bank)
+    want = oracle._biased_matmul(bf16_np(x), values, sizes, bias.numpy(), dtype="bfloat16", factor=factor)
+    scatter = torch.from_numpy(np.random.default_rng(5).permutation(x.shape[0]).astype(np.int32))
+    prepared = ops.prepare(bank.to("cuda"))
+    got = ops.grouped_gemm(x.cuda(), prepared, torch.from_numpy(offsets).cuda(), bias=held.cuda(), scatter=scatter.cuda())
+    got = bf16_np(got)[scatter.numpy()]
+    assert np.abs(got - want).max() <= 2 ** -8 * np.abs(want).max()
+    assert (got == want).mean() > 0.97
+    # a product whose rounding comes before the bias would differ: the bias is of the outputs' size
+    late = oracle.bf16_round(oracle.grouped_matmul(bf16_np(x), values, sizes, factor=factor) + held.numpy()[np.repeat(
+        np.arange(len(sizes)), sizes)])
+    assert (late != want).mean() > 0.01
+
+
+@pytest.mark.parametrize("quant", ["fp8_channel", "fp8_block", "mxfp4", "nvfp4"])
+@pytest.mark.parametrize("label,sizes", SIZES, ids=[s[0] for s in SIZES])
+def test_interleaved_gate_up_with_the_clamped_gating(ops, quant, label, sizes):
+    # weights large enough that some sums pass the clamp at 7
+    bank, x, bias, offsets = bank_case(quant, len(sizes), 256, 512, sizes, seed=3 * len(label) + len(quant), scale=0.2)
+    held = bias.to(torch.bfloat16).float()
+    values, factor = dequantized(bank)
+    projected = oracle._biased_matmul(bf16_np(x), values, sizes, bias.numpy(), dtype="bfloat16", factor=factor)
+    assert (projected > 7).mean() > 0.005 and (projected < -7).mean() > 0.005
+    want = oracle.gpt_oss_gating(projected)
+    rng = np.random.default_rng(9)
+    gather = rng.integers(0, x.shape[0], size=x.shape[0]).astype(np.int32)
+    want_gathered = oracle.gpt_oss_gating(oracle._biased_matmul(bf16_np(x)[gather], values, sizes, bias.numpy(), dtype="bfloat16",
+                                                                factor=factor))
+    prepared = ops.prepare(bank.to("cuda"))
+    od = torch.from_numpy(offsets).cuda()
+    got = bf16_np(ops.gateup_interleaved(x.cuda(), prepared, od, bias=held.cuda(), limit=7.0))
+    assert got.shape == (x.shape[0], 256)
+    # the kernel's own projection is within one bf16 ulp of the oracle's; gate it with the oracle's arithmetic
+    own = bf16_np(ops.grouped_gemm(x.cuda(), prepared, od, bias=held.cuda()))
+    assert np.array_equal(got, oracle.gpt_oss_gating(own)) or (got == oracle.gpt_oss_gating(own)).mean() > 0.999
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= 2e-2 * scale
+    assert (got == want).mean() > 0.9
+    got_gathered = bf16_np(ops.gateup_interleaved(x.cuda(), prepared, od, bias=held.cuda(), gather=torch.from_numpy(gather).cuda()))
+    assert np.abs(got_gathered - want_gathered).max() <= 2e-2 * scale and (got_gathered == want_gathered).mean() > 0.9
+
+
+def test_unrouted_tail_rows_of_the_gated_product_are_zero(ops):
+    bank, x, bias, offsets = bank_case("mxfp4", 2, 256, 256, [5, 6], seed=2)
+    rows = 40
+    xs = torch.cat([x, torch.ones((rows - x.shape[0], 256), dtype=torch.bfloat16)]).cuda()
+    got = bf16_np(ops.gateup_interleaved(xs, ops.prepare(bank.to("cuda")), torch.from_numpy(offsets).cuda(),
+                                         bias=bias.to(torch.bfloat16).float().cuda(), rows=rows))
+    assert got.shape == (rows, 128) and np.all(got[11:] == 0) and np.any(got[:11] != 0)
+
+
+@pytest.mark.parametrize("quant", ["mxfp4", "fp8_block"])
+def test_gpt_oss_layer_matches_the_oracle(quant):
+    from dew_amd import gpt_oss
+
+    tokens, hidden, intermediate, experts, top_k = 96, 256, 256, 8, 4
+    rng = np.random.default_rng(11)
+    x = torch.from_numpy(rng.standard_normal((2, tokens // 2, hidden)).astype(np.float32)).to(torch.bfloat16)
+    router_kernel = torch.from_numpy((rng.standard_normal((hidden, experts)) * hidden ** -0.5).astype(np.float32))
+    router_bias = torch.from_numpy((rng.standard_normal(experts) * 0.1).astype(np.float32))
+    gate_up = quantize(torch.from_numpy((rng.standard_normal((experts, hidden, 2 * intermediate)) * hidden ** -0.5).astype(np.float32)), quant)
+    down = quantize(torch.from_numpy((rng.standard_normal((experts, intermediate, hidden)) * intermediate ** -0.5).astype(np.float32)), quant)
+    gate_bias = torch.from_numpy(rng.standard_normal((experts, 2 * intermediate)).astype(np.float32))
+    down_bias = torch.from_numpy(rng.standard_normal((experts, hidden)).astype(np.float32))
+    gate_up_values, gate_up_factor = dequantized(gate_up)
+    down_values, down_factor = dequantized(down)
+    want, trace = oracle.gpt_oss_mlp(bf16_np(x), router_kernel.numpy(), router_bias.numpy(), gate_up_values, gate_bias.numpy(),
+                                     down_values, down_bias.numpy(), top_k_count=top_k, factors=(gate_up_factor, down_factor))
+    variables = {"params": {"router": {"kernel": router_kernel.cuda(), "bias": router_bias.cuda()},
+                            "experts": {"gate_up_proj_bias": gate_bias.cuda(), "down_proj_bias": down_bias.cuda()}},
+                 "quantization": {"experts": {"gate_up_proj": gate_up.to("cuda"), "down_proj": down.to("cuda")}}}
+    layer = gpt_oss.GptOssMLP(hidden, intermediate, experts, top_k)
+    got = layer.apply(variables, x.cuda())
+    assert got.shape == x.shape and got.dtype == torch.bfloat16
+    logits = bf16_np(layer._bound(variables, ()).logits(x.cuda())).reshape(-1, experts)
+    assert np.abs(logits - trace["logits"]).max() <= 1e-5 * max(1.0, np.abs(trace["logits"]).max())
+    peak_error, elementwise = oracle.relative_errors(bf16_np(got).reshape(want.shape), want)
+    assert peak_error <= 2e-2 and elementwise <= 2e-2          # max|got - want| / max|want| and element-wise with an rms floor
+    assert peak_error <= 8e-3
+
+
+def test_gpt_oss_requirements_are_refused_by_name(ops):
+    from dew_amd import gemm, selection
+
+    bank, x, bias, offsets = bank_case("mxfp4", 2, 256, 256, [5, 6], seed=2)
+    sizes = gemm.GroupSizes.of(torch.tensor([5, 6], dtype=torch.int32, device="cuda"))
+    with pytest.raises(selection.KernelRefused, match="epilogue"):
+        gemm.gemm(x.cuda(), bank.to("cuda"), sizes, epilogue="plus_bias", epilogue_operands=(bias[:, :8].cuda(),),
+                  implementation="hip")
+    with pytest.raises(selection.KernelRefused, match="epilogue"):
+        gemm.gemm(x.cuda(), bank.to("cuda"), sizes, epilogue="gpt_oss_gated", epilogue_operands=(None, -1.0), implementation="hip")
+    out = gemm.gemm(x.cuda(), bank.to("cuda"), sizes, epilogue="gpt_oss_gated", epilogue_operands=(None, 7.0))
+    assert out.shape == (11, 128)

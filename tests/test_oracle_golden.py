@@ -253,3 +253,33 @@ def test_bf16_combine_weighs_in_fp32_and_rounds_once():
     slots = np.array([[[1.0], [-1.0]]], np.float32)                   # tests/test_moe_precision.py:652-674
     weights = np.array([[0.5 + 2 ** -11, 0.5 - 2 ** -11]], np.float32)
     assert oracle.combine(slots, weights)[0, 0] == 2.0 ** -10
+
+
+def test_gpt_oss_mlp_matches_the_reference_fixture():
+    """tests/fixtures/gpt_oss/moe.npz of the reference, at its own test's tolerance (tests/test_gpt_oss.py:45-66)."""
+    held = golden("gpt_oss/moe.npz")
+
+    def run(down_bias):
+        out, _ = oracle.gpt_oss_mlp(held["hidden"], held["router.weight"].T, held["router.bias"], held["experts.gate_up_proj"],
+                                    held["experts.gate_up_proj_bias"], held["experts.down_proj"], down_bias,
+                                    top_k_count=2, dtype="float32")
+        return out
+
+    np.testing.assert_allclose(run(held["experts.down_proj_bias"]), held["output"], atol=1.6e-4, rtol=0)
+    assert np.abs(run(np.zeros_like(held["experts.down_proj_bias"])) - held["output"]).max() > 0.5
+
+
+def test_gpt_oss_gating_rounds_every_operation_in_bf16():
+    """Hand-followed cases: gate 1, up 0.5 -> t = bf16(1.703125) ; s = bf16(logistic(1.703125)) = 0.84765625;
+    q = bf16(1 * s); u1 = 1.5; out = bf16(1.5 * 0.84765625) = 1.2734375 (1.271484375 rounds to 8 bits). Clamps: gate
+    9 -> 7, up -9 -> -7 gives (1 - 7) * bf16(7 * bf16(logistic(bf16(7 * 1.703125))))."""
+    out = oracle.gpt_oss_gating(np.array([[1.0, 0.5, 9.0, -9.0]], np.float32))
+    s = oracle.bf16_round(np.float32(1.0) / (np.float32(1.0) + np.exp(np.float32(-1.703125))))
+    assert s == np.float32(0.84765625)
+    assert out[0, 0] == oracle.bf16_round(np.float32(1.5) * s) == np.float32(1.2734375)
+    t = oracle.bf16_round(np.float32(7.0 * 1.703125))
+    s7 = oracle.bf16_round(np.float32(1.0) / (np.float32(1.0) + np.exp(-t)))
+    assert out[0, 1] == oracle.bf16_round(np.float32(-6.0) * oracle.bf16_round(np.float32(7.0) * s7))
+    # fp32 mode rounds nowhere and uses 1.702 itself
+    exact = oracle.gpt_oss_gating(np.array([[1.0, 0.5]], np.float32), dtype="float32")
+    assert abs(exact[0, 0] - 1.5 / (1 + np.exp(-1.702))) < 1e-6
