@@ -42,9 +42,10 @@ const char* dew_moe_kernel_fields(void) { return "name,tile_m,tile_n,tile_k,wave
 const char* dew_moe_kernels(void) {
   return "route,1 token/wave,-,-,4,-,f32 logits\n"
          "permute_small|permute_count+scan+scatter,2048 slots/block,-,-,4,-,i32 ballot+LDS histogram\n"
-         "grouped_gemm<large>,256,256 (paired 2x128),64,4 (1x4),v_mfma_f32_32x32x16_bf16,bf16 rows via global_load_lds x nvfp4|mxfp4 fragments from global\n"
-         "grouped_gemm<medium>,128,128 (paired 2x128),64,4 (1x4),v_mfma_f32_32x32x16_bf16,bf16 x {fp8 block|fp8 channel|nvfp4|mxfp4}\n"
+         "grouped_gemm<large>,256,256 (paired 2x128),64,4 (1x4),v_mfma_f32_32x32x16_bf16,bf16 rows via global_load_lds x nvfp4|mxfp4 fragments from global; 1 block/CU\n"
+         "grouped_gemm<medium>,128,256 (paired 2x128) | 128,64,4 (1x4),v_mfma_f32_32x32x16_bf16,bf16 x {fp8 block|fp8 channel|nvfp4|mxfp4}; 2 blocks/CU\n"
          "grouped_gemm<decode>,32,128 (paired 2x128),64,4 (1x4),v_mfma_f32_32x32x16_bf16,weight streaming for groups under 24 rows\n"
+         "grouped_gemm epilogues,-,-,-,-,-,plain (+bias) | swiglu of two banks | interleaved gate/up clamped 1.702 gating (+bias); tile staged in LDS and stored as whole rows\n"
          "combine,8 columns/lane,-,-,4,-,bf16 slots x f32 weights\n";
 }
 
