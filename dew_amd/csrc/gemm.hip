@@ -101,6 +101,15 @@ __device__ __forceinline__ bf16x8_t fragment_fp4_pow2(uint32_t word, float scale
       __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 3))});
 }
 
+// Dynamic LDS of a block: the three-stage ring of A rows, or the staged output tile where that is larger
+// (the 32-row tile of 256 columns).
+template <int BM, int BN, int MODE>
+constexpr size_t shared_bytes() {
+  constexpr size_t ring = 3 * static_cast<size_t>(BM) * BK * 2;
+  constexpr size_t staged = static_cast<size_t>(BM / ((BN == 256 && BM > 32) ? 2 : 1)) * ((MODE == 2 ? BN / 2 : BN) / 2 + 4) * 4;
+  return ring > staged ? ring : staged;
+}
+
 // Instruction order of one phase of the main loop, stated to the scheduler: `MFMAS` matrix instructions in a
 // row, the phase's `DSR` operand reads issued one behind each of the first of them (so they are long done
 // when the next phase multiplies them), and the phase's other work (vector ALU, LDS stores, global loads)
@@ -454,13 +463,13 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     factor0 = 256.0f * p.w0.tensor_scale[expert];
     if (PAIRED) factor1 = 256.0f * p.w1.tensor_scale[expert];
   }
-  constexpr int kPasses = BN == 256 ? 2 : 1;
+  constexpr int kPasses = (BN == 256 && TI > 1) ? 2 : 1;
   constexpr int kPassTiles = TI / kPasses, kPassRows = BM / kPasses;
   constexpr int kRowDwords = kOutBN / 2 + 4;  // a staged row: the tile's output columns in bf16 and 16 bytes of padding
   constexpr int kRowChunks = kOutBN / 8;      // 16-byte pieces of an output row
   constexpr int kStoreIters = kPassRows * kRowChunks / kThreads;
   static_assert(kPassRows * kRowChunks % kThreads == 0, "whole store rounds");
-  static_assert(TI % kPasses == 0 && kPassRows * kRowDwords * 4 <= kStages * kStageChunks * 16, "staged tile fits the A ring");
+  static_assert(TI % kPasses == 0 && kPassRows * kRowDwords * 4 <= shared_bytes<BM, BN, MODE>(), "staged tile fits the LDS");
   uint32_t* staged = reinterpret_cast<uint32_t*>(lds);
   const bool odd_lane = lane & 1;
   const int out_width = kGated ? p.width / 2 : p.width, out_n0 = kGated ? n0 / 2 : n0;
@@ -544,7 +553,7 @@ static int check_bank(const char* who, const dew_moe_bank* bank, const char* nam
 
 template <int FORMAT, int MODE, int BM, int BN, int WM, int WN>
 static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
-  constexpr size_t kShared = 3 * static_cast<size_t>(BM) * BK * sizeof(bf16_t);
+  constexpr size_t kShared = shared_bytes<BM, BN, MODE>();
   auto kernel = grouped_gemm_kernel<FORMAT, MODE, BM, BN, WM, WN>;
   static bool configured = false;  // dynamic LDS above 64 KiB must be opted into once per kernel
   if (!configured) {
@@ -568,7 +577,12 @@ template <int FORMAT, int MODE>
 static int launch_format(const char* who, const GemmParams& p, hipStream_t stream) {
   constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4;  // the 256-row tiles are kept to the FP4 banks
   const int average = p.rows / p.experts;
-  if (average < 24) return launch_tile<FORMAT, MODE, 32, 128, 1, 4>(who, p, stream);
+  if (average < 24) {
+    // one bank: 256 columns a block where that still leaves every CU several blocks, so that a launch is one round
+    if (MODE != kSwigluOfTwo && p.width % 256 == 0 && static_cast<long long>(p.experts) * (p.width / 256) >= 768)
+      return launch_tile<FORMAT, MODE, 32, 256, 1, 4>(who, p, stream);
+    return launch_tile<FORMAT, MODE, 32, 128, 1, 4>(who, p, stream);
+  }
   if constexpr (MODE == kSwigluOfTwo) {
     if (kFp4 && average >= 768 && p.width % 256 == 0) return launch_tile<FORMAT, MODE, 256, 128, 1, 4>(who, p, stream);
     return launch_tile<FORMAT, MODE, 128, 128, 1, 4>(who, p, stream);
