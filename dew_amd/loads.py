@@ -1,0 +1,122 @@
+"""A quantized checkpoint's expert banks taken to the kernels' formats at load time, without decoding a value:
+the host-side mirror of the reference's `packed_banks` / `with_banks` (src/dew/interop/quantized_loads.py:106-168)
+for MXFP4 sources (gpt-oss's `*_blocks` / `*_scales`), and the same service for FP8 128 x 128 block sources
+(`weight` / `weight_scale_inv`, which the reference decodes at load, src/dew/interop/codecs.py:638-648).
+
+Tensors may live on the host or the device; every step is a torch index or bit operation, so a bank loaded to the
+GPU is re-laid there. The banks go into the `'quantization'` collection at the path their parameter had.
+"""
+
+import dataclasses
+import logging
+from collections.abc import Mapping
+
+import torch
+
+from . import codecs, formats
+
+_log = logging.getLogger(__name__)
+
+MXFP4_SUFFIXES = ("_blocks", "_scales")
+"""The two tensors an MXFP4 weight is stored as (src/dew/interop/codecs.py:463)."""
+FP8_SUFFIXES = (".weight", ".weight_scale_inv")
+
+
+@dataclasses.dataclass(frozen=True)
+class Unread:
+    """The shape and dtype of a leaf whose values are held elsewhere (the reference's `unread.Unread`)."""
+
+    shape: tuple
+    dtype: torch.dtype
+
+
+def source_quantization(config: Mapping) -> str | None:
+    found = config.get("quantization_config") or {}
+    return found.get("quant_method")
+
+
+def packed_banks(tensors: Mapping[str, torch.Tensor], config: Mapping) -> tuple[dict, dict]:
+    """`tensors` with each MXFP4 expert bank taken out of the source's decoding, and those banks by their source
+    names (`formats.NvFp4`, exactly the MXFP4 values: `codecs.mxfp4_as_nvfp4`); in each one's place an `Unread`
+    of its decoded shape. A bank whose depth is no whole NVFP4 stages, whose experts' group powers span past one
+    tensor scale's reach, or that holds no experts stays as the source states it and is named in the log."""
+    if source_quantization(config) != "mxfp4":
+        raise ValueError("packed_experts serves an MXFP4 source's expert banks (gpt-oss's quant_method mxfp4); "
+                         f"this source's quantization is {config.get('quantization_config')!r}")
+    tensors, banks = dict(tensors), {}
+    names = sorted(name[:-len(MXFP4_SUFFIXES[0])] for name in tensors
+                   if name.endswith(MXFP4_SUFFIXES[0]) and name[:-len(MXFP4_SUFFIXES[0])] + MXFP4_SUFFIXES[1] in tensors)
+    for name in names:
+        blocks, scales = (tensors[name + suffix] for suffix in MXFP4_SUFFIXES)
+        powers = None
+        if blocks.ndim != 4:
+            reason = "it holds no experts"
+        elif blocks.shape[2] * codecs.GROUP % formats.NVFP4_STAGE:
+            reason = f"its depth {blocks.shape[2] * codecs.GROUP} is no whole {formats.NVFP4_STAGE}-deep stages"
+        else:
+            powers = codecs.mxfp4_tensor_powers(blocks, scales)
+            reason = "its experts' group powers span past one tensor scale's reach"
+        if powers is None:
+            _log.warning("packed_experts: %s stays dense: %s", name, reason)
+            continue
+        experts, outputs, groups, _ = blocks.shape
+        banks[name] = formats.NvFp4.of(*codecs.mxfp4_as_nvfp4(blocks, scales, powers))
+        for suffix in MXFP4_SUFFIXES:
+            del tensors[name + suffix]
+        tensors[name] = Unread((experts, groups * codecs.GROUP, outputs), torch.float32)
+    return tensors, banks
+
+
+def fp8_block_bank(weights, scale_invs) -> formats.Fp8Blocks:
+    """One projection's experts, each stored `[out, in]` e4m3 with `[out/128, in/128]` fp32 inverse scales
+    (DeepSeek-V3 / Qwen3-FP8 checkpoints), as the `[E, in, out]` bank the kernels multiply, still quantized."""
+    codes = torch.stack([weight.view(torch.uint8).transpose(0, 1) for weight in weights]).contiguous()
+    scales = torch.stack([scale.to(torch.float32).transpose(0, 1) for scale in scale_invs]).contiguous()
+    experts, depth, width = codes.shape
+    if depth % 128 or width % 128 or tuple(scales.shape) != (experts, depth // 128, width // 128):
+        raise ValueError(f"an FP8 block bank is [E, in, out] in whole 128s with [E, in/128, out/128] scales, got codes "
+                         f"{tuple(codes.shape)} and scales {tuple(scales.shape)}")
+    return formats.Fp8Blocks(codes, scales)
+
+
+def fp8_expert_banks(tensors: Mapping[str, torch.Tensor], prefix: str, experts: int,
+                     projections=("gate_proj", "up_proj", "down_proj")) -> tuple[dict, dict]:
+    """`tensors` without `prefix.{e}.{projection}.weight[_scale_inv]` for e < experts, and the stacked FP8 block
+    banks by projection name."""
+    tensors, banks = dict(tensors), {}
+    for projection in projections:
+        names = [f"{prefix}.{e}.{projection}" for e in range(experts)]
+        banks[projection] = fp8_block_bank([tensors[name + FP8_SUFFIXES[0]] for name in names],
+                                           [tensors[name + FP8_SUFFIXES[1]] for name in names])
+        for name in names:
+            for suffix in FP8_SUFFIXES:
+                del tensors[name + suffix]
+    return tensors, banks
+
+
+def with_banks(variables: Mapping, paths: Mapping[str, tuple], banks: Mapping) -> dict:
+    """`variables` with each bank in `'quantization'` under the path its source name binds (`paths[name]`, a
+    path into `'params'`), the leaf there taken out of `'params'`; a name that binds no path is refused
+    (src/dew/interop/quantized_loads.py:146-168)."""
+    if not banks:
+        return dict(variables)
+    params = _copied(variables.get("params", {}))
+    held = _copied(variables.get("quantization", {}))
+    for name, bank in banks.items():
+        path = paths.get(name)
+        if not path:
+            raise ValueError(f"{name} binds no path, which a packed bank does not take: it holds a whole "
+                             "[experts, in, out] matrix at one path")
+        node = params
+        for key in path[:-1]:
+            node = node.get(key, {})
+        node.pop(path[-1], None)
+        node = held
+        for key in path[:-1]:
+            node = node.setdefault(key, {})
+        node[path[-1]] = bank
+    return {**variables, "params": params, "quantization": held}
+
+
+def _copied(tree):
+    return {key: _copied(value) if isinstance(value, dict) else value for key, value in tree.items()}
