@@ -135,8 +135,10 @@ __global__ __launch_bounds__(kPermuteThreads) void permute_scatter_kernel(Permut
   }
 }
 
-// All of the above in one launch for at most kSlotsPerBlock slots (a decode step): one block counts, scans
-// and scatters, with the LDS histogram as the only intermediate.
+// All of the above in one launch for at most kSmallSlots slots (a decode step, a small prefill): one block
+// counts, scans and scatters, each wavefront a contiguous run of the slots, with the LDS histogram as the only
+// intermediate.
+constexpr int kSmallSlots = 2048;  // beyond this three launches over many blocks are faster (measured at 4096)
 __global__ __launch_bounds__(kPermuteThreads) void permute_small_kernel(PermuteParams p) {
   extern __shared__ int32_t running[];  // [kPermuteWaves][buckets] then [buckets + 1] totals
   int32_t* totals = running + kPermuteWaves * p.buckets;
@@ -256,7 +258,7 @@ extern "C" int dew_moe_permute(const int32_t* indices, int32_t tokens, int32_t t
   uintptr_t base = (reinterpret_cast<uintptr_t>(workspace) + 255) & ~static_cast<uintptr_t>(255);
   p.counts = reinterpret_cast<int32_t*>(base);
   p.bases = p.counts + static_cast<size_t>(p.blocks) * p.buckets;
-  if (p.blocks <= 1) {
+  if (slots <= kSmallSlots) {  // one block does it all faster than three launches
     hipLaunchKernelGGL(permute_small_kernel, dim3(1), dim3(kPermuteThreads),
                        sizeof(int32_t) * ((kPermuteWaves + 1) * p.buckets + 1), s, p);
     return launched("permute_small_kernel");
