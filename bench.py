@@ -75,7 +75,7 @@ def build_workload(case, device, seed=0):
 class Stepper:
     """One step of the hot path, launch by launch, with optional HIP events around the gate/up launch."""
 
-    def __init__(self, case, data):
+    def __init__(self, case, data, split=False):
         import torch
 
         from dew_amd import gemm, ops
@@ -86,6 +86,7 @@ class Stepper:
         tokens = case.tokens
         self.dense_offsets = torch.tensor([0, tokens], dtype=torch.int32, device=data["x"].device)
         self.events = []
+        self.split = split
 
     def __call__(self, timed: bool = False):
         torch, ops, case, data = self.torch, self.ops, self.case, self.data
@@ -94,11 +95,22 @@ class Stepper:
         if timed:
             start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             start.record()
-        hidden = ops.gateup_swiglu(data["x"], self.gate, self.up, plan.offsets, gather=plan.rows)
+        routed = case.tokens * case.top_k
+        if self.split and ops.prefers_split(self.gate, routed):
+            # an MXFP4 bank and groups of hundreds of rows: rows as two e4m3 terms, scaled matrix instructions
+            pieces = ops.split_rows(data["x"])
+            if timed:
+                start.record()
+            hidden = ops.gateup_swiglu_split(*pieces, self.gate, self.up, plan.offsets, gather=plan.rows)
+        else:
+            hidden = ops.gateup_swiglu(data["x"], self.gate, self.up, plan.offsets, gather=plan.rows)
         if timed:
             stop.record()
             self.events.append((start, stop))
-        slots = ops.grouped_gemm(hidden, self.down, plan.offsets, scatter=plan.order)
+        if self.split and ops.prefers_split(self.down, routed):
+            slots = ops.grouped_gemm_split(*ops.split_rows(hidden), self.down, plan.offsets, scatter=plan.order)
+        else:
+            slots = ops.grouped_gemm(hidden, self.down, plan.offsets, scatter=plan.order)
         addend = None
         if self.shared is not None:
             shared_hidden = ops.gateup_swiglu(data["x"], self.shared[0], self.shared[1], self.dense_offsets)
@@ -203,6 +215,9 @@ def main():
     parser.add_argument("--calibrate-copy", action="store_true",
                         help="only run the plain copy probe (1 GiB read + 1 GiB written, 5 launches): the known traffic "
                              "that rocprofv3's FETCH_SIZE / WRITE_SIZE are scaled by")
+    parser.add_argument("--split", action="store_true",
+                        help="MXFP4 banks with groups of hundreds of rows: rows split into two e4m3 terms and the scaled matrix "
+                             "instruction instead of the bf16 one (same exact products; the default measured faster overall)")
     parser.add_argument("--graph", choices=["auto", "on", "off"], default="auto",
                         help="replay the step as one captured HIP graph (auto: for the launch-bound configs c1 and c3)")
     args = parser.parse_args()
@@ -226,7 +241,7 @@ def main():
         return
     case = CONFIGS[args.config]
     data = build_workload(case, device)
-    stepper = Stepper(case, data)
+    stepper = Stepper(case, data, split=args.split)
 
     graphed = args.graph == "on" or (args.graph == "auto" and args.config in ("c1", "c3"))
     for _ in range(args.warmup):
@@ -287,7 +302,8 @@ def main():
                              "frac_of_sustained": round(roofline["achieved"] / (sustained_copy if decode else sustained_mfma), 4),
                              "note": "measured in this run by dew_moe_probe_mfma / dew_moe_probe_copy: the rate the chip holds on "
                                      "random data at its power limit, below the published peak"}
-    roofline["kernel"] = "grouped_gemm_kernel<paired gate/up + SwiGLU>"
+    roofline["kernel"] = "grouped_gemm_kernel<paired gate/up + SwiGLU>" + (
+        " on split rows (v_mfma_scale_f32_32x32x64_f8f6f4, two e4m3 terms x FP4)" if args.split and case.quant == "mxfp4" else "")
     roofline["kernel_ms"] = round(gateup_ms, 4)
 
     result = {

@@ -30,6 +30,12 @@ typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;  // a 16-byte register quad (native vector: stays in VGPRs)
+typedef __attribute__((ext_vector_type(8))) int i32x8_t;       // an operand of the scaled matrix instruction
+
+// Kernel-side format of an MXFP4 bank multiplied by activation rows already split into two e4m3 terms
+// (dew_moe_split_rows): v_mfma_scale_f32_32x32x64_f8f6f4 takes the FP4 codes and their power-of-two block scales
+// as they are stored, so the weights are not dequantized at all.
+constexpr int kFormatMxSplit = 5;
 
 constexpr int BK = 64;
 constexpr int kThreads = 256;
@@ -49,6 +55,7 @@ struct GemmParams {
   const int32_t* scatter;
   BankView w0, w1;
   bf16_t* out;
+  const uint8_t* a_scale;  // split activations: each source row's e8m0 scale
   const float* bias;  // [experts, width] values of the compute dtype held in fp32, or null
   float limit;        // the interleaved gated epilogue's clamp
   int experts, depth, width, rows, m_tile_bound;
@@ -137,8 +144,9 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   constexpr bool kGated = MODE == kInterleavedGated;
   constexpr int kOutBN = kGated ? BN / 2 : BN;  // output columns of the tile
   static_assert(WM * WN == 4 && BM % (32 * WM) == 0 && BN % (32 * WN) == 0 && BM % 32 == 0, "tile shape");
-  constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4;
-  constexpr bool kPow2 = FORMAT == DEW_MOE_W_MXFP4;
+  constexpr bool kSplit = FORMAT == kFormatMxSplit;
+  constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4 || kSplit;
+  constexpr bool kPow2 = FORMAT == DEW_MOE_W_MXFP4 || kSplit;
   constexpr int kMatrices = PAIRED ? 2 : 1;
   constexpr int kAtomK = kFp4 ? 64 : 32;       // depth an atom covers
   constexpr int kAtoms = BK / kAtomK;          // 16-byte loads a lane makes per 32-column tile per step
@@ -241,6 +249,18 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     const int source = p.gather ? p.gather[sorted] : sorted;
     a_src[i] = p.x + static_cast<size_t>(source) * p.depth + chunk * 8;
   }
+  // Split activations: the lane's row of each row tile carries one e8m0 scale; the hi term multiplies under it
+  // (byte 0) and the lo term under 2^-4 of it (byte 1).
+  int a_scale_word[TI];
+#pragma unroll
+  for (int i = 0; i < TI; ++i) {
+    a_scale_word[i] = 0;
+    if constexpr (kSplit) {
+      const int sorted = row0 + min(wm0 + 32 * i + lane % 32, valid_rows - 1);
+      const int byte = p.a_scale[p.gather ? p.gather[sorted] : sorted];
+      a_scale_word[i] = byte | ((byte - 4) << 8);
+    }
+  }
   auto load_a = [&](u32x4_t* stage, int step, auto begin, auto end) __attribute__((always_inline)) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass, which only needs the kernel's stub, does not know the builtin
 #pragma unroll
@@ -296,7 +316,22 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
 
   // ---- fragments: slice kk of a step is 16 depths; a lane's are the 8 its weight bytes cover ----
   bf16x8_t a_frag[2][TI], b_frag[2][kTiles];
+  i32x8_t a_term[2][kSplit ? TI : 1];  // split activations: [0] the hi term of a step, [1] its lo term
   float fp4_scale[kTiles];
+  // a term of a 32-depth block is 32 bytes: the lane's block lane / 32 of the step holds hi in its chunks 0-1, lo in 2-3
+  auto fetch_term = [&](const u32x4_t* stage, auto term) __attribute__((always_inline)) {
+    if constexpr (kSplit) {
+#pragma unroll
+      for (int i = 0; i < TI; ++i) {
+        const int row = wm0 + 32 * i + lane % 32;
+        const u32x4_t first = stage[swizzled(row, 4 * (lane / 32) + 2 * term.value)];
+        const u32x4_t second = stage[swizzled(row, 4 * (lane / 32) + 2 * term.value + 1)];
+        a_term[term.value][i] = i32x8_t{static_cast<int>(first[0]), static_cast<int>(first[1]), static_cast<int>(first[2]),
+                                        static_cast<int>(first[3]), static_cast<int>(second[0]), static_cast<int>(second[1]),
+                                        static_cast<int>(second[2]), static_cast<int>(second[3])};
+      }
+    }
+  };
   auto fetch = [&](const u32x4_t* stage, auto kk, auto into) __attribute__((always_inline)) {
     const int chunk = kFp4 ? 4 * (lane / 32) + kk.value : 4 * (kk.value / 2) + 2 * (lane / 32) + kk.value % 2;
 #pragma unroll
@@ -339,6 +374,25 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
 #pragma unroll
         for (int j = 0; j < TJ; ++j)
           acc[m][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_frag[from.value][i], b_frag[from.value][m * TJ + j], acc[m][i][j], 0, 0, 0);
+  };
+
+  // Split activations: one scaled instruction multiplies 64 depths of one term by the stored FP4 codes under
+  // both operands' power-of-two scales; the block scale byte is the e4m3 of a normal power of two, 2^(field - 7).
+  auto multiply_term = [&](auto set, auto term) __attribute__((always_inline)) {
+    if constexpr (kSplit) {
+#pragma unroll
+      for (int m = 0; m < kMatrices; ++m)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+          const u32x4_t& raw = b_regs[set.value][m * TJ + j][0];
+          const i32x8_t codes = {static_cast<int>(raw[0]), static_cast<int>(raw[1]), static_cast<int>(raw[2]), static_cast<int>(raw[3]), 0, 0, 0, 0};
+          const int b_scale = static_cast<int>(((s_regs[set.value][m * TJ + j] >> 3) & 15u) + 120u);
+#pragma unroll
+          for (int i = 0; i < TI; ++i)
+            acc[m][i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_term[term.value][i], codes, acc[m][i][j], 0, 4, term.value,
+                                                                        a_scale_word[i], 0, b_scale);
+        }
+    }
   };
 
   // ---- pipeline. At the top of step s: LDS stage s % 3 holds the A rows of step s and the loads of step s + 1
@@ -387,6 +441,36 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     u32x4_t* next = lds + next_index * kStageChunks;
     u32x4_t* fill = lds + fill_index * kStageChunks;
     const int ahead_a = min(step + 2, steps - 1), ahead_b = min(step + kSets - 1, steps - 1);
+    if constexpr (kSplit) {
+      // two phases a step: the hi term multiplies while the lo term is read, then the barrier, then the lo term
+      // multiplies while the next step's hi term is read; each phase issues half of the step's global loads
+      constexpr std::integral_constant<int, kRowLoads / 2> ah{};
+      constexpr std::integral_constant<int, kTiles / 2> bh{};
+      constexpr int kSplitMfmas = kMatrices * TI * TJ;
+      constexpr int kSplitLoads = kRowLoads / 2 + (kTiles / 2) * kLoadsPerTile;
+      static_assert(kRowLoads % 2 == 0 && kTiles % 2 == 0, "two even halves of loads");
+      // younger than the last A load of the step before: only this phase's loads are sure to be
+      constexpr int kSplitWait = (kSplitLoads & 0xF) | (7 << 4) | (0 << 8) | ((kSplitLoads >> 4) << 14);
+      fetch_term(current, c1);
+      multiply_term(set, c0);
+      load_a(fill, ahead_a, c0, ah);
+      load_b(filling, ahead_b, c0, bh);
+      schedule_phase<0, kSplitMfmas, 2 * TI, 0, 2 * kTiles + 2 * kSplitLoads, kSplitLoads>();
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_waitcnt(last_steps.value ? kWaitAll : kSplitWait);
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+      fetch_term(next, c0);
+      multiply_term(set, c1);
+      load_a(fill, ahead_a, ah, a4);
+      load_b(filling, ahead_b, bh, b4);
+      schedule_phase<0, kSplitMfmas, 2 * TI, 0, 2 * kTiles + 2 * kSplitLoads, kSplitLoads>();
+      __builtin_amdgcn_sched_barrier(0);
+      stage_index = next_index;
+      return;
+    }
     fetch(current, c1, c1);
     dequantize(set, c1, c1, step);
     multiply(c0);
@@ -436,8 +520,12 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   __builtin_amdgcn_s_waitcnt(kWaitAll);
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
-  fetch(lds, c0, c0);
-  dequantize(c0, c0, c0, 0);
+  if constexpr (kSplit) {
+    fetch_term(lds, c0);
+  } else {
+    fetch(lds, c0, c0);
+    dequantize(c0, c0, c0, 0);
+  }
   int step = 0;
   for (; step + kSets <= steps; step += kSets) {
     iterate(c0, step, std::false_type{});
@@ -460,8 +548,9 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   // kernel's time). Tiles of 256 columns are staged in two passes of BM / 2 rows.
   float factor0 = 1.0f, factor1 = 1.0f;
   if (kFp4) {  // the 2^8 the decode owes times the expert's tensor scale (src/dew/nn/kernels/gemm.py:660-662)
-    factor0 = 256.0f * p.w0.tensor_scale[expert];
-    if (PAIRED) factor1 = 256.0f * p.w1.tensor_scale[expert];
+    // (the scaled instruction applies the block scales themselves, not their 2^-8)
+    factor0 = (kSplit ? 1.0f : 256.0f) * p.w0.tensor_scale[expert];
+    if (PAIRED) factor1 = (kSplit ? 1.0f : 256.0f) * p.w1.tensor_scale[expert];
   }
   constexpr int kPasses = (BN == 256 && TI > 1) ? 2 : 1;
   constexpr int kPassTiles = TI / kPasses, kPassRows = BM / kPasses;
@@ -646,6 +735,56 @@ extern "C" int dew_moe_grouped_gemm(const void* x, const int32_t* gather, const 
                                     const dew_moe_bank* w, const int32_t* scatter, void* out, int32_t rows,
                                     void* stream) {
   return dew_moe_grouped_gemm_bias(x, gather, offsets, w, nullptr, scatter, out, rows, stream);
+}
+
+extern "C" int dew_moe_grouped_gemm_split(const void* x_split, const uint8_t* x_scale, const int32_t* gather, const int32_t* offsets,
+                                          const dew_moe_bank* w, const float* bias, const int32_t* scatter, void* out,
+                                          int32_t rows, void* stream) {
+  using namespace dew;
+  const char* who = "dew_moe_grouped_gemm_split";
+  if (int rc = check_bank(who, w, "weight")) return rc;
+  DEW_REQUIRE(w->format == DEW_MOE_W_MXFP4 && w->width % 256 == 0,
+              "%s: split activations multiply an MXFP4 bank (power-of-two block scales) whose width is whole 256s; this one is "
+              "format %d, width %d", who, w->format, w->width);
+  DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
+  if (rows == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(x_scale, "%s: the rows' scales must not be null", who);
+  GemmParams p{};
+  if (int rc = fill_single(who, p, x_split, gather, offsets, w, bias, scatter, out, rows)) return rc;
+  p.a_scale = x_scale;
+  return launch_tile<kFormatMxSplit, kPlain, 256, 256, 1, 4>(who, p, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int dew_moe_gateup_swiglu_split(const void* x_split, const uint8_t* x_scale, const int32_t* gather,
+                                           const int32_t* offsets, const dew_moe_bank* gate, const dew_moe_bank* up, void* hidden,
+                                           int32_t rows, void* stream) {
+  using namespace dew;
+  const char* who = "dew_moe_gateup_swiglu_split";
+  if (int rc = check_bank(who, gate, "gate")) return rc;
+  if (int rc = check_bank(who, up, "up")) return rc;
+  DEW_REQUIRE(gate->format == DEW_MOE_W_MXFP4 && up->format == DEW_MOE_W_MXFP4,
+              "%s: split activations multiply MXFP4 banks (power-of-two block scales); these are formats %d and %d", who,
+              gate->format, up->format);
+  DEW_REQUIRE(gate->experts == up->experts && gate->depth == up->depth && gate->width == up->width,
+              "%s: gate [%d, %d, %d] and up [%d, %d, %d] differ", who, gate->experts, gate->depth, gate->width, up->experts,
+              up->depth, up->width);
+  DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
+  if (rows == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(x_split && x_scale && offsets && hidden, "%s: x_split, x_scale, offsets and hidden must not be null", who);
+  DEW_REQUIRE(aligned16(x_split) && aligned16(hidden), "%s: x_split and hidden must be 16-byte aligned", who);
+  GemmParams p{};
+  p.x = static_cast<const bf16_t*>(x_split);
+  p.a_scale = x_scale;
+  p.gather = gather;
+  p.offsets = offsets;
+  p.w0 = BankView{static_cast<const uint8_t*>(gate->codes), gate->scales, gate->tensor_scale};
+  p.w1 = BankView{static_cast<const uint8_t*>(up->codes), up->scales, up->tensor_scale};
+  p.out = static_cast<bf16_t*>(hidden);
+  p.experts = gate->experts;
+  p.depth = gate->depth;
+  p.width = gate->width;
+  p.rows = rows;
+  return launch_tile<kFormatMxSplit, kSwigluOfTwo, 256, 128, 1, 4>(who, p, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int dew_moe_gateup_interleaved(const void* x, const int32_t* gather, const int32_t* offsets,

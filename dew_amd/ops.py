@@ -265,6 +265,55 @@ def combine(slots: torch.Tensor, weights: torch.Tensor, addend: torch.Tensor | N
     return out
 
 
+def split_rows(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """bf16 rows `[rows, depth]` as two e4m3 terms per element: (`split` uint8 `[rows, depth * 2]`, each 64 depths as
+    four 32-byte pieces in the scaled matrix instruction's operand order; `scale` uint8 `[rows]`, e8m0) with
+    `x = 2^(scale - 127) * (hi + lo / 16)`."""
+    _device(x, "x", torch.bfloat16)
+    rows, depth = x.shape
+    split = torch.empty((rows, depth * 2), dtype=torch.uint8, device=x.device)
+    scale = torch.empty((rows,), dtype=torch.uint8, device=x.device)
+    _lib.check(_lib.library().dew_moe_split_rows(_ptr(x), _ptr(split), _ptr(scale), rows, depth, _stream()), "dew_moe_split_rows")
+    return split, scale
+
+
+def prefers_split(bank: PreparedBank, rows: int) -> bool:
+    """Whether a product of `rows` rows through `bank` is better run on split rows (`split_rows` then the `_split`
+    launches): an MXFP4 bank of whole 256-column strips whose groups average the 256-row tiles' fill."""
+    experts, _, width = bank.shape
+    return bank.descriptor.format == _lib.W_MXFP4 and width % 256 == 0 and rows // experts >= 768
+
+
+def grouped_gemm_split(split: torch.Tensor, scale: torch.Tensor, bank: PreparedBank, offsets: torch.Tensor, *,
+                       gather: torch.Tensor | None = None, scatter: torch.Tensor | None = None, rows: int | None = None,
+                       bias: torch.Tensor | None = None) -> torch.Tensor:
+    """`grouped_gemm` on rows already split into two e4m3 terms (`split_rows`), for an MXFP4 bank."""
+    experts, depth, width = bank.shape
+    if split.dtype != torch.uint8 or split.shape[-1] != 2 * depth or scale.dtype != torch.uint8 or scale.numel() != split.shape[0]:
+        raise KernelError(f"split rows are uint8 [rows, {2 * depth}] with one uint8 scale a row")
+    rows = (gather.numel() if gather is not None else split.shape[0]) if rows is None else rows
+    bias = _expert_bias(bias, experts, width)
+    out = torch.empty((rows, width), dtype=torch.bfloat16, device=split.device)
+    _lib.check(_lib.library().dew_moe_grouped_gemm_split(_ptr(split), _ptr(scale), _ptr(gather), _ptr(offsets), bank.descriptor,
+                                                         _ptr(bias), _ptr(scatter), _ptr(out), rows, _stream()),
+               "dew_moe_grouped_gemm_split")
+    return out
+
+
+def gateup_swiglu_split(split: torch.Tensor, scale: torch.Tensor, gate: PreparedBank, up: PreparedBank, offsets: torch.Tensor, *,
+                        gather: torch.Tensor | None = None, rows: int | None = None) -> torch.Tensor:
+    """`gateup_swiglu` on rows already split into two e4m3 terms (`split_rows`), for MXFP4 banks."""
+    experts, depth, width = gate.shape
+    if split.dtype != torch.uint8 or split.shape[-1] != 2 * depth or scale.dtype != torch.uint8 or scale.numel() != split.shape[0]:
+        raise KernelError(f"split rows are uint8 [rows, {2 * depth}] with one uint8 scale a row")
+    rows = (gather.numel() if gather is not None else split.shape[0]) if rows is None else rows
+    hidden = torch.empty((rows, width), dtype=torch.bfloat16, device=split.device)
+    _lib.check(_lib.library().dew_moe_gateup_swiglu_split(_ptr(split), _ptr(scale), _ptr(gather), _ptr(offsets), gate.descriptor,
+                                                          up.descriptor, _ptr(hidden), rows, _stream()),
+               "dew_moe_gateup_swiglu_split")
+    return hidden
+
+
 # ---- measurement aids ---------------------------------------------------------------------------------
 
 

@@ -125,6 +125,27 @@ int dew_moe_gateup_interleaved(const void* x, const int32_t* gather, const int32
                                const dew_moe_bank* gate_up /* prepared, [E,K,2F] */, const float* bias /* nullable [E,2F] */,
                                float limit, void* hidden /* bf16 [rows,F] */, int32_t rows, void* stream);
 
+/* Activation rows as two FP8 (e4m3) terms for the scaled matrix instructions (no counterpart in the reference:
+ * its products take bf16 operands, src/dew/nn/moe.py:675-677, and this keeps their values): x = s (hi + lo / 16)
+ * with s = 2^(scale[row] - 127) one power of two per row, exact for every element within 2^-11 of its row's
+ * largest magnitude and to 2^-21 of that magnitude otherwise. split[row] holds each 64 depths as four 32-byte
+ * pieces in the scaled instruction's operand order (hi then lo of depths 0-15 and 32-47, hi then lo of depths
+ * 16-31 and 48-63): depth * 2 bytes a row, like the bf16 source.                                            */
+int dew_moe_split_rows(const void* x /* bf16 [rows, depth] */, void* split /* [rows, depth * 2] bytes */,
+                       uint8_t* scale /* [rows] e8m0 */, int32_t rows, int32_t depth, void* stream);
+
+/* The grouped products on rows split by dew_moe_split_rows, for MXFP4 banks (every block scale a power of two,
+ * DEW_MOE_W_MXFP4 after dew_moe_prepare_bank) whose width is whole 256s: v_mfma_scale_f32_32x32x64_f8f6f4 multiplies
+ * each e4m3 term by the FP4 codes as stored, under both operands' power-of-two scales, so no weight is dequantized
+ * and every product is the exact bf16 x weight product of dew_moe_grouped_gemm_bias / dew_moe_gateup_swiglu; only
+ * the order of the fp32 sums differs. 256-row tiles: meant for groups of several hundred rows.            */
+int dew_moe_grouped_gemm_split(const void* x_split, const uint8_t* x_scale, const int32_t* gather,
+                               const int32_t* offsets, const dew_moe_bank* w, const float* bias,
+                               const int32_t* scatter, void* out, int32_t rows, void* stream);
+int dew_moe_gateup_swiglu_split(const void* x_split, const uint8_t* x_scale, const int32_t* gather,
+                                const int32_t* offsets, const dew_moe_bank* gate, const dew_moe_bank* up,
+                                void* hidden, int32_t rows, void* stream);
+
 /* gate and up in one launch with the SwiGLU epilogue: hidden[i] = swiglu(x[gather[i]] @ Wg[e], .. @ Wu[e])
  * with the reference's rounding sequence (src/dew/nn/activations.py:267-278): both products rounded to
  * bf16, a = bf16(g * logistic(g)), hidden = bf16(a * u).                                                */

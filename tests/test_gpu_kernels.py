@@ -283,3 +283,54 @@ def test_depths_that_leave_steps_after_the_unrolled_loop(ops, quant, depth, labe
     got_gate = bf16_np(got_gate)
     assert np.abs(got_gate - want_gate).max() <= 2 ** -8 * np.abs(want_gate).max() + 1e-6
     assert (got_gate == want_gate).mean() > 0.97
+
+
+def test_split_rows_is_exact_within_eleven_binades_of_the_row_maximum(ops):
+    rng = np.random.default_rng(17)
+    rows, depth = 64, 512
+    x = rng.standard_normal((rows, depth)).astype(np.float32)
+    x[8:16] *= 10.0 ** rng.uniform(-4, 4, size=(8, depth)).astype(np.float32)     # twenty-six binades in a row
+    x[16] = 0.0
+    x[17, 5] = 3.0e4                                                                # one outlier over a row of ~1
+    x[18] *= 1e-30
+    xb = torch.from_numpy(x).to(torch.bfloat16)
+    split, scale = ops.split_rows(xb.cuda())
+    # each 64 depths: [group][term][half][16] with depth = 32 half + 16 group + j
+    split, scale = split.cpu().numpy().reshape(rows, depth // 64, 2, 2, 2, 16), scale.cpu().numpy()
+    table = oracle._e4m3_table()
+    s = np.ldexp(np.float64(1), scale.astype(np.int64) - 127)[:, None]
+    terms = table[split].astype(np.float64)                                        # [rows, 64s, group, term, half, 16]
+    values = terms[:, :, :, 0] + terms[:, :, :, 1] / 16                            # [rows, 64s, group, half, 16]
+    rebuilt = values.transpose(0, 1, 3, 2, 4).reshape(rows, depth) * s             # depth order: half, group, j
+    want = xb.float().numpy().astype(np.float64)
+    largest = np.abs(want).max(axis=1, keepdims=True)
+    near = np.abs(want) >= largest * 2.0 ** -11
+    assert np.array_equal(rebuilt[near], want[near])
+    assert (np.abs(rebuilt - want) <= largest * 2.0 ** -21).all()
+    assert np.all((largest[:, 0] == 0) | ((largest[:, 0] / s[:, 0] >= 128) & (largest[:, 0] / s[:, 0] < 256)))
+
+
+@pytest.mark.parametrize("depth", [256, 768, 1280])
+def test_split_activations_give_the_bf16_products_on_mxfp4_banks(ops, depth):
+    """Two e4m3 terms times the stored FP4 codes under power-of-two scales are the exact bf16 x weight products:
+    the scaled-instruction kernels agree with the bf16 kernels up to the order of the fp32 sums."""
+    sizes = [700, 0, 290, 5]
+    gate, x, offsets = grouped_case("mxfp4", len(sizes), depth, 256, sizes, seed=depth + 1)
+    up, _, _ = grouped_case("mxfp4", len(sizes), depth, 256, sizes, seed=depth + 2)
+    gate_values, gate_factor = dequantized(gate)
+    up_values, up_factor = dequantized(up)
+    rng = np.random.default_rng(depth)
+    gather = rng.integers(0, x.shape[0], size=x.shape[0]).astype(np.int32)
+    scatter = rng.permutation(x.shape[0]).astype(np.int32)
+    rows = bf16_np(x)[gather]
+    want_gate = oracle.grouped_matmul(rows, gate_values, sizes, factor=gate_factor)
+    want = oracle.swiglu(want_gate, oracle.grouped_matmul(rows, up_values, sizes, factor=up_factor))
+    xd, od, gd, sd = x.cuda(), torch.from_numpy(offsets).cuda(), torch.from_numpy(gather).cuda(), torch.from_numpy(scatter).cuda()
+    pg, pu = ops.prepare(gate.to("cuda")), ops.prepare(up.to("cuda"))
+    split, scale = ops.split_rows(xd)
+    got_gate = bf16_np(ops.grouped_gemm_split(split, scale, pg, od, gather=gd, scatter=sd))[scatter]
+    plain_gate = bf16_np(ops.grouped_gemm(xd, pg, od, gather=gd))
+    assert np.abs(got_gate - want_gate).max() <= 2 ** -8 * np.abs(want_gate).max()
+    assert (got_gate == want_gate).mean() > 0.97 and (got_gate == plain_gate).mean() > 0.97
+    fused = bf16_np(ops.gateup_swiglu_split(split, scale, pg, pu, od, gather=gd))
+    assert np.abs(fused - want).max() <= 2 ** -6 * np.abs(want).max() and (fused == want).mean() > 0.9
