@@ -552,13 +552,13 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     factor0 = (kSplit ? 1.0f : 256.0f) * p.w0.tensor_scale[expert];
     if (PAIRED) factor1 = (kSplit ? 1.0f : 256.0f) * p.w1.tensor_scale[expert];
   }
-  constexpr int kPasses = (BN == 256 && TI > 1) ? 2 : 1;
-  constexpr int kPassTiles = TI / kPasses, kPassRows = BM / kPasses;
+  constexpr int kPasses = (BN == 256 && BM > 32) ? 2 : 1;
+  constexpr int kPassTiles = BM / 32 / kPasses, kPassRows = BM / kPasses;  // row tiles of the block a pass stages
   constexpr int kRowDwords = kOutBN / 2 + 4;  // a staged row: the tile's output columns in bf16 and 16 bytes of padding
   constexpr int kRowChunks = kOutBN / 8;      // 16-byte pieces of an output row
   constexpr int kStoreIters = kPassRows * kRowChunks / kThreads;
   static_assert(kPassRows * kRowChunks % kThreads == 0, "whole store rounds");
-  static_assert(TI % kPasses == 0 && kPassRows * kRowDwords * 4 <= shared_bytes<BM, BN, MODE>(), "staged tile fits the LDS");
+  static_assert((BM / 32) % kPasses == 0 && kPassRows * kRowDwords * 4 <= shared_bytes<BM, BN, MODE>(), "staged tile fits the LDS");
   uint32_t* staged = reinterpret_cast<uint32_t*>(lds);
   const bool odd_lane = lane & 1;
   const int out_width = kGated ? p.width / 2 : p.width, out_n0 = kGated ? n0 / 2 : n0;
@@ -579,8 +579,10 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
       out_rows[it] = p.scatter ? p.scatter[sorted] : sorted;
     }
 #pragma unroll
-    for (int ii = 0; ii < kPassTiles; ++ii) {
-      const int i = pass * kPassTiles + ii;
+    for (int i = 0; i < TI; ++i) {
+      const int block_tile = wm0 / 32 + i;  // this wavefront's row tile i among the block's
+      if (block_tile / kPassTiles != pass) continue;
+      const int ii = block_tile % kPassTiles;
 #pragma unroll
       for (int q = 0; q < 16; q += 2) {
         const int row = 32 * ii + 8 * (q / 4) + 4 * (lane / 32) + q % 4 + (odd_lane ? 1 : 0);  // within the pass
@@ -752,7 +754,7 @@ extern "C" int dew_moe_grouped_gemm_split(const void* x_split, const uint8_t* x_
   GemmParams p{};
   if (int rc = fill_single(who, p, x_split, gather, offsets, w, bias, scatter, out, rows)) return rc;
   p.a_scale = x_scale;
-  return launch_tile<kFormatMxSplit, kPlain, 256, 256, 1, 4>(who, p, static_cast<hipStream_t>(stream));
+  return launch_tile<kFormatMxSplit, kPlain, 256, 256, 2, 2>(who, p, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int dew_moe_gateup_swiglu_split(const void* x_split, const uint8_t* x_scale, const int32_t* gather,
@@ -784,7 +786,7 @@ extern "C" int dew_moe_gateup_swiglu_split(const void* x_split, const uint8_t* x
   p.depth = gate->depth;
   p.width = gate->width;
   p.rows = rows;
-  return launch_tile<kFormatMxSplit, kSwigluOfTwo, 256, 128, 1, 4>(who, p, static_cast<hipStream_t>(stream));
+  return launch_tile<kFormatMxSplit, kSwigluOfTwo, 256, 128, 2, 2>(who, p, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int dew_moe_gateup_interleaved(const void* x, const int32_t* gather, const int32_t* offsets,

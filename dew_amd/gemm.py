@@ -105,7 +105,7 @@ names are refused as unlowerable."""
 SPLIT_ROWS = False
 """Whether large-group products on MXFP4 banks run on rows split into two e4m3 terms and the scaled matrix
 instruction (`ops.split_rows`, `ops.*_split`). The products are the same exact ones; measured on C2 the gate/up
-launch is 2.7 % faster and the whole step 4 % slower (the split of the hidden rows is a pass of its own), so the
+launch is 5 % faster and the whole step no faster (the split of the hidden rows is a pass of its own), so the
 bf16 instructions stay the default."""
 
 
