@@ -224,8 +224,8 @@ extern "C" int dew_moe_route(const float* logits, const float* bias, int32_t tok
                              int32_t expert_groups, int32_t groups_per_token, float* weights,
                              int32_t* indices, void* stream) {
   using namespace dew;
-  DEW_REQUIRE(logits && weights && indices, "dew_moe_route: logits, weights and indices must not be null");
   DEW_REQUIRE(tokens >= 0 && experts >= 1, "dew_moe_route: tokens %d experts %d", tokens, experts);
+  DEW_REQUIRE(tokens == 0 || (logits && weights && indices), "dew_moe_route: logits, weights and indices must not be null");
   DEW_REQUIRE(experts <= kWave * kMaxPerLane, "dew_moe_route: at most %d experts, got %d", kWave * kMaxPerLane,
               experts);
   DEW_REQUIRE(top_k >= 1 && top_k <= experts && top_k <= kWave, "dew_moe_route: top_k %d of %d experts (at most %d)",

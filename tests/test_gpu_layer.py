@@ -136,3 +136,43 @@ def test_a_named_kernel_that_cannot_run_is_refused_by_name():
         layer.apply(variables, x, logits=logits)
     with pytest.raises(selection.KernelRefused, match="bf16"), selection.chosen(grouped_matmul="hip"):
         layer.apply(variables, x.float(), logits=logits)
+
+
+def test_no_tokens_give_no_rows_and_no_launch_fails():
+    """An empty batch goes through every entry point and the whole layer and comes back empty."""
+    from dew_amd import ops
+
+    case = CASES["c3-one-token"]
+    data = inputs(case, seed=2)
+    layer, variables = layer_and_variables(case, data)
+    x = data["x"][:0].cuda()
+    logits = data["logits"][:0].cuda()
+    weights, indices = ops.route(logits, case.top_k, **case.router)
+    assert weights.shape == (0, case.top_k) and indices.shape == (0, case.top_k)
+    plan = ops.sort_by_expert(indices, case.experts)
+    assert plan.sizes.tolist() == [0] * case.experts and plan.offsets.tolist() == [0] * (case.experts + 1)
+    assert plan.order.numel() == 0 and plan.rows.numel() == 0
+    out = layer.apply(variables, x, logits=logits)
+    assert out.shape == (0, case.d_model) and out.dtype == torch.bfloat16
+
+
+def test_more_experts_than_one_scan_round_and_every_expert_chosen():
+    """512 experts (the tile search scans them 256 at a time) of which most are idle, and a router whose top-k is
+    all of its experts."""
+    from dew_amd import ops
+
+    rng = np.random.default_rng(8)
+    experts, depth, width = 512, 256, 128
+    sizes = np.zeros(experts, np.int64)
+    sizes[[3, 255, 256, 300, 511]] = [40, 1, 130, 7, 64]
+    from test_gpu_kernels import grouped_case, bf16_np
+    bank, x, offsets = grouped_case("fp8_block", experts, depth, width, sizes.tolist(), seed=4)
+    values, factor = dequantized(bank)
+    want = oracle.grouped_matmul(bf16_np(x), values, sizes.tolist(), factor=factor)
+    got = bf16_np(ops.grouped_gemm(x.cuda(), ops.prepare(bank.to("cuda")), torch.from_numpy(offsets).cuda()))
+    assert np.abs(got - want).max() <= 2 ** -8 * np.abs(want).max() and (got == want).mean() > 0.97
+    logits = torch.from_numpy(rng.standard_normal((33, 8)).astype(np.float32))
+    weights, indices = ops.route(logits.cuda(), 8, score_function="softmax", normalize_weights=True)
+    want_weights, want_indices = oracle.route(logits.numpy(), 8, score_function="softmax", normalize_weights=True)
+    assert np.array_equal(indices.cpu().numpy(), want_indices) and np.array_equal(weights.cpu().numpy(), want_weights)
+    assert np.array_equal(np.sort(indices.cpu().numpy(), -1), np.tile(np.arange(8), (33, 1)))
