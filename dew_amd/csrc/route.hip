@@ -55,17 +55,21 @@ __device__ __forceinline__ bool better(float v, int i, const Best& than) {
   return v > than.value || (v == than.value && i < than.index);
 }
 
+// The wavefront's best (value, index): the largest value by a butterfly of maxima, then the lowest index among the
+// lanes that hold it. Almost always one lane does, found by a ballot and read with one cross-lane move; ties walk
+// the ballot's set bits. Half the cross-lane traffic of reducing value and index together.
 __device__ __forceinline__ Best wave_best(Best b) {
-#pragma unroll
-  for (int offset = 32; offset >= 1; offset >>= 1) {
-    const float v = __shfl_xor(b.value, offset, kWave);
-    const int i = __shfl_xor(b.index, offset, kWave);
-    if (better(v, i, b)) {
-      b.value = v;
-      b.index = i;
-    }
+  const float top = wave_max(b.value);
+  unsigned long long holders = __ballot(b.value == top);
+  Best best;
+  best.value = top;
+  best.index = 0x7fffffff;
+  while (holders != 0ull) {
+    const int lane = __builtin_ctzll(holders);
+    best.index = min(best.index, __builtin_amdgcn_readlane(b.index, lane));
+    holders &= holders - 1ull;
   }
-  return b;
+  return best;
 }
 
 struct RouteParams {
