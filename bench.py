@@ -260,13 +260,13 @@ def main():
             graph.replay()
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - began
-        # the dominant kernel's duration, by HIP events around eager launches of it on the same inputs
+        # The dominant kernel's duration: HIP events around its launch inside eager steps on the same inputs. A
+        # millisecond of queued work ahead of each step lets the host run ahead, so the step's launches follow each
+        # other on the device as they do in the graph and the events bracket the kernel, not the host's launch path.
+        operands = torch.randn(16384, device=device).to(torch.bfloat16)
         for _ in range(args.steps):
-            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            start.record()
-            ops.gateup_swiglu(data["x"], stepper.gate, stepper.up, plan.offsets, gather=plan.rows)
-            stop.record()
-            stepper.events.append((start, stop))
+            ops.probe_mfma(operands, 1200)
+            stepper(timed=True)
         torch.cuda.synchronize()
     else:
         began = time.perf_counter()
