@@ -2,12 +2,17 @@
 // weights dequantized to bf16 in registers (exactly the values the reference's load produces), fp32
 // accumulation in v_mfma_f32_32x32x16_bf16, one rounding to bf16.
 //
-//   out[scatter[i], :] = bf16( sum_k x[gather[i], k] * W[e(i)][k, :] )       (expert_projection)
-//   hidden[i, :] = swiglu(x[gather[i]] @ Wg[e], x[gather[i]] @ Wu[e])        (paired gate/up + epilogue)
+//   out[scatter[i], :] = bf16( sum_k x[gather[i], k] * W[e(i)][k, :] + bias[e(i)] )   (expert_projection)
+//   hidden[i, :] = swiglu(x[gather[i]] @ Wg[e], x[gather[i]] @ Wu[e])                 (paired gate/up + epilogue)
+//   hidden[i, :] = gated pairs of one interleaved bank's columns                       (GPT-OSS's gate_up)
 //
-// Work decomposition: a 256-thread block (4 wavefronts, 2 x 2) owns a BM-row x BN-column tile of one expert's
-// group (two such tiles, gate and up, when paired) and walks the depth in 64-deep steps. Tiles are enumerated
-// on the device from `offsets` (no host read of the routing); experts with no rows own no tiles.
+// Work decomposition: a 256-thread block (4 wavefronts side by side along the columns) owns a BM-row x BN-column
+// tile of one expert's group (two such tiles, gate and up, when paired) and walks the depth in 64-deep steps.
+// Tiles are enumerated on the device from `offsets` (no host read of the routing); experts with no rows own no
+// tiles. The finished tile is staged in the LDS and leaves as whole rows.
+//
+// For MXFP4 banks there is a second operand path (kFormatMxSplit): activation rows split beforehand into two e4m3
+// terms and multiplied by the stored FP4 codes with v_mfma_scale_f32_32x32x64_f8f6f4, nothing dequantized.
 //
 // Operand paths, shaped by what the LDS of this chip costs (measured: ds_read_b128 ~230 B/clk a CU,
 // ds_write_b128 ~70 B/clk):
