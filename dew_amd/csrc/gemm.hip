@@ -669,24 +669,43 @@ static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
 // Tile choice from what the host knows (rows and experts; the routing itself stays on the device): 256-row
 // tiles when the average group fills them, 128-row tiles otherwise, and for decode-sized groups a 32-row tile
 // whose four wavefronts split the columns, so that thousands of wavefronts stream the weights at once.
+// Rows of the block tile, from what the host knows (rows and experts; the routing itself stays on the device).
+// Two rules, both measured over group sizes of 8 .. 1024 rows on four model shapes. Fill: the tile about as tall as
+// the average group (a 128-row tile over 32-row groups multiplies three empty rows for each real one, and takes 1.3
+// to 2 times as long as 32-row tiles). Occupancy: a launch of fewer tiles than CUs halves its tile until there are
+// enough (8 experts x 512 rows x 512 columns: 144 tiles of 128 rows take 16.5 us, 272 tiles of 64 rows 11.7 us).
+// 256-row tiles, which fill every accumulator register, are kept to FP4 banks whose groups fill them.
+static int forced_tile_rows = 0;  // dew_moe_tile_rows: 0 leaves the choice to the rules below
+
+static int tile_rows(const GemmParams& p, bool fp4) {
+  if (forced_tile_rows != 0) return forced_tile_rows;
+  const int average = p.rows / p.experts;
+  if (fp4 && average >= 768 && p.width % 256 == 0) return 256;
+  int rows = average <= 36 ? 32 : average <= 72 ? 64 : 128;
+  const long long strips = p.width / 128;
+  while (rows > 32 && (p.rows / rows + p.experts / 2) * strips < 256) rows /= 2;
+  return rows;
+}
+
 template <int FORMAT, int MODE>
 static int launch_format(const char* who, const GemmParams& p, hipStream_t stream) {
-  constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4;  // the 256-row tiles are kept to the FP4 banks
-  const int average = p.rows / p.experts;
-  if (average < 24) {
-    // one bank: 256 columns a block where that still leaves every CU several blocks, so that a launch is one round
-    if (MODE != kSwigluOfTwo && p.width % 256 == 0 && static_cast<long long>(p.experts) * (p.width / 256) >= 768)
-      return launch_tile<FORMAT, MODE, 32, 256, 1, 4>(who, p, stream);
-    return launch_tile<FORMAT, MODE, 32, 128, 1, 4>(who, p, stream);
-  }
-  if constexpr (MODE == kSwigluOfTwo) {
-    if (kFp4 && average >= 768 && p.width % 256 == 0) return launch_tile<FORMAT, MODE, 256, 128, 1, 4>(who, p, stream);
-    return launch_tile<FORMAT, MODE, 128, 128, 1, 4>(who, p, stream);
-  } else {
-    if (kFp4 && average >= 768 && p.width % 256 == 0) return launch_tile<FORMAT, MODE, 256, 256, 1, 4>(who, p, stream);
-    if (p.width % 256 == 0 && static_cast<long long>(p.rows / 128 + 1) * (p.width / 256) >= 512)
-      return launch_tile<FORMAT, MODE, 128, 256, 1, 4>(who, p, stream);  // enough tiles to fill the chip twice over
-    return launch_tile<FORMAT, MODE, 128, 128, 1, 4>(who, p, stream);
+  constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4;
+  constexpr bool kPaired = MODE == kSwigluOfTwo;
+  switch (tile_rows(p, kFp4)) {
+    case 32:
+      // one bank: 256 columns a block where that still leaves every CU several blocks, so that a launch is one round
+      if (!kPaired && p.width % 256 == 0 && static_cast<long long>(p.experts) * (p.width / 256) >= 768)
+        return launch_tile<FORMAT, MODE, 32, 256, 1, 4>(who, p, stream);
+      return launch_tile<FORMAT, MODE, 32, 128, 1, 4>(who, p, stream);
+    case 64:
+      return launch_tile<FORMAT, MODE, 64, 128, 1, 4>(who, p, stream);
+    case 256:
+      if (kPaired || p.width % 256 == 0) return launch_tile<FORMAT, MODE, 256, kPaired ? 128 : 256, 1, 4>(who, p, stream);
+      [[fallthrough]];  // one bank whose width is not whole 256s: the 128-row tile
+    default:
+      if (!kPaired && p.width % 256 == 0 && static_cast<long long>(p.rows / 128 + 1) * (p.width / 256) >= 512)
+        return launch_tile<FORMAT, MODE, 128, 256, 1, 4>(who, p, stream);  // enough tiles to fill the chip twice over
+      return launch_tile<FORMAT, MODE, 128, 128, 1, 4>(who, p, stream);
   }
 }
 
@@ -724,6 +743,14 @@ static int fill_single(const char* who, GemmParams& p, const void* x, const int3
 }
 
 }  // namespace dew
+
+extern "C" int dew_moe_tile_rows(int32_t rows) {
+  using namespace dew;
+  DEW_REQUIRE(rows == 0 || rows == 32 || rows == 64 || rows == 128 || rows == 256,
+              "dew_moe_tile_rows: tiles are 32, 64, 128 or 256 rows (0 = chosen per launch), not %d", rows);
+  forced_tile_rows = rows;
+  return DEW_MOE_OK;
+}
 
 extern "C" int dew_moe_grouped_gemm_bias(const void* x, const int32_t* gather, const int32_t* offsets,
                                          const dew_moe_bank* w, const float* bias, const int32_t* scatter, void* out,

@@ -2,6 +2,7 @@
 contiguity), allocates its outputs with torch (device memory and streams are torch's here; the arithmetic is
 the library's) and calls the C ABI on torch's current stream. No function reads a device value on the host."""
 
+import contextlib
 import dataclasses
 
 import torch
@@ -275,6 +276,17 @@ def split_rows(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     scale = torch.empty((rows,), dtype=torch.uint8, device=x.device)
     _lib.check(_lib.library().dew_moe_split_rows(_ptr(x), _ptr(split), _ptr(scale), rows, depth, _stream()), "dew_moe_split_rows")
     return split, scale
+
+
+@contextlib.contextmanager
+def tile_rows(rows: int):
+    """Within the block every grouped product uses block tiles of `rows` rows (32, 64, 128, 256) instead of the
+    per-launch choice: for tuning, and for tests that must reach one tile's code whatever the problem's size."""
+    _lib.check(_lib.library().dew_moe_tile_rows(rows), "dew_moe_tile_rows")
+    try:
+        yield
+    finally:
+        _lib.check(_lib.library().dew_moe_tile_rows(0), "dew_moe_tile_rows")
 
 
 def prefers_split(bank: PreparedBank, rows: int) -> bool:

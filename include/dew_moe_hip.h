@@ -101,6 +101,11 @@ size_t dew_moe_prepared_bytes(int32_t format, int32_t experts, int32_t depth, in
 int dew_moe_prepare_bank(const dew_moe_bank* reference, void* prepared, dew_moe_bank* out /* host */,
                          void* stream);
 
+/* Tuning and testing knob (no counterpart in the reference): every later grouped product of this process uses
+ * block tiles of `rows` rows (32, 64, 128 or 256; 256 with FP4 banks whose width is whole 256s); 0, the default,
+ * chooses per launch from the rows, experts and width.                                                      */
+int dew_moe_tile_rows(int32_t rows);
+
 /* ---- Grouped products (src/dew/nn/moe.py:666-770 expert_projection / paired_projections; replaces the
  *      launches of kernels/cutlass/ffi.cu:180-220 behind src/dew/nn/kernels/grouped_matmul.py:1826-1831) --
  * Sorted position i in [offsets[e], offsets[e+1]) belongs to expert e and reads row gather[i] of x (row i

@@ -109,15 +109,17 @@ def grouped_case(quant, experts, depth, width, sizes, seed):
 SIZES = [("ragged", [130, 0, 1, 257, 64, 0, 127, 5]), ("single", [3]), ("even", [128, 128, 128, 128])]
 
 
+@pytest.mark.parametrize("tile", [0, 32, 64, 128])
 @pytest.mark.parametrize("quant", ["fp8_channel", "fp8_block", "mxfp4", "nvfp4"])
 @pytest.mark.parametrize("label,sizes", SIZES, ids=[s[0] for s in SIZES])
-def test_grouped_gemm_matches_the_dequantized_fp32_sum(ops, quant, label, sizes):
+def test_grouped_gemm_matches_the_dequantized_fp32_sum(ops, quant, label, sizes, tile):
     """bf16 x decoded-weight products are exact in fp32, so kernel and oracle differ by summation order
     alone before the one bf16 rounding: allow one bf16 ulp (2^-8 relative) plus an fp32-sum floor."""
     bank, x, offsets = grouped_case(quant, len(sizes), 512, 256, sizes, seed=len(sizes) * 7 + len(quant))
     values, factor = dequantized(bank)
     want = oracle.grouped_matmul(bf16_np(x), values, sizes, factor=factor)
-    got = bf16_np(ops.grouped_gemm(x.cuda(), ops.prepare(bank.to("cuda")), torch.from_numpy(offsets).cuda()))
+    with ops.tile_rows(tile):
+        got = bf16_np(ops.grouped_gemm(x.cuda(), ops.prepare(bank.to("cuda")), torch.from_numpy(offsets).cuda()))
     scale = np.abs(want).max()
     assert np.abs(got - want).max() <= 2 ** -8 * scale
     assert (np.abs(got - want) <= 2 ** -7 * np.abs(want) + 1e-5 * scale).all()
@@ -160,8 +162,9 @@ def test_grouped_gemm_gathers_scatters_and_zeroes_unrouted_rows(ops):
     assert np.abs(got - want).max() <= 2 ** -8 * np.abs(want).max()
 
 
+@pytest.mark.parametrize("tile", [0, 32, 64, 128])
 @pytest.mark.parametrize("quant", ["fp8_channel", "fp8_block", "mxfp4", "nvfp4"])
-def test_gateup_swiglu_matches_the_two_products_and_the_rounded_epilogue(ops, quant):
+def test_gateup_swiglu_matches_the_two_products_and_the_rounded_epilogue(ops, quant, tile):
     sizes = [100, 0, 37, 200]
     rng = np.random.default_rng(21)
     gate, x, offsets = grouped_case(quant, 4, 512, 256, sizes, seed=1)
@@ -175,8 +178,9 @@ def test_gateup_swiglu_matches_the_two_products_and_the_rounded_epilogue(ops, qu
     want = oracle.swiglu(want_gate, want_up)
     xd, od, gd = x.cuda(), torch.from_numpy(offsets).cuda(), torch.from_numpy(gather).cuda()
     pg, pu = ops.prepare(gate.to("cuda")), ops.prepare(up.to("cuda"))
-    fused = bf16_np(ops.gateup_swiglu(xd, pg, pu, od, gather=gd))
-    apart = ops.swiglu(ops.grouped_gemm(xd, pg, od, gather=gd), ops.grouped_gemm(xd, pu, od, gather=gd))
+    with ops.tile_rows(tile):
+        fused = bf16_np(ops.gateup_swiglu(xd, pg, pu, od, gather=gd))
+        apart = ops.swiglu(ops.grouped_gemm(xd, pg, od, gather=gd), ops.grouped_gemm(xd, pu, od, gather=gd))
     assert np.array_equal(fused, bf16_np(apart))           # the fused epilogue is the unfused arithmetic
     scale = np.abs(want).max()
     # a one-ulp difference in gate or up moves the product by up to ~3 ulp of the result
@@ -263,10 +267,12 @@ def test_probes_run_and_the_copy_probe_copies(ops):
 
 @pytest.mark.parametrize("quant", ["fp8_channel", "fp8_block", "mxfp4", "nvfp4"])
 @pytest.mark.parametrize("depth", [128, 384, 640, 896])
-@pytest.mark.parametrize("label,sizes", [("decode", [3, 0, 9]), ("medium", [150, 70, 1]), ("large", [800])])
-def test_depths_that_leave_steps_after_the_unrolled_loop(ops, quant, depth, label, sizes):
+@pytest.mark.parametrize("label,sizes,tile", [("decode", [3, 0, 9], 32), ("small", [40, 70, 1], 64), ("medium", [150, 70, 1], 128),
+                                               ("large", [800], 256)])
+def test_depths_that_leave_steps_after_the_unrolled_loop(ops, quant, depth, label, sizes, tile):
     """Depth / 64 steps that are not a multiple of the main loop's unroll (3 or 4) end in separately compiled
-    steps; both launches must still agree with the oracle and with each other."""
+    steps; both launches must still agree with the oracle and with each other. Each tile height is forced, since
+    problems this small would all be given 32-row tiles."""
     if quant in ("mxfp4", "nvfp4"):
         depth = 2 * depth  # an NvFp4 bank's depth is whole 256s
     gate, x, offsets = grouped_case(quant, len(sizes), depth, 256, sizes, seed=depth + len(quant))
@@ -276,9 +282,10 @@ def test_depths_that_leave_steps_after_the_unrolled_loop(ops, quant, depth, labe
     want_gate = oracle.grouped_matmul(rows, gate_values, sizes, factor=gate_factor)
     xd, od = x.cuda(), torch.from_numpy(offsets).cuda()
     pg, pu = ops.prepare(gate.to("cuda")), ops.prepare(up.to("cuda"))
-    fused = bf16_np(ops.gateup_swiglu(xd, pg, pu, od))
-    got_gate = ops.grouped_gemm(xd, pg, od)
-    apart = bf16_np(ops.swiglu(got_gate, ops.grouped_gemm(xd, pu, od)))
+    with ops.tile_rows(tile):
+        fused = bf16_np(ops.gateup_swiglu(xd, pg, pu, od))
+        got_gate = ops.grouped_gemm(xd, pg, od)
+        apart = bf16_np(ops.swiglu(got_gate, ops.grouped_gemm(xd, pu, od)))
     assert np.array_equal(fused, apart)
     got_gate = bf16_np(got_gate)
     assert np.abs(got_gate - want_gate).max() <= 2 ** -8 * np.abs(want_gate).max() + 1e-6
