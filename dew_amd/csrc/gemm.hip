@@ -680,7 +680,7 @@ static int forced_tile_rows = 0;  // dew_moe_tile_rows: 0 leaves the choice to t
 static int tile_rows(const GemmParams& p, bool fp4) {
   if (forced_tile_rows != 0) return forced_tile_rows;
   const int average = p.rows / p.experts;
-  if (fp4 && average >= 768 && p.width % 256 == 0) return 256;
+  if (fp4 && average >= 1024 && p.width % 256 == 0) return 256;  // below, the half tile a group wastes outweighs its gain
   int rows = average <= 36 ? 32 : average <= 72 ? 64 : 128;
   const long long strips = p.width / 128;
   while (rows > 32 && (p.rows / rows + p.experts / 2) * strips < 256) rows /= 2;

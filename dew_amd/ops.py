@@ -293,7 +293,7 @@ def prefers_split(bank: PreparedBank, rows: int) -> bool:
     """Whether a product of `rows` rows through `bank` is better run on split rows (`split_rows` then the `_split`
     launches): an MXFP4 bank of whole 256-column strips whose groups average the 256-row tiles' fill."""
     experts, _, width = bank.shape
-    return bank.descriptor.format == _lib.W_MXFP4 and width % 256 == 0 and rows // experts >= 768
+    return bank.descriptor.format == _lib.W_MXFP4 and width % 256 == 0 and rows // experts >= 1024
 
 
 def grouped_gemm_split(split: torch.Tensor, scale: torch.Tensor, bank: PreparedBank, offsets: torch.Tensor, *,
