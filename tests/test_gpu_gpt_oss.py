@@ -46,7 +46,7 @@ def test_the_bias_meets_the_fp32_sums_before_their_one_rounding(ops, quant, labe
     prepared = ops.prepare(bank.to("cuda"))
     got = ops.grouped_gemm(x.cuda(), prepared, torch.from_numpy(offsets).cuda(), bias=held.cuda(), scatter=scatter.cuda())
     got = bf16_np(got)[scatter.numpy()]
-    assert np.abs(got - want).max() <= 2 ** -8 * np.abs(want).max()
+    assert np.abs(got - want).max() <= 2 ** -7 * np.abs(want).max()
     assert (got == want).mean() > 0.97
     # a product whose rounding comes before the bias would differ: the bias is of the outputs' size
     late = oracle.bf16_round(oracle.grouped_matmul(bf16_np(x), values, sizes, factor=factor) + held.numpy()[np.repeat(

@@ -114,14 +114,14 @@ SIZES = [("ragged", [130, 0, 1, 257, 64, 0, 127, 5]), ("single", [3]), ("even", 
 @pytest.mark.parametrize("label,sizes", SIZES, ids=[s[0] for s in SIZES])
 def test_grouped_gemm_matches_the_dequantized_fp32_sum(ops, quant, label, sizes, tile):
     """bf16 x decoded-weight products are exact in fp32, so kernel and oracle differ by summation order
-    alone before the one bf16 rounding: allow one bf16 ulp (2^-8 relative) plus an fp32-sum floor."""
+    alone before the one bf16 rounding: allow one bf16 ulp of the largest output (at most 2^-7 of it)."""
     bank, x, offsets = grouped_case(quant, len(sizes), 512, 256, sizes, seed=len(sizes) * 7 + len(quant))
     values, factor = dequantized(bank)
     want = oracle.grouped_matmul(bf16_np(x), values, sizes, factor=factor)
     with ops.tile_rows(tile):
         got = bf16_np(ops.grouped_gemm(x.cuda(), ops.prepare(bank.to("cuda")), torch.from_numpy(offsets).cuda()))
     scale = np.abs(want).max()
-    assert np.abs(got - want).max() <= 2 ** -8 * scale
+    assert np.abs(got - want).max() <= 2 ** -7 * scale
     assert (np.abs(got - want) <= 2 ** -7 * np.abs(want) + 1e-5 * scale).all()
     assert (got == want).mean() > 0.97                     # nearly every element rounds identically
 
@@ -159,7 +159,7 @@ def test_grouped_gemm_gathers_scatters_and_zeroes_unrouted_rows(ops):
     got = bf16_np(ops.grouped_gemm(tokens.cuda(), ops.prepare(bank.to("cuda")), torch.from_numpy(offsets).cuda(),
                                    gather=torch.from_numpy(gather).cuda(), scatter=torch.from_numpy(scatter).cuda(), rows=rows))
     assert not got[scatter[200:]].any()
-    assert np.abs(got - want).max() <= 2 ** -8 * np.abs(want).max()
+    assert np.abs(got - want).max() <= 2 ** -7 * np.abs(want).max()
 
 
 @pytest.mark.parametrize("tile", [0, 32, 64, 128])
@@ -249,7 +249,7 @@ def test_large_tile_kernels_match_the_oracle(ops, quant):
     with ops.tile_rows(256):
         got_gate = bf16_np(ops.grouped_gemm(xd, pg, od))
         fused = bf16_np(ops.gateup_swiglu(xd, pg, pu, od))
-    assert np.abs(got_gate - want_gate).max() <= 2 ** -8 * np.abs(want_gate).max() and (got_gate == want_gate).mean() > 0.97
+    assert np.abs(got_gate - want_gate).max() <= 2 ** -7 * np.abs(want_gate).max() and (got_gate == want_gate).mean() > 0.97
     assert np.abs(fused - want).max() <= 2 ** -6 * np.abs(want).max() and (fused == want).mean() > 0.9
 
 
@@ -290,7 +290,7 @@ def test_depths_that_leave_steps_after_the_unrolled_loop(ops, quant, depth, labe
         apart = bf16_np(ops.swiglu(got_gate, ops.grouped_gemm(xd, pu, od)))
     assert np.array_equal(fused, apart)
     got_gate = bf16_np(got_gate)
-    assert np.abs(got_gate - want_gate).max() <= 2 ** -8 * np.abs(want_gate).max() + 1e-6
+    assert np.abs(got_gate - want_gate).max() <= 2 ** -7 * np.abs(want_gate).max() + 1e-6
     assert (got_gate == want_gate).mean() > 0.97
 
 
@@ -339,7 +339,7 @@ def test_split_activations_give_the_bf16_products_on_mxfp4_banks(ops, depth):
     split, scale = ops.split_rows(xd)
     got_gate = bf16_np(ops.grouped_gemm_split(split, scale, pg, od, gather=gd, scatter=sd))[scatter]
     plain_gate = bf16_np(ops.grouped_gemm(xd, pg, od, gather=gd))
-    assert np.abs(got_gate - want_gate).max() <= 2 ** -8 * np.abs(want_gate).max()
+    assert np.abs(got_gate - want_gate).max() <= 2 ** -7 * np.abs(want_gate).max()
     assert (got_gate == want_gate).mean() > 0.97 and (got_gate == plain_gate).mean() > 0.97
     fused = bf16_np(ops.gateup_swiglu_split(split, scale, pg, pu, od, gather=gd))
     assert np.abs(fused - want).max() <= 2 ** -6 * np.abs(want).max() and (fused == want).mean() > 0.9

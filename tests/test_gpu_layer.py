@@ -170,7 +170,7 @@ def test_more_experts_than_one_scan_round_and_every_expert_chosen():
     values, factor = dequantized(bank)
     want = oracle.grouped_matmul(bf16_np(x), values, sizes.tolist(), factor=factor)
     got = bf16_np(ops.grouped_gemm(x.cuda(), ops.prepare(bank.to("cuda")), torch.from_numpy(offsets).cuda()))
-    assert np.abs(got - want).max() <= 2 ** -8 * np.abs(want).max() and (got == want).mean() > 0.97
+    assert np.abs(got - want).max() <= 2 ** -7 * np.abs(want).max() and (got == want).mean() > 0.97
     logits = torch.from_numpy(rng.standard_normal((33, 8)).astype(np.float32))
     weights, indices = ops.route(logits.cuda(), 8, score_function="softmax", normalize_weights=True)
     want_weights, want_indices = oracle.route(logits.numpy(), 8, score_function="softmax", normalize_weights=True)
