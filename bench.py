@@ -75,7 +75,7 @@ def build_workload(case, device, seed=0):
 class Stepper:
     """One step of the hot path, launch by launch, with optional HIP events around the gate/up launch."""
 
-    def __init__(self, case, data, split=False):
+    def __init__(self, case, data, split=True):
         import torch
 
         from dew_amd import gemm, ops
@@ -95,27 +95,36 @@ class Stepper:
         if timed:
             start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             start.record()
-        routed = case.tokens * case.top_k
-        if self.split and ops.prefers_split(self.gate, routed):
-            # an MXFP4 bank and groups of hundreds of rows: rows as two e4m3 terms, scaled matrix instructions
-            pieces = ops.split_rows(data["x"])
-            if timed:
-                start.record()
-            hidden = ops.gateup_swiglu_split(*pieces, self.gate, self.up, plan.offsets, gather=plan.rows)
-        else:
-            hidden = ops.gateup_swiglu(data["x"], self.gate, self.up, plan.offsets, gather=plan.rows)
-        if timed:
-            stop.record()
-            self.events.append((start, stop))
-        if self.split and ops.prefers_split(self.down, routed):
-            slots = ops.grouped_gemm_split(*ops.split_rows(hidden), self.down, plan.offsets, scatter=plan.order)
-        else:
-            slots = ops.grouped_gemm(hidden, self.down, plan.offsets, scatter=plan.order)
+        slots = self.project(plan, (start, stop) if timed else None)
         addend = None
         if self.shared is not None:
             shared_hidden = ops.gateup_swiglu(data["x"], self.shared[0], self.shared[1], self.dense_offsets)
             addend = ops.grouped_gemm(shared_hidden, self.shared[2], self.dense_offsets)
         return ops.combine(slots.view(case.tokens, case.top_k, case.d_model), weights, addend), plan
+
+    def on_split_rows(self):
+        """Whether the routed experts run on split rows and the scaled matrix instruction (the library's rule)."""
+        return self.split and self.ops.prefers_split_pair(self.gate, self.up, self.down, self.case.tokens * self.case.top_k)
+
+    def project(self, plan, events=None):
+        """The routed experts' two launches: [T * k, D] rows at their slots. `events` bracket the gate/up launch."""
+        ops, data = self.ops, self.data
+        if self.on_split_rows():
+            # MXFP4 banks and groups of a thousand rows: the rows as two e4m3 terms and the scaled matrix instruction;
+            # the gate/up launch writes its hidden rows already split, so the only extra pass is the split of x
+            pieces = ops.split_rows(data["x"])
+            if events:
+                events[0].record()
+            hidden = ops.gateup_swiglu_split_out(*pieces, self.gate, self.up, plan.offsets, gather=plan.rows)
+            if events:
+                events[1].record()
+                self.events.append(events)
+            return ops.grouped_gemm_split_blocks(*hidden, self.down, plan.offsets, scatter=plan.order)
+        hidden = ops.gateup_swiglu(data["x"], self.gate, self.up, plan.offsets, gather=plan.rows)
+        if events:
+            events[1].record()
+            self.events.append(events)
+        return ops.grouped_gemm(hidden, self.down, plan.offsets, scatter=plan.order)
 
     def gateup_ms(self):
         return sum(start.elapsed_time(stop) for start, stop in self.events) / max(1, len(self.events))
@@ -215,9 +224,9 @@ def main():
     parser.add_argument("--calibrate-copy", action="store_true",
                         help="only run the plain copy probe (1 GiB read + 1 GiB written, 5 launches): the known traffic "
                              "that rocprofv3's FETCH_SIZE / WRITE_SIZE are scaled by")
-    parser.add_argument("--split", action="store_true",
-                        help="MXFP4 banks with groups of hundreds of rows: rows split into two e4m3 terms and the scaled matrix "
-                             "instruction instead of the bf16 one (same exact products; the default measured faster overall)")
+    parser.add_argument("--bf16-operands", action="store_true",
+                        help="keep MXFP4 banks with groups of a thousand rows on the bf16 matrix instruction too (the default "
+                             "there: rows split into two e4m3 terms and the scaled instruction, the library's own choice)")
     parser.add_argument("--graph", choices=["auto", "on", "off"], default="auto",
                         help="replay the step as one captured HIP graph (auto: for the launch-bound configs c1 and c3)")
     args = parser.parse_args()
@@ -241,7 +250,7 @@ def main():
         return
     case = CONFIGS[args.config]
     data = build_workload(case, device)
-    stepper = Stepper(case, data, split=args.split)
+    stepper = Stepper(case, data, split=not args.bf16_operands)
 
     graphed = args.graph == "on" or (args.graph == "auto" and args.config in ("c1", "c3"))
     for _ in range(args.warmup):
@@ -291,10 +300,17 @@ def main():
                     "unit": "GB/s", "traffic": None}
     else:
         roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAKS["bf16_mfma"], "unit": "TFLOP/s", "traffic": None,
-                    "peak_note": "dense bf16 MFMA: the kernel multiplies bf16 activations by weights dequantized exactly to "
-                                 "bf16 (v_mfma_f32_32x32x16_bf16)",
+                    "peak_note": ("the kernel multiplies each bf16 activation as two e4m3 terms by the stored FP4 codes "
+                                  "(v_mfma_scale_f32_32x32x64_f8f6f4, which runs at the dense fp8 rate, 5.0 PFLOP/s published): "
+                                  "two instruction flops per algorithmic flop, so the algorithm's ceiling is 2.5 PFLOP/s, the "
+                                  "dense bf16 peak; achieved counts algorithmic flops only") if stepper.on_split_rows() else
+                                 ("dense bf16 MFMA: the kernel multiplies bf16 activations by weights dequantized exactly to "
+                                  "bf16 (v_mfma_f32_32x32x16_bf16)"),
                     "frac_of_fp8_peak": round(achieved / PEAKS["fp8_mfma"], 4), "frac_of_fp4_peak": round(achieved / PEAKS["fp4_mfma"], 4)}
     roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
+    if not decode and stepper.on_split_rows():
+        roofline["executed"] = {"tflops": round(2 * achieved, 1), "frac_of_fp8_peak": round(2 * achieved / PEAKS["fp8_mfma"], 4),
+                                "note": "instruction flops: both terms' products"}
     roofline["traffic"] = measured_traffic(args.config)
     roofline["algorithmic"] = {"per_launch": gateup_bytes if decode else gateup_flops, "unit": "bytes" if decode else "flop"}
     sustained_mfma, sustained_copy = sustained_rates(device)
@@ -303,7 +319,7 @@ def main():
                              "note": "measured in this run by dew_moe_probe_mfma / dew_moe_probe_copy: the rate the chip holds on "
                                      "random data at its power limit, below the published peak"}
     roofline["kernel"] = "grouped_gemm_kernel<paired gate/up + SwiGLU>" + (
-        " on split rows (v_mfma_scale_f32_32x32x64_f8f6f4, two e4m3 terms x FP4)" if args.split and case.quant == "mxfp4" else "")
+        " on split rows (v_mfma_scale_f32_32x32x64_f8f6f4, two e4m3 terms x FP4)" if stepper.on_split_rows() else "")
     roofline["kernel_ms"] = round(gateup_ms, 4)
 
     result = {
@@ -322,8 +338,7 @@ def main():
         baseline, (slots, want) = cpu_baseline(case, data, out, plan)
         result["cpu_baseline"] = baseline
         # parity on the sample at full size: the device's down-projection rows for those slots
-        hidden = ops.gateup_swiglu(data["x"], stepper.gate, stepper.up, plan.offsets, gather=plan.rows)
-        projected = ops.grouped_gemm(hidden, stepper.down, plan.offsets, scatter=plan.order).float().cpu().numpy()
+        projected = stepper.project(plan).float().cpu().numpy()
         got = projected[slots]
         scale = float(np.abs(want).max())
         result["sample_parity"] = {"max_abs_over_max_ref": round(float(np.abs(got - want).max() / scale), 6),

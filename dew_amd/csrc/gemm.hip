@@ -41,11 +41,13 @@ typedef __attribute__((ext_vector_type(8))) int i32x8_t;       // an operand of 
 // (dew_moe_split_rows): v_mfma_scale_f32_32x32x64_f8f6f4 takes the FP4 codes and their power-of-two block scales
 // as they are stored, so the weights are not dequantized at all.
 constexpr int kFormatMxSplit = 5;
+constexpr int kFormatMxSplitBlocks = 6;  // the same with one activation scale per row and 128 depths, not per row
 
 constexpr int BK = 64;
 constexpr int kThreads = 256;
 constexpr int kChunksPerRow = BK / 8;  // 16-byte chunks in an LDS row
 constexpr int kMaxDepthBlocks = 256;   // FP8 128 x 128 blocks: depth up to 32768
+constexpr int kMaxBlockScaleDepth = 24576;  // block-scaled split rows: 256 rows x 192 scale bytes fit the LDS behind the ring
 
 struct BankView {
   const uint8_t* codes;
@@ -60,15 +62,18 @@ struct GemmParams {
   const int32_t* scatter;
   BankView w0, w1;
   bf16_t* out;
-  const uint8_t* a_scale;  // split activations: each source row's e8m0 scale
+  const uint8_t* a_scale;  // split activations: each source row's e8m0 scale, or its row of block_scale_pitch(depth) of them
+  uint8_t* out_scale;      // split output: each written row's block_scale_pitch(width) e8m0 scales, one for 128 columns
   const float* bias;  // [experts, width] values of the compute dtype held in fp32, or null
   float limit;        // the interleaved gated epilogue's clamp
   int experts, depth, width, rows, m_tile_bound;
 };
 
-// What the epilogue writes: the rounded product (plus bias); SwiGLU of two banks' products; or, for one bank
-// whose columns interleave gate (even) and up (odd), the clamped quick-GELU gating of each column pair.
-enum Epilogue { kPlain = 0, kSwigluOfTwo = 1, kInterleavedGated = 2 };
+// What the epilogue writes: the rounded product (plus bias); SwiGLU of two banks' products; for one bank whose
+// columns interleave gate (even) and up (odd), the clamped quick-GELU gating of each column pair; or the SwiGLU of
+// two banks' products already split into two e4m3 terms under one scale per row and 128 columns, which is what the
+// next product's scaled matrix instructions read (kFormatMxSplitBlocks).
+enum Epilogue { kPlain = 0, kSwigluOfTwo = 1, kInterleavedGated = 2, kSwigluOfTwoSplit = 3 };
 
 // LDS index of 16-byte chunk `chunk` of row `row` (128-byte rows). The chunk is xor-swizzled by
 // f(row) = ((row >> 1) & 7) ^ ((row & 1) << 2), chosen against the measured service order of gfx950's LDS:
@@ -113,6 +118,9 @@ __device__ __forceinline__ bf16x8_t fragment_fp4_pow2(uint32_t word, float scale
       __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 3))});
 }
 
+// Bytes of one row's block scales (one e8m0 byte for 128 elements), padded to whole 16-byte loads.
+__host__ __device__ constexpr int block_scale_pitch(int elements) { return (elements / 128 + 15) / 16 * 16; }
+
 // Dynamic LDS of a block: the three-stage ring of A rows, or the staged output tile where that is larger
 // (the 32-row tile of 256 columns).
 template <int BM, int BN, int MODE>
@@ -145,11 +153,13 @@ __device__ __forceinline__ void schedule_phase() {
 // bytes); each owns (BM/WM) x (BN/WN) of every matrix as 32 x 32 MFMA tiles.
 template <int FORMAT, int MODE, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 : 1) * BN == 256) ? 2 : 1) void grouped_gemm_kernel(GemmParams p) {
-  constexpr bool PAIRED = MODE == kSwigluOfTwo;
+  constexpr bool PAIRED = MODE == kSwigluOfTwo || MODE == kSwigluOfTwoSplit;
+  constexpr bool kSplitOut = MODE == kSwigluOfTwoSplit;
   constexpr bool kGated = MODE == kInterleavedGated;
   constexpr int kOutBN = kGated ? BN / 2 : BN;  // output columns of the tile
   static_assert(WM * WN == 4 && BM % (32 * WM) == 0 && BN % (32 * WN) == 0 && BM % 32 == 0, "tile shape");
-  constexpr bool kSplit = FORMAT == kFormatMxSplit;
+  constexpr bool kSplit = FORMAT == kFormatMxSplit || FORMAT == kFormatMxSplitBlocks;
+  constexpr bool kBlockScales = FORMAT == kFormatMxSplitBlocks;
   constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4 || kSplit;
   constexpr bool kPow2 = FORMAT == DEW_MOE_W_MXFP4 || kSplit;
   constexpr int kMatrices = PAIRED ? 2 : 1;
@@ -233,6 +243,9 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
       const int sorted = tail_begin + item / (kOutBN / 8);
       const int row = p.scatter ? p.scatter[sorted] : sorted;
       *reinterpret_cast<u32x4_t*>(p.out + static_cast<size_t>(row) * out_width + out_n0 + (item % (kOutBN / 8)) * 8) = u32x4_t{0, 0, 0, 0};
+      if constexpr (kSplitOut) {  // zero terms under a unit scale
+        if (item % (kOutBN / 8) == 0) p.out_scale[static_cast<size_t>(sorted) * block_scale_pitch(p.width) + n0 / 128] = 127;
+      }
     }
     return;
   }
@@ -262,10 +275,42 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     a_scale_word[i] = 0;
     if constexpr (kSplit) {
       const int sorted = row0 + min(wm0 + 32 * i + lane % 32, valid_rows - 1);
-      const int byte = p.a_scale[p.gather ? p.gather[sorted] : sorted];
-      a_scale_word[i] = byte | ((byte - 4) << 8);
+      const int source = p.gather ? p.gather[sorted] : sorted;
+      if constexpr (!kBlockScales) {
+        const int byte = p.a_scale[source];
+        a_scale_word[i] = byte | ((byte - 4) << 8);
+      }
     }
   }
+  // Block scales change every 128 depths (two steps). The tile's rows' scales, all depths of them, are copied into
+  // the LDS behind the ring before the loop (thread t copies row t, 16 bytes a load), and the loop reads its bytes
+  // from there into two sets of registers, the one of the next 128 depths while this one multiplies. (Read from
+  // global memory inside the loop they cost 14 to 20 % of the kernel, however early they were issued: every byte
+  // is a first touch of its cache line, and the vmcnt wait of each step's barrier, which counts loads in order,
+  // stalled on them.)
+  const int a_pitch = block_scale_pitch(p.depth);
+  uint8_t* block_scales = reinterpret_cast<uint8_t*>(lds + kStages * kStageChunks);
+  if constexpr (kBlockScales) {
+    static_assert(!kBlockScales || BM == kThreads, "one thread copies one row's scales");
+    const int sorted = row0 + min(tid, valid_rows - 1);
+    const int source = p.gather ? p.gather[sorted] : sorted;
+    const u32x4_t* from = reinterpret_cast<const u32x4_t*>(p.a_scale + static_cast<size_t>(source) * a_pitch);
+    u32x4_t* to = reinterpret_cast<u32x4_t*>(block_scales + tid * a_pitch);
+    for (int piece = 0; piece < a_pitch / 16; ++piece) to[piece] = from[piece];
+  }
+  int a_block_word[2][kBlockScales ? TI : 1], a_block_byte[kBlockScales ? TI : 1];
+  auto load_block_scales = [&](int block) __attribute__((always_inline)) {
+    if constexpr (kBlockScales) {
+#pragma unroll
+      for (int i = 0; i < TI; ++i) a_block_byte[i] = block_scales[(wm0 + 32 * i + lane % 32) * a_pitch + block];
+    }
+  };
+  auto form_block_words = [&](auto buffer) __attribute__((always_inline)) {
+    if constexpr (kBlockScales) {
+#pragma unroll
+      for (int i = 0; i < TI; ++i) a_block_word[buffer.value][i] = a_block_byte[i] | ((a_block_byte[i] - 4) << 8);
+    }
+  };
   auto load_a = [&](u32x4_t* stage, int step, auto begin, auto end) __attribute__((always_inline)) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass, which only needs the kernel's stub, does not know the builtin
 #pragma unroll
@@ -385,6 +430,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   // both operands' power-of-two scales; the block scale byte is the e4m3 of a normal power of two, 2^(field - 7).
   auto multiply_term = [&](auto set, auto term) __attribute__((always_inline)) {
     if constexpr (kSplit) {
+      constexpr int kBuffer = (set.value / 2) % 2;  // block scales: steps 0, 1 of the unrolled four read set 0, steps 2, 3 set 1
 #pragma unroll
       for (int m = 0; m < kMatrices; ++m)
 #pragma unroll
@@ -393,9 +439,11 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
           const i32x8_t codes = {static_cast<int>(raw[0]), static_cast<int>(raw[1]), static_cast<int>(raw[2]), static_cast<int>(raw[3]), 0, 0, 0, 0};
           const int b_scale = static_cast<int>(((s_regs[set.value][m * TJ + j] >> 3) & 15u) + 120u);
 #pragma unroll
-          for (int i = 0; i < TI; ++i)
+          for (int i = 0; i < TI; ++i) {
             acc[m][i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_term[term.value][i], codes, acc[m][i][j], 0, 4, term.value,
-                                                                        a_scale_word[i], 0, b_scale);
+                                                                        kBlockScales ? a_block_word[kBuffer][i] : a_scale_word[i], 0,
+                                                                        b_scale);
+          }
         }
     }
   };
@@ -467,6 +515,10 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
       __builtin_amdgcn_s_barrier();
       asm volatile("" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
+      // block scales: the bytes of the next 128 depths are read from the LDS in the second phase of an even step
+      // and formed into words in the second phase of the odd step that follows, one phase before they multiply
+      if constexpr (kBlockScales && set.value % 2 == 0) load_block_scales(min(step / 2 + 1, p.depth / 128 - 1));
+      if constexpr (kBlockScales && set.value % 2 == 1) form_block_words(std::integral_constant<int, 1 - (set.value / 2) % 2>{});
       fetch_term(next, c0);
       multiply_term(set, c1);
       load_a(fill, ahead_a, ah, a4);
@@ -526,6 +578,8 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
   if constexpr (kSplit) {
+    load_block_scales(0);
+    form_block_words(c0);
     fetch_term(lds, c0);
   } else {
     fetch(lds, c0, c0);
@@ -624,9 +678,53 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     for (int it = 0; it < kStoreIters; ++it) {
       const int item = tid + it * kThreads;
       const int staged_row = item / kRowChunks, chunk = item % kRowChunks;
-      if (pass * kPassRows + staged_row < valid_rows)
-        *reinterpret_cast<u32x4_t*>(p.out + static_cast<size_t>(out_rows[it]) * out_width + out_n0 + chunk * 8) =
-            *reinterpret_cast<const u32x4_t*>(staged + staged_row * kRowDwords + chunk * 4);
+      const bool valid = pass * kPassRows + staged_row < valid_rows;
+      const u32x4_t words = *reinterpret_cast<const u32x4_t*>(staged + staged_row * kRowDwords + chunk * 4);
+      if constexpr (kSplitOut) {
+        // The row's 128 columns of this tile as two e4m3 terms under one scale (dew_moe_split_rows' arithmetic on a
+        // 128-column block): the 16 lanes that hold the row's chunks agree on its largest exponent field, each
+        // converts its 8 values and writes their hi and lo bytes where the scaled instruction's operand order puts
+        // them (split.hip: each 64 depths as [group 0 hi][group 0 lo][group 1 hi][group 1 lo]).
+        static_assert(!kSplitOut || kRowChunks == 16, "a row's chunks fill one 16-lane row of the wavefront");
+        uint32_t largest = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) largest = max(largest, max((words[i] >> 7) & 0xFFu, (words[i] >> 23) & 0xFFu));
+        largest = max(largest, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(largest), 0xB1, 0xF, 0xF, true)));   // lane ^ 1
+        largest = max(largest, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(largest), 0x4E, 0xF, 0xF, true)));   // lane ^ 2
+        largest = max(largest, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(largest), 0x141, 0xF, 0xF, true)));  // 7 - lane in each 8
+        largest = max(largest, static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(largest), 0x140, 0xF, 0xF, true)));  // 15 - lane
+        const int field = min(max(static_cast<int>(largest), 16), 254);
+        const int hi_byte = field - 7;
+        const float inverse = __uint_as_float(static_cast<uint32_t>(254 - hi_byte) << 23);
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          v[2 * i] = __uint_as_float(words[i] << 16) * inverse;
+          v[2 * i + 1] = __uint_as_float(words[i] & 0xFFFF0000u) * inverse;
+        }
+        uint32_t hi[2], lo[2];
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+          hi[w] = __builtin_amdgcn_cvt_pk_fp8_f32(v[4 * w], v[4 * w + 1], 0, false);
+          hi[w] = __builtin_amdgcn_cvt_pk_fp8_f32(v[4 * w + 2], v[4 * w + 3], hi[w], true);
+          const auto first = __builtin_amdgcn_cvt_pk_f32_fp8(hi[w], false), second = __builtin_amdgcn_cvt_pk_f32_fp8(hi[w], true);
+          lo[w] = __builtin_amdgcn_cvt_pk_fp8_f32((v[4 * w] - first[0]) * 16.0f, (v[4 * w + 1] - first[1]) * 16.0f, 0, false);
+          lo[w] = __builtin_amdgcn_cvt_pk_fp8_f32((v[4 * w + 2] - second[0]) * 16.0f, (v[4 * w + 3] - second[1]) * 16.0f, lo[w], true);
+        }
+        if (valid) {
+          const int within = chunk % 8, half = within / 4, group = (within % 4) / 2, piece = within % 2;
+          uint8_t* block = reinterpret_cast<uint8_t*>(p.out + static_cast<size_t>(out_rows[it]) * out_width + out_n0) +
+                           (chunk / 8) * 128 + group * 64 + half * 16 + piece * 8;
+          *reinterpret_cast<uint32_t*>(block) = hi[0];
+          *reinterpret_cast<uint32_t*>(block + 4) = hi[1];
+          *reinterpret_cast<uint32_t*>(block + 32) = lo[0];
+          *reinterpret_cast<uint32_t*>(block + 36) = lo[1];
+          if (chunk == 0)
+            p.out_scale[static_cast<size_t>(row0 + pass * kPassRows + staged_row) * block_scale_pitch(p.width) + n0 / 128] = static_cast<uint8_t>(hi_byte);
+        }
+      } else {
+        if (valid) *reinterpret_cast<u32x4_t*>(p.out + static_cast<size_t>(out_rows[it]) * out_width + out_n0 + chunk * 8) = words;
+      }
     }
   }
 }
@@ -649,7 +747,9 @@ static int check_bank(const char* who, const dew_moe_bank* bank, const char* nam
 
 template <int FORMAT, int MODE, int BM, int BN, int WM, int WN>
 static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
-  constexpr size_t kShared = shared_bytes<BM, BN, MODE>();
+  // block-scaled activations keep their tile's scales behind the ring (reserved at their largest: kMaxBlockScaleDepth)
+  constexpr size_t kShared = shared_bytes<BM, BN, MODE>() +
+                             (FORMAT == kFormatMxSplitBlocks ? static_cast<size_t>(BM) * block_scale_pitch(kMaxBlockScaleDepth) : 0);
   auto kernel = grouped_gemm_kernel<FORMAT, MODE, BM, BN, WM, WN>;
   static bool configured = false;  // dynamic LDS above 64 KiB must be opted into once per kernel
   if (!configured) {
@@ -819,6 +919,60 @@ extern "C" int dew_moe_gateup_swiglu_split(const void* x_split, const uint8_t* x
   p.width = gate->width;
   p.rows = rows;
   return launch_tile<kFormatMxSplit, kSwigluOfTwo, 256, 128, 2, 2>(who, p, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int dew_moe_grouped_gemm_split_blocks(const void* x_split, const uint8_t* x_scales, const int32_t* gather,
+                                                 const int32_t* offsets, const dew_moe_bank* w, const float* bias,
+                                                 const int32_t* scatter, void* out, int32_t rows, void* stream) {
+  using namespace dew;
+  const char* who = "dew_moe_grouped_gemm_split_blocks";
+  if (int rc = check_bank(who, w, "weight")) return rc;
+  DEW_REQUIRE(w->format == DEW_MOE_W_MXFP4 && w->width % 256 == 0,
+              "%s: split activations multiply an MXFP4 bank (power-of-two block scales) whose width is whole 256s; this one is "
+              "format %d, width %d", who, w->format, w->width);
+  DEW_REQUIRE(w->depth <= kMaxBlockScaleDepth, "%s: bank depth %d is above %d (a tile's block scales are kept in the LDS)", who,
+              w->depth, kMaxBlockScaleDepth);
+  DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
+  if (rows == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(x_scales && aligned16(x_scales), "%s: the rows' scales must not be null and must be 16-byte aligned", who);
+  GemmParams p{};
+  if (int rc = fill_single(who, p, x_split, gather, offsets, w, bias, scatter, out, rows)) return rc;
+  p.a_scale = x_scales;
+  return launch_tile<kFormatMxSplitBlocks, kPlain, 256, 256, 2, 2>(who, p, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int dew_moe_gateup_swiglu_split_out(const void* x_split, const uint8_t* x_scale, const int32_t* gather,
+                                               const int32_t* offsets, const dew_moe_bank* gate, const dew_moe_bank* up,
+                                               void* hidden_split, uint8_t* hidden_scales, int32_t rows, void* stream) {
+  using namespace dew;
+  const char* who = "dew_moe_gateup_swiglu_split_out";
+  if (int rc = check_bank(who, gate, "gate")) return rc;
+  if (int rc = check_bank(who, up, "up")) return rc;
+  DEW_REQUIRE(gate->format == DEW_MOE_W_MXFP4 && up->format == DEW_MOE_W_MXFP4,
+              "%s: split activations multiply MXFP4 banks (power-of-two block scales); these are formats %d and %d", who,
+              gate->format, up->format);
+  DEW_REQUIRE(gate->experts == up->experts && gate->depth == up->depth && gate->width == up->width,
+              "%s: gate [%d, %d, %d] and up [%d, %d, %d] differ", who, gate->experts, gate->depth, gate->width, up->experts,
+              up->depth, up->width);
+  DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
+  if (rows == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(x_split && x_scale && offsets && hidden_split && hidden_scales,
+              "%s: x_split, x_scale, offsets, hidden_split and hidden_scales must not be null", who);
+  DEW_REQUIRE(aligned16(x_split) && aligned16(hidden_split), "%s: x_split and hidden_split must be 16-byte aligned", who);
+  GemmParams p{};
+  p.x = static_cast<const bf16_t*>(x_split);
+  p.a_scale = x_scale;
+  p.gather = gather;
+  p.offsets = offsets;
+  p.w0 = BankView{static_cast<const uint8_t*>(gate->codes), gate->scales, gate->tensor_scale};
+  p.w1 = BankView{static_cast<const uint8_t*>(up->codes), up->scales, up->tensor_scale};
+  p.out = static_cast<bf16_t*>(hidden_split);
+  p.out_scale = hidden_scales;
+  p.experts = gate->experts;
+  p.depth = gate->depth;
+  p.width = gate->width;
+  p.rows = rows;
+  return launch_tile<kFormatMxSplit, kSwigluOfTwoSplit, 256, 128, 2, 2>(who, p, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int dew_moe_gateup_interleaved(const void* x, const int32_t* gather, const int32_t* offsets,

@@ -220,6 +220,12 @@ class ExpertMLP(_Module):
     def _project(self, tokens: Gathered, sizes: GroupSizes, kernels) -> torch.Tensor:
         """src/dew/nn/moe.py:1305-1326."""
         gate_w, up_w, down_w = kernels
+        if self.fused and self.dtype in (None, torch.bfloat16):
+            # large groups on MXFP4 banks: both launches on the scaled matrix instruction, the hidden rows never in bf16
+            out = gemm.swiglu_mlp_on_split_rows(tokens.tokens, gate_w, up_w, down_w, sizes, gather=tokens.rows,
+                                                scatter=tokens.slots, implementation=_implementation(self.implementation))
+            if out is not None:
+                return out
         if self.fused:
             hidden = gated_projections(tokens, gate_w, up_w, sizes, self.dtype, self.implementation, self.precision)
         else:

@@ -296,6 +296,18 @@ def prefers_split(bank: PreparedBank, rows: int) -> bool:
     return bank.descriptor.format == _lib.W_MXFP4 and width % 256 == 0 and rows // experts >= 1024
 
 
+MAX_BLOCK_SCALE_DEPTH = 24576
+"""`grouped_gemm_split_blocks` keeps a tile's rows' block scales in the LDS: 256 rows of 192 bytes at most."""
+
+
+def prefers_split_pair(gate: PreparedBank, up: PreparedBank, down: PreparedBank, rows: int) -> bool:
+    """Whether a SwiGLU expert MLP of `rows` rows is better run as `gateup_swiglu_split_out` then
+    `grouped_gemm_split_blocks`: all three banks as `prefers_split` wants them, the down bank's depth the gate's width
+    and within the LDS's room for its scales."""
+    return prefers_split(gate, rows) and prefers_split(up, rows) and prefers_split(down, rows) and \
+        gate.shape == up.shape and down.shape[1] == gate.shape[2] and down.shape[1] <= MAX_BLOCK_SCALE_DEPTH
+
+
 def grouped_gemm_split(split: torch.Tensor, scale: torch.Tensor, bank: PreparedBank, offsets: torch.Tensor, *,
                        gather: torch.Tensor | None = None, scatter: torch.Tensor | None = None, rows: int | None = None,
                        bias: torch.Tensor | None = None) -> torch.Tensor:
@@ -324,6 +336,46 @@ def gateup_swiglu_split(split: torch.Tensor, scale: torch.Tensor, gate: Prepared
                                                           up.descriptor, _ptr(hidden), rows, _stream()),
                "dew_moe_gateup_swiglu_split")
     return hidden
+
+
+def block_scale_pitch(elements: int) -> int:
+    """Bytes of one row's block scales: one for 128 elements, padded to whole 16-byte loads."""
+    return (elements // 128 + 15) // 16 * 16
+
+
+def gateup_swiglu_split_out(split: torch.Tensor, scale: torch.Tensor, gate: PreparedBank, up: PreparedBank,
+                            offsets: torch.Tensor, *, gather: torch.Tensor | None = None,
+                            rows: int | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """`gateup_swiglu_split` whose hidden rows leave already split: (`hidden_split` uint8 `[rows, F * 2]`,
+    `hidden_scales` uint8 `[rows, block_scale_pitch(F)]`), one scale per row and 128 columns (byte b of a row scales its
+    columns 128 b .. 128 b + 127; the pad bytes are not written), for `grouped_gemm_split_blocks`."""
+    experts, depth, width = gate.shape
+    if split.dtype != torch.uint8 or split.shape[-1] != 2 * depth or scale.dtype != torch.uint8 or scale.numel() != split.shape[0]:
+        raise KernelError(f"split rows are uint8 [rows, {2 * depth}] with one uint8 scale a row")
+    rows = (gather.numel() if gather is not None else split.shape[0]) if rows is None else rows
+    hidden = torch.empty((rows, width * 2), dtype=torch.uint8, device=split.device)
+    scales = torch.empty((rows, block_scale_pitch(width)), dtype=torch.uint8, device=split.device)
+    _lib.check(_lib.library().dew_moe_gateup_swiglu_split_out(_ptr(split), _ptr(scale), _ptr(gather), _ptr(offsets), gate.descriptor,
+                                                              up.descriptor, _ptr(hidden), _ptr(scales), rows, _stream()),
+               "dew_moe_gateup_swiglu_split_out")
+    return hidden, scales
+
+
+def grouped_gemm_split_blocks(split: torch.Tensor, scales: torch.Tensor, bank: PreparedBank, offsets: torch.Tensor, *,
+                              gather: torch.Tensor | None = None, scatter: torch.Tensor | None = None, rows: int | None = None,
+                              bias: torch.Tensor | None = None) -> torch.Tensor:
+    """`grouped_gemm` on rows split with one scale per row and 128 depths (`gateup_swiglu_split_out`'s), MXFP4 bank."""
+    experts, depth, width = bank.shape
+    if split.dtype != torch.uint8 or split.shape[-1] != 2 * depth or scales.dtype != torch.uint8 or \
+            tuple(scales.shape) != (split.shape[0], block_scale_pitch(depth)) or not scales.is_contiguous():
+        raise KernelError(f"split rows are uint8 [rows, {2 * depth}] with uint8 scales [rows, {block_scale_pitch(depth)}]")
+    rows = (gather.numel() if gather is not None else split.shape[0]) if rows is None else rows
+    bias = _expert_bias(bias, experts, width)
+    out = torch.empty((rows, width), dtype=torch.bfloat16, device=split.device)
+    _lib.check(_lib.library().dew_moe_grouped_gemm_split_blocks(_ptr(split), _ptr(scales), _ptr(gather), _ptr(offsets),
+                                                                bank.descriptor, _ptr(bias), _ptr(scatter), _ptr(out), rows, _stream()),
+               "dew_moe_grouped_gemm_split_blocks")
+    return out
 
 
 # ---- measurement aids ---------------------------------------------------------------------------------

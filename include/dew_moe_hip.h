@@ -150,6 +150,19 @@ int dew_moe_grouped_gemm_split(const void* x_split, const uint8_t* x_scale, cons
 int dew_moe_gateup_swiglu_split(const void* x_split, const uint8_t* x_scale, const int32_t* gather,
                                 const int32_t* offsets, const dew_moe_bank* gate, const dew_moe_bank* up,
                                 void* hidden, int32_t rows, void* stream);
+/* The pair that keeps the whole expert MLP on the scaled instruction without a split pass between its products:
+ * the gate/up launch writes its SwiGLU rows already split, two e4m3 terms under one scale per row and 128 columns
+ * (hidden_split [rows, F * 2] bytes in dew_moe_split_rows' order; hidden_scales [rows, P] e8m0 bytes, byte b of a
+ * row the scale of its columns 128 b .. 128 b + 127, with P = F / 128 rounded up to a multiple of 16 and the base
+ * 16-byte aligned; the values are the bf16 hidden rows of dew_moe_gateup_swiglu, exactly, within 2^-11 of each
+ * block's largest magnitude), and the down launch reads rows split that way (x_scales [source rows, P of K]; K up to
+ * 24576: a tile keeps its rows' scales in the LDS).                                                              */
+int dew_moe_gateup_swiglu_split_out(const void* x_split, const uint8_t* x_scale, const int32_t* gather,
+                                    const int32_t* offsets, const dew_moe_bank* gate, const dew_moe_bank* up,
+                                    void* hidden_split, uint8_t* hidden_scales, int32_t rows, void* stream);
+int dew_moe_grouped_gemm_split_blocks(const void* x_split, const uint8_t* x_scales, const int32_t* gather,
+                                      const int32_t* offsets, const dew_moe_bank* w, const float* bias,
+                                      const int32_t* scatter, void* out, int32_t rows, void* stream);
 
 /* gate and up in one launch with the SwiGLU epilogue: hidden[i] = swiglu(x[gather[i]] @ Wg[e], .. @ Wu[e])
  * with the reference's rounding sequence (src/dew/nn/activations.py:267-278): both products rounded to

@@ -52,8 +52,8 @@ def test_full_size_configuration(name):
 
     # the busiest expert's first rows through all three projections against the oracle, and the combine from the slots
     _, (sampled_slots, want_down) = bench.cpu_baseline(case, data, out, plan, budget_rows=48)
-    hidden = ops.gateup_swiglu(data["x"], stepper.gate, stepper.up, plan.offsets, gather=plan.rows)
-    slots = ops.grouped_gemm(hidden, stepper.down, plan.offsets, scatter=plan.order)
+    slots = stepper.project(plan)                                   # c2: on split rows, the library's rule for its groups
+    assert stepper.on_split_rows() == (name == "c2")
     got_down = slots[torch.from_numpy(sampled_slots).to(device).long()].float().cpu().numpy()
     peak, elementwise = oracle.relative_errors(got_down, want_down)
     assert peak <= 2e-2 and elementwise <= 2e-2, (peak, elementwise)

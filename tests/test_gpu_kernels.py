@@ -343,3 +343,43 @@ def test_split_activations_give_the_bf16_products_on_mxfp4_banks(ops, depth):
     assert (got_gate == want_gate).mean() > 0.97 and (got_gate == plain_gate).mean() > 0.97
     fused = bf16_np(ops.gateup_swiglu_split(split, scale, pg, pu, od, gather=gd))
     assert np.abs(fused - want).max() <= 2 ** -6 * np.abs(want).max() and (fused == want).mean() > 0.9
+
+
+@pytest.mark.parametrize("depth,width", [(256, 512), (768, 2304)])     # 4 and 18 blocks of scales a row: one and two 16-byte pieces
+def test_the_expert_mlp_stays_on_split_rows_without_a_pass_between_its_products(ops, depth, width):
+    """gate/up writes its SwiGLU rows already split (one scale per row and 128 columns), down reads them: the hidden
+    rows are the bf16 ones exactly, and the output agrees with the bf16 kernels and the oracle."""
+    sizes = [700, 0, 290, 5]
+    gate, x, offsets = grouped_case("mxfp4", len(sizes), depth, width, sizes, seed=depth + 11)
+    up, _, _ = grouped_case("mxfp4", len(sizes), depth, width, sizes, seed=depth + 12)
+    down, _, _ = grouped_case("mxfp4", len(sizes), width, 256, sizes, seed=depth + 13)
+    rng = np.random.default_rng(depth)
+    padded = x.shape[0] + 9                                            # unrouted sorted positions past the last group
+    gather = np.concatenate([rng.integers(0, x.shape[0], size=x.shape[0]), np.zeros(9)]).astype(np.int32)
+    xd, od, gd = x.cuda(), torch.from_numpy(offsets).cuda(), torch.from_numpy(gather).cuda()
+    pg, pu, pd = (ops.prepare(bank.to("cuda")) for bank in (gate, up, down))
+    hidden = ops.gateup_swiglu(xd, pg, pu, od, gather=gd, rows=padded)
+    hidden_split, hidden_scales = ops.gateup_swiglu_split_out(*ops.split_rows(xd), pg, pu, od, gather=gd, rows=padded)
+    # the split rows rebuilt on the host are the bf16 hidden rows
+    rows = padded
+    pieces = hidden_split.cpu().numpy().reshape(rows, width // 64, 2, 2, 2, 16)
+    terms = oracle._e4m3_table()[pieces].astype(np.float64)
+    values = (terms[:, :, :, 0] + terms[:, :, :, 1] / 16).transpose(0, 1, 3, 2, 4).reshape(rows, width // 128, 128)
+    assert tuple(hidden_scales.shape) == (rows, ops.block_scale_pitch(width))
+    s = np.ldexp(np.float64(1), hidden_scales.cpu().numpy()[:, :width // 128].astype(np.int64) - 127)[:, :, None]
+    rebuilt = (values * s).reshape(rows, width)
+    want_hidden = bf16_np(hidden).astype(np.float64)
+    largest = np.abs(want_hidden.reshape(rows, width // 128, 128)).max(axis=2, keepdims=True)
+    near = (np.abs(want_hidden.reshape(rows, width // 128, 128)) >= largest * 2.0 ** -11).reshape(rows, width)
+    split_hidden_matches = (rebuilt == want_hidden)
+    assert (split_hidden_matches | ~near).mean() > 0.97          # up to fp32 summation order in the two kernels' products
+    assert np.abs(rebuilt - want_hidden).max() <= 2 ** -6 * np.abs(want_hidden).max()
+    assert np.all(rebuilt[x.shape[0]:] == 0)
+    out = bf16_np(ops.grouped_gemm_split_blocks(hidden_split, hidden_scales, pd, od, rows=padded))
+    plain = bf16_np(ops.grouped_gemm(hidden, pd, od, rows=padded))
+    down_values, down_factor = dequantized(down)
+    want = oracle.grouped_matmul(bf16_np(hidden)[:x.shape[0]], down_values, sizes, factor=down_factor)
+    assert np.all(out[x.shape[0]:] == 0)
+    scale = np.abs(want).max()
+    assert np.abs(out[:x.shape[0]] - want).max() <= 2 ** -5 * scale and np.abs(out - plain).max() <= 2 ** -5 * scale
+    assert (out == plain).mean() > 0.9

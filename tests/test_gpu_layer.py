@@ -82,6 +82,32 @@ def test_layer_matches_the_oracle(name):
     assert np.array_equal(unfused, got)
 
 
+def test_large_groups_on_mxfp4_banks_run_on_split_rows_and_agree_with_the_bf16_launches(monkeypatch):
+    """Groups of a thousand rows on MXFP4 banks take the two launches on the scaled matrix instruction (rows as two
+    e4m3 terms); the layer's output is within the bar of the oracle either way and nearly all of it is identical."""
+    from dew_amd import gemm, ops
+
+    case = CONFIGS["c2"].scaled(tokens=4608, d_model=512, d_ff=768)       # 9216 routed rows over 8 experts
+    data = inputs(case, seed=3)
+    layer, variables = layer_and_variables(case, data)
+    x, logits = data["x"].cuda(), data["logits"].cuda()
+    calls = []
+    split_out = ops.gateup_swiglu_split_out
+    monkeypatch.setattr(ops, "gateup_swiglu_split_out", lambda *a, **k: calls.append(1) or split_out(*a, **k))
+    assert gemm.SPLIT_ROWS
+    got = layer.apply(variables, x, logits=logits).float().cpu().numpy()
+    assert calls == [1]
+    monkeypatch.setattr(gemm, "SPLIT_ROWS", False)
+    plain = layer.apply(variables, x, logits=logits).float().cpu().numpy()
+    assert calls == [1]
+    want, _ = oracle_output(case, data)
+    for name, value in (("split rows", got), ("bf16 operands", plain)):
+        by_max, by_element = oracle.relative_errors(value, want)
+        print(f"\n{name}: max|d|/max|ref| = {by_max:.3e}, element-wise max rel = {by_element:.3e}, identical = {(value == want).mean():.4f}")
+        assert by_max <= TOLERANCE and by_element <= TOLERANCE
+    assert (got == plain).mean() > 0.9 and np.abs(got - plain).max() <= 2.0 ** -6 * np.abs(plain).max()
+
+
 def test_layer_multiplies_its_own_gate_kernel_when_no_logits_are_given():
     from dew_amd import moe
 
