@@ -42,6 +42,11 @@ typedef __attribute__((ext_vector_type(8))) int i32x8_t;       // an operand of 
 // as they are stored, so the weights are not dequantized at all.
 constexpr int kFormatMxSplit = 5;
 constexpr int kFormatMxSplitBlocks = 6;  // the same with one activation scale per row and 128 depths, not per row
+// Kernel-side format of an FP8 128 x 128 block bank whose scales are powers of two, multiplied by rows quantized to
+// e4m3 a 1 x 128 tile at a time under power-of-two scales (dew_moe_quantize_rows_fp8): the blockwise FP8 recipe's
+// product. The same instruction takes both operands' codes and scales as stored; a step is 128 depths, its two
+// 64-deep halves taking the places of the split rows' two terms.
+constexpr int kFormatFp8Rows = 7;
 
 constexpr int BK = 64;
 constexpr int kThreads = 256;
@@ -158,13 +163,16 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   constexpr bool kGated = MODE == kInterleavedGated;
   constexpr int kOutBN = kGated ? BN / 2 : BN;  // output columns of the tile
   static_assert(WM * WN == 4 && BM % (32 * WM) == 0 && BN % (32 * WN) == 0 && BM % 32 == 0, "tile shape");
-  constexpr bool kSplit = FORMAT == kFormatMxSplit || FORMAT == kFormatMxSplitBlocks;
-  constexpr bool kBlockScales = FORMAT == kFormatMxSplitBlocks;
-  constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4 || kSplit;
-  constexpr bool kPow2 = FORMAT == DEW_MOE_W_MXFP4 || kSplit;
+  constexpr bool kFp8Rows = FORMAT == kFormatFp8Rows;
+  constexpr bool kSplit = FORMAT == kFormatMxSplit || FORMAT == kFormatMxSplitBlocks || kFp8Rows;  // A arrives as 8-bit codes
+  constexpr bool kBlockScales = FORMAT == kFormatMxSplitBlocks || kFp8Rows;
+  constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4 || (kSplit && !kFp8Rows);
+  constexpr bool kPow2 = FORMAT == DEW_MOE_W_MXFP4 || (kSplit && !kFp8Rows);
+  constexpr bool kBlockBank = FORMAT == DEW_MOE_W_FP8_BLOCK || kFp8Rows;  // one fp32 scale per 128 x 128 weights
   constexpr int kMatrices = PAIRED ? 2 : 1;
   constexpr int kAtomK = kFp4 ? 64 : 32;       // depth an atom covers
-  constexpr int kAtoms = BK / kAtomK;          // 16-byte loads a lane makes per 32-column tile per step
+  constexpr int kStepDepth = kFp8Rows ? 128 : BK;  // depth a step covers: always 128 bytes of an A row
+  constexpr int kAtoms = kStepDepth / kAtomK;  // 16-byte loads a lane makes per 32-column tile per step
   constexpr int kRowLoads = BM / 32;           // A rows a lane loads per step
   constexpr int TI = BM / (32 * WM), TJ = BN / (32 * WN);  // MFMA tiles per wavefront: rows, columns of each matrix
   constexpr int kTiles = kMatrices * TJ;       // weight tiles a wavefront multiplies
@@ -180,8 +188,8 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   __shared__ int wave_tiles[4];
   __shared__ int found[3];  // expert, first sorted row of the tile, total m-tiles
   // FP8 128 x 128 blocks: the scales of the block's column blocks down the whole depth, read once
-  constexpr int kScaleColumns = FORMAT == DEW_MOE_W_FP8_BLOCK ? kMatrices * (BN / 128) : 1;
-  __shared__ float depth_scales[kScaleColumns][FORMAT == DEW_MOE_W_FP8_BLOCK ? kMaxDepthBlocks : 1];
+  constexpr int kScaleColumns = kBlockBank ? kMatrices * (BN / 128) : 1;
+  __shared__ float depth_scales[kScaleColumns][kBlockBank ? kMaxDepthBlocks : 1];
 
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
 
@@ -252,7 +260,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
 
   const int row0 = found[1];
   const int valid_rows = min(BM, p.offsets[expert + 1] - row0);
-  const int steps = p.depth / BK;
+  const int steps = p.depth / kStepDepth;
   const int wm0 = (wave / WN) * (BM / WM), wn0 = (wave % WN) * (BN / WN);
 
   // ---- A loader. One global_load_lds_dwordx4 of a wavefront fills 1 KiB of LDS, lane l landing at byte 16 l:
@@ -265,7 +273,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     const int chunk = (lane % 8) ^ (((row >> 1) & 7) ^ ((row & 1) << 2));
     const int sorted = row0 + min(row, valid_rows - 1);
     const int source = p.gather ? p.gather[sorted] : sorted;
-    a_src[i] = p.x + static_cast<size_t>(source) * p.depth + chunk * 8;
+    a_src[i] = p.x + static_cast<size_t>(source) * (kFp8Rows ? p.depth / 2 : p.depth) + chunk * 8;  // a row of e4m3 codes is depth bytes
   }
   // Split activations: the lane's row of each row tile carries one e8m0 scale; the hi term multiplies under it
   // (byte 0) and the lo term under 2^-4 of it (byte 1).
@@ -308,7 +316,8 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   auto form_block_words = [&](auto buffer) __attribute__((always_inline)) {
     if constexpr (kBlockScales) {
 #pragma unroll
-      for (int i = 0; i < TI; ++i) a_block_word[buffer.value][i] = a_block_byte[i] | ((a_block_byte[i] - 4) << 8);
+      for (int i = 0; i < TI; ++i)  // quantized rows have the one term: the byte is the word
+        a_block_word[buffer.value][i] = kFp8Rows ? a_block_byte[i] : a_block_byte[i] | ((a_block_byte[i] - 4) << 8);
     }
   };
   auto load_a = [&](u32x4_t* stage, int step, auto begin, auto end) __attribute__((always_inline)) {
@@ -340,7 +349,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
       channel_scale[t] = static_cast<const float*>(scales)[static_cast<size_t>(expert) * p.width + column + lane % 32];
     }
   }
-  if constexpr (FORMAT == DEW_MOE_W_FP8_BLOCK) {
+  if constexpr (kBlockBank) {
     const int depth_blocks = p.depth / 128, width_blocks = p.width / 128;
     for (int item = tid; item < kScaleColumns * depth_blocks; item += kThreads) {
       const int which = item / depth_blocks, block = item % depth_blocks;
@@ -428,21 +437,39 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
 
   // Split activations: one scaled instruction multiplies 64 depths of one term by the stored FP4 codes under
   // both operands' power-of-two scales; the block scale byte is the e4m3 of a normal power of two, 2^(field - 7).
-  auto multiply_term = [&](auto set, auto term) __attribute__((always_inline)) {
+  int unscalable = 0;  // quantized rows: mantissa bits met in a weight block scale (the instruction takes powers of two only)
+  auto multiply_term = [&](auto set, auto term, int step) __attribute__((always_inline)) {
     if constexpr (kSplit) {
-      constexpr int kBuffer = (set.value / 2) % 2;  // block scales: steps 0, 1 of the unrolled four read set 0, steps 2, 3 set 1
+      // block scales: of the unrolled four steps, steps 0, 1 read set 0 and steps 2, 3 set 1 (a scale holds for two
+      // 64-deep steps); quantized rows' 128-deep steps alternate
+      constexpr int kBuffer = kFp8Rows ? set.value % 2 : (set.value / 2) % 2;
 #pragma unroll
       for (int m = 0; m < kMatrices; ++m)
 #pragma unroll
         for (int j = 0; j < TJ; ++j) {
-          const u32x4_t& raw = b_regs[set.value][m * TJ + j][0];
-          const i32x8_t codes = {static_cast<int>(raw[0]), static_cast<int>(raw[1]), static_cast<int>(raw[2]), static_cast<int>(raw[3]), 0, 0, 0, 0};
-          const int b_scale = static_cast<int>(((s_regs[set.value][m * TJ + j] >> 3) & 15u) + 120u);
+          if constexpr (kFp8Rows) {
+            // both operands e4m3: the half's 64 depths are two 32-deep atoms of the bank, in the operand's own order
+            const u32x4_t& first = b_regs[set.value][m * TJ + j][2 * term.value];
+            const u32x4_t& second = b_regs[set.value][m * TJ + j][2 * term.value + 1];
+            const i32x8_t codes = {static_cast<int>(first[0]), static_cast<int>(first[1]), static_cast<int>(first[2]), static_cast<int>(first[3]),
+                                   static_cast<int>(second[0]), static_cast<int>(second[1]), static_cast<int>(second[2]), static_cast<int>(second[3])};
+            const uint32_t bits = __float_as_uint(depth_scales[m * (BN / 128) + (wn0 + 32 * j) / 128][step]);
+            unscalable |= (bits & 0x807FFFFFu) | ((bits >> 23) == 0u) | ((bits >> 23) == 255u);
+            const int b_scale = static_cast<int>(bits >> 23);
 #pragma unroll
-          for (int i = 0; i < TI; ++i) {
-            acc[m][i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_term[term.value][i], codes, acc[m][i][j], 0, 4, term.value,
-                                                                        kBlockScales ? a_block_word[kBuffer][i] : a_scale_word[i], 0,
-                                                                        b_scale);
+            for (int i = 0; i < TI; ++i)
+              acc[m][i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_term[term.value][i], codes, acc[m][i][j], 0, 0, 0,
+                                                                          a_block_word[kBuffer][i], 0, b_scale);
+          } else {
+            const u32x4_t& raw = b_regs[set.value][m * TJ + j][0];
+            const i32x8_t codes = {static_cast<int>(raw[0]), static_cast<int>(raw[1]), static_cast<int>(raw[2]), static_cast<int>(raw[3]), 0, 0, 0, 0};
+            const int b_scale = static_cast<int>(((s_regs[set.value][m * TJ + j] >> 3) & 15u) + 120u);
+#pragma unroll
+            for (int i = 0; i < TI; ++i) {
+              acc[m][i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_term[term.value][i], codes, acc[m][i][j], 0, 4, term.value,
+                                                                          kBlockScales ? a_block_word[kBuffer][i] : a_scale_word[i], 0,
+                                                                          b_scale);
+            }
           }
         }
     }
@@ -505,7 +532,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
       // younger than the last A load of the step before: only this phase's loads are sure to be
       constexpr int kSplitWait = (kSplitLoads & 0xF) | (7 << 4) | (0 << 8) | ((kSplitLoads >> 4) << 14);
       fetch_term(current, c1);
-      multiply_term(set, c0);
+      multiply_term(set, c0, step);
       load_a(fill, ahead_a, c0, ah);
       load_b(filling, ahead_b, c0, bh);
       schedule_phase<0, kSplitMfmas, 2 * TI, 0, 2 * kTiles + 2 * kSplitLoads, kSplitLoads>();
@@ -517,10 +544,15 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
       __builtin_amdgcn_sched_barrier(0);
       // block scales: the bytes of the next 128 depths are read from the LDS in the second phase of an even step
       // and formed into words in the second phase of the odd step that follows, one phase before they multiply
-      if constexpr (kBlockScales && set.value % 2 == 0) load_block_scales(min(step / 2 + 1, p.depth / 128 - 1));
-      if constexpr (kBlockScales && set.value % 2 == 1) form_block_words(std::integral_constant<int, 1 - (set.value / 2) % 2>{});
+      if constexpr (kFp8Rows) {  // a step is the 128 depths of one scale: the next step's, into the other set
+        load_block_scales(min(step + 1, steps - 1));
+        form_block_words(std::integral_constant<int, 1 - set.value % 2>{});
+      } else {
+        if constexpr (kBlockScales && set.value % 2 == 0) load_block_scales(min(step / 2 + 1, p.depth / 128 - 1));
+        if constexpr (kBlockScales && set.value % 2 == 1) form_block_words(std::integral_constant<int, 1 - (set.value / 2) % 2>{});
+      }
       fetch_term(next, c0);
-      multiply_term(set, c1);
+      multiply_term(set, c1, step);
       load_a(fill, ahead_a, ah, a4);
       load_b(filling, ahead_b, bh, b4);
       schedule_phase<0, kSplitMfmas, 2 * TI, 0, 2 * kTiles + 2 * kSplitLoads, kSplitLoads>();
@@ -606,6 +638,9 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   // the tile leaves as full cache lines (direct 4-byte stores of 64-byte row pieces took a quarter of the
   // kernel's time). Tiles of 256 columns are staged in two passes of BM / 2 rows.
   float factor0 = 1.0f, factor1 = 1.0f;
+  // quantized rows: a weight block scale that is no normal power of two cannot enter the instruction; the tile is
+  // then written as NaN rather than as the product under another scale
+  if (kFp8Rows && unscalable != 0) factor0 = factor1 = __uint_as_float(0x7FC00000u);
   if (kFp4) {  // the 2^8 the decode owes times the expert's tensor scale (src/dew/nn/kernels/gemm.py:660-662)
     // (the scaled instruction applies the block scales themselves, not their 2^-8)
     factor0 = (kSplit ? 1.0f : 256.0f) * p.w0.tensor_scale[expert];
@@ -749,7 +784,7 @@ template <int FORMAT, int MODE, int BM, int BN, int WM, int WN>
 static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
   // block-scaled activations keep their tile's scales behind the ring (reserved at their largest: kMaxBlockScaleDepth)
   constexpr size_t kShared = shared_bytes<BM, BN, MODE>() +
-                             (FORMAT == kFormatMxSplitBlocks ? static_cast<size_t>(BM) * block_scale_pitch(kMaxBlockScaleDepth) : 0);
+                             (FORMAT == kFormatMxSplitBlocks || FORMAT == kFormatFp8Rows ? static_cast<size_t>(BM) * block_scale_pitch(kMaxBlockScaleDepth) : 0);
   auto kernel = grouped_gemm_kernel<FORMAT, MODE, BM, BN, WM, WN>;
   static bool configured = false;  // dynamic LDS above 64 KiB must be opted into once per kernel
   if (!configured) {
@@ -939,6 +974,25 @@ extern "C" int dew_moe_grouped_gemm_split_blocks(const void* x_split, const uint
   if (int rc = fill_single(who, p, x_split, gather, offsets, w, bias, scatter, out, rows)) return rc;
   p.a_scale = x_scales;
   return launch_tile<kFormatMxSplitBlocks, kPlain, 256, 256, 2, 2>(who, p, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int dew_moe_grouped_gemm_fp8_rows(const void* x_codes, const uint8_t* x_scales, const int32_t* gather,
+                                             const int32_t* offsets, const dew_moe_bank* w, const float* bias,
+                                             const int32_t* scatter, void* out, int32_t rows, void* stream) {
+  using namespace dew;
+  const char* who = "dew_moe_grouped_gemm_fp8_rows";
+  if (int rc = check_bank(who, w, "weight")) return rc;
+  DEW_REQUIRE(w->format == DEW_MOE_W_FP8_BLOCK, "%s: quantized rows multiply an FP8 128 x 128 block bank; this one is format %d", who,
+              w->format);
+  DEW_REQUIRE(w->depth <= kMaxBlockScaleDepth, "%s: bank depth %d is above %d (a tile's block scales are kept in the LDS)", who,
+              w->depth, kMaxBlockScaleDepth);
+  DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
+  if (rows == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(x_scales && aligned16(x_scales), "%s: the rows' scales must not be null and must be 16-byte aligned", who);
+  GemmParams p{};
+  if (int rc = fill_single(who, p, x_codes, gather, offsets, w, bias, scatter, out, rows)) return rc;
+  p.a_scale = x_scales;
+  return launch_tile<kFormatFp8Rows, kPlain, 256, 128, 2, 2>(who, p, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int dew_moe_gateup_swiglu_split_out(const void* x_split, const uint8_t* x_scale, const int32_t* gather,

@@ -378,6 +378,53 @@ def grouped_gemm_split_blocks(split: torch.Tensor, scales: torch.Tensor, bank: P
     return out
 
 
+def quantize_rows_fp8(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """bf16 rows `[rows, K]` as the blockwise FP8 recipe quantizes them (1 x 128 tiles, power-of-two scales):
+    (`codes` uint8 `[rows, K]`, each 128 depths in the scaled matrix instruction's operand order; `scales` uint8
+    `[rows, block_scale_pitch(K)]`, the scales' e8m0 bytes)."""
+    _device(x, "x", torch.bfloat16)
+    rows, depth = x.shape
+    codes = torch.empty((rows, depth), dtype=torch.uint8, device=x.device)
+    scales = torch.empty((rows, block_scale_pitch(depth)), dtype=torch.uint8, device=x.device)
+    _lib.check(_lib.library().dew_moe_quantize_rows_fp8(_ptr(x), _ptr(codes), _ptr(scales), rows, depth, _stream()),
+               "dew_moe_quantize_rows_fp8")
+    return codes, scales
+
+
+def operand_order_fp8(codes: torch.Tensor) -> torch.Tensor:
+    """e4m3 codes `[rows, K]` in depth order -> the order `quantize_rows_fp8` writes and `grouped_gemm_fp8_rows`
+    reads: of each 128 depths, byte 16 (4 g + 2 t + h) + b holds depth 64 t + 32 h + 16 g + b."""
+    rows, depth = codes.shape
+    return codes.view(rows, depth // 128, 2, 2, 2, 16).permute(0, 1, 4, 2, 3, 5).contiguous().view(rows, depth)
+
+
+def depth_order_fp8(codes: torch.Tensor) -> torch.Tensor:
+    """The inverse of `operand_order_fp8`."""
+    rows, depth = codes.shape
+    return codes.view(rows, depth // 128, 2, 2, 2, 16).permute(0, 1, 3, 4, 2, 5).contiguous().view(rows, depth)
+
+
+def grouped_gemm_fp8_rows(codes: torch.Tensor, scales: torch.Tensor, bank: PreparedBank, offsets: torch.Tensor, *,
+                          gather: torch.Tensor | None = None, scatter: torch.Tensor | None = None, rows: int | None = None,
+                          bias: torch.Tensor | None = None) -> torch.Tensor:
+    """The blockwise FP8 recipe's product: `quantize_rows_fp8`'s rows times an FP8 128 x 128 block bank whose scales
+    are powers of two, each 128-deep block's exact partial under its row's and its block's scale, fp32 sums, one
+    rounding to bf16 `[rows, N]`."""
+    experts, depth, width = bank.shape
+    if codes.dtype != torch.uint8 or codes.shape[-1] != depth or scales.dtype != torch.uint8 or \
+            tuple(scales.shape) != (codes.shape[0], block_scale_pitch(depth)) or not scales.is_contiguous():
+        raise KernelError(f"quantized rows are uint8 [rows, {depth}] with uint8 scales [rows, {block_scale_pitch(depth)}]")
+    if bank.descriptor.format != _lib.W_FP8_BLOCK:
+        raise KernelError("quantized rows multiply an FP8 128 x 128 block bank")
+    rows = (gather.numel() if gather is not None else codes.shape[0]) if rows is None else rows
+    bias = _expert_bias(bias, experts, width)
+    out = torch.empty((rows, width), dtype=torch.bfloat16, device=codes.device)
+    _lib.check(_lib.library().dew_moe_grouped_gemm_fp8_rows(_ptr(codes), _ptr(scales), _ptr(gather), _ptr(offsets), bank.descriptor,
+                                                            _ptr(bias), _ptr(scatter), _ptr(out), rows, _stream()),
+               "dew_moe_grouped_gemm_fp8_rows")
+    return out
+
+
 # ---- measurement aids ---------------------------------------------------------------------------------
 
 

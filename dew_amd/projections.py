@@ -1,0 +1,118 @@
+"""The blockwise FP8 recipe's projection, forward only, shaped as the reference's
+(`src/dew/nn/kernels/projections.py:50-60,96-204`: `blockwise_fp8_projection`, `recipe_projection`,
+`rows_quantized`, `blocks_quantized`; product `gemm.blockwise_fp8_product` `src/dew/nn/kernels/gemm.py:764-793`).
+
+DeepSeek-V3's recipe: activations quantized to E4M3 a 1 x 128 tile at a time along the depth, weights a
+128 x 128 block at a time, both under power-of-two scales; each 128-deep block's partial, exact, times its
+row's and its block's scale, summed in fp32, rounded once. On gfx950 both operands enter
+`v_mfma_scale_f32_32x32x64_f8f6f4` as stored, codes and scales: the rows' quantizer is one HBM-bound launch
+(`ops.quantize_rows_fp8`) and the product one grouped launch (`ops.grouped_gemm_fp8_rows`). A group's rows need
+no padding to whole 128-row blocks here (the launch finds its tiles from the group offsets), so
+`recipe_projection` takes ragged groups as they are; the zero rows the reference pads with add nothing there.
+The recipe's gradients (its own FP8 products of requantized operands) are not part of this package.
+"""
+
+import dataclasses
+
+import torch
+
+from . import formats, gemm, ops
+
+SCALE_DEPTH = 128
+"""The recipe's block: activations 1 x 128, weights 128 x 128 (`templates.product.SCALE_DEPTH`)."""
+
+_E4M3_MAX = 448.0
+_AMAX_FLOOR = 1e-4
+
+
+def _power_of_two_ceil(value: torch.Tensor) -> torch.Tensor:
+    """The least power of two >= `value`, off its fp32 bits (src/dew/nn/fake_quant.py:48-57)."""
+    bits = value.contiguous().view(torch.int32)
+    field = ((bits >> 23) & 0xFF) + ((bits & 0x7FFFFF) != 0).to(torch.int32)
+    return (field << 23).view(torch.float32)
+
+
+def blocks_quantized(w: torch.Tensor) -> formats.Fp8Blocks:
+    """`w [groups, depth, width]` as E4M3 codes a 128 x 128 block at a time, each block's scale the least power
+    of two >= max(amax, 1e-4) * f32(1 / 448) (src/dew/nn/kernels/projections.py:185-196 over
+    src/dew/nn/fake_quant.py:117-128): the bank the recipe's product multiplies, made once where the weights are
+    held fixed."""
+    values = w.to(torch.float32)
+    groups, depth, width = values.shape
+    if depth % SCALE_DEPTH or width % SCALE_DEPTH:
+        raise ValueError(f"a {depth} x {width} matrix holds no whole {SCALE_DEPTH}-wide blocks")
+    edge = SCALE_DEPTH
+    tiles = values.reshape(groups, depth // edge, edge, width // edge, edge)
+    amax = tiles.abs().amax(dim=(2, 4)).clamp_min(torch.tensor(_AMAX_FLOOR, dtype=torch.float32, device=values.device))
+    scale = _power_of_two_ceil(amax * torch.tensor(1 / _E4M3_MAX, dtype=torch.float32, device=values.device))
+    quotient = (tiles / scale[:, :, None, :, None]).clamp(-_E4M3_MAX, _E4M3_MAX)
+    codes = quotient.to(torch.float8_e4m3fn).view(torch.uint8).reshape(groups, depth, width).contiguous()
+    return formats.Fp8Blocks(codes, scale.contiguous())
+
+
+@dataclasses.dataclass(frozen=True)
+class QuantizedRows:
+    """Rows as `ops.quantize_rows_fp8` writes them: `codes [rows, K]` uint8, each 128 depths in the scaled matrix
+    instruction's operand order, and `scales [rows, P]` their tiles' e8m0 bytes."""
+
+    codes: torch.Tensor
+    scales: torch.Tensor
+
+    def values(self) -> tuple[torch.Tensor, torch.Tensor]:
+        """(codes in depth order `[rows, K]` uint8, scales fp32 `[rows, K / 128]`): the reference's `rows_quantized`."""
+        blocks = self.codes.shape[1] // SCALE_DEPTH
+        scales = (self.scales[:, :blocks].to(torch.int32) << 23).view(torch.float32)
+        return ops.depth_order_fp8(self.codes), scales
+
+
+def rows_quantized(x: torch.Tensor) -> QuantizedRows:
+    """`x [rows, K]` bf16 as E4M3 codes a 1 x 128 tile at a time along the depth and each tile's power-of-two scale
+    (src/dew/nn/kernels/projections.py:176-182), on the device."""
+    return QuantizedRows(*ops.quantize_rows_fp8(x.contiguous()))
+
+
+def _offsets(group_sizes, rows: int, device) -> torch.Tensor:
+    if group_sizes is None:
+        return torch.tensor([0, rows], dtype=torch.int32, device=device)
+    return gemm.GroupSizes.of(group_sizes).offsets
+
+
+def blockwise_fp8_product(lhs: QuantizedRows, kernel, group_sizes, *, out_dtype=torch.bfloat16, bias=None,
+                          gather=None, scatter=None) -> torch.Tensor:
+    """Each group's quantized rows times its matrix of the FP8 block bank `kernel` (`formats.Fp8Blocks` with
+    power-of-two scales, or its prepared form), each 128-deep block's exact partial under its rows' and its block's
+    scales, fp32 sums (+ `bias [groups, width]`), one rounding (src/dew/nn/kernels/gemm.py:764-793). Scales that
+    are not powers of two have no place in the instruction: the launch writes NaN where it meets one."""
+    if out_dtype != torch.bfloat16:
+        raise ValueError(f"the launch writes bfloat16, not {out_dtype}")
+    bank = gemm.prepared(kernel)
+    rows = lhs.codes.shape[0] if gather is None else gather.numel()
+    return ops.grouped_gemm_fp8_rows(lhs.codes, lhs.scales, bank, _offsets(group_sizes, rows, lhs.codes.device),
+                                     gather=gather, scatter=scatter, bias=bias)
+
+
+def blockwise_fp8_projection(x: torch.Tensor, w, group_blocks, *, out_dtype=torch.bfloat16) -> torch.Tensor:
+    """Each group's rows of `x [rows, depth]` times its matrix of `w [groups, depth, width]` in the blockwise FP8
+    recipe; group `g` holds `group_blocks[g]` whole 128-row blocks, in order (src/dew/nn/kernels/projections.py:
+    50-60). `w` is the weights (quantized here, `blocks_quantized`) or a bank already quantized."""
+    bank = w if isinstance(w, (formats.Fp8Blocks, ops.PreparedBank)) else blocks_quantized(w)
+    sizes = (torch.as_tensor(group_blocks, device=x.device).to(torch.int32) * SCALE_DEPTH).contiguous()
+    return blockwise_fp8_product(rows_quantized(x), bank, sizes, out_dtype=out_dtype)
+
+
+def recipe_projection(rows: torch.Tensor, matrix, group_sizes=None, *, out_dtype=torch.bfloat16, bias=None):
+    """`rows @ matrix` in the blockwise FP8 recipe: a dense projection's (`matrix [in, out]`, every row its one
+    group's) or experts' (`[groups, in, out]`, `group_sizes` counting each group's leading rows, any past their sum
+    zero), `bias [groups, out]` added to the fp32 sums before the one rounding
+    (src/dew/nn/kernels/projections.py:96-140). None where the widths hold no whole 128-wide blocks
+    (`recipe_refusal`'s 'block_shape', :62-83): the caller then keeps the projection in the run's dtypes."""
+    if isinstance(matrix, (formats.Fp8Blocks, ops.PreparedBank)):
+        bank = matrix
+    else:
+        stacked = matrix if matrix.dim() == 3 else matrix[None]
+        if stacked.shape[1] % SCALE_DEPTH or stacked.shape[2] % SCALE_DEPTH:
+            return None
+        bank = blocks_quantized(stacked)
+    if bias is not None:
+        bias = bias.reshape(bank.shape[0], bank.shape[2]).to(torch.float32).contiguous()  # widened as it is stored (:141)
+    return blockwise_fp8_product(rows_quantized(rows), bank, group_sizes, out_dtype=out_dtype, bias=bias)

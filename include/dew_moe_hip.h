@@ -164,6 +164,23 @@ int dew_moe_grouped_gemm_split_blocks(const void* x_split, const uint8_t* x_scal
                                       const int32_t* offsets, const dew_moe_bank* w, const float* bias,
                                       const int32_t* scatter, void* out, int32_t rows, void* stream);
 
+/* The blockwise FP8 recipe's forward product (DeepSeek-V3's 1 x 128 activation tiles, 128 x 128 weight blocks):
+ * `rows_quantized` src/dew/nn/kernels/projections.py:176-182 and `blockwise_fp8_product`
+ * src/dew/nn/kernels/gemm.py:764-793 (its portable sum: `step_scaled` src/dew/nn/kernels/xla_products.py:147-173).
+ * dew_moe_quantize_rows_fp8: x bf16 [rows, K] -> e4m3 codes a 1 x 128 tile at a time, amax floored at 1e-4, scale the
+ * least power of two >= amax * f32(1 / 448) (src/dew/nn/fake_quant.py:117-128). codes [rows, K] bytes hold each 128
+ * depths in the scaled matrix instruction's operand order: byte 16 (4 g + 2 t + h) + b is depth 64 t + 32 h + 16 g + b;
+ * scales [rows, P] are the scales' e8m0 bytes (value 2^(byte - 127)), P = K / 128 rounded up to a multiple of 16.
+ * dew_moe_grouped_gemm_fp8_rows: out[scatter[i]] = bf16( sum over 128-deep blocks of (codes x codes, exact) x row
+ * scale x weight block scale (+ bias) ) for an FP8 128 x 128 block bank (prepared) whose scales are powers of two, as
+ * the recipe's `blocks_quantized` makes them: both operands enter v_mfma_scale_f32_32x32x64_f8f6f4 as stored. A weight
+ * block scale that is no normal power of two makes the tiles that meet it NaN. K up to 24576, rows in 256-row tiles. */
+int dew_moe_quantize_rows_fp8(const void* x /* bf16 [rows, K] */, void* codes /* [rows, K] bytes */,
+                              uint8_t* scales /* [rows, P] e8m0 */, int32_t rows, int32_t depth, void* stream);
+int dew_moe_grouped_gemm_fp8_rows(const void* x_codes, const uint8_t* x_scales, const int32_t* gather,
+                                  const int32_t* offsets, const dew_moe_bank* w, const float* bias,
+                                  const int32_t* scatter, void* out, int32_t rows, void* stream);
+
 /* gate and up in one launch with the SwiGLU epilogue: hidden[i] = swiglu(x[gather[i]] @ Wg[e], .. @ Wu[e])
  * with the reference's rounding sequence (src/dew/nn/activations.py:267-278): both products rounded to
  * bf16, a = bf16(g * logistic(g)), hidden = bf16(a * u).                                                */

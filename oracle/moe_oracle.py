@@ -25,6 +25,15 @@ What pins each function (tests/test_oracle_golden.py):
 * `grouped_matmul`: tools/grouped_oracle.py:20-27 semantics (float64 per-group product) on integer inputs,
   where fp32 sums are exact.
 
+* `rows_quantized` / `blocks_quantized` / `blockwise_fp8_product` (the blockwise FP8 recipe): no byte fixture in
+  the reference (its tests hold the product to a float64 truth, tests/test_gemm_blockwise.py:20-40 over
+  tests/blockwise_matrix.py); pinned by what the arithmetic fixes: `e4m3_rounded` against a brute-force nearest
+  neighbour (ties to the even code) over every fp32 midpoint and grid point of E4M3FN, `power_of_two_ceil` on
+  exact powers and their neighbours, the scale rule on amax = 448 * 2^k and on the 1e-4 floor, the quantized
+  blocks reproducing tests/fixtures/codecs/deepgemm_fp8.npz's ue8m0 codes and scales wherever the two rules
+  agree (they differ only in how amax / 448 is rounded before the ceiling), and the product against the float64
+  sum of the dequantized operands at the reference's own bound.
+
 Parity unpinned (no byte fixture in the reference, closed form only): the exact bits of the softmax
 denominator's compensated sum (src/dew/nn/precision.py:1832); it moves router weights by at most one fp32
 ulp and no index. `gpt_oss_gating`'s bf16 mode: where each bf16 rounding falls follows JAX's arithmetic on
@@ -371,6 +380,124 @@ def grouped_matmul(x, w, sizes, *, dtype="bfloat16", factor=None, accumulate=F32
             out[start:start + size] = summed.astype(F32)
         start += size
     return bf16_round(out) if dtype == "bfloat16" else out
+
+
+# --------------------------------------------------------------------------------------------------
+# The blockwise FP8 recipe's forward product (activations quantized 1 x 128, weights 128 x 128)
+# --------------------------------------------------------------------------------------------------
+
+SCALE_DEPTH = 128
+E4M3_MAX = F32(448.0)
+
+
+def power_of_two_ceil(value):
+    """The least power of two >= `value` read off its fp32 bits: its exponent, plus one where any fraction
+    bit is set (src/dew/nn/fake_quant.py:48-57; normal values only, which a floored amax / 448 always is)."""
+    bits = np.ascontiguousarray(value, F32).view(np.uint32)
+    field = (bits >> np.uint32(23)) & np.uint32(0xFF)
+    field = field + ((bits & np.uint32(0x7FFFFF)) != 0)
+    return (field.astype(np.uint32) << np.uint32(23)).view(F32)
+
+
+def e4m3_rounded(values):
+    """fp32 values within +-448 rounded to E4M3FN, ties to even, by arithmetic (src/dew/nn/fake_quant.py:60-76):
+    the quantum is 2^(max(exponent, -6) - 3); the quotient by it is exact and `rint` ties to the even multiple."""
+    values = np.ascontiguousarray(values, F32)
+    exponent = ((values.view(np.uint32) >> np.uint32(23)) & np.uint32(0xFF)).astype(np.int32) - 127
+    quantum = np.exp2(np.maximum(exponent, -6) - 3).astype(F32)
+    return (np.rint(values / quantum) * quantum).astype(F32)
+
+
+def e4m3_bytes(values):
+    """The float8_e4m3fn byte of each value already on the E4M3FN grid (the `.astype(float8_e4m3fn)` of an exact
+    value; -0.0 keeps its sign)."""
+    values = np.ascontiguousarray(values, F32)
+    magnitudes = E4M3[:0x7F].astype(F32)  # ascending, 0 .. 448
+    index = np.searchsorted(magnitudes, np.abs(values))
+    assert np.array_equal(magnitudes[index], np.abs(values)), "a value off the E4M3FN grid"
+    return (index | np.where(np.signbit(values), 0x80, 0)).astype(np.uint8)
+
+
+def fp8_scaled_blocks(x, block):
+    """`x` in fp32 blocks of `block` channels and each block's power-of-two scale: amax floored at 1e-4, the scale
+    the ceiling power of two of amax * f32(1 / 448) (src/dew/nn/fake_quant.py:117-122)."""
+    blocks = np.asarray(x, F32).reshape(*np.shape(x)[:-1], -1, block)
+    amax = np.maximum(np.abs(blocks).max(axis=-1, keepdims=True), F32(1e-4)).astype(F32)
+    return blocks, power_of_two_ceil(amax * F32(1 / 448.0))
+
+
+def fp8_codes(values):
+    """src/dew/nn/fake_quant.py:125-128: clamp to +-448, round to E4M3FN."""
+    return e4m3_rounded(np.clip(np.asarray(values, F32), -E4M3_MAX, E4M3_MAX))
+
+
+def rows_quantized(x):
+    """`x [..., n]` as E4M3 values a 1 x 128 tile at a time along its last axis and each tile's power-of-two scale
+    `[..., n / 128]` (src/dew/nn/kernels/projections.py:176-182). Returns (values on the E4M3 grid, scales)."""
+    blocks, scale = fp8_scaled_blocks(x, SCALE_DEPTH)
+    return fp8_codes(blocks / scale).reshape(np.shape(x)), scale[..., 0]
+
+
+def blocks_quantized(w):
+    """`w [groups, depth, width]` as E4M3 values a 128 x 128 block at a time and each block's power-of-two scale
+    `[groups, depth / 128, width / 128]` (src/dew/nn/kernels/projections.py:185-196)."""
+    w = np.asarray(w, F32)
+    groups, depth, width = w.shape
+    edge = SCALE_DEPTH
+    tiled = w.reshape(groups, depth // edge, edge, width // edge, edge).transpose(0, 1, 3, 2, 4)
+    blocks, scale = fp8_scaled_blocks(tiled.reshape(groups, depth // edge, width // edge, -1), edge * edge)
+    codes = fp8_codes(blocks / scale).reshape(tiled.shape).transpose(0, 1, 3, 2, 4)
+    return codes.reshape(w.shape), scale[..., 0, 0]
+
+
+def twice_scaled(product, first, second):
+    """`product` times two scales in the order whose intermediate is a normal fp32
+    (src/dew/nn/precision.py:1782-1791)."""
+    product, first, second = np.broadcast_arrays(np.asarray(product, F32), np.asarray(first, F32), np.asarray(second, F32))
+    tiny = np.finfo(F32).tiny
+    with np.errstate(over="ignore", under="ignore"):
+        once = (product * first).astype(F32)
+        kept = np.isfinite(once) & ((np.abs(once) >= tiny) | (product == 0))
+        return (np.where(kept, once, (product * second).astype(F32)) * np.where(kept, second, first)).astype(F32)
+
+
+def blockwise_fp8_product(lhs, kernel, group_sizes, row_scales, column_scales, *, dtype="bfloat16", bias=None):
+    """Each group's rows of `lhs [rows, depth]` (E4M3 values) times its matrix of `kernel [groups, depth, width]`
+    (E4M3 values), each 128-deep block's partial, summed exactly and rounded to fp32, times its rows' scales
+    (`row_scales [depth / 128, rows]`) and its group's column scales (`column_scales [groups, depth / 128, width / c]`)
+    before it is added, in the blocks' order, into the fp32 sum; one rounding to `dtype`; rows past the groups are
+    zero (src/dew/nn/kernels/gemm.py:764-793 over src/dew/nn/kernels/xla_products.py:147-173). `bias [groups,
+    width]` is added to the fp32 sums before the rounding (src/dew/nn/kernels/projections.py:107-140).
+    The partial of 128 products of 8-bit-mantissa values is exact in float64."""
+    lhs, kernel = np.asarray(lhs, F32), np.asarray(kernel, F32)
+    row_scales, column_scales = np.asarray(row_scales, F32), np.asarray(column_scales, F32)
+    blocks, rows = row_scales.shape
+    groups, _, scaled = column_scales.shape
+    width = kernel.shape[2]
+    assert lhs.shape == (rows, blocks * SCALE_DEPTH) and kernel.shape[:2] == (groups, blocks * SCALE_DEPTH) and width % scaled == 0
+    total = np.zeros((rows, width), F32)
+    start = 0
+    for group, size in enumerate(np.asarray(group_sizes).tolist()):
+        span = slice(start, start + size)
+        for index in range(blocks if size else 0):
+            depth = slice(index * SCALE_DEPTH, (index + 1) * SCALE_DEPTH)
+            partial = (lhs[span, depth].astype(np.float64) @ kernel[group, depth].astype(np.float64)).astype(F32)
+            columns = np.repeat(column_scales[group, index], width // scaled)[None, :]
+            total[span] = total[span] + twice_scaled(partial, row_scales[index, span, None], columns)
+        if bias is not None and size:
+            total[span] = total[span] + np.asarray(bias, F32)[group][None, :]
+        start += size
+    return bf16_round(total) if dtype == "bfloat16" else total
+
+
+def blockwise_fp8_projection(x, w, group_sizes, *, dtype="bfloat16", bias=None):
+    """Each group's rows of `x` times its matrix of `w` in the blockwise FP8 recipe: both quantized
+    (`rows_quantized`, `blocks_quantized`), their product `blockwise_fp8_product`
+    (src/dew/nn/kernels/projections.py:199-204; with ragged groups and a bias, `recipe_projection` :96-140, whose
+    zero padding rows add nothing)."""
+    rows, rows_scales = rows_quantized(x)
+    blocks, blocks_scales = blocks_quantized(w)
+    return blockwise_fp8_product(rows, blocks, group_sizes, rows_scales.T, blocks_scales, dtype=dtype, bias=bias)
 
 
 def swiglu(gate, up, *, dtype="bfloat16", limit=None, exp=np.exp):

@@ -1,0 +1,144 @@
+"""The blockwise FP8 recipe's forward product on the device (rows quantized 1 x 128, weights 128 x 128, power-of-two
+scales, both operands through the scaled matrix instruction) against the CPU oracle.
+
+Bars: the rows' quantizer bit for bit (codes and scales are byte work); the product within one bf16 ulp of the
+largest output (kernel and oracle multiply the same codes exactly and differ in the order of the fp32 sums alone)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from dew_amd import ops
+
+    return ops
+
+
+def bf16_np(tensor):
+    return tensor.float().cpu().numpy()
+
+
+def rows_case(rows, depth, seed):
+    """Rows with the quantizer's corner tiles among ordinary ones."""
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((rows, depth)).astype(np.float32) * rng.choice([1e-3, 0.1, 1.0, 30.0], size=(rows, 1)).astype(np.float32)
+    x[0, :128] = 0.0                                   # an all-zero tile: the 1e-4 floor sets its scale
+    x[1, :128] = np.linspace(-1e-5, 1e-5, 128)         # under the floor: tiny codes, negative ones rounding to -0
+    x[2, :128] = np.clip(x[2, :128], -0.875, 0.875)
+    x[2, 5] = 0.875                                    # amax = 448 * 2^-9: amax * f32(1 / 448) decides the scale
+    x[3, :128] = np.clip(x[3, :128], -448.0, 448.0)
+    x[3, 77] = -448.0                                  # amax = 448 exactly
+    x[4, 128:256] *= 1e30                              # a huge tile beside ordinary ones
+    x[5, :128] = 2.0 ** -130                           # bf16 subnormals
+    return torch.from_numpy(x).to(torch.bfloat16)
+
+
+@pytest.mark.parametrize("rows,depth", [(7, 128), (33, 384), (260, 4096)])
+def test_rows_are_quantized_bit_for_bit(ops, rows, depth):
+    x = rows_case(rows, depth, seed=rows)
+    codes, scales = ops.quantize_rows_fp8(x.cuda())
+    want_values, want_scales = oracle.rows_quantized(bf16_np(x))
+    want_codes = oracle.e4m3_bytes(want_values)
+    got_codes = ops.depth_order_fp8(codes).cpu().numpy()
+    got_scales = scales.cpu().numpy()[:, :depth // 128]
+    assert np.array_equal(np.ldexp(np.float32(1), got_scales.astype(np.int32) - 127), want_scales)
+    assert np.array_equal(got_codes, want_codes)
+    assert np.array_equal(ops.operand_order_fp8(ops.depth_order_fp8(codes)).cpu().numpy(), codes.cpu().numpy())
+
+
+def weights_case(groups, depth, width, seed):
+    rng = np.random.default_rng(seed)
+    w = (rng.standard_normal((groups, depth, width)) * 0.02).astype(np.float32)
+    w[0, :128, :128] *= 50.0                           # blocks of different scales
+    w[-1, -128:, -128:] = 0.0                          # an all-zero block
+    return w
+
+
+SIZES = [("ragged", [130, 0, 1, 257, 64, 0, 127, 5]), ("single", [3]), ("blocks", [256, 128, 0, 384])]
+
+
+@pytest.mark.parametrize("label,sizes", SIZES, ids=[s[0] for s in SIZES])
+@pytest.mark.parametrize("depth,width", [(256, 128), (1152, 384)])
+def test_the_recipes_product_matches_the_oracle(ops, label, sizes, depth, width):
+    from dew_amd import projections
+
+    groups, rows = len(sizes), int(np.sum(sizes))
+    rng = np.random.default_rng(depth + rows)
+    x = torch.from_numpy(rng.standard_normal((rows + 6, depth)).astype(np.float32)).to(torch.bfloat16)   # 6 rows past the groups
+    w = weights_case(groups, depth, width, seed=depth)
+    bias = torch.from_numpy(rng.standard_normal((groups, width)).astype(np.float32) * 0.1)
+    sizes_device = torch.tensor(sizes, dtype=torch.int32).cuda()
+    bank = projections.blocks_quantized(torch.from_numpy(w)).to("cuda")
+    for with_bias in (None, bias):
+        got = bf16_np(projections.recipe_projection(x.cuda(), bank, sizes_device, bias=None if with_bias is None else with_bias.cuda()))
+        padded = list(sizes) + [0]
+        want = oracle.blockwise_fp8_projection(bf16_np(x), w, sizes, bias=None if with_bias is None else with_bias.numpy())
+        assert np.all(got[rows:] == 0) and np.all(want[rows:] == 0)
+        scale = np.abs(want).max()
+        assert np.abs(got - want).max() <= 2.0 ** -7 * scale
+        assert (got == want).mean() > 0.97
+    # the product alone from the quantized operands, against the float64 sum of the dequantized blocks (the
+    # reference's own truth, tests/blockwise_matrix.py): what one bf16 rounding of an fp32 sum allows
+    values, scales = oracle.rows_quantized(bf16_np(x))
+    blocks, block_scales = oracle.blocks_quantized(w)
+    truth = np.zeros((rows + 6, width))
+    start = 0
+    for group, size in enumerate(sizes):
+        lhs = (values[start:start + size].reshape(size, depth // 128, 128) * scales[start:start + size, :, None]).reshape(size, depth)
+        rhs = blocks[group] * np.repeat(np.repeat(block_scales[group], 128, axis=0), 128, axis=1)
+        truth[start:start + size] = lhs.astype(np.float64) @ rhs.astype(np.float64)
+        start += size
+    got = bf16_np(projections.recipe_projection(x.cuda(), bank, sizes_device))
+    assert np.abs(got - truth).max() <= 2.0 ** -8 * np.abs(truth).max() * 1.01
+
+
+def test_gathered_rows_and_scattered_outputs(ops):
+    from dew_amd import projections
+
+    sizes, depth, width = [200, 56, 300], 512, 256
+    rows = sum(sizes)
+    rng = np.random.default_rng(9)
+    x = torch.from_numpy(rng.standard_normal((400, depth)).astype(np.float32)).to(torch.bfloat16)
+    gather = rng.integers(0, 400, size=rows).astype(np.int32)
+    scatter = rng.permutation(rows).astype(np.int32)
+    w = weights_case(len(sizes), depth, width, seed=4)
+    bank = projections.blocks_quantized(torch.from_numpy(w)).to("cuda")
+    quantized = projections.rows_quantized(x.cuda())
+    got = bf16_np(projections.blockwise_fp8_product(quantized, bank, torch.tensor(sizes, dtype=torch.int32).cuda(),
+                                                    gather=torch.from_numpy(gather).cuda(), scatter=torch.from_numpy(scatter).cuda()))
+    want = oracle.blockwise_fp8_projection(bf16_np(x)[gather], w, sizes)
+    placed = np.zeros_like(want)
+    placed[scatter] = want
+    assert np.abs(got - placed).max() <= 2.0 ** -7 * np.abs(want).max() and (got == placed).mean() > 0.97
+
+
+def test_group_blocks_count_whole_128_row_blocks(ops):
+    from dew_amd import projections
+
+    blocks, depth, width = [2, 0, 1], 256, 128
+    rng = np.random.default_rng(2)
+    x = torch.from_numpy(rng.standard_normal((384, depth)).astype(np.float32)).to(torch.bfloat16)
+    w = weights_case(3, depth, width, seed=8)
+    got = bf16_np(projections.blockwise_fp8_projection(x.cuda(), torch.from_numpy(w).cuda(), blocks))
+    want = oracle.blockwise_fp8_projection(bf16_np(x), w, [256, 0, 128])
+    assert np.abs(got - want).max() <= 2.0 ** -7 * np.abs(want).max() and (got == want).mean() > 0.97
+
+
+def test_a_block_scale_that_is_no_power_of_two_is_not_multiplied_silently(ops):
+    from dew_amd import formats, projections
+
+    depth, width = 256, 256
+    rng = np.random.default_rng(3)
+    x = torch.from_numpy(rng.standard_normal((40, depth)).astype(np.float32)).to(torch.bfloat16)
+    bank = projections.blocks_quantized(torch.from_numpy(weights_case(1, depth, width, seed=5)))
+    scales = bank.scale_inv.clone()
+    scales[0, 1, 1] *= 1.5                              # a checkpoint's fp32 block scale, not the recipe's
+    spoiled = formats.Fp8Blocks(bank.codes, scales).to("cuda")
+    got = bf16_np(projections.recipe_projection(x.cuda(), spoiled, torch.tensor([40], dtype=torch.int32).cuda()))
+    assert np.isnan(got[:, 128:]).all() and np.isfinite(got[:, :128]).all()

@@ -1,0 +1,115 @@
+"""The blockwise FP8 recipe on the CPU: what pins the oracle's restatement (no byte fixture of the reference covers
+it, so each piece is held to what the arithmetic fixes), and the host mirror's weight quantizer against the oracle."""
+
+import pathlib
+
+import numpy as np
+import torch
+
+from oracle import moe_oracle as oracle
+
+GOLDEN = pathlib.Path(__file__).parent / "golden"
+
+
+def test_e4m3_rounding_is_nearest_with_ties_to_the_even_code():
+    """Brute force over every grid point, every midpoint between neighbours, and random values: the nearest E4M3FN
+    magnitude, a tie going to the even code."""
+    magnitudes = oracle.E4M3[:0x7F].astype(np.float64)
+    rng = np.random.default_rng(0)
+    values = np.concatenate([magnitudes, -magnitudes, (magnitudes[1:] + magnitudes[:-1]) / 2, rng.uniform(-448, 448, 5000),
+                             rng.standard_normal(5000) * 0.01, [2.0 ** -10, -2.0 ** -10, 3 * 2.0 ** -10, 447.9, -448.0]]).astype(np.float32)
+    got = oracle.e4m3_rounded(values)
+    distance = np.abs(magnitudes[None, :] - np.abs(values.astype(np.float64))[:, None])
+    best = distance.min(axis=1, keepdims=True)
+    tied = distance == best
+    index = np.where(tied.sum(axis=1) == 1, tied.argmax(axis=1), (tied & (np.arange(127) % 2 == 0)).argmax(axis=1))
+    assert np.array_equal(np.abs(got), magnitudes[index].astype(np.float32))
+    assert np.array_equal(np.signbit(got), np.signbit(values))                 # -2^-10 rounds to -0
+    assert np.array_equal(oracle.E4M3[oracle.e4m3_bytes(got)], got)
+
+
+def test_the_scale_is_the_least_power_of_two_at_or_above_amax_over_448():
+    assert np.array_equal(oracle.power_of_two_ceil(np.array([1, np.nextafter(np.float32(1), 2), 0.5, 0.75, 3, 4, 2.0 ** -20], np.float32)),
+                          np.array([1, 2, 0.5, 1, 4, 4, 2.0 ** -20], np.float32))
+    block = np.zeros((6, 128), np.float32)
+    block[0, 3] = 448.0                     # 448 * f32(1 / 448) rounds to 1 exactly: scale 1, code 448
+    block[1, 3] = 449.0                     # just above: scale 2
+    block[2, 3] = 0.875                     # 448 * 2^-9
+    block[3, 3] = 1e-5                      # under the floor: the floor's scale, 2^-22 (1e-4 / 448 = 2.2e-7 < 2^-22 = 2.4e-7)
+    block[5, 3] = -3.0
+    values, scales = oracle.rows_quantized(block)
+    assert scales[:, 0].tolist() == [1.0, 2.0, 2.0 ** -9, 2.0 ** -22, 2.0 ** -22, 2.0 ** -7]
+    assert values[0, 3] == 448.0 and values[1, 3] == 224.0 and values[2, 3] == 448.0 and values[5, 3] == -384.0
+    assert values[3, 3] == oracle.e4m3_rounded(np.float32(1e-5) / np.float32(2.0 ** -22))
+    # what a tile stands for is within half a code step of its source, 2^-4 of the tile's largest magnitude at most
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((50, 256)).astype(np.float32)
+    values, scales = oracle.rows_quantized(x)
+    rebuilt = (values.reshape(50, 2, 128) * scales[:, :, None]).reshape(50, 256)
+    assert np.abs(rebuilt - x).max() <= 2.0 ** -4 * np.abs(x).max()
+    assert np.abs(values).max() <= 448 and (np.abs(values).reshape(50, 2, 128).max(axis=2) >= 224).all()  # the least such scale
+
+
+def test_the_weight_blocks_agree_with_deepgemms_ue8m0_cast_where_the_rules_coincide():
+    """DeepGEMM's ue8m0 cast (the reference's fixture) takes the ceiling power of two of amax / 448, the recipe of
+    amax * f32(1 / 448): the same scale unless the two roundings of the quotient straddle a power of two, and then
+    the same codes."""
+    with np.load(GOLDEN / "codecs" / "deepgemm_fp8.npz") as held:
+        for name in ("random/256x384/128",):
+            weight = held[f"{name}/weight"]
+            values, scales = oracle.blocks_quantized(weight[None])
+            assert np.array_equal(scales[0], held[f"{name}/scales/ue8m0"])
+            assert np.array_equal(oracle.e4m3_bytes(values[0]), held[f"{name}/codes/ue8m0"])
+
+
+def test_the_product_scales_each_blocks_partial_before_it_is_added():
+    """Against the float64 sum of the dequantized operands (the reference's own truth for this product,
+    tests/test_gemm_blockwise.py:20-40): fp32's accuracy, with general (not power-of-two) scales as its test
+    draws them; rows past the groups are zero; swapping the two scale operands' roles changes the result."""
+    rng = np.random.default_rng(2)
+    sizes, depth, width = [40, 0, 25], 384, 256
+    rows = sum(sizes) + 3
+    lhs = oracle.e4m3_rounded(np.clip(rng.standard_normal((rows, depth)) * 100, -448, 448).astype(np.float32))
+    kernel = oracle.e4m3_rounded(np.clip(rng.standard_normal((3, depth, width)) * 100, -448, 448).astype(np.float32))
+    row_scales = rng.uniform(0.5, 2.0, size=(depth // 128, rows)).astype(np.float32)
+    column_scales = rng.uniform(0.5, 2.0, size=(3, depth // 128, width // 128)).astype(np.float32)
+    got = oracle.blockwise_fp8_product(lhs, kernel, sizes, row_scales, column_scales, dtype="float32")
+    truth = np.zeros((rows, width))
+    start = 0
+    for group, size in enumerate(sizes):
+        for block in range(depth // 128):
+            span = slice(128 * block, 128 * block + 128)
+            partial = lhs[start:start + size, span].astype(np.float64) @ kernel[group, span].astype(np.float64)
+            truth[start:start + size] += partial * row_scales[block, start:start + size, None] * np.repeat(column_scales[group, block], 128)[None, :]
+        start += size
+    assert np.all(got[sum(sizes):] == 0)
+    assert np.abs(got - truth).max() <= 4 * 2.0 ** -24 * np.abs(truth).max()
+    swapped = oracle.blockwise_fp8_product(lhs, kernel, sizes, row_scales[::-1], column_scales, dtype="float32")
+    assert np.abs(swapped - truth).max() > 1e-3 * np.abs(truth).max()
+    # scaling twice keeps extreme scales in range whichever comes first (src/dew/nn/precision.py:1782-1791)
+    assert oracle.twice_scaled(np.float32(2.0 ** 100), np.float32(2.0 ** 100), np.float32(2.0 ** -120)) == np.float32(2.0 ** 80)
+    assert oracle.twice_scaled(np.float32(2.0 ** -100), np.float32(2.0 ** -100), np.float32(2.0 ** 120)) == np.float32(2.0 ** -80)
+
+
+def weights_case(groups, depth, width, seed):
+    rng = np.random.default_rng(seed)
+    w = (rng.standard_normal((groups, depth, width)) * 0.02).astype(np.float32)
+    w[0, :128, :128] *= 50.0
+    w[-1, -128:, -128:] = 0.0
+    return w
+
+
+def test_the_host_mirror_quantizes_weight_blocks_as_the_oracle_does():
+    from dew_amd import projections
+
+    w = weights_case(3, 384, 256, seed=1)
+    bank = projections.blocks_quantized(torch.from_numpy(w))
+    want_values, want_scales = oracle.blocks_quantized(w)
+    assert np.array_equal(bank.scale_inv.numpy(), want_scales)
+    assert np.array_equal(bank.codes.numpy(), oracle.e4m3_bytes(want_values))
+
+
+def test_shapes_without_whole_blocks_are_left_to_the_caller():
+    from dew_amd import projections
+
+    assert projections.recipe_projection(torch.zeros((4, 192), dtype=torch.bfloat16), torch.zeros((192, 128))) is None
