@@ -25,6 +25,7 @@
 //     A lane's 16 bytes hold a run of consecutive depths, so the depth order inside a 64-deep step is permuted
 //     (the same permutation on the A side: only the LDS chunk a lane reads changes).
 #include <type_traits>
+#include <utility>
 
 #include "common.h"
 
@@ -133,6 +134,12 @@ constexpr size_t shared_bytes() {
   constexpr size_t ring = 3 * static_cast<size_t>(BM) * BK * 2;
   constexpr size_t staged = static_cast<size_t>(BM / ((BN == 256 && BM > 32) ? 2 : 1)) * ((MODE == 2 ? BN / 2 : BN) / 2 + 4) * 4;
   return ring > staged ? ring : staged;
+}
+
+// f(integral_constant<B>), f(integral_constant<B + 1>), ...: a loop whose index is a constant expression in its body.
+template <int B, int... Is, class F>
+__device__ __forceinline__ void static_range(std::integer_sequence<int, Is...>, F&& f) {
+  (f(std::integral_constant<int, B + Is>{}), ...);
 }
 
 // Instruction order of one phase of the main loop, stated to the scheduler: `MFMAS` matrix instructions in a
@@ -273,7 +280,9 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     const int chunk = (lane % 8) ^ (((row >> 1) & 7) ^ ((row & 1) << 2));
     const int sorted = row0 + min(row, valid_rows - 1);
     const int source = p.gather ? p.gather[sorted] : sorted;
-    a_src[i] = p.x + static_cast<size_t>(source) * (kFp8Rows ? p.depth / 2 : p.depth) + chunk * 8;  // a row of e4m3 codes is depth bytes
+    // (a row of e4m3 codes is depth bytes.) Less the load's immediate offset, which the instruction adds back: see load_a
+    a_src[i] = p.x + static_cast<size_t>(source) * (kFp8Rows ? p.depth / 2 : p.depth) + chunk * 8 - (i % 4) * 512;
+    asm volatile("" : "+v"(a_src[i]));  // kept as computed: the compiler otherwise re-adds the bias at every load
   }
   // Split activations: the lane's row of each row tile carries one e8m0 scale; the hi term multiplies under it
   // (byte 0) and the lo term under 2^-4 of it (byte 1).
@@ -320,31 +329,37 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
         a_block_word[buffer.value][i] = kFp8Rows ? a_block_byte[i] : a_block_byte[i] | ((a_block_byte[i] - 4) << 8);
     }
   };
+  // The LDS address of such a load is M0 + its immediate offset + 16 lane, and M0 costs three instructions to set
+  // (a lane read, the move, a wait state): four loads share one M0, the base of their first, and reach their own
+  // KiB of the stage through the immediate offset, which the global address is biased against (a_src above).
   auto load_a = [&](u32x4_t* stage, int step, auto begin, auto end) __attribute__((always_inline)) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass, which only needs the kernel's stub, does not know the builtin
-#pragma unroll
-    for (int i = begin.value; i < end.value; ++i)
+    static_range<decltype(begin)::value>(std::make_integer_sequence<int, decltype(end)::value - decltype(begin)::value>{}, [&](auto index) {
+      constexpr int i = decltype(index)::value, first = i / 4 * 4;
       __builtin_amdgcn_global_load_lds(a_src[i] + static_cast<size_t>(step) * BK,
-                                       (__attribute__((address_space(3))) void*)(stage + (wave * kRowLoads + i) * 64), 16, 0, 0);
+                                       (__attribute__((address_space(3))) void*)(stage + (wave * kRowLoads + first) * 64), 16,
+                                       (i - first) * 1024, 0);
+    });
 #endif
   };
 
   // ---- B loader: tile t = (matrix, 32-column tile j of the wavefront); the lane's piece of each atom ----
   const uint8_t* b_src[kTiles];
-  const uint16_t* b_scale_src[kTiles];  // FP4: the lane's two e4m3 block scales of each atom
-  float channel_scale[kTiles];          // FP8 channel: the lane's column scale
+  const uint8_t* b_scale_src[kTiles];  // FP4: the lane's two e4m3 block scales of each atom
+  float channel_scale[kTiles];         // FP8 channel: the lane's column scale
   const int n_atoms = p.width / 32, k_atoms = p.depth / kAtomK;
+  const uint32_t b_lane = lane * 16, b_scale_lane = lane * 2;
 #pragma unroll
   for (int t = 0; t < kTiles; ++t) {
     const int matrix = t / TJ, column = n0 + wn0 + 32 * (t % TJ);
     const uint8_t* codes = matrix == 0 ? p.w0.codes : p.w1.codes;
     const void* scales = matrix == 0 ? p.w0.scales : p.w1.scales;
     const size_t first_atom = (static_cast<size_t>(expert) * n_atoms + column / 32) * k_atoms;
-    b_src[t] = codes + first_atom * kAtomBytes + lane * 16;
+    b_src[t] = codes + first_atom * kAtomBytes + b_lane;
     b_scale_src[t] = nullptr;
     channel_scale[t] = 1.0f;
     if (kFp4) {
-      b_scale_src[t] = static_cast<const uint16_t*>(scales) + first_atom * 64 + lane;
+      b_scale_src[t] = static_cast<const uint8_t*>(scales) + first_atom * 128 + b_scale_lane;
     } else if (FORMAT == DEW_MOE_W_FP8_CHANNEL) {
       channel_scale[t] = static_cast<const float*>(scales)[static_cast<size_t>(expert) * p.width + column + lane % 32];
     }
@@ -369,7 +384,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
 #pragma unroll
       for (int a = 0; a < kAtoms; ++a)
         b_regs[set.value][t][a] = *reinterpret_cast<const u32x4_t*>(b_src[t] + (static_cast<size_t>(step) * kAtoms + a) * kAtomBytes);
-      if (kFp4) __builtin_memcpy(&s_regs[set.value][t], b_scale_src[t] + static_cast<size_t>(step) * 64, sizeof(uint32_t));
+      if (kFp4) __builtin_memcpy(&s_regs[set.value][t], b_scale_src[t] + static_cast<size_t>(step) * 128, sizeof(uint32_t));
     }
   };
 
