@@ -79,6 +79,8 @@ struct RouteParams {
   int32_t* indices;
   int tokens, experts, top_k, score_function, normalize, expert_groups, groups_per_token;
   float scaling;
+  float* scores;  // nullable [T, E]: the activated scores, as the router sows them for the balance statistics
+  float* log_z;   // nullable [T]: logsumexp of the logits (the z-loss's log partition)
 };
 
 template <int kPerLane>  // experts <= 64 * kPerLane
@@ -118,6 +120,30 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
   } else {
 #pragma unroll
     for (int i = 0; i < kPerLane; ++i) score[i] = 1.0f / (1.0f + exp_f32(-logit[i]));
+  }
+
+  // What the router sows beside its choices (src/dew/nn/moe.py:474-479): the scores, and the log partition
+  // max + log(sum exp(logit - max)) of the logits whatever the score function.
+  if (p.scores != nullptr && active) {
+#pragma unroll
+    for (int i = 0; i < kPerLane; ++i) {
+      const int e = lane + kWave * i;
+      if (e < p.experts) p.scores[static_cast<size_t>(token) * p.experts + e] = score[i];
+    }
+  }
+  if (p.log_z != nullptr) {
+    float m = ninf;
+#pragma unroll
+    for (int i = 0; i < kPerLane; ++i) m = fmaxf(m, logit[i]);
+    m = wave_max(m);
+    double partial = 0.0;
+#pragma unroll
+    for (int i = 0; i < kPerLane; ++i) {
+      const int e = lane + kWave * i;
+      if (e < p.experts) partial = partial + static_cast<double>(exp_f32(logit[i] - m));
+    }
+    const float total = wave_sum_once(partial);
+    if (active && lane == 0) p.log_z[token] = m + logf(total);
   }
 
 #pragma unroll
@@ -227,6 +253,14 @@ extern "C" int dew_moe_route(const float* logits, const float* bias, int32_t tok
                              int32_t top_k, int32_t score_function, int32_t normalize, float scaling,
                              int32_t expert_groups, int32_t groups_per_token, float* weights,
                              int32_t* indices, void* stream) {
+  return dew_moe_route_sown(logits, bias, tokens, experts, top_k, score_function, normalize, scaling, expert_groups,
+                            groups_per_token, weights, indices, nullptr, nullptr, stream);
+}
+
+extern "C" int dew_moe_route_sown(const float* logits, const float* bias, int32_t tokens, int32_t experts,
+                                  int32_t top_k, int32_t score_function, int32_t normalize, float scaling,
+                                  int32_t expert_groups, int32_t groups_per_token, float* weights,
+                                  int32_t* indices, float* scores, float* log_z, void* stream) {
   using namespace dew;
   DEW_REQUIRE(tokens >= 0 && experts >= 1, "dew_moe_route: tokens %d experts %d", tokens, experts);
   DEW_REQUIRE(tokens == 0 || (logits && weights && indices), "dew_moe_route: logits, weights and indices must not be null");
@@ -249,7 +283,7 @@ extern "C" int dew_moe_route(const float* logits, const float* bias, int32_t tok
   }
   if (tokens == 0) return DEW_MOE_OK;
   RouteParams p{logits, bias, weights, indices, tokens, experts, top_k, score_function, normalize ? 1 : 0,
-                expert_groups, groups_per_token, scaling};
+                expert_groups, groups_per_token, scaling, scores, log_z};
   const int blocks = (tokens + kRouteWaves - 1) / kRouteWaves;
   const size_t shared = expert_groups > 1 ? sizeof(float) * kRouteWaves * experts : 0;
   const dim3 grid(blocks), block(kWave * kRouteWaves);
@@ -264,4 +298,39 @@ extern "C" int dew_moe_route(const float* logits, const float* bias, int32_t tok
     hipLaunchKernelGGL(route_kernel<kMaxPerLane>, grid, block, shared, s, p);
   }
   return launched("route_kernel");
+}
+
+namespace dew {
+
+// The aux-loss-free balancing step on the selection bias (src/dew/nn/moe.py:271-300 `load_balance_update`, applied
+// as src/dew/objectives/routing.py:342-345): an expert that took more slots than the average loses `rate`, one that
+// took fewer gains it, one exactly at the floor of the average gains it only if the average has a remainder.
+__global__ __launch_bounds__(256) void balance_bias_kernel(const int32_t* __restrict__ counts, float* __restrict__ bias,
+                                                           float rate, int experts) {
+  __shared__ long long partial[256];
+  long long sum = 0;
+  for (int e = threadIdx.x; e < experts; e += 256) sum += counts[e];
+  partial[threadIdx.x] = sum;
+  __syncthreads();
+  for (int half = 128; half >= 1; half >>= 1) {
+    if (threadIdx.x < half) partial[threadIdx.x] += partial[threadIdx.x + half];
+    __syncthreads();
+  }
+  const long long total = partial[0];
+  const long long average = total / experts, remainder = total % experts;
+  for (int e = threadIdx.x; e < experts; e += 256) {
+    const long long count = counts[e];
+    const float direction = count > average ? -1.0f : (count < average || remainder > 0) ? 1.0f : 0.0f;
+    bias[e] = bias[e] + rate * direction;
+  }
+}
+
+}  // namespace dew
+
+extern "C" int dew_moe_balance_bias(const int32_t* counts, float* bias, float rate, int32_t experts, void* stream) {
+  using namespace dew;
+  DEW_REQUIRE(experts >= 1, "dew_moe_balance_bias: experts %d", experts);
+  DEW_REQUIRE(counts && bias, "dew_moe_balance_bias: counts and bias must not be null");
+  hipLaunchKernelGGL(balance_bias_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(stream), counts, bias, rate, experts);
+  return launched("balance_bias_kernel");
 }

@@ -158,20 +158,43 @@ class Router(_Module):
         kernel = _at(self.variables["params"], (*self.path, "kernel"))
         return ops.router_logits(x.reshape(-1, x.shape[-1]).contiguous(), kernel).reshape(*x.shape[:-1], self.num_experts)
 
-    def routed(self, logits: torch.Tensor):
-        """(weights, indices) from the logits on (src/dew/nn/moe.py:466-494)."""
+    def routed(self, logits: torch.Tensor, sown: dict | None = None):
+        """(weights, indices) from the logits on (src/dew/nn/moe.py:466-494). A caller that opens the 'router'
+        collection passes `sown`, a dict: it receives what the reference's router sows there (:474-479), the
+        choices under 'indices', the activated scores under 'scores' and each position's log partition
+        `logsumexp(logits)` under 'log_z', written by the same launch."""
         bias = _at(self.variables.get("moe"), (*self.path, "e_score_correction_bias")) if self.expert_bias else None
         if self.expert_bias and bias is None:
             raise KeyError(f"no moe/{'/'.join(self.path)}/e_score_correction_bias")
-        return ops.route(logits, self.top_k, score_function=self.score_function,
-                         normalize_weights=self.normalize_weights, bias=bias,
-                         routed_scaling_factor=self.routed_scaling_factor, expert_groups=self.expert_groups,
-                         groups_per_token=self.groups_per_token)
+        found = ops.route(logits, self.top_k, score_function=self.score_function,
+                          normalize_weights=self.normalize_weights, bias=bias,
+                          routed_scaling_factor=self.routed_scaling_factor, expert_groups=self.expert_groups,
+                          groups_per_token=self.groups_per_token, sown=sown is not None)
+        if sown is not None:
+            sown.update(indices=found[1], scores=found[2], log_z=found[3])
+        return found[0], found[1]
 
     def __call__(self, x, tokens=None, media=None, routes=None, blocks=None):
         if tokens is not None or media is not None or routes is not None or blocks is not None:
             raise ValueError("hash, media, replayed and block routing are not part of the HIP router")
         return self.routed(self.logits(x))
+
+
+def load_balance_update(counts: torch.Tensor, rate: float) -> torch.Tensor:
+    """Bias displacement from per-expert integer counts (src/dew/nn/moe.py:271-300): `-rate` for an expert above
+    the floor of the average count, `+rate` for one below it, or at it while the average has a remainder, else 0."""
+    return ops.balance_bias(torch.zeros(counts.shape, dtype=torch.float32, device=counts.device), counts.to(torch.int32), rate)
+
+
+def updated_bias(bias: torch.Tensor, counts: torch.Tensor, rate: float) -> torch.Tensor:
+    """The selection bias after one balancing step (src/dew/objectives/routing.py:342-345), a new tensor."""
+    return ops.balance_bias(bias.clone(), counts.to(torch.int32).contiguous(), rate)
+
+
+def router_counts(indices: torch.Tensor, num_experts: int) -> torch.Tensor:
+    """The slots each expert was chosen for (src/dew/objectives/routing.py:312-340 over one router call whose
+    queries are all real): the sizes of the dispatch sort."""
+    return ops.sort_by_expert(indices.reshape(-1, indices.shape[-1]), num_experts).sizes
 
 
 def _sorted_locally(indices: torch.Tensor, num_experts: int):

@@ -39,8 +39,9 @@ def device_check() -> None:
 
 def route(logits: torch.Tensor, top_k: int, *, score_function: str = "softmax", normalize_weights: bool = True,
           bias: torch.Tensor | None = None, routed_scaling_factor: float = 1.0, expert_groups: int = 1,
-          groups_per_token: int = 1):
-    """(weights fp32 `[..., k]`, indices int32 `[..., k]`) of router `logits [..., E]` (fp32)."""
+          groups_per_token: int = 1, sown: bool = False):
+    """(weights fp32 `[..., k]`, indices int32 `[..., k]`) of router `logits [..., E]` (fp32); with `sown`, also what
+    the router sows for the balance statistics: (weights, indices, scores fp32 `[..., E]`, log_z fp32 `[...]`)."""
     scores = {"softmax": _lib.SCORE_SOFTMAX, "sigmoid": _lib.SCORE_SIGMOID}
     if score_function not in scores:
         raise KernelError(f"score_function must be one of {list(scores)}, got {score_function!r}")
@@ -53,11 +54,29 @@ def route(logits: torch.Tensor, top_k: int, *, score_function: str = "softmax", 
     tokens = logits.numel() // experts
     weights = torch.empty((*logits.shape[:-1], top_k), dtype=torch.float32, device=logits.device)
     indices = torch.empty((*logits.shape[:-1], top_k), dtype=torch.int32, device=logits.device)
+    if sown:
+        activated = torch.empty_like(logits)
+        log_z = torch.empty(logits.shape[:-1], dtype=torch.float32, device=logits.device)
+        _lib.check(_lib.library().dew_moe_route_sown(
+            _ptr(logits), _ptr(bias), tokens, experts, top_k, scores[score_function], int(bool(normalize_weights)),
+            float(routed_scaling_factor), expert_groups, groups_per_token, _ptr(weights), _ptr(indices), _ptr(activated),
+            _ptr(log_z), _stream()), "dew_moe_route_sown")
+        return weights, indices, activated, log_z
     _lib.check(_lib.library().dew_moe_route(
         _ptr(logits), _ptr(bias), tokens, experts, top_k, scores[score_function], int(bool(normalize_weights)),
         float(routed_scaling_factor), expert_groups, groups_per_token, _ptr(weights), _ptr(indices), _stream()),
         "dew_moe_route")
     return weights, indices
+
+
+def balance_bias(bias: torch.Tensor, counts: torch.Tensor, rate: float) -> torch.Tensor:
+    """The aux-loss-free balancing step, in place: `bias[e] += rate * direction(counts)[e]` (the reference's
+    `load_balance_update`), `counts` the int32 slots each expert took (`sort_by_expert(...).sizes`)."""
+    _device(bias, "bias", torch.float32), _device(counts, "counts", torch.int32)
+    if bias.shape != counts.shape or bias.dim() != 1:
+        raise KernelError(f"bias {tuple(bias.shape)} and counts {tuple(counts.shape)} are one value per expert")
+    _lib.check(_lib.library().dew_moe_balance_bias(_ptr(counts), _ptr(bias), float(rate), bias.numel(), _stream()), "dew_moe_balance_bias")
+    return bias
 
 
 def router_logits(x: torch.Tensor, kernel: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:

@@ -71,6 +71,19 @@ int dew_moe_route(const float* logits, const float* bias /* nullable */, int32_t
                   int32_t expert_groups, int32_t groups_per_token, float* weights /* [T,k] */,
                   int32_t* indices /* [T,k] */, void* stream);
 
+/* dew_moe_route that also writes what the router sows for the balance statistics (src/dew/nn/moe.py:474-479): the
+ * activated scores[T,E] and log_z[T] = logsumexp of the logits (either may be null).                            */
+int dew_moe_route_sown(const float* logits, const float* bias /* nullable */, int32_t tokens, int32_t experts,
+                       int32_t top_k, int32_t score_function, int32_t normalize, float scaling,
+                       int32_t expert_groups, int32_t groups_per_token, float* weights, int32_t* indices,
+                       float* scores /* nullable [T,E] */, float* log_z /* nullable [T] */, void* stream);
+
+/* The aux-loss-free balancing step (`load_balance_update` src/dew/nn/moe.py:271-300, applied to the selection bias as
+ * `_updated_bias` src/dew/objectives/routing.py:342-345): bias[e] += rate * direction, direction -1 where counts[e]
+ * is above floor(sum / E), +1 where below it or equal with a remainder, else 0. counts = dew_moe_permute's sizes. */
+int dew_moe_balance_bias(const int32_t* counts /* [E] */, float* bias /* [E], updated in place */, float rate,
+                         int32_t experts, void* stream);
+
 /* Gate logits (src/dew/nn/moe.py:526-534): logits[T,E] = f32(x[T,D] bf16) @ kernel[D,E] f32, IEEE fp32, plus
  * bias[E] where the router has one (GPT-OSS's, src/dew/nn/gpt_oss.py:163-165).                              */
 int dew_moe_router_logits(const void* x /* bf16 [T,D] */, const float* kernel /* [D,E] */,

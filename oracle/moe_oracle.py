@@ -25,6 +25,9 @@ What pins each function (tests/test_oracle_golden.py):
 * `grouped_matmul`: tools/grouped_oracle.py:20-27 semantics (float64 per-group product) on integer inputs,
   where fp32 sums are exact.
 
+* `load_balance_update`: the known answer of tests/test_moe.py:326-336 (counts 3, 1, 0, 0 at rate 0.001).
+* `router_statistics`: closed forms (scores = exp(logits - log_z) for softmax; log_z(logits + c) = log_z + c; the
+  z-loss's log partition against a float64 logsumexp).
 * `rows_quantized` / `blocks_quantized` / `blockwise_fp8_product` (the blockwise FP8 recipe): no byte fixture in
   the reference (its tests hold the product to a float64 truth, tests/test_gemm_blockwise.py:20-40 over
   tests/blockwise_matrix.py); pinned by what the arithmetic fixes: `e4m3_rounded` against a brute-force nearest
@@ -329,6 +332,26 @@ def route(logits, top_k_count, *, score_function="softmax", normalize_weights=Tr
             total = (total + F32(weight_sum_epsilon)).astype(F32)
             weights = (weights / total[..., None]).astype(F32)
     return (weights * F32(routed_scaling_factor)).astype(F32), indices
+
+
+def router_statistics(logits, *, score_function="softmax"):
+    """What the router sows beside its choices (src/dew/nn/moe.py:474-479): the activated scores `[T, E]`
+    (`_activated`, :536-541) and the log partition of the logits `[T]`, `jax.nn.logsumexp`'s max + log(sum(exp(x -
+    max))) in fp32."""
+    logits = np.asarray(logits, F32)
+    scores = expert_softmax(logits) if score_function == "softmax" else logistic(logits)
+    top = logits.max(axis=-1, keepdims=True)
+    log_z = (top[..., 0] + np.log(np.exp((logits - top).astype(np.float64)).sum(axis=-1)).astype(F32)).astype(F32)
+    return scores, log_z
+
+
+def load_balance_update(counts, rate):
+    """src/dew/nn/moe.py:271-300, the integer branch: direction -1 where a count is above floor(sum / E), +1 where
+    below it or (at it) the sum leaves a remainder, else 0; times `rate` in fp32."""
+    counts = np.asarray(counts, np.int64)
+    average, remainder = divmod(int(counts.sum()), counts.size)
+    direction = np.where(counts > average, -1, np.where((counts < average) | (remainder > 0), 1, 0))
+    return (F32(rate) * direction.astype(F32)).astype(F32)
 
 
 def router_logits(x, kernel):

@@ -202,3 +202,29 @@ def test_more_experts_than_one_scan_round_and_every_expert_chosen():
     want_weights, want_indices = oracle.route(logits.numpy(), 8, score_function="softmax", normalize_weights=True)
     assert np.array_equal(indices.cpu().numpy(), want_indices) and np.array_equal(weights.cpu().numpy(), want_weights)
     assert np.array_equal(np.sort(indices.cpu().numpy(), -1), np.tile(np.arange(8), (33, 1)))
+
+
+@pytest.mark.parametrize("score_function,experts,top_k,groups", [("softmax", 8, 2, (1, 1)), ("sigmoid", 256, 8, (8, 4)), ("softmax", 130, 4, (1, 1))])
+def test_the_router_sows_its_scores_and_log_partition_and_the_bias_balances(score_function, experts, top_k, groups):
+    """The launch that routes also writes what the reference's router sows for the balance statistics; the choices
+    are the plain launch's bit for bit, scores and log partition within 1e-6 of the oracle's, and one balancing
+    step of the selection bias from the dispatch's own counts is the oracle's bit for bit."""
+    from dew_amd import moe, ops
+
+    rng = np.random.default_rng(experts)
+    logits = torch.from_numpy((rng.standard_normal((500, experts)) * 2).astype(np.float32)).cuda()
+    bias = torch.from_numpy((rng.standard_normal(experts) * 0.1).astype(np.float32)).cuda() if score_function == "sigmoid" else None
+    options = dict(score_function=score_function, bias=bias, expert_groups=groups[0], groups_per_token=groups[1])
+    weights, indices = ops.route(logits, top_k, **options)
+    sown_weights, sown_indices, scores, log_z = ops.route(logits, top_k, sown=True, **options)
+    assert torch.equal(weights, sown_weights) and torch.equal(indices, sown_indices)
+    want_scores, want_log_z = oracle.router_statistics(logits.cpu().numpy(), score_function=score_function)
+    assert np.abs(scores.cpu().numpy() - want_scores).max() <= 1e-6
+    assert np.abs(log_z.cpu().numpy() - want_log_z).max() <= 1e-6 * max(1.0, np.abs(want_log_z).max())
+    counts = moe.router_counts(indices, experts)
+    assert np.array_equal(counts.cpu().numpy(), np.bincount(indices.cpu().numpy().ravel(), minlength=experts))
+    start = torch.zeros(experts, dtype=torch.float32).cuda() if bias is None else bias
+    stepped = moe.updated_bias(start, counts, 0.001)
+    want = start.cpu().numpy() + oracle.load_balance_update(counts.cpu().numpy(), 0.001)
+    assert np.array_equal(stepped.cpu().numpy(), want.astype(np.float32))
+    assert np.array_equal(moe.load_balance_update(counts, 0.25).cpu().numpy(), oracle.load_balance_update(counts.cpu().numpy(), 0.25))

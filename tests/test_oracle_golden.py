@@ -283,3 +283,26 @@ def test_gpt_oss_gating_rounds_every_operation_in_bf16():
     # fp32 mode rounds nowhere and uses 1.702 itself
     exact = oracle.gpt_oss_gating(np.array([[1.0, 0.5]], np.float32), dtype="float32")
     assert abs(exact[0, 0] - 1.5 / (1 + np.exp(-1.702))) < 1e-6
+
+
+def test_the_balance_update_pushes_against_the_busy_experts():
+    """The reference's own known answer (tests/test_moe.py:326-336): over four experts, three slots on expert 0 and
+    one on expert 1 average one each, so expert 0 loses bias, expert 1 holds and the idle two gain."""
+    assert np.array_equal(oracle.load_balance_update([3, 1, 0, 0], 0.001), np.array([-0.001, 0.0, 0.001, 0.001], np.float32))
+    # a remainder tips the experts at the floor of the average upwards
+    assert np.array_equal(oracle.load_balance_update([2, 1, 1, 1], 0.5), np.array([-0.5, 0.5, 0.5, 0.5], np.float32))
+    assert np.array_equal(oracle.load_balance_update([2, 2, 2, 2], 0.5), np.zeros(4, np.float32))
+
+
+def test_the_sown_statistics_are_the_scores_and_the_log_partition():
+    rng = np.random.default_rng(5)
+    logits = (rng.standard_normal((40, 24)) * 3).astype(np.float32)
+    scores, log_z = oracle.router_statistics(logits)
+    wide = logits.astype(np.float64)
+    truth = np.log(np.exp(wide - wide.max(axis=1, keepdims=True)).sum(axis=1)) + wide.max(axis=1)
+    assert np.abs(log_z - truth).max() <= 1e-6 * np.abs(truth).max()
+    assert np.abs(scores - np.exp(wide - truth[:, None])).max() <= 1e-6            # softmax = exp(logit - log_z)
+    shifted = oracle.router_statistics(logits + np.float32(8.0))[1]
+    assert np.abs(shifted - (log_z + 8.0)).max() <= 1e-5
+    sigmoid, same = oracle.router_statistics(logits, score_function="sigmoid")
+    assert np.array_equal(same, log_z) and np.abs(sigmoid - 1 / (1 + np.exp(-wide))).max() <= 1e-6
