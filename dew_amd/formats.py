@@ -193,3 +193,23 @@ class Fp8Channels:
 
     def to(self, device) -> "Fp8Channels":
         return Fp8Channels(self.codes.to(device), self.scales.to(device))
+
+
+@dataclasses.dataclass(frozen=True)
+class Layered:
+    """An expert kernel read in place from a run's stack (src/dew/nn/moe.py:595-606): `stack` the bank of every
+    layer's experts along one axis (`[layers * E, K, N]`, any of the quantized formats or its prepared form) and
+    the `layer` read of `layers`. The grouped launch reads the layer's matrices where they lie."""
+
+    stack: object
+    layer: int
+    layers: int
+
+    @property
+    def shape(self):
+        total, depth, width = self.stack.shape
+        return (total // self.layers, depth, width)
+
+    @property
+    def dtype(self):
+        return torch.bfloat16

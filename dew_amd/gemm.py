@@ -50,7 +50,7 @@ class GroupedCase:
     epilogue_operands: tuple = ()
 
 
-_BANKS = (formats.NvFp4, formats.Fp8Blocks, formats.Fp8Channels, ops.PreparedBank)
+_BANKS = (formats.NvFp4, formats.Fp8Blocks, formats.Fp8Channels, formats.Layered, ops.PreparedBank)
 
 
 def _shape(bank):
@@ -114,6 +114,8 @@ def prepared(bank) -> ops.PreparedBank:
     """The bank's one-time device re-layout, cached on the bank object."""
     if isinstance(bank, ops.PreparedBank):
         return bank
+    if isinstance(bank, formats.Layered):  # the layer's matrices where they lie in the stack
+        return prepared(bank.stack).layer(int(bank.layer), int(bank.layers))
     held = getattr(bank, "_prepared", None)
     if held is None:
         held = ops.prepare(bank)

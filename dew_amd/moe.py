@@ -21,7 +21,7 @@ from typing import NamedTuple
 
 import torch
 
-from . import gemm, ops, selection
+from . import formats, gemm, ops, selection
 from .gemm import GroupSizes
 
 GROUPED_MATMULS = ("auto", "hip", "xla", "pallas")
@@ -43,6 +43,9 @@ class Gathered(NamedTuple):
     tokens: torch.Tensor
     rows: torch.Tensor
     slots: torch.Tensor
+
+
+Layered = formats.Layered
 
 
 def _implementation(implementation: str) -> str | None:

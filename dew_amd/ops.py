@@ -150,6 +150,24 @@ class PreparedBank:
     def experts(self):
         return self.shape[0]
 
+    def layer(self, index: int, layers: int) -> "PreparedBank":
+        """Layer `index` of a bank that stacks `layers` layers' experts along its expert axis (`[layers * E, K, N]`),
+        read where it lies: the same buffers, the descriptor's pointers moved to the layer's first expert (the
+        reference's `Layered` read, src/dew/nn/moe.py:595-606 and `gemm._grouped`'s `first`,
+        src/dew/nn/kernels/gemm.py:1763-1778), so no layer is copied out of the stack."""
+        total, depth, width = self.shape
+        if layers < 1 or total % layers or not 0 <= index < layers:
+            raise KernelError(f"layer {index} of {layers} in a bank of {total} matrices")
+        experts = total // layers
+        first = index * experts
+        held = self.descriptor
+        fp4 = held.format in (_lib.W_NVFP4, _lib.W_MXFP4)
+        codes = depth * width // 2 if fp4 else depth * width
+        scales = {_lib.W_FP8_BLOCK: (depth // 128) * (width // 128) * 4, _lib.W_FP8_CHANNEL: width * 4}.get(held.format, width * (depth // 16))
+        view = _lib.Bank(held.format, held.layout, experts, depth, width, held.codes + first * codes, held.scales + first * scales,
+                         None if not held.tensor_scale else held.tensor_scale + first * 4)
+        return PreparedBank(view, (experts, depth, width), self.keep)
+
 
 def prepare(bank) -> PreparedBank:
     """The one-time re-layout of a `formats.NvFp4`, `formats.Fp8Blocks` or `formats.Fp8Channels` bank."""

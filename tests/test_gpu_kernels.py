@@ -2,6 +2,8 @@
 Integer outputs (indices, sizes, offsets, order, rows) and router weights must match bit for bit; products
 are compared with the tolerance stated beside each check."""
 
+import dataclasses
+
 import numpy as np
 import pytest
 import torch
@@ -383,3 +385,28 @@ def test_the_expert_mlp_stays_on_split_rows_without_a_pass_between_its_products(
     scale = np.abs(want).max()
     assert np.abs(out[:x.shape[0]] - want).max() <= 2 ** -5 * scale and np.abs(out - plain).max() <= 2 ** -5 * scale
     assert (out == plain).mean() > 0.9
+
+
+@pytest.mark.parametrize("quant", ["fp8_block", "fp8_channel", "mxfp4", "nvfp4"])
+def test_a_layer_of_a_stacked_bank_is_read_where_it_lies(ops, quant):
+    """`Layered(stack, layer)`: the grouped product of one layer's experts out of a bank stacking three layers', from
+    the stack's own buffers, is the product of that layer's bank prepared alone, bit for bit."""
+    from dew_amd import gemm, moe
+
+    layers, experts, depth, width = 3, 4, 512, 256
+    sizes = [70, 0, 33, 129]
+    banks = [grouped_case(quant, experts, depth, width, sizes, seed=17 + layer) for layer in range(layers)]
+    x, offsets = banks[0][1].cuda(), torch.from_numpy(banks[0][2]).cuda()
+    first = banks[0][0]
+    joined = {field.name: torch.cat([getattr(bank, field.name) for bank, _, _ in banks]) for field in dataclasses.fields(first)
+              if field.name != "form"}
+    stacked = type(first)(**joined)
+    stack = ops.prepare(stacked.to("cuda"))
+    assert stack.shape == (layers * experts, depth, width)
+    for layer in range(layers):
+        alone = ops.grouped_gemm(x, ops.prepare(banks[layer][0].to("cuda")), offsets)
+        assert torch.equal(ops.grouped_gemm(x, stack.layer(layer, layers), offsets), alone)
+        through = gemm.gemm(x, moe.Layered(stack, layer, layers), gemm.GroupSizes(torch.tensor(sizes, dtype=torch.int32).cuda(), offsets))
+        assert torch.equal(through, alone)
+    with pytest.raises(Exception):
+        stack.layer(3, layers)
