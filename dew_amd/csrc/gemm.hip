@@ -189,7 +189,9 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   // MFMAs for each A fragment read from LDS) runs two blocks a CU (256 registers a lane each),
   // which FP8's 32 raw bytes a lane a tile a step only fit with three sets; two resident blocks cover the
   // shorter lookahead.
-  constexpr int kSets = (!kFp4 && BM == 128 && kMatrices * BN == 256) ? 3 : 4;
+  // Quantized rows on the full 256 x 256 tile: a step's weights are 64 registers a lane, of which two sets fit
+  // beside the accumulators (a load then has most of a 2048-cycle step to land).
+  constexpr int kSets = (kFp8Rows && BN == 256) ? 2 : (!kFp4 && BM == 128 && kMatrices * BN == 256) ? 3 : 4;
 
   extern __shared__ u32x4_t lds[];  // a ring of three stages of A: BM rows of 128 bytes each
   __shared__ int wave_tiles[4];
@@ -539,10 +541,15 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     if constexpr (kSplit) {
       // two phases a step: the hi term multiplies while the lo term is read, then the barrier, then the lo term
       // multiplies while the next step's hi term is read; each phase issues half of the step's global loads
-      constexpr std::integral_constant<int, kRowLoads / 2> ah{};
-      constexpr std::integral_constant<int, kTiles / 2> bh{};
+      // (With two weight sets the next step's weights are needed at its very start: all of them are issued in the
+      // first phase and the A rows in the second, so that the wait for the weights leaves the A rows in flight and
+      // neither has less than a phase to land. Issued half and half, the weights were the youngest loads at the
+      // step's end and the wait for them drained the memory pipeline every step.)
+      constexpr bool kWeightsFirst = kSets == 2;
+      constexpr std::integral_constant<int, kWeightsFirst ? 0 : kRowLoads / 2> ah{};
+      constexpr std::integral_constant<int, kWeightsFirst ? kTiles : kTiles / 2> bh{};
       constexpr int kSplitMfmas = kMatrices * TI * TJ;
-      constexpr int kSplitLoads = kRowLoads / 2 + (kTiles / 2) * kLoadsPerTile;
+      constexpr int kSplitLoads = ah.value + bh.value * kLoadsPerTile;  // the first phase's, the younger ones at the barrier
       static_assert(kRowLoads % 2 == 0 && kTiles % 2 == 0, "two even halves of loads");
       // younger than the last A load of the step before: only this phase's loads are sure to be
       constexpr int kSplitWait = (kSplitLoads & 0xF) | (7 << 4) | (0 << 8) | ((kSplitLoads >> 4) << 14);
@@ -570,8 +577,16 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
       multiply_term(set, c1, step);
       load_a(fill, ahead_a, ah, a4);
       load_b(filling, ahead_b, bh, b4);
-      schedule_phase<0, kSplitMfmas, 2 * TI, 0, 2 * kTiles + 2 * kSplitLoads, kSplitLoads>();
+      constexpr int kSecondLoads = kRowLoads - ah.value + (kTiles - bh.value) * kLoadsPerTile;
+      schedule_phase<0, kSplitMfmas, 2 * TI, 0, 2 * kTiles + 2 * kSecondLoads, kSecondLoads>();
       __builtin_amdgcn_sched_barrier(0);
+      if constexpr (kWeightsFirst) {
+        // the next step's weights have landed once only this phase's A rows are still in flight (stated here: left
+        // to itself the compiler waits for every load before the step's first multiply)
+        constexpr int kWeightsLanded = (kSecondLoads & 0xF) | (7 << 4) | (0xF << 8) | ((kSecondLoads >> 4) << 14);
+        if (!last_steps.value) __builtin_amdgcn_s_waitcnt(kWeightsLanded);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       stage_index = next_index;
       return;
     }
@@ -616,7 +631,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     stage_index = next_index;
   };
   load_b(c0, 0, c0, all_tiles);
-  load_b(c1, min(1, steps - 1), c0, all_tiles);
+  if constexpr (kSets >= 3) load_b(c1, min(1, steps - 1), c0, all_tiles);
   if constexpr (kSets == 4) load_b(c2, min(2, steps - 1), c0, all_tiles);
   load_a(lds, 0, c0, a4);
   load_a(lds + kStageChunks, min(1, steps - 1), c0, a4);
@@ -636,11 +651,13 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   for (; step + kSets <= steps; step += kSets) {
     iterate(c0, step, std::false_type{});
     iterate(c1, step + 1, std::false_type{});
-    iterate(c2, step + 2, std::false_type{});
+    if constexpr (kSets >= 3) iterate(c2, step + 2, std::false_type{});
     if constexpr (kSets == 4) iterate(c3, step + 3, std::false_type{});
   }
   if (step < steps) iterate(c0, step++, std::true_type{});  // the last steps % kSets steps
-  if (step < steps) iterate(c1, step++, std::true_type{});
+  if constexpr (kSets >= 3) {
+    if (step < steps) iterate(c1, step++, std::true_type{});
+  }
   if constexpr (kSets == 4) {
     if (step < steps) iterate(c2, step++, std::true_type{});
   }
@@ -653,9 +670,6 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   // the tile leaves as full cache lines (direct 4-byte stores of 64-byte row pieces took a quarter of the
   // kernel's time). Tiles of 256 columns are staged in two passes of BM / 2 rows.
   float factor0 = 1.0f, factor1 = 1.0f;
-  // quantized rows: a weight block scale that is no normal power of two cannot enter the instruction; the tile is
-  // then written as NaN rather than as the product under another scale
-  if (kFp8Rows && unscalable != 0) factor0 = factor1 = __uint_as_float(0x7FC00000u);
   if (kFp4) {  // the 2^8 the decode owes times the expert's tensor scale (src/dew/nn/kernels/gemm.py:660-662)
     // (the scaled instruction applies the block scales themselves, not their 2^-8)
     factor0 = (kSplit ? 1.0f : 256.0f) * p.w0.tensor_scale[expert];
@@ -676,6 +690,14 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
 #pragma unroll
   for (int j = 0; j < TJ; ++j)
     bias[j] = (!PAIRED && p.bias) ? p.bias[static_cast<size_t>(expert) * p.width + n0 + wn0 + 32 * j + lane % 32] : 0.0f;
+  // quantized rows: a weight block scale that is no normal power of two cannot enter the instruction; the tile is
+  // then written as NaN (through the addend every sum meets) rather than as the product under another scale
+  if (kFp8Rows && unscalable != 0) {
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) bias[j] = __uint_as_float(0x7FC00000u);
+  }
+  // bytes of (neighbour's pair, own pair) that make the lane's staged pair: see the swap below
+  const uint32_t swap_select = odd_lane ? 0x03020706u : 0x05040100u;
   __builtin_amdgcn_s_barrier();  // every wavefront has read its last A fragments: the ring is free
 #pragma unroll
   for (int pass = 0; pass < kPasses; ++pass) {
@@ -708,16 +730,20 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
             const bf16_t value = odd_lane ? gated_pair_rounded(got, mine[1], p.limit) : gated_pair_rounded(mine[0], got, p.limit);
             reinterpret_cast<bf16_t*>(staged)[row * (2 * kRowDwords) + (wn0 + 32 * j + lane % 32) / 2] = value;
           } else {
-            uint32_t mine[2];
-#pragma unroll
-            for (int r = 0; r < 2; ++r) {
-              mine[r] = PAIRED ? swiglu_rounded(acc[0][i][j][q + r] * factor0, acc[kMatrices - 1][i][j][q + r] * factor1)
-                               : f32_to_bf16(acc[0][i][j][q + r] * factor0 + bias[j]);
+            // the lane's rows q (low half) and q + 1 (high half) of its column, rounded
+            uint32_t mine;
+            if constexpr (PAIRED) {
+              mine = swiglu_rounded(acc[0][i][j][q] * factor0, acc[kMatrices - 1][i][j][q] * factor1) |
+                     (static_cast<uint32_t>(swiglu_rounded(acc[0][i][j][q + 1] * factor0, acc[kMatrices - 1][i][j][q + 1] * factor1)) << 16);
+            } else if constexpr (kFp4) {
+              mine = pack_bf16(acc[0][i][j][q] * factor0 + bias[j], acc[0][i][j][q + 1] * factor0 + bias[j]);
+            } else {
+              mine = pack_bf16(acc[0][i][j][q] + bias[j], acc[0][i][j][q + 1] + bias[j]);
             }
-            // even lane keeps row q and sends its row q + 1; odd lane keeps row q + 1 and sends its row q
-            const uint32_t sent = odd_lane ? mine[0] : mine[1];
-            const uint32_t got = __builtin_amdgcn_mov_dpp(sent, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
-            const uint32_t packed = odd_lane ? (got | (mine[1] << 16)) : (mine[0] | (got << 16));
+            // the even lane keeps row q of both columns and the odd lane row q + 1: each takes the neighbour's pair
+            // (quad_perm [1,0,3,2]) and picks its four bytes out of the two pairs with one byte permute
+            const uint32_t other = __builtin_amdgcn_mov_dpp(mine, 0xB1, 0xF, 0xF, true);
+            const uint32_t packed = __builtin_amdgcn_perm(other, mine, swap_select);
             staged[row * kRowDwords + (wn0 + 32 * j + (lane % 32 & ~1)) / 2] = packed;
           }
         }
@@ -1007,6 +1033,7 @@ extern "C" int dew_moe_grouped_gemm_fp8_rows(const void* x_codes, const uint8_t*
   GemmParams p{};
   if (int rc = fill_single(who, p, x_codes, gather, offsets, w, bias, scatter, out, rows)) return rc;
   p.a_scale = x_scales;
+  if (p.width % 256 == 0) return launch_tile<kFormatFp8Rows, kPlain, 256, 256, 2, 2>(who, p, static_cast<hipStream_t>(stream));
   return launch_tile<kFormatFp8Rows, kPlain, 256, 128, 2, 2>(who, p, static_cast<hipStream_t>(stream));
 }
 
