@@ -395,13 +395,21 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   i32x8_t a_term[2][kSplit ? TI : 1];  // split activations: [0] the hi term of a step, [1] its lo term
   float fp4_scale[kTiles];
   // a term of a 32-depth block is 32 bytes: the lane's block lane / 32 of the step holds hi in its chunks 0-1, lo in 2-3
+  // The lane's four chunks of its first row tile, as chunk indices into a stage: computed once, so that a phase's
+  // reads are the stage's base plus one of these plus 32 rows (a constant) a row tile further.
+  int term_chunk[2][2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int piece = 0; piece < 2; ++piece) term_chunk[t][piece] = swizzled(wm0 + lane % 32, 4 * (lane / 32) + 2 * t + piece);
   auto fetch_term = [&](const u32x4_t* stage, auto term) __attribute__((always_inline)) {
     if constexpr (kSplit) {
+      const u32x4_t* first_piece = stage + term_chunk[term.value][0];
+      const u32x4_t* second_piece = stage + term_chunk[term.value][1];
 #pragma unroll
       for (int i = 0; i < TI; ++i) {
-        const int row = wm0 + 32 * i + lane % 32;
-        const u32x4_t first = stage[swizzled(row, 4 * (lane / 32) + 2 * term.value)];
-        const u32x4_t second = stage[swizzled(row, 4 * (lane / 32) + 2 * term.value + 1)];
+        const u32x4_t first = first_piece[32 * i * kChunksPerRow];  // the swizzle reads a row's low four bits only
+        const u32x4_t second = second_piece[32 * i * kChunksPerRow];
         a_term[term.value][i] = i32x8_t{static_cast<int>(first[0]), static_cast<int>(first[1]), static_cast<int>(first[2]),
                                         static_cast<int>(first[3]), static_cast<int>(second[0]), static_cast<int>(second[1]),
                                         static_cast<int>(second[2]), static_cast<int>(second[3])};
