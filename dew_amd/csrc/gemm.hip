@@ -41,13 +41,18 @@ typedef __attribute__((ext_vector_type(8))) int i32x8_t;       // an operand of 
 // Kernel-side format of an MXFP4 bank multiplied by activation rows already split into two e4m3 terms
 // (dew_moe_split_rows): v_mfma_scale_f32_32x32x64_f8f6f4 takes the FP4 codes and their power-of-two block scales
 // as they are stored, so the weights are not dequantized at all.
-constexpr int kFormatMxSplit = 5;
-constexpr int kFormatMxSplitBlocks = 6;  // the same with one activation scale per row and 128 depths, not per row
+constexpr int kFormatMxSplit = 16;
+constexpr int kFormatMxSplitBlocks = 17;  // the same with one activation scale per row and 128 depths, not per row
 // Kernel-side format of an FP8 128 x 128 block bank whose scales are powers of two, multiplied by rows quantized to
 // e4m3 a 1 x 128 tile at a time under power-of-two scales (dew_moe_quantize_rows_fp8): the blockwise FP8 recipe's
 // product. The same instruction takes both operands' codes and scales as stored; a step is 128 depths, its two
 // 64-deep halves taking the places of the split rows' two terms.
-constexpr int kFormatFp8Rows = 7;
+constexpr int kFormatFp8Rows = 18;
+// Kernel-side format of an MXFP8 bank (DEW_MOE_W_MXFP8: e4m3 codes, one E8M0 scale per column and 32 depths)
+// multiplied by MXFP8 rows (dew_moe_quantize_rows_mxfp8): OCP MX as the instruction defines it, each lane handing
+// in the scale byte of its row (column) and 32-deep block. The rows' scale bytes ride the A ring, a dword a row a
+// step; the weights' come with their atoms, a dword a column a step.
+constexpr int kFormatMxFp8Rows = 19;
 
 constexpr int BK = 64;
 constexpr int kThreads = 256;
@@ -170,15 +175,17 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   constexpr bool kGated = MODE == kInterleavedGated;
   constexpr int kOutBN = kGated ? BN / 2 : BN;  // output columns of the tile
   static_assert(WM * WN == 4 && BM % (32 * WM) == 0 && BN % (32 * WN) == 0 && BM % 32 == 0, "tile shape");
-  constexpr bool kFp8Rows = FORMAT == kFormatFp8Rows;
-  constexpr bool kSplit = FORMAT == kFormatMxSplit || FORMAT == kFormatMxSplitBlocks || kFp8Rows;  // A arrives as 8-bit codes
+  constexpr bool kFp8Rows = FORMAT == kFormatFp8Rows;   // e4m3 rows, one scale per row and 128 depths; 128 x 128 weight scales
+  constexpr bool kMxRows = FORMAT == kFormatMxFp8Rows;  // e4m3 rows and weights, one scale per row (column) and 32 depths
+  constexpr bool kFp8A = kFp8Rows || kMxRows;           // both operands e4m3 codes: a step is 128 depths
+  constexpr bool kSplit = FORMAT == kFormatMxSplit || FORMAT == kFormatMxSplitBlocks || kFp8A;  // A arrives as 8-bit codes
   constexpr bool kBlockScales = FORMAT == kFormatMxSplitBlocks || kFp8Rows;
-  constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4 || (kSplit && !kFp8Rows);
-  constexpr bool kPow2 = FORMAT == DEW_MOE_W_MXFP4 || (kSplit && !kFp8Rows);
+  constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4 || (kSplit && !kFp8A);
+  constexpr bool kPow2 = FORMAT == DEW_MOE_W_MXFP4 || (kSplit && !kFp8A);
   constexpr bool kBlockBank = FORMAT == DEW_MOE_W_FP8_BLOCK || kFp8Rows;  // one fp32 scale per 128 x 128 weights
   constexpr int kMatrices = PAIRED ? 2 : 1;
   constexpr int kAtomK = kFp4 ? 64 : 32;       // depth an atom covers
-  constexpr int kStepDepth = kFp8Rows ? 128 : BK;  // depth a step covers: always 128 bytes of an A row
+  constexpr int kStepDepth = kFp8A ? 128 : BK;  // depth a step covers: always 128 bytes of an A row
   constexpr int kAtoms = kStepDepth / kAtomK;  // 16-byte loads a lane makes per 32-column tile per step
   constexpr int kRowLoads = BM / 32;           // A rows a lane loads per step
   constexpr int TI = BM / (32 * WM), TJ = BN / (32 * WN);  // MFMA tiles per wavefront: rows, columns of each matrix
@@ -191,7 +198,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   // shorter lookahead.
   // Quantized rows on the full 256 x 256 tile: a step's weights are 64 registers a lane, of which two sets fit
   // beside the accumulators (a load then has most of a 2048-cycle step to land).
-  constexpr int kSets = (kFp8Rows && BN == 256) ? 2 : (!kFp4 && BM == 128 && kMatrices * BN == 256) ? 3 : 4;
+  constexpr int kSets = (kFp8A && BN == 256) ? 2 : (!kFp4 && BM == 128 && kMatrices * BN == 256) ? 3 : 4;
 
   extern __shared__ u32x4_t lds[];  // a ring of three stages of A: BM rows of 128 bytes each
   __shared__ int wave_tiles[4];
@@ -283,7 +290,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     const int sorted = row0 + min(row, valid_rows - 1);
     const int source = p.gather ? p.gather[sorted] : sorted;
     // (a row of e4m3 codes is depth bytes.) Less the load's immediate offset, which the instruction adds back: see load_a
-    a_src[i] = p.x + static_cast<size_t>(source) * (kFp8Rows ? p.depth / 2 : p.depth) + chunk * 8 - (i % 4) * 512;
+    a_src[i] = p.x + static_cast<size_t>(source) * (kFp8A ? p.depth / 2 : p.depth) + chunk * 8 - (i % 4) * 512;
     asm volatile("" : "+v"(a_src[i]));  // kept as computed: the compiler otherwise re-adds the bias at every load
   }
   // Split activations: the lane's row of each row tile carries one e8m0 scale; the hi term multiplies under it
@@ -345,6 +352,33 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
 #endif
   };
 
+  // MXFP8 rows: a step's four scale bytes of each row, one dword a row, ride the ring beside the A rows: thread t
+  // fetches row t's (one 4-byte LDS-DMA load a wavefront a step), into BM dwords a stage behind the ring.
+  uint32_t* a_mx_stage = reinterpret_cast<uint32_t*>(lds + kStages * kStageChunks);
+  const uint8_t* a_mx_src = nullptr;
+  (void)a_mx_src;  // (the host pass compiles no load)
+  if constexpr (kMxRows) {
+    static_assert(!kMxRows || BM == kThreads, "one thread fetches one row's scales");
+    const int sorted = row0 + min(tid, valid_rows - 1);
+    const int source = p.gather ? p.gather[sorted] : sorted;
+    a_mx_src = p.a_scale + static_cast<size_t>(source) * (p.depth / 32);
+  }
+  auto load_a_scales = [&](int stage_number, int step) __attribute__((always_inline)) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    if constexpr (kMxRows)
+      __builtin_amdgcn_global_load_lds(a_mx_src + 4 * step, (__attribute__((address_space(3))) void*)(a_mx_stage + stage_number * BM + wave * 64),
+                                       4, 0, 0);
+#endif
+  };
+  uint32_t a_mx_word[2][kMxRows ? TI : 1];  // the lane's rows' scale dwords of a step, shifted so that byte 2 t is term t's
+  auto fetch_a_scales = [&](auto buffer, int stage_number) __attribute__((always_inline)) {
+    if constexpr (kMxRows) {
+#pragma unroll
+      for (int i = 0; i < TI; ++i)
+        a_mx_word[buffer.value][i] = a_mx_stage[stage_number * BM + wm0 + 32 * i + lane % 32] >> (8 * (lane / 32));
+    }
+  };
+
   // ---- B loader: tile t = (matrix, 32-column tile j of the wavefront); the lane's piece of each atom ----
   const uint8_t* b_src[kTiles];
   const uint8_t* b_scale_src[kTiles];  // FP4: the lane's two e4m3 block scales of each atom
@@ -362,6 +396,9 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     channel_scale[t] = 1.0f;
     if (kFp4) {
       b_scale_src[t] = static_cast<const uint8_t*>(scales) + first_atom * 128 + b_scale_lane;
+    } else if (kMxRows) {  // [E][N / 32][K / 128][32 columns][4 bytes]: the lane's column's dword of each step
+      b_scale_src[t] = static_cast<const uint8_t*>(scales) +
+                       (static_cast<size_t>(expert) * n_atoms + column / 32) * (p.depth / 128) * 128 + (lane % 32) * 4;
     } else if (FORMAT == DEW_MOE_W_FP8_CHANNEL) {
       channel_scale[t] = static_cast<const float*>(scales)[static_cast<size_t>(expert) * p.width + column + lane % 32];
     }
@@ -386,7 +423,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
 #pragma unroll
       for (int a = 0; a < kAtoms; ++a)
         b_regs[set.value][t][a] = *reinterpret_cast<const u32x4_t*>(b_src[t] + (static_cast<size_t>(step) * kAtoms + a) * kAtomBytes);
-      if (kFp4) __builtin_memcpy(&s_regs[set.value][t], b_scale_src[t] + static_cast<size_t>(step) * 128, sizeof(uint32_t));
+      if (kFp4 || kMxRows) __builtin_memcpy(&s_regs[set.value][t], b_scale_src[t] + static_cast<size_t>(step) * 128, sizeof(uint32_t));
     }
   };
 
@@ -467,24 +504,34 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     if constexpr (kSplit) {
       // block scales: of the unrolled four steps, steps 0, 1 read set 0 and steps 2, 3 set 1 (a scale holds for two
       // 64-deep steps); quantized rows' 128-deep steps alternate
-      constexpr int kBuffer = kFp8Rows ? set.value % 2 : (set.value / 2) % 2;
+      constexpr int kBuffer = kFp8A ? set.value % 2 : (set.value / 2) % 2;
 #pragma unroll
       for (int m = 0; m < kMatrices; ++m)
 #pragma unroll
         for (int j = 0; j < TJ; ++j) {
-          if constexpr (kFp8Rows) {
+          if constexpr (kFp8A) {
             // both operands e4m3: the half's 64 depths are two 32-deep atoms of the bank, in the operand's own order
             const u32x4_t& first = b_regs[set.value][m * TJ + j][2 * term.value];
             const u32x4_t& second = b_regs[set.value][m * TJ + j][2 * term.value + 1];
             const i32x8_t codes = {static_cast<int>(first[0]), static_cast<int>(first[1]), static_cast<int>(first[2]), static_cast<int>(first[3]),
                                    static_cast<int>(second[0]), static_cast<int>(second[1]), static_cast<int>(second[2]), static_cast<int>(second[3])};
-            const uint32_t bits = __float_as_uint(depth_scales[m * (BN / 128) + (wn0 + 32 * j) / 128][step]);
-            unscalable |= (bits & 0x807FFFFFu) | ((bits >> 23) == 0u) | ((bits >> 23) == 255u);
-            const int b_scale = static_cast<int>(bits >> 23);
+            if constexpr (kMxRows) {
+              // each lane hands in the scale of its row (column) and its lane group's 32 of the half's 64 depths:
+              // byte 2 term + lane / 32 of the step's dword, brought to byte 2 term by the shift
+              const int b_scale = static_cast<int>(s_regs[set.value][m * TJ + j] >> (8 * (lane / 32)));
 #pragma unroll
-            for (int i = 0; i < TI; ++i)
-              acc[m][i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_term[term.value][i], codes, acc[m][i][j], 0, 0, 0,
-                                                                          a_block_word[kBuffer][i], 0, b_scale);
+              for (int i = 0; i < TI; ++i)
+                acc[m][i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_term[term.value][i], codes, acc[m][i][j], 0, 0, 2 * term.value,
+                                                                            static_cast<int>(a_mx_word[kBuffer][i]), 2 * term.value, b_scale);
+            } else {
+              const uint32_t bits = __float_as_uint(depth_scales[m * (BN / 128) + (wn0 + 32 * j) / 128][step]);
+              unscalable |= (bits & 0x807FFFFFu) | ((bits >> 23) == 0u) | ((bits >> 23) == 255u);
+              const int b_scale = static_cast<int>(bits >> 23);
+#pragma unroll
+              for (int i = 0; i < TI; ++i)
+                acc[m][i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_term[term.value][i], codes, acc[m][i][j], 0, 0, 0,
+                                                                            a_block_word[kBuffer][i], 0, b_scale);
+            }
           } else {
             const u32x4_t& raw = b_regs[set.value][m * TJ + j][0];
             const i32x8_t codes = {static_cast<int>(raw[0]), static_cast<int>(raw[1]), static_cast<int>(raw[2]), static_cast<int>(raw[3]), 0, 0, 0, 0};
@@ -525,7 +572,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   constexpr std::integral_constant<int, kTiles> all_tiles{};
   constexpr int kMfmas = kMatrices * TI * TJ;
   constexpr int kDequantOps = kTiles * (kPow2 ? 5 : 17);  // vector instructions to dequantize one slice
-  constexpr int kLoadsPerTile = kAtoms + (kFp4 ? 1 : 0);
+  constexpr int kLoadsPerTile = kAtoms + (kFp4 || kMxRows ? 1 : 0);
   constexpr int kLoadsPerPhase = (kRowLoads + 3) / 4 + ((kTiles + 3) / 4) * kLoadsPerTile;
   // s_waitcnt vmcnt(kYounger) lgkmcnt(0): everything but the kYounger youngest vector-memory operations is done.
   // Younger than the last A load of step s + 1 (issued during step s - 1, in the last phase that has one) are
@@ -574,7 +621,10 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
       __builtin_amdgcn_sched_barrier(0);
       // block scales: the bytes of the next 128 depths are read from the LDS in the second phase of an even step
       // and formed into words in the second phase of the odd step that follows, one phase before they multiply
-      if constexpr (kFp8Rows) {  // a step is the 128 depths of one scale: the next step's, into the other set
+      if constexpr (kMxRows) {
+        fetch_a_scales(std::integral_constant<int, 1 - set.value % 2>{}, next_index);  // the next step's, landed before the barrier
+        load_a_scales(fill_index, ahead_a);
+      } else if constexpr (kFp8Rows) {  // a step is the 128 depths of one scale: the next step's, into the other set
         load_block_scales(min(step + 1, steps - 1));
         form_block_words(std::integral_constant<int, 1 - set.value % 2>{});
       } else {
@@ -585,7 +635,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
       multiply_term(set, c1, step);
       load_a(fill, ahead_a, ah, a4);
       load_b(filling, ahead_b, bh, b4);
-      constexpr int kSecondLoads = kRowLoads - ah.value + (kTiles - bh.value) * kLoadsPerTile;
+      constexpr int kSecondLoads = kRowLoads - ah.value + (kTiles - bh.value) * kLoadsPerTile + (kMxRows ? 1 : 0);
       schedule_phase<0, kSplitMfmas, 2 * TI, 0, 2 * kTiles + 2 * kSecondLoads, kSecondLoads>();
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (kWeightsFirst) {
@@ -643,6 +693,8 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   if constexpr (kSets == 4) load_b(c2, min(2, steps - 1), c0, all_tiles);
   load_a(lds, 0, c0, a4);
   load_a(lds + kStageChunks, min(1, steps - 1), c0, a4);
+  load_a_scales(0, 0);
+  load_a_scales(1, min(1, steps - 1));
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_waitcnt(kWaitAll);
   __builtin_amdgcn_s_barrier();
@@ -650,6 +702,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   if constexpr (kSplit) {
     load_block_scales(0);
     form_block_words(c0);
+    fetch_a_scales(c0, 0);
     fetch_term(lds, c0);
   } else {
     fetch(lds, c0, c0);
@@ -817,7 +870,7 @@ static int check_bank(const char* who, const dew_moe_bank* bank, const char* nam
   DEW_REQUIRE(bank, "%s: %s bank must not be null", who, name);
   DEW_REQUIRE(bank->layout == DEW_MOE_LAYOUT_PREPARED, "%s: %s bank is in the reference layout; call dew_moe_prepare_bank once at load", who, name);
   DEW_REQUIRE(bank->format == DEW_MOE_W_FP8_BLOCK || bank->format == DEW_MOE_W_FP8_CHANNEL || bank->format == DEW_MOE_W_NVFP4 ||
-                  bank->format == DEW_MOE_W_MXFP4,
+                  bank->format == DEW_MOE_W_MXFP4 || bank->format == DEW_MOE_W_MXFP8,
               "%s: %s bank has unknown format %d", who, name, bank->format);
   DEW_REQUIRE(bank->experts >= 1 && bank->experts <= 4096, "%s: %s bank has %d experts", who, name, bank->experts);
   DEW_REQUIRE(bank->depth >= 128 && bank->depth % 128 == 0, "%s: %s bank depth %d is not a multiple of 128", who, name, bank->depth);
@@ -833,7 +886,8 @@ template <int FORMAT, int MODE, int BM, int BN, int WM, int WN>
 static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
   // block-scaled activations keep their tile's scales behind the ring (reserved at their largest: kMaxBlockScaleDepth)
   constexpr size_t kShared = shared_bytes<BM, BN, MODE>() +
-                             (FORMAT == kFormatMxSplitBlocks || FORMAT == kFormatFp8Rows ? static_cast<size_t>(BM) * block_scale_pitch(kMaxBlockScaleDepth) : 0);
+                             (FORMAT == kFormatMxSplitBlocks || FORMAT == kFormatFp8Rows ? static_cast<size_t>(BM) * block_scale_pitch(kMaxBlockScaleDepth) : 0) +
+                             (FORMAT == kFormatMxFp8Rows ? 3 * static_cast<size_t>(BM) * 4 : 0);  // MXFP8 rows: a dword a row a stage
   auto kernel = grouped_gemm_kernel<FORMAT, MODE, BM, BN, WM, WN>;
   static bool configured = false;  // dynamic LDS above 64 KiB must be opted into once per kernel
   if (!configured) {
@@ -902,6 +956,8 @@ static int launch(const char* who, const GemmParams& p, int format, hipStream_t 
       return launch_format<DEW_MOE_W_FP8_CHANNEL, MODE>(who, p, stream);
     case DEW_MOE_W_MXFP4:
       return launch_format<DEW_MOE_W_MXFP4, MODE>(who, p, stream);
+    case DEW_MOE_W_MXFP8:
+      return fail(DEW_MOE_EINVAL, "%s: an MXFP8 bank multiplies MXFP8 rows (dew_moe_grouped_gemm_mxfp8_rows), not bf16 rows", who);
     default:
       return launch_format<DEW_MOE_W_NVFP4, MODE>(who, p, stream);
   }
@@ -1043,6 +1099,23 @@ extern "C" int dew_moe_grouped_gemm_fp8_rows(const void* x_codes, const uint8_t*
   p.a_scale = x_scales;
   if (p.width % 256 == 0) return launch_tile<kFormatFp8Rows, kPlain, 256, 256, 2, 2>(who, p, static_cast<hipStream_t>(stream));
   return launch_tile<kFormatFp8Rows, kPlain, 256, 128, 2, 2>(who, p, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int dew_moe_grouped_gemm_mxfp8_rows(const void* x_codes, const uint8_t* x_scales, const int32_t* gather,
+                                               const int32_t* offsets, const dew_moe_bank* w, const float* bias,
+                                               const int32_t* scatter, void* out, int32_t rows, void* stream) {
+  using namespace dew;
+  const char* who = "dew_moe_grouped_gemm_mxfp8_rows";
+  if (int rc = check_bank(who, w, "weight")) return rc;
+  DEW_REQUIRE(w->format == DEW_MOE_W_MXFP8, "%s: MXFP8 rows multiply an MXFP8 bank; this one is format %d", who, w->format);
+  DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
+  if (rows == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(x_scales && (reinterpret_cast<uintptr_t>(x_scales) & 3u) == 0, "%s: the rows' scales must not be null and must be 4-byte aligned", who);
+  GemmParams p{};
+  if (int rc = fill_single(who, p, x_codes, gather, offsets, w, bias, scatter, out, rows)) return rc;
+  p.a_scale = x_scales;
+  if (p.width % 256 == 0) return launch_tile<kFormatMxFp8Rows, kPlain, 256, 256, 2, 2>(who, p, static_cast<hipStream_t>(stream));
+  return launch_tile<kFormatMxFp8Rows, kPlain, 256, 128, 2, 2>(who, p, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int dew_moe_gateup_swiglu_split_out(const void* x_split, const uint8_t* x_scale, const int32_t* gather,

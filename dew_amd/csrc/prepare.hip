@@ -90,6 +90,30 @@ __global__ __launch_bounds__(256) void prepare_nvfp4_codes_kernel(const uint32_t
   }
 }
 
+// MXFP8 (K-major codes [E][N][K], scales [E][N][K / 32]): the same 32 n x 32 k atoms as the FP8 banks', a lane's 16
+// bytes contiguous in its column's row of the source; the scales as [E][N / 32][K / 128][32 columns][4 bytes], so that
+// a 32-column tile's scales of one 128-deep step are one 128-byte line.
+__global__ __launch_bounds__(256) void prepare_mxfp8_kernel(const uint8_t* __restrict__ codes, const uint8_t* __restrict__ scales,
+                                                            uint8_t* __restrict__ out, uint32_t* __restrict__ scales_out, int experts,
+                                                            int depth, int width) {
+  const int k_atoms = depth / 32, n_atoms = width / 32;
+  const long long total = static_cast<long long>(experts) * n_atoms * k_atoms * 64;
+  for (long long item = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; item < total;
+       item += static_cast<long long>(gridDim.x) * blockDim.x) {
+    const int lane = static_cast<int>(item % 64);
+    const long long atom = item / 64;
+    const int ka = static_cast<int>(atom % k_atoms);
+    const int na = static_cast<int>((atom / k_atoms) % n_atoms);
+    const int e = static_cast<int>(atom / (static_cast<long long>(k_atoms) * n_atoms));
+    const int n = na * 32 + lane % 32;
+    const size_t column = static_cast<size_t>(e) * width + n;
+    *reinterpret_cast<uint4*>(out + item * 16) = *reinterpret_cast<const uint4*>(codes + column * depth + ka * 32 + 16 * (lane / 32));
+    if (ka % 4 == 0 && lane < 32)  // the column's four scale bytes of this 128-deep step
+      scales_out[((static_cast<size_t>(e) * n_atoms + na) * (depth / 128) + ka / 4) * 32 + lane] =
+          *reinterpret_cast<const uint32_t*>(scales + column * (depth / 32) + ka);
+  }
+}
+
 // Also notes in *general whether any scale is not a normal power of two (mantissa bits set, or a zero or
 // subnormal exponent).
 __global__ __launch_bounds__(256) void prepare_nvfp4_scales_kernel(const uint8_t* __restrict__ scales,
@@ -122,6 +146,7 @@ extern "C" size_t dew_moe_prepared_bytes(int32_t format, int32_t experts, int32_
   if (experts <= 0 || depth <= 0 || width <= 0) return 0;
   size_t bytes = dew::codes_bytes(format, experts, depth, width);
   if (format == DEW_MOE_W_NVFP4) bytes += static_cast<size_t>(experts) * width * (depth / 16) + 256;  // + a flag word
+  if (format == DEW_MOE_W_MXFP8) bytes += static_cast<size_t>(experts) * width * (depth / 32);
   return bytes;
 }
 
@@ -129,7 +154,8 @@ extern "C" int dew_moe_prepare_bank(const dew_moe_bank* ref, void* prepared, dew
   using namespace dew;
   DEW_REQUIRE(ref && prepared && out, "dew_moe_prepare_bank: bank, prepared buffer and out must not be null");
   DEW_REQUIRE(ref->layout == DEW_MOE_LAYOUT_REFERENCE, "dew_moe_prepare_bank: the bank is already prepared");
-  DEW_REQUIRE(ref->format == DEW_MOE_W_FP8_BLOCK || ref->format == DEW_MOE_W_FP8_CHANNEL || ref->format == DEW_MOE_W_NVFP4,
+  DEW_REQUIRE(ref->format == DEW_MOE_W_FP8_BLOCK || ref->format == DEW_MOE_W_FP8_CHANNEL || ref->format == DEW_MOE_W_NVFP4 ||
+                  ref->format == DEW_MOE_W_MXFP8,
               "dew_moe_prepare_bank: unknown weight format %d", ref->format);
   DEW_REQUIRE(ref->experts >= 1 && ref->depth >= 1 && ref->width >= 1, "dew_moe_prepare_bank: bank [%d, %d, %d]",
               ref->experts, ref->depth, ref->width);
@@ -160,6 +186,16 @@ extern "C" int dew_moe_prepare_bank(const dew_moe_bank* ref, void* prepared, dew
     if (hipMemcpyAsync(&found, general, sizeof(found), hipMemcpyDeviceToHost, s) != hipSuccess || hipStreamSynchronize(s) != hipSuccess)
       return fail(DEW_MOE_ELAUNCH, "dew_moe_prepare_bank: reading the scale summary back failed: %s", hipGetErrorString(hipGetLastError()));
     if (!found) out->format = DEW_MOE_W_MXFP4;
+  } else if (ref->format == DEW_MOE_W_MXFP8) {
+    DEW_REQUIRE(ref->depth % 128 == 0, "dew_moe_prepare_bank: an MXFP8 bank's depth is whole 128s, not %d", ref->depth);
+    DEW_REQUIRE(aligned16(ref->codes) && (reinterpret_cast<uintptr_t>(ref->scales) & 3u) == 0,
+                "dew_moe_prepare_bank: MXFP8 codes must be 16-byte and scales 4-byte aligned");
+    uint8_t* scales_out = static_cast<uint8_t*>(prepared) + codes_bytes(ref->format, ref->experts, ref->depth, ref->width);
+    hipLaunchKernelGGL(prepare_mxfp8_kernel, dim3(grid), dim3(256), 0, s, static_cast<const uint8_t*>(ref->codes),
+                       static_cast<const uint8_t*>(ref->scales), static_cast<uint8_t*>(prepared), reinterpret_cast<uint32_t*>(scales_out),
+                       ref->experts, ref->depth, ref->width);
+    if (int rc = launched("prepare_mxfp8_kernel")) return rc;
+    out->scales = scales_out;
   } else {
     DEW_REQUIRE(ref->depth % 128 == 0, "dew_moe_prepare_bank: an FP8 bank's depth is whole 128s, not %d", ref->depth);
     hipLaunchKernelGGL(prepare_fp8_kernel, dim3(grid), dim3(256), 0, s, static_cast<const uint8_t*>(ref->codes),

@@ -196,6 +196,43 @@ class Fp8Channels:
 
 
 @dataclasses.dataclass(frozen=True)
+class MxFp8:
+    """An MXFP8 bank of matrices, K-major as a product reads them (the reference's `MxFp8` operand,
+    src/dew/nn/kernels/formats.py:186-194): e4m3 `codes [E, N, K]` (uint8) and one E8M0 `scales [E, N, K / 32]` byte
+    (uint8) every 32 depths, value = code * 2^(byte - 127). Standing for `W [E, K, N]`."""
+
+    codes: torch.Tensor
+    scales: torch.Tensor
+
+    @classmethod
+    def quantized(cls, weight: torch.Tensor) -> "MxFp8":
+        """`weight [E, K, N]` quantized along the depth by OCP MX's rule (`MxFp8.quantized`,
+        src/dew/nn/kernels/formats.py:195-229): each 32 depths' scale 2^(largest magnitude's exponent - 8), codes
+        rounded to e4m3, ties to even, saturating at +-448; a block of zeros takes the least scale."""
+        matrices = weight.to(torch.float32).transpose(1, 2).contiguous()      # [E, N, K]
+        experts, width, depth = matrices.shape
+        blocks = matrices.reshape(experts, width, depth // 32, 32)
+        largest = blocks.abs().amax(dim=-1, keepdim=True)
+        field = (largest.contiguous().view(torch.int32) >> 23) & 0xFF          # 0 for zero and subnormal magnitudes
+        byte = (field - 8).clamp(0, 254)
+        inverse = ((254 - byte) << 23).view(torch.float32)                     # 2^(127 - byte)
+        codes = (blocks * inverse).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8)
+        return cls(codes.reshape(experts, width, depth).contiguous(), byte[..., 0].to(torch.uint8).contiguous())
+
+    @property
+    def shape(self):
+        experts, width, depth = self.codes.shape
+        return (experts, depth, width)
+
+    @property
+    def dtype(self):
+        return torch.bfloat16
+
+    def to(self, device) -> "MxFp8":
+        return MxFp8(self.codes.to(device), self.scales.to(device))
+
+
+@dataclasses.dataclass(frozen=True)
 class Layered:
     """An expert kernel read in place from a run's stack (src/dew/nn/moe.py:595-606): `stack` the bank of every
     layer's experts along one axis (`[layers * E, K, N]`, any of the quantized formats or its prepared form) and

@@ -51,6 +51,7 @@ class GroupedCase:
 
 
 _BANKS = (formats.NvFp4, formats.Fp8Blocks, formats.Fp8Channels, formats.Layered, ops.PreparedBank)
+# (formats.MxFp8 multiplies MXFP8 rows only: projections.mxfp8_product)
 
 
 def _shape(bank):

@@ -170,7 +170,7 @@ class PreparedBank:
 
 
 def prepare(bank) -> PreparedBank:
-    """The one-time re-layout of a `formats.NvFp4`, `formats.Fp8Blocks` or `formats.Fp8Channels` bank."""
+    """The one-time re-layout of a `formats.NvFp4`, `formats.Fp8Blocks`, `formats.Fp8Channels` or `formats.MxFp8` bank."""
     if isinstance(bank, PreparedBank):
         return bank
     if isinstance(bank, formats.NvFp4):
@@ -184,6 +184,9 @@ def prepare(bank) -> PreparedBank:
     elif isinstance(bank, formats.Fp8Channels):
         fmt, codes, scales, tensor = _lib.W_FP8_CHANNEL, bank.codes, bank.scales, None
         _device(codes, "Fp8Channels.codes", torch.uint8), _device(scales, "Fp8Channels.scales", torch.float32)
+    elif isinstance(bank, formats.MxFp8):
+        fmt, codes, scales, tensor = _lib.W_MXFP8, bank.codes, bank.scales, None
+        _device(codes, "MxFp8.codes", torch.uint8), _device(scales, "MxFp8.scales", torch.uint8)
     else:
         raise KernelError(f"no HIP kernel multiplies a {type(bank).__name__} bank")
     experts, depth, width = bank.shape
@@ -426,6 +429,38 @@ def quantize_rows_fp8(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     _lib.check(_lib.library().dew_moe_quantize_rows_fp8(_ptr(x), _ptr(codes), _ptr(scales), rows, depth, _stream()),
                "dew_moe_quantize_rows_fp8")
     return codes, scales
+
+
+def quantize_rows_mxfp8(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """bf16 rows `[rows, K]` as MXFP8 (OCP MX: one E8M0 scale every 32 depths): (`codes` uint8 `[rows, K]`, each 128
+    depths in the scaled matrix instruction's operand order; `scales` uint8 `[rows, K / 32]` in depth order)."""
+    _device(x, "x", torch.bfloat16)
+    rows, depth = x.shape
+    codes = torch.empty((rows, depth), dtype=torch.uint8, device=x.device)
+    scales = torch.empty((rows, depth // 32), dtype=torch.uint8, device=x.device)
+    _lib.check(_lib.library().dew_moe_quantize_rows_mxfp8(_ptr(x), _ptr(codes), _ptr(scales), rows, depth, _stream()),
+               "dew_moe_quantize_rows_mxfp8")
+    return codes, scales
+
+
+def grouped_gemm_mxfp8_rows(codes: torch.Tensor, scales: torch.Tensor, bank: PreparedBank, offsets: torch.Tensor, *,
+                            gather: torch.Tensor | None = None, scatter: torch.Tensor | None = None, rows: int | None = None,
+                            bias: torch.Tensor | None = None) -> torch.Tensor:
+    """The MXFP8 recipe's product: `quantize_rows_mxfp8`'s rows times a prepared `formats.MxFp8` bank, every product of
+    (code x scale) values exact, fp32 sums, one rounding to bf16 `[rows, N]`."""
+    experts, depth, width = bank.shape
+    if codes.dtype != torch.uint8 or codes.shape[-1] != depth or scales.dtype != torch.uint8 or \
+            tuple(scales.shape) != (codes.shape[0], depth // 32) or not scales.is_contiguous():
+        raise KernelError(f"MXFP8 rows are uint8 [rows, {depth}] with uint8 scales [rows, {depth // 32}]")
+    if bank.descriptor.format != _lib.W_MXFP8:
+        raise KernelError("MXFP8 rows multiply an MXFP8 bank")
+    rows = (gather.numel() if gather is not None else codes.shape[0]) if rows is None else rows
+    bias = _expert_bias(bias, experts, width)
+    out = torch.empty((rows, width), dtype=torch.bfloat16, device=codes.device)
+    _lib.check(_lib.library().dew_moe_grouped_gemm_mxfp8_rows(_ptr(codes), _ptr(scales), _ptr(gather), _ptr(offsets), bank.descriptor,
+                                                              _ptr(bias), _ptr(scatter), _ptr(out), rows, _stream()),
+               "dew_moe_grouped_gemm_mxfp8_rows")
+    return out
 
 
 def operand_order_fp8(codes: torch.Tensor) -> torch.Tensor:

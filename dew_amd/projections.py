@@ -116,3 +116,47 @@ def recipe_projection(rows: torch.Tensor, matrix, group_sizes=None, *, out_dtype
     if bias is not None:
         bias = bias.reshape(bank.shape[0], bank.shape[2]).to(torch.float32).contiguous()  # widened as it is stored (:141)
     return blockwise_fp8_product(rows_quantized(rows), bank, group_sizes, out_dtype=out_dtype, bias=bias)
+
+
+# ---- the MXFP8 recipe (OCP MX) ---------------------------------------------------------------------------
+
+
+@dataclasses.dataclass(frozen=True)
+class MxFp8Rows:
+    """Rows as `ops.quantize_rows_mxfp8` writes them: `codes [rows, K]` uint8, each 128 depths in the scaled matrix
+    instruction's operand order, and `scales [rows, K / 32]` E8M0 bytes in depth order."""
+
+    codes: torch.Tensor
+    scales: torch.Tensor
+
+    def values(self) -> tuple[torch.Tensor, torch.Tensor]:
+        """(codes in depth order, scales): the reference's `MxFp8.quantized(x)` fields."""
+        return ops.depth_order_fp8(self.codes), self.scales
+
+
+def mxfp8_rows(x: torch.Tensor) -> MxFp8Rows:
+    """`MxFp8.quantized(x)` for rows `[rows, K]` bf16 (src/dew/nn/kernels/formats.py:195-229), on the device."""
+    return MxFp8Rows(*ops.quantize_rows_mxfp8(x.contiguous()))
+
+
+def mxfp8_product(lhs: MxFp8Rows, matrices, group_sizes, *, out_dtype=torch.bfloat16, bias=None, gather=None,
+                  scatter=None) -> torch.Tensor:
+    """Each group's MXFP8 rows times its matrix of the MXFP8 bank `matrices` (`formats.MxFp8`, or its prepared form):
+    every (code x scale) product exact, fp32 sums (+ `bias [groups, width]`), one rounding
+    (src/dew/nn/kernels/gemm.py:882-892, with its `gather`)."""
+    if out_dtype != torch.bfloat16:
+        raise ValueError(f"the launch writes bfloat16, not {out_dtype}")
+    bank = gemm.prepared(matrices)
+    rows = lhs.codes.shape[0] if gather is None else gather.numel()
+    return ops.grouped_gemm_mxfp8_rows(lhs.codes, lhs.scales, bank, _offsets(group_sizes, rows, lhs.codes.device),
+                                       gather=gather, scatter=scatter, bias=bias)
+
+
+def mxfp8_projection(x: torch.Tensor, w, group_blocks, *, out_dtype=torch.bfloat16) -> torch.Tensor:
+    """Each group's rows of `x [rows, depth]` times its matrix of `w [groups, depth, width]` in the MXFP8 recipe, both
+    quantized along the depth (src/dew/nn/kernels/projections.py:231-258); group `g` holds `group_blocks[g]` whole
+    128-row blocks. `w` is the weights (quantized here) or an MXFP8 bank already quantized."""
+    bank = w if isinstance(w, (formats.MxFp8, ops.PreparedBank)) else formats.MxFp8.quantized(w)
+    sizes = (torch.as_tensor(group_blocks, device=x.device).to(torch.int32) * SCALE_DEPTH).contiguous()
+    return mxfp8_product(mxfp8_rows(x), bank, sizes, out_dtype=out_dtype)
+

@@ -36,8 +36,11 @@ enum {
   DEW_MOE_W_NVFP4 = 3,       /* codes = NvFp4.words u32 [E,N,K/8] (staged order, GF(2)-encoded);        */
                              /* scales = NvFp4.scales e4m3 bytes [E,N,K/16]; tensor_scale f32 [E].      */
                              /* MXFP4 banks arrive in this form (codecs.mxfp4_as_nvfp4).                */
-  DEW_MOE_W_MXFP4 = 4        /* prepared banks only: an NVFP4 bank whose block scales are all powers of */
+  DEW_MOE_W_MXFP4 = 4,       /* prepared banks only: an NVFP4 bank whose block scales are all powers of */
                              /* two, as an MXFP4 checkpoint's are; dew_moe_prepare_bank finds it so.    */
+  DEW_MOE_W_MXFP8 = 5        /* OCP MXFP8, K-major as `formats.MxFp8` holds a product's matrices: codes */
+                             /* u8 e4m3 [E,N,K]; scales u8 e8m0 [E,N,K/32]. For dew_moe_grouped_gemm_   */
+                             /* mxfp8_rows only.                                                        */
 };
 
 enum { DEW_MOE_LAYOUT_REFERENCE = 0, DEW_MOE_LAYOUT_PREPARED = 1 };
@@ -188,6 +191,19 @@ int dew_moe_grouped_gemm_split_blocks(const void* x_split, const uint8_t* x_scal
  * scale x weight block scale (+ bias) ) for an FP8 128 x 128 block bank (prepared) whose scales are powers of two, as
  * the recipe's `blocks_quantized` makes them: both operands enter v_mfma_scale_f32_32x32x64_f8f6f4 as stored. A weight
  * block scale that is no normal power of two makes the tiles that meet it NaN. K up to 24576, rows in 256-row tiles. */
+/* The MXFP8 recipe's forward product (OCP MX: e4m3 codes, one power-of-two E8M0 scale every 32 depths of both
+ * operands): `MxFp8.quantized` src/dew/nn/kernels/formats.py:186-229 and `mxfp8_product`
+ * src/dew/nn/kernels/gemm.py:882-892. dew_moe_quantize_rows_mxfp8: x bf16 [rows, K] -> codes [rows, K] bytes in the
+ * operand order of dew_moe_quantize_rows_fp8 and scales [rows, K / 32] E8M0 bytes in depth order (scale = 2^(largest
+ * magnitude's exponent - 8), byte 0 for a block of zeros; codes saturate at +-448). dew_moe_grouped_gemm_mxfp8_rows:
+ * out[scatter[i]] = bf16( sum of exact (code x scale) products (+ bias) ) with a DEW_MOE_W_MXFP8 bank (prepared):
+ * v_mfma_scale_f32_32x32x64_f8f6f4 takes the codes and the per-32 scales of both operands as they are stored, which
+ * is the instruction's own format. K whole 128s, N whole 128s, rows in 256-row tiles.                           */
+int dew_moe_quantize_rows_mxfp8(const void* x /* bf16 [rows, K] */, void* codes /* [rows, K] bytes */,
+                                uint8_t* scales /* [rows, K / 32] e8m0 */, int32_t rows, int32_t depth, void* stream);
+int dew_moe_grouped_gemm_mxfp8_rows(const void* x_codes, const uint8_t* x_scales, const int32_t* gather,
+                                    const int32_t* offsets, const dew_moe_bank* w, const float* bias,
+                                    const int32_t* scatter, void* out, int32_t rows, void* stream);
 int dew_moe_quantize_rows_fp8(const void* x /* bf16 [rows, K] */, void* codes /* [rows, K] bytes */,
                               uint8_t* scales /* [rows, P] e8m0 */, int32_t rows, int32_t depth, void* stream);
 int dew_moe_grouped_gemm_fp8_rows(const void* x_codes, const uint8_t* x_scales, const int32_t* gather,

@@ -37,6 +37,11 @@ What pins each function (tests/test_oracle_golden.py):
   agree (they differ only in how amax / 448 is rounded before the ceiling), and the product against the float64
   sum of the dequantized operands at the reference's own bound.
 
+* `mxfp8_quantized` / `mxfp8_product` (the MXFP8 recipe): OCP MX's rule as the reference states it, pinned by its
+  invariants (a block's largest magnitude over its scale in [256, 512), so its code is 256 .. 448; 448 .. 512
+  saturates; a zero block takes byte 0; the scale byte is the largest magnitude's fp32 exponent field less 8) and
+  by the decoded operands reproducing the source within half a code step.
+
 Parity unpinned (no byte fixture in the reference, closed form only): the exact bits of the softmax
 denominator's compensated sum (src/dew/nn/precision.py:1832); it moves router weights by at most one fp32
 ulp and no index. `gpt_oss_gating`'s bf16 mode: where each bf16 rounding falls follows JAX's arithmetic on
@@ -521,6 +526,63 @@ def blockwise_fp8_projection(x, w, group_sizes, *, dtype="bfloat16", bias=None):
     rows, rows_scales = rows_quantized(x)
     blocks, blocks_scales = blocks_quantized(w)
     return blockwise_fp8_product(rows, blocks, group_sizes, rows_scales.T, blocks_scales, dtype=dtype, bias=bias)
+
+
+# --------------------------------------------------------------------------------------------------
+# The MXFP8 recipe's forward product (OCP MX: E4M3 codes, a power-of-two E8M0 scale every 32 depths)
+# --------------------------------------------------------------------------------------------------
+
+MX_DEPTH = 32
+
+
+def mxfp8_quantized(x):
+    """`x [..., depth]` as MXFP8 by OCP MX's rule (src/dew/nn/kernels/formats.py:195-229): each 32 depths' scale 2
+    to the power of its largest magnitude's binary exponent less 8, so that the magnitude over the scale lies in
+    [256, 512); each value over its scale rounded to E4M3, ties to even, saturating at +-448; a block of zeros
+    takes the least scale 2^-127; exponents clipped to +-127. Returns (E4M3 values `[..., depth]`, E8M0 bytes
+    `[..., depth / 32]`: scale = 2^(byte - 127))."""
+    x = np.asarray(x, F32)
+    blocks = x.reshape(*x.shape[:-1], x.shape[-1] // MX_DEPTH, MX_DEPTH)
+    largest = np.abs(blocks).max(axis=-1, keepdims=True)
+    binade = np.frexp(largest)[1]
+    exponent = np.clip(np.where(largest > 0, binade - 1 - 8, -127), -127, 127).astype(np.int32)
+    scaled = np.ldexp(blocks.astype(np.float64), -exponent).astype(F32)  # exact: a power of two, within fp32's range
+    return fp8_codes(scaled).reshape(x.shape), (exponent[..., 0] + 127).astype(np.uint8)
+
+
+def mxfp8_decoded(values, scales):
+    """src/dew/nn/kernels/formats.py:231-243: each E4M3 value times its block's scale 2^(byte - 127), in float64
+    (exact)."""
+    exponents = np.repeat(np.asarray(scales).astype(np.int32) - 127, MX_DEPTH, axis=-1)
+    return np.ldexp(np.asarray(values, np.float64), exponents)
+
+
+def mxfp8_product(lhs, lhs_scales, matrices, matrix_scales, group_sizes, *, dtype="bfloat16", bias=None):
+    """Each group's rows of `lhs [rows, depth]` times its matrix of `matrices [groups, width, depth]` (K-major), both
+    MXFP8: each value its code times its 32 depths' scale, every product exact, summed in fp32 and rounded once
+    (src/dew/nn/kernels/gemm.py:882-892); rows past the groups zero. The sum is formed exactly (float64) and
+    rounded to fp32, which any order of fp32 additions reaches to a few ulps."""
+    left = mxfp8_decoded(lhs, lhs_scales)
+    right = mxfp8_decoded(matrices, matrix_scales)
+    rows, width = left.shape[0], right.shape[1]
+    total = np.zeros((rows, width), F32)
+    start = 0
+    for group, size in enumerate(np.asarray(group_sizes).tolist()):
+        if size:
+            summed = (left[start:start + size] @ right[group].T).astype(F32)
+            if bias is not None:
+                summed = summed + np.asarray(bias, F32)[group][None, :]
+            total[start:start + size] = summed
+        start += size
+    return bf16_round(total) if dtype == "bfloat16" else total
+
+
+def mxfp8_projection(x, w, group_sizes, *, dtype="bfloat16", bias=None):
+    """`x [rows, depth]` and `w [groups, depth, width]` both quantized along the depth, their `mxfp8_product`
+    (src/dew/nn/kernels/projections.py:231-258)."""
+    rows, row_scales = mxfp8_quantized(x)
+    matrices, matrix_scales = mxfp8_quantized(np.swapaxes(np.asarray(w, F32), 1, 2))
+    return mxfp8_product(rows, row_scales, matrices, matrix_scales, group_sizes, dtype=dtype, bias=bias)
 
 
 def swiglu(gate, up, *, dtype="bfloat16", limit=None, exp=np.exp):

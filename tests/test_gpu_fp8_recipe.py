@@ -142,3 +142,74 @@ def test_a_block_scale_that_is_no_power_of_two_is_not_multiplied_silently(ops):
     spoiled = formats.Fp8Blocks(bank.codes, scales).to("cuda")
     got = bf16_np(projections.recipe_projection(x.cuda(), spoiled, torch.tensor([40], dtype=torch.int32).cuda()))
     assert np.isnan(got[:, 128:]).all() and np.isfinite(got[:, :128]).all()
+
+
+# ---- the MXFP8 recipe -----------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("rows,depth", [(7, 128), (33, 384), (260, 4096)])
+def test_mxfp8_rows_are_quantized_bit_for_bit(ops, rows, depth):
+    x = rows_case(rows, depth, seed=rows + 1)
+    codes, scales = ops.quantize_rows_mxfp8(x.cuda())
+    want_values, want_scales = oracle.mxfp8_quantized(bf16_np(x))
+    assert np.array_equal(scales.cpu().numpy(), want_scales)
+    assert np.array_equal(ops.depth_order_fp8(codes).cpu().numpy(), oracle.e4m3_bytes(want_values))
+
+
+@pytest.mark.parametrize("label,sizes", SIZES, ids=[s[0] for s in SIZES])
+@pytest.mark.parametrize("depth,width", [(256, 128), (1152, 384), (512, 512)])
+def test_the_mxfp8_product_matches_the_oracle(ops, label, sizes, depth, width):
+    """Every scale differs by row, column and 32-deep block here, so a lane that handed the instruction another
+    block's or another row's scale would be off by powers of two."""
+    from dew_amd import formats, projections
+
+    groups, rows = len(sizes), int(np.sum(sizes))
+    rng = np.random.default_rng(depth + rows + 1)
+    spread = np.exp2(rng.integers(-6, 7, size=(rows + 6, depth // 32))).repeat(32, axis=1)
+    x = torch.from_numpy((rng.standard_normal((rows + 6, depth)) * spread).astype(np.float32)).to(torch.bfloat16)
+    w = weights_case(groups, depth, width, seed=depth + 1) * np.exp2(rng.integers(-4, 5, size=(groups, depth // 32, width))).repeat(32, axis=1)
+    w = w.astype(np.float32)
+    bias = torch.from_numpy(rng.standard_normal((groups, width)).astype(np.float32) * 0.1)
+    sizes_device = torch.tensor(sizes, dtype=torch.int32).cuda()
+    bank = formats.MxFp8.quantized(torch.from_numpy(w)).to("cuda")
+    quantized = projections.mxfp8_rows(x.cuda())
+    for with_bias in (None, bias):
+        got = bf16_np(projections.mxfp8_product(quantized, bank, sizes_device, bias=None if with_bias is None else with_bias.cuda()))
+        want = oracle.mxfp8_projection(bf16_np(x), w, sizes, bias=None if with_bias is None else with_bias.numpy())
+        assert np.all(got[rows:] == 0) and np.all(want[rows:] == 0)
+        scale = np.abs(want).max()
+        assert np.abs(got - want).max() <= 2.0 ** -7 * scale
+        assert (got == want).mean() > 0.97
+
+
+def test_mxfp8_gathered_rows_scattered_outputs_and_whole_blocks(ops):
+    from dew_amd import formats, projections
+
+    sizes, depth, width = [200, 56, 300], 512, 256
+    rows = sum(sizes)
+    rng = np.random.default_rng(19)
+    x = torch.from_numpy(rng.standard_normal((400, depth)).astype(np.float32)).to(torch.bfloat16)
+    gather = rng.integers(0, 400, size=rows).astype(np.int32)
+    scatter = rng.permutation(rows).astype(np.int32)
+    w = weights_case(len(sizes), depth, width, seed=14)
+    bank = formats.MxFp8.quantized(torch.from_numpy(w)).to("cuda")
+    got = bf16_np(projections.mxfp8_product(projections.mxfp8_rows(x.cuda()), bank, torch.tensor(sizes, dtype=torch.int32).cuda(),
+                                            gather=torch.from_numpy(gather).cuda(), scatter=torch.from_numpy(scatter).cuda()))
+    want = oracle.mxfp8_projection(bf16_np(x)[gather], w, sizes)
+    placed = np.zeros_like(want)
+    placed[scatter] = want
+    assert np.abs(got - placed).max() <= 2.0 ** -7 * np.abs(want).max() and (got == placed).mean() > 0.97
+    blocks = [2, 0, 1]
+    x = torch.from_numpy(rng.standard_normal((384, depth)).astype(np.float32)).to(torch.bfloat16)
+    got = bf16_np(projections.mxfp8_projection(x.cuda(), torch.from_numpy(w).cuda(), blocks))
+    want = oracle.mxfp8_projection(bf16_np(x), w, [256, 0, 128])
+    assert np.abs(got - want).max() <= 2.0 ** -7 * np.abs(want).max() and (got == want).mean() > 0.97
+
+
+def test_an_mxfp8_bank_is_refused_by_the_bf16_products(ops):
+    from dew_amd import formats
+
+    bank = ops.prepare(formats.MxFp8.quantized(torch.from_numpy(weights_case(1, 256, 128, seed=2))).to("cuda"))
+    x = torch.zeros((8, 256), dtype=torch.bfloat16).cuda()
+    with pytest.raises(Exception, match="MXFP8"):
+        ops.grouped_gemm(x, bank, torch.tensor([0, 8], dtype=torch.int32).cuda())

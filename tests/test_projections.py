@@ -113,3 +113,38 @@ def test_shapes_without_whole_blocks_are_left_to_the_caller():
     from dew_amd import projections
 
     assert projections.recipe_projection(torch.zeros((4, 192), dtype=torch.bfloat16), torch.zeros((192, 128))) is None
+
+
+def test_mxfp8_quantizes_by_the_ocp_rule():
+    """A block's largest magnitude over its scale lies in [256, 512), so its code is 256 .. 448 (448 .. 512 saturates);
+    the scale byte is that magnitude's fp32 exponent field less 8; zeros and magnitudes under 2^-119 take byte 0."""
+    rng = np.random.default_rng(7)
+    x = (rng.standard_normal((64, 256)) * rng.choice([1e-4, 1.0, 3e4], size=(64, 1))).astype(np.float32)
+    x[0, :32] = 0.0
+    x[1, :32] = np.float32(2.0 ** -130)
+    x[2, :32] = 0.0
+    x[2, 5] = 511.0                                   # 511 / 2 = 255.5 -> code 256; under its own scale 2^0 it would saturate
+    x[3, :32] = 0.0
+    x[3, 7] = -480.0                                  # scale 2^0: -480 saturates to -448
+    values, scales = oracle.mxfp8_quantized(x)
+    top = np.abs(values).reshape(64, 8, 32).max(axis=2)
+    nonzero = np.abs(x).reshape(64, 8, 32).max(axis=2) >= 2.0 ** -118
+    assert ((top >= 256) & (top <= 448))[nonzero].all()
+    field = (np.abs(x).reshape(64, 8, 32).max(axis=2).astype(np.float32).view(np.uint32) >> 23).astype(np.int32)
+    assert np.array_equal(scales, np.clip(field - 8, 0, 254).astype(np.uint8))
+    assert scales[0, 0] == 0 and values[0, :32].max() == 0 and scales[1, 0] == 0 and values[1, 0] == 0.125
+    assert scales[2, 0] == 127 and values[2, 5] == 448.0 and scales[3, 0] == 127 and values[3, 7] == -448.0
+    decoded = oracle.mxfp8_decoded(values, scales)
+    unsaturated = np.abs(values) < 448
+    assert (np.abs(decoded - x)[unsaturated] <= np.repeat(np.ldexp(1.0, scales.astype(np.int32) - 127 + 4), 32, axis=1)[unsaturated]).all()
+
+
+def test_the_host_mirror_quantizes_an_mxfp8_bank_as_the_oracle_does():
+    from dew_amd import formats
+
+    w = weights_case(2, 256, 128, seed=3)
+    bank = formats.MxFp8.quantized(torch.from_numpy(w))
+    want_values, want_scales = oracle.mxfp8_quantized(np.swapaxes(w, 1, 2))
+    assert bank.shape == (2, 256, 128)
+    assert np.array_equal(bank.scales.numpy(), want_scales)
+    assert np.array_equal(bank.codes.numpy(), oracle.e4m3_bytes(want_values))
