@@ -47,8 +47,9 @@ const char* dew_moe_kernels(void) {
          "grouped_gemm<decode>,32,128 (paired 2x128),64,4 (1x4),v_mfma_f32_32x32x16_bf16,weight streaming for groups under 24 rows\n"
          "grouped_gemm epilogues,-,-,-,-,-,plain (+bias) | swiglu of two banks | interleaved gate/up clamped 1.702 gating (+bias); tile staged in LDS and stored as whole rows\n"
          "grouped_gemm<split rows>,256,256 (paired 2x128),64,4 (2x2),v_mfma_scale_f32_32x32x64_f8f6f4,two e4m3 terms per bf16 activation x mxfp4 codes as stored; SwiGLU rows written already split\n"
-         "grouped_gemm<fp8 rows>,256,128,128,4 (2x2),v_mfma_scale_f32_32x32x64_f8f6f4,e4m3 rows (1x128 power-of-two scales) x fp8 128x128 blocks (power-of-two scales)\n"
-         "split_rows | quantize_rows_fp8,1 row/wave,-,-,4,-,bf16 rows -> e4m3 terms | e4m3 codes in operand order + e8m0 scales\n"
+         "grouped_gemm<fp8 rows>,256,256 | 128,128,4 (2x2),v_mfma_scale_f32_32x32x64_f8f6f4,e4m3 rows (1x128 power-of-two scales) x fp8 128x128 blocks (power-of-two scales)\n"
+         "grouped_gemm<mxfp8 rows>,256,256,128,4 (2x2),v_mfma_scale_f32_32x32x64_f8f6f4,OCP MXFP8 rows x MXFP8 bank: e4m3 codes and E8M0 scales per 32 depths of both operands as stored\n"
+         "split_rows | quantize_rows_fp8 | quantize_rows_mxfp8,1 row/wave,-,-,4,-,bf16 rows -> e4m3 terms | e4m3 codes in operand order + e8m0 scales\n"
          "combine,8 columns/lane,-,-,4,-,bf16 slots x f32 weights\n";
 }
 
