@@ -604,13 +604,14 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
       constexpr std::integral_constant<int, kWeightsFirst ? 0 : kRowLoads / 2> ah{};
       constexpr std::integral_constant<int, kWeightsFirst ? kTiles : kTiles / 2> bh{};
       constexpr int kSplitMfmas = kMatrices * TI * TJ;
-      constexpr int kSplitLoads = ah.value + bh.value * kLoadsPerTile;  // the first phase's, the younger ones at the barrier
+      constexpr int kSplitLoads = ah.value + bh.value * kLoadsPerTile + (kMxRows ? 1 : 0);  // the first phase's, the younger ones at the barrier
       static_assert(kRowLoads % 2 == 0 && kTiles % 2 == 0, "two even halves of loads");
       // younger than the last A load of the step before: only this phase's loads are sure to be
       constexpr int kSplitWait = (kSplitLoads & 0xF) | (7 << 4) | (0 << 8) | ((kSplitLoads >> 4) << 14);
       fetch_term(current, c1);
       multiply_term(set, c0, step);
       load_a(fill, ahead_a, c0, ah);
+      load_a_scales(fill_index, ahead_a);  // (MXFP8 rows: the step's scale dwords, with this phase's loads)
       load_b(filling, ahead_b, c0, bh);
       schedule_phase<0, kSplitMfmas, 2 * TI, 0, 2 * kTiles + 2 * kSplitLoads, kSplitLoads>();
       __builtin_amdgcn_sched_barrier(0);
@@ -623,7 +624,6 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
       // and formed into words in the second phase of the odd step that follows, one phase before they multiply
       if constexpr (kMxRows) {
         fetch_a_scales(std::integral_constant<int, 1 - set.value % 2>{}, next_index);  // the next step's, landed before the barrier
-        load_a_scales(fill_index, ahead_a);
       } else if constexpr (kFp8Rows) {  // a step is the 128 depths of one scale: the next step's, into the other set
         load_block_scales(min(step + 1, steps - 1));
         form_block_words(std::integral_constant<int, 1 - set.value % 2>{});
@@ -635,7 +635,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
       multiply_term(set, c1, step);
       load_a(fill, ahead_a, ah, a4);
       load_b(filling, ahead_b, bh, b4);
-      constexpr int kSecondLoads = kRowLoads - ah.value + (kTiles - bh.value) * kLoadsPerTile + (kMxRows ? 1 : 0);
+      constexpr int kSecondLoads = kRowLoads - ah.value + (kTiles - bh.value) * kLoadsPerTile;
       schedule_phase<0, kSplitMfmas, 2 * TI, 0, 2 * kTiles + 2 * kSecondLoads, kSecondLoads>();
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (kWeightsFirst) {
