@@ -110,7 +110,7 @@ class Stepper:
         """The routed experts' two launches: [T * k, D] rows at their slots. `events` bracket the gate/up launch."""
         ops, data = self.ops, self.data
         if self.on_split_rows():
-            # MXFP4 banks and groups of a thousand rows: the rows as two e4m3 terms and the scaled matrix instruction;
+            # MXFP4 banks and groups of hundreds of rows: the rows as two e4m3 terms and the scaled matrix instruction;
             # the gate/up launch writes its hidden rows already split, so the only extra pass is the split of x
             pieces = ops.split_rows(data["x"])
             if events:
@@ -225,7 +225,7 @@ def main():
                         help="only run the plain copy probe (1 GiB read + 1 GiB written, 5 launches): the known traffic "
                              "that rocprofv3's FETCH_SIZE / WRITE_SIZE are scaled by")
     parser.add_argument("--bf16-operands", action="store_true",
-                        help="keep MXFP4 banks with groups of a thousand rows on the bf16 matrix instruction too (the default "
+                        help="keep MXFP4 banks with groups of hundreds of rows on the bf16 matrix instruction too (the default "
                              "there: rows split into two e4m3 terms and the scaled instruction, the library's own choice)")
     parser.add_argument("--graph", choices=["auto", "on", "off"], default="auto",
                         help="replay the step as one captured HIP graph (auto: for the launch-bound configs c1 and c3)")

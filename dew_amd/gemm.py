@@ -104,7 +104,7 @@ names are refused as unlowerable."""
 
 
 SPLIT_ROWS = True
-"""Whether an expert MLP of MXFP4 banks with groups of a thousand rows or more runs on rows split into two e4m3
+"""Whether an expert MLP of MXFP4 banks with groups of 384 rows or more (`ops.prefers_split`) runs on rows split into two e4m3
 terms and the scaled matrix instruction (`swiglu_mlp_on_split_rows`). The products are the same exact ones (an
 element loses bits only below 2^-11 of the largest of its 128 neighbours); measured on 16384 tokens of
 4096 -> 14336 -> 4096 over 8 experts the two launches take 5.45 + 2.48 ms against 5.75 + 2.54 ms on bf16
