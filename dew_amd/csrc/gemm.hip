@@ -78,6 +78,11 @@ struct GemmParams {
   const float* bias;  // [experts, width] values of the compute dtype held in fp32, or null
   float limit;        // the interleaved gated epilogue's clamp
   int experts, depth, width, rows, m_tile_bound;
+  // A launch normally multiplies every group in tiles of its BM rows, the last of a group partly empty. Where that
+  // waste matters two launches share the groups: the taller tiles' launch leaves (skip_tails) a last tile that would
+  // hold at most BM / 2 rows to a launch of tiles half as tall, which multiplies (tail_of = the taller tile's rows)
+  // only those last rows, the ones past a group's whole tiles of tail_of rows where they are at most its own BM.
+  int skip_tails, tail_of;
 };
 
 // What the epilogue writes: the rounded product (plus bias); SwiGLU of two banks' products; for one bank whose
@@ -234,7 +239,14 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     int start = 0, tiles = 0;
     if (e < p.experts) {
       start = p.offsets[e];
-      tiles = (p.offsets[e + 1] - start + BM - 1) / BM;
+      const int size = p.offsets[e + 1] - start;
+      if (p.tail_of > 0) {
+        const int rest = size % p.tail_of;
+        tiles = rest >= 1 && rest <= BM ? 1 : 0;
+        start += size - rest;
+      } else {
+        tiles = size / BM + (size % BM > (p.skip_tails ? BM / 2 : 0) ? 1 : 0);
+      }
     }
     int inclusive = tiles;
 #pragma unroll
@@ -259,6 +271,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   const int expert = found[0];
 
   if (expert < 0) {
+    if (p.tail_of > 0) return;  // (the taller tiles' launch zeroes them)
     // Past the last real tile: zero the rows no expert owns (sorted positions offsets[E] .. rows).
     const int tail_begin = p.offsets[p.experts] + (m_tile - found[2]) * BM;
     const int tail_end = min(tail_begin + BM, p.rows);
@@ -897,7 +910,7 @@ static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
     configured = true;
   }
   // every expert may end in a partial tile, and the zeroed tail may add one more
-  p.m_tile_bound = (p.rows + BM - 1) / BM + p.experts + 1;
+  p.m_tile_bound = p.tail_of > 0 ? p.experts : (p.rows + BM - 1) / BM + p.experts + 1;
   const int total = p.m_tile_bound * (p.width / BN);
   const int blocks = ((total + 255) / 256) * 256;  // whole chunks of 32 tiles for each of the 8 XCDs
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreads), kShared, stream, p);
@@ -940,10 +953,23 @@ static int launch_format(const char* who, const GemmParams& p, hipStream_t strea
     case 256:
       if (kPaired || p.width % 256 == 0) return launch_tile<FORMAT, MODE, 256, kPaired ? 128 : 256, 1, 4>(who, p, stream);
       [[fallthrough]];  // one bank whose width is not whole 256s: the 128-row tile
-    default:
+    default: {
+      // Groups of a few hundred rows end in a 128-row tile that is half empty on average. With enough groups and
+      // strips for a launch of their own (256 tiles), last tiles of at most 64 rows go to the 64-row tile: measured on
+      // 256 groups of 256 +- 16 rows, 2.5 tiles a group become 2 and a 64-row one.
+      const bool shared = forced_tile_rows == 0 && static_cast<long long>(p.experts) * (p.width / 128) >= 256;
+      GemmParams taller = p;
+      taller.skip_tails = shared ? 1 : 0;
+      int status;
       if (!kPaired && p.width % 256 == 0 && static_cast<long long>(p.rows / 128 + 1) * (p.width / 256) >= 512)
-        return launch_tile<FORMAT, MODE, 128, 256, 1, 4>(who, p, stream);  // enough tiles to fill the chip twice over
-      return launch_tile<FORMAT, MODE, 128, 128, 1, 4>(who, p, stream);
+        status = launch_tile<FORMAT, MODE, 128, 256, 1, 4>(who, taller, stream);  // enough tiles to fill the chip twice over
+      else
+        status = launch_tile<FORMAT, MODE, 128, 128, 1, 4>(who, taller, stream);
+      if (status != DEW_MOE_OK || !shared) return status;
+      GemmParams rest = p;
+      rest.tail_of = 128;
+      return launch_tile<FORMAT, MODE, 64, 128, 1, 4>(who, rest, stream);
+    }
   }
 }
 

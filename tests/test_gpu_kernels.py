@@ -410,3 +410,35 @@ def test_a_layer_of_a_stacked_bank_is_read_where_it_lies(ops, quant):
         assert torch.equal(through, alone)
     with pytest.raises(Exception):
         stack.layer(3, layers)
+
+
+@pytest.mark.parametrize("quant", ["fp8_block", "fp8_channel", "mxfp4", "nvfp4"])
+def test_last_tiles_of_at_most_64_rows_go_to_a_launch_of_their_own(ops, quant):
+    """With 32 groups over 8 strips the 128-row tiles' launch leaves each group's last rows, where they are at most
+    64, to a launch of 64-row tiles: every remainder from none to a full tile, both products and the paired one, are
+    the single launch's bit for bit (a row's sum does not depend on the tile it sits in), and rows past the groups
+    are zero."""
+    remainders = [0, 1, 2, 31, 63, 64, 65, 100, 127, 128, 129, 192, 193, 255, 256, 257]
+    sizes = [remainders[i % 16] + 128 * (i % 3) for i in range(32)]
+    depth, width = 256, 1024
+    bank, x, offsets = grouped_case(quant, len(sizes), depth, width, sizes, seed=41)
+    up, _, _ = grouped_case(quant, len(sizes), depth, width, sizes, seed=42)
+    rows = int(np.sum(sizes))
+    rng = np.random.default_rng(5)
+    padded = rows + 37
+    gather = np.concatenate([rng.integers(0, rows, size=rows), np.zeros(37)]).astype(np.int32)
+    scatter = rng.permutation(padded).astype(np.int32)
+    xd, od = x.cuda(), torch.from_numpy(offsets).cuda()
+    gd, sd = torch.from_numpy(gather).cuda(), torch.from_numpy(scatter).cuda()
+    pb, pu = ops.prepare(bank.to("cuda")), ops.prepare(up.to("cuda"))
+    shared = ops.grouped_gemm(xd, pb, od, gather=gd, scatter=sd, rows=padded)
+    hidden = ops.gateup_swiglu(xd, pb, pu, od, gather=gd, rows=padded)
+    with ops.tile_rows(128):
+        single = ops.grouped_gemm(xd, pb, od, gather=gd, scatter=sd, rows=padded)
+        single_hidden = ops.gateup_swiglu(xd, pb, pu, od, gather=gd, rows=padded)
+    assert torch.equal(shared, single) and torch.equal(hidden, single_hidden)
+    values, factor = dequantized(bank)
+    want = oracle.grouped_matmul(bf16_np(x)[gather[:rows]], values, sizes, factor=factor)
+    got = bf16_np(shared)
+    assert np.all(got[scatter[rows:]] == 0)
+    assert np.abs(got[scatter[:rows]] - want).max() <= 2 ** -7 * np.abs(want).max()
