@@ -98,7 +98,105 @@ __global__ __launch_bounds__(64 * kQuantizeWaves) void quantize_rows_mxfp8_kerne
   }
 }
 
+// The NVFP4 recipe's rows (reference src/dew/nn/kernels/formats.py:263-274 over src/dew/algebra/bits.py:941-982):
+// E2M1 codes under an E4M3 scale every 16 depths and one tensor scale over the whole operand. The scaled matrix
+// instruction takes power-of-two scales of 32 depths only, so this operand goes to the bf16 instruction: each value is
+// written as what it stands for short of the tensor scale, code x block scale, which bf16 holds exactly (5 significant
+// bits), and the product applies the tensor scale to its fp32 sums with the bank's.
+// Two passes, because the tensor scale needs the whole operand's largest magnitude first.
+__global__ __launch_bounds__(256) void absmax_clear_kernel(uint32_t* __restrict__ largest) { *largest = 0u; }
+
+__global__ __launch_bounds__(256) void absmax_kernel(const bf16_t* __restrict__ x, long long chunks, uint32_t* __restrict__ largest) {
+  uint32_t mine = 0;  // magnitudes of bf16 values order as their bit patterns do
+  for (long long chunk = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; chunk < chunks;
+       chunk += static_cast<long long>(gridDim.x) * blockDim.x) {
+    const u32x4_t words = reinterpret_cast<const u32x4_t*>(x)[chunk];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) mine = max(mine, max(words[i] & 0x7FFFu, (words[i] >> 16) & 0x7FFFu));
+  }
+#pragma unroll
+  for (int offset = 32; offset >= 1; offset >>= 1) mine = max(mine, static_cast<uint32_t>(__shfl_xor(static_cast<int>(mine), offset, 64)));
+  if (threadIdx.x % 64 == 0 && mine != 0) atomicMax(largest, mine);
+}
+
+__device__ __forceinline__ float e2m1_nearest(float magnitude) {
+  // ties to the even code: 0.25 -> 0, 0.75 -> 1, 1.25 -> 1, 1.75 -> 2, 2.5 -> 2, 3.5 -> 4, 5 -> 4
+  float value = magnitude > 0.25f ? 0.5f : 0.0f;
+  value = magnitude >= 0.75f ? 1.0f : value;
+  value = magnitude > 1.25f ? 1.5f : value;
+  value = magnitude >= 1.75f ? 2.0f : value;
+  value = magnitude > 2.5f ? 3.0f : value;
+  value = magnitude >= 3.5f ? 4.0f : value;
+  return magnitude > 5.0f ? 6.0f : value;
+}
+
+__global__ __launch_bounds__(64 * kQuantizeWaves) void quantize_rows_nvfp4_kernel(const bf16_t* __restrict__ x, const uint32_t* __restrict__ largest,
+                                                                                bf16_t* __restrict__ out, float* __restrict__ tensor_scale,
+                                                                                int rows, int depth) {
+  const float top = __uint_as_float(*largest << 16);
+  // largest / (6 * 448), fp32's least normal at least; 1 for an operand of zeros
+  const float tensor = top > 0.0f ? fmaxf(top / 2688.0f, 1.17549435e-38f) : 1.0f;
+  if (blockIdx.x == 0 && threadIdx.x == 0) *tensor_scale = tensor;
+  const int lane = threadIdx.x % 64;
+  const int row = blockIdx.x * kQuantizeWaves + threadIdx.x / 64;
+  if (row >= rows) return;
+  const bf16_t* source = x + static_cast<size_t>(row) * depth;
+  bf16_t* target = out + static_cast<size_t>(row) * depth;
+  for (int chunk = lane; chunk < depth / 8; chunk += 64) {  // 8 depths a lane, 2 lanes a block of 16
+    const u32x4_t words = *reinterpret_cast<const u32x4_t*>(source + chunk * 8);
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = __uint_as_float(words[i] << 16);
+      v[2 * i + 1] = __uint_as_float(words[i] & 0xFFFF0000u);
+    }
+    float block = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) block = fmaxf(block, fabsf(v[i]));
+    block = fmaxf(block, __shfl_xor(block, 1, 64));
+    // the least e4m3 at or above blockmax / tensor / 6: the nearest one, and the next where that lies below
+    const float ratio = (block / tensor) / 6.0f;
+    uint32_t byte = __builtin_amdgcn_cvt_pk_fp8_f32(fminf(ratio, 448.0f), 0.0f, 0, false) & 0xFFu;
+    if (__builtin_amdgcn_cvt_f32_fp8(byte, 0) < ratio) byte = min(byte + 1u, 0x7Eu);
+    const float each = __builtin_amdgcn_cvt_f32_fp8(byte, 0);
+    u32x4_t packed;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float pair[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const float source_value = v[2 * i + h];
+        const float quotient = each > 0.0f ? (source_value / tensor) / each : 0.0f;
+        pair[h] = copysignf(e2m1_nearest(fabsf(quotient)) * each, quotient);  // code x block scale: exact in bf16
+      }
+      packed[i] = (__float_as_uint(pair[0]) >> 16) | (__float_as_uint(pair[1]) & 0xFFFF0000u);
+    }
+    *reinterpret_cast<u32x4_t*>(target + chunk * 8) = packed;
+  }
+}
+
 }  // namespace dew
+
+extern "C" int dew_moe_quantize_rows_nvfp4(const void* x, void* values, float* tensor_scale, uint32_t* workspace, int32_t rows,
+                                           int32_t depth, void* stream) {
+  using namespace dew;
+  DEW_REQUIRE(rows >= 0 && depth >= 16 && depth % 16 == 0, "dew_moe_quantize_rows_nvfp4: rows %d, depth %d (whole 16s)", rows, depth);
+  DEW_REQUIRE(tensor_scale && workspace, "dew_moe_quantize_rows_nvfp4: tensor_scale and the 4-byte workspace must not be null");
+  DEW_REQUIRE(rows == 0 || (x && values), "dew_moe_quantize_rows_nvfp4: x and values must not be null");
+  DEW_REQUIRE(depth % 8 == 0 && aligned16(x) && aligned16(values), "dew_moe_quantize_rows_nvfp4: x and values must be 16-byte aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(absmax_clear_kernel, dim3(1), dim3(1), 0, s, workspace);
+  if (int rc = launched("absmax_clear_kernel")) return rc;
+  const long long chunks = static_cast<long long>(rows) * depth / 8;
+  if (chunks > 0) {
+    const int blocks = static_cast<int>(min((chunks + 255) / 256, 256ll * 16));
+    hipLaunchKernelGGL(absmax_kernel, dim3(blocks), dim3(256), 0, s, static_cast<const bf16_t*>(x), chunks, workspace);
+    if (int rc = launched("absmax_kernel")) return rc;
+  }
+  hipLaunchKernelGGL(quantize_rows_nvfp4_kernel, dim3(max(1, (rows + kQuantizeWaves - 1) / kQuantizeWaves)), dim3(64 * kQuantizeWaves), 0, s,
+                     static_cast<const bf16_t*>(x), workspace, static_cast<bf16_t*>(values), tensor_scale, rows, depth);
+  return launched("quantize_rows_nvfp4_kernel");
+}
 
 extern "C" int dew_moe_quantize_rows_mxfp8(const void* x, void* codes, uint8_t* scales, int32_t rows, int32_t depth, void* stream) {
   using namespace dew;

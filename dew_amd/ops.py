@@ -150,6 +150,16 @@ class PreparedBank:
     def experts(self):
         return self.shape[0]
 
+    def scaled(self, by: torch.Tensor) -> "PreparedBank":
+        """The same NVFP4 bank with every expert's tensor scale times `by` (a one-element device tensor): how a
+        product of two NVFP4 operands owes both tensor scales to its fp32 sums."""
+        held = self.descriptor
+        if held.format not in (_lib.W_NVFP4, _lib.W_MXFP4):
+            raise KernelError("only an NVFP4 bank carries tensor scales")
+        scales = (self.keep[2].to(torch.float32) * by.to(torch.float32)).contiguous()
+        view = _lib.Bank(held.format, held.layout, held.experts, held.depth, held.width, held.codes, held.scales, _ptr(scales))
+        return PreparedBank(view, self.shape, (*self.keep, scales))
+
     def layer(self, index: int, layers: int) -> "PreparedBank":
         """Layer `index` of a bank that stacks `layers` layers' experts along its expert axis (`[layers * E, K, N]`),
         read where it lies: the same buffers, the descriptor's pointers moved to the layer's first expert (the
@@ -435,6 +445,20 @@ def quantize_rows_fp8(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     _lib.check(_lib.library().dew_moe_quantize_rows_fp8(_ptr(x), _ptr(codes), _ptr(scales), rows, depth, _stream()),
                "dew_moe_quantize_rows_fp8")
     return codes, scales
+
+
+def quantize_rows_nvfp4(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """bf16 rows `[rows, K]` quantized to NVFP4 along the depth (E2M1 under an E4M3 scale every 16 depths and one tensor
+    scale): (`values` bf16 `[rows, K]`, each what its code times its block's scale stands for, exactly; `scale` fp32
+    `[1]`, the tensor scale the product owes)."""
+    _device(x, "x", torch.bfloat16)
+    rows, depth = x.shape
+    values = torch.empty_like(x)
+    scale = torch.empty(1, dtype=torch.float32, device=x.device)
+    workspace = torch.empty(1, dtype=torch.int32, device=x.device)
+    _lib.check(_lib.library().dew_moe_quantize_rows_nvfp4(_ptr(x), _ptr(values), _ptr(scale), _ptr(workspace), rows, depth, _stream()),
+               "dew_moe_quantize_rows_nvfp4")
+    return values, scale
 
 
 def quantize_rows_mxfp8(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:

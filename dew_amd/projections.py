@@ -160,3 +160,54 @@ def mxfp8_projection(x: torch.Tensor, w, group_blocks, *, out_dtype=torch.bfloat
     sizes = (torch.as_tensor(group_blocks, device=x.device).to(torch.int32) * SCALE_DEPTH).contiguous()
     return mxfp8_product(mxfp8_rows(x), bank, sizes, out_dtype=out_dtype)
 
+
+# ---- the NVFP4 recipe ------------------------------------------------------------------------------------
+
+
+@dataclasses.dataclass(frozen=True)
+class NvFp4Rows:
+    """Rows quantized to NVFP4 (`ops.quantize_rows_nvfp4`): `values [rows, K]` bf16, each its E2M1 code times its 16
+    depths' E4M3 scale (exact), and the operand's tensor `scale [1]` fp32."""
+
+    values: torch.Tensor
+    scale: torch.Tensor
+
+
+def nvfp4_rows(x: torch.Tensor) -> NvFp4Rows:
+    """`NvFp4Block.quantized(x)` for rows `[rows, K]` bf16 (src/dew/nn/kernels/formats.py:263-274), on the device."""
+    return NvFp4Rows(*ops.quantize_rows_nvfp4(x.contiguous()))
+
+
+def nvfp4_matrices(w: torch.Tensor) -> formats.NvFp4:
+    """`w [groups, depth, width]` as the recipe quantizes its matrices: NVFP4 along the depth, all of them under one
+    tensor scale (`NvFp4Block.quantized(swapaxes(w, 1, 2))` flattens the groups into one operand,
+    src/dew/nn/kernels/projections.py:243-247), packed as the bank the kernels multiply."""
+    from . import codecs
+
+    groups, depth, width = w.shape
+    together = w.to(torch.float32).permute(1, 0, 2).reshape(depth, groups * width)
+    codes, scales, tensor = codecs.nvfp4_coded(together)
+    codes = codes.reshape(depth, groups, width).permute(1, 0, 2).contiguous()
+    scales = scales.reshape(depth // 16, groups, width).permute(1, 0, 2).contiguous()
+    return formats.NvFp4.of(codes, scales, tensor.reshape(1).expand(groups).contiguous())
+
+
+def nvfp4_block_product(lhs: NvFp4Rows, matrices, group_sizes, *, out_dtype=torch.bfloat16, gather=None, scatter=None) -> torch.Tensor:
+    """Each group's NVFP4 rows times its matrix of the NVFP4 bank `matrices`: every (code x block scale) product exact,
+    fp32 sums, times both tensor scales, one rounding (src/dew/nn/kernels/gemm.py:937-947). The rows' values are
+    exact in bf16, so this is the bank's bf16-operand launch with the rows' tensor scale folded into the bank's."""
+    if out_dtype != torch.bfloat16:
+        raise ValueError(f"the launch writes bfloat16, not {out_dtype}")
+    bank = gemm.prepared(matrices).scaled(lhs.scale)
+    rows = lhs.values.shape[0] if gather is None else gather.numel()
+    return ops.grouped_gemm(lhs.values, bank, _offsets(group_sizes, rows, lhs.values.device), gather=gather, scatter=scatter)
+
+
+def nvfp4_projection(x: torch.Tensor, w, group_blocks, *, out_dtype=torch.bfloat16) -> torch.Tensor:
+    """Each group's rows of `x [rows, depth]` times its matrix of `w [groups, depth, width]` in the NVFP4 recipe, both
+    quantized along the depth (src/dew/nn/kernels/projections.py:261-275); group `g` holds `group_blocks[g]` whole
+    128-row blocks. `w` is the weights (quantized here, `nvfp4_matrices`) or an NVFP4 bank already quantized."""
+    bank = w if isinstance(w, (formats.NvFp4, ops.PreparedBank)) else nvfp4_matrices(w)
+    sizes = (torch.as_tensor(group_blocks, device=x.device).to(torch.int32) * SCALE_DEPTH).contiguous()
+    return nvfp4_block_product(nvfp4_rows(x), bank, sizes, out_dtype=out_dtype)
+

@@ -204,6 +204,15 @@ int dew_moe_quantize_rows_mxfp8(const void* x /* bf16 [rows, K] */, void* codes 
 int dew_moe_grouped_gemm_mxfp8_rows(const void* x_codes, const uint8_t* x_scales, const int32_t* gather,
                                     const int32_t* offsets, const dew_moe_bank* w, const float* bias,
                                     const int32_t* scatter, void* out, int32_t rows, void* stream);
+/* The NVFP4 recipe's rows (`NvFp4Block.quantized` src/dew/nn/kernels/formats.py:263-274 over `bits.nvfp4_coded`
+ * src/dew/algebra/bits.py:941-982): E2M1 codes under an E4M3 scale every 16 depths and one tensor scale (the
+ * operand's largest magnitude over 6 x 448). The instruction has no such operand (its block scales are powers of two
+ * over 32 depths), so the rows are written as the bf16 values they stand for short of the tensor scale (code x block
+ * scale, exact in bf16) and multiplied by the NVFP4 bank through dew_moe_grouped_gemm with the two tensor scales'
+ * product as the bank's (`nvfp4_block_product` src/dew/nn/kernels/gemm.py:937-947). workspace: 4 bytes of device
+ * memory; tensor_scale: one device float, written.                                                               */
+int dew_moe_quantize_rows_nvfp4(const void* x /* bf16 [rows, K] */, void* values /* bf16 [rows, K] */,
+                                float* tensor_scale, uint32_t* workspace, int32_t rows, int32_t depth, void* stream);
 int dew_moe_quantize_rows_fp8(const void* x /* bf16 [rows, K] */, void* codes /* [rows, K] bytes */,
                               uint8_t* scales /* [rows, P] e8m0 */, int32_t rows, int32_t depth, void* stream);
 int dew_moe_grouped_gemm_fp8_rows(const void* x_codes, const uint8_t* x_scales, const int32_t* gather,

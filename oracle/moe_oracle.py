@@ -42,6 +42,11 @@ What pins each function (tests/test_oracle_golden.py):
   saturates; a zero block takes byte 0; the scale byte is the largest magnitude's fp32 exponent field less 8) and
   by the decoded operands reproducing the source within half a code step.
 
+* `nvfp4_quantized` (the NVFP4 recipe's operands): the closed form the reference's own test states
+  (tests/test_algebra_bits.py:510-528), checked against the bank quantizer's pins (tests/test_codecs.py) and by
+  brute force over the E2M1 grid for the rounding; `nvfp4_block_product` against the float64 sum of the decoded
+  operands.
+
 Parity unpinned (no byte fixture in the reference, closed form only): the exact bits of the softmax
 denominator's compensated sum (src/dew/nn/precision.py:1832); it moves router weights by at most one fp32
 ulp and no index. `gpt_oss_gating`'s bf16 mode: where each bf16 rounding falls follows JAX's arithmetic on
@@ -583,6 +588,61 @@ def mxfp8_projection(x, w, group_sizes, *, dtype="bfloat16", bias=None):
     rows, row_scales = mxfp8_quantized(x)
     matrices, matrix_scales = mxfp8_quantized(np.swapaxes(np.asarray(w, F32), 1, 2))
     return mxfp8_product(rows, row_scales, matrices, matrix_scales, group_sizes, dtype=dtype, bias=bias)
+
+
+# --------------------------------------------------------------------------------------------------
+# The NVFP4 recipe's forward product (E2M1 codes, an E4M3 scale every 16 depths, one tensor scale)
+# --------------------------------------------------------------------------------------------------
+
+
+def nvfp4_quantized(x):
+    """`x [..., depth]` as NVFP4 along its depth (`NvFp4Block.quantized`, src/dew/nn/kernels/formats.py:263-274, over
+    `bits.nvfp4_coded`, src/dew/algebra/bits.py:941-982, in the closed form its test states,
+    tests/test_algebra_bits.py:510-528): one tensor scale, the largest magnitude over 6 x 448 (fp32's least normal
+    at least; 1 for a zero tensor); each 16 depths' scale the least E4M3 at or above its largest magnitude over the
+    tensor scale over 6; each value, divided by the tensor scale and then by its block's, rounded to E2M1, ties to
+    even; a zero block's codes zero. Every quotient an IEEE fp32 division. Returns (E2M1 values `[..., depth]`, E4M3
+    scale values `[..., depth / 16]`, the tensor scale)."""
+    x = np.asarray(x, F32)
+    largest = F32(np.abs(x).max()) if x.size else F32(0)
+    tensor = np.maximum(largest / F32(6 * 448), np.finfo(F32).tiny).astype(F32) if largest > 0 else F32(1)
+    blocks = np.abs(x).reshape(*x.shape[:-1], x.shape[-1] // 16, 16)
+    ratio = ((blocks.max(axis=-1) / tensor).astype(F32) / F32(6)).astype(F32)
+    table = E4M3[:0x7F].astype(F32)
+    scales = table[np.minimum(np.searchsorted(table, ratio), table.size - 1)]
+    each = np.repeat(scales, 16, axis=-1)
+    positive = each > 0
+    quotient = np.where(positive, ((x / tensor).astype(F32) / np.where(positive, each, F32(1))).astype(F32), F32(0))
+    grid = E2M1[:8].astype(np.float64)
+    magnitude = np.abs(quotient.astype(np.float64))
+    below = np.searchsorted((grid[1:] + grid[:-1]) / 2, magnitude, side="left")    # a tie stays with the lower code
+    above = np.searchsorted((grid[1:] + grid[:-1]) / 2, magnitude, side="right")   # a tie goes to the upper code
+    code = np.where((above != below) & (above % 2 == 1), below, above)             # ... whichever is even
+    return (np.copysign(grid[code], quotient)).astype(F32), scales, tensor
+
+
+def nvfp4_block_product(lhs, lhs_scales, lhs_scale, matrices, matrix_scales, matrix_scale, group_sizes, *, dtype="bfloat16"):
+    """Each group's rows of `lhs [rows, depth]` times its matrix of `matrices [groups, width, depth]`, both NVFP4:
+    each code times its sixteen depths' scale, every product exact, summed in fp32, times both tensor scales, rounded
+    once (src/dew/nn/kernels/gemm.py:937-947). The sum is formed exactly and rounded to fp32."""
+    left = np.asarray(lhs, np.float64) * np.repeat(np.asarray(lhs_scales, np.float64), 16, axis=-1)
+    right = np.asarray(matrices, np.float64) * np.repeat(np.asarray(matrix_scales, np.float64), 16, axis=-1)
+    total = np.zeros((left.shape[0], right.shape[1]), F32)
+    start = 0
+    for group, size in enumerate(np.asarray(group_sizes).tolist()):
+        if size:
+            total[start:start + size] = (left[start:start + size] @ right[group].T).astype(F32)
+        start += size
+    total = twice_scaled(total, F32(lhs_scale), F32(matrix_scale))
+    return bf16_round(total) if dtype == "bfloat16" else total
+
+
+def nvfp4_projection(x, w, group_sizes, *, dtype="bfloat16"):
+    """`x [rows, depth]` and `w [groups, depth, width]` both quantized along the depth (the matrices under one tensor
+    scale together), their `nvfp4_block_product` (src/dew/nn/kernels/projections.py:261-275)."""
+    rows = nvfp4_quantized(x)
+    matrices = nvfp4_quantized(np.swapaxes(np.asarray(w, F32), 1, 2))
+    return nvfp4_block_product(*rows, *matrices, group_sizes, dtype=dtype)
 
 
 def swiglu(gate, up, *, dtype="bfloat16", limit=None, exp=np.exp):

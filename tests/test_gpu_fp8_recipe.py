@@ -213,3 +213,38 @@ def test_an_mxfp8_bank_is_refused_by_the_bf16_products(ops):
     x = torch.zeros((8, 256), dtype=torch.bfloat16).cuda()
     with pytest.raises(Exception, match="MXFP8"):
         ops.grouped_gemm(x, bank, torch.tensor([0, 8], dtype=torch.int32).cuda())
+
+
+# ---- the NVFP4 recipe -----------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("rows,depth", [(7, 128), (33, 384), (260, 4096)])
+def test_nvfp4_rows_are_quantized_bit_for_bit(ops, rows, depth):
+    rng = np.random.default_rng(rows)
+    x = (rng.standard_normal((rows, depth)) * rng.choice([1e-3, 0.1, 1.0, 30.0], size=(rows, 1))).astype(np.float32)
+    x[0, :16] = 0.0                                   # a zero block: zero codes
+    x[1, :16] = np.linspace(-1e-5, 1e-5, 16)          # far under the tensor's largest: the least scales, tiny codes
+    x = torch.from_numpy(x).to(torch.bfloat16)
+    values, scale = ops.quantize_rows_nvfp4(x.cuda())
+    want_values, want_scales, want_tensor = oracle.nvfp4_quantized(bf16_np(x))
+    assert scale.item() == want_tensor
+    assert np.array_equal(bf16_np(values), want_values * np.repeat(want_scales, 16, axis=1))
+    zeros, one = ops.quantize_rows_nvfp4(torch.zeros((3, 64), dtype=torch.bfloat16).cuda())
+    assert one.item() == 1.0 and not zeros.any()
+
+
+@pytest.mark.parametrize("label,sizes", SIZES, ids=[s[0] for s in SIZES])
+def test_the_nvfp4_product_matches_the_oracle(ops, label, sizes):
+    from dew_amd import projections
+
+    depth, width = 512, 256
+    groups, rows = len(sizes), int(np.sum(sizes))
+    rng = np.random.default_rng(rows + 3)
+    x = torch.from_numpy(rng.standard_normal((rows + 6, depth)).astype(np.float32)).to(torch.bfloat16)
+    w = weights_case(groups, depth, width, seed=21)
+    bank = projections.nvfp4_matrices(torch.from_numpy(w)).to("cuda")
+    got = bf16_np(projections.nvfp4_block_product(projections.nvfp4_rows(x.cuda()), bank, torch.tensor(sizes, dtype=torch.int32).cuda()))
+    want = oracle.nvfp4_projection(bf16_np(x), w, sizes)
+    assert np.all(got[rows:] == 0) and np.all(want[rows:] == 0)
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= 2.0 ** -7 * scale and (got == want).mean() > 0.97

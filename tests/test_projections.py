@@ -148,3 +148,22 @@ def test_the_host_mirror_quantizes_an_mxfp8_bank_as_the_oracle_does():
     assert bank.shape == (2, 256, 128)
     assert np.array_equal(bank.scales.numpy(), want_scales)
     assert np.array_equal(bank.codes.numpy(), oracle.e4m3_bytes(want_values))
+
+
+def test_the_nvfp4_operand_follows_the_bank_quantizers_closed_form():
+    """The recipe's operand rule is the bank quantizer's (tests/test_codecs.py pins that one against the reference's own
+    statement); here the oracle's restatement against it, the zero block, and the decoded operand within half a code
+    step of its source."""
+    from dew_amd import codecs
+
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal((40, 256)) * rng.choice([0.01, 1.0, 50.0], size=(40, 1))).astype(np.float32)
+    x[3, 16:32] = 0.0
+    values, scales, tensor = oracle.nvfp4_quantized(x)
+    codes, held, scale = codecs.nvfp4_coded(torch.from_numpy(x.T.copy()))
+    assert tensor == scale.item() == np.float32(np.abs(x).max()) / np.float32(6 * 448)
+    assert np.array_equal(oracle.E4M3[held.numpy()].T, scales) and np.array_equal(oracle.E2M1[codes.numpy()].T, values)
+    assert not values[3, 16:32].any() and np.abs(values).max() <= 6
+    decoded = values * np.repeat(scales, 16, axis=1) * tensor
+    assert (np.abs(decoded - x) <= 0.5 * np.repeat(scales, 16, axis=1) * tensor * 2.0 + 1e-30).all()   # the widest step is 2
+    assert oracle.nvfp4_quantized(np.zeros((2, 32), np.float32))[2] == 1.0
