@@ -53,6 +53,11 @@ constexpr int kFormatFp8Rows = 18;
 // in the scale byte of its row (column) and 32-deep block. The rows' scale bytes ride the A ring, a dword a row a
 // step; the weights' come with their atoms, a dword a column a step.
 constexpr int kFormatMxFp8Rows = 19;
+// The same instruction stream as a kernel gradient (each group's rows contracted: out[g] = lhs_t[:, group g's tokens] x
+// rhs_t[:, group g's tokens]^T): the "rows" are the lhs_t's (the same `window_rows` of them for every group), the
+// "bank" is the rhs_t quantized along the tokens and laid out as an MXFP8 bank of one expert whose depth is all the
+// tokens, and group g contracts the window of 128-token blocks its offsets name (dew_moe_kernel_gradient_mxfp8).
+constexpr int kFormatMxFp8Window = 20;
 
 constexpr int BK = 64;
 constexpr int kThreads = 256;
@@ -83,13 +88,18 @@ struct GemmParams {
   // hold at most BM / 2 rows to a launch of tiles half as tall, which multiplies (tail_of = the taller tile's rows)
   // only those last rows, the ones past a group's whole tiles of tail_of rows where they are at most its own BM.
   int skip_tails, tail_of;
+  // A kernel gradient (kFormatMxFp8Window): every group multiplies the same window_rows rows over its own window of
+  // the depth, tokens windows[g] .. windows[g + 1] in whole 128s; `depth` is then all the tokens.
+  const int32_t* windows;
+  int window_rows;
+  float* out_f32;  // the product in fp32 (kPlainF32) instead of `out`
 };
 
 // What the epilogue writes: the rounded product (plus bias); SwiGLU of two banks' products; for one bank whose
 // columns interleave gate (even) and up (odd), the clamped quick-GELU gating of each column pair; or the SwiGLU of
 // two banks' products already split into two e4m3 terms under one scale per row and 128 columns, which is what the
 // next product's scaled matrix instructions read (kFormatMxSplitBlocks).
-enum Epilogue { kPlain = 0, kSwigluOfTwo = 1, kInterleavedGated = 2, kSwigluOfTwoSplit = 3 };
+enum Epilogue { kPlain = 0, kSwigluOfTwo = 1, kInterleavedGated = 2, kSwigluOfTwoSplit = 3, kPlainF32 = 4 };
 
 // LDS index of 16-byte chunk `chunk` of row `row` (128-byte rows). The chunk is xor-swizzled by
 // f(row) = ((row >> 1) & 7) ^ ((row & 1) << 2), chosen against the measured service order of gfx950's LDS:
@@ -181,7 +191,8 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   constexpr int kOutBN = kGated ? BN / 2 : BN;  // output columns of the tile
   static_assert(WM * WN == 4 && BM % (32 * WM) == 0 && BN % (32 * WN) == 0 && BM % 32 == 0, "tile shape");
   constexpr bool kFp8Rows = FORMAT == kFormatFp8Rows;   // e4m3 rows, one scale per row and 128 depths; 128 x 128 weight scales
-  constexpr bool kMxRows = FORMAT == kFormatMxFp8Rows;  // e4m3 rows and weights, one scale per row (column) and 32 depths
+  constexpr bool kWindow = FORMAT == kFormatMxFp8Window;  // a kernel gradient: the same rows for every group, its own depths
+  constexpr bool kMxRows = FORMAT == kFormatMxFp8Rows || kWindow;  // e4m3 rows and weights, one scale per row (column) and 32 depths
   constexpr bool kFp8A = kFp8Rows || kMxRows;           // both operands e4m3 codes: a step is 128 depths
   constexpr bool kSplit = FORMAT == kFormatMxSplit || FORMAT == kFormatMxSplitBlocks || kFp8A;  // A arrives as 8-bit codes
   constexpr bool kBlockScales = FORMAT == kFormatMxSplitBlocks || kFp8Rows;
@@ -238,8 +249,8 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     const int e = base + tid;
     int start = 0, tiles = 0;
     if (e < p.experts) {
-      start = p.offsets[e];
-      const int size = p.offsets[e + 1] - start;
+      start = kWindow ? e * p.window_rows : p.offsets[e];
+      const int size = kWindow ? p.window_rows : p.offsets[e + 1] - start;
       if (p.tail_of > 0) {
         const int rest = size % p.tail_of;
         tiles = rest >= 1 && rest <= BM ? 1 : 0;
@@ -271,7 +282,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   const int expert = found[0];
 
   if (expert < 0) {
-    if (p.tail_of > 0) return;  // (the taller tiles' launch zeroes them)
+    if (kWindow || p.tail_of > 0) return;  // (the taller tiles' launch zeroes them; a kernel gradient has no rows past its groups)
     // Past the last real tile: zero the rows no expert owns (sorted positions offsets[E] .. rows).
     const int tail_begin = p.offsets[p.experts] + (m_tile - found[2]) * BM;
     const int tail_end = min(tail_begin + BM, p.rows);
@@ -288,8 +299,20 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   }
 
   const int row0 = found[1];
-  const int valid_rows = min(BM, p.offsets[expert + 1] - row0);
-  const int steps = p.depth / kStepDepth;
+  const int valid_rows = min(BM, (kWindow ? (expert + 1) * p.window_rows : p.offsets[expert + 1]) - row0);
+  // a kernel gradient's group contracts its own whole 128-token blocks of the depth
+  const int first_step = kWindow ? min(max(p.windows[expert], 0), p.depth) / kStepDepth : 0;
+  const int steps = kWindow ? max(min(max(p.windows[expert + 1], 0), p.depth) / kStepDepth - first_step, 0) : p.depth / kStepDepth;
+  if (kWindow && steps == 0) {  // an empty group's gradient is zero
+    for (int item = tid; item < valid_rows * (BN / 4); item += kThreads) {
+      const size_t at = static_cast<size_t>(row0 + item / (BN / 4)) * p.width + n0 + (item % (BN / 4)) * 4;
+      if (MODE == kPlainF32)
+        *reinterpret_cast<u32x4_t*>(p.out_f32 + at) = u32x4_t{0, 0, 0, 0};
+      else
+        *reinterpret_cast<uint2*>(p.out + at) = uint2{0, 0};
+    }
+    return;
+  }
   const int wm0 = (wave / WN) * (BM / WM), wn0 = (wave % WN) * (BN / WN);
 
   // ---- A loader. One global_load_lds_dwordx4 of a wavefront fills 1 KiB of LDS, lane l landing at byte 16 l:
@@ -301,9 +324,9 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     const int row = (wave * kRowLoads + i) * 8 + lane / 8;
     const int chunk = (lane % 8) ^ (((row >> 1) & 7) ^ ((row & 1) << 2));
     const int sorted = row0 + min(row, valid_rows - 1);
-    const int source = p.gather ? p.gather[sorted] : sorted;
+    const int source = kWindow ? sorted - expert * p.window_rows : p.gather ? p.gather[sorted] : sorted;
     // (a row of e4m3 codes is depth bytes.) Less the load's immediate offset, which the instruction adds back: see load_a
-    a_src[i] = p.x + static_cast<size_t>(source) * (kFp8A ? p.depth / 2 : p.depth) + chunk * 8 - (i % 4) * 512;
+    a_src[i] = p.x + static_cast<size_t>(source) * (kFp8A ? p.depth / 2 : p.depth) + first_step * (kStepDepth / 2) + chunk * 8 - (i % 4) * 512;
     asm volatile("" : "+v"(a_src[i]));  // kept as computed: the compiler otherwise re-adds the bias at every load
   }
   // Split activations: the lane's row of each row tile carries one e8m0 scale; the hi term multiplies under it
@@ -373,8 +396,8 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   if constexpr (kMxRows) {
     static_assert(!kMxRows || BM == kThreads, "one thread fetches one row's scales");
     const int sorted = row0 + min(tid, valid_rows - 1);
-    const int source = p.gather ? p.gather[sorted] : sorted;
-    a_mx_src = p.a_scale + static_cast<size_t>(source) * (p.depth / 32);
+    const int source = kWindow ? sorted - expert * p.window_rows : p.gather ? p.gather[sorted] : sorted;
+    a_mx_src = p.a_scale + static_cast<size_t>(source) * (p.depth / 32) + first_step * 4;
   }
   auto load_a_scales = [&](int stage_number, int step) __attribute__((always_inline)) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -403,7 +426,8 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     const int matrix = t / TJ, column = n0 + wn0 + 32 * (t % TJ);
     const uint8_t* codes = matrix == 0 ? p.w0.codes : p.w1.codes;
     const void* scales = matrix == 0 ? p.w0.scales : p.w1.scales;
-    const size_t first_atom = (static_cast<size_t>(expert) * n_atoms + column / 32) * k_atoms;
+    // (a kernel gradient's one "expert" holds every group's tokens: the group's window starts first_step steps in)
+    const size_t first_atom = (static_cast<size_t>(kWindow ? 0 : expert) * n_atoms + column / 32) * k_atoms + first_step * kAtoms;
     b_src[t] = codes + first_atom * kAtomBytes + b_lane;
     b_scale_src[t] = nullptr;
     channel_scale[t] = 1.0f;
@@ -411,7 +435,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
       b_scale_src[t] = static_cast<const uint8_t*>(scales) + first_atom * 128 + b_scale_lane;
     } else if (kMxRows) {  // [E][N / 32][K / 128][32 columns][4 bytes]: the lane's column's dword of each step
       b_scale_src[t] = static_cast<const uint8_t*>(scales) +
-                       (static_cast<size_t>(expert) * n_atoms + column / 32) * (p.depth / 128) * 128 + (lane % 32) * 4;
+                       ((static_cast<size_t>(kWindow ? 0 : expert) * n_atoms + column / 32) * (p.depth / 128) + first_step) * 128 + (lane % 32) * 4;
     } else if (FORMAT == DEW_MOE_W_FP8_CHANNEL) {
       channel_scale[t] = static_cast<const float*>(scales)[static_cast<size_t>(expert) * p.width + column + lane % 32];
     }
@@ -749,6 +773,21 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     factor0 = (kSplit ? 1.0f : 256.0f) * p.w0.tensor_scale[expert];
     if (PAIRED) factor1 = (kSplit ? 1.0f : 256.0f) * p.w1.tensor_scale[expert];
   }
+  if constexpr (MODE == kPlainF32) {
+    // the fp32 sums as they are: a lane group's 32 lanes write 128 contiguous bytes of a row
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const int row = wm0 + 32 * i + 8 * (q / 4) + 4 * (lane / 32) + q % 4;
+        if (row < valid_rows) {
+          float* out_row = p.out_f32 + static_cast<size_t>(row0 + row) * p.width + n0 + wn0 + lane % 32;
+#pragma unroll
+          for (int j = 0; j < TJ; ++j) out_row[32 * j] = acc[0][i][j][q];
+        }
+      }
+    return;
+  }
   constexpr int kPasses = (BN == 256 && BM > 32) ? 2 : 1;
   constexpr int kPassTiles = BM / 32 / kPasses, kPassRows = BM / kPasses;  // row tiles of the block a pass stages
   constexpr int kRowDwords = kOutBN / 2 + 4;  // a staged row: the tile's output columns in bf16 and 16 bytes of padding
@@ -900,7 +939,7 @@ static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
   // block-scaled activations keep their tile's scales behind the ring (reserved at their largest: kMaxBlockScaleDepth)
   constexpr size_t kShared = shared_bytes<BM, BN, MODE>() +
                              (FORMAT == kFormatMxSplitBlocks || FORMAT == kFormatFp8Rows ? static_cast<size_t>(BM) * block_scale_pitch(kMaxBlockScaleDepth) : 0) +
-                             (FORMAT == kFormatMxFp8Rows ? 3 * static_cast<size_t>(BM) * 4 : 0);  // MXFP8 rows: a dword a row a stage
+                             (FORMAT == kFormatMxFp8Rows || FORMAT == kFormatMxFp8Window ? 3 * static_cast<size_t>(BM) * 4 : 0);  // MXFP8 rows: a dword a row a stage
   auto kernel = grouped_gemm_kernel<FORMAT, MODE, BM, BN, WM, WN>;
   static bool configured = false;  // dynamic LDS above 64 KiB must be opted into once per kernel
   if (!configured) {
@@ -911,6 +950,7 @@ static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
   }
   // every expert may end in a partial tile, and the zeroed tail may add one more
   p.m_tile_bound = p.tail_of > 0 ? p.experts : (p.rows + BM - 1) / BM + p.experts + 1;
+  if (FORMAT == kFormatMxFp8Window) p.m_tile_bound = p.experts * ((p.window_rows + BM - 1) / BM);  // every group the same whole rows
   const int total = p.m_tile_bound * (p.width / BN);
   const int blocks = ((total + 255) / 256) * 256;  // whole chunks of 32 tiles for each of the 8 XCDs
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreads), kShared, stream, p);
@@ -1142,6 +1182,47 @@ extern "C" int dew_moe_grouped_gemm_mxfp8_rows(const void* x_codes, const uint8_
   p.a_scale = x_scales;
   if (p.width % 256 == 0) return launch_tile<kFormatMxFp8Rows, kPlain, 256, 256, 2, 2>(who, p, static_cast<hipStream_t>(stream));
   return launch_tile<kFormatMxFp8Rows, kPlain, 256, 128, 2, 2>(who, p, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int dew_moe_kernel_gradient_mxfp8(const void* lhs_t_codes, const uint8_t* lhs_t_scales, const dew_moe_bank* rhs_t,
+                                             const int32_t* offsets, void* out, int32_t out_is_f32, int32_t depth, int32_t groups,
+                                             void* stream) {
+  using namespace dew;
+  const char* who = "dew_moe_kernel_gradient_mxfp8";
+  DEW_REQUIRE(rhs_t, "%s: the rhs_t bank must not be null", who);
+  DEW_REQUIRE(rhs_t->format == DEW_MOE_W_MXFP8 && rhs_t->layout == DEW_MOE_LAYOUT_PREPARED && rhs_t->experts == 1,
+              "%s: rhs_t is one prepared MXFP8 matrix [width, tokens] (dew_moe_quantize_columns_*, as a bank), not format %d, layout %d, %d experts",
+              who, rhs_t->format, rhs_t->layout, rhs_t->experts);
+  const int tokens = rhs_t->depth;
+  DEW_REQUIRE(tokens >= 0 && tokens % 128 == 0, "%s: %d tokens are not whole 128-token blocks", who, tokens);
+  DEW_REQUIRE(rhs_t->width >= 128 && rhs_t->width % 128 == 0, "%s: width %d is not a multiple of 128", who, rhs_t->width);
+  DEW_REQUIRE(depth >= 128 && depth % 128 == 0, "%s: depth %d is not a multiple of 128", who, depth);
+  DEW_REQUIRE(groups >= 1 && groups <= 4096, "%s: %d groups", who, groups);
+  DEW_REQUIRE(static_cast<long long>(groups) * depth < (1ll << 31), "%s: %d groups of %d rows overflow the row index", who, groups, depth);
+  DEW_REQUIRE(offsets && out && aligned16(out), "%s: offsets and out must not be null, out 16-byte aligned", who);
+  DEW_REQUIRE(tokens == 0 || (lhs_t_codes && lhs_t_scales && rhs_t->codes && rhs_t->scales), "%s: the operands' codes and scales must not be null", who);
+  DEW_REQUIRE(aligned16(lhs_t_codes) && aligned16(rhs_t->codes) && (reinterpret_cast<uintptr_t>(lhs_t_scales) & 3u) == 0,
+              "%s: codes must be 16-byte and the lhs_t's scales 4-byte aligned", who);
+  GemmParams p{};
+  p.x = static_cast<const bf16_t*>(lhs_t_codes);
+  p.a_scale = lhs_t_scales;
+  p.windows = offsets;
+  p.window_rows = depth;
+  p.w0 = BankView{static_cast<const uint8_t*>(rhs_t->codes), rhs_t->scales, nullptr};
+  p.w1 = p.w0;
+  p.out = static_cast<bf16_t*>(out);
+  p.out_f32 = static_cast<float*>(out);
+  p.experts = groups;
+  p.depth = tokens;
+  p.width = rhs_t->width;
+  p.rows = groups * depth;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (out_is_f32) {
+    if (p.width % 256 == 0) return launch_tile<kFormatMxFp8Window, kPlainF32, 256, 256, 2, 2>(who, p, s);
+    return launch_tile<kFormatMxFp8Window, kPlainF32, 256, 128, 2, 2>(who, p, s);
+  }
+  if (p.width % 256 == 0) return launch_tile<kFormatMxFp8Window, kPlain, 256, 256, 2, 2>(who, p, s);
+  return launch_tile<kFormatMxFp8Window, kPlain, 256, 128, 2, 2>(who, p, s);
 }
 
 extern "C" int dew_moe_gateup_swiglu_split_out(const void* x_split, const uint8_t* x_scale, const int32_t* gather,

@@ -175,7 +175,119 @@ __global__ __launch_bounds__(64 * kQuantizeWaves) void quantize_rows_nvfp4_kerne
   }
 }
 
+// A kernel gradient's operands: x [tokens, dim] quantized ALONG THE TOKENS and written transposed, for the product
+// that contracts each group's tokens (reference src/dew/nn/kernels/projections.py:211-224 `rows_quantized(x.T)`, and
+// :263-275 `MxFp8.quantized(x.T)`). MX false: the blockwise FP8 recipe's 1 x 128 tiles (128 tokens of one column under
+// the scale rule of quantize_rows_fp8_kernel, its byte written for each of the tile's four 32-token blocks); MX true: OCP
+// MX blocks of 32 tokens (quantize_rows_mxfp8_kernel's rule). BANK false writes the lhs_t operand: codes [dim, tokens]
+// in the row operand's order within each 128 tokens (see the head of this file) and scales [dim, tokens / 32]. BANK true
+// writes the rhs_t operand as a prepared MXFP8 bank of one expert, depth = tokens, width = dim: codes as 32 column x 32
+// token atoms [dim / 32][tokens / 32][64 lanes][16 bytes] (lane 32 g + c holds tokens 16 g .. 16 g + 15 of column c) and
+// scales [dim / 32][tokens / 128][32 columns][4 bytes].
+// A block takes 128 tokens x 64 columns through the LDS: thread (column c, quarter a) owns the 32 tokens of block a.
+// HBM-bound: 2 bytes read and 1 written per element.
+template <bool MX, bool BANK>
+__global__ __launch_bounds__(256) void quantize_columns_kernel(const bf16_t* __restrict__ x, uint8_t* __restrict__ codes,
+                                                               uint32_t* __restrict__ scales, int tokens, int dim) {
+  __shared__ uint32_t tile[128][33];     // 128 tokens x 64 columns of bf16, a dword of padding a row
+  __shared__ float quarter_amax[4][64];
+  __shared__ uint32_t scale_word[64];    // a column's four scale bytes
+  __shared__ u32x4_t staged[64][8];      // the lhs_t operand's 64 rows of 128 bytes, chunk xor-swizzled by the row
+  const int tid = threadIdx.x;
+  const int t0 = blockIdx.x * 128, d0 = blockIdx.y * 64;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int item = tid + 256 * k, row = item / 8, chunk = item % 8;
+    const u32x4_t words = *reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(t0 + row) * dim + d0 + chunk * 8);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) tile[row][chunk * 4 + i] = words[i];
+  }
+  if (tid < 64) scale_word[tid] = 0;
+  __syncthreads();
+  const int c = tid % 64, quarter = tid / 64;
+  float v[32];
+  float largest = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 32; ++i) {
+    const uint32_t word = tile[32 * quarter + i][c / 2];
+    v[i] = __uint_as_float(c % 2 ? word & 0xFFFF0000u : word << 16);
+    largest = fmaxf(largest, fabsf(v[i]));
+  }
+  uint32_t byte;
+  if constexpr (MX) {
+    const int field = static_cast<int>(__float_as_uint(largest) >> 23);
+    byte = static_cast<uint32_t>(min(max(field - 8, 0), 254));
+  } else {
+    quarter_amax[quarter][c] = largest;
+    __syncthreads();
+    const float amax = fmaxf(fmaxf(quarter_amax[0][c], quarter_amax[1][c]), fmaxf(quarter_amax[2][c], quarter_amax[3][c]));
+    const uint32_t bits = __float_as_uint(fmaxf(amax, 1e-4f) * 0x1.24924ap-9f);  // f32(1 / 448)
+    byte = min(max((bits >> 23) + ((bits & 0x7FFFFFu) != 0u ? 1u : 0u), 1u), 253u);
+  }
+  const float inverse = __uint_as_float((254u - byte) << 23);
+  uint32_t packed[8];
+#pragma unroll
+  for (int w = 0; w < 8; ++w) {
+    float q[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) q[i] = MX ? fminf(fmaxf(v[4 * w + i] * inverse, -448.0f), 448.0f) : v[4 * w + i] * inverse;
+    packed[w] = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false);
+    packed[w] = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], packed[w], true);
+  }
+  atomicOr(&scale_word[c], byte << (8 * quarter));
+  const u32x4_t low = {packed[0], packed[1], packed[2], packed[3]}, high = {packed[4], packed[5], packed[6], packed[7]};
+  if constexpr (BANK) {
+    uint8_t* atom = codes + ((static_cast<size_t>((d0 + c) / 32) * (tokens / 32) + t0 / 32 + quarter) * 64 + c % 32) * 16;
+    *reinterpret_cast<u32x4_t*>(atom) = low;
+    *reinterpret_cast<u32x4_t*>(atom + 512) = high;
+    __syncthreads();
+    if (tid < 64) scales[(static_cast<size_t>((d0 + tid) / 32) * (tokens / 128) + t0 / 128) * 32 + tid % 32] = scale_word[tid];
+  } else {
+    // tokens 32 a + 16 g + b of the 128 sit at byte 16 (4 g + a) + b
+    staged[c][quarter ^ (c & 7)] = low;
+    staged[c][(4 + quarter) ^ (c & 7)] = high;
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int item = tid + 256 * k, row = item / 8, chunk = item % 8;
+      *reinterpret_cast<u32x4_t*>(codes + static_cast<size_t>(d0 + row) * tokens + t0 + chunk * 16) = staged[row][chunk ^ (row & 7)];
+    }
+    if (tid < 64) scales[static_cast<size_t>(d0 + tid) * (tokens / 128) + t0 / 128] = scale_word[tid];
+  }
+}
+
+static int quantize_columns(const char* who, bool mx, const void* x, void* codes, void* scales, int tokens, int dim, int as_bank,
+                            void* stream) {
+  DEW_REQUIRE(tokens >= 0 && tokens % 128 == 0, "%s: %d tokens are not whole 128-token blocks", who, tokens);
+  DEW_REQUIRE(dim >= 128 && dim % 128 == 0, "%s: %d columns (whole 128s)", who, dim);
+  if (tokens == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(tokens / 128 <= 65535 * 32, "%s: %d tokens", who, tokens);
+  DEW_REQUIRE(x && codes && scales, "%s: x, codes and scales must not be null", who);
+  DEW_REQUIRE(aligned16(x) && aligned16(codes) && aligned16(scales), "%s: x, codes and scales must be 16-byte aligned", who);
+  const dim3 grid(tokens / 128, dim / 64);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, dim3(256), 0, s, static_cast<const bf16_t*>(x), static_cast<uint8_t*>(codes),
+                       static_cast<uint32_t*>(scales), tokens, dim);
+  };
+  if (mx && as_bank) launch(quantize_columns_kernel<true, true>);
+  else if (mx) launch(quantize_columns_kernel<true, false>);
+  else if (as_bank) launch(quantize_columns_kernel<false, true>);
+  else launch(quantize_columns_kernel<false, false>);
+  return launched("quantize_columns_kernel");
+}
+
 }  // namespace dew
+
+extern "C" int dew_moe_quantize_columns_fp8(const void* x, void* codes, void* scales, int32_t tokens, int32_t dim, int32_t as_bank,
+                                            void* stream) {
+  return dew::quantize_columns("dew_moe_quantize_columns_fp8", false, x, codes, scales, tokens, dim, as_bank, stream);
+}
+
+extern "C" int dew_moe_quantize_columns_mxfp8(const void* x, void* codes, void* scales, int32_t tokens, int32_t dim, int32_t as_bank,
+                                              void* stream) {
+  return dew::quantize_columns("dew_moe_quantize_columns_mxfp8", true, x, codes, scales, tokens, dim, as_bank, stream);
+}
 
 extern "C" int dew_moe_quantize_rows_nvfp4(const void* x, void* values, float* tensor_scale, uint32_t* workspace, int32_t rows,
                                            int32_t depth, void* stream) {

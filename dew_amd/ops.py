@@ -493,6 +493,50 @@ def grouped_gemm_mxfp8_rows(codes: torch.Tensor, scales: torch.Tensor, bank: Pre
     return out
 
 
+def quantize_columns(x: torch.Tensor, *, mx: bool, as_bank: bool):
+    """bf16 `[tokens, dim]` quantized along the tokens and written transposed, a kernel gradient's operand
+    (`dew_moe_quantize_columns_fp8` for the blockwise FP8 recipe's 1 x 128 tiles, `_mxfp8` for MX blocks of 32 tokens).
+    The lhs_t operand (`as_bank` false): (`codes` uint8 `[dim, tokens]`, each 128 tokens in the row operand's order;
+    `scales` uint8 `[dim, tokens / 32]`). The rhs_t operand (`as_bank`): a `PreparedBank` of one MXFP8 matrix, depth
+    the tokens, width `dim`."""
+    _device(x, "x", torch.bfloat16)
+    tokens, dim = x.shape
+    call = _lib.library().dew_moe_quantize_columns_mxfp8 if mx else _lib.library().dew_moe_quantize_columns_fp8
+    name = "dew_moe_quantize_columns_mxfp8" if mx else "dew_moe_quantize_columns_fp8"
+    if as_bank:
+        buffer = torch.empty(max(tokens * dim + tokens // 32 * dim, 16), dtype=torch.uint8, device=x.device)
+        codes, scales = buffer[:tokens * dim], buffer[tokens * dim:tokens * dim + tokens // 32 * dim]
+    else:
+        codes = torch.empty((dim, tokens), dtype=torch.uint8, device=x.device)
+        scales = torch.empty((dim, tokens // 32), dtype=torch.uint8, device=x.device)
+    _lib.check(call(_ptr(x), _ptr(codes), _ptr(scales), tokens, dim, int(as_bank), _stream()), name)
+    if not as_bank:
+        return codes, scales
+    view = _lib.Bank(_lib.W_MXFP8, _lib.LAYOUT_PREPARED, 1, tokens, dim, _ptr(codes), _ptr(scales), None)
+    return PreparedBank(view, (1, tokens, dim), (buffer,))
+
+
+def kernel_gradient_mxfp8(codes: torch.Tensor, scales: torch.Tensor, rhs_t: PreparedBank, offsets: torch.Tensor, *,
+                          out_dtype=torch.bfloat16) -> torch.Tensor:
+    """Each group's tokens contracted: `out[g] = lhs_t[:, tokens of g] @ rhs_t[:, tokens of g]^T`, `[groups, depth,
+    width]` in bf16 or fp32, from `quantize_columns`' operands (`codes [depth, tokens]`, `scales [depth, tokens / 32]`,
+    the bank `[width, tokens]`); `offsets` int32 `[groups + 1]` in whole 128-token blocks; an empty group's is zero."""
+    _, tokens, width = rhs_t.shape
+    depth = codes.shape[0]
+    if codes.dtype != torch.uint8 or tuple(codes.shape) != (depth, tokens) or scales.dtype != torch.uint8 or \
+            tuple(scales.shape) != (depth, tokens // 32) or not codes.is_contiguous() or not scales.is_contiguous():
+        raise KernelError(f"the lhs_t operand is uint8 [depth, {tokens}] with uint8 scales [depth, {tokens // 32}]")
+    if out_dtype not in (torch.bfloat16, torch.float32):
+        raise KernelError(f"a kernel gradient is written in bfloat16 or float32, not {out_dtype}")
+    _device(offsets, "offsets", torch.int32)
+    groups = offsets.numel() - 1
+    out = torch.empty((groups, depth, width), dtype=out_dtype, device=codes.device)
+    _lib.check(_lib.library().dew_moe_kernel_gradient_mxfp8(_ptr(codes), _ptr(scales), rhs_t.descriptor, _ptr(offsets), _ptr(out),
+                                                            int(out_dtype == torch.float32), depth, groups, _stream()),
+               "dew_moe_kernel_gradient_mxfp8")
+    return out
+
+
 def operand_order_fp8(codes: torch.Tensor) -> torch.Tensor:
     """e4m3 codes `[rows, K]` in depth order -> the order `quantize_rows_fp8` writes and `grouped_gemm_fp8_rows`
     reads: of each 128 depths, byte 16 (4 g + 2 t + h) + b holds depth 64 t + 32 h + 16 g + b."""

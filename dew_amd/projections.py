@@ -211,3 +211,37 @@ def nvfp4_projection(x: torch.Tensor, w, group_blocks, *, out_dtype=torch.bfloat
     sizes = (torch.as_tensor(group_blocks, device=x.device).to(torch.int32) * SCALE_DEPTH).contiguous()
     return nvfp4_block_product(nvfp4_rows(x), bank, sizes, out_dtype=out_dtype)
 
+
+# ---- the recipes' gradients ------------------------------------------------------------------------------
+
+
+def _group_offsets(group_blocks, device) -> torch.Tensor:
+    sizes = torch.as_tensor(group_blocks, device=device).to(torch.int64) * SCALE_DEPTH
+    return torch.cat([sizes.new_zeros(1), sizes.cumsum(0)]).to(torch.int32).contiguous()
+
+
+def kernel_gradient(x: torch.Tensor, cotangent: torch.Tensor, group_blocks, *, mx: bool, out_dtype=torch.bfloat16) -> torch.Tensor:
+    """A recipe's gradient for the matrices, `[groups, depth, width]`: each group's tokens of `x [tokens, depth]` and
+    `cotangent [tokens, width]` contracted after both are quantized ALONG THE TOKENS: the blockwise FP8 recipe's
+    1 x 128 tiles (`rows_quantized(x.T)`, `blockwise_fp8_kernel_gradient`, src/dew/nn/kernels/projections.py:220-223)
+    or, `mx`, MXFP8's blocks of 32 tokens (src/dew/nn/kernels/projections.py:268-274). Group `g` holds
+    `group_blocks[g]` whole 128-token blocks; an empty group's gradient is zero."""
+    codes, scales = ops.quantize_columns(x.contiguous(), mx=mx, as_bank=False)
+    bank = ops.quantize_columns(cotangent.contiguous(), mx=mx, as_bank=True)
+    return ops.kernel_gradient_mxfp8(codes, scales, bank, _group_offsets(group_blocks, x.device), out_dtype=out_dtype)
+
+
+def blockwise_fp8_gradients(x: torch.Tensor, w: torch.Tensor, cotangent: torch.Tensor, group_blocks, *, out_dtype=torch.bfloat16):
+    """`_projection_backward` (src/dew/nn/kernels/projections.py:211-224) -> (d_x, d_w). The input's gradient is the
+    recipe's own product of the requantized cotangent and the matrices' blocks transposed (a 128 x 128 block and its
+    scale transpose as they are); the matrices' is `kernel_gradient`."""
+    d_x = blockwise_fp8_projection(cotangent, w.transpose(1, 2).contiguous(), group_blocks, out_dtype=x.dtype)
+    return d_x, kernel_gradient(x, cotangent, group_blocks, mx=False, out_dtype=out_dtype)
+
+
+def mxfp8_gradients(x: torch.Tensor, w: torch.Tensor, cotangent: torch.Tensor, group_blocks, *, out_dtype=torch.bfloat16):
+    """`_mx_backward` (src/dew/nn/kernels/projections.py:263-275) -> (d_x, d_w): the MXFP8 product of the cotangent and
+    the matrices, both quantized along the width, and `kernel_gradient` with a scale every 32 tokens."""
+    d_x = mxfp8_projection(cotangent, w.transpose(1, 2).contiguous(), group_blocks, out_dtype=x.dtype)
+    return d_x, kernel_gradient(x, cotangent, group_blocks, mx=True, out_dtype=out_dtype)
+

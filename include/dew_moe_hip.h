@@ -204,6 +204,33 @@ int dew_moe_quantize_rows_mxfp8(const void* x /* bf16 [rows, K] */, void* codes 
 int dew_moe_grouped_gemm_mxfp8_rows(const void* x_codes, const uint8_t* x_scales, const int32_t* gather,
                                     const int32_t* offsets, const dew_moe_bank* w, const float* bias,
                                     const int32_t* scatter, void* out, int32_t rows, void* stream);
+/* The recipes' kernel gradients: each group's tokens contracted, out[g] = x[group g's tokens]^T @ dy[group g's
+ * tokens] -> [groups, K, N]. Blockwise FP8: `_projection_backward` src/dew/nn/kernels/projections.py:211-224
+ * (`rows_quantized(x.T)`, `rows_quantized(cotangent.T)`) and `blockwise_fp8_kernel_gradient`
+ * src/dew/nn/kernels/gemm.py:795-819 (each 128-token block's exact partial times its rows' and columns' scales, fp32
+ * sums; the recipe's scales are powers of two, taken here as E8M0 bytes). MXFP8: `_mx_backward`
+ * src/dew/nn/kernels/projections.py:263-275 (`MxFp8.quantized(x.T)`, every 32 tokens a scale; the reference multiplies
+ * the decoded operands in bf16 with fp32 sums, `gemm_t` src/dew/nn/kernels/gemm.py:418-431, which the scaled products
+ * equal term for term).
+ * dew_moe_quantize_columns_fp8 / _mxfp8: x bf16 [tokens, dim] quantized along the TOKENS (1 x 128 tiles under
+ * dew_moe_quantize_rows_fp8's scale rule, or 32-token MX blocks under dew_moe_quantize_rows_mxfp8's) and written
+ * transposed. as_bank 0 (the lhs_t operand): codes [dim, tokens] bytes in the row operand's order within each 128
+ * tokens, scales [dim, tokens / 32] E8M0 bytes (the FP8 tile's byte repeated for its four 32s). as_bank 1 (the rhs_t
+ * operand): the layout of a prepared DEW_MOE_W_MXFP8 bank of one expert, depth = tokens, width = dim: codes
+ * [dim / 32][tokens / 32][64][16] bytes, then scales [dim / 32][tokens / 128][32][4]; wrap them in a dew_moe_bank
+ * {MXFP8, PREPARED, experts 1, depth tokens, width dim}. tokens whole 128s (a recipe pads each group to them), dim
+ * whole 128s.
+ * dew_moe_kernel_gradient_mxfp8: out [groups, depth, width] (bf16, or fp32 where out_is_f32) from the lhs_t operand
+ * [depth, tokens] and the rhs_t bank [width, tokens]; group g contracts tokens offsets[g] .. offsets[g + 1], whole
+ * 128-token blocks (device int32 [groups + 1]); an empty group's matrix is zero. Both operands enter
+ * v_mfma_scale_f32_32x32x64_f8f6f4 as stored, 256 x 256 tiles.                                                    */
+int dew_moe_quantize_columns_fp8(const void* x /* bf16 [tokens, dim] */, void* codes, void* scales, int32_t tokens,
+                                 int32_t dim, int32_t as_bank, void* stream);
+int dew_moe_quantize_columns_mxfp8(const void* x /* bf16 [tokens, dim] */, void* codes, void* scales, int32_t tokens,
+                                   int32_t dim, int32_t as_bank, void* stream);
+int dew_moe_kernel_gradient_mxfp8(const void* lhs_t_codes, const uint8_t* lhs_t_scales, const dew_moe_bank* rhs_t,
+                                  const int32_t* offsets, void* out, int32_t out_is_f32, int32_t depth, int32_t groups,
+                                  void* stream);
 /* The NVFP4 recipe's rows (`NvFp4Block.quantized` src/dew/nn/kernels/formats.py:263-274 over `bits.nvfp4_coded`
  * src/dew/algebra/bits.py:941-982): E2M1 codes under an E4M3 scale every 16 depths and one tensor scale (the
  * operand's largest magnitude over 6 x 448). The instruction has no such operand (its block scales are powers of two

@@ -591,6 +591,59 @@ def mxfp8_projection(x, w, group_sizes, *, dtype="bfloat16", bias=None):
 
 
 # --------------------------------------------------------------------------------------------------
+# The recipes' gradients: the input's is the recipe's own product of the requantized cotangent and the matrices
+# quantized along the width; the matrices' contracts each group's tokens
+# --------------------------------------------------------------------------------------------------
+
+
+def kernel_gradient(lhs_t, rhs_t, group_sizes, *, dtype="bfloat16"):
+    """Each group's tokens contracted: `out[g] = lhs_t[:, tokens of g] @ rhs_t[:, tokens of g].T` for operands
+    `[depth, tokens]` and `[width, tokens]` already decoded to their values (float64, exact), summed exactly, rounded to
+    fp32 and then to `dtype`; an empty group's is zero (`gemm_t`, src/dew/nn/kernels/gemm.py:418-431; the definition the
+    reference's own test writes out, tests/test_gemm_blockwise.py:97-107)."""
+    lhs_t, rhs_t = np.asarray(lhs_t, np.float64), np.asarray(rhs_t, np.float64)
+    out = np.zeros((len(group_sizes), lhs_t.shape[0], rhs_t.shape[0]), F32)
+    start = 0
+    for group, size in enumerate(np.asarray(group_sizes, np.int64)):
+        out[group] = (lhs_t[:, start:start + size] @ rhs_t[:, start:start + size].T).astype(F32)
+        start += size
+    return bf16_round(out) if dtype == "bfloat16" else out
+
+
+def blockwise_fp8_kernel_gradient(lhs_t, rhs_t, group_blocks, row_scales, column_scales, *, dtype="bfloat16"):
+    """src/dew/nn/kernels/gemm.py:795-819: E4M3 values `lhs_t [depth, rows]` and `rhs_t [width, rows]`, each 128-row
+    block's partial times its depth rows' scales (`row_scales [rows / 128, depth]`) and its columns'
+    (`column_scales [rows / 128, width]`), added into its group's sum."""
+    left = np.asarray(lhs_t, np.float64) * np.repeat(np.asarray(row_scales, np.float64).T, SCALE_DEPTH, axis=1)
+    right = np.asarray(rhs_t, np.float64) * np.repeat(np.asarray(column_scales, np.float64).T, SCALE_DEPTH, axis=1)
+    return kernel_gradient(left, right, np.asarray(group_blocks) * SCALE_DEPTH, dtype=dtype)
+
+
+def blockwise_fp8_gradients(x, w, cotangent, group_blocks, *, dtype="bfloat16"):
+    """`_projection_backward` (src/dew/nn/kernels/projections.py:211-224): the input's gradient is the recipe's product
+    of the cotangent, requantized along the width, and the matrices' blocks transposed; the matrices' is the kernel
+    gradient of `x.T` and `cotangent.T`, each quantized along the tokens. Returns (d_x, d_w)."""
+    sizes = np.asarray(group_blocks) * SCALE_DEPTH
+    dy, dy_scales = rows_quantized(cotangent)
+    blocks, blocks_scales = blocks_quantized(w)
+    d_x = blockwise_fp8_product(dy, np.swapaxes(blocks, 1, 2), sizes, dy_scales.T, np.swapaxes(blocks_scales, 1, 2), dtype=dtype)
+    rows_t, rows_t_scales = rows_quantized(np.asarray(x, F32).T)
+    dy_t, dy_t_scales = rows_quantized(np.asarray(cotangent, F32).T)
+    return d_x, blockwise_fp8_kernel_gradient(rows_t, dy_t, group_blocks, rows_t_scales.T, dy_t_scales.T, dtype=dtype)
+
+
+def mxfp8_gradients(x, w, cotangent, group_blocks, *, dtype="bfloat16"):
+    """`_mx_backward` (src/dew/nn/kernels/projections.py:263-275): d_x = the MXFP8 product of the cotangent and the
+    matrices both quantized along the width; d_w = each group's tokens contracted over `x.T` and `cotangent.T`
+    quantized along the tokens, every 32 a scale, and decoded (exact in bf16), fp32 sums. Returns (d_x, d_w)."""
+    sizes = np.asarray(group_blocks) * SCALE_DEPTH
+    d_x = mxfp8_product(*mxfp8_quantized(cotangent), *mxfp8_quantized(np.asarray(w, F32)), sizes, dtype=dtype)
+    rows_t = mxfp8_decoded(*mxfp8_quantized(np.asarray(x, F32).T))
+    dy_t = mxfp8_decoded(*mxfp8_quantized(np.asarray(cotangent, F32).T))
+    return d_x, kernel_gradient(rows_t, dy_t, sizes, dtype=dtype)
+
+
+# --------------------------------------------------------------------------------------------------
 # The NVFP4 recipe's forward product (E2M1 codes, an E4M3 scale every 16 depths, one tensor scale)
 # --------------------------------------------------------------------------------------------------
 
