@@ -50,6 +50,7 @@ const char* dew_moe_kernels(void) {
          "grouped_gemm<fp8 rows>,256,256 | 128,128,4 (2x2),v_mfma_scale_f32_32x32x64_f8f6f4,e4m3 rows (1x128 power-of-two scales) x fp8 128x128 blocks (power-of-two scales)\n"
          "grouped_gemm<mxfp8 rows>,256,256,128,4 (2x2),v_mfma_scale_f32_32x32x64_f8f6f4,OCP MXFP8 rows x MXFP8 bank: e4m3 codes and E8M0 scales per 32 depths of both operands as stored\n"
          "split_rows | quantize_rows_fp8 | quantize_rows_mxfp8,1 row/wave,-,-,4,-,bf16 rows -> e4m3 terms | e4m3 codes in operand order + e8m0 scales\n"
+         "grouped_gemm<bf16>,32|64|128|256,128|256,64,3,v_mfma_f32_32x32x16_bf16,unquantized bf16 matrices as fragment atoms: no dequantization\n"
          "grouped_gemm<mxfp8 window>,256,256 | 128,128,4 (2x2),v_mfma_scale_f32_32x32x64_f8f6f4,a kernel gradient: each group's window of 128-token steps of lhs_t rows x the rhs_t bank; bf16 or fp32 out\n"
          "quantize_columns,128 tokens x 64 columns/block,-,-,4,-,bf16 [tokens x dim] -> e4m3 along the tokens and transposed: operand rows or bank atoms + e8m0 scales\n"
          "absmax + quantize_rows_nvfp4,1 row/wave,-,-,4,-,bf16 rows -> bf16 (e2m1 code x e4m3 scale) + the tensor scale\n"

@@ -184,7 +184,7 @@ __device__ __forceinline__ void schedule_phase() {
 // four wavefronts sit WM x WN (1 x 4: side by side along the columns, so no two of them need the same weight
 // bytes); each owns (BM/WM) x (BN/WN) of every matrix as 32 x 32 MFMA tiles.
 template <int FORMAT, int MODE, int BM, int BN, int WM, int WN>
-__global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 : 1) * BN == 256) ? 2 : 1) void grouped_gemm_kernel(GemmParams p) {
+__global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 && (MODE == kSwigluOfTwo ? 2 : 1) * BN == 256) ? 2 : 1) void grouped_gemm_kernel(GemmParams p) {
   constexpr bool PAIRED = MODE == kSwigluOfTwo || MODE == kSwigluOfTwoSplit;
   constexpr bool kSplitOut = MODE == kSwigluOfTwoSplit;
   constexpr bool kGated = MODE == kInterleavedGated;
@@ -200,7 +200,8 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   constexpr bool kPow2 = FORMAT == DEW_MOE_W_MXFP4 || (kSplit && !kFp8A);
   constexpr bool kBlockBank = FORMAT == DEW_MOE_W_FP8_BLOCK || kFp8Rows;  // one fp32 scale per 128 x 128 weights
   constexpr int kMatrices = PAIRED ? 2 : 1;
-  constexpr int kAtomK = kFp4 ? 64 : 32;       // depth an atom covers
+  constexpr bool kBf16 = FORMAT == DEW_MOE_W_BF16;  // unquantized matrices: the atoms are the fragments themselves
+  constexpr int kAtomK = kFp4 ? 64 : kBf16 ? 16 : 32;  // depth an atom covers
   constexpr int kStepDepth = kFp8A ? 128 : BK;  // depth a step covers: always 128 bytes of an A row
   constexpr int kAtoms = kStepDepth / kAtomK;  // 16-byte loads a lane makes per 32-column tile per step
   constexpr int kRowLoads = BM / 32;           // A rows a lane loads per step
@@ -214,7 +215,8 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   // shorter lookahead.
   // Quantized rows on the full 256 x 256 tile: a step's weights are 64 registers a lane, of which two sets fit
   // beside the accumulators (a load then has most of a 2048-cycle step to land).
-  constexpr int kSets = (kFp8A && BN == 256) ? 2 : (!kFp4 && BM == 128 && kMatrices * BN == 256) ? 3 : 4;
+  // (bf16 matrices: a step's raw data is twice FP8's, three sets of it fit beside the 256-row tile's accumulators)
+  constexpr int kSets = (kFp8A && BN == 256) ? 2 : (kBf16 || (!kFp4 && BM == 128 && kMatrices * BN == 256)) ? 3 : 4;
 
   extern __shared__ u32x4_t lds[];  // a ring of three stages of A: BM rows of 128 bytes each
   __shared__ int wave_tiles[4];
@@ -491,7 +493,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
     }
   };
   auto fetch = [&](const u32x4_t* stage, auto kk, auto into) __attribute__((always_inline)) {
-    const int chunk = kFp4 ? 4 * (lane / 32) + kk.value : 4 * (kk.value / 2) + 2 * (lane / 32) + kk.value % 2;
+    const int chunk = kFp4 ? 4 * (lane / 32) + kk.value : kBf16 ? 2 * kk.value + lane / 32 : 4 * (kk.value / 2) + 2 * (lane / 32) + kk.value % 2;
 #pragma unroll
     for (int i = 0; i < TI; ++i)
       a_frag[into.value][i] = __builtin_bit_cast(bf16x8_t, stage[swizzled(wm0 + 32 * i + lane % 32, chunk)]);
@@ -505,6 +507,8 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
                                         : __builtin_amdgcn_cvt_f32_fp8(s_regs[set.value][t], 1)) * 0.00390625f;
         const uint32_t word = b_regs[set.value][t][0][kk.value];
         b_frag[into.value][t] = kPow2 ? fragment_fp4_pow2(word, fp4_scale[t]) : fragment_fp4(word, fp4_scale[t]);
+      } else if constexpr (kBf16) {
+        b_frag[into.value][t] = __builtin_bit_cast(bf16x8_t, b_regs[set.value][t][kk.value]);
       } else {
         const float scale = FORMAT == DEW_MOE_W_FP8_BLOCK
                                 ? depth_scales[(t / TJ) * (BN / 128) + (wn0 + 32 * (t % TJ)) / 128][step / (128 / BK)]
@@ -608,7 +612,7 @@ __global__ __launch_bounds__(kThreads, (BM == 128 && (MODE == kSwigluOfTwo ? 2 :
   constexpr std::integral_constant<int, kTiles> b4{};
   constexpr std::integral_constant<int, kTiles> all_tiles{};
   constexpr int kMfmas = kMatrices * TI * TJ;
-  constexpr int kDequantOps = kTiles * (kPow2 ? 5 : 17);  // vector instructions to dequantize one slice
+  constexpr int kDequantOps = kBf16 ? 0 : kTiles * (kPow2 ? 5 : 17);  // vector instructions to dequantize one slice
   constexpr int kLoadsPerTile = kAtoms + (kFp4 || kMxRows ? 1 : 0);
   constexpr int kLoadsPerPhase = (kRowLoads + 3) / 4 + ((kTiles + 3) / 4) * kLoadsPerTile;
   // s_waitcnt vmcnt(kYounger) lgkmcnt(0): everything but the kYounger youngest vector-memory operations is done.
@@ -922,13 +926,13 @@ static int check_bank(const char* who, const dew_moe_bank* bank, const char* nam
   DEW_REQUIRE(bank, "%s: %s bank must not be null", who, name);
   DEW_REQUIRE(bank->layout == DEW_MOE_LAYOUT_PREPARED, "%s: %s bank is in the reference layout; call dew_moe_prepare_bank once at load", who, name);
   DEW_REQUIRE(bank->format == DEW_MOE_W_FP8_BLOCK || bank->format == DEW_MOE_W_FP8_CHANNEL || bank->format == DEW_MOE_W_NVFP4 ||
-                  bank->format == DEW_MOE_W_MXFP4 || bank->format == DEW_MOE_W_MXFP8,
+                  bank->format == DEW_MOE_W_MXFP4 || bank->format == DEW_MOE_W_MXFP8 || bank->format == DEW_MOE_W_BF16,
               "%s: %s bank has unknown format %d", who, name, bank->format);
   DEW_REQUIRE(bank->experts >= 1 && bank->experts <= 4096, "%s: %s bank has %d experts", who, name, bank->experts);
   DEW_REQUIRE(bank->depth >= 128 && bank->depth % 128 == 0, "%s: %s bank depth %d is not a multiple of 128", who, name, bank->depth);
   DEW_REQUIRE(bank->depth <= 128 * kMaxDepthBlocks, "%s: %s bank depth %d is above %d", who, name, bank->depth, 128 * kMaxDepthBlocks);
   DEW_REQUIRE(bank->width % 128 == 0 && bank->width >= 128, "%s: %s bank width %d is not a multiple of 128", who, name, bank->width);
-  DEW_REQUIRE(bank->codes && bank->scales, "%s: %s bank codes and scales must not be null", who, name);
+  DEW_REQUIRE(bank->codes && (bank->scales || bank->format == DEW_MOE_W_BF16), "%s: %s bank codes and scales must not be null", who, name);
   DEW_REQUIRE((bank->format != DEW_MOE_W_NVFP4 && bank->format != DEW_MOE_W_MXFP4) || bank->tensor_scale, "%s: %s NVFP4 bank needs tensor scales", who, name);
   DEW_REQUIRE(aligned16(bank->codes), "%s: %s bank codes must be 16-byte aligned", who, name);
   return DEW_MOE_OK;
@@ -980,7 +984,8 @@ static int tile_rows(const GemmParams& p, bool fp4) {
 
 template <int FORMAT, int MODE>
 static int launch_format(const char* who, const GemmParams& p, hipStream_t stream) {
-  constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4;
+  // (256-row tiles: the banks whose weights cost the vector unit little or nothing to bring to bf16)
+  constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4 || FORMAT == DEW_MOE_W_BF16;
   constexpr bool kPaired = MODE == kSwigluOfTwo;
   switch (tile_rows(p, kFp4)) {
     case 32:
@@ -1022,6 +1027,8 @@ static int launch(const char* who, const GemmParams& p, int format, hipStream_t 
       return launch_format<DEW_MOE_W_FP8_CHANNEL, MODE>(who, p, stream);
     case DEW_MOE_W_MXFP4:
       return launch_format<DEW_MOE_W_MXFP4, MODE>(who, p, stream);
+    case DEW_MOE_W_BF16:
+      return launch_format<DEW_MOE_W_BF16, MODE>(who, p, stream);
     case DEW_MOE_W_MXFP8:
       return fail(DEW_MOE_EINVAL, "%s: an MXFP8 bank multiplies MXFP8 rows (dew_moe_grouped_gemm_mxfp8_rows), not bf16 rows", who);
     default:

@@ -41,6 +41,29 @@ __global__ __launch_bounds__(256) void prepare_fp8_kernel(const uint8_t* __restr
   }
 }
 
+// bf16 matrices [E][K][N] -> atoms of 32 n x 16 k: lane 32 g + n holds depths 8 g .. 8 g + 7 of column n, the 16 bytes
+// the bf16 matrix instruction takes from it for one 16-deep slice. Atom order [E][N / 32][K / 16].
+__global__ __launch_bounds__(256) void prepare_bf16_kernel(const uint16_t* __restrict__ weights, uint8_t* __restrict__ out,
+                                                           int experts, int depth, int width) {
+  const int k_atoms = depth / 16, n_atoms = width / 32;
+  const long long total = static_cast<long long>(experts) * n_atoms * k_atoms * 64;
+  for (long long item = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; item < total;
+       item += static_cast<long long>(gridDim.x) * blockDim.x) {
+    const int lane = static_cast<int>(item % 64);
+    const long long atom = item / 64;
+    const int ka = static_cast<int>(atom % k_atoms);
+    const int na = static_cast<int>((atom / k_atoms) % n_atoms);
+    const int e = static_cast<int>(atom / (static_cast<long long>(k_atoms) * n_atoms));
+    const uint16_t* src = weights + (static_cast<size_t>(e) * depth + ka * 16 + 8 * (lane / 32)) * width + na * 32 + lane % 32;
+    uint32_t words[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      words[q] = static_cast<uint32_t>(src[static_cast<size_t>(2 * q) * width]) |
+                 (static_cast<uint32_t>(src[static_cast<size_t>(2 * q + 1) * width]) << 16);
+    *reinterpret_cast<uint4*>(out + item * 16) = make_uint4(words[0], words[1], words[2], words[3]);
+  }
+}
+
 // The eight E2M1 nibbles of a stored word (sign in bit 3), code j at bits 4 j of the result.
 __device__ __forceinline__ uint32_t nvfp4_natural_word(uint32_t s) {
   const uint32_t mask = 0x81C081C0u;
@@ -137,7 +160,7 @@ __global__ __launch_bounds__(256) void prepare_nvfp4_scales_kernel(const uint8_t
 
 static size_t codes_bytes(int format, int experts, int depth, int width) {
   const size_t elements = static_cast<size_t>(experts) * depth * width;
-  return format == DEW_MOE_W_NVFP4 ? elements / 2 : elements;
+  return format == DEW_MOE_W_NVFP4 ? elements / 2 : format == DEW_MOE_W_BF16 ? elements * 2 : elements;
 }
 
 }  // namespace dew
@@ -155,11 +178,11 @@ extern "C" int dew_moe_prepare_bank(const dew_moe_bank* ref, void* prepared, dew
   DEW_REQUIRE(ref && prepared && out, "dew_moe_prepare_bank: bank, prepared buffer and out must not be null");
   DEW_REQUIRE(ref->layout == DEW_MOE_LAYOUT_REFERENCE, "dew_moe_prepare_bank: the bank is already prepared");
   DEW_REQUIRE(ref->format == DEW_MOE_W_FP8_BLOCK || ref->format == DEW_MOE_W_FP8_CHANNEL || ref->format == DEW_MOE_W_NVFP4 ||
-                  ref->format == DEW_MOE_W_MXFP8,
+                  ref->format == DEW_MOE_W_MXFP8 || ref->format == DEW_MOE_W_BF16,
               "dew_moe_prepare_bank: unknown weight format %d", ref->format);
   DEW_REQUIRE(ref->experts >= 1 && ref->depth >= 1 && ref->width >= 1, "dew_moe_prepare_bank: bank [%d, %d, %d]",
               ref->experts, ref->depth, ref->width);
-  DEW_REQUIRE(ref->codes && ref->scales, "dew_moe_prepare_bank: codes and scales must not be null");
+  DEW_REQUIRE(ref->codes && (ref->scales || ref->format == DEW_MOE_W_BF16), "dew_moe_prepare_bank: codes and scales must not be null");
   DEW_REQUIRE(ref->width % 128 == 0, "dew_moe_prepare_bank: width %d is not a multiple of 128", ref->width);
   DEW_REQUIRE((reinterpret_cast<uintptr_t>(prepared) & 255u) == 0, "dew_moe_prepare_bank: prepared buffer must be 256-byte aligned");
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -186,6 +209,12 @@ extern "C" int dew_moe_prepare_bank(const dew_moe_bank* ref, void* prepared, dew
     if (hipMemcpyAsync(&found, general, sizeof(found), hipMemcpyDeviceToHost, s) != hipSuccess || hipStreamSynchronize(s) != hipSuccess)
       return fail(DEW_MOE_ELAUNCH, "dew_moe_prepare_bank: reading the scale summary back failed: %s", hipGetErrorString(hipGetLastError()));
     if (!found) out->format = DEW_MOE_W_MXFP4;
+  } else if (ref->format == DEW_MOE_W_BF16) {
+    DEW_REQUIRE(ref->depth % 128 == 0, "dew_moe_prepare_bank: a bf16 bank's depth is whole 128s, not %d", ref->depth);
+    hipLaunchKernelGGL(prepare_bf16_kernel, dim3(grid), dim3(256), 0, s, static_cast<const uint16_t*>(ref->codes),
+                       static_cast<uint8_t*>(prepared), ref->experts, ref->depth, ref->width);
+    if (int rc = launched("prepare_bf16_kernel")) return rc;
+    out->scales = nullptr;
   } else if (ref->format == DEW_MOE_W_MXFP8) {
     DEW_REQUIRE(ref->depth % 128 == 0, "dew_moe_prepare_bank: an MXFP8 bank's depth is whole 128s, not %d", ref->depth);
     DEW_REQUIRE(aligned16(ref->codes) && (reinterpret_cast<uintptr_t>(ref->scales) & 3u) == 0,

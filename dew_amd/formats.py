@@ -196,6 +196,30 @@ class Fp8Channels:
 
 
 @dataclasses.dataclass(frozen=True)
+class Bf16:
+    """Unquantized matrices `[E, K, N]` bf16 as the reference's experts hold them (`experts/*_proj/kernel`,
+    src/dew/nn/moe.py:1231-1235): the grouped product's plain operand (`expert_projection`,
+    src/dew/nn/moe.py:666-726), wrapped so that its one-time re-layout for the matrix cores is kept with it."""
+
+    weights: torch.Tensor
+
+    def __post_init__(self):
+        if self.weights.dtype != torch.bfloat16 or self.weights.ndim != 3:
+            raise ValueError(f"a bf16 bank is bfloat16 [E, K, N], not {self.weights.dtype} {tuple(self.weights.shape)}")
+
+    @property
+    def shape(self):
+        return tuple(self.weights.shape)
+
+    @property
+    def dtype(self):
+        return torch.bfloat16
+
+    def to(self, device) -> "Bf16":
+        return Bf16(self.weights.to(device))
+
+
+@dataclasses.dataclass(frozen=True)
 class MxFp8:
     """An MXFP8 bank of matrices, K-major as a product reads them (the reference's `MxFp8` operand,
     src/dew/nn/kernels/formats.py:186-194): e4m3 `codes [E, N, K]` (uint8) and one E8M0 `scales [E, N, K / 32]` byte

@@ -50,12 +50,17 @@ class GroupedCase:
     epilogue_operands: tuple = ()
 
 
-_BANKS = (formats.NvFp4, formats.Fp8Blocks, formats.Fp8Channels, formats.Layered, ops.PreparedBank)
+_BANKS = (formats.NvFp4, formats.Fp8Blocks, formats.Fp8Channels, formats.Bf16, formats.Layered, ops.PreparedBank)
 # (formats.MxFp8 multiplies MXFP8 rows only: projections.mxfp8_product)
 
 
 def _shape(bank):
-    return bank.shape
+    return tuple(bank.shape)
+
+
+def _is_bank(matrices) -> bool:
+    """A bank the kernels multiply: one of the formats, or the reference's plain operand, bf16 `[E, K, N]`."""
+    return isinstance(matrices, _BANKS) or (torch.is_tensor(matrices) and matrices.dtype == torch.bfloat16 and matrices.ndim == 3)
 
 
 def _bias_fits(case, bias) -> bool:
@@ -77,9 +82,9 @@ _EPILOGUES = {
 
 HIP = Kernel("hip", (
     Requirement("device", lambda c: c.lhs.is_cuda, "the rows are not on the GPU; the HIP kernels have no CPU path"),
-    Requirement("quantized-bank", lambda c: isinstance(c.rhs, _BANKS) and (c.paired is None or isinstance(c.paired, _BANKS)),
-                lambda c: f"the matrices are {type(c.rhs).__name__}; the kernels multiply NvFp4, Fp8Blocks and "
-                          f"Fp8Channels banks", row="dense bf16 banks"),
+    Requirement("quantized-bank", lambda c: _is_bank(c.rhs) and (c.paired is None or _is_bank(c.paired)),
+                lambda c: f"the matrices are {type(c.rhs).__name__}; the kernels multiply NvFp4, Fp8Blocks, Fp8Channels "
+                          f"and Bf16 banks", row="matrices of other dtypes"),
     Requirement("bf16", lambda c: c.lhs.dtype == torch.bfloat16 and c.compute == torch.bfloat16 and c.out_dtype == torch.bfloat16,
                 lambda c: f"rows {c.lhs.dtype}, compute {c.compute}, out {c.out_dtype}; the kernels compute and write bfloat16",
                 row="fp32 outputs"),
@@ -115,6 +120,8 @@ def prepared(bank) -> ops.PreparedBank:
     """The bank's one-time device re-layout, cached on the bank object."""
     if isinstance(bank, ops.PreparedBank):
         return bank
+    if torch.is_tensor(bank):  # the reference's plain operand: re-laid at every call, since a parameter may have changed
+        return ops.prepare(formats.Bf16(bank.contiguous()))
     if isinstance(bank, formats.Layered):  # the layer's matrices where they lie in the stack
         return prepared(bank.stack).layer(int(bank.layer), int(bank.layers))
     held = getattr(bank, "_prepared", None)

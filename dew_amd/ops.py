@@ -173,14 +173,17 @@ class PreparedBank:
         held = self.descriptor
         fp4 = held.format in (_lib.W_NVFP4, _lib.W_MXFP4)
         codes = depth * width // 2 if fp4 else depth * width
+        codes = depth * width * 2 if held.format == _lib.W_BF16 else codes
         scales = {_lib.W_FP8_BLOCK: (depth // 128) * (width // 128) * 4, _lib.W_FP8_CHANNEL: width * 4}.get(held.format, width * (depth // 16))
-        view = _lib.Bank(held.format, held.layout, experts, depth, width, held.codes + first * codes, held.scales + first * scales,
+        view = _lib.Bank(held.format, held.layout, experts, depth, width, held.codes + first * codes,
+                         None if not held.scales else held.scales + first * scales,
                          None if not held.tensor_scale else held.tensor_scale + first * 4)
         return PreparedBank(view, (experts, depth, width), self.keep)
 
 
 def prepare(bank) -> PreparedBank:
-    """The one-time re-layout of a `formats.NvFp4`, `formats.Fp8Blocks`, `formats.Fp8Channels` or `formats.MxFp8` bank."""
+    """The one-time re-layout of a `formats.NvFp4`, `formats.Fp8Blocks`, `formats.Fp8Channels`, `formats.MxFp8` or
+    `formats.Bf16` bank."""
     if isinstance(bank, PreparedBank):
         return bank
     if isinstance(bank, formats.NvFp4):
@@ -197,6 +200,9 @@ def prepare(bank) -> PreparedBank:
     elif isinstance(bank, formats.MxFp8):
         fmt, codes, scales, tensor = _lib.W_MXFP8, bank.codes, bank.scales, None
         _device(codes, "MxFp8.codes", torch.uint8), _device(scales, "MxFp8.scales", torch.uint8)
+    elif isinstance(bank, formats.Bf16):
+        fmt, codes, scales, tensor = _lib.W_BF16, bank.weights, None, None
+        _device(codes, "Bf16.weights", torch.bfloat16)
     else:
         raise KernelError(f"no HIP kernel multiplies a {type(bank).__name__} bank")
     experts, depth, width = bank.shape

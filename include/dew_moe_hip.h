@@ -38,9 +38,11 @@ enum {
                              /* MXFP4 banks arrive in this form (codecs.mxfp4_as_nvfp4).                */
   DEW_MOE_W_MXFP4 = 4,       /* prepared banks only: an NVFP4 bank whose block scales are all powers of */
                              /* two, as an MXFP4 checkpoint's are; dew_moe_prepare_bank finds it so.    */
-  DEW_MOE_W_MXFP8 = 5        /* OCP MXFP8, K-major as `formats.MxFp8` holds a product's matrices: codes */
+  DEW_MOE_W_MXFP8 = 5,       /* OCP MXFP8, K-major as `formats.MxFp8` holds a product's matrices: codes */
                              /* u8 e4m3 [E,N,K]; scales u8 e8m0 [E,N,K/32]. For dew_moe_grouped_gemm_   */
                              /* mxfp8_rows only.                                                        */
+  DEW_MOE_W_BF16 = 6         /* unquantized matrices as the reference holds them: codes bf16 [E,K,N]    */
+                             /* (`experts/*_proj/kernel`, src/dew/nn/moe.py:1231-1235); no scales.      */
 };
 
 enum { DEW_MOE_LAYOUT_REFERENCE = 0, DEW_MOE_LAYOUT_PREPARED = 1 };

@@ -51,6 +51,8 @@ def quantize(weight: torch.Tensor, quant: str):
         powers = codecs.mxfp4_tensor_powers(blocks, scales)
         assert powers is not None, "an N(0, 0.02) bank's group powers fit E4M3"
         return formats.NvFp4.of(*codecs.mxfp4_as_nvfp4(blocks, scales, powers))
+    if quant == "bf16":
+        return formats.Bf16(weight.to(torch.bfloat16))
     raise ValueError(quant)
 
 
@@ -89,4 +91,6 @@ def dequantized(bank):
         return oracle.dequantize_fp8_blocks(bank.codes.cpu().numpy(), bank.scale_inv.cpu().numpy()), None
     if isinstance(bank, formats.Fp8Channels):
         return oracle.dequantize_fp8_channels(bank.codes.cpu().numpy(), bank.scales.cpu().numpy()), None
+    if isinstance(bank, formats.Bf16):
+        return bank.weights.float().cpu().numpy(), None
     raise TypeError(type(bank))

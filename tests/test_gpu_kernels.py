@@ -112,7 +112,7 @@ SIZES = [("ragged", [130, 0, 1, 257, 64, 0, 127, 5]), ("single", [3]), ("even", 
 
 
 @pytest.mark.parametrize("tile", [0, 32, 64, 128])
-@pytest.mark.parametrize("quant", ["fp8_channel", "fp8_block", "mxfp4", "nvfp4"])
+@pytest.mark.parametrize("quant", ["fp8_channel", "fp8_block", "mxfp4", "nvfp4", "bf16"])
 @pytest.mark.parametrize("label,sizes", SIZES, ids=[s[0] for s in SIZES])
 def test_grouped_gemm_matches_the_dequantized_fp32_sum(ops, quant, label, sizes, tile):
     """bf16 x decoded-weight products are exact in fp32, so kernel and oracle differ by summation order
@@ -165,7 +165,7 @@ def test_grouped_gemm_gathers_scatters_and_zeroes_unrouted_rows(ops):
 
 
 @pytest.mark.parametrize("tile", [0, 32, 64, 128])
-@pytest.mark.parametrize("quant", ["fp8_channel", "fp8_block", "mxfp4", "nvfp4"])
+@pytest.mark.parametrize("quant", ["fp8_channel", "fp8_block", "mxfp4", "nvfp4", "bf16"])
 def test_gateup_swiglu_matches_the_two_products_and_the_rounded_epilogue(ops, quant, tile):
     sizes = [100, 0, 37, 200]
     rng = np.random.default_rng(21)
@@ -234,7 +234,7 @@ def test_entry_points_refuse_what_they_cannot_run(ops):
                          torch.zeros(3, dtype=torch.int32, device="cuda"))
 
 
-@pytest.mark.parametrize("quant", ["mxfp4", "nvfp4"])
+@pytest.mark.parametrize("quant", ["mxfp4", "nvfp4", "bf16"])
 def test_large_tile_kernels_match_the_oracle(ops, quant):
     """The 256-row tiles (paired 256 x 2 x 128, one bank 256 x 256), which launches take for FP4 banks whose groups
     average 1024 rows or more; forced here so that a small problem reaches them."""
@@ -269,7 +269,7 @@ def test_probes_run_and_the_copy_probe_copies(ops):
     assert ops.probe_mfma(torch.randn(16384, device="cuda").to(torch.bfloat16), 10) == 1024 * 4 * 10 * 16 * 32768.0
 
 
-@pytest.mark.parametrize("quant", ["fp8_channel", "fp8_block", "mxfp4", "nvfp4"])
+@pytest.mark.parametrize("quant", ["fp8_channel", "fp8_block", "mxfp4", "nvfp4", "bf16"])
 @pytest.mark.parametrize("depth", [128, 384, 640, 896])
 @pytest.mark.parametrize("label,sizes,tile", [("decode", [3, 0, 9], 32), ("small", [40, 70, 1], 64), ("medium", [150, 70, 1], 128),
                                                ("large", [800], 256)])
@@ -387,7 +387,7 @@ def test_the_expert_mlp_stays_on_split_rows_without_a_pass_between_its_products(
     assert (out == plain).mean() > 0.9
 
 
-@pytest.mark.parametrize("quant", ["fp8_block", "fp8_channel", "mxfp4", "nvfp4"])
+@pytest.mark.parametrize("quant", ["fp8_block", "fp8_channel", "mxfp4", "nvfp4", "bf16"])
 def test_a_layer_of_a_stacked_bank_is_read_where_it_lies(ops, quant):
     """`Layered(stack, layer)`: the grouped product of one layer's experts out of a bank stacking three layers', from
     the stack's own buffers, is the product of that layer's bank prepared alone, bit for bit."""
@@ -412,7 +412,7 @@ def test_a_layer_of_a_stacked_bank_is_read_where_it_lies(ops, quant):
         stack.layer(3, layers)
 
 
-@pytest.mark.parametrize("quant", ["fp8_block", "fp8_channel", "mxfp4", "nvfp4"])
+@pytest.mark.parametrize("quant", ["fp8_block", "fp8_channel", "mxfp4", "nvfp4", "bf16"])
 def test_last_tiles_of_at_most_64_rows_go_to_a_launch_of_their_own(ops, quant):
     """With 32 groups over 8 strips the 128-row tiles' launch leaves each group's last rows, where they are at most
     64, to a launch of 64-row tiles: every remainder from none to a full tile, both products and the paired one, are
