@@ -58,6 +58,9 @@ constexpr int kFormatMxFp8Rows = 19;
 // "bank" is the rhs_t quantized along the tokens and laid out as an MXFP8 bank of one expert whose depth is all the
 // tokens, and group g contracts the window of 128-token blocks its offsets name (dew_moe_kernel_gradient_mxfp8).
 constexpr int kFormatMxFp8Window = 20;
+// The kernel gradient of bf16 operands (the reference's `gemm_t`): lhs_t rows [depth, tokens] bf16 and the rhs_t as a
+// DEW_MOE_W_BF16 bank of one expert whose depth is all the tokens; windows in whole 64-token steps.
+constexpr int kFormatBf16Window = 21;
 
 constexpr int BK = 64;
 constexpr int kThreads = 256;
@@ -93,6 +96,8 @@ struct GemmParams {
   const int32_t* windows;
   int window_rows;
   float* out_f32;  // the product in fp32 (kPlainF32) instead of `out`
+  const float* factor0;  // a kernel gradient's fp32 sums times *factor0 * *factor1 before the rounding (each may be null):
+  const float* factor1;  // the tensor scales of NVFP4 operands
 };
 
 // What the epilogue writes: the rounded product (plus bias); SwiGLU of two banks' products; for one bank whose
@@ -191,8 +196,8 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   constexpr int kOutBN = kGated ? BN / 2 : BN;  // output columns of the tile
   static_assert(WM * WN == 4 && BM % (32 * WM) == 0 && BN % (32 * WN) == 0 && BM % 32 == 0, "tile shape");
   constexpr bool kFp8Rows = FORMAT == kFormatFp8Rows;   // e4m3 rows, one scale per row and 128 depths; 128 x 128 weight scales
-  constexpr bool kWindow = FORMAT == kFormatMxFp8Window;  // a kernel gradient: the same rows for every group, its own depths
-  constexpr bool kMxRows = FORMAT == kFormatMxFp8Rows || kWindow;  // e4m3 rows and weights, one scale per row (column) and 32 depths
+  constexpr bool kWindow = FORMAT == kFormatMxFp8Window || FORMAT == kFormatBf16Window;  // a kernel gradient: the same rows for every group, its own depths
+  constexpr bool kMxRows = FORMAT == kFormatMxFp8Rows || FORMAT == kFormatMxFp8Window;  // e4m3 rows and weights, one scale per row (column) and 32 depths
   constexpr bool kFp8A = kFp8Rows || kMxRows;           // both operands e4m3 codes: a step is 128 depths
   constexpr bool kSplit = FORMAT == kFormatMxSplit || FORMAT == kFormatMxSplitBlocks || kFp8A;  // A arrives as 8-bit codes
   constexpr bool kBlockScales = FORMAT == kFormatMxSplitBlocks || kFp8Rows;
@@ -200,7 +205,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   constexpr bool kPow2 = FORMAT == DEW_MOE_W_MXFP4 || (kSplit && !kFp8A);
   constexpr bool kBlockBank = FORMAT == DEW_MOE_W_FP8_BLOCK || kFp8Rows;  // one fp32 scale per 128 x 128 weights
   constexpr int kMatrices = PAIRED ? 2 : 1;
-  constexpr bool kBf16 = FORMAT == DEW_MOE_W_BF16;  // unquantized matrices: the atoms are the fragments themselves
+  constexpr bool kBf16 = FORMAT == DEW_MOE_W_BF16 || FORMAT == kFormatBf16Window;  // unquantized matrices: the atoms are the fragments themselves
   constexpr int kAtomK = kFp4 ? 64 : kBf16 ? 16 : 32;  // depth an atom covers
   constexpr int kStepDepth = kFp8A ? 128 : BK;  // depth a step covers: always 128 bytes of an A row
   constexpr int kAtoms = kStepDepth / kAtomK;  // 16-byte loads a lane makes per 32-column tile per step
@@ -302,7 +307,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
 
   const int row0 = found[1];
   const int valid_rows = min(BM, (kWindow ? (expert + 1) * p.window_rows : p.offsets[expert + 1]) - row0);
-  // a kernel gradient's group contracts its own whole 128-token blocks of the depth
+  // a kernel gradient's group contracts its own whole steps of the depth (128 tokens of e4m3 codes, 64 of bf16)
   const int first_step = kWindow ? min(max(p.windows[expert], 0), p.depth) / kStepDepth : 0;
   const int steps = kWindow ? max(min(max(p.windows[expert + 1], 0), p.depth) / kStepDepth - first_step, 0) : p.depth / kStepDepth;
   if (kWindow && steps == 0) {  // an empty group's gradient is zero
@@ -328,7 +333,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
     const int sorted = row0 + min(row, valid_rows - 1);
     const int source = kWindow ? sorted - expert * p.window_rows : p.gather ? p.gather[sorted] : sorted;
     // (a row of e4m3 codes is depth bytes.) Less the load's immediate offset, which the instruction adds back: see load_a
-    a_src[i] = p.x + static_cast<size_t>(source) * (kFp8A ? p.depth / 2 : p.depth) + first_step * (kStepDepth / 2) + chunk * 8 - (i % 4) * 512;
+    a_src[i] = p.x + static_cast<size_t>(source) * (kFp8A ? p.depth / 2 : p.depth) + first_step * (kFp8A ? kStepDepth / 2 : kStepDepth) + chunk * 8 - (i % 4) * 512;
     asm volatile("" : "+v"(a_src[i]));  // kept as computed: the compiler otherwise re-adds the bias at every load
   }
   // Split activations: the lane's row of each row tile carries one e8m0 scale; the hi term multiplies under it
@@ -777,6 +782,8 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
     factor0 = (kSplit ? 1.0f : 256.0f) * p.w0.tensor_scale[expert];
     if (PAIRED) factor1 = (kSplit ? 1.0f : 256.0f) * p.w1.tensor_scale[expert];
   }
+  float window_factor = 1.0f;
+  if constexpr (kWindow) window_factor = (p.factor0 ? *p.factor0 : 1.0f) * (p.factor1 ? *p.factor1 : 1.0f);
   if constexpr (MODE == kPlainF32) {
     // the fp32 sums as they are: a lane group's 32 lanes write 128 contiguous bytes of a row
 #pragma unroll
@@ -787,7 +794,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
         if (row < valid_rows) {
           float* out_row = p.out_f32 + static_cast<size_t>(row0 + row) * p.width + n0 + wn0 + lane % 32;
 #pragma unroll
-          for (int j = 0; j < TJ; ++j) out_row[32 * j] = acc[0][i][j][q];
+          for (int j = 0; j < TJ; ++j) out_row[32 * j] = acc[0][i][j][q] * window_factor;
         }
       }
     return;
@@ -854,6 +861,8 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
                      (static_cast<uint32_t>(swiglu_rounded(acc[0][i][j][q + 1] * factor0, acc[kMatrices - 1][i][j][q + 1] * factor1)) << 16);
             } else if constexpr (kFp4) {
               mine = pack_bf16(acc[0][i][j][q] * factor0 + bias[j], acc[0][i][j][q + 1] * factor0 + bias[j]);
+            } else if constexpr (kWindow) {
+              mine = pack_bf16(acc[0][i][j][q] * window_factor, acc[0][i][j][q + 1] * window_factor);
             } else {
               mine = pack_bf16(acc[0][i][j][q] + bias[j], acc[0][i][j][q + 1] + bias[j]);
             }
@@ -954,7 +963,7 @@ static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
   }
   // every expert may end in a partial tile, and the zeroed tail may add one more
   p.m_tile_bound = p.tail_of > 0 ? p.experts : (p.rows + BM - 1) / BM + p.experts + 1;
-  if (FORMAT == kFormatMxFp8Window) p.m_tile_bound = p.experts * ((p.window_rows + BM - 1) / BM);  // every group the same whole rows
+  if (FORMAT == kFormatMxFp8Window || FORMAT == kFormatBf16Window) p.m_tile_bound = p.experts * ((p.window_rows + BM - 1) / BM);  // every group the same whole rows
   const int total = p.m_tile_bound * (p.width / BN);
   const int blocks = ((total + 255) / 256) * 256;  // whole chunks of 32 tiles for each of the 8 XCDs
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreads), kShared, stream, p);
@@ -1230,6 +1239,47 @@ extern "C" int dew_moe_kernel_gradient_mxfp8(const void* lhs_t_codes, const uint
   }
   if (p.width % 256 == 0) return launch_tile<kFormatMxFp8Window, kPlain, 256, 256, 2, 2>(who, p, s);
   return launch_tile<kFormatMxFp8Window, kPlain, 256, 128, 2, 2>(who, p, s);
+}
+
+extern "C" int dew_moe_kernel_gradient_bf16(const void* lhs_t, const dew_moe_bank* rhs_t, const int32_t* offsets, const float* lhs_scale,
+                                            const float* rhs_scale, void* out, int32_t out_is_f32, int32_t depth, int32_t groups,
+                                            void* stream) {
+  using namespace dew;
+  const char* who = "dew_moe_kernel_gradient_bf16";
+  DEW_REQUIRE(rhs_t, "%s: the rhs_t bank must not be null", who);
+  DEW_REQUIRE(rhs_t->format == DEW_MOE_W_BF16 && rhs_t->layout == DEW_MOE_LAYOUT_PREPARED && rhs_t->experts == 1,
+              "%s: rhs_t is one prepared bf16 matrix [width, tokens] (dew_moe_transpose_columns, as a bank), not format %d, layout %d, %d experts",
+              who, rhs_t->format, rhs_t->layout, rhs_t->experts);
+  const int tokens = rhs_t->depth;
+  DEW_REQUIRE(tokens >= 0 && tokens % 128 == 0, "%s: %d tokens are not whole 128s", who, tokens);
+  DEW_REQUIRE(rhs_t->width >= 128 && rhs_t->width % 128 == 0, "%s: width %d is not a multiple of 128", who, rhs_t->width);
+  DEW_REQUIRE(depth >= 128 && depth % 128 == 0, "%s: depth %d is not a multiple of 128", who, depth);
+  DEW_REQUIRE(groups >= 1 && groups <= 4096, "%s: %d groups", who, groups);
+  DEW_REQUIRE(static_cast<long long>(groups) * depth < (1ll << 31), "%s: %d groups of %d rows overflow the row index", who, groups, depth);
+  DEW_REQUIRE(offsets && out && aligned16(out), "%s: offsets and out must not be null, out 16-byte aligned", who);
+  DEW_REQUIRE(tokens == 0 || (lhs_t && rhs_t->codes), "%s: the operands must not be null", who);
+  DEW_REQUIRE(aligned16(lhs_t) && aligned16(rhs_t->codes), "%s: the operands must be 16-byte aligned", who);
+  GemmParams p{};
+  p.x = static_cast<const bf16_t*>(lhs_t);
+  p.windows = offsets;
+  p.window_rows = depth;
+  p.factor0 = lhs_scale;
+  p.factor1 = rhs_scale;
+  p.w0 = BankView{static_cast<const uint8_t*>(rhs_t->codes), nullptr, nullptr};
+  p.w1 = p.w0;
+  p.out = static_cast<bf16_t*>(out);
+  p.out_f32 = static_cast<float*>(out);
+  p.experts = groups;
+  p.depth = tokens;
+  p.width = rhs_t->width;
+  p.rows = groups * depth;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (out_is_f32) {
+    if (p.width % 256 == 0) return launch_tile<kFormatBf16Window, kPlainF32, 256, 256, 1, 4>(who, p, s);
+    return launch_tile<kFormatBf16Window, kPlainF32, 256, 128, 1, 4>(who, p, s);
+  }
+  if (p.width % 256 == 0) return launch_tile<kFormatBf16Window, kPlain, 256, 256, 1, 4>(who, p, s);
+  return launch_tile<kFormatBf16Window, kPlain, 256, 128, 1, 4>(who, p, s);
 }
 
 extern "C" int dew_moe_gateup_swiglu_split_out(const void* x_split, const uint8_t* x_scale, const int32_t* gather,

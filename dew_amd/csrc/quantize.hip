@@ -256,6 +256,120 @@ __global__ __launch_bounds__(256) void quantize_columns_kernel(const bf16_t* __r
   }
 }
 
+// A kernel gradient's bf16 operands: x [tokens, dim] written transposed, as it is (`gemm_t`'s operands, reference
+// src/dew/nn/kernels/gemm.py:418-431) or, NVFP4 true, quantized ALONG THE TOKENS to the NVFP4 recipe's values (E2M1
+// codes under an E4M3 scale every 16 tokens, the tensor scale left to the product: quantize_rows_nvfp4_kernel's
+// arithmetic, reference src/dew/nn/kernels/projections.py:330-335). BANK false: rows [dim, tokens] bf16. BANK true: a
+// prepared DEW_MOE_W_BF16 bank of one expert, depth = tokens, width = dim: atoms [dim / 32][tokens / 16][64 lanes][8
+// bf16], lane 32 g + c holding tokens 8 g .. 8 g + 7 of column c. The same 128-token x 64-column tile and thread
+// ownership as quantize_columns_kernel.
+template <bool NVFP4, bool BANK>
+__global__ __launch_bounds__(256) void transpose_columns_kernel(const bf16_t* __restrict__ x, const uint32_t* __restrict__ largest,
+                                                                uint8_t* __restrict__ out, float* __restrict__ tensor_scale,
+                                                                int tokens, int dim) {
+  __shared__ uint32_t tile[128][33];
+  __shared__ u32x4_t staged[64][16];  // the rows operand's 64 rows of 256 bytes, chunk xor-swizzled by the row
+  const int tid = threadIdx.x;
+  const int t0 = blockIdx.x * 128, d0 = blockIdx.y * 64;
+  float tensor = 1.0f;
+  if constexpr (NVFP4) {
+    const float top = __uint_as_float(*largest << 16);
+    tensor = top > 0.0f ? fmaxf(top / 2688.0f, 1.17549435e-38f) : 1.0f;
+    if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) *tensor_scale = tensor;
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int item = tid + 256 * k, row = item / 8, chunk = item % 8;
+    const u32x4_t words = *reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(t0 + row) * dim + d0 + chunk * 8);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) tile[row][chunk * 4 + i] = words[i];
+  }
+  __syncthreads();
+  const int c = tid % 64, quarter = tid / 64;
+  uint32_t bits[32];  // the thread's 32 tokens of column c as bf16 patterns
+#pragma unroll
+  for (int i = 0; i < 32; ++i) {
+    const uint32_t word = tile[32 * quarter + i][c / 2];
+    bits[i] = c % 2 ? word >> 16 : word & 0xFFFFu;
+  }
+  if constexpr (NVFP4) {
+#pragma unroll
+    for (int block = 0; block < 2; ++block) {
+      float largest_of_block = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) largest_of_block = fmaxf(largest_of_block, fabsf(__uint_as_float(bits[16 * block + i] << 16)));
+      const float ratio = (largest_of_block / tensor) / 6.0f;
+      uint32_t byte = __builtin_amdgcn_cvt_pk_fp8_f32(fminf(ratio, 448.0f), 0.0f, 0, false) & 0xFFu;
+      if (__builtin_amdgcn_cvt_f32_fp8(byte, 0) < ratio) byte = min(byte + 1u, 0x7Eu);
+      const float each = __builtin_amdgcn_cvt_f32_fp8(byte, 0);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float value = __uint_as_float(bits[16 * block + i] << 16);
+        const float quotient = each > 0.0f ? (value / tensor) / each : 0.0f;
+        bits[16 * block + i] = __float_as_uint(copysignf(e2m1_nearest(fabsf(quotient)) * each, quotient)) >> 16;
+      }
+    }
+  }
+  u32x4_t pieces[4];  // 8 tokens each
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pieces[j][i] = bits[8 * j + 2 * i] | (bits[8 * j + 2 * i + 1] << 16);
+  if constexpr (BANK) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {  // piece j: atom 2 quarter + j / 2 of the tile's eight, lane group j % 2
+      const size_t atom = static_cast<size_t>((d0 + c) / 32) * (tokens / 16) + t0 / 16 + 2 * quarter + j / 2;
+      *reinterpret_cast<u32x4_t*>(out + (atom * 64 + 32 * (j % 2) + c % 32) * 16) = pieces[j];
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) staged[c][(4 * quarter + j) ^ (c & 15)] = pieces[j];
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int item = tid + 256 * k, row = item / 16, chunk = item % 16;
+      *reinterpret_cast<u32x4_t*>(out + (static_cast<size_t>(d0 + row) * tokens + t0) * 2 + chunk * 16) = staged[row][chunk ^ (row & 15)];
+    }
+  }
+}
+
+static int transpose_columns(const char* who, bool nvfp4, const void* x, void* out, float* tensor_scale, uint32_t* workspace, int tokens,
+                             int dim, int as_bank, void* stream) {
+  DEW_REQUIRE(tokens >= 0 && tokens % 128 == 0, "%s: %d tokens are not whole 128s", who, tokens);
+  DEW_REQUIRE(dim >= 128 && dim % 128 == 0, "%s: %d columns (whole 128s)", who, dim);
+  DEW_REQUIRE(!nvfp4 || (tensor_scale && workspace), "%s: tensor_scale and the 4-byte workspace must not be null", who);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (nvfp4) {
+    hipLaunchKernelGGL(absmax_clear_kernel, dim3(1), dim3(1), 0, s, workspace);
+    if (int rc = launched("absmax_clear_kernel")) return rc;
+  }
+  if (tokens == 0) {
+    if (nvfp4) {  // an operand of no tokens: the unit scale
+      hipLaunchKernelGGL(quantize_rows_nvfp4_kernel, dim3(1), dim3(64 * kQuantizeWaves), 0, s, static_cast<const bf16_t*>(nullptr), workspace,
+                         static_cast<bf16_t*>(nullptr), tensor_scale, 0, 0);
+      return launched("quantize_rows_nvfp4_kernel");
+    }
+    return DEW_MOE_OK;
+  }
+  DEW_REQUIRE(tokens / 128 <= 65535 * 32, "%s: %d tokens", who, tokens);
+  DEW_REQUIRE(x && out && aligned16(x) && aligned16(out), "%s: x and out must not be null and must be 16-byte aligned", who);
+  if (nvfp4) {
+    const long long chunks = static_cast<long long>(tokens) * dim / 8;
+    const int blocks = static_cast<int>(min((chunks + 255) / 256, 256ll * 16));
+    hipLaunchKernelGGL(absmax_kernel, dim3(blocks), dim3(256), 0, s, static_cast<const bf16_t*>(x), chunks, workspace);
+    if (int rc = launched("absmax_kernel")) return rc;
+  }
+  const dim3 grid(tokens / 128, dim / 64);
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, dim3(256), 0, s, static_cast<const bf16_t*>(x), workspace, static_cast<uint8_t*>(out), tensor_scale, tokens, dim);
+  };
+  if (nvfp4 && as_bank) launch(transpose_columns_kernel<true, true>);
+  else if (nvfp4) launch(transpose_columns_kernel<true, false>);
+  else if (as_bank) launch(transpose_columns_kernel<false, true>);
+  else launch(transpose_columns_kernel<false, false>);
+  return launched("transpose_columns_kernel");
+}
+
 static int quantize_columns(const char* who, bool mx, const void* x, void* codes, void* scales, int tokens, int dim, int as_bank,
                             void* stream) {
   DEW_REQUIRE(tokens >= 0 && tokens % 128 == 0, "%s: %d tokens are not whole 128-token blocks", who, tokens);
@@ -278,6 +392,15 @@ static int quantize_columns(const char* who, bool mx, const void* x, void* codes
 }
 
 }  // namespace dew
+
+extern "C" int dew_moe_transpose_columns(const void* x, void* out, int32_t tokens, int32_t dim, int32_t as_bank, void* stream) {
+  return dew::transpose_columns("dew_moe_transpose_columns", false, x, out, nullptr, nullptr, tokens, dim, as_bank, stream);
+}
+
+extern "C" int dew_moe_quantize_columns_nvfp4(const void* x, void* values, float* tensor_scale, uint32_t* workspace, int32_t tokens,
+                                              int32_t dim, int32_t as_bank, void* stream) {
+  return dew::transpose_columns("dew_moe_quantize_columns_nvfp4", true, x, values, tensor_scale, workspace, tokens, dim, as_bank, stream);
+}
 
 extern "C" int dew_moe_quantize_columns_fp8(const void* x, void* codes, void* scales, int32_t tokens, int32_t dim, int32_t as_bank,
                                             void* stream) {

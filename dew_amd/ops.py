@@ -543,6 +543,52 @@ def kernel_gradient_mxfp8(codes: torch.Tensor, scales: torch.Tensor, rhs_t: Prep
     return out
 
 
+def transpose_columns(x: torch.Tensor, *, nvfp4: bool = False, as_bank: bool):
+    """bf16 `[tokens, dim]` written transposed, a bf16 kernel gradient's operand (`dew_moe_transpose_columns`), or, `nvfp4`,
+    its NVFP4 values along the tokens short of the tensor scale (`dew_moe_quantize_columns_nvfp4`). The lhs_t operand
+    (`as_bank` false) is bf16 `[dim, tokens]`; the rhs_t operand a `PreparedBank` of one bf16 matrix, depth the tokens,
+    width `dim`. Returns (operand, tensor scale f32 `[1]` or None)."""
+    _device(x, "x", torch.bfloat16)
+    tokens, dim = x.shape
+    out = torch.empty((dim, tokens) if not as_bank else (max(tokens * dim, 8),), dtype=torch.bfloat16, device=x.device)
+    scale = None
+    if nvfp4:
+        scale = torch.empty(1, dtype=torch.float32, device=x.device)
+        workspace = torch.empty(1, dtype=torch.int32, device=x.device)
+        _lib.check(_lib.library().dew_moe_quantize_columns_nvfp4(_ptr(x), _ptr(out), _ptr(scale), _ptr(workspace), tokens, dim,
+                                                                 int(as_bank), _stream()), "dew_moe_quantize_columns_nvfp4")
+    else:
+        _lib.check(_lib.library().dew_moe_transpose_columns(_ptr(x), _ptr(out), tokens, dim, int(as_bank), _stream()),
+                   "dew_moe_transpose_columns")
+    if not as_bank:
+        return out, scale
+    view = _lib.Bank(_lib.W_BF16, _lib.LAYOUT_PREPARED, 1, tokens, dim, _ptr(out), None, None)
+    return PreparedBank(view, (1, tokens, dim), (out,)), scale
+
+
+def kernel_gradient_bf16(lhs_t: torch.Tensor, rhs_t: PreparedBank, offsets: torch.Tensor, *, lhs_scale: torch.Tensor | None = None,
+                         rhs_scale: torch.Tensor | None = None, out_dtype=torch.bfloat16) -> torch.Tensor:
+    """Each group's tokens contracted over bf16 operands: `out[g] = lhs_t[:, tokens of g] @ rhs_t[:, tokens of g]^T` times
+    the two scales, `[groups, depth, width]` in bf16 or fp32; `lhs_t [depth, tokens]` bf16 and the bank `[width, tokens]`
+    from `transpose_columns`; `offsets` int32 `[groups + 1]` in whole 64-token steps; an empty group's is zero."""
+    _, tokens, width = rhs_t.shape
+    _device(lhs_t, "lhs_t", torch.bfloat16), _device(offsets, "offsets", torch.int32)
+    depth = lhs_t.shape[0]
+    if tuple(lhs_t.shape) != (depth, tokens) or rhs_t.descriptor.format != _lib.W_BF16:
+        raise KernelError(f"the lhs_t operand is bfloat16 [depth, {tokens}] and the rhs_t a bf16 bank")
+    if out_dtype not in (torch.bfloat16, torch.float32):
+        raise KernelError(f"a kernel gradient is written in bfloat16 or float32, not {out_dtype}")
+    for name, scale in (("lhs_scale", lhs_scale), ("rhs_scale", rhs_scale)):
+        if scale is not None:
+            _device(scale, name, torch.float32)
+    groups = offsets.numel() - 1
+    out = torch.empty((groups, depth, width), dtype=out_dtype, device=lhs_t.device)
+    _lib.check(_lib.library().dew_moe_kernel_gradient_bf16(_ptr(lhs_t), rhs_t.descriptor, _ptr(offsets), _ptr(lhs_scale), _ptr(rhs_scale),
+                                                           _ptr(out), int(out_dtype == torch.float32), depth, groups, _stream()),
+               "dew_moe_kernel_gradient_bf16")
+    return out
+
+
 def operand_order_fp8(codes: torch.Tensor) -> torch.Tensor:
     """e4m3 codes `[rows, K]` in depth order -> the order `quantize_rows_fp8` writes and `grouped_gemm_fp8_rows`
     reads: of each 128 depths, byte 16 (4 g + 2 t + h) + b holds depth 64 t + 32 h + 16 g + b."""

@@ -245,3 +245,16 @@ def mxfp8_gradients(x: torch.Tensor, w: torch.Tensor, cotangent: torch.Tensor, g
     d_x = mxfp8_projection(cotangent, w.transpose(1, 2).contiguous(), group_blocks, out_dtype=x.dtype)
     return d_x, kernel_gradient(x, cotangent, group_blocks, mx=True, out_dtype=out_dtype)
 
+
+def nvfp4_gradients(x: torch.Tensor, w: torch.Tensor, cotangent: torch.Tensor, group_blocks, *, out_dtype=torch.bfloat16):
+    """`_nvfp4_backward` (src/dew/nn/kernels/projections.py:322-337) -> (d_x, d_w): the NVFP4 product of the cotangent
+    and the matrices, both quantized along the width; and each group's tokens contracted over `x` and the cotangent
+    quantized along the tokens, every 16 a scale. The decoded operands short of their tensor scales are exact in bf16,
+    so the contraction is the bf16 kernel gradient with both tensor scales applied to its fp32 sums."""
+    d_x = nvfp4_projection(cotangent, w.transpose(1, 2).contiguous(), group_blocks, out_dtype=x.dtype)
+    rows, rows_scale = ops.transpose_columns(x.contiguous(), nvfp4=True, as_bank=False)
+    bank, bank_scale = ops.transpose_columns(cotangent.contiguous(), nvfp4=True, as_bank=True)
+    d_w = ops.kernel_gradient_bf16(rows, bank, _group_offsets(group_blocks, x.device), lhs_scale=rows_scale, rhs_scale=bank_scale,
+                                   out_dtype=out_dtype)
+    return d_x, d_w
+

@@ -233,6 +233,25 @@ int dew_moe_quantize_columns_mxfp8(const void* x /* bf16 [tokens, dim] */, void*
 int dew_moe_kernel_gradient_mxfp8(const void* lhs_t_codes, const uint8_t* lhs_t_scales, const dew_moe_bank* rhs_t,
                                   const int32_t* offsets, void* out, int32_t out_is_f32, int32_t depth, int32_t groups,
                                   void* stream);
+/* The kernel gradient of bf16 operands: the reference's `gemm_t` src/dew/nn/kernels/gemm.py:418-431 (each group's rows
+ * of lhs transposed times its rows of rhs, fp32 sums), and with it the NVFP4 recipe's `_nvfp4_backward`
+ * src/dew/nn/kernels/projections.py:322-337 (both operands quantized along the tokens, every 16 a scale, decoded, the
+ * tensor scales applied).
+ * dew_moe_transpose_columns: x bf16 [tokens, dim] -> the lhs_t operand, rows [dim, tokens] bf16 (as_bank 0), or the
+ * rhs_t operand in the layout of a prepared DEW_MOE_W_BF16 bank of one expert, depth = tokens, width = dim (as_bank 1:
+ * atoms [dim / 32][tokens / 16][64][8 bf16]). dew_moe_quantize_columns_nvfp4: the same with every value replaced by its
+ * NVFP4 value short of the tensor scale (E2M1 code x the E4M3 scale of its 16 tokens; dew_moe_quantize_rows_nvfp4's
+ * arithmetic along the tokens) and *tensor_scale written; workspace is 4 bytes of device memory.
+ * dew_moe_kernel_gradient_bf16: out [groups, depth, width] (bf16, or fp32 where out_is_f32) = lhs_t[:, tokens of g] x
+ * rhs_t[:, tokens of g]^T, exact products, fp32 sums, times *lhs_scale x *rhs_scale (device floats, each may be null),
+ * one rounding. Group g contracts tokens offsets[g] .. offsets[g + 1], whole 64-token steps. 256 x 256 tiles.        */
+int dew_moe_transpose_columns(const void* x /* bf16 [tokens, dim] */, void* out, int32_t tokens, int32_t dim,
+                              int32_t as_bank, void* stream);
+int dew_moe_quantize_columns_nvfp4(const void* x /* bf16 [tokens, dim] */, void* values, float* tensor_scale,
+                                   uint32_t* workspace, int32_t tokens, int32_t dim, int32_t as_bank, void* stream);
+int dew_moe_kernel_gradient_bf16(const void* lhs_t, const dew_moe_bank* rhs_t, const int32_t* offsets,
+                                 const float* lhs_scale, const float* rhs_scale, void* out, int32_t out_is_f32,
+                                 int32_t depth, int32_t groups, void* stream);
 /* The NVFP4 recipe's rows (`NvFp4Block.quantized` src/dew/nn/kernels/formats.py:263-274 over `bits.nvfp4_coded`
  * src/dew/algebra/bits.py:941-982): E2M1 codes under an E4M3 scale every 16 depths and one tensor scale (the
  * operand's largest magnitude over 6 x 448). The instruction has no such operand (its block scales are powers of two

@@ -643,6 +643,20 @@ def mxfp8_gradients(x, w, cotangent, group_blocks, *, dtype="bfloat16"):
     return d_x, kernel_gradient(rows_t, dy_t, sizes, dtype=dtype)
 
 
+def nvfp4_gradients(x, w, cotangent, group_blocks, *, dtype="bfloat16"):
+    """`_nvfp4_backward` (src/dew/nn/kernels/projections.py:322-337): d_x = the NVFP4 block product of the cotangent and
+    the matrices both quantized along the width; d_w = each group's tokens contracted over `x.T` and `cotangent.T`
+    quantized along the tokens (every 16 a scale) and decoded with their tensor scales, summed at the highest precision.
+    Returns (d_x, d_w). (`nvfp4_quantized` and `nvfp4_projection` are defined below.)"""
+    sizes = np.asarray(group_blocks) * SCALE_DEPTH
+    d_x = nvfp4_projection(cotangent, np.swapaxes(np.asarray(w, F32), 1, 2), sizes, dtype=dtype)
+    decoded = []
+    for operand in (x, cotangent):
+        values, scales, tensor = nvfp4_quantized(np.asarray(operand, F32).T)
+        decoded.append(values.astype(np.float64) * np.repeat(scales.astype(np.float64), 16, axis=1) * np.float64(tensor))
+    return d_x, kernel_gradient(decoded[0], decoded[1], sizes, dtype=dtype)
+
+
 # --------------------------------------------------------------------------------------------------
 # The NVFP4 recipe's forward product (E2M1 codes, an E4M3 scale every 16 depths, one tensor scale)
 # --------------------------------------------------------------------------------------------------

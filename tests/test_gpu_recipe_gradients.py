@@ -111,3 +111,83 @@ def test_the_input_gradient_is_the_recipes_own_product(ops, mx):
     assert np.abs(bf16_np(d_x) - want_x).max() <= 2.0 ** -7 * np.abs(want_x).max()
     assert np.abs(bf16_np(d_w) - want_w).max() <= 2.0 ** -7 * np.abs(want_w).max()
     assert (bf16_np(d_x) == want_x).mean() > 0.97 and (bf16_np(d_w) == want_w).mean() > 0.97
+
+
+# ---- bf16 operands: the reference's gemm_t, and the NVFP4 recipe's kernel gradient ------------------------------
+
+
+def bf16_bank_rows(bank, tokens, dim):
+    """A `transpose_columns(as_bank=True)` bank's matrix `[dim, tokens]`."""
+    atoms = bank.keep[0][:tokens * dim].cpu().view(dim // 32, tokens // 16, 2, 32, 8)
+    return atoms.permute(0, 3, 1, 2, 4).reshape(dim, tokens)
+
+
+@pytest.mark.parametrize("tokens,dim", [(128, 128), (384, 256), (1024, 640)])
+def test_tokens_are_transposed_bit_for_bit_in_both_layouts(ops, tokens, dim):
+    x = tokens_case(tokens, dim, seed=tokens + dim + 3)
+    rows, none = ops.transpose_columns(x.cuda(), as_bank=False)
+    assert none is None and torch.equal(rows.cpu(), x.T)
+    bank, _ = ops.transpose_columns(x.cuda(), as_bank=True)
+    assert torch.equal(bf16_bank_rows(bank, tokens, dim), x.T)
+    # the NVFP4 values along the tokens: the oracle's quantizer on the transpose
+    want_values, want_scales, want_tensor = oracle.nvfp4_quantized(bf16_np(x).T)
+    want = want_values * np.repeat(want_scales, 16, axis=1)
+    rows, scale = ops.transpose_columns(x.cuda(), nvfp4=True, as_bank=False)
+    assert scale.item() == want_tensor and np.array_equal(bf16_np(rows), want)
+    bank, scale = ops.transpose_columns(x.cuda(), nvfp4=True, as_bank=True)
+    assert scale.item() == want_tensor and np.array_equal(bf16_np(bf16_bank_rows(bank, tokens, dim)), want)
+
+
+@pytest.mark.parametrize("label,blocks", GROUPS, ids=[g[0] for g in GROUPS])
+@pytest.mark.parametrize("depth,width", [(256, 256), (384, 384), (128, 512)])
+def test_gemm_t_matches_the_oracle(ops, label, blocks, depth, width):
+    from dew_amd import gemm
+
+    tokens = 128 * sum(blocks)
+    rng = np.random.default_rng(depth + tokens)
+    x = torch.from_numpy(rng.standard_normal((tokens, depth)).astype(np.float32)).to(torch.bfloat16)
+    dy = torch.from_numpy(rng.standard_normal((tokens, width)).astype(np.float32)).to(torch.bfloat16)
+    sizes = np.asarray(blocks) * 128
+    want = oracle.kernel_gradient(bf16_np(x).T, bf16_np(dy).T, sizes, dtype="float32")
+    scale = np.abs(want).max()
+    device_sizes = torch.tensor(sizes, dtype=torch.int32).cuda()
+    got = gemm.gemm_t(x.cuda(), dy.cuda(), device_sizes, out_dtype=torch.float32).cpu().numpy()
+    for group, count in enumerate(blocks):
+        if count == 0:
+            assert not got[group].any()
+    assert np.abs(got - want).max() <= 2.0 ** -18 * scale
+    rounded = bf16_np(gemm.gemm_t(x.cuda(), dy.cuda(), device_sizes))
+    assert np.abs(rounded - oracle.bf16_round(want)).max() <= 2.0 ** -7 * scale
+    assert (rounded == oracle.bf16_round(want)).mean() > 0.99
+
+
+def test_gemm_t_takes_groups_of_whole_64_row_steps(ops):
+    from dew_amd import gemm
+
+    sizes = np.asarray([64, 192, 0, 128])
+    rng = np.random.default_rng(9)
+    x = torch.from_numpy(rng.standard_normal((384, 128)).astype(np.float32)).to(torch.bfloat16)
+    dy = torch.from_numpy(rng.standard_normal((384, 256)).astype(np.float32)).to(torch.bfloat16)
+    want = oracle.kernel_gradient(bf16_np(x).T, bf16_np(dy).T, sizes, dtype="float32")
+    got = gemm.gemm_t(x.cuda(), dy.cuda(), torch.tensor(sizes, dtype=torch.int32).cuda(), out_dtype=torch.float32).cpu().numpy()
+    assert np.abs(got - want).max() <= 2.0 ** -18 * np.abs(want).max()
+
+
+def test_the_nvfp4_gradients_match_the_oracle(ops):
+    from dew_amd import projections
+
+    blocks, depth, width = (1, 0, 2, 1), 256, 512        # (an NVFP4 bank's depth, here also the width, is whole 256s)
+    tokens = 128 * sum(blocks)
+    rng = np.random.default_rng(6)
+    x = torch.from_numpy(rng.standard_normal((tokens, depth)).astype(np.float32)).to(torch.bfloat16)
+    dy = torch.from_numpy(rng.standard_normal((tokens, width)).astype(np.float32)).to(torch.bfloat16)
+    w = torch.from_numpy((rng.standard_normal((len(blocks), depth, width)) * 0.05).astype(np.float32)).to(torch.bfloat16)
+    want_x, want_w = oracle.nvfp4_gradients(bf16_np(x), bf16_np(w), bf16_np(dy), blocks)
+    d_x, d_w = projections.nvfp4_gradients(x.cuda(), w.cuda(), dy.cuda(), blocks)
+    assert d_x.shape == x.shape and d_w.shape == w.shape
+    assert np.abs(bf16_np(d_x) - want_x).max() <= 2.0 ** -7 * np.abs(want_x).max()
+    assert np.abs(bf16_np(d_w) - want_w).max() <= 2.0 ** -7 * np.abs(want_w).max()
+    assert (bf16_np(d_x) == want_x).mean() > 0.97 and (bf16_np(d_w) == want_w).mean() > 0.97
+    wide = projections.nvfp4_gradients(x.cuda(), w.cuda(), dy.cuda(), blocks, out_dtype=torch.float32)[1].cpu().numpy()
+    exact = oracle.nvfp4_gradients(bf16_np(x), bf16_np(w), bf16_np(dy), blocks, dtype="float32")[1]
+    assert np.abs(wide - exact).max() <= 2.0 ** -18 * np.abs(exact).max()

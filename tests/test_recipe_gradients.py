@@ -65,3 +65,20 @@ def test_the_mxfp8_gradients_are_exact_where_the_format_is():
     d_x, d_w = oracle.mxfp8_gradients(x, w, dy, BLOCKS, dtype="float32")
     want_x, want_w = _exact_gradients(x, w, dy)
     assert np.array_equal(d_x, want_x) and np.array_equal(d_w, want_w)
+
+
+def test_the_nvfp4_gradients_are_exact_where_the_format_is():
+    """E2M1 holds {0, .5, 1, 1.5, 2, 3, 4, 6}: operands drawn from them with every operand's largest magnitude 6 (the
+    tensor scale is then 1 / 448 and every block scale 448 or, for blocks whose largest is 3, 224)."""
+    rng = np.random.default_rng(3)
+    grid = np.array([0, 0.5, 1, 1.5, 2, 3, 4, 6, -0.5, -1, -1.5, -2, -3, -4, -6], np.float32)
+    depth, width, tokens = 128, 256, 128 * sum(BLOCKS)
+    x, dy = rng.choice(grid, size=(tokens, depth)), rng.choice(grid, size=(tokens, width))
+    w = rng.choice(grid, size=(len(BLOCKS), depth, width))
+    for each in (x, dy):
+        each[::16, :], each[:, ::16] = 6.0, 6.0     # every block of 16, along either axis, holds a 6
+    w[:, ::16, :], w[:, :, ::16] = 6.0, 6.0
+    d_x, d_w = oracle.nvfp4_gradients(x, w, dy, BLOCKS, dtype="float32")
+    want_x, want_w = _exact_gradients(x, w, dy)
+    assert np.abs(d_x - want_x).max() <= 2.0 ** -21 * np.abs(want_x).max()      # (448 x 1 / 448 rounds in fp32)
+    assert np.abs(d_w - want_w).max() <= 2.0 ** -21 * np.abs(want_w).max()
