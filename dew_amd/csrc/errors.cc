@@ -52,6 +52,8 @@ const char* dew_moe_kernels(void) {
          "split_rows | quantize_rows_fp8 | quantize_rows_mxfp8,1 row/wave,-,-,4,-,bf16 rows -> e4m3 terms | e4m3 codes in operand order + e8m0 scales\n"
          "grouped_gemm<bf16>,32|64|128|256,128|256,64,3,v_mfma_f32_32x32x16_bf16,unquantized bf16 matrices as fragment atoms: no dequantization\n"
          "grouped_gemm<mxfp8 window>,256,256 | 128,128,4 (2x2),v_mfma_scale_f32_32x32x64_f8f6f4,a kernel gradient: each group's window of 128-token steps of lhs_t rows x the rhs_t bank; bf16 or fp32 out\n"
+         "grouped_gemm<bf16 window>,256,256 | 128,64,3,v_mfma_f32_32x32x16_bf16,gemm_t: each group's window of 64-token steps of bf16 lhs_t rows x the bf16 rhs_t bank; tensor scales on the sums\n"
+         "transpose_columns,128 tokens x 64 columns/block,-,-,4,-,bf16 [tokens x dim] transposed (or its NVFP4 values along the tokens): rows or bf16 bank atoms\n"
          "quantize_columns,128 tokens x 64 columns/block,-,-,4,-,bf16 [tokens x dim] -> e4m3 along the tokens and transposed: operand rows or bank atoms + e8m0 scales\n"
          "absmax + quantize_rows_nvfp4,1 row/wave,-,-,4,-,bf16 rows -> bf16 (e2m1 code x e4m3 scale) + the tensor scale\n"
          "combine,8 columns/lane,-,-,4,-,bf16 slots x f32 weights\n";
