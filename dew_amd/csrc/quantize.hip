@@ -263,14 +263,61 @@ __global__ __launch_bounds__(256) void quantize_columns_kernel(const bf16_t* __r
 // prepared DEW_MOE_W_BF16 bank of one expert, depth = tokens, width = dim: atoms [dim / 32][tokens / 16][64 lanes][8
 // bf16], lane 32 g + c holding tokens 8 g .. 8 g + 7 of column c. The same 128-token x 64-column tile and thread
 // ownership as quantize_columns_kernel.
+// With `offsets` (groups + 1 of them) the groups are ragged: each is written from a whole 64-token step on, its last
+// step filled with zeros, so that the product's windows need no mask; `tokens` is then the padded extent (at least
+// the rows plus 64 a group, in whole 128s), the tokens past the last group are zeros, and `padded` receives the
+// groups' offsets in the written order. Every block scans the group sizes itself (at most 4096 of them).
+constexpr int kMaxPaddedGroups = 4096;
+
 template <bool NVFP4, bool BANK>
 __global__ __launch_bounds__(256) void transpose_columns_kernel(const bf16_t* __restrict__ x, const uint32_t* __restrict__ largest,
                                                                 uint8_t* __restrict__ out, float* __restrict__ tensor_scale,
-                                                                int tokens, int dim) {
+                                                                int tokens, int dim, const int32_t* __restrict__ offsets, int groups,
+                                                                int32_t* __restrict__ padded, int rows) {
   __shared__ uint32_t tile[128][33];
   __shared__ u32x4_t staged[64][16];  // the rows operand's 64 rows of 256 bytes, chunk xor-swizzled by the row
+  __shared__ int source_row[128];     // the row of x each of the block's tokens is, -1 for a token of padding
+  __shared__ int starts[kMaxPaddedGroups + 1];
+  __shared__ int partial[256];
   const int tid = threadIdx.x;
   const int t0 = blockIdx.x * 128, d0 = blockIdx.y * 64;
+  if (offsets == nullptr) {
+    if (tid < 128) source_row[tid] = t0 + tid;
+  } else {
+    // padded start of every group: an exclusive scan of the sizes rounded up to whole 64s
+    const int each = (groups + 255) / 256;
+    int sum = 0;
+    for (int g = tid * each; g < min((tid + 1) * each, groups); ++g) sum += (offsets[g + 1] - offsets[g] + 63) / 64 * 64;
+    partial[tid] = sum;
+    __syncthreads();
+    for (int offset = 1; offset < 256; offset <<= 1) {
+      const int other = tid >= offset ? partial[tid - offset] : 0;
+      __syncthreads();
+      partial[tid] += other;
+      __syncthreads();
+    }
+    int running = partial[tid] - sum;
+    for (int g = tid * each; g < min((tid + 1) * each, groups); ++g) {
+      starts[g] = running;
+      running += (offsets[g + 1] - offsets[g] + 63) / 64 * 64;
+    }
+    if (tid == 255) starts[groups] = partial[255];
+    __syncthreads();
+    if (blockIdx.x == 0 && blockIdx.y == 0)
+      for (int g = tid; g <= groups; g += 256) padded[g] = starts[g];
+    if (tid < 128) {
+      const int token = t0 + tid;
+      int low = 0, high = groups;  // the last group that starts at or before the token
+      while (high - low > 1) {
+        const int middle = (low + high) / 2;
+        if (starts[middle] <= token) low = middle; else high = middle;
+      }
+      const int within = token - starts[low];
+      const int source = offsets[low] + within;  // (offsets that leave x's rows read nothing)
+      source_row[tid] = (token < starts[groups] && within < offsets[low + 1] - offsets[low] && source >= 0 && source < rows) ? source : -1;
+    }
+  }
+  __syncthreads();
   float tensor = 1.0f;
   if constexpr (NVFP4) {
     const float top = __uint_as_float(*largest << 16);
@@ -280,7 +327,9 @@ __global__ __launch_bounds__(256) void transpose_columns_kernel(const bf16_t* __
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
     const int item = tid + 256 * k, row = item / 8, chunk = item % 8;
-    const u32x4_t words = *reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(t0 + row) * dim + d0 + chunk * 8);
+    const int source = source_row[row];
+    u32x4_t words = {0, 0, 0, 0};
+    if (source >= 0) words = *reinterpret_cast<const u32x4_t*>(x + static_cast<size_t>(source) * dim + d0 + chunk * 8);
 #pragma unroll
     for (int i = 0; i < 4; ++i) tile[row][chunk * 4 + i] = words[i];
   }
@@ -334,8 +383,15 @@ __global__ __launch_bounds__(256) void transpose_columns_kernel(const bf16_t* __
 }
 
 static int transpose_columns(const char* who, bool nvfp4, const void* x, void* out, float* tensor_scale, uint32_t* workspace, int tokens,
-                             int dim, int as_bank, void* stream) {
+                             int dim, int as_bank, void* stream, int rows = -1, const int32_t* offsets = nullptr, int groups = 0,
+                             int32_t* padded = nullptr) {
+  if (rows < 0) rows = tokens;  // (ragged groups: `rows` of x are written into `tokens` padded ones)
   DEW_REQUIRE(tokens >= 0 && tokens % 128 == 0, "%s: %d tokens are not whole 128s", who, tokens);
+  if (offsets) {
+    DEW_REQUIRE(groups >= 1 && groups <= kMaxPaddedGroups && padded, "%s: %d groups (at most %d) and their padded offsets", who, groups, kMaxPaddedGroups);
+    DEW_REQUIRE(rows >= 0 && static_cast<long long>(tokens) >= static_cast<long long>(rows) + 64ll * groups,
+                "%s: %d padded tokens do not hold %d rows in %d groups of whole 64s", who, tokens, rows, groups);
+  }
   DEW_REQUIRE(dim >= 128 && dim % 128 == 0, "%s: %d columns (whole 128s)", who, dim);
   DEW_REQUIRE(!nvfp4 || (tensor_scale && workspace), "%s: tensor_scale and the 4-byte workspace must not be null", who);
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -354,14 +410,15 @@ static int transpose_columns(const char* who, bool nvfp4, const void* x, void* o
   DEW_REQUIRE(tokens / 128 <= 65535 * 32, "%s: %d tokens", who, tokens);
   DEW_REQUIRE(x && out && aligned16(x) && aligned16(out), "%s: x and out must not be null and must be 16-byte aligned", who);
   if (nvfp4) {
-    const long long chunks = static_cast<long long>(tokens) * dim / 8;
+    const long long chunks = static_cast<long long>(rows) * dim / 8;
     const int blocks = static_cast<int>(min((chunks + 255) / 256, 256ll * 16));
     hipLaunchKernelGGL(absmax_kernel, dim3(blocks), dim3(256), 0, s, static_cast<const bf16_t*>(x), chunks, workspace);
     if (int rc = launched("absmax_kernel")) return rc;
   }
   const dim3 grid(tokens / 128, dim / 64);
   auto launch = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, grid, dim3(256), 0, s, static_cast<const bf16_t*>(x), workspace, static_cast<uint8_t*>(out), tensor_scale, tokens, dim);
+    hipLaunchKernelGGL(kernel, grid, dim3(256), 0, s, static_cast<const bf16_t*>(x), workspace, static_cast<uint8_t*>(out), tensor_scale, tokens, dim,
+                       offsets, groups, padded, rows);
   };
   if (nvfp4 && as_bank) launch(transpose_columns_kernel<true, true>);
   else if (nvfp4) launch(transpose_columns_kernel<true, false>);
@@ -395,6 +452,14 @@ static int quantize_columns(const char* who, bool mx, const void* x, void* codes
 
 extern "C" int dew_moe_transpose_columns(const void* x, void* out, int32_t tokens, int32_t dim, int32_t as_bank, void* stream) {
   return dew::transpose_columns("dew_moe_transpose_columns", false, x, out, nullptr, nullptr, tokens, dim, as_bank, stream);
+}
+
+extern "C" int dew_moe_transpose_groups(const void* x, const int32_t* offsets, void* out, int32_t* padded_offsets, int32_t rows,
+                                        int32_t padded_tokens, int32_t dim, int32_t groups, int32_t as_bank, void* stream) {
+  using namespace dew;
+  DEW_REQUIRE(offsets, "dew_moe_transpose_groups: offsets must not be null");
+  return transpose_columns("dew_moe_transpose_groups", false, x, out, nullptr, nullptr, padded_tokens, dim, as_bank, stream, rows, offsets, groups,
+                           padded_offsets);
 }
 
 extern "C" int dew_moe_quantize_columns_nvfp4(const void* x, void* values, float* tensor_scale, uint32_t* workspace, int32_t tokens,

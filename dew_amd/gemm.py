@@ -161,16 +161,22 @@ def gemm(lhs: torch.Tensor, rhs, group_sizes, *, paired=None, gather: torch.Tens
             ops.grouped_gemm(lhs, second, groups.offsets, gather=gather))
 
 
-def gemm_t(lhs: torch.Tensor, rhs: torch.Tensor, group_sizes, *, out_dtype=torch.bfloat16) -> torch.Tensor:
+def gemm_t(lhs: torch.Tensor, rhs: torch.Tensor, group_sizes, *, out_dtype=torch.bfloat16, whole_steps: bool = False) -> torch.Tensor:
     """Each group's rows of `lhs [rows, depth]` transposed times its rows of `rhs [rows, width]`: `[groups, depth,
     width]` in `out_dtype`, an empty group's zero, exact bf16 products summed in fp32 (the reference's `gemm_t`,
     src/dew/nn/kernels/gemm.py:418-431: a grouped product's kernel gradient). Both operands are written transposed
-    first (one pass each) so that the contraction runs along contiguous tokens. The groups are whole 64-row steps (a
-    recipe pads them to 128s); `rows` whole 128s."""
+    first (one pass each) so that the contraction runs along contiguous tokens, each group from a whole 64-token step
+    on with zeros filling its last step, so the groups are of any sizes and rows past them add nothing. A caller whose
+    groups are whole 64-row steps and whose rows whole 128s (a recipe pads them so) says `whole_steps` and saves the
+    padding."""
     groups = GroupSizes.of(group_sizes)
-    rows_t, _ = ops.transpose_columns(lhs.contiguous(), as_bank=False)
-    bank, _ = ops.transpose_columns(rhs.contiguous(), as_bank=True)
-    return ops.kernel_gradient_bf16(rows_t, bank, groups.offsets, out_dtype=out_dtype)
+    if whole_steps:
+        rows_t, _ = ops.transpose_columns(lhs.contiguous(), as_bank=False)
+        bank, _ = ops.transpose_columns(rhs.contiguous(), as_bank=True)
+        return ops.kernel_gradient_bf16(rows_t, bank, groups.offsets, out_dtype=out_dtype)
+    rows_t, padded = ops.transpose_groups(lhs.contiguous(), groups.offsets, as_bank=False)
+    bank, _ = ops.transpose_groups(rhs.contiguous(), groups.offsets, as_bank=True)
+    return ops.kernel_gradient_bf16(rows_t, bank, padded, out_dtype=out_dtype)
 
 
 def swiglu_mlp_on_split_rows(lhs: torch.Tensor, gate, up, down, group_sizes, *, gather: torch.Tensor | None = None,

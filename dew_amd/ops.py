@@ -566,6 +566,24 @@ def transpose_columns(x: torch.Tensor, *, nvfp4: bool = False, as_bank: bool):
     return PreparedBank(view, (1, tokens, dim), (out,)), scale
 
 
+def transpose_groups(x: torch.Tensor, offsets: torch.Tensor, *, as_bank: bool):
+    """`transpose_columns` for ragged groups (`dew_moe_transpose_groups`): each group of `x [rows, dim]`'s rows is written
+    from a whole 64-token step on, zeros filling its last step. Returns (operand over the padded tokens, the groups'
+    padded offsets int32 `[groups + 1]`, which are `kernel_gradient_bf16`'s)."""
+    _device(x, "x", torch.bfloat16), _device(offsets, "offsets", torch.int32)
+    rows, dim = x.shape
+    groups = offsets.numel() - 1
+    tokens = (rows + 64 * groups + 127) // 128 * 128
+    out = torch.empty((dim, tokens) if not as_bank else (tokens * dim,), dtype=torch.bfloat16, device=x.device)
+    padded = torch.empty(groups + 1, dtype=torch.int32, device=x.device)
+    _lib.check(_lib.library().dew_moe_transpose_groups(_ptr(x), _ptr(offsets), _ptr(out), _ptr(padded), rows, tokens, dim, groups,
+                                                       int(as_bank), _stream()), "dew_moe_transpose_groups")
+    if not as_bank:
+        return out, padded
+    view = _lib.Bank(_lib.W_BF16, _lib.LAYOUT_PREPARED, 1, tokens, dim, _ptr(out), None, None)
+    return PreparedBank(view, (1, tokens, dim), (out,)), padded
+
+
 def kernel_gradient_bf16(lhs_t: torch.Tensor, rhs_t: PreparedBank, offsets: torch.Tensor, *, lhs_scale: torch.Tensor | None = None,
                          rhs_scale: torch.Tensor | None = None, out_dtype=torch.bfloat16) -> torch.Tensor:
     """Each group's tokens contracted over bf16 operands: `out[g] = lhs_t[:, tokens of g] @ rhs_t[:, tokens of g]^T` times

@@ -247,6 +247,14 @@ int dew_moe_kernel_gradient_mxfp8(const void* lhs_t_codes, const uint8_t* lhs_t_
  * one rounding. Group g contracts tokens offsets[g] .. offsets[g + 1], whole 64-token steps. 256 x 256 tiles.        */
 int dew_moe_transpose_columns(const void* x /* bf16 [tokens, dim] */, void* out, int32_t tokens, int32_t dim,
                               int32_t as_bank, void* stream);
+/* dew_moe_transpose_groups: dew_moe_transpose_columns for ragged groups (`gemm_t`'s `group_sizes` are any sizes): x bf16
+ * [rows, dim], group g its rows offsets[g] .. offsets[g + 1] (device int32 [groups + 1]); each group is written from a
+ * whole 64-token step on and its last step filled with zeros, into padded_tokens tokens (whole 128s, at least rows +
+ * 64 * groups; the rest zeros); padded_offsets [groups + 1] receives the groups' offsets in the written order, which
+ * are dew_moe_kernel_gradient_bf16's. At most 4096 groups.                                                        */
+int dew_moe_transpose_groups(const void* x /* bf16 [rows, dim] */, const int32_t* offsets, void* out,
+                             int32_t* padded_offsets, int32_t rows, int32_t padded_tokens, int32_t dim, int32_t groups,
+                             int32_t as_bank, void* stream);
 int dew_moe_quantize_columns_nvfp4(const void* x /* bf16 [tokens, dim] */, void* values, float* tensor_scale,
                                    uint32_t* workspace, int32_t tokens, int32_t dim, int32_t as_bank, void* stream);
 int dew_moe_kernel_gradient_bf16(const void* lhs_t, const dew_moe_bank* rhs_t, const int32_t* offsets,

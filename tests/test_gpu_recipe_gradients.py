@@ -161,16 +161,39 @@ def test_gemm_t_matches_the_oracle(ops, label, blocks, depth, width):
     assert (rounded == oracle.bf16_round(want)).mean() > 0.99
 
 
-def test_gemm_t_takes_groups_of_whole_64_row_steps(ops):
+RAGGED = [("ragged", [130, 0, 1, 257, 64, 0, 127, 5]), ("single", [3]), ("steps", [64, 192, 0, 128]), ("tail", [100, 30])]
+
+
+@pytest.mark.parametrize("label,sizes", RAGGED, ids=[r[0] for r in RAGGED])
+def test_gemm_t_takes_groups_of_any_sizes(ops, label, sizes):
+    """Each group padded to whole 64-token steps by the transposer: every boundary inside a step, empty groups, rows
+    past the last group (which belong to no group and add nothing), and the same groups as whole steps."""
     from dew_amd import gemm
 
-    sizes = np.asarray([64, 192, 0, 128])
-    rng = np.random.default_rng(9)
-    x = torch.from_numpy(rng.standard_normal((384, 128)).astype(np.float32)).to(torch.bfloat16)
-    dy = torch.from_numpy(rng.standard_normal((384, 256)).astype(np.float32)).to(torch.bfloat16)
+    sizes = np.asarray(sizes)
+    rows = int(sizes.sum()) + 9                         # nine rows no group owns
+    rng = np.random.default_rng(rows)
+    x = torch.from_numpy(rng.standard_normal((rows, 128)).astype(np.float32)).to(torch.bfloat16)
+    dy = torch.from_numpy(rng.standard_normal((rows, 256)).astype(np.float32)).to(torch.bfloat16)
     want = oracle.kernel_gradient(bf16_np(x).T, bf16_np(dy).T, sizes, dtype="float32")
-    got = gemm.gemm_t(x.cuda(), dy.cuda(), torch.tensor(sizes, dtype=torch.int32).cuda(), out_dtype=torch.float32).cpu().numpy()
+    device_sizes = torch.tensor(sizes, dtype=torch.int32).cuda()
+    got = gemm.gemm_t(x.cuda(), dy.cuda(), device_sizes, out_dtype=torch.float32).cpu().numpy()
     assert np.abs(got - want).max() <= 2.0 ** -18 * np.abs(want).max()
+    for group, size in enumerate(sizes):
+        if size == 0:
+            assert not got[group].any()
+    rows_t, padded = ops.transpose_groups(x.cuda(), torch.tensor(np.concatenate([[0], np.cumsum(sizes)]), dtype=torch.int32).cuda(), as_bank=False)
+    starts = np.concatenate([[0], np.cumsum((sizes + 63) // 64 * 64)])
+    assert padded.cpu().tolist() == starts.tolist()
+    held = bf16_np(rows_t)
+    for group, size in enumerate(sizes):
+        first = int(np.sum(sizes[:group]))
+        assert np.array_equal(held[:, starts[group]:starts[group] + size], bf16_np(x)[first:first + size].T)
+        assert not held[:, starts[group] + size:starts[group + 1]].any()
+    assert not held[:, starts[-1]:].any()
+    if label == "steps":
+        whole = gemm.gemm_t(x[:384].cuda(), dy[:384].cuda(), device_sizes, out_dtype=torch.float32, whole_steps=True).cpu().numpy()
+        assert np.array_equal(whole, got)
 
 
 def test_the_nvfp4_gradients_match_the_oracle(ops):
