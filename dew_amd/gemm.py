@@ -188,6 +188,8 @@ def swiglu_mlp_on_split_rows(lhs: torch.Tensor, gate, up, down, group_sizes, *, 
     them, so no bf16 hidden rows are written at all. The same selector decides the call."""
     if not SPLIT_ROWS or not (torch.is_tensor(lhs) and lhs.is_cuda and lhs.dtype == torch.bfloat16):
         return None
+    if any(torch.is_tensor(bank) or isinstance(bank, formats.Bf16) for bank in (gate, up, down)):
+        return None  # unquantized matrices have no FP4 codes for the scaled instruction (and a plain tensor is not re-laid to find out)
     named = None if implementation in (None, "auto") else implementation
     selection.select(GROUPED, GroupedCase(lhs, gate, up, "swiglu"), named)
     first, second, third = prepared(gate), prepared(up), prepared(down)

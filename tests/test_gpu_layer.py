@@ -228,3 +228,26 @@ def test_the_router_sows_its_scores_and_log_partition_and_the_bias_balances(scor
     want = start.cpu().numpy() + oracle.load_balance_update(counts.cpu().numpy(), 0.001)
     assert np.array_equal(stepped.cpu().numpy(), want.astype(np.float32))
     assert np.array_equal(moe.load_balance_update(counts, 0.25).cpu().numpy(), oracle.load_balance_update(counts.cpu().numpy(), 0.25))
+
+
+def test_unquantized_bf16_experts_run_through_the_layer_as_plain_tensors():
+    """The reference's own operand: bf16 `[E, K, N]` parameters handed to the layer as tensors (re-laid at every call)
+    give the products of the same matrices wrapped as `formats.Bf16` (re-laid once), bit for bit, and match the
+    oracle's layer on the decoded (here: identical) weights."""
+    from dew_amd import formats, gemm
+
+    rng = np.random.default_rng(77)
+    experts, depth, width, sizes = 4, 256, 384, [70, 0, 129, 33]
+    rows = int(np.sum(sizes))
+    x = torch.from_numpy(rng.standard_normal((rows, depth)).astype(np.float32)).to(torch.bfloat16).cuda()
+    gate, up = (torch.from_numpy((rng.standard_normal((experts, depth, width)) * 0.05).astype(np.float32)).to(torch.bfloat16).cuda()
+                for _ in range(2))
+    group_sizes = torch.tensor(sizes, dtype=torch.int32).cuda()
+    plain = gemm.gemm(x, gate, group_sizes, paired=up, epilogue="swiglu")
+    kept = gemm.gemm(x, formats.Bf16(gate), group_sizes, paired=formats.Bf16(up), epilogue="swiglu")
+    assert torch.equal(plain, kept)
+    want = oracle.swiglu(oracle.grouped_matmul(x.float().cpu().numpy(), gate.float().cpu().numpy(), sizes),
+                         oracle.grouped_matmul(x.float().cpu().numpy(), up.float().cpu().numpy(), sizes))
+    got = plain.float().cpu().numpy()
+    assert np.abs(got - want).max() <= 2.0 ** -6 * np.abs(want).max() and (got == want).mean() > 0.9
+
