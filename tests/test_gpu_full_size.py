@@ -67,3 +67,43 @@ def test_full_size_configuration(name):
         dense = ops.gateup_swiglu(data["x"], stepper.shared[0], stepper.shared[1], stepper.dense_offsets)
         want_out = (want_out.float() + ops.grouped_gemm(dense, stepper.shared[2], stepper.dense_offsets).float()).to(torch.bfloat16)
     assert torch.equal(out, want_out)
+
+
+@pytest.mark.parametrize("recipe", ["blockwise_fp8", "mxfp8", "bf16"])
+def test_full_size_kernel_gradient_partitions_its_tokens(recipe):
+    """Mixtral-8x7B's gate projection at the benchmark's routed rows (32768 x 4096 x 14336), where no CPU sum follows:
+    the gradient of one group holding every token is the sum of the eight groups' gradients (the same products in
+    other windows: fp32 rounding of the sums apart), a group's gradient does not depend on its neighbours, and a
+    sample of its elements is the oracle's exact sum of the same quantized operands."""
+    from dew_amd import gemm, ops, projections
+
+    device = torch.device("cuda:0")
+    generator = torch.Generator(device=device).manual_seed(0)
+    tokens, depth, width, groups = 32768, 4096, 14336, 8
+    x = torch.randn((tokens, depth), device=device, generator=generator).to(torch.bfloat16)
+    dy = torch.randn((tokens, width), device=device, generator=generator).to(torch.bfloat16)
+    each = tokens // groups // 128
+    if recipe == "bf16":
+        gradient = lambda blocks: gemm.gemm_t(x, dy, torch.tensor(blocks, dtype=torch.int32, device=device) * 128,
+                                              out_dtype=torch.float32, whole_steps=True)
+    else:
+        gradient = lambda blocks: projections.kernel_gradient(x, dy, blocks, mx=recipe == "mxfp8", out_dtype=torch.float32)
+    apart = gradient([each] * groups)
+    whole = gradient([each * groups])[0]
+    scale = float(whole.abs().max())
+    assert float((apart.sum(dim=0) - whole).abs().max()) <= 2.0 ** -12 * scale
+    uneven = gradient([each, 0, 2 * each, each] + [each] * (groups - 4))
+    assert torch.equal(uneven[0], apart[0]) and not bool(uneven[1].any()) and torch.equal(uneven[3], apart[3])
+    # group 5's first 64 x 64 elements against the exact sums of the same operands
+    span = slice(5 * each * 128, 6 * each * 128)
+    left, right = x[span, :64].float().cpu().numpy(), dy[span, :64].float().cpu().numpy()
+    if recipe == "bf16":
+        want = oracle.kernel_gradient(left.T, right.T, [each * 128], dtype="float32")[0]
+    elif recipe == "mxfp8":
+        want = oracle.kernel_gradient(oracle.mxfp8_decoded(*oracle.mxfp8_quantized(left.T)), oracle.mxfp8_decoded(*oracle.mxfp8_quantized(right.T)),
+                                      [each * 128], dtype="float32")[0]
+    else:
+        (lv, ls), (rv, rs) = oracle.rows_quantized(left.T), oracle.rows_quantized(right.T)
+        want = oracle.blockwise_fp8_kernel_gradient(lv, rv, [each], ls.T, rs.T, dtype="float32")[0]
+    got = apart[5, :64, :64].cpu().numpy()
+    assert np.abs(got - want).max() <= 2.0 ** -12 * np.abs(want).max()
