@@ -47,6 +47,12 @@ What pins each function (tests/test_oracle_golden.py):
   brute force over the E2M1 grid for the rounding; `nvfp4_block_product` against the float64 sum of the decoded
   operands.
 
+* `kernel_gradient` / `blockwise_fp8_kernel_gradient` and the recipes' `*_gradients` (tests/test_recipe_gradients.py):
+  the kernel gradient against the block-by-block definition the reference's own test writes out
+  (tests/test_gemm_blockwise.py:97-107, with its shapes, its empty group and scales drawn from [0.5, 2)); both
+  gradients of each recipe against the exact derivative (d_x = dy @ w^T, d_w[g] = x_g^T @ dy_g) on operands the format
+  holds exactly, where quantizing changes nothing: a wrong axis, transpose, group window or scale pairing fails it.
+
 Parity unpinned (no byte fixture in the reference, closed form only): the exact bits of the softmax
 denominator's compensated sum (src/dew/nn/precision.py:1832); it moves router weights by at most one fp32
 ulp and no index. `gpt_oss_gating`'s bf16 mode: where each bf16 rounding falls follows JAX's arithmetic on
