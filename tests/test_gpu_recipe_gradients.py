@@ -214,3 +214,35 @@ def test_the_nvfp4_gradients_match_the_oracle(ops):
     wide = projections.nvfp4_gradients(x.cuda(), w.cuda(), dy.cuda(), blocks, out_dtype=torch.float32)[1].cpu().numpy()
     exact = oracle.nvfp4_gradients(bf16_np(x), bf16_np(w), bf16_np(dy), blocks, dtype="float32")[1]
     assert np.abs(wide - exact).max() <= 2.0 ** -18 * np.abs(exact).max()
+
+
+def test_the_gradients_entry_points_refuse_what_they_cannot_run(ops):
+    from dew_amd._lib import KernelError
+
+    odd = torch.zeros((100, 128), dtype=torch.bfloat16, device="cuda")
+    whole = torch.zeros((128, 128), dtype=torch.bfloat16, device="cuda")
+    narrow = torch.zeros((128, 64), dtype=torch.bfloat16, device="cuda")
+    offsets = torch.tensor([0, 128], dtype=torch.int32, device="cuda")
+    for call in (lambda x: ops.quantize_columns(x, mx=False, as_bank=False), lambda x: ops.quantize_columns(x, mx=True, as_bank=True),
+                 lambda x: ops.transpose_columns(x, as_bank=False), lambda x: ops.transpose_columns(x, nvfp4=True, as_bank=True)):
+        with pytest.raises(KernelError, match="whole 128"):
+            call(odd)                                   # tokens in whole 128s (ragged groups go through transpose_groups)
+        with pytest.raises(KernelError, match="whole 128"):
+            call(narrow)                                # columns in whole 128s
+        with pytest.raises(KernelError, match="GPU"):
+            call(whole.cpu())
+    codes, scales = ops.quantize_columns(whole, mx=True, as_bank=False)
+    fp8_bank, (bf16_bank, _) = ops.quantize_columns(whole, mx=True, as_bank=True), ops.transpose_columns(whole, as_bank=True)
+    with pytest.raises(KernelError, match="MXFP8"):
+        ops._lib.check(ops._lib.library().dew_moe_kernel_gradient_mxfp8(codes.data_ptr(), scales.data_ptr(), bf16_bank.descriptor, offsets.data_ptr(),
+                                                                        whole.data_ptr(), 0, 128, 1, None), "dew_moe_kernel_gradient_mxfp8")
+    with pytest.raises(KernelError, match="bf16"):
+        ops.kernel_gradient_bf16(whole, fp8_bank, offsets)
+    with pytest.raises(KernelError, match="float32"):
+        ops.kernel_gradient_mxfp8(codes, scales, fp8_bank, offsets, out_dtype=torch.float16)
+    # an operand of no tokens: nothing to contract, every group's gradient zero
+    none = torch.zeros((0, 128), dtype=torch.bfloat16, device="cuda")
+    rows_t, _ = ops.transpose_columns(none, as_bank=False)
+    empty_bank, _ = ops.transpose_columns(none, as_bank=True)
+    zero = ops.kernel_gradient_bf16(rows_t, empty_bank, torch.zeros(3, dtype=torch.int32, device="cuda"), out_dtype=torch.float32)
+    assert zero.shape == (2, 128, 128) and not zero.any()
