@@ -10,7 +10,7 @@ from pathlib import Path
 LIBRARY = Path(__file__).resolve().parent / "libdew_moe_hip.so"
 
 W_FP8_BLOCK, W_FP8_CHANNEL, W_NVFP4, W_MXFP4, W_MXFP8, W_BF16 = 1, 2, 3, 4, 5, 6
-LAYOUT_REFERENCE, LAYOUT_PREPARED = 0, 1
+LAYOUT_REFERENCE, LAYOUT_PREPARED, LAYOUT_REFERENCE_KMAJOR = 0, 1, 2
 SCORE_SOFTMAX, SCORE_SIGMOID = 0, 1
 
 EXPORTS = (

@@ -37,7 +37,7 @@ def products(recipe: str, x, w, dy, blocks, offsets):
     """(name, prepare call, product call) for the recipe's three products, operands prepared once outside the timing."""
     sizes = offsets[1:] - offsets[:-1]
     if recipe == "bf16":
-        bank, bank_t = ops.prepare(formats.Bf16(w)), ops.prepare(formats.Bf16(w.transpose(1, 2).contiguous()))
+        bank, bank_t = ops.prepare(formats.Bf16(w)), ops.prepare(formats.Bf16(w).T)
         rows_t, _ = ops.transpose_columns(x, as_bank=False)
         dy_bank, _ = ops.transpose_columns(dy, as_bank=True)
         return [("forward", None, lambda: ops.grouped_gemm(x, bank, offsets)),

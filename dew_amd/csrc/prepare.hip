@@ -64,6 +64,24 @@ __global__ __launch_bounds__(256) void prepare_bf16_kernel(const uint16_t* __res
   }
 }
 
+// The same atoms from matrices held K-major, [E][N][K] (a bf16 bank read as its transpose): a lane's 8 depths are 16
+// contiguous bytes of its column's row.
+__global__ __launch_bounds__(256) void prepare_bf16_kmajor_kernel(const uint16_t* __restrict__ weights, uint8_t* __restrict__ out,
+                                                                  int experts, int depth, int width) {
+  const int k_atoms = depth / 16, n_atoms = width / 32;
+  const long long total = static_cast<long long>(experts) * n_atoms * k_atoms * 64;
+  for (long long item = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; item < total;
+       item += static_cast<long long>(gridDim.x) * blockDim.x) {
+    const int lane = static_cast<int>(item % 64);
+    const long long atom = item / 64;
+    const int ka = static_cast<int>(atom % k_atoms);
+    const int na = static_cast<int>((atom / k_atoms) % n_atoms);
+    const int e = static_cast<int>(atom / (static_cast<long long>(k_atoms) * n_atoms));
+    const uint16_t* src = weights + (static_cast<size_t>(e) * width + na * 32 + lane % 32) * depth + ka * 16 + 8 * (lane / 32);
+    *reinterpret_cast<uint4*>(out + item * 16) = *reinterpret_cast<const uint4*>(src);
+  }
+}
+
 // The eight E2M1 nibbles of a stored word (sign in bit 3), code j at bits 4 j of the result.
 __device__ __forceinline__ uint32_t nvfp4_natural_word(uint32_t s) {
   const uint32_t mask = 0x81C081C0u;
@@ -176,7 +194,8 @@ extern "C" size_t dew_moe_prepared_bytes(int32_t format, int32_t experts, int32_
 extern "C" int dew_moe_prepare_bank(const dew_moe_bank* ref, void* prepared, dew_moe_bank* out, void* stream) {
   using namespace dew;
   DEW_REQUIRE(ref && prepared && out, "dew_moe_prepare_bank: bank, prepared buffer and out must not be null");
-  DEW_REQUIRE(ref->layout == DEW_MOE_LAYOUT_REFERENCE, "dew_moe_prepare_bank: the bank is already prepared");
+  DEW_REQUIRE(ref->layout == DEW_MOE_LAYOUT_REFERENCE || (ref->layout == DEW_MOE_LAYOUT_REFERENCE_KMAJOR && ref->format == DEW_MOE_W_BF16),
+              "dew_moe_prepare_bank: the bank is already prepared (layout %d)", ref->layout);
   DEW_REQUIRE(ref->format == DEW_MOE_W_FP8_BLOCK || ref->format == DEW_MOE_W_FP8_CHANNEL || ref->format == DEW_MOE_W_NVFP4 ||
                   ref->format == DEW_MOE_W_MXFP8 || ref->format == DEW_MOE_W_BF16,
               "dew_moe_prepare_bank: unknown weight format %d", ref->format);
@@ -211,8 +230,14 @@ extern "C" int dew_moe_prepare_bank(const dew_moe_bank* ref, void* prepared, dew
     if (!found) out->format = DEW_MOE_W_MXFP4;
   } else if (ref->format == DEW_MOE_W_BF16) {
     DEW_REQUIRE(ref->depth % 128 == 0, "dew_moe_prepare_bank: a bf16 bank's depth is whole 128s, not %d", ref->depth);
-    hipLaunchKernelGGL(prepare_bf16_kernel, dim3(grid), dim3(256), 0, s, static_cast<const uint16_t*>(ref->codes),
-                       static_cast<uint8_t*>(prepared), ref->experts, ref->depth, ref->width);
+    if (ref->layout == DEW_MOE_LAYOUT_REFERENCE_KMAJOR) {
+      DEW_REQUIRE(aligned16(ref->codes), "dew_moe_prepare_bank: K-major bf16 matrices must be 16-byte aligned");
+      hipLaunchKernelGGL(prepare_bf16_kmajor_kernel, dim3(grid), dim3(256), 0, s, static_cast<const uint16_t*>(ref->codes),
+                         static_cast<uint8_t*>(prepared), ref->experts, ref->depth, ref->width);
+    } else {
+      hipLaunchKernelGGL(prepare_bf16_kernel, dim3(grid), dim3(256), 0, s, static_cast<const uint16_t*>(ref->codes),
+                         static_cast<uint8_t*>(prepared), ref->experts, ref->depth, ref->width);
+    }
     if (int rc = launched("prepare_bf16_kernel")) return rc;
     out->scales = nullptr;
   } else if (ref->format == DEW_MOE_W_MXFP8) {

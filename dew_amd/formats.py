@@ -202,6 +202,7 @@ class Bf16:
     src/dew/nn/moe.py:666-726), wrapped so that its one-time re-layout for the matrix cores is kept with it."""
 
     weights: torch.Tensor
+    transposed: bool = False   # the same memory as the matrices of the transposed product (an input gradient's)
 
     def __post_init__(self):
         if self.weights.dtype != torch.bfloat16 or self.weights.ndim != 3:
@@ -209,14 +210,20 @@ class Bf16:
 
     @property
     def shape(self):
-        return tuple(self.weights.shape)
+        experts, depth, width = self.weights.shape
+        return (experts, width, depth) if self.transposed else (experts, depth, width)
 
     @property
     def dtype(self):
         return torch.bfloat16
 
+    @property
+    def T(self) -> "Bf16":
+        """The bank of every matrix's transpose, over the same memory: what an input gradient multiplies by."""
+        return Bf16(self.weights, not self.transposed)
+
     def to(self, device) -> "Bf16":
-        return Bf16(self.weights.to(device))
+        return Bf16(self.weights.to(device), self.transposed)
 
 
 @dataclasses.dataclass(frozen=True)

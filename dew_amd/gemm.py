@@ -121,6 +121,8 @@ def prepared(bank) -> ops.PreparedBank:
     if isinstance(bank, ops.PreparedBank):
         return bank
     if torch.is_tensor(bank):  # the reference's plain operand: re-laid at every call, since a parameter may have changed
+        if not bank.is_contiguous() and bank.transpose(1, 2).is_contiguous():
+            return ops.prepare(formats.Bf16(bank.transpose(1, 2), transposed=True))  # `w.transpose(1, 2)`: read where it lies
         return ops.prepare(formats.Bf16(bank.contiguous()))
     if isinstance(bank, formats.Layered):  # the layer's matrices where they lie in the stack
         return prepared(bank.stack).layer(int(bank.layer), int(bank.layers))

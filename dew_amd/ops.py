@@ -207,7 +207,8 @@ def prepare(bank) -> PreparedBank:
         raise KernelError(f"no HIP kernel multiplies a {type(bank).__name__} bank")
     experts, depth, width = bank.shape
     lib = _lib.library()
-    reference = _lib.Bank(fmt, _lib.LAYOUT_REFERENCE, experts, depth, width, _ptr(codes), _ptr(scales), _ptr(tensor))
+    layout = _lib.LAYOUT_REFERENCE_KMAJOR if isinstance(bank, formats.Bf16) and bank.transposed else _lib.LAYOUT_REFERENCE
+    reference = _lib.Bank(fmt, layout, experts, depth, width, _ptr(codes), _ptr(scales), _ptr(tensor))
     buffer = torch.empty(lib.dew_moe_prepared_bytes(fmt, experts, depth, width), dtype=torch.uint8, device=codes.device)
     out = _lib.Bank()
     _lib.check(lib.dew_moe_prepare_bank(reference, _ptr(buffer), out, _stream()), "dew_moe_prepare_bank")

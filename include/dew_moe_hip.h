@@ -42,10 +42,13 @@ enum {
                              /* u8 e4m3 [E,N,K]; scales u8 e8m0 [E,N,K/32]. For dew_moe_grouped_gemm_   */
                              /* mxfp8_rows only.                                                        */
   DEW_MOE_W_BF16 = 6         /* unquantized matrices as the reference holds them: codes bf16 [E,K,N]    */
-                             /* (`experts/*_proj/kernel`, src/dew/nn/moe.py:1231-1235); no scales.      */
+                             /* (`experts/*_proj/kernel`, src/dew/nn/moe.py:1231-1235); no scales. With */
+                             /* DEW_MOE_LAYOUT_REFERENCE_KMAJOR, codes bf16 [E,N,K]: the same memory    */
+                             /* read as the transposed matrices (an input gradient's: depth and width   */
+                             /* are then the transposed product's).                                     */
 };
 
-enum { DEW_MOE_LAYOUT_REFERENCE = 0, DEW_MOE_LAYOUT_PREPARED = 1 };
+enum { DEW_MOE_LAYOUT_REFERENCE = 0, DEW_MOE_LAYOUT_PREPARED = 1, DEW_MOE_LAYOUT_REFERENCE_KMAJOR = 2 };
 
 typedef struct dew_moe_bank {
   int32_t format;            /* DEW_MOE_W_*                                                             */

@@ -250,4 +250,11 @@ def test_unquantized_bf16_experts_run_through_the_layer_as_plain_tensors():
                          oracle.grouped_matmul(x.float().cpu().numpy(), up.float().cpu().numpy(), sizes))
     got = plain.float().cpu().numpy()
     assert np.abs(got - want).max() <= 2.0 ** -6 * np.abs(want).max() and (got == want).mean() > 0.9
+    # an input gradient's matrices: the transposed view is read where it lies, no copy of the transpose is made
+    dy = torch.from_numpy(rng.standard_normal((rows, width)).astype(np.float32)).to(torch.bfloat16).cuda()
+    copied = gemm.gemm(dy, gate.transpose(1, 2).contiguous(), group_sizes)
+    assert torch.equal(gemm.gemm(dy, gate.transpose(1, 2), group_sizes), copied)
+    assert torch.equal(gemm.gemm(dy, formats.Bf16(gate).T, group_sizes), copied)
+    want = oracle.grouped_matmul(dy.float().cpu().numpy(), gate.float().cpu().numpy().transpose(0, 2, 1), sizes)
+    assert np.abs(copied.float().cpu().numpy() - want).max() <= 2.0 ** -7 * np.abs(want).max()
 
