@@ -246,3 +246,26 @@ def test_the_gradients_entry_points_refuse_what_they_cannot_run(ops):
     empty_bank, _ = ops.transpose_columns(none, as_bank=True)
     zero = ops.kernel_gradient_bf16(rows_t, empty_bank, torch.zeros(3, dtype=torch.int32, device="cuda"), out_dtype=torch.float32)
     assert zero.shape == (2, 128, 128) and not zero.any()
+
+
+@pytest.mark.parametrize("kind", ["mxfp8", "bf16"])
+def test_kernel_gradients_over_more_groups_than_a_block_has_threads(ops, kind):
+    """300 groups of 0 .. 2 blocks each (the tile search scans the groups 256 at a time; the padded transposer scans
+    them in runs): every group's gradient against the oracle's, the empty ones zero."""
+    from dew_amd import gemm, projections
+
+    rng = np.random.default_rng(300)
+    blocks = rng.integers(0, 3, size=300)
+    depth, width, tokens = 128, 256, 128 * int(blocks.sum())
+    x = torch.from_numpy(rng.standard_normal((tokens, depth)).astype(np.float32)).to(torch.bfloat16)
+    dy = torch.from_numpy(rng.standard_normal((tokens, width)).astype(np.float32)).to(torch.bfloat16)
+    if kind == "mxfp8":
+        want = oracle.mxfp8_gradients(bf16_np(x), np.zeros((300, depth, width), np.float32), bf16_np(dy), blocks, dtype="float32")[1]
+        got = projections.kernel_gradient(x.cuda(), dy.cuda(), blocks, mx=True, out_dtype=torch.float32).cpu().numpy()
+        bar = 2.0 ** -13
+    else:
+        want = oracle.kernel_gradient(bf16_np(x).T, bf16_np(dy).T, blocks * 128, dtype="float32")
+        got = gemm.gemm_t(x.cuda(), dy.cuda(), torch.tensor(blocks * 128, dtype=torch.int32).cuda(), out_dtype=torch.float32).cpu().numpy()
+        bar = 2.0 ** -18
+    assert np.abs(got - want).max() <= bar * np.abs(want).max()
+    assert not got[blocks == 0].any()
