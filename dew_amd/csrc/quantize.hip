@@ -108,8 +108,18 @@ __global__ __launch_bounds__(256) void absmax_clear_kernel(uint32_t* __restrict_
 
 __global__ __launch_bounds__(256) void absmax_kernel(const bf16_t* __restrict__ x, long long chunks, uint32_t* __restrict__ largest) {
   uint32_t mine = 0;  // magnitudes of bf16 values order as their bit patterns do
-  for (long long chunk = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; chunk < chunks;
-       chunk += static_cast<long long>(gridDim.x) * blockDim.x) {
+  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+  long long chunk = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  for (; chunk + 3 * stride < chunks; chunk += 4 * stride) {  // four loads in flight a lane
+    u32x4_t words[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) words[k] = reinterpret_cast<const u32x4_t*>(x)[chunk + k * stride];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mine = max(mine, max(words[k][i] & 0x7FFFu, (words[k][i] >> 16) & 0x7FFFu));
+  }
+  for (; chunk < chunks; chunk += stride) {
     const u32x4_t words = reinterpret_cast<const u32x4_t*>(x)[chunk];
 #pragma unroll
     for (int i = 0; i < 4; ++i) mine = max(mine, max(words[i] & 0x7FFFu, (words[i] >> 16) & 0x7FFFu));
