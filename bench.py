@@ -231,8 +231,8 @@ def main():
                         help="replay the step as one captured HIP graph (auto: for the launch-bound configs c1 and c3)")
     args = parser.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (expert-parallel sharding is described "
-                 "in DESIGN.md, not built). Run with --gpus 1.")
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the path would shard by expert over "
+                 "an all-to-all each way; that is designed, not built). Run with --gpus 1.")
 
     import numpy as np
     import torch
