@@ -100,12 +100,33 @@ def blockwise_fp8_projection(x: torch.Tensor, w, group_blocks, *, out_dtype=torc
     return blockwise_fp8_product(rows_quantized(x), bank, sizes, out_dtype=out_dtype)
 
 
-def recipe_projection(rows: torch.Tensor, matrix, group_sizes=None, *, out_dtype=torch.bfloat16, bias=None):
-    """`rows @ matrix` in the blockwise FP8 recipe: a dense projection's (`matrix [in, out]`, every row its one
+def recipe_projection(rows: torch.Tensor, matrix, group_sizes=None, *, out_dtype=torch.bfloat16, bias=None,
+                      recipe: str = "blockwise_fp8"):
+    """`rows @ matrix` in a low-precision recipe (`'blockwise_fp8'`, `'mxfp8'` or `'nvfp4'`: the reference reads the
+    run's, `recipe_role`; here the caller names it): a dense projection's (`matrix [in, out]`, every row its one
     group's) or experts' (`[groups, in, out]`, `group_sizes` counting each group's leading rows, any past their sum
     zero), `bias [groups, out]` added to the fp32 sums before the one rounding
-    (src/dew/nn/kernels/projections.py:96-140). None where the widths hold no whole 128-wide blocks
-    (`recipe_refusal`'s 'block_shape', :62-83): the caller then keeps the projection in the run's dtypes."""
+    (src/dew/nn/kernels/projections.py:96-140). The reference pads each group with zero rows to whole 128-row blocks
+    for its launches; a zero row changes no other row's quantization and adds nothing, and these launches take ragged
+    groups as they are. None where the widths hold no whole 128-wide blocks (`recipe_refusal`'s 'block_shape',
+    :62-83): the caller then keeps the projection in the run's dtypes."""
+    if recipe not in ("blockwise_fp8", "mxfp8", "nvfp4"):
+        raise ValueError(f"no recipe {recipe!r}: 'blockwise_fp8', 'mxfp8' or 'nvfp4'")
+    if recipe != "blockwise_fp8":
+        if isinstance(matrix, (formats.MxFp8, formats.NvFp4, ops.PreparedBank)):
+            bank = matrix
+        else:
+            stacked = matrix if matrix.dim() == 3 else matrix[None]
+            if stacked.shape[1] % SCALE_DEPTH or stacked.shape[2] % SCALE_DEPTH or (recipe == "nvfp4" and stacked.shape[1] % 256):
+                return None  # (an NVFP4 bank's depth is whole 256s)
+            bank = formats.MxFp8.quantized(stacked) if recipe == "mxfp8" else nvfp4_matrices(stacked)
+        if bias is not None:
+            bias = bias.reshape(bank.shape[0], bank.shape[2]).to(torch.float32).contiguous()
+        if group_sizes is None:
+            group_sizes = torch.tensor([rows.shape[0]], dtype=torch.int32, device=rows.device)
+        if recipe == "mxfp8":
+            return mxfp8_product(mxfp8_rows(rows), bank, group_sizes, out_dtype=out_dtype, bias=bias)
+        return nvfp4_block_product(nvfp4_rows(rows), bank, group_sizes, out_dtype=out_dtype, bias=bias)
     if isinstance(matrix, (formats.Fp8Blocks, ops.PreparedBank)):
         bank = matrix
     else:
@@ -192,7 +213,8 @@ def nvfp4_matrices(w: torch.Tensor) -> formats.NvFp4:
     return formats.NvFp4.of(codes, scales, tensor.reshape(1).expand(groups).contiguous())
 
 
-def nvfp4_block_product(lhs: NvFp4Rows, matrices, group_sizes, *, out_dtype=torch.bfloat16, gather=None, scatter=None) -> torch.Tensor:
+def nvfp4_block_product(lhs: NvFp4Rows, matrices, group_sizes, *, out_dtype=torch.bfloat16, bias=None, gather=None,
+                        scatter=None) -> torch.Tensor:
     """Each group's NVFP4 rows times its matrix of the NVFP4 bank `matrices`: every (code x block scale) product exact,
     fp32 sums, times both tensor scales, one rounding (src/dew/nn/kernels/gemm.py:937-947). The rows' values are
     exact in bf16, so this is the bank's bf16-operand launch with the rows' tensor scale folded into the bank's."""
@@ -200,7 +222,7 @@ def nvfp4_block_product(lhs: NvFp4Rows, matrices, group_sizes, *, out_dtype=torc
         raise ValueError(f"the launch writes bfloat16, not {out_dtype}")
     bank = gemm.prepared(matrices).scaled(lhs.scale)
     rows = lhs.values.shape[0] if gather is None else gather.numel()
-    return ops.grouped_gemm(lhs.values, bank, _offsets(group_sizes, rows, lhs.values.device), gather=gather, scatter=scatter)
+    return ops.grouped_gemm(lhs.values, bank, _offsets(group_sizes, rows, lhs.values.device), gather=gather, scatter=scatter, bias=bias)
 
 
 def nvfp4_projection(x: torch.Tensor, w, group_blocks, *, out_dtype=torch.bfloat16) -> torch.Tensor:

@@ -694,7 +694,7 @@ def nvfp4_quantized(x):
     return (np.copysign(grid[code], quotient)).astype(F32), scales, tensor
 
 
-def nvfp4_block_product(lhs, lhs_scales, lhs_scale, matrices, matrix_scales, matrix_scale, group_sizes, *, dtype="bfloat16"):
+def nvfp4_block_product(lhs, lhs_scales, lhs_scale, matrices, matrix_scales, matrix_scale, group_sizes, *, dtype="bfloat16", bias=None):
     """Each group's rows of `lhs [rows, depth]` times its matrix of `matrices [groups, width, depth]`, both NVFP4:
     each code times its sixteen depths' scale, every product exact, summed in fp32, times both tensor scales, rounded
     once (src/dew/nn/kernels/gemm.py:937-947). The sum is formed exactly and rounded to fp32."""
@@ -707,15 +707,20 @@ def nvfp4_block_product(lhs, lhs_scales, lhs_scale, matrices, matrix_scales, mat
             total[start:start + size] = (left[start:start + size] @ right[group].T).astype(F32)
         start += size
     total = twice_scaled(total, F32(lhs_scale), F32(matrix_scale))
+    if bias is not None:  # each group's bias meets its rows' fp32 sums before the one rounding (projections.py:137-139)
+        start = 0
+        for group, size in enumerate(np.asarray(group_sizes).tolist()):
+            total[start:start + size] = (total[start:start + size] + np.asarray(bias, F32)[group]).astype(F32)
+            start += size
     return bf16_round(total) if dtype == "bfloat16" else total
 
 
-def nvfp4_projection(x, w, group_sizes, *, dtype="bfloat16"):
+def nvfp4_projection(x, w, group_sizes, *, dtype="bfloat16", bias=None):
     """`x [rows, depth]` and `w [groups, depth, width]` both quantized along the depth (the matrices under one tensor
     scale together), their `nvfp4_block_product` (src/dew/nn/kernels/projections.py:261-275)."""
     rows = nvfp4_quantized(x)
     matrices = nvfp4_quantized(np.swapaxes(np.asarray(w, F32), 1, 2))
-    return nvfp4_block_product(*rows, *matrices, group_sizes, dtype=dtype)
+    return nvfp4_block_product(*rows, *matrices, group_sizes, dtype=dtype, bias=bias)
 
 
 def swiglu(gate, up, *, dtype="bfloat16", limit=None, exp=np.exp):

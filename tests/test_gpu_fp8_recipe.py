@@ -248,3 +248,33 @@ def test_the_nvfp4_product_matches_the_oracle(ops, label, sizes):
     assert np.all(got[rows:] == 0) and np.all(want[rows:] == 0)
     scale = np.abs(want).max()
     assert np.abs(got - want).max() <= 2.0 ** -7 * scale and (got == want).mean() > 0.97
+
+
+@pytest.mark.parametrize("recipe", ["mxfp8", "nvfp4"])
+@pytest.mark.parametrize("label,sizes", SIZES, ids=[s[0] for s in SIZES])
+def test_recipe_projection_takes_every_recipe_with_ragged_groups_and_a_bias(ops, recipe, label, sizes):
+    """`recipe_projection` from the weights themselves: ragged groups as they are (the reference pads them with zero
+    rows, which change nothing), rows past the groups zero, the bias on the fp32 sums; and a dense projection's one
+    group."""
+    from dew_amd import projections
+
+    depth, width = 512, 256
+    groups, rows = len(sizes), int(np.sum(sizes))
+    rng = np.random.default_rng(rows + len(recipe))
+    x = torch.from_numpy(rng.standard_normal((rows + 6, depth)).astype(np.float32)).to(torch.bfloat16)
+    w = weights_case(groups, depth, width, seed=31)
+    bias = torch.from_numpy(rng.standard_normal((groups, width)).astype(np.float32) * 0.1)
+    sizes_device = torch.tensor(sizes, dtype=torch.int32).cuda()
+    truth = oracle.mxfp8_projection if recipe == "mxfp8" else oracle.nvfp4_projection
+    for with_bias in (None, bias):
+        got = bf16_np(projections.recipe_projection(x.cuda(), torch.from_numpy(w).cuda(), sizes_device, recipe=recipe,
+                                                    bias=None if with_bias is None else with_bias.cuda()))
+        want = truth(bf16_np(x), w, sizes, bias=None if with_bias is None else with_bias.numpy())
+        assert np.all(got[rows:] == 0) and np.all(want[rows:] == 0)
+        assert np.abs(got - want).max() <= 2.0 ** -7 * np.abs(want).max() and (got == want).mean() > 0.97
+    dense = bf16_np(projections.recipe_projection(x.cuda(), torch.from_numpy(w[0]).cuda(), recipe=recipe))
+    want = truth(bf16_np(x), w[:1], [rows + 6])
+    assert np.abs(dense - want).max() <= 2.0 ** -7 * np.abs(want).max() and (dense == want).mean() > 0.97
+    assert projections.recipe_projection(x.cuda(), torch.zeros((192, 128), device="cuda"), recipe=recipe) is None
+    with pytest.raises(ValueError):
+        projections.recipe_projection(x.cuda(), torch.from_numpy(w).cuda(), sizes_device, recipe="int8")
