@@ -140,6 +140,22 @@ __device__ __forceinline__ float e2m1_nearest(float magnitude) {
   return magnitude > 5.0f ? 6.0f : value;
 }
 
+// The same choice times the block scale, without the quotient: for y = x / tensor and the block scale `each` (an e4m3
+// value, four significant bits), fl(y / each) > t exactly where y > t each, and >= likewise, for each of the seven
+// thresholds t (at most three significant bits, so t each is exact): a y above t each lies at least one ulp of t each
+// above it, which is more than half an ulp of t above t in the quotient (their ratio is 1 / m or 2 / m for each's
+// significand m < 2), so the quotient rounds past t; at or below, it cannot round above. One IEEE division an element
+// instead of two.
+__device__ __forceinline__ float e2m1_scaled(float magnitude, float each) {
+  float value = magnitude > 0.25f * each ? 0.5f * each : 0.0f;
+  value = magnitude >= 0.75f * each ? each : value;
+  value = magnitude > 1.25f * each ? 1.5f * each : value;
+  value = magnitude >= 1.75f * each ? 2.0f * each : value;
+  value = magnitude > 2.5f * each ? 3.0f * each : value;
+  value = magnitude >= 3.5f * each ? 4.0f * each : value;
+  return magnitude > 5.0f * each ? 6.0f * each : value;
+}
+
 __global__ __launch_bounds__(64 * kQuantizeWaves) void quantize_rows_nvfp4_kernel(const bf16_t* __restrict__ x, const uint32_t* __restrict__ largest,
                                                                                 bf16_t* __restrict__ out, float* __restrict__ tensor_scale,
                                                                                 int rows, int depth) {
@@ -176,8 +192,8 @@ __global__ __launch_bounds__(64 * kQuantizeWaves) void quantize_rows_nvfp4_kerne
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         const float source_value = v[2 * i + h];
-        const float quotient = each > 0.0f ? (source_value / tensor) / each : 0.0f;
-        pair[h] = copysignf(e2m1_nearest(fabsf(quotient)) * each, quotient);  // code x block scale: exact in bf16
+        const float over_tensor = each > 0.0f ? source_value / tensor : 0.0f;
+        pair[h] = copysignf(e2m1_scaled(fabsf(over_tensor), each), over_tensor);  // code x block scale: exact in bf16
       }
       packed[i] = (__float_as_uint(pair[0]) >> 16) | (__float_as_uint(pair[1]) & 0xFFFF0000u);
     }
@@ -364,8 +380,8 @@ __global__ __launch_bounds__(256) void transpose_columns_kernel(const bf16_t* __
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const float value = __uint_as_float(bits[16 * block + i] << 16);
-        const float quotient = each > 0.0f ? (value / tensor) / each : 0.0f;
-        bits[16 * block + i] = __float_as_uint(copysignf(e2m1_nearest(fabsf(quotient)) * each, quotient)) >> 16;
+        const float over_tensor = each > 0.0f ? value / tensor : 0.0f;
+        bits[16 * block + i] = __float_as_uint(copysignf(e2m1_scaled(fabsf(over_tensor), each), over_tensor)) >> 16;
       }
     }
   }

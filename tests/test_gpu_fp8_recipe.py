@@ -278,3 +278,18 @@ def test_recipe_projection_takes_every_recipe_with_ragged_groups_and_a_bias(ops,
     assert projections.recipe_projection(x.cuda(), torch.zeros((192, 128), device="cuda"), recipe=recipe) is None
     with pytest.raises(ValueError):
         projections.recipe_projection(x.cuda(), torch.from_numpy(w).cuda(), sizes_device, recipe="int8")
+
+
+def test_the_nvfp4_quantizers_choose_the_oracles_codes_over_millions_of_elements(ops):
+    """The device compares x / tensor with (threshold x block scale) where the oracle, as the reference, rounds
+    (x / tensor) / scale and compares with the threshold: the same choice for every element (rows over 17 binades of
+    scale, so block scales and quotients of every size meet), along the depth and along the tokens."""
+    rng = np.random.default_rng(12)
+    x = (rng.standard_normal((2048, 2048)) * np.exp2(rng.integers(-8, 9, size=(2048, 1)))).astype(np.float32)
+    x = torch.from_numpy(x).to(torch.bfloat16)
+    for transposed in (False, True):
+        source = bf16_np(x).T if transposed else bf16_np(x)
+        values, scales, tensor = oracle.nvfp4_quantized(source)
+        want = values * np.repeat(scales, 16, axis=1)
+        got, scale = ops.transpose_columns(x.cuda(), nvfp4=True, as_bank=False) if transposed else ops.quantize_rows_nvfp4(x.cuda())
+        assert scale.item() == tensor and np.array_equal(bf16_np(got), want)
