@@ -194,7 +194,7 @@ def sustained_rates(device):
     bytes read plus bytes written), each timed with HIP events over several launches after a warm-up."""
     import torch
 
-    from dew_amd import ops
+    from bench_aids import probes as ops
 
     operands = torch.randn(16384, device=device).to(torch.bfloat16)
     ops.probe_mfma(operands, 2000)
@@ -273,8 +273,9 @@ def main():
         # millisecond of queued work ahead of each step lets the host run ahead, so the step's launches follow each
         # other on the device as they do in the graph and the events bracket the kernel, not the host's launch path.
         operands = torch.randn(16384, device=device).to(torch.bfloat16)
+        from bench_aids import probes
         for _ in range(args.steps):
-            ops.probe_mfma(operands, 1200)
+            probes.probe_mfma(operands, 1200)
             stepper(timed=True)
         torch.cuda.synchronize()
     else:
@@ -316,7 +317,7 @@ def main():
     sustained_mfma, sustained_copy = sustained_rates(device)
     roofline["sustained"] = {"bf16_mfma_random_operands_tflops": sustained_mfma, "plain_copy_gbs": sustained_copy,
                              "frac_of_sustained": round(roofline["achieved"] / (sustained_copy if decode else sustained_mfma), 4),
-                             "note": "measured in this run by dew_moe_probe_mfma / dew_moe_probe_copy: the rate the chip holds on "
+                             "note": "measured in this run by bench_aids' MFMA and copy probes: the rate the chip holds on "
                                      "random data at its power limit, below the published peak"}
     roofline["kernel"] = "grouped_gemm_kernel<paired gate/up + SwiGLU>" + (
         " on split rows (v_mfma_scale_f32_32x32x64_f8f6f4, two e4m3 terms x FP4)" if stepper.on_split_rows() else "")

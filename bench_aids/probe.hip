@@ -1,13 +1,17 @@
 // Measurement aids for the roofline report: what this chip sustains, measured in the same run as the kernels.
-//   dew_moe_probe_mfma  back-to-back v_mfma_f32_32x32x16_bf16 on caller-supplied operands, nothing else in
+//   dew_bench_probe_mfma back-to-back v_mfma_f32_32x32x16_bf16 on caller-supplied operands, nothing else in
 //                       the loop. With operands of random sign, exponent and mantissa the matrix cores draw
 //                       more power than with constants and the clock settles lower: the sustained rate the
 //                       GEMM kernels can approach on real data.
-//   dew_moe_probe_copy  a plain 16-byte-per-lane copy: the HBM rate a streaming kernel sustains, and the known
+//   dew_bench_probe_copy a plain 16-byte-per-lane copy: the HBM rate a streaming kernel sustains, and the known
 //                       traffic the FETCH_SIZE / WRITE_SIZE counters are scaled by.
-#include "common.h"
+//
+// Built into its own small library (libdew_bench_probes.so) beside the benchmarks that use it: it is no part of the
+// MoE kernels' C ABI.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
 
-namespace dew {
+namespace dew_bench {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
@@ -44,22 +48,24 @@ __global__ __launch_bounds__(256) void probe_copy_kernel(const u32x4_t* __restri
     dst[i] = src[i];
 }
 
-}  // namespace dew
+}  // namespace dew_bench
 
-extern "C" int dew_moe_probe_mfma(const void* operands, int32_t iters, float* sink, double* flops, void* stream) {
-  using namespace dew;
-  DEW_REQUIRE(operands && sink && iters >= 1, "dew_moe_probe_mfma: operands (32 KiB), sink (1 MiB) and iters >= 1");
-  DEW_REQUIRE(aligned16(operands), "dew_moe_probe_mfma: operands must be 16-byte aligned");
+// Both return 0, 1 for arguments that do not fit (null or misaligned pointers, sizes that are not whole 16 bytes), or 3
+// for a failed launch.
+extern "C" int dew_bench_probe_mfma(const void* operands /* 32 KiB of bf16 */, int32_t iters, float* sink /* 1 MiB */,
+                                    double* flops /* host, nullable */, void* stream) {
+  using namespace dew_bench;
+  if (!operands || !sink || iters < 1 || (reinterpret_cast<uintptr_t>(operands) & 15u) != 0) return 1;
   hipLaunchKernelGGL(probe_mfma_kernel, dim3(kProbeBlocks), dim3(256), 0, static_cast<hipStream_t>(stream),
                      static_cast<const u32x4_t*>(operands), sink, iters);
   if (flops) *flops = static_cast<double>(kProbeBlocks) * 4 * iters * 16 * (2.0 * 32 * 32 * 16);
-  return launched("probe_mfma_kernel");
+  return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 
-extern "C" int dew_moe_probe_copy(const void* src, void* dst, size_t bytes, void* stream) {
-  using namespace dew;
-  DEW_REQUIRE(src && dst && bytes % 16 == 0 && aligned16(src) && aligned16(dst), "dew_moe_probe_copy: 16-byte aligned buffers and size");
+extern "C" int dew_bench_probe_copy(const void* src, void* dst, size_t bytes, void* stream) {
+  using namespace dew_bench;
+  if (!src || !dst || bytes % 16 != 0 || ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) != 0) return 1;
   hipLaunchKernelGGL(probe_copy_kernel, dim3(256 * 32), dim3(256), 0, static_cast<hipStream_t>(stream),
                      static_cast<const u32x4_t*>(src), static_cast<u32x4_t*>(dst), bytes / 16);
-  return launched("probe_copy_kernel");
+  return hipGetLastError() == hipSuccess ? 0 : 3;
 }

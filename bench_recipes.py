@@ -2,7 +2,7 @@
 and NVFP4 recipes and for plain bf16 matrices, the forward product, the input's gradient and the matrices' gradient
 (each with the passes that quantize or transpose its operands timed beside it). One JSON line a product.
 
-    python -m dew_amd.bench_recipes [--shape mixtral|deepseek] [--steps 5]
+    python bench_recipes.py [--shape mixtral|deepseek] [--steps 5]
 
 `tflops` counts 2 x rows x depth x width for the product alone; `prepare_us` is the operands' quantizing / transposing
 passes of that product (the matrices' own quantization, done once a step for all three products, is not timed)."""
@@ -12,7 +12,7 @@ import json
 
 import torch
 
-from . import formats, gemm, ops, projections
+from dew_amd import formats, gemm, ops, projections
 
 SHAPES = {
     # groups, rows a group, depth, width: the gate/up and the down projection of each model's experts

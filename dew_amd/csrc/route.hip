@@ -151,7 +151,9 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
     const int e = lane + kWave * i;
     float s = score[i];
     if (p.bias != nullptr && e < p.experts) s = s + p.bias[e];
-    select[i] = e < p.experts ? s : ninf;
+    // A NaN selection (a NaN in the bias or the logits) is never preferred: it competes as -inf, so every round still
+    // finds an expert in range (no comparison with NaN holds, and a round without a candidate would name no expert).
+    select[i] = (e < p.experts && s == s) ? s : ninf;
   }
 
   if (p.expert_groups > 1) {
@@ -216,7 +218,7 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
     }
     b = wave_best(b);
     if ((b.index % kWave) == lane) taken_mask |= 1u << (b.index / kWave);
-    if (lane == round) my_choice = b.index;
+    if (lane == round) my_choice = min(b.index, p.experts - 1);
   }
 
   // gate weights: lane j < k owns the j-th choice

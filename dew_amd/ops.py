@@ -145,6 +145,8 @@ class PreparedBank:
     descriptor: _lib.Bank
     shape: tuple
     keep: tuple
+    first: int = 0
+    """The bank's first expert within the buffers `keep` holds (a layer of a stack starts inside them)."""
 
     @property
     def experts(self):
@@ -156,9 +158,10 @@ class PreparedBank:
         held = self.descriptor
         if held.format not in (_lib.W_NVFP4, _lib.W_MXFP4):
             raise KernelError("only an NVFP4 bank carries tensor scales")
-        scales = (self.keep[2].to(torch.float32) * by.to(torch.float32)).contiguous()
+        own = self.keep[2].reshape(-1)[self.first:self.first + self.experts]  # a layer's experts within its stack's scales
+        scales = (own.to(torch.float32) * by.to(torch.float32)).contiguous()
         view = _lib.Bank(held.format, held.layout, held.experts, held.depth, held.width, held.codes, held.scales, _ptr(scales))
-        return PreparedBank(view, self.shape, (*self.keep, scales))
+        return PreparedBank(view, self.shape, (self.keep[0], self.keep[1], scales), 0)
 
     def layer(self, index: int, layers: int) -> "PreparedBank":
         """Layer `index` of a bank that stacks `layers` layers' experts along its expert axis (`[layers * E, K, N]`),
@@ -174,11 +177,16 @@ class PreparedBank:
         fp4 = held.format in (_lib.W_NVFP4, _lib.W_MXFP4)
         codes = depth * width // 2 if fp4 else depth * width
         codes = depth * width * 2 if held.format == _lib.W_BF16 else codes
-        scales = {_lib.W_FP8_BLOCK: (depth // 128) * (width // 128) * 4, _lib.W_FP8_CHANNEL: width * 4}.get(held.format, width * (depth // 16))
+        strides = {_lib.W_FP8_BLOCK: (depth // 128) * (width // 128) * 4, _lib.W_FP8_CHANNEL: width * 4,
+                   _lib.W_NVFP4: width * (depth // 16), _lib.W_MXFP4: width * (depth // 16), _lib.W_MXFP8: width * (depth // 32),
+                   _lib.W_BF16: 0}
+        if held.format not in strides:
+            raise KernelError(f"no layer stride is known for a prepared bank of format {held.format}")
+        scales = strides[held.format]
         view = _lib.Bank(held.format, held.layout, experts, depth, width, held.codes + first * codes,
                          None if not held.scales else held.scales + first * scales,
                          None if not held.tensor_scale else held.tensor_scale + first * 4)
-        return PreparedBank(view, (experts, depth, width), self.keep)
+        return PreparedBank(view, (experts, depth, width), self.keep, self.first + first)
 
 
 def prepare(bank) -> PreparedBank:
@@ -228,24 +236,37 @@ def _expert_bias(bias: torch.Tensor | None, experts: int, width: int) -> torch.T
     return bias
 
 
+def _product_rows(operand: torch.Tensor, name: str, offsets: torch.Tensor, experts: int, gather, scatter, rows) -> int:
+    """What every grouped product's launch trusts and only the host can see, checked before any pointer leaves: the
+    row operand on the device and contiguous, `offsets` int32 `[E + 1]` on the device, `gather` / `scatter` int32,
+    contiguous, on the device and covering every row, and no more rows asked than the operand (without a gather)
+    holds. Returns the rows of the launch."""
+    _device(operand, name)
+    _device(offsets, "offsets", torch.int32)
+    if offsets.numel() != experts + 1:
+        raise KernelError(f"offsets has {offsets.numel()} entries, the bank {experts} experts")
+    for label, index in (("gather", gather), ("scatter", scatter)):
+        if index is not None:
+            _device(index, label, torch.int32)
+    rows = (gather.numel() if gather is not None else operand.shape[0]) if rows is None else int(rows)
+    if rows < 0:
+        raise KernelError(f"{rows} rows asked")
+    if gather is None and rows > operand.shape[0]:
+        raise KernelError(f"{rows} rows asked of {name} of {operand.shape[0]}")
+    if (gather is not None and gather.numel() < rows) or (scatter is not None and scatter.numel() < rows):
+        raise KernelError("gather and scatter must cover every row")
+    return rows
+
+
 def grouped_gemm(x: torch.Tensor, bank: PreparedBank, offsets: torch.Tensor, *, gather: torch.Tensor | None = None,
                  scatter: torch.Tensor | None = None, rows: int | None = None,
                  bias: torch.Tensor | None = None) -> torch.Tensor:
     """`out[scatter[i]] = x[gather[i]] @ W[expert of sorted position i] (+ bias[expert])`, bf16 `[rows, N]`."""
-    _device(x, "x", torch.bfloat16), _device(offsets, "offsets", torch.int32)
+    _device(x, "x", torch.bfloat16)
     experts, depth, width = bank.shape
     if x.shape[-1] != depth:
         raise KernelError(f"x rows are {x.shape[-1]} deep, the bank {depth}")
-    if offsets.numel() != experts + 1:
-        raise KernelError(f"offsets has {offsets.numel()} entries, the bank {experts} experts")
-    for name, index in (("gather", gather), ("scatter", scatter)):
-        if index is not None:
-            _device(index, name, torch.int32)
-    rows = (gather.numel() if gather is not None else x.shape[0]) if rows is None else rows
-    if gather is None and rows > x.shape[0]:
-        raise KernelError(f"{rows} rows asked of an x of {x.shape[0]}")
-    if (gather is not None and gather.numel() < rows) or (scatter is not None and scatter.numel() < rows):
-        raise KernelError("gather and scatter must cover every row")
+    rows = _product_rows(x, "x", offsets, experts, gather, scatter, rows)
     bias = _expert_bias(bias, experts, width)
     out = torch.empty((rows, width), dtype=torch.bfloat16, device=x.device)
     _lib.check(_lib.library().dew_moe_grouped_gemm_bias(_ptr(x), _ptr(gather), _ptr(offsets), bank.descriptor, _ptr(bias),
@@ -259,17 +280,11 @@ def gateup_interleaved(x: torch.Tensor, gate_up: PreparedBank, offsets: torch.Te
     """GPT-OSS's fused projection and gating, one launch: `p = x[gather[i]] @ W[e] + bias[e]` with gate in the even
     columns and up in the odd ones, `hidden = (clip(up) + 1) * min(gate, limit) * logistic(1.702 min(gate, limit))`,
     bf16 `[rows, N / 2]`."""
-    _device(x, "x", torch.bfloat16), _device(offsets, "offsets", torch.int32)
+    _device(x, "x", torch.bfloat16)
     experts, depth, width = gate_up.shape
     if x.shape[-1] != depth:
         raise KernelError(f"x rows are {x.shape[-1]} deep, the bank {depth}")
-    if offsets.numel() != experts + 1:
-        raise KernelError(f"offsets has {offsets.numel()} entries, the bank {experts} experts")
-    if gather is not None:
-        _device(gather, "gather", torch.int32)
-    rows = (gather.numel() if gather is not None else x.shape[0]) if rows is None else rows
-    if gather is None and rows > x.shape[0]:
-        raise KernelError(f"{rows} rows asked of an x of {x.shape[0]}")
+    rows = _product_rows(x, "x", offsets, experts, gather, None, rows)
     bias = _expert_bias(bias, experts, width)
     hidden = torch.empty((rows, width // 2), dtype=torch.bfloat16, device=x.device)
     _lib.check(_lib.library().dew_moe_gateup_interleaved(_ptr(x), _ptr(gather), _ptr(offsets), gate_up.descriptor, _ptr(bias),
@@ -281,17 +296,13 @@ def gateup_interleaved(x: torch.Tensor, gate_up: PreparedBank, offsets: torch.Te
 def gateup_swiglu(x: torch.Tensor, gate: PreparedBank, up: PreparedBank, offsets: torch.Tensor, *,
                   gather: torch.Tensor | None = None, rows: int | None = None) -> torch.Tensor:
     """`hidden[i] = swiglu(x[gather[i]] @ Wg[e], x[gather[i]] @ Wu[e])`, bf16 `[rows, F]`, one launch."""
-    _device(x, "x", torch.bfloat16), _device(offsets, "offsets", torch.int32)
+    _device(x, "x", torch.bfloat16)
     experts, depth, width = gate.shape
     if x.shape[-1] != depth:
         raise KernelError(f"x rows are {x.shape[-1]} deep, the banks {depth}")
-    if offsets.numel() != experts + 1:
-        raise KernelError(f"offsets has {offsets.numel()} entries, the banks {experts} experts")
-    if gather is not None:
-        _device(gather, "gather", torch.int32)
-    rows = (gather.numel() if gather is not None else x.shape[0]) if rows is None else rows
-    if gather is None and rows > x.shape[0]:
-        raise KernelError(f"{rows} rows asked of an x of {x.shape[0]}")
+    if up.shape != gate.shape:
+        raise KernelError(f"gate {gate.shape} and up {up.shape} differ")
+    rows = _product_rows(x, "x", offsets, experts, gather, None, rows)
     hidden = torch.empty((rows, width), dtype=torch.bfloat16, device=x.device)
     _lib.check(_lib.library().dew_moe_gateup_swiglu(_ptr(x), _ptr(gather), _ptr(offsets), gate.descriptor, up.descriptor,
                                                     _ptr(hidden), rows, _stream()), "dew_moe_gateup_swiglu")
@@ -378,7 +389,8 @@ def grouped_gemm_split(split: torch.Tensor, scale: torch.Tensor, bank: PreparedB
     experts, depth, width = bank.shape
     if split.dtype != torch.uint8 or split.shape[-1] != 2 * depth or scale.dtype != torch.uint8 or scale.numel() != split.shape[0]:
         raise KernelError(f"split rows are uint8 [rows, {2 * depth}] with one uint8 scale a row")
-    rows = (gather.numel() if gather is not None else split.shape[0]) if rows is None else rows
+    _device(scale, "scale", torch.uint8)
+    rows = _product_rows(split, "split", offsets, experts, gather, scatter, rows)
     bias = _expert_bias(bias, experts, width)
     out = torch.empty((rows, width), dtype=torch.bfloat16, device=split.device)
     _lib.check(_lib.library().dew_moe_grouped_gemm_split(_ptr(split), _ptr(scale), _ptr(gather), _ptr(offsets), bank.descriptor,
@@ -393,7 +405,10 @@ def gateup_swiglu_split(split: torch.Tensor, scale: torch.Tensor, gate: Prepared
     experts, depth, width = gate.shape
     if split.dtype != torch.uint8 or split.shape[-1] != 2 * depth or scale.dtype != torch.uint8 or scale.numel() != split.shape[0]:
         raise KernelError(f"split rows are uint8 [rows, {2 * depth}] with one uint8 scale a row")
-    rows = (gather.numel() if gather is not None else split.shape[0]) if rows is None else rows
+    _device(scale, "scale", torch.uint8)
+    if up.shape != gate.shape:
+        raise KernelError(f"gate {gate.shape} and up {up.shape} differ")
+    rows = _product_rows(split, "split", offsets, experts, gather, None, rows)
     hidden = torch.empty((rows, width), dtype=torch.bfloat16, device=split.device)
     _lib.check(_lib.library().dew_moe_gateup_swiglu_split(_ptr(split), _ptr(scale), _ptr(gather), _ptr(offsets), gate.descriptor,
                                                           up.descriptor, _ptr(hidden), rows, _stream()),
@@ -415,7 +430,10 @@ def gateup_swiglu_split_out(split: torch.Tensor, scale: torch.Tensor, gate: Prep
     experts, depth, width = gate.shape
     if split.dtype != torch.uint8 or split.shape[-1] != 2 * depth or scale.dtype != torch.uint8 or scale.numel() != split.shape[0]:
         raise KernelError(f"split rows are uint8 [rows, {2 * depth}] with one uint8 scale a row")
-    rows = (gather.numel() if gather is not None else split.shape[0]) if rows is None else rows
+    _device(scale, "scale", torch.uint8)
+    if up.shape != gate.shape:
+        raise KernelError(f"gate {gate.shape} and up {up.shape} differ")
+    rows = _product_rows(split, "split", offsets, experts, gather, None, rows)
     hidden = torch.empty((rows, width * 2), dtype=torch.uint8, device=split.device)
     scales = torch.empty((rows, block_scale_pitch(width)), dtype=torch.uint8, device=split.device)
     _lib.check(_lib.library().dew_moe_gateup_swiglu_split_out(_ptr(split), _ptr(scale), _ptr(gather), _ptr(offsets), gate.descriptor,
@@ -432,7 +450,8 @@ def grouped_gemm_split_blocks(split: torch.Tensor, scales: torch.Tensor, bank: P
     if split.dtype != torch.uint8 or split.shape[-1] != 2 * depth or scales.dtype != torch.uint8 or \
             tuple(scales.shape) != (split.shape[0], block_scale_pitch(depth)) or not scales.is_contiguous():
         raise KernelError(f"split rows are uint8 [rows, {2 * depth}] with uint8 scales [rows, {block_scale_pitch(depth)}]")
-    rows = (gather.numel() if gather is not None else split.shape[0]) if rows is None else rows
+    _device(scales, "scales", torch.uint8)
+    rows = _product_rows(split, "split", offsets, experts, gather, scatter, rows)
     bias = _expert_bias(bias, experts, width)
     out = torch.empty((rows, width), dtype=torch.bfloat16, device=split.device)
     _lib.check(_lib.library().dew_moe_grouped_gemm_split_blocks(_ptr(split), _ptr(scales), _ptr(gather), _ptr(offsets),
@@ -491,7 +510,8 @@ def grouped_gemm_mxfp8_rows(codes: torch.Tensor, scales: torch.Tensor, bank: Pre
         raise KernelError(f"MXFP8 rows are uint8 [rows, {depth}] with uint8 scales [rows, {depth // 32}]")
     if bank.descriptor.format != _lib.W_MXFP8:
         raise KernelError("MXFP8 rows multiply an MXFP8 bank")
-    rows = (gather.numel() if gather is not None else codes.shape[0]) if rows is None else rows
+    _device(scales, "scales", torch.uint8)
+    rows = _product_rows(codes, "codes", offsets, experts, gather, scatter, rows)
     bias = _expert_bias(bias, experts, width)
     out = torch.empty((rows, width), dtype=torch.bfloat16, device=codes.device)
     _lib.check(_lib.library().dew_moe_grouped_gemm_mxfp8_rows(_ptr(codes), _ptr(scales), _ptr(gather), _ptr(offsets), bank.descriptor,
@@ -633,36 +653,11 @@ def grouped_gemm_fp8_rows(codes: torch.Tensor, scales: torch.Tensor, bank: Prepa
         raise KernelError(f"quantized rows are uint8 [rows, {depth}] with uint8 scales [rows, {block_scale_pitch(depth)}]")
     if bank.descriptor.format != _lib.W_FP8_BLOCK:
         raise KernelError("quantized rows multiply an FP8 128 x 128 block bank")
-    rows = (gather.numel() if gather is not None else codes.shape[0]) if rows is None else rows
+    _device(scales, "scales", torch.uint8)
+    rows = _product_rows(codes, "codes", offsets, experts, gather, scatter, rows)
     bias = _expert_bias(bias, experts, width)
     out = torch.empty((rows, width), dtype=torch.bfloat16, device=codes.device)
     _lib.check(_lib.library().dew_moe_grouped_gemm_fp8_rows(_ptr(codes), _ptr(scales), _ptr(gather), _ptr(offsets), bank.descriptor,
                                                             _ptr(bias), _ptr(scatter), _ptr(out), rows, _stream()),
                "dew_moe_grouped_gemm_fp8_rows")
     return out
-
-
-# ---- measurement aids ---------------------------------------------------------------------------------
-
-
-def probe_mfma(operands: torch.Tensor, iters: int) -> float:
-    """Launch the back-to-back MFMA probe on `operands` (bf16, 16384 values); returns its FLOP count."""
-    import ctypes
-
-    _device(operands, "operands", torch.bfloat16)
-    if operands.numel() < 16384:
-        raise KernelError("the MFMA probe reads 16384 bf16 operands")
-    sink = torch.empty(1024 * 256, dtype=torch.float32, device=operands.device)
-    flops = ctypes.c_double(0.0)
-    _lib.check(_lib.library().dew_moe_probe_mfma(_ptr(operands), iters, _ptr(sink), ctypes.byref(flops), _stream()), "dew_moe_probe_mfma")
-    return flops.value
-
-
-def probe_copy(src: torch.Tensor, dst: torch.Tensor) -> int:
-    """Launch the plain copy probe; returns the bytes copied (read once, written once)."""
-    _device(src, "src"), _device(dst, "dst")
-    size = src.numel() * src.element_size()
-    if size != dst.numel() * dst.element_size() or size % 16:
-        raise KernelError("the copy probe takes two buffers of one size, a multiple of 16 bytes")
-    _lib.check(_lib.library().dew_moe_probe_copy(_ptr(src), _ptr(dst), size, _stream()), "dew_moe_probe_copy")
-    return size

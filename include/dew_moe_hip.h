@@ -295,15 +295,6 @@ int dew_moe_combine(const void* slots /* bf16 [T,k,D] */, const float* weights /
                     const void* addend /* nullable */, void* out /* bf16 [T,D] */, int32_t tokens,
                     int32_t top_k, int32_t width, void* stream);
 
-/* ---- Measurement aids (no counterpart in the reference; used by the benchmark's roofline report) ---------
- * dew_moe_probe_mfma: back-to-back v_mfma_f32_32x32x16_bf16 on the caller's operands (32 KiB of bf16, any
- * values; random ones show the rate the matrix cores sustain on real data), 1024 blocks x `iters` x 16
- * instructions a wavefront; writes 1 MiB of sums to `sink` and the FLOP count to *flops (host, nullable).
- * dew_moe_probe_copy: dst[i] = src[i], 16 bytes a lane: the streaming rate of HBM and the known traffic that
- * the FETCH_SIZE / WRITE_SIZE counters are scaled by.                                                      */
-int dew_moe_probe_mfma(const void* operands, int32_t iters, float* sink, double* flops /* host */, void* stream);
-int dew_moe_probe_copy(const void* src, void* dst, size_t bytes, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

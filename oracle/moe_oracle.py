@@ -308,11 +308,9 @@ def top_k(values, k):
     return np.take_along_axis(values, order, axis=-1), order.astype(np.int32)
 
 
-def route(logits, top_k_count, *, score_function="softmax", normalize_weights=True, bias=None,
-          routed_scaling_factor=1.0, expert_groups=1, groups_per_token=1, group_score="top2",
-          weight_sum_epsilon=1e-20):
-    """`Router.__call__` from its logits on (src/dew/nn/moe.py:466-494): scores, selection (bias,
-    group-limited mask :496-565), top-k, weights. Returns (weights fp32 [T, k], indices int32 [T, k])."""
+def selection_scores(logits, *, score_function="softmax", bias=None, expert_groups=1, groups_per_token=1, group_score="top2"):
+    """(scores, selection) of `Router.__call__` (src/dew/nn/moe.py:466-470, 516-524): the activated scores and what the
+    top-k runs over, the scores plus the bias with the experts outside a token's best groups at -inf (:496-565)."""
     logits = np.asarray(logits, F32)
     experts = logits.shape[-1]
     if score_function == "softmax":
@@ -324,6 +322,9 @@ def route(logits, top_k_count, *, score_function="softmax", normalize_weights=Tr
     else:
         raise ValueError(score_function)
     selection = scores if bias is None else (scores + np.asarray(bias, F32)).astype(F32)
+    # A NaN selection competes as -inf (the HIP router's rule): none of the reference's tests feeds its `lax.top_k` a
+    # NaN, so this is a choice of this restatement, made so that every choice stays an expert in range.
+    selection = np.where(np.isnan(selection), F32(-np.inf), selection)
     if expert_groups > 1:
         per_group = experts // expert_groups
         grouped = selection.reshape(*selection.shape[:-1], expert_groups, per_group)
@@ -336,6 +337,32 @@ def route(logits, top_k_count, *, score_function="softmax", normalize_weights=Tr
         kept = np.zeros(group_scores.shape, bool)
         np.put_along_axis(kept, groups, True, axis=-1)
         selection = np.where(np.repeat(kept, per_group, axis=-1), selection, F32(-np.inf))
+    return scores, selection
+
+
+def top_k_margin(selection, top_k_count):
+    """The least gap, over the tokens, between the last selection chosen and the best one left out, as (gap, the gap in
+    units of the chosen value's fp32 spacing, token). A gap of zero is a tie, which the lower index wins in every
+    implementation; a gap of a few spacings is where two exponentials that round differently could choose differently."""
+    selection = np.asarray(selection, F32)
+    if selection.shape[-1] <= top_k_count:
+        return float("inf"), float("inf"), -1
+    ranked = -np.sort(-selection.reshape(-1, selection.shape[-1]), axis=-1)
+    last, left = ranked[:, top_k_count - 1], ranked[:, top_k_count]
+    gap = (last.astype(np.float64) - left.astype(np.float64))
+    gap[~np.isfinite(left)] = np.inf
+    token = int(gap.argmin())
+    return float(gap[token]), float(gap[token] / np.spacing(np.abs(last[token]))), token
+
+
+def route(logits, top_k_count, *, score_function="softmax", normalize_weights=True, bias=None,
+          routed_scaling_factor=1.0, expert_groups=1, groups_per_token=1, group_score="top2",
+          weight_sum_epsilon=1e-20):
+    """`Router.__call__` from its logits on (src/dew/nn/moe.py:466-494): scores, selection (bias,
+    group-limited mask :496-565), top-k, weights. Returns (weights fp32 [T, k], indices int32 [T, k])."""
+    logits = np.asarray(logits, F32)
+    scores, selection = selection_scores(logits, score_function=score_function, bias=bias, expert_groups=expert_groups,
+                                         groups_per_token=groups_per_token, group_score=group_score)
     _, indices = top_k(selection, top_k_count)
     if normalize_weights and score_function == "softmax":
         weights = expert_softmax(np.take_along_axis(logits, indices, axis=-1))        # moe.py:194-199,485

@@ -58,6 +58,26 @@ def test_router_matches_the_oracle_bit_for_bit(ops, name, experts, k, settings, 
     assert np.array_equal(got_w.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
 
 
+def test_a_nan_selection_bias_is_never_chosen_and_every_choice_stays_in_range(ops):
+    """A NaN in the selection bias makes that expert's selection NaN for every token. It competes as -inf: never
+    chosen while k others remain, and when fewer remain the lowest remaining indices fill in, all within range."""
+    rng = np.random.default_rng(3)
+    experts, k, tokens = 64, 6, 257
+    logits = rng.standard_normal((tokens, experts)).astype(np.float32)
+    settings = dict(score_function="sigmoid", normalize_weights=True, routed_scaling_factor=1.5)
+    for poisoned in ([5], list(range(60)), list(range(64))):
+        bias = (rng.standard_normal(experts) * 0.1).astype(np.float32)
+        bias[poisoned] = np.nan
+        want_w, want_i = oracle.route(logits, k, bias=bias, **settings)
+        got_w, got_i = ops.route(torch.from_numpy(logits).cuda(), k, bias=torch.from_numpy(bias).cuda(), **settings)
+        got_i = got_i.cpu().numpy()
+        assert got_i.min() >= 0 and got_i.max() < experts
+        assert np.array_equal(got_i, want_i)
+        assert np.array_equal(got_w.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
+        if len(poisoned) <= experts - k:
+            assert not np.isin(got_i, poisoned).any()
+
+
 def test_router_reproduces_the_reference_fixtures_on_the_device(ops):
     from conftest import golden
     for name, settings in (("mixtral", dict(score_function="softmax", normalize_weights=True)),
@@ -262,11 +282,13 @@ def test_an_mxfp4_bank_is_recognized_at_preparation_and_a_general_bank_is_not(op
     assert ops.prepare(quantize(weight, "nvfp4").to("cuda")).descriptor.format == _lib.W_NVFP4
 
 
-def test_probes_run_and_the_copy_probe_copies(ops):
+def test_the_benchmarks_probes_run_and_the_copy_probe_copies():
+    from bench_aids import probes
+
     src = torch.arange(1 << 20, dtype=torch.int32, device="cuda")
     dst = torch.zeros_like(src)
-    assert ops.probe_copy(src, dst) == 4 << 20 and torch.equal(src, dst)
-    assert ops.probe_mfma(torch.randn(16384, device="cuda").to(torch.bfloat16), 10) == 1024 * 4 * 10 * 16 * 32768.0
+    assert probes.probe_copy(src, dst) == 4 << 20 and torch.equal(src, dst)
+    assert probes.probe_mfma(torch.randn(16384, device="cuda").to(torch.bfloat16), 10) == 1024 * 4 * 10 * 16 * 32768.0
 
 
 @pytest.mark.parametrize("quant", ["fp8_channel", "fp8_block", "mxfp4", "nvfp4", "bf16"])
@@ -410,6 +432,37 @@ def test_a_layer_of_a_stacked_bank_is_read_where_it_lies(ops, quant):
         assert torch.equal(through, alone)
     with pytest.raises(Exception):
         stack.layer(3, layers)
+
+
+def test_a_layer_of_a_stacked_mxfp8_bank_and_a_scaled_layer_are_read_where_they_lie(ops):
+    """The two reads of a stack that move more than the codes: an MXFP8 bank's scale lines (one byte every 32 depths,
+    half an NVFP4 bank's stride) and `layer(i).scaled(by)`, which owes layer i's own tensor scales, not the stack's
+    first ones. Both against the layer's bank prepared alone, bit for bit."""
+    from dew_amd import formats
+
+    layers, experts, depth, width = 4, 3, 512, 256
+    sizes = [70, 0, 129]
+    rng = np.random.default_rng(23)
+    offsets = torch.tensor(np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)).cuda()
+    x = torch.from_numpy(rng.standard_normal((sum(sizes), depth)).astype(np.float32)).to(torch.bfloat16).cuda()
+    spread = np.exp2(rng.integers(-4, 5, size=(layers * experts, depth // 32, width))).repeat(32, axis=1)
+    weights = torch.from_numpy((rng.standard_normal((layers * experts, depth, width)) * 0.02 * spread).astype(np.float32))
+    stack = ops.prepare(formats.MxFp8.quantized(weights).to("cuda"))
+    codes, scales = ops.quantize_rows_mxfp8(x)
+    for layer in range(layers):
+        alone = ops.prepare(formats.MxFp8.quantized(weights[layer * experts:(layer + 1) * experts]).to("cuda"))
+        want = ops.grouped_gemm_mxfp8_rows(codes, scales, alone, offsets)
+        assert torch.equal(ops.grouped_gemm_mxfp8_rows(codes, scales, stack.layer(layer, layers), offsets), want), layer
+
+    banks = [grouped_case("nvfp4", experts, depth, width, sizes, seed=50 + layer)[0] for layer in range(layers)]
+    first = banks[0]
+    joined = {field.name: torch.cat([getattr(bank, field.name) for bank in banks]) for field in dataclasses.fields(first)
+              if torch.is_tensor(getattr(first, field.name)) and field.name != "form"}
+    stack = ops.prepare(type(first)(**joined).to("cuda"))
+    by = torch.tensor([0.375], device="cuda")
+    for layer in range(layers):
+        want = ops.grouped_gemm(x, ops.prepare(banks[layer].to("cuda")).scaled(by), offsets)
+        assert torch.equal(ops.grouped_gemm(x, stack.layer(layer, layers).scaled(by), offsets), want), layer
 
 
 @pytest.mark.parametrize("quant", ["fp8_block", "fp8_channel", "mxfp4", "nvfp4", "bf16"])

@@ -306,3 +306,16 @@ def test_the_sown_statistics_are_the_scores_and_the_log_partition():
     assert np.abs(shifted - (log_z + 8.0)).max() <= 1e-5
     sigmoid, same = oracle.router_statistics(logits, score_function="sigmoid")
     assert np.array_equal(same, log_z) and np.abs(sigmoid - 1 / (1 + np.exp(-wide))).max() <= 1e-6
+
+
+def test_a_nan_selection_competes_as_minus_infinity():
+    """The router's rule for a NaN selection (a NaN bias entry): never preferred, and every choice an expert in range."""
+    rng = np.random.default_rng(3)
+    logits = rng.standard_normal((9, 16)).astype(np.float32)
+    bias = np.zeros(16, np.float32)
+    bias[[2, 7]] = np.nan
+    _, indices = oracle.route(logits, 4, score_function="sigmoid", bias=bias)
+    assert not np.isin(indices, [2, 7]).any() and indices.min() >= 0 and indices.max() < 16
+    bias[:] = np.nan
+    _, indices = oracle.route(logits, 4, score_function="sigmoid", bias=bias)
+    assert np.array_equal(indices, np.tile(np.arange(4, dtype=np.int32), (9, 1)))
