@@ -7,6 +7,8 @@
 //   scatter each wavefront ranks its 64 slots among themselves with ballots (match-any over the id's bits),
 //           adds the running count of earlier slots, and writes order[] / rows[]
 // Slots whose id is >= experts (a dropped slot's sentinel) sort last, in slot order, outside every group.
+#include <mutex>
+
 #include "common.h"
 
 namespace dew {
@@ -228,22 +230,13 @@ extern "C" size_t dew_moe_permute_workspace_bytes(int32_t slots, int32_t experts
   return 2 * blocks * (static_cast<size_t>(experts) + 1) * sizeof(int32_t) + 256;
 }
 
-extern "C" int dew_moe_permute(const int32_t* indices, int32_t tokens, int32_t top_k, int32_t experts,
-                               int32_t* sizes, int32_t* offsets, int32_t* order, int32_t* rows,
-                               void* workspace, size_t workspace_bytes, void* stream) {
-  using namespace dew;
-  DEW_REQUIRE(tokens >= 0 && top_k >= 1, "dew_moe_permute: tokens %d top_k %d", tokens, top_k);
-  DEW_REQUIRE(experts >= 1 && experts <= kMaxExperts, "dew_moe_permute: experts %d (at most %d)", experts,
-              kMaxExperts);
-  DEW_REQUIRE(static_cast<int64_t>(tokens) * top_k < (1ll << 30), "dew_moe_permute: %d x %d slots overflow int32",
-              tokens, top_k);
-  DEW_REQUIRE(sizes && offsets, "dew_moe_permute: sizes and offsets must not be null");
+namespace dew {
+
+// The sort's launches, given where the per-block counts and bases live (the caller's workspace or the library's own
+// scratch array): `counts` holds 2 * blocks * buckets int32, 256-byte aligned.
+static int permute_launches(const int32_t* indices, int32_t tokens, int32_t top_k, int32_t experts, int32_t* sizes,
+                            int32_t* offsets, int32_t* order, int32_t* rows, int32_t* counts, hipStream_t s) {
   const int slots = tokens * top_k;
-  DEW_REQUIRE(slots == 0 || (indices && order && rows), "dew_moe_permute: indices, order and rows must not be null");
-  DEW_REQUIRE(workspace && workspace_bytes >= dew_moe_permute_workspace_bytes(slots, experts),
-              "dew_moe_permute: workspace of %zu bytes, need %zu", workspace_bytes,
-              dew_moe_permute_workspace_bytes(slots, experts));
-  hipStream_t s = static_cast<hipStream_t>(stream);
   PermuteParams p;
   p.ids = indices;
   p.sizes = sizes;
@@ -255,24 +248,87 @@ extern "C" int dew_moe_permute(const int32_t* indices, int32_t tokens, int32_t t
   p.top_k = top_k;
   p.buckets = experts + 1;
   p.blocks = (slots + kSlotsPerBlock - 1) / kSlotsPerBlock;
-  uintptr_t base = (reinterpret_cast<uintptr_t>(workspace) + 255) & ~static_cast<uintptr_t>(255);
-  p.counts = reinterpret_cast<int32_t*>(base);
+  p.counts = counts;
   p.bases = p.counts + static_cast<size_t>(p.blocks) * p.buckets;
   if (slots <= kSmallSlots) {  // one block does it all faster than three launches
     hipLaunchKernelGGL(permute_small_kernel, dim3(1), dim3(kPermuteThreads),
                        sizeof(int32_t) * ((kPermuteWaves + 1) * p.buckets + 1), s, p);
     return launched("permute_small_kernel");
   }
-  if (p.blocks > 0) {
-    hipLaunchKernelGGL(permute_count_kernel, dim3(p.blocks), dim3(kPermuteThreads), sizeof(int32_t) * p.buckets, s, p);
-    if (int rc = launched("permute_count_kernel")) return rc;
-  }
+  hipLaunchKernelGGL(permute_count_kernel, dim3(p.blocks), dim3(kPermuteThreads), sizeof(int32_t) * p.buckets, s, p);
+  if (int rc = launched("permute_count_kernel")) return rc;
   hipLaunchKernelGGL(permute_scan_kernel, dim3(1), dim3(kPermuteThreads), sizeof(int32_t) * (p.buckets + 1), s, p);
   if (int rc = launched("permute_scan_kernel")) return rc;
-  if (p.blocks > 0) {
-    hipLaunchKernelGGL(permute_scatter_kernel, dim3(p.blocks), dim3(kPermuteThreads),
-                       sizeof(int32_t) * kPermuteWaves * p.buckets, s, p);
-    if (int rc = launched("permute_scatter_kernel")) return rc;
-  }
+  hipLaunchKernelGGL(permute_scatter_kernel, dim3(p.blocks), dim3(kPermuteThreads),
+                     sizeof(int32_t) * kPermuteWaves * p.buckets, s, p);
+  return launched("permute_scatter_kernel");
+}
+
+static int permute_arguments(const char* who, const int32_t* indices, int32_t tokens, int32_t top_k, int32_t experts,
+                             const int32_t* sizes, const int32_t* offsets, const int32_t* order, const int32_t* rows) {
+  DEW_REQUIRE(tokens >= 0 && top_k >= 1, "%s: tokens %d top_k %d", who, tokens, top_k);
+  DEW_REQUIRE(experts >= 1 && experts <= kMaxExperts, "%s: experts %d (at most %d)", who, experts, kMaxExperts);
+  DEW_REQUIRE(static_cast<int64_t>(tokens) * top_k < (1ll << 30), "%s: %d x %d slots overflow int32", who, tokens, top_k);
+  DEW_REQUIRE(sizes && offsets, "%s: sizes and offsets must not be null", who);
+  DEW_REQUIRE(tokens * top_k == 0 || (indices && order && rows), "%s: indices, order and rows must not be null", who);
   return DEW_MOE_OK;
+}
+
+// The library's own scratch for dew_moe_permute_static: the per-block counts and bases of the three-launch sort.
+// Every GPU the library runs on holds its own copy of the array until the process ends. The array's name is a
+// host-side stand-in for it, not a device address: host code uses the address hipGetSymbolAddress returns for the
+// current device, looked up once a device and kept.
+constexpr size_t kStaticScratchBytes = DEW_MOE_PERMUTE_STATIC_BYTES;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static void* scratch_of_device[kMaxDevices];  // null until the device's first call
+static std::mutex scratch_lookup;
+
+static int static_scratch(const char* who, void** out) {
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices)
+    return fail(DEW_MOE_EDEVICE, "%s: no HIP device below %d is current", who, kMaxDevices);
+  std::lock_guard<std::mutex> hold(scratch_lookup);
+  if (scratch_of_device[device] == nullptr) {
+    void* address = nullptr;
+    const hipError_t status = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
+    if (status != hipSuccess || address == nullptr)
+      return fail(DEW_MOE_ELAUNCH, "%s: hipGetSymbolAddress of the scratch array on device %d: %s", who, device,
+                  hipGetErrorString(status));
+    scratch_of_device[device] = address;
+  }
+  *out = scratch_of_device[device];
+  return DEW_MOE_OK;
+}
+
+}  // namespace dew
+
+extern "C" int dew_moe_permute(const int32_t* indices, int32_t tokens, int32_t top_k, int32_t experts,
+                               int32_t* sizes, int32_t* offsets, int32_t* order, int32_t* rows,
+                               void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace dew;
+  if (int rc = permute_arguments("dew_moe_permute", indices, tokens, top_k, experts, sizes, offsets, order, rows)) return rc;
+  const int slots = tokens * top_k;
+  DEW_REQUIRE(workspace && workspace_bytes >= dew_moe_permute_workspace_bytes(slots, experts),
+              "dew_moe_permute: workspace of %zu bytes, need %zu", workspace_bytes,
+              dew_moe_permute_workspace_bytes(slots, experts));
+  const uintptr_t base = (reinterpret_cast<uintptr_t>(workspace) + 255) & ~static_cast<uintptr_t>(255);
+  return permute_launches(indices, tokens, top_k, experts, sizes, offsets, order, rows, reinterpret_cast<int32_t*>(base),
+                          static_cast<hipStream_t>(stream));
+}
+
+extern "C" int dew_moe_permute_static(const int32_t* indices, int32_t tokens, int32_t top_k, int32_t experts,
+                                      int32_t* sizes, int32_t* offsets, int32_t* order, int32_t* rows, void* stream) {
+  using namespace dew;
+  const char* who = "dew_moe_permute_static";
+  if (int rc = permute_arguments(who, indices, tokens, top_k, experts, sizes, offsets, order, rows)) return rc;
+  const size_t need = dew_moe_permute_workspace_bytes(tokens * top_k, experts);
+  DEW_REQUIRE(need <= kStaticScratchBytes,
+              "%s: %d slots over %d experts need %zu bytes of scratch, the library's own array holds %zu; use dew_moe_permute "
+              "with a workspace", who, tokens * top_k, experts, need, kStaticScratchBytes);
+  void* base = nullptr;
+  if (int rc = static_scratch(who, &base)) return rc;
+  // every int32 of the counts and bases a call reads is written earlier in the same call: nothing to clear
+  return permute_launches(indices, tokens, top_k, experts, sizes, offsets, order, rows, static_cast<int32_t*>(base),
+                          static_cast<hipStream_t>(stream));
 }

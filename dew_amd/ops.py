@@ -135,6 +135,23 @@ def sort_by_expert(indices: torch.Tensor, num_experts: int) -> Plan:
     return Plan(order, rows, sizes, offsets)
 
 
+def sort_by_expert_into(indices: torch.Tensor, num_experts: int, plan: Plan) -> Plan:
+    """`sort_by_expert` written into a `Plan` the caller already holds, through `dew_moe_permute_static`: no device
+    memory is allocated (the sort's scratch is the library's own array), for steps that run where nothing may
+    allocate. Sorts within `dew_moe_permute_static`'s limit only; calls that overlap on one GPU race."""
+    _device(indices, "indices", torch.int32)
+    top_k = indices.shape[-1]
+    tokens = indices.numel() // top_k
+    for name, tensor, count in (("sizes", plan.sizes, num_experts), ("offsets", plan.offsets, num_experts + 1),
+                                ("order", plan.order, tokens * top_k), ("rows", plan.rows, tokens * top_k)):
+        _device(tensor, name, torch.int32)
+        if tensor.numel() < count:
+            raise KernelError(f"plan.{name} holds {tensor.numel()} values, the sort writes {count}")
+    _lib.check(_lib.library().dew_moe_permute_static(_ptr(indices), tokens, top_k, num_experts, _ptr(plan.sizes), _ptr(plan.offsets),
+                                                     _ptr(plan.order), _ptr(plan.rows), _stream()), "dew_moe_permute_static")
+    return plan
+
+
 # ---- banks ----------------------------------------------------------------------------------------------
 
 

@@ -107,6 +107,18 @@ int dew_moe_permute(const int32_t* indices /* [T,k] */, int32_t tokens, int32_t 
                     int32_t* sizes, int32_t* offsets, int32_t* order, int32_t* rows, void* workspace,
                     size_t workspace_bytes, void* stream);
 
+/* dew_moe_permute for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc) and so have no workspace to hand in; no counterpart in the reference, whose FFI
+ * handler takes its workspace from XLA's ScratchAllocator. The sort's per-block counts live in an array of
+ * DEW_MOE_PERMUTE_STATIC_BYTES that the library itself holds on every GPU it runs on until the process ends; a
+ * problem whose dew_moe_permute_workspace_bytes() is larger is refused (slots / 2048 blocks x (experts + 1) x 8 bytes:
+ * 1 MiB covers e.g. 2^20 slots over 255 experts). Calls on one GPU share that array: calls that overlap on
+ * different streams of one GPU race; calls in stream order need nothing cleared between them. The call allocates and
+ * frees nothing; outputs are identical to dew_moe_permute's.                                                    */
+#define DEW_MOE_PERMUTE_STATIC_BYTES ((size_t)1 << 20)
+int dew_moe_permute_static(const int32_t* indices /* [T,k] */, int32_t tokens, int32_t top_k, int32_t experts,
+                           int32_t* sizes, int32_t* offsets, int32_t* order, int32_t* rows, void* stream);
+
 /* offsets[E+1] = exclusive prefix of group sizes[E] (implicit in jax.lax.ragged_dot's group_sizes,
  * src/dew/nn/kernels/xla_products.py:86-115; explicit at src/dew/nn/moe.py:1172).                        */
 int dew_moe_group_offsets(const int32_t* sizes, int32_t experts, int32_t* offsets, void* stream);
