@@ -4,16 +4,20 @@ A step is one pass of the hot path over one batch of synthetic input already res
 sort by expert -> gate/up grouped GEMM with the SwiGLU epilogue -> down grouped GEMM scattered to slot
 order -> weighted combine (+ shared expert where the config has one). Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--only] [--no-cpu-baseline]
 
-`value` is algorithmic TFLOP/s of the whole step: 6 * R * D * F (+ 6 * T * D * F_shared), the reference's
-own convention of three projections per dispatched row (src/dew/nn/moe.py:1275-1281), over the measured step
-time. `roofline` is the dominant kernel alone (the paired gate/up launch: two thirds of the FLOPs), timed
-with HIP events recorded on the launch stream around every one of its launches in the timed region.
-`cpu_baseline` is the CPU oracle on a bounded sample of the same workload, on this box's host cores.
+The line's top level is the `--config` workload (default c2, the one the metric is quoted on). `value` is
+algorithmic TFLOP/s of the whole step: 6 * R * D * F (+ 6 * T * D * F_shared), the reference's own convention of
+three projections per dispatched row (src/dew/nn/moe.py:1275-1281), over the measured step time. `roofline` is
+the dominant kernel alone (the paired gate/up launch: two thirds of the FLOPs), timed with HIP events recorded on
+the launch stream around every one of its launches in the timed region. `cpu_baseline` is the CPU oracle on a
+bounded sample of the same workload, on this box's host cores. `configs` holds the same measurement for each of
+the five workloads c1 .. c5 (step time, the dominant kernel against its roofline, parity of a full-size sample
+against the CPU oracle, and the least top-k margin of the routing); `--only` leaves it out.
 """
 
 import argparse
+import gc
 import json
 import os
 import sys
@@ -26,6 +30,12 @@ sys.path.insert(0, str(ROOT / "tests"))
 
 PEAKS = {"bf16_mfma": 2500.0, "fp8_mfma": 5000.0, "fp4_mfma": 10100.0, "hbm_gbs": 8000.0}
 """MI355X published dense peaks, TFLOP/s and GB/s."""
+
+ALL_CONFIGS = ("c1", "c2", "c3", "c4", "c5")
+GRAPHED = ("c1", "c3")
+"""The launch-bound workloads: their step is replayed as one captured HIP graph."""
+DECODE = ("c3",)
+"""The workloads whose dominant kernel is bound by HBM bandwidth, not by the matrix cores."""
 
 
 def build_workload(case, device, seed=0):
@@ -130,11 +140,10 @@ class Stepper:
         return sum(start.elapsed_time(stop) for start, stop in self.events) / max(1, len(self.events))
 
 
-def cpu_baseline(case, data, out, plan, budget_rows=192):
-    """The CPU oracle (dequantize -> bf16-exact fp32 GEMMs -> SwiGLU -> down) on a bounded sample: the
-    busiest expert's first `budget_rows` sorted rows, all three projections at full width. Also checks the
-    GPU's hidden-to-output path for those rows against it."""
-    import numpy as np
+def oracle_sample(case, data, plan, budget_rows=192):
+    """The CPU oracle (dequantize -> bf16-exact fp32 GEMMs -> SwiGLU -> down) on a bounded sample of the workload: the
+    busiest expert's first `budget_rows` sorted rows, all three projections at full width. Returns the timing as the
+    `cpu_baseline` object and (the slots of those rows, the oracle's down-projection rows for them)."""
     import torch
     from moe_cases import dequantized
 
@@ -175,13 +184,19 @@ def cpu_baseline(case, data, out, plan, budget_rows=192):
 
 
 # HBM bytes one launch of the dominant (gate/up) kernel moved, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (KiB per
-# dispatch, two runs of this file per workload), each scaled by what the same counter reads for the plain copy probe of known
-# size (--calibrate-copy: FETCH_SIZE reads half of the bytes fetched, WRITE_SIZE all of the bytes written). The counters
-# cannot be read from inside this process, so the figures sit here and are refreshed with the summaries kept beside the
-# kernel traces; a workload without an entry reports null.
+# dispatch, two runs of `bench.py --config cN --only` per workload), each scaled by what the same counter reads for the plain
+# copy probe of known size (--calibrate-copy: FETCH_SIZE reads half of the bytes fetched, WRITE_SIZE all of the bytes
+# written). The counters cannot be read from inside this process, so the figures sit here, taken from the summaries under
+# profiles/ named in COUNTED_FROM; `roofline.traffic_source` says so in the line. A workload without an entry reports null.
 COUNTER_SCALE = {"FETCH_SIZE": 2.0, "WRITE_SIZE": 1.0}
-COUNTED_KIB = {"c2": {"FETCH_SIZE": 3105088.8, "WRITE_SIZE": 946747.0},
-               "c3": {"FETCH_SIZE": 194873.3, "WRITE_SIZE": 768.0}}
+COUNTED_KIB = {"c1": {"FETCH_SIZE": 8891.1, "WRITE_SIZE": 8192.0},
+               "c2": {"FETCH_SIZE": 3105110.7, "WRITE_SIZE": 946751.4},
+               "c3": {"FETCH_SIZE": 194866.8, "WRITE_SIZE": 768.0},
+               "c4": {"FETCH_SIZE": 4908110.0 + 1961998.4, "WRITE_SIZE": 244552.0 + 17592.0},   # the 128-row tiles' launch + the last tiles' 64-row launch
+               "c5": {"FETCH_SIZE": 976239.3, "WRITE_SIZE": 229376.0}}
+COUNTED_FROM = {"c1": "profiles/grouped_gemm_c1_small_fp8_channel.txt", "c2": "profiles/grouped_gemm_c2_prefill_mxfp4.txt",
+                "c3": "profiles/grouped_gemm_c3_decode_fp8.txt", "c4": "profiles/grouped_gemm_c4_prefill_fp8_blocks.txt",
+                "c5": "profiles/grouped_gemm_c5_prefill_nvfp4.txt"}
 
 
 def measured_traffic(config):
@@ -194,65 +209,39 @@ def sustained_rates(device):
     bytes read plus bytes written), each timed with HIP events over several launches after a warm-up."""
     import torch
 
-    from bench_aids import probes as ops
+    from bench_aids import probes
 
     operands = torch.randn(16384, device=device).to(torch.bfloat16)
-    ops.probe_mfma(operands, 2000)
+    probes.probe_mfma(operands, 2000)
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
-    flops = sum(ops.probe_mfma(operands, 20000) for _ in range(3))
+    flops = sum(probes.probe_mfma(operands, 20000) for _ in range(3))
     stop.record()
     torch.cuda.synchronize()
     mfma = flops / (start.elapsed_time(stop) * 1e-3) / 1e12
     src = torch.empty(1 << 30, dtype=torch.uint8, device=device).random_()
     dst = torch.empty_like(src)
-    ops.probe_copy(src, dst)
+    probes.probe_copy(src, dst)
     start.record()
-    moved = sum(2 * ops.probe_copy(src, dst) for _ in range(5))
+    moved = sum(2 * probes.probe_copy(src, dst) for _ in range(5))
     stop.record()
     torch.cuda.synchronize()
     return round(mfma, 1), round(moved / (start.elapsed_time(stop) * 1e-3) / 1e9, 1)
 
 
-def main():
-    parser = argparse.ArgumentParser()
-    parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=20)
-    parser.add_argument("--warmup", type=int, default=3)
-    parser.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
-    parser.add_argument("--no-cpu-baseline", action="store_true")
-    parser.add_argument("--calibrate-copy", action="store_true",
-                        help="only run the plain copy probe (1 GiB read + 1 GiB written, 5 launches): the known traffic "
-                             "that rocprofv3's FETCH_SIZE / WRITE_SIZE are scaled by")
-    parser.add_argument("--bf16-operands", action="store_true",
-                        help="keep MXFP4 banks with groups of hundreds of rows on the bf16 matrix instruction too (the default "
-                             "there: rows split into two e4m3 terms and the scaled instruction, the library's own choice)")
-    parser.add_argument("--graph", choices=["auto", "on", "off"], default="auto",
-                        help="replay the step as one captured HIP graph (auto: for the launch-bound configs c1 and c3)")
-    args = parser.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the path would shard by expert over "
-                 "an all-to-all each way; that is designed, not built). Run with --gpus 1.")
-
-    import numpy as np
+def measure(config, args, device, sustained, with_cpu_baseline):
+    """One workload, measured: its part of the line (ms_per_step, value, config, roofline, sample_parity,
+    min_topk_margin and, where asked, cpu_baseline)."""
     import torch
     from moe_cases import CONFIGS
 
-    from dew_amd import ops
+    from bench_aids import probes
+    from oracle import moe_oracle as oracle
 
-    ops.device_check()
-    device = torch.device("cuda:0")
-    torch.cuda.set_device(device)
-    if args.calibrate_copy:
-        mfma, copy = sustained_rates(device)
-        print(json.dumps({"probe_copy_bytes_read_per_launch": 1 << 30, "probe_copy_bytes_written_per_launch": 1 << 30,
-                          "sustained_copy_gbs": copy, "sustained_bf16_mfma_tflops": mfma}))
-        return
-    case = CONFIGS[args.config]
+    case = CONFIGS[config]
     data = build_workload(case, device)
     stepper = Stepper(case, data, split=not args.bf16_operands)
-
-    graphed = args.graph == "on" or (args.graph == "auto" and args.config in ("c1", "c3"))
+    graphed = args.graph == "on" or (args.graph == "auto" and config in GRAPHED)
     for _ in range(args.warmup):
         stepper()
     torch.cuda.synchronize()
@@ -273,7 +262,6 @@ def main():
         # millisecond of queued work ahead of each step lets the host run ahead, so the step's launches follow each
         # other on the device as they do in the graph and the events bracket the kernel, not the host's launch path.
         operands = torch.randn(16384, device=device).to(torch.bfloat16)
-        from bench_aids import probes
         for _ in range(args.steps):
             probes.probe_mfma(operands, 1200)
             stepper(timed=True)
@@ -291,30 +279,34 @@ def main():
     gateup_flops = 4.0 * routed_rows * case.d_model * case.d_ff
     gateup_ms = stepper.gateup_ms()
     achieved = gateup_flops / (gateup_ms * 1e-3) / 1e12
-    decode = args.config == "c3"
+    decode = config in DECODE
     bytes_per_weight = 0.5 if case.quant in ("mxfp4", "nvfp4") else 1.0
     touched = int((plan.sizes > 0).sum().item())
+    # bandwidth view: the touched experts' gate and up codes read once + activations in, hidden out
+    gateup_bytes = touched * 2 * case.d_model * case.d_ff * bytes_per_weight + case.tokens * case.d_model * 2 + routed_rows * case.d_ff * 2
+    gateup_gbs = gateup_bytes / (gateup_ms * 1e-3) / 1e9
+    sustained_mfma, sustained_copy = sustained
     if decode:
-        # bandwidth view: the touched experts' gate and up codes read once + activations in, hidden out
-        gateup_bytes = touched * 2 * case.d_model * case.d_ff * bytes_per_weight + case.tokens * case.d_model * 2 + routed_rows * case.d_ff * 2
-        roofline = {"bound": "hbm", "achieved": round(gateup_bytes / (gateup_ms * 1e-3) / 1e9, 1), "peak": PEAKS["hbm_gbs"],
-                    "unit": "GB/s", "traffic": None}
+        roofline = {"bound": "hbm", "achieved": round(gateup_gbs, 1), "peak": PEAKS["hbm_gbs"], "unit": "GB/s"}
     else:
-        roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAKS["bf16_mfma"], "unit": "TFLOP/s", "traffic": None,
+        roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAKS["bf16_mfma"], "unit": "TFLOP/s",
                     "peak_note": ("the kernel multiplies each bf16 activation as two e4m3 terms by the stored FP4 codes "
                                   "(v_mfma_scale_f32_32x32x64_f8f6f4, which runs at the dense fp8 rate, 5.0 PFLOP/s published): "
                                   "two instruction flops per algorithmic flop, so the algorithm's ceiling is 2.5 PFLOP/s, the "
                                   "dense bf16 peak; achieved counts algorithmic flops only") if stepper.on_split_rows() else
                                  ("dense bf16 MFMA: the kernel multiplies bf16 activations by weights dequantized exactly to "
                                   "bf16 (v_mfma_f32_32x32x16_bf16)"),
-                    "frac_of_fp8_peak": round(achieved / PEAKS["fp8_mfma"], 4), "frac_of_fp4_peak": round(achieved / PEAKS["fp4_mfma"], 4)}
+                    "frac_of_fp8_peak": round(achieved / PEAKS["fp8_mfma"], 4), "frac_of_fp4_peak": round(achieved / PEAKS["fp4_mfma"], 4),
+                    "hbm_view": {"algorithmic_bytes": gateup_bytes, "gbs": round(gateup_gbs, 1),
+                                 "frac_of_hbm_peak": round(gateup_gbs / PEAKS["hbm_gbs"], 4)}}
     roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
     if not decode and stepper.on_split_rows():
         roofline["executed"] = {"tflops": round(2 * achieved, 1), "frac_of_fp8_peak": round(2 * achieved / PEAKS["fp8_mfma"], 4),
                                 "note": "instruction flops: both terms' products"}
-    roofline["traffic"] = measured_traffic(args.config)
+    roofline["traffic"] = measured_traffic(config)
+    roofline["traffic_source"] = (f"stored: rocprofv3 --pmc FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 of this command's gate/up launch, "
+                                  f"{COUNTED_FROM[config]}; not measured in this run") if config in COUNTED_KIB else None
     roofline["algorithmic"] = {"per_launch": gateup_bytes if decode else gateup_flops, "unit": "bytes" if decode else "flop"}
-    sustained_mfma, sustained_copy = sustained_rates(device)
     roofline["sustained"] = {"bf16_mfma_random_operands_tflops": sustained_mfma, "plain_copy_gbs": sustained_copy,
                              "frac_of_sustained": round(roofline["achieved"] / (sustained_copy if decode else sustained_mfma), 4),
                              "note": "measured in this run by bench_aids' MFMA and copy probes: the rate the chip holds on "
@@ -324,26 +316,93 @@ def main():
     roofline["kernel_ms"] = round(gateup_ms, 4)
 
     result = {
-        "metric": "grouped-GEMM TFLOP/s & % MFMA peak (prefill); HBM GB/s & % peak (decode)",
-        "value": round(flops / (ms_per_step * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"{args.config}: T={case.tokens} D={case.d_model} F={case.d_ff} E={case.experts} k={case.top_k} "
+        "value": round(flops / (ms_per_step * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "ms_per_step": round(ms_per_step, 4),
+        "config": {"workload": f"{config}: T={case.tokens} D={case.d_model} F={case.d_ff} E={case.experts} k={case.top_k} "
                                f"{case.quant} weights, {case.router['score_function']} router"
                                + (" + shared expert" if case.shared else ""),
                    "routed_rows": routed_rows, "experts_touched": touched, "launch": "hip graph replay" if graphed else "eager",
                    "algorithmic_flops": flops},
         "roofline": roofline,
     }
-    if not args.no_cpu_baseline:
-        baseline, (slots, want) = cpu_baseline(case, data, out, plan)
-        result["cpu_baseline"] = baseline
+    # the routing's least top-k margin: how close the last chosen selection comes to the best one left out
+    router = {k: v for k, v in case.router.items() if k in ("score_function", "expert_groups", "groups_per_token")}
+    _, selection = oracle.selection_scores(data["logits"].cpu().numpy(), bias=None if data["bias"] is None else data["bias"].cpu().numpy(),
+                                           **router)
+    gap, spacings, token = oracle.top_k_margin(selection, case.top_k)
+    finite = gap != float("inf")
+    result["min_topk_margin"] = {"value": gap if finite else None, "fp32_spacings": round(spacings, 1) if finite else None, "token": token,
+                                 "note": "least gap over the tokens between the k-th selection and the best one left out; 0 is an "
+                                         "exact tie (the lower index wins everywhere)"}
+    if with_cpu_baseline or not args.no_parity:
+        baseline, (slots, want) = oracle_sample(case, data, plan)
+        if with_cpu_baseline:
+            result["cpu_baseline"] = baseline
         # parity on the sample at full size: the device's down-projection rows for those slots
-        projected = stepper.project(plan).float().cpu().numpy()
-        got = projected[slots]
-        scale = float(np.abs(want).max())
-        result["sample_parity"] = {"max_abs_over_max_ref": round(float(np.abs(got - want).max() / scale), 6),
-                                   "rows": int(len(slots))}
+        got = stepper.project(plan).float().cpu().numpy()[slots]
+        by_max, by_element = oracle.relative_errors(got, want)
+        result["sample_parity"] = {"max_abs_over_max_ref": round(float(by_max), 6), "elementwise": round(float(by_element), 6),
+                                   "identical_frac": round(float((got == want).mean()), 5), "rows": int(len(slots)),
+                                   "bar": 2e-2}
+    del stepper, data, out, plan
+    gc.collect()
+    torch.cuda.empty_cache()
+    return result
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=20)
+    parser.add_argument("--warmup", type=int, default=3)
+    parser.add_argument("--config", default="c2", choices=list(ALL_CONFIGS), help="the workload of the line's top level")
+    parser.add_argument("--only", action="store_true", help="measure the --config workload alone (no `configs` object)")
+    parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--no-parity", action="store_true", help="skip the CPU oracle's sample (profiling runs)")
+    parser.add_argument("--calibrate-copy", action="store_true",
+                        help="only run the plain copy probe (1 GiB read + 1 GiB written, 5 launches): the known traffic "
+                             "that rocprofv3's FETCH_SIZE / WRITE_SIZE are scaled by")
+    parser.add_argument("--bf16-operands", action="store_true",
+                        help="keep MXFP4 banks with groups of hundreds of rows on the bf16 matrix instruction too (the default "
+                             "there: rows split into two e4m3 terms and the scaled instruction, the library's own choice)")
+    parser.add_argument("--graph", choices=["auto", "on", "off"], default="auto",
+                        help="replay the step as one captured HIP graph (auto: for the launch-bound configs c1 and c3)")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the path would shard by expert over "
+                 "an all-to-all each way; that is designed, not built). Run with --gpus 1.")
+
+    import torch
+
+    from dew_amd import ops
+
+    ops.device_check()
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    sustained = sustained_rates(device)
+    if args.calibrate_copy:
+        print(json.dumps({"probe_copy_bytes_read_per_launch": 1 << 30, "probe_copy_bytes_written_per_launch": 1 << 30,
+                          "sustained_copy_gbs": sustained[1], "sustained_bf16_mfma_tflops": sustained[0]}))
+        return
+    top = measure(args.config, args, device, sustained, with_cpu_baseline=not args.no_cpu_baseline)
+    result = {
+        "metric": "grouped-GEMM TFLOP/s & % MFMA peak (prefill); HBM GB/s & % peak (decode)",
+        "value": top["value"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": top["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic", "config": top["config"], "roofline": top["roofline"],
+    }
+    for name in ("cpu_baseline", "sample_parity", "min_topk_margin"):
+        if name in top:
+            result[name] = top[name]
+    if not args.only:
+        per_config = {}
+        for config in ALL_CONFIGS:
+            if config == args.config:
+                measured = {k: v for k, v in top.items() if k != "cpu_baseline"}
+            else:
+                print(f"[bench] measuring {config}", file=sys.stderr, flush=True)
+                measured = measure(config, args, device, sustained, with_cpu_baseline=False)
+            per_config[config] = measured
+        result["configs"] = per_config
     print(json.dumps(result))
 
 
