@@ -24,6 +24,7 @@
 //     dequantizes one 16-deep slice at a time in the shadow of the previous slice's matrix instructions.
 //     A lane's 16 bytes hold a run of consecutive depths, so the depth order inside a 64-deep step is permuted
 //     (the same permutation on the A side: only the LDS chunk a lane reads changes).
+#include <mutex>
 #include <type_traits>
 #include <utility>
 
@@ -77,7 +78,8 @@ struct BankView {
 struct GemmParams {
   const bf16_t* x;
   const int32_t* gather;
-  const int32_t* offsets;
+  const int32_t* offsets;  // [experts + 1] exclusive prefix of the group sizes, or null where `sizes` is given
+  const int32_t* sizes;    // [experts] group sizes as jax.lax.ragged_dot takes them: the prefix is then formed in the tile search
   const int32_t* scatter;
   BankView w0, w1;
   bf16_t* out;
@@ -224,8 +226,8 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   constexpr int kSets = (kFp8A && BN == 256) ? 2 : (kBf16 || (!kFp4 && BM == 128 && kMatrices * BN == 256)) ? 3 : 4;
 
   extern __shared__ u32x4_t lds[];  // a ring of three stages of A: BM rows of 128 bytes each
-  __shared__ int wave_tiles[4];
-  __shared__ int found[3];  // expert, first sorted row of the tile, total m-tiles
+  __shared__ int wave_tiles[4], wave_rows[4];
+  __shared__ int found[5];  // expert, first sorted row of the tile, total m-tiles, the expert's last row + 1, rows in all groups
   // FP8 128 x 128 blocks: the scales of the block's column blocks down the whole depth, read once
   constexpr int kScaleColumns = kBlockBank ? kMatrices * (BN / 128) : 1;
   __shared__ float depth_scales[kScaleColumns][kBlockBank ? kMaxDepthBlocks : 1];
@@ -249,15 +251,32 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   const int m_tile = group * kGroupM + within % group_m;
   const int n0 = (within / group_m) * BN;
 
-  // ---- which expert owns m-tile `m_tile`? inclusive scan of ceil(size / BM) over the experts ----
+  // ---- which expert owns m-tile `m_tile`? inclusive scan of ceil(size / BM) over the experts (and, where the caller
+  // gave group sizes instead of their prefix, of the sizes themselves: an expert's first row) ----
   if (tid == 0) found[0] = -1;
-  int carried = 0;
+  int carried = 0, carried_rows = 0;
   for (int base = 0; base < p.experts; base += kThreads) {
     const int e = base + tid;
-    int start = 0, tiles = 0;
-    if (e < p.experts) {
+    int start = 0, tiles = 0, size = 0;
+    if (e < p.experts) size = kWindow ? p.window_rows : p.sizes ? max(p.sizes[e], 0) : p.offsets[e + 1] - p.offsets[e];
+    if (p.sizes && !kWindow) {  // (uniform) exclusive prefix of the sizes
+      int inclusive_rows = size;
+#pragma unroll
+      for (int offset = 1; offset < 64; offset <<= 1) {
+        const int other = __shfl_up(inclusive_rows, offset, 64);
+        if (lane >= offset) inclusive_rows += other;
+      }
+      __syncthreads();
+      if (lane == 63) wave_rows[wave] = inclusive_rows;
+      __syncthreads();
+      start = carried_rows + inclusive_rows - size;
+      for (int w = 0; w < wave; ++w) start += wave_rows[w];
+      carried_rows += wave_rows[0] + wave_rows[1] + wave_rows[2] + wave_rows[3];
+    } else if (e < p.experts) {
       start = kWindow ? e * p.window_rows : p.offsets[e];
-      const int size = kWindow ? p.window_rows : p.offsets[e + 1] - start;
+    }
+    const int group_end = start + size;
+    if (e < p.experts) {
       if (p.tail_of > 0) {
         const int rest = size % p.tail_of;
         tiles = rest >= 1 && rest <= BM ? 1 : 0;
@@ -281,17 +300,21 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
     if (tiles > 0 && m_tile >= first && m_tile < first + tiles) {
       found[0] = e;
       found[1] = start + (m_tile - first) * BM;
+      found[3] = group_end;
     }
     carried += wave_tiles[0] + wave_tiles[1] + wave_tiles[2] + wave_tiles[3];
   }
-  if (tid == 0) found[2] = carried;
+  if (tid == 0) {
+    found[2] = carried;
+    found[4] = p.sizes ? carried_rows : 0;  // the rows the groups hold (read from the prefix's last entry otherwise)
+  }
   __syncthreads();
   const int expert = found[0];
 
   if (expert < 0) {
     if (kWindow || p.tail_of > 0) return;  // (the taller tiles' launch zeroes them; a kernel gradient has no rows past its groups)
     // Past the last real tile: zero the rows no expert owns (sorted positions offsets[E] .. rows).
-    const int tail_begin = p.offsets[p.experts] + (m_tile - found[2]) * BM;
+    const int tail_begin = (p.sizes ? found[4] : p.offsets[p.experts]) + (m_tile - found[2]) * BM;
     const int tail_end = min(tail_begin + BM, p.rows);
     const int out_width = kGated ? p.width / 2 : p.width, out_n0 = kGated ? n0 / 2 : n0;
     for (int item = tid; item < (tail_end - tail_begin) * (kOutBN / 8); item += kThreads) {
@@ -306,7 +329,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   }
 
   const int row0 = found[1];
-  const int valid_rows = min(BM, (kWindow ? (expert + 1) * p.window_rows : p.offsets[expert + 1]) - row0);
+  const int valid_rows = min(BM, found[3] - row0);
   // a kernel gradient's group contracts its own whole steps of the depth (128 tokens of e4m3 codes, 64 of bf16)
   const int first_step = kWindow ? min(max(p.windows[expert], 0), p.depth) / kStepDepth : 0;
   const int steps = kWindow ? max(min(max(p.windows[expert + 1], 0), p.depth) / kStepDepth - first_step, 0) : p.depth / kStepDepth;
@@ -954,13 +977,12 @@ static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
                              (FORMAT == kFormatMxSplitBlocks || FORMAT == kFormatFp8Rows ? static_cast<size_t>(BM) * block_scale_pitch(kMaxBlockScaleDepth) : 0) +
                              (FORMAT == kFormatMxFp8Rows || FORMAT == kFormatMxFp8Window ? 3 * static_cast<size_t>(BM) * 4 : 0);  // MXFP8 rows: a dword a row a stage
   auto kernel = grouped_gemm_kernel<FORMAT, MODE, BM, BN, WM, WN>;
-  static bool configured = false;  // dynamic LDS above 64 KiB must be opted into once per kernel
-  if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            static_cast<int>(kShared)) != hipSuccess)
-      return fail(DEW_MOE_ELAUNCH, "%s: cannot reserve %zu bytes of LDS", who, kShared);
-    configured = true;
-  }
+  static std::once_flag configured;  // dynamic LDS above 64 KiB must be opted into once per kernel (whichever thread calls first)
+  static hipError_t reserved = hipSuccess;
+  std::call_once(configured, [&] {
+    reserved = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kShared));
+  });
+  if (reserved != hipSuccess) return fail(DEW_MOE_ELAUNCH, "%s: cannot reserve %zu bytes of LDS", who, kShared);
   // every expert may end in a partial tile, and the zeroed tail may add one more
   p.m_tile_bound = p.tail_of > 0 ? p.experts : (p.rows + BM - 1) / BM + p.experts + 1;
   if (FORMAT == kFormatMxFp8Window || FORMAT == kFormatBf16Window) p.m_tile_bound = p.experts * ((p.window_rows + BM - 1) / BM);  // every group the same whole rows
@@ -979,7 +1001,7 @@ static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
 // to 2 times as long as 32-row tiles). Occupancy: a launch of fewer tiles than CUs halves its tile until there are
 // enough (8 experts x 512 rows x 512 columns: 144 tiles of 128 rows take 16.5 us, 272 tiles of 64 rows 11.7 us).
 // 256-row tiles, which fill every accumulator register, are kept to FP4 banks whose groups fill them.
-static int forced_tile_rows = 0;  // dew_moe_tile_rows: 0 leaves the choice to the rules below
+static thread_local int forced_tile_rows = 0;  // dew_moe_tile_rows, per calling thread: 0 leaves the choice to the rules below
 
 static int tile_rows(const GemmParams& p, bool fp4) {
   if (forced_tile_rows != 0) return forced_tile_rows;
@@ -1046,8 +1068,10 @@ static int launch(const char* who, const GemmParams& p, int format, hipStream_t 
 }
 
 static int fill_single(const char* who, GemmParams& p, const void* x, const int32_t* gather, const int32_t* offsets,
-                       const dew_moe_bank* w, const float* bias, const int32_t* scatter, void* out, int32_t rows) {
-  DEW_REQUIRE(x && offsets && out, "%s: x, offsets and out must not be null", who);
+                       const dew_moe_bank* w, const float* bias, const int32_t* scatter, void* out, int32_t rows,
+                       const int32_t* sizes = nullptr) {
+  DEW_REQUIRE(x && (offsets || sizes) && out, "%s: x, the groups' offsets (or sizes) and out must not be null", who);
+  p.sizes = sizes;
   DEW_REQUIRE(aligned16(x) && aligned16(out), "%s: x and out must be 16-byte aligned", who);
   p.x = static_cast<const bf16_t*>(x);
   p.gather = gather;
@@ -1074,17 +1098,27 @@ extern "C" int dew_moe_tile_rows(int32_t rows) {
   return DEW_MOE_OK;
 }
 
-extern "C" int dew_moe_grouped_gemm_bias(const void* x, const int32_t* gather, const int32_t* offsets,
-                                         const dew_moe_bank* w, const float* bias, const int32_t* scatter, void* out,
-                                         int32_t rows, void* stream) {
+static int grouped_gemm_of(const char* who, const void* x, const int32_t* gather, const int32_t* offsets, const int32_t* sizes,
+                           const dew_moe_bank* w, const float* bias, const int32_t* scatter, void* out, int32_t rows, void* stream) {
   using namespace dew;
-  const char* who = "dew_moe_grouped_gemm";
   if (int rc = check_bank(who, w, "weight")) return rc;
   DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
   if (rows == 0) return DEW_MOE_OK;
   GemmParams p{};
-  if (int rc = fill_single(who, p, x, gather, offsets, w, bias, scatter, out, rows)) return rc;
+  if (int rc = fill_single(who, p, x, gather, offsets, w, bias, scatter, out, rows, sizes)) return rc;
   return launch<kPlain>(who, p, w->format, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int dew_moe_grouped_gemm_bias(const void* x, const int32_t* gather, const int32_t* offsets,
+                                         const dew_moe_bank* w, const float* bias, const int32_t* scatter, void* out,
+                                         int32_t rows, void* stream) {
+  return grouped_gemm_of("dew_moe_grouped_gemm", x, gather, offsets, nullptr, w, bias, scatter, out, rows, stream);
+}
+
+extern "C" int dew_moe_grouped_gemm_sizes(const void* x, const int32_t* gather, const int32_t* group_sizes,
+                                          const dew_moe_bank* w, const float* bias, const int32_t* scatter, void* out,
+                                          int32_t rows, void* stream) {
+  return grouped_gemm_of("dew_moe_grouped_gemm_sizes", x, gather, nullptr, group_sizes, w, bias, scatter, out, rows, stream);
 }
 
 extern "C" int dew_moe_grouped_gemm(const void* x, const int32_t* gather, const int32_t* offsets,
@@ -1331,11 +1365,9 @@ extern "C" int dew_moe_gateup_interleaved(const void* x, const int32_t* gather, 
   return launch<kInterleavedGated>(who, p, gate_up->format, static_cast<hipStream_t>(stream));
 }
 
-extern "C" int dew_moe_gateup_swiglu(const void* x, const int32_t* gather, const int32_t* offsets,
-                                     const dew_moe_bank* gate, const dew_moe_bank* up, void* hidden, int32_t rows,
-                                     void* stream) {
+static int gateup_swiglu_of(const char* who, const void* x, const int32_t* gather, const int32_t* offsets, const int32_t* sizes,
+                            const dew_moe_bank* gate, const dew_moe_bank* up, void* hidden, int32_t rows, void* stream) {
   using namespace dew;
-  const char* who = "dew_moe_gateup_swiglu";
   if (int rc = check_bank(who, gate, "gate")) return rc;
   if (int rc = check_bank(who, up, "up")) return rc;
   DEW_REQUIRE(gate->format == up->format && gate->experts == up->experts && gate->depth == up->depth && gate->width == up->width,
@@ -1343,12 +1375,13 @@ extern "C" int dew_moe_gateup_swiglu(const void* x, const int32_t* gather, const
               gate->width, gate->format, up->experts, up->depth, up->width, up->format);
   DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
   if (rows == 0) return DEW_MOE_OK;
-  DEW_REQUIRE(x && offsets && hidden, "%s: x, offsets and hidden must not be null", who);
+  DEW_REQUIRE(x && (offsets || sizes) && hidden, "%s: x, the groups' offsets (or sizes) and hidden must not be null", who);
   DEW_REQUIRE(aligned16(x) && aligned16(hidden), "%s: x and hidden must be 16-byte aligned", who);
   GemmParams p{};
   p.x = static_cast<const bf16_t*>(x);
   p.gather = gather;
   p.offsets = offsets;
+  p.sizes = sizes;
   p.scatter = nullptr;
   p.w0 = BankView{static_cast<const uint8_t*>(gate->codes), gate->scales, gate->tensor_scale};
   p.w1 = BankView{static_cast<const uint8_t*>(up->codes), up->scales, up->tensor_scale};
@@ -1358,4 +1391,16 @@ extern "C" int dew_moe_gateup_swiglu(const void* x, const int32_t* gather, const
   p.width = gate->width;
   p.rows = rows;
   return launch<kSwigluOfTwo>(who, p, gate->format, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int dew_moe_gateup_swiglu(const void* x, const int32_t* gather, const int32_t* offsets,
+                                     const dew_moe_bank* gate, const dew_moe_bank* up, void* hidden, int32_t rows,
+                                     void* stream) {
+  return gateup_swiglu_of("dew_moe_gateup_swiglu", x, gather, offsets, nullptr, gate, up, hidden, rows, stream);
+}
+
+extern "C" int dew_moe_gateup_swiglu_sizes(const void* x, const int32_t* gather, const int32_t* group_sizes,
+                                           const dew_moe_bank* gate, const dew_moe_bank* up, void* hidden, int32_t rows,
+                                           void* stream) {
+  return gateup_swiglu_of("dew_moe_gateup_swiglu_sizes", x, gather, nullptr, group_sizes, gate, up, hidden, rows, stream);
 }

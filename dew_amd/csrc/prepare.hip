@@ -176,17 +176,148 @@ __global__ __launch_bounds__(256) void prepare_nvfp4_scales_kernel(const uint8_t
   }
 }
 
+// FP8 codes held K-major, [E][N][K], as a DeepSeek-style checkpoint stores each expert's `weight [out, in]`
+// (src/dew/interop/codecs.py:670-703): the same 32 n x 32 k atoms, a lane's 16 bytes contiguous in the source.
+__global__ __launch_bounds__(256) void prepare_fp8_kmajor_kernel(const uint8_t* __restrict__ codes, uint8_t* __restrict__ out,
+                                                                 int experts, int depth, int width) {
+  const int k_atoms = depth / 32, n_atoms = width / 32;
+  const long long total = static_cast<long long>(experts) * n_atoms * k_atoms * 64;
+  for (long long item = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; item < total;
+       item += static_cast<long long>(gridDim.x) * blockDim.x) {
+    const int lane = static_cast<int>(item % 64);
+    const long long atom = item / 64;
+    const int ka = static_cast<int>(atom % k_atoms);
+    const int na = static_cast<int>((atom / k_atoms) % n_atoms);
+    const int e = static_cast<int>(atom / (static_cast<long long>(k_atoms) * n_atoms));
+    const size_t column = static_cast<size_t>(e) * width + na * 32 + lane % 32;
+    *reinterpret_cast<uint4*>(out + item * 16) = *reinterpret_cast<const uint4*>(codes + column * depth + ka * 32 + 16 * (lane / 32));
+  }
+}
+
+// The 128 x 128 block scales into the prepared buffer as [E][K / 128][N / 128] fp32, from that layout or, `kmajor`,
+// from a checkpoint's `weight_scale_inv [E][N / 128][K / 128]`.
+__global__ __launch_bounds__(256) void prepare_block_scales_kernel(const float* __restrict__ scales, float* __restrict__ out,
+                                                                   int experts, int depth_blocks, int width_blocks, int kmajor) {
+  const int total = experts * depth_blocks * width_blocks;
+  for (int item = blockIdx.x * blockDim.x + threadIdx.x; item < total; item += gridDim.x * blockDim.x) {
+    const int nb = item % width_blocks, kb = (item / width_blocks) % depth_blocks, e = item / (width_blocks * depth_blocks);
+    out[item] = kmajor ? scales[(static_cast<size_t>(e) * width_blocks + nb) * depth_blocks + kb] : scales[item];
+  }
+}
+
+__global__ void fill_words_kernel(uint32_t* __restrict__ words, int count, uint32_t value) {
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < count; i += gridDim.x * blockDim.x) words[i] = value;
+}
+
+// ---- An MXFP4 checkpoint's own tensors (`*_blocks [E][N][K / 32][16]` bytes, low nibble the even element, and
+// `*_scales [E][N][K / 32]` E8M0 bytes, src/dew/interop/codecs.py:193-224) straight to the prepared FP4 bank, with
+// the arithmetic of the reference's `mxfp4_tensor_powers` / `mxfp4_as_nvfp4` (src/dew/interop/codecs.py:238-284) and
+// no value decoded: an expert's tensor scale is 2^k with k its largest group power (of the groups that hold a nonzero
+// magnitude) less 8, a group's E4M3 block scale 2^(its power - k), twice, and 2^8 for a group of zeros.
+// summary[e] = {largest scale byte + 1 of the groups holding a magnitude (0: none), least such byte}; flags[1] is
+// set by a 0xff scale byte.
+struct Mxfp4Survey {
+  uint32_t top_plus_one, bottom;
+};
+
+__device__ __forceinline__ bool holds_magnitude(const uint4& block) {
+  return ((block.x | block.y | block.z | block.w) & 0x77777777u) != 0u;
+}
+
+__global__ void mxfp4_survey_start_kernel(Mxfp4Survey* __restrict__ summary, int experts) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e < experts) summary[e] = Mxfp4Survey{0u, 0xFFFFFFFFu};
+}
+
+__global__ __launch_bounds__(256) void mxfp4_survey_kernel(const uint4* __restrict__ blocks, const uint8_t* __restrict__ scales,
+                                                           Mxfp4Survey* __restrict__ summary, uint32_t* __restrict__ flags,
+                                                           int experts, long long per_expert) {
+  // per_expert (= N * K / 32) is a multiple of 64: a wavefront's 64 groups belong to one expert
+  const long long total = static_cast<long long>(experts) * per_expert;
+  for (long long base = (static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x) & ~63ll; base < total;
+       base += static_cast<long long>(gridDim.x) * blockDim.x) {
+    const long long item = base + threadIdx.x % 64;
+    const uint32_t byte = scales[item];
+    const bool held = holds_magnitude(blocks[item]);
+    uint32_t top = held ? byte + 1u : 0u, bottom = held ? byte : 0xFFFFFFFFu, nan = byte == 255u ? 1u : 0u;
+#pragma unroll
+    for (int offset = 32; offset >= 1; offset >>= 1) {
+      top = max(top, static_cast<uint32_t>(__shfl_xor(static_cast<int>(top), offset, 64)));
+      bottom = min(bottom, static_cast<uint32_t>(__shfl_xor(static_cast<int>(bottom), offset, 64)));
+      nan |= static_cast<uint32_t>(__shfl_xor(static_cast<int>(nan), offset, 64));
+    }
+    if (threadIdx.x % 64 == 0) {
+      const int e = static_cast<int>(base / per_expert);
+      if (top != 0u) {
+        atomicMax(&summary[e].top_plus_one, top);
+        atomicMin(&summary[e].bottom, bottom);
+      }
+      if (nan) atomicOr(flags + 1, 1u);
+    }
+  }
+}
+
+// One thread an expert: its power k and tensor scale 2^k; flags[1] set where the bank cannot be one NVFP4 bank (its
+// group powers spread past E4M3's 17 binades, or 2^k leaves fp32's normal range). summary[e].bottom then holds k.
+__global__ void mxfp4_powers_kernel(Mxfp4Survey* __restrict__ summary, float* __restrict__ tensor_scale, uint32_t* __restrict__ flags,
+                                    int experts) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= experts) return;
+  const bool any = summary[e].top_plus_one != 0u;
+  const int top = any ? static_cast<int>(summary[e].top_plus_one) - 1 - 127 : 8;
+  const int bottom = any ? static_cast<int>(summary[e].bottom) - 127 : 8;
+  const int power = top - 8;
+  if (top - bottom > 17 || power < -126 || power > 127) atomicOr(flags + 1, 1u);
+  tensor_scale[e] = __uint_as_float(static_cast<uint32_t>(min(max(power, -126), 127) + 127) << 23);
+  summary[e].bottom = static_cast<uint32_t>(power);
+}
+
+// One thread per (expert, column, 32-deep group): its 16 bytes are a lane's piece of an FP4 atom as they are, and its
+// scale the lane's two equal E4M3 bytes. flags[0] is set by a block scale below E4M3's normal range (2^-7 .. 2^-9),
+// which the scaled conversions cannot take as an exponent: the bank is then multiplied as a general NVFP4 bank.
+__global__ __launch_bounds__(256) void prepare_mxfp4_blocks_kernel(const uint4* __restrict__ blocks, const uint8_t* __restrict__ scales,
+                                                                   const Mxfp4Survey* __restrict__ summary, uint8_t* __restrict__ codes_out,
+                                                                   uint16_t* __restrict__ scales_out, uint32_t* __restrict__ flags,
+                                                                   int experts, int depth, int width) {
+  const int groups = depth / 32, n_atoms = width / 32, k_atoms = depth / 64;
+  const long long total = static_cast<long long>(experts) * width * groups;
+  for (long long item = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; item < total;
+       item += static_cast<long long>(gridDim.x) * blockDim.x) {
+    // consecutive threads take consecutive columns of one group, so their 16-byte writes fill an atom's lanes in order
+    const int n = static_cast<int>(item % width);
+    const int group = static_cast<int>((item / width) % groups);
+    const int e = static_cast<int>(item / (static_cast<long long>(width) * groups));
+    const size_t source = (static_cast<size_t>(e) * width + n) * groups + group;
+    const uint4 block = blocks[source];
+    const int local = holds_magnitude(block) ? static_cast<int>(scales[source]) - 127 - static_cast<int>(summary[e].bottom) : 8;
+    const int clamped = min(max(local, -9), 8);
+    const uint32_t e4m3 = clamped >= -6 ? static_cast<uint32_t>(clamped + 7) << 3 : 1u << (clamped + 9);
+    if (clamped < -6) atomicOr(flags, 1u);
+    const size_t atom = (static_cast<size_t>(e) * n_atoms + n / 32) * k_atoms + group / 2;
+    const int lane = 32 * (group % 2) + n % 32;
+    *reinterpret_cast<uint4*>(codes_out + atom * kAtomBytes + lane * 16) = block;
+    scales_out[atom * 64 + lane] = static_cast<uint16_t>(e4m3 | (e4m3 << 8));
+  }
+}
+
 static size_t codes_bytes(int format, int experts, int depth, int width) {
   const size_t elements = static_cast<size_t>(experts) * depth * width;
-  return format == DEW_MOE_W_NVFP4 ? elements / 2 : format == DEW_MOE_W_BF16 ? elements * 2 : elements;
+  return (format == DEW_MOE_W_NVFP4 || format == DEW_MOE_W_MXFP4_BLOCKS) ? elements / 2 : format == DEW_MOE_W_BF16 ? elements * 2 : elements;
 }
+
+// Behind an FP4 bank's codes and scales: 256 bytes of flag words, then (a checkpoint's MXFP4 tensors) the experts'
+// tensor scales and the survey's two words an expert.
+static size_t fp4_scales_bytes(int experts, int depth, int width) { return static_cast<size_t>(experts) * width * (depth / 16); }
 
 }  // namespace dew
 
 extern "C" size_t dew_moe_prepared_bytes(int32_t format, int32_t experts, int32_t depth, int32_t width) {
   if (experts <= 0 || depth <= 0 || width <= 0) return 0;
   size_t bytes = dew::codes_bytes(format, experts, depth, width);
-  if (format == DEW_MOE_W_NVFP4) bytes += static_cast<size_t>(experts) * width * (depth / 16) + 256;  // + a flag word
+  if (format == DEW_MOE_W_NVFP4) bytes += dew::fp4_scales_bytes(experts, depth, width) + 256;  // + a flag word
+  if (format == DEW_MOE_W_MXFP4_BLOCKS)  // + flag words, tensor scales, the survey
+    bytes += dew::fp4_scales_bytes(experts, depth, width) + 256 + (static_cast<size_t>(experts) * 12 + 255) / 256 * 256;
+  if (format == DEW_MOE_W_FP8_BLOCK) bytes += static_cast<size_t>(experts) * (depth / 128) * (width / 128) * sizeof(float);  // its block scales
   if (format == DEW_MOE_W_MXFP8) bytes += static_cast<size_t>(experts) * width * (depth / 32);
   return bytes;
 }
@@ -194,10 +325,12 @@ extern "C" size_t dew_moe_prepared_bytes(int32_t format, int32_t experts, int32_
 extern "C" int dew_moe_prepare_bank(const dew_moe_bank* ref, void* prepared, dew_moe_bank* out, void* stream) {
   using namespace dew;
   DEW_REQUIRE(ref && prepared && out, "dew_moe_prepare_bank: bank, prepared buffer and out must not be null");
-  DEW_REQUIRE(ref->layout == DEW_MOE_LAYOUT_REFERENCE || (ref->layout == DEW_MOE_LAYOUT_REFERENCE_KMAJOR && ref->format == DEW_MOE_W_BF16),
-              "dew_moe_prepare_bank: the bank is already prepared (layout %d)", ref->layout);
+  DEW_REQUIRE(ref->layout == DEW_MOE_LAYOUT_REFERENCE ||
+                  (ref->layout == DEW_MOE_LAYOUT_REFERENCE_KMAJOR && (ref->format == DEW_MOE_W_BF16 || ref->format == DEW_MOE_W_FP8_BLOCK)),
+              "dew_moe_prepare_bank: the bank is already prepared, or K-major in a format held one way only (layout %d, format %d)",
+              ref->layout, ref->format);
   DEW_REQUIRE(ref->format == DEW_MOE_W_FP8_BLOCK || ref->format == DEW_MOE_W_FP8_CHANNEL || ref->format == DEW_MOE_W_NVFP4 ||
-                  ref->format == DEW_MOE_W_MXFP8 || ref->format == DEW_MOE_W_BF16,
+                  ref->format == DEW_MOE_W_MXFP8 || ref->format == DEW_MOE_W_BF16 || ref->format == DEW_MOE_W_MXFP4_BLOCKS,
               "dew_moe_prepare_bank: unknown weight format %d", ref->format);
   DEW_REQUIRE(ref->experts >= 1 && ref->depth >= 1 && ref->width >= 1, "dew_moe_prepare_bank: bank [%d, %d, %d]",
               ref->experts, ref->depth, ref->width);
@@ -219,7 +352,8 @@ extern "C" int dew_moe_prepare_bank(const dew_moe_bank* ref, void* prepared, dew
                        codes_out, ref->experts, ref->depth, ref->width);
     if (int rc = launched("prepare_nvfp4_codes_kernel")) return rc;
     uint32_t* general = reinterpret_cast<uint32_t*>(scales_out + static_cast<size_t>(ref->experts) * ref->width * (ref->depth / 16));
-    if (hipMemsetAsync(general, 0, sizeof(uint32_t), s) != hipSuccess) return fail(DEW_MOE_ELAUNCH, "dew_moe_prepare_bank: memset failed");
+    hipLaunchKernelGGL(fill_words_kernel, dim3(1), dim3(64), 0, s, general, 1, 0u);  // (a kernel, not a memset node: a caller may capture this)
+    if (int rc = launched("fill_words_kernel")) return rc;
     hipLaunchKernelGGL(prepare_nvfp4_scales_kernel, dim3(grid), dim3(256), 0, s, static_cast<const uint8_t*>(ref->scales),
                        reinterpret_cast<uint16_t*>(scales_out), ref->experts, ref->depth, ref->width, general);
     if (int rc = launched("prepare_nvfp4_scales_kernel")) return rc;
@@ -228,6 +362,34 @@ extern "C" int dew_moe_prepare_bank(const dew_moe_bank* ref, void* prepared, dew
     if (hipMemcpyAsync(&found, general, sizeof(found), hipMemcpyDeviceToHost, s) != hipSuccess || hipStreamSynchronize(s) != hipSuccess)
       return fail(DEW_MOE_ELAUNCH, "dew_moe_prepare_bank: reading the scale summary back failed: %s", hipGetErrorString(hipGetLastError()));
     if (!found) out->format = DEW_MOE_W_MXFP4;
+  } else if (ref->format == DEW_MOE_W_MXFP4_BLOCKS) {
+    DEW_REQUIRE(ref->depth % 256 == 0, "dew_moe_prepare_bank: an FP4 bank's depth is whole 256s, not %d", ref->depth);
+    DEW_REQUIRE(aligned16(ref->codes), "dew_moe_prepare_bank: blocks must be 16-byte aligned");
+    uint8_t* codes_out = static_cast<uint8_t*>(prepared);
+    uint8_t* scales_out = codes_out + codes_bytes(ref->format, ref->experts, ref->depth, ref->width);
+    uint32_t* flags = reinterpret_cast<uint32_t*>(scales_out + fp4_scales_bytes(ref->experts, ref->depth, ref->width));
+    float* tensor_scale = reinterpret_cast<float*>(flags + 64);
+    Mxfp4Survey* summary = reinterpret_cast<Mxfp4Survey*>(tensor_scale + ref->experts);
+    const uint4* blocks = static_cast<const uint4*>(ref->codes);
+    const uint8_t* bytes = static_cast<const uint8_t*>(ref->scales);
+    const long long per_expert = static_cast<long long>(ref->width) * (ref->depth / 32);
+    hipLaunchKernelGGL(fill_words_kernel, dim3(1), dim3(64), 0, s, flags, 2, 0u);
+    if (int rc = launched("fill_words_kernel")) return rc;
+    hipLaunchKernelGGL(mxfp4_survey_start_kernel, dim3((ref->experts + 255) / 256), dim3(256), 0, s, summary, ref->experts);
+    hipLaunchKernelGGL(mxfp4_survey_kernel, dim3(grid), dim3(256), 0, s, blocks, bytes, summary, flags, ref->experts, per_expert);
+    if (int rc = launched("mxfp4_survey_kernel")) return rc;
+    hipLaunchKernelGGL(mxfp4_powers_kernel, dim3((ref->experts + 255) / 256), dim3(256), 0, s, summary, tensor_scale, flags, ref->experts);
+    hipLaunchKernelGGL(prepare_mxfp4_blocks_kernel, dim3(grid), dim3(256), 0, s, blocks, bytes, summary, codes_out,
+                       reinterpret_cast<uint16_t*>(scales_out), flags, ref->experts, ref->depth, ref->width);
+    if (int rc = launched("prepare_mxfp4_blocks_kernel")) return rc;
+    uint32_t found[2] = {1, 1};
+    if (hipMemcpyAsync(found, flags, sizeof(found), hipMemcpyDeviceToHost, s) != hipSuccess || hipStreamSynchronize(s) != hipSuccess)
+      return fail(DEW_MOE_ELAUNCH, "dew_moe_prepare_bank: reading the scale summary back failed: %s", hipGetErrorString(hipGetLastError()));
+    DEW_REQUIRE(!found[1], "dew_moe_prepare_bank: this MXFP4 bank is no one NVFP4 bank (an expert's group powers spread past 17 binades, "
+                           "a tensor scale leaves float32's normal range, or a scale byte is 0xff): it stays dense");
+    out->format = found[0] ? DEW_MOE_W_NVFP4 : DEW_MOE_W_MXFP4;
+    out->scales = scales_out;
+    out->tensor_scale = tensor_scale;
   } else if (ref->format == DEW_MOE_W_BF16) {
     DEW_REQUIRE(ref->depth % 128 == 0, "dew_moe_prepare_bank: a bf16 bank's depth is whole 128s, not %d", ref->depth);
     if (ref->layout == DEW_MOE_LAYOUT_REFERENCE_KMAJOR) {
@@ -252,9 +414,23 @@ extern "C" int dew_moe_prepare_bank(const dew_moe_bank* ref, void* prepared, dew
     out->scales = scales_out;
   } else {
     DEW_REQUIRE(ref->depth % 128 == 0, "dew_moe_prepare_bank: an FP8 bank's depth is whole 128s, not %d", ref->depth);
-    hipLaunchKernelGGL(prepare_fp8_kernel, dim3(grid), dim3(256), 0, s, static_cast<const uint8_t*>(ref->codes),
-                       static_cast<uint8_t*>(prepared), ref->experts, ref->depth, ref->width);
+    const bool kmajor = ref->layout == DEW_MOE_LAYOUT_REFERENCE_KMAJOR;
+    if (kmajor) {
+      DEW_REQUIRE(aligned16(ref->codes), "dew_moe_prepare_bank: K-major FP8 codes must be 16-byte aligned");
+      hipLaunchKernelGGL(prepare_fp8_kmajor_kernel, dim3(grid), dim3(256), 0, s, static_cast<const uint8_t*>(ref->codes),
+                         static_cast<uint8_t*>(prepared), ref->experts, ref->depth, ref->width);
+    } else {
+      hipLaunchKernelGGL(prepare_fp8_kernel, dim3(grid), dim3(256), 0, s, static_cast<const uint8_t*>(ref->codes),
+                         static_cast<uint8_t*>(prepared), ref->experts, ref->depth, ref->width);
+    }
     if (int rc = launched("prepare_fp8_kernel")) return rc;
+    if (ref->format == DEW_MOE_W_FP8_BLOCK) {  // the block scales travel with the codes, in the order the products read
+      float* scales_out = reinterpret_cast<float*>(static_cast<uint8_t*>(prepared) + codes_bytes(ref->format, ref->experts, ref->depth, ref->width));
+      hipLaunchKernelGGL(prepare_block_scales_kernel, dim3(64), dim3(256), 0, s, static_cast<const float*>(ref->scales), scales_out,
+                         ref->experts, ref->depth / 128, ref->width / 128, kmajor ? 1 : 0);
+      if (int rc = launched("prepare_block_scales_kernel")) return rc;
+      out->scales = scales_out;
+    }
   }
   return DEW_MOE_OK;
 }

@@ -151,6 +151,10 @@ class Fp8Blocks:
 
     codes: torch.Tensor
     scale_inv: torch.Tensor
+    kmajor: bool = False
+    """The tensors as such a checkpoint stores them, stacked by expert: `codes [E, N, K]` (each expert's `weight [out,
+    in]`) and `scale_inv [E, N/128, K/128]`; the bank still stands for `W [E, K, N]`, and its re-layout for the matrix
+    cores reads them where they lie."""
 
     @classmethod
     def quantized(cls, weight: torch.Tensor) -> "Fp8Blocks":
@@ -160,14 +164,44 @@ class Fp8Blocks:
 
     @property
     def shape(self):
-        return tuple(self.codes.shape)
+        experts, first, second = self.codes.shape
+        return (experts, second, first) if self.kmajor else (experts, first, second)
 
     @property
     def dtype(self):
         return torch.bfloat16
 
     def to(self, device) -> "Fp8Blocks":
-        return Fp8Blocks(self.codes.to(device), self.scale_inv.to(device))
+        return Fp8Blocks(self.codes.to(device), self.scale_inv.to(device), self.kmajor)
+
+
+@dataclasses.dataclass(frozen=True)
+class Mxfp4Blocks:
+    """An MXFP4 checkpoint's expert bank as the checkpoint stores it (gpt-oss's `*_blocks` / `*_scales`,
+    src/dew/interop/codecs.py:193-224): `blocks [E, N, K/32, 16]` uint8, two E2M1 codes a byte (low nibble the even
+    element), and `scales [E, N, K/32]` E8M0 bytes; standing for `W [E, K, N]`. The reference turns such a bank into
+    its `NvFp4` on the host (`mxfp4_as_nvfp4`, src/dew/interop/codecs.py:265-284); here the device re-layout takes
+    these bytes straight to the same prepared bank (`DEW_MOE_W_MXFP4_BLOCKS`)."""
+
+    blocks: torch.Tensor
+    scales: torch.Tensor
+
+    def __post_init__(self):
+        if self.blocks.ndim != 4 or self.blocks.shape[-1] != 16 or tuple(self.scales.shape) != tuple(self.blocks.shape[:3]):
+            raise ValueError(f"an MXFP4 bank is blocks [E, N, K/32, 16] with scales [E, N, K/32], got {tuple(self.blocks.shape)} "
+                             f"and {tuple(self.scales.shape)}")
+
+    @property
+    def shape(self):
+        experts, width, groups, _ = self.blocks.shape
+        return (experts, 32 * groups, width)
+
+    @property
+    def dtype(self):
+        return torch.bfloat16
+
+    def to(self, device) -> "Mxfp4Blocks":
+        return Mxfp4Blocks(self.blocks.to(device), self.scales.to(device))
 
 
 @dataclasses.dataclass(frozen=True)

@@ -36,6 +36,14 @@ class GroupSizes:
         sizes = group_sizes.to(torch.int32).contiguous()
         return cls(sizes, ops.group_offsets(sizes))
 
+    @staticmethod
+    def operands(group_sizes) -> dict:
+        """The groups as a product's keywords: the prefix where the caller holds it (`GroupSizes`), else the plain
+        `group_sizes [E]` as the reference's FFI takes them, the prefix then formed inside the launch."""
+        if isinstance(group_sizes, GroupSizes):
+            return dict(offsets=group_sizes.offsets)
+        return dict(offsets=None, sizes=group_sizes.to(torch.int32).contiguous())
+
 
 @dataclasses.dataclass(frozen=True)
 class GroupedCase:
@@ -50,7 +58,7 @@ class GroupedCase:
     epilogue_operands: tuple = ()
 
 
-_BANKS = (formats.NvFp4, formats.Fp8Blocks, formats.Fp8Channels, formats.Bf16, formats.Layered, ops.PreparedBank)
+_BANKS = (formats.NvFp4, formats.Fp8Blocks, formats.Fp8Channels, formats.Bf16, formats.Mxfp4Blocks, formats.Layered, ops.PreparedBank)
 # (formats.MxFp8 multiplies MXFP8 rows only: projections.mxfp8_product)
 
 
@@ -144,23 +152,24 @@ def gemm(lhs: torch.Tensor, rhs, group_sizes, *, paired=None, gather: torch.Tens
     case = GroupedCase(lhs, rhs, paired, epilogue, out_dtype, compute, tuple(epilogue_operands))
     named = None if implementation in (None, "auto") else implementation
     selection.select(GROUPED, case, named)
-    groups = GroupSizes.of(group_sizes)
     first = prepared(rhs)
     if epilogue == "gpt_oss_gated":
         if scatter is not None:
             raise selection.KernelRefused(GROUPED_MATMUL, "hip", selection.Refusal("gated-scatter", "the gated product writes sorted rows"), iter(()))
-        return ops.gateup_interleaved(lhs, first, groups.offsets, bias=epilogue_operands[0], limit=float(epilogue_operands[1]),
-                                      gather=gather)
+        return ops.gateup_interleaved(lhs, first, GroupSizes.of(group_sizes).offsets, bias=epilogue_operands[0],
+                                      limit=float(epilogue_operands[1]), gather=gather)
+    groups = GroupSizes.operands(group_sizes)    # no prefix launch where the caller holds sizes only
+    offsets = groups.pop("offsets")
     if paired is None:
         bias = epilogue_operands[0] if epilogue == "plus_bias" else None
-        return ops.grouped_gemm(lhs, first, groups.offsets, gather=gather, scatter=scatter, bias=bias)
+        return ops.grouped_gemm(lhs, first, offsets, gather=gather, scatter=scatter, bias=bias, **groups)
     second = prepared(paired)
     if scatter is not None:
         raise selection.KernelRefused(GROUPED_MATMUL, "hip", selection.Refusal("pair-scatter", "a paired product writes sorted rows"), iter(()))
     if epilogue == "swiglu":
-        return ops.gateup_swiglu(lhs, first, second, groups.offsets, gather=gather)
-    return (ops.grouped_gemm(lhs, first, groups.offsets, gather=gather),
-            ops.grouped_gemm(lhs, second, groups.offsets, gather=gather))
+        return ops.gateup_swiglu(lhs, first, second, offsets, gather=gather, **groups)
+    return (ops.grouped_gemm(lhs, first, offsets, gather=gather, **groups),
+            ops.grouped_gemm(lhs, second, offsets, gather=gather, **groups))
 
 
 def gemm_t(lhs: torch.Tensor, rhs: torch.Tensor, group_sizes, *, out_dtype=torch.bfloat16, whole_steps: bool = False) -> torch.Tensor:

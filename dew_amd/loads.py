@@ -35,11 +35,16 @@ def source_quantization(config: Mapping) -> str | None:
     return found.get("quant_method")
 
 
-def packed_banks(tensors: Mapping[str, torch.Tensor], config: Mapping) -> tuple[dict, dict]:
+def packed_banks(tensors: Mapping[str, torch.Tensor], config: Mapping, *, device_codec: bool | None = None) -> tuple[dict, dict]:
     """`tensors` with each MXFP4 expert bank taken out of the source's decoding, and those banks by their source
-    names (`formats.NvFp4`, exactly the MXFP4 values: `codecs.mxfp4_as_nvfp4`); in each one's place an `Unread`
-    of its decoded shape. A bank whose depth is no whole NVFP4 stages, whose experts' group powers span past one
-    tensor scale's reach, or that holds no experts stays as the source states it and is named in the log."""
+    names; in each one's place an `Unread` of its decoded shape. A bank whose depth is no whole NVFP4 stages, whose
+    experts' group powers span past one tensor scale's reach, or that holds no experts stays as the source states it
+    and is named in the log.
+
+    A bank is the reference's `formats.NvFp4` (exactly the MXFP4 values: `codecs.mxfp4_as_nvfp4` then `NvFp4.of`, torch
+    index and bit operations wherever the tensors live), or, with `device_codec` (the default for tensors on the GPU),
+    `formats.Mxfp4Blocks`: the checkpoint's own two tensors, which the device re-layout takes straight to the same
+    prepared bank (`dew_moe_prepare_bank` on `DEW_MOE_W_MXFP4_BLOCKS`) with no NvFp4 words formed in between."""
     if source_quantization(config) != "mxfp4":
         raise ValueError("packed_experts serves an MXFP4 source's expert banks (gpt-oss's quant_method mxfp4); "
                          f"this source's quantization is {config.get('quantization_config')!r}")
@@ -48,35 +53,58 @@ def packed_banks(tensors: Mapping[str, torch.Tensor], config: Mapping) -> tuple[
                    if name.endswith(MXFP4_SUFFIXES[0]) and name[:-len(MXFP4_SUFFIXES[0])] + MXFP4_SUFFIXES[1] in tensors)
     for name in names:
         blocks, scales = (tensors[name + suffix] for suffix in MXFP4_SUFFIXES)
+        on_device = blocks.is_cuda if device_codec is None else device_codec
         powers = None
         if blocks.ndim != 4:
             reason = "it holds no experts"
         elif blocks.shape[2] * codecs.GROUP % formats.NVFP4_STAGE:
             reason = f"its depth {blocks.shape[2] * codecs.GROUP} is no whole {formats.NVFP4_STAGE}-deep stages"
+        elif on_device:
+            # the device re-layout itself finds an expert whose group powers spread too far, and refuses the bank by name
+            from . import gemm, ops
+
+            bank = formats.Mxfp4Blocks(blocks.view(torch.uint8).contiguous(), scales.view(torch.uint8).contiguous())
+            try:
+                gemm.prepared(bank)
+                powers = True
+            except ops.KernelError as refusal:
+                reason = str(refusal)
         else:
             powers = codecs.mxfp4_tensor_powers(blocks, scales)
             reason = "its experts' group powers span past one tensor scale's reach"
+            bank = None if powers is None else formats.NvFp4.of(*codecs.mxfp4_as_nvfp4(blocks, scales, powers))
         if powers is None:
             _log.warning("packed_experts: %s stays dense: %s", name, reason)
             continue
         experts, outputs, groups, _ = blocks.shape
-        banks[name] = formats.NvFp4.of(*codecs.mxfp4_as_nvfp4(blocks, scales, powers))
+        banks[name] = bank
         for suffix in MXFP4_SUFFIXES:
             del tensors[name + suffix]
         tensors[name] = Unread((experts, groups * codecs.GROUP, outputs), torch.float32)
     return tensors, banks
 
 
-def fp8_block_bank(weights, scale_invs) -> formats.Fp8Blocks:
+def fp8_block_bank(weights, scale_invs, *, device_codec: bool | None = None) -> formats.Fp8Blocks:
     """One projection's experts, each stored `[out, in]` e4m3 with `[out/128, in/128]` fp32 inverse scales
-    (DeepSeek-V3 / Qwen3-FP8 checkpoints), as the `[E, in, out]` bank the kernels multiply, still quantized."""
-    codes = torch.stack([weight.view(torch.uint8).transpose(0, 1) for weight in weights]).contiguous()
-    scales = torch.stack([scale.to(torch.float32).transpose(0, 1) for scale in scale_invs]).contiguous()
-    experts, depth, width = codes.shape
-    if depth % 128 or width % 128 or tuple(scales.shape) != (experts, depth // 128, width // 128):
+    (DeepSeek-V3 / Qwen3-FP8 checkpoints), as the bank the kernels multiply, still quantized: `[E, in, out]` codes
+    transposed here, or, with `device_codec` (the default for tensors on the GPU), the tensors stacked as they are
+    (`Fp8Blocks(kmajor=True)`), which the device re-layout reads where they lie."""
+    weights, scale_invs = list(weights), list(scale_invs)
+    on_device = weights[0].is_cuda if device_codec is None else device_codec
+    if on_device:
+        codes = torch.stack([weight.view(torch.uint8) for weight in weights]).contiguous()
+        scales = torch.stack([scale.to(torch.float32) for scale in scale_invs]).contiguous()
+        experts, width, depth = codes.shape
+        expected = (experts, width // 128, depth // 128)
+    else:
+        codes = torch.stack([weight.view(torch.uint8).transpose(0, 1) for weight in weights]).contiguous()
+        scales = torch.stack([scale.to(torch.float32).transpose(0, 1) for scale in scale_invs]).contiguous()
+        experts, depth, width = codes.shape
+        expected = (experts, depth // 128, width // 128)
+    if depth % 128 or width % 128 or tuple(scales.shape) != expected:
         raise ValueError(f"an FP8 block bank is [E, in, out] in whole 128s with [E, in/128, out/128] scales, got codes "
                          f"{tuple(codes.shape)} and scales {tuple(scales.shape)}")
-    return formats.Fp8Blocks(codes, scales)
+    return formats.Fp8Blocks(codes, scales, kmajor=on_device)
 
 
 def fp8_expert_banks(tensors: Mapping[str, torch.Tensor], prefix: str, experts: int,

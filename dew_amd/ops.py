@@ -207,8 +207,9 @@ class PreparedBank:
 
 
 def prepare(bank) -> PreparedBank:
-    """The one-time re-layout of a `formats.NvFp4`, `formats.Fp8Blocks`, `formats.Fp8Channels`, `formats.MxFp8` or
-    `formats.Bf16` bank."""
+    """The one-time re-layout of a `formats.NvFp4`, `formats.Fp8Blocks` (either way round), `formats.Fp8Channels`,
+    `formats.MxFp8`, `formats.Bf16` or `formats.Mxfp4Blocks` bank. An MXFP4 checkpoint's bank that is no one NVFP4
+    bank (the reference keeps it dense) raises `KernelError`."""
     if isinstance(bank, PreparedBank):
         return bank
     if isinstance(bank, formats.NvFp4):
@@ -219,6 +220,12 @@ def prepare(bank) -> PreparedBank:
     elif isinstance(bank, formats.Fp8Blocks):
         fmt, codes, scales, tensor = _lib.W_FP8_BLOCK, bank.codes, bank.scale_inv, None
         _device(codes, "Fp8Blocks.codes", torch.uint8), _device(scales, "Fp8Blocks.scale_inv", torch.float32)
+        blocks = (bank.shape[2] // 128, bank.shape[1] // 128) if bank.kmajor else (bank.shape[1] // 128, bank.shape[2] // 128)
+        if tuple(scales.shape) != (bank.shape[0], *blocks):
+            raise KernelError(f"Fp8Blocks.scale_inv is {tuple(scales.shape)}, the bank's blocks {(bank.shape[0], *blocks)}")
+    elif isinstance(bank, formats.Mxfp4Blocks):
+        fmt, codes, scales, tensor = _lib.W_MXFP4_BLOCKS, bank.blocks, bank.scales, None
+        _device(codes, "Mxfp4Blocks.blocks", torch.uint8), _device(scales, "Mxfp4Blocks.scales", torch.uint8)
     elif isinstance(bank, formats.Fp8Channels):
         fmt, codes, scales, tensor = _lib.W_FP8_CHANNEL, bank.codes, bank.scales, None
         _device(codes, "Fp8Channels.codes", torch.uint8), _device(scales, "Fp8Channels.scales", torch.float32)
@@ -232,11 +239,15 @@ def prepare(bank) -> PreparedBank:
         raise KernelError(f"no HIP kernel multiplies a {type(bank).__name__} bank")
     experts, depth, width = bank.shape
     lib = _lib.library()
-    layout = _lib.LAYOUT_REFERENCE_KMAJOR if isinstance(bank, formats.Bf16) and bank.transposed else _lib.LAYOUT_REFERENCE
+    kmajor = (isinstance(bank, formats.Bf16) and bank.transposed) or (isinstance(bank, formats.Fp8Blocks) and bank.kmajor)
+    layout = _lib.LAYOUT_REFERENCE_KMAJOR if kmajor else _lib.LAYOUT_REFERENCE
     reference = _lib.Bank(fmt, layout, experts, depth, width, _ptr(codes), _ptr(scales), _ptr(tensor))
     buffer = torch.empty(lib.dew_moe_prepared_bytes(fmt, experts, depth, width), dtype=torch.uint8, device=codes.device)
     out = _lib.Bank()
     _lib.check(lib.dew_moe_prepare_bank(reference, _ptr(buffer), out, _stream()), "dew_moe_prepare_bank")
+    if isinstance(bank, formats.Mxfp4Blocks):  # its tensor scales were written into the prepared buffer
+        at = out.tensor_scale - buffer.data_ptr()
+        tensor = buffer[at:at + 4 * experts].view(torch.float32)
     return PreparedBank(out, (experts, depth, width), (buffer, scales, tensor))
 
 
@@ -253,15 +264,22 @@ def _expert_bias(bias: torch.Tensor | None, experts: int, width: int) -> torch.T
     return bias
 
 
-def _product_rows(operand: torch.Tensor, name: str, offsets: torch.Tensor, experts: int, gather, scatter, rows) -> int:
+def _product_rows(operand: torch.Tensor, name: str, offsets: torch.Tensor, experts: int, gather, scatter, rows, sizes=None) -> int:
     """What every grouped product's launch trusts and only the host can see, checked before any pointer leaves: the
     row operand on the device and contiguous, `offsets` int32 `[E + 1]` on the device, `gather` / `scatter` int32,
     contiguous, on the device and covering every row, and no more rows asked than the operand (without a gather)
     holds. Returns the rows of the launch."""
     _device(operand, name)
-    _device(offsets, "offsets", torch.int32)
-    if offsets.numel() != experts + 1:
-        raise KernelError(f"offsets has {offsets.numel()} entries, the bank {experts} experts")
+    if offsets is None and sizes is not None:   # the groups as `group_sizes [E]`: the launch forms the prefix itself
+        _device(sizes, "group_sizes", torch.int32)
+        if sizes.numel() != experts:
+            raise KernelError(f"group_sizes has {sizes.numel()} entries, the bank {experts} experts")
+    else:
+        if offsets is None:
+            raise KernelError("a grouped product takes the groups' offsets [E + 1] or their sizes [E]")
+        _device(offsets, "offsets", torch.int32)
+        if offsets.numel() != experts + 1:
+            raise KernelError(f"offsets has {offsets.numel()} entries, the bank {experts} experts")
     for label, index in (("gather", gather), ("scatter", scatter)):
         if index is not None:
             _device(index, label, torch.int32)
@@ -275,17 +293,22 @@ def _product_rows(operand: torch.Tensor, name: str, offsets: torch.Tensor, exper
     return rows
 
 
-def grouped_gemm(x: torch.Tensor, bank: PreparedBank, offsets: torch.Tensor, *, gather: torch.Tensor | None = None,
+def grouped_gemm(x: torch.Tensor, bank: PreparedBank, offsets: torch.Tensor | None, *, gather: torch.Tensor | None = None,
                  scatter: torch.Tensor | None = None, rows: int | None = None,
-                 bias: torch.Tensor | None = None) -> torch.Tensor:
-    """`out[scatter[i]] = x[gather[i]] @ W[expert of sorted position i] (+ bias[expert])`, bf16 `[rows, N]`."""
+                 bias: torch.Tensor | None = None, sizes: torch.Tensor | None = None) -> torch.Tensor:
+    """`out[scatter[i]] = x[gather[i]] @ W[expert of sorted position i] (+ bias[expert])`, bf16 `[rows, N]`. The groups
+    are `offsets [E + 1]`, or, where that is None, `sizes [E]` (the launch then forms the prefix on the device)."""
     _device(x, "x", torch.bfloat16)
     experts, depth, width = bank.shape
     if x.shape[-1] != depth:
         raise KernelError(f"x rows are {x.shape[-1]} deep, the bank {depth}")
-    rows = _product_rows(x, "x", offsets, experts, gather, scatter, rows)
+    rows = _product_rows(x, "x", offsets, experts, gather, scatter, rows, sizes)
     bias = _expert_bias(bias, experts, width)
     out = torch.empty((rows, width), dtype=torch.bfloat16, device=x.device)
+    if offsets is None:
+        _lib.check(_lib.library().dew_moe_grouped_gemm_sizes(_ptr(x), _ptr(gather), _ptr(sizes), bank.descriptor, _ptr(bias),
+                                                             _ptr(scatter), _ptr(out), rows, _stream()), "dew_moe_grouped_gemm_sizes")
+        return out
     _lib.check(_lib.library().dew_moe_grouped_gemm_bias(_ptr(x), _ptr(gather), _ptr(offsets), bank.descriptor, _ptr(bias),
                                                         _ptr(scatter), _ptr(out), rows, _stream()), "dew_moe_grouped_gemm")
     return out
@@ -310,17 +333,22 @@ def gateup_interleaved(x: torch.Tensor, gate_up: PreparedBank, offsets: torch.Te
     return hidden
 
 
-def gateup_swiglu(x: torch.Tensor, gate: PreparedBank, up: PreparedBank, offsets: torch.Tensor, *,
-                  gather: torch.Tensor | None = None, rows: int | None = None) -> torch.Tensor:
-    """`hidden[i] = swiglu(x[gather[i]] @ Wg[e], x[gather[i]] @ Wu[e])`, bf16 `[rows, F]`, one launch."""
+def gateup_swiglu(x: torch.Tensor, gate: PreparedBank, up: PreparedBank, offsets: torch.Tensor | None, *,
+                  gather: torch.Tensor | None = None, rows: int | None = None, sizes: torch.Tensor | None = None) -> torch.Tensor:
+    """`hidden[i] = swiglu(x[gather[i]] @ Wg[e], x[gather[i]] @ Wu[e])`, bf16 `[rows, F]`, one launch. The groups are
+    `offsets [E + 1]`, or, where that is None, `sizes [E]`."""
     _device(x, "x", torch.bfloat16)
     experts, depth, width = gate.shape
     if x.shape[-1] != depth:
         raise KernelError(f"x rows are {x.shape[-1]} deep, the banks {depth}")
     if up.shape != gate.shape:
         raise KernelError(f"gate {gate.shape} and up {up.shape} differ")
-    rows = _product_rows(x, "x", offsets, experts, gather, None, rows)
+    rows = _product_rows(x, "x", offsets, experts, gather, None, rows, sizes)
     hidden = torch.empty((rows, width), dtype=torch.bfloat16, device=x.device)
+    if offsets is None:
+        _lib.check(_lib.library().dew_moe_gateup_swiglu_sizes(_ptr(x), _ptr(gather), _ptr(sizes), gate.descriptor, up.descriptor,
+                                                              _ptr(hidden), rows, _stream()), "dew_moe_gateup_swiglu_sizes")
+        return hidden
     _lib.check(_lib.library().dew_moe_gateup_swiglu(_ptr(x), _ptr(gather), _ptr(offsets), gate.descriptor, up.descriptor,
                                                     _ptr(hidden), rows, _stream()), "dew_moe_gateup_swiglu")
     return hidden

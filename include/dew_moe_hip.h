@@ -41,12 +41,19 @@ enum {
   DEW_MOE_W_MXFP8 = 5,       /* OCP MXFP8, K-major as `formats.MxFp8` holds a product's matrices: codes */
                              /* u8 e4m3 [E,N,K]; scales u8 e8m0 [E,N,K/32]. For dew_moe_grouped_gemm_   */
                              /* mxfp8_rows only.                                                        */
-  DEW_MOE_W_BF16 = 6         /* unquantized matrices as the reference holds them: codes bf16 [E,K,N]    */
+  DEW_MOE_W_BF16 = 6,        /* unquantized matrices as the reference holds them: codes bf16 [E,K,N]    */
                              /* (`experts/*_proj/kernel`, src/dew/nn/moe.py:1231-1235); no scales. With */
                              /* DEW_MOE_LAYOUT_REFERENCE_KMAJOR, codes bf16 [E,N,K]: the same memory    */
                              /* read as the transposed matrices (an input gradient's: depth and width   */
                              /* are then the transposed product's).                                     */
+  DEW_MOE_W_MXFP4_BLOCKS = 7 /* an MXFP4 checkpoint's own tensors, for dew_moe_prepare_bank only: codes =  */
+                             /* `*_blocks` u8 [E,N,K/32,16] (low nibble the even element), scales =       */
+                             /* `*_scales` E8M0 u8 [E,N,K/32] (src/dew/interop/codecs.py:193-224). The    */
+                             /* prepared bank is DEW_MOE_W_MXFP4 (or _NVFP4) and holds its tensor scales. */
 };
+/* With DEW_MOE_LAYOUT_REFERENCE_KMAJOR a DEW_MOE_W_FP8_BLOCK bank is a DeepSeek-style checkpoint's own tensors stacked by
+ * expert: codes = `weight` e4m3 [E,N,K] ([out, in]), scales = `weight_scale_inv` f32 [E,N/128,K/128]
+ * (src/dew/interop/codecs.py:670-703).                                                                            */
 
 enum { DEW_MOE_LAYOUT_REFERENCE = 0, DEW_MOE_LAYOUT_PREPARED = 1, DEW_MOE_LAYOUT_REFERENCE_KMAJOR = 2 };
 
@@ -129,14 +136,19 @@ int dew_moe_group_offsets(const int32_t* sizes, int32_t experts, int32_t* offset
  * bank at load; `prepared` must hold dew_moe_prepared_bytes() bytes, 256-byte aligned. `out` describes
  * the prepared bank and is what the GEMM entry points take. For an NVFP4 bank the call waits for the
  * stream once, to read back whether every block scale is a power of two (then out->format is
- * DEW_MOE_W_MXFP4 and the kernels convert codes and scale in one hardware instruction).                 */
+ * DEW_MOE_W_MXFP4 and the kernels convert codes and scale in one hardware instruction). A checkpoint's MXFP4
+ * tensors (DEW_MOE_W_MXFP4_BLOCKS) become the same prepared bank as the reference's own conversion of them would
+ * (`mxfp4_tensor_powers`, `mxfp4_as_nvfp4`, src/dew/interop/codecs.py:238-284, then `NvFp4.of`), without a value or a
+ * word decoded; where the reference keeps such a bank dense (an expert's group powers spread past 17 binades, a 0xff
+ * scale byte) the call refuses it by name. Load time only: the call synchronizes and is not for a captured step.  */
 size_t dew_moe_prepared_bytes(int32_t format, int32_t experts, int32_t depth, int32_t width);
 int dew_moe_prepare_bank(const dew_moe_bank* reference, void* prepared, dew_moe_bank* out /* host */,
                          void* stream);
 
-/* Tuning and testing knob (no counterpart in the reference): every later grouped product of this process uses
- * block tiles of `rows` rows (32, 64, 128 or 256; 256 with FP4 banks whose width is whole 256s); 0, the default,
- * chooses per launch from the rows, experts and width.                                                      */
+/* Tuning and testing knob (no counterpart in the reference): every later grouped product launched by the CALLING
+ * THREAD uses block tiles of `rows` rows (32, 64, 128 or 256; 256 with FP4 banks whose width is whole 256s); 0, the
+ * default, chooses per launch from the rows, experts and width. The setting is thread-local: other threads' launches
+ * (an FFI thread pool's) keep their own choice.                                                              */
 int dew_moe_tile_rows(int32_t rows);
 
 /* ---- Grouped products (src/dew/nn/moe.py:666-770 expert_projection / paired_projections; replaces the
@@ -148,6 +160,16 @@ int dew_moe_tile_rows(int32_t rows);
 int dew_moe_grouped_gemm(const void* x /* bf16 [*,K] */, const int32_t* gather, const int32_t* offsets,
                          const dew_moe_bank* w /* prepared, [E,K,N] */, const int32_t* scatter,
                          void* out /* bf16 [rows,N] */, int32_t rows, void* stream);
+
+/* dew_moe_grouped_gemm_bias and dew_moe_gateup_swiglu taking the groups as the reference's FFI targets take them:
+ * `group_sizes s32[E]`, the operand of jax.lax.ragged_dot and of dew_cutlass_grouped_gemm (kernels/cutlass/ffi.cu:180-198,
+ * groups.cuh:19-30). The exclusive prefix is formed on the device inside each block's tile search, so a launch class
+ * that holds sizes needs no prefix launch; everything else is the entry point of the same name without `_sizes`.   */
+int dew_moe_grouped_gemm_sizes(const void* x, const int32_t* gather, const int32_t* group_sizes /* [E] */,
+                               const dew_moe_bank* w, const float* bias /* nullable */, const int32_t* scatter, void* out,
+                               int32_t rows, void* stream);
+int dew_moe_gateup_swiglu_sizes(const void* x, const int32_t* gather, const int32_t* group_sizes /* [E] */,
+                                const dew_moe_bank* gate, const dew_moe_bank* up, void* hidden, int32_t rows, void* stream);
 
 /* The same with each expert's bias[E,N] (values of the compute dtype held in fp32) added to its rows' fp32
  * sums before their one rounding (src/dew/nn/moe.py:729-742 _biased / _plus_bias; NULL = none).          */

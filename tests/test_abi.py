@@ -27,7 +27,8 @@ def test_introspection_strings_and_size_queries():
     fields = lib.dew_moe_kernel_fields().decode().split(",")
     for line in lib.dew_moe_kernels().decode().strip().splitlines():
         assert len(line.split(",")) == len(fields)
-    assert lib.dew_moe_prepared_bytes(_lib.W_FP8_BLOCK, 2, 256, 128) == 2 * 256 * 128
+    assert lib.dew_moe_prepared_bytes(_lib.W_FP8_BLOCK, 2, 256, 128) == 2 * 256 * 128 + 2 * 2 * 1 * 4   # codes + block scales
+    assert lib.dew_moe_prepared_bytes(_lib.W_FP8_CHANNEL, 2, 256, 128) == 2 * 256 * 128
     assert lib.dew_moe_prepared_bytes(_lib.W_NVFP4, 2, 256, 128) == 2 * 256 * 128 // 2 + 2 * 128 * 16 + 256
     assert lib.dew_moe_permute_workspace_bytes(4096, 8) >= 2 * 2 * 9 * 4
 

@@ -495,3 +495,30 @@ def test_last_tiles_of_at_most_64_rows_go_to_a_launch_of_their_own(ops, quant):
     got = bf16_np(shared)
     assert np.all(got[scatter[rows:]] == 0)
     assert np.abs(got[scatter[:rows]] - want).max() <= 2 ** -7 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("quant", ["fp8_block", "mxfp4", "bf16"])
+def test_group_sizes_in_place_of_their_prefix_give_the_same_products(ops, quant):
+    """The reference's FFI operand is `group_sizes [E]` (kernels/cutlass/ffi.cu:185-198): handed in as they are, the
+    launch forms the prefix in its tile search. Same bits as with the prefix, for both entry points, every tile
+    height, ragged and empty groups, rows past the groups zero; more than 256 groups walk the search's second round."""
+    from dew_amd import gemm
+
+    for sizes, depth, width in (([130, 0, 1, 257, 64, 0, 127, 5], 256, 256), ([3] * 150 + [0] * 60 + [7] * 90, 256, 128)):
+        bank, x, offsets = grouped_case(quant, len(sizes), depth, width, sizes, seed=len(sizes))
+        up, _, _ = grouped_case(quant, len(sizes), depth, width, sizes, seed=len(sizes) + 1)
+        rows = int(np.sum(sizes))
+        padded = rows + 9
+        gather = torch.from_numpy(np.concatenate([np.random.default_rng(1).integers(0, rows, size=rows), np.zeros(9)]).astype(np.int32)).cuda()
+        scatter = torch.from_numpy(np.random.default_rng(2).permutation(padded).astype(np.int32)).cuda()
+        xd, od, sd = x.cuda(), torch.from_numpy(offsets).cuda(), torch.tensor(sizes, dtype=torch.int32).cuda()
+        pb, pu = ops.prepare(bank.to("cuda")), ops.prepare(up.to("cuda"))
+        for tile in (0, 32, 64, 128):
+            with ops.tile_rows(tile):
+                want = ops.grouped_gemm(xd, pb, od, gather=gather, scatter=scatter, rows=padded)
+                got = ops.grouped_gemm(xd, pb, None, sizes=sd, gather=gather, scatter=scatter, rows=padded)
+                assert torch.equal(got, want), (quant, tile, len(sizes))
+                want = ops.gateup_swiglu(xd, pb, pu, od, gather=gather, rows=padded)
+                assert torch.equal(ops.gateup_swiglu(xd, pb, pu, None, sizes=sd, gather=gather, rows=padded), want)
+        assert torch.equal(gemm.gemm(xd, pb, sd, gather=gather[:rows]), ops.grouped_gemm(xd, pb, od, gather=gather[:rows]))
+        assert torch.equal(gemm.gemm(xd, pb, sd, paired=pu, epilogue="swiglu"), ops.gateup_swiglu(xd, pb, pu, od, rows=rows))
