@@ -85,14 +85,25 @@ def build_workload(case, device, seed=0):
 class Stepper:
     """One step of the hot path, launch by launch, with optional HIP events around the gate/up launch."""
 
-    def __init__(self, case, data, split=True):
+    def __init__(self, case, data, split=True, fuse_shared=True):
         import torch
 
-        from dew_amd import gemm, ops
+        from dew_amd import gemm, moe, ops
 
         self.torch, self.ops, self.case, self.data = torch, ops, case, data
-        self.gate, self.up, self.down = (gemm.prepared(data["banks"][n]) for n in ("gate", "up", "down"))
-        self.shared = None if data["shared"] is None else tuple(gemm.prepared(data["shared"][n]) for n in ("gate", "up", "down"))
+        names = ("gate", "up", "down")
+        # a shared expert of the routed experts' shape and format rides the routed launches as their group #E (the layer's
+        # own rule, moe.with_shared_expert); else it is a dense MLP of its own and the combine adds its output
+        stack = None
+        if data["shared"] is not None and fuse_shared:
+            stack = moe.with_shared_expert(tuple(data["banks"][n] for n in names), tuple(data["shared"][n] for n in names))
+        self.fused_shared = stack is not None
+        if self.fused_shared:
+            self.gate, self.up, self.down = (gemm.prepared(bank) for bank in stack)
+            self.shared = None
+        else:
+            self.gate, self.up, self.down = (gemm.prepared(data["banks"][n]) for n in names)
+            self.shared = None if data["shared"] is None else tuple(gemm.prepared(data["shared"][n]) for n in names)
         tokens = case.tokens
         self.dense_offsets = torch.tensor([0, tokens], dtype=torch.int32, device=data["x"].device)
         self.events = []
@@ -101,16 +112,17 @@ class Stepper:
     def __call__(self, timed: bool = False):
         torch, ops, case, data = self.torch, self.ops, self.case, self.data
         weights, indices = ops.route(data["logits"], case.top_k, bias=data["bias"], **case.router)
-        plan = ops.sort_by_expert(indices, case.experts)
+        plan = ops.sort_by_expert(indices, case.experts, case.tokens if self.fused_shared else 0)
         if timed:
             start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             start.record()
         slots = self.project(plan, (start, stop) if timed else None)
-        addend = None
+        routed = case.tokens * case.top_k
+        addend = slots[routed:] if self.fused_shared else None
         if self.shared is not None:
             shared_hidden = ops.gateup_swiglu(data["x"], self.shared[0], self.shared[1], self.dense_offsets)
             addend = ops.grouped_gemm(shared_hidden, self.shared[2], self.dense_offsets)
-        return ops.combine(slots.view(case.tokens, case.top_k, case.d_model), weights, addend), plan
+        return ops.combine(slots[:routed].view(case.tokens, case.top_k, case.d_model), weights, addend), plan
 
     def on_split_rows(self):
         """Whether the routed experts run on split rows and the scaled matrix instruction (the library's rule)."""
@@ -150,7 +162,7 @@ def oracle_sample(case, data, plan, budget_rows=192):
     from dew_amd import formats
     from oracle import moe_oracle as oracle
 
-    sizes = plan.sizes.cpu().numpy()
+    sizes = plan.sizes.cpu().numpy()[:case.experts]      # (a fused shared expert is group #E of the plan: not sampled here)
     offsets = plan.offsets.cpu().numpy()
     expert = int(sizes.argmax())
     rows = int(min(budget_rows, sizes[expert]))
@@ -240,7 +252,7 @@ def measure(config, args, device, sustained, with_cpu_baseline):
 
     case = CONFIGS[config]
     data = build_workload(case, device)
-    stepper = Stepper(case, data, split=not args.bf16_operands)
+    stepper = Stepper(case, data, split=not args.bf16_operands, fuse_shared=not args.separate_shared)
     graphed = args.graph == "on" or (args.graph == "auto" and config in GRAPHED)
     for _ in range(args.warmup):
         stepper()
@@ -276,14 +288,15 @@ def measure(config, args, device, sustained, with_cpu_baseline):
 
     routed_rows = case.tokens * case.top_k
     flops = 6.0 * routed_rows * case.d_model * case.d_ff + (6.0 * case.tokens * case.d_model * case.d_ff if case.shared else 0.0)
-    gateup_flops = 4.0 * routed_rows * case.d_model * case.d_ff
+    gateup_rows = routed_rows + (case.tokens if stepper.fused_shared else 0)   # the launch multiplies a fused shared expert's rows too
+    gateup_flops = 4.0 * gateup_rows * case.d_model * case.d_ff
     gateup_ms = stepper.gateup_ms()
     achieved = gateup_flops / (gateup_ms * 1e-3) / 1e12
     decode = config in DECODE
     bytes_per_weight = 0.5 if case.quant in ("mxfp4", "nvfp4") else 1.0
-    touched = int((plan.sizes > 0).sum().item())
+    touched = int((plan.sizes[:case.experts] > 0).sum().item())
     # bandwidth view: the touched experts' gate and up codes read once + activations in, hidden out
-    gateup_bytes = touched * 2 * case.d_model * case.d_ff * bytes_per_weight + case.tokens * case.d_model * 2 + routed_rows * case.d_ff * 2
+    gateup_bytes = (touched + (1 if stepper.fused_shared else 0)) * 2 * case.d_model * case.d_ff * bytes_per_weight + case.tokens * case.d_model * 2 + gateup_rows * case.d_ff * 2
     gateup_gbs = gateup_bytes / (gateup_ms * 1e-3) / 1e9
     sustained_mfma, sustained_copy = sustained
     if decode:
@@ -320,7 +333,8 @@ def measure(config, args, device, sustained, with_cpu_baseline):
         "config": {"workload": f"{config}: T={case.tokens} D={case.d_model} F={case.d_ff} E={case.experts} k={case.top_k} "
                                f"{case.quant} weights, {case.router['score_function']} router"
                                + (" + shared expert" if case.shared else ""),
-                   "routed_rows": routed_rows, "experts_touched": touched, "launch": "hip graph replay" if graphed else "eager",
+                   "routed_rows": routed_rows, "experts_touched": touched,
+                   **({"shared_expert": "group #E of the routed launches" if stepper.fused_shared else "two launches of its own"} if case.shared else {}), "launch": "hip graph replay" if graphed else "eager",
                    "algorithmic_flops": flops},
         "roofline": roofline,
     }
@@ -364,6 +378,9 @@ def main():
     parser.add_argument("--bf16-operands", action="store_true",
                         help="keep MXFP4 banks with groups of hundreds of rows on the bf16 matrix instruction too (the default "
                              "there: rows split into two e4m3 terms and the scaled instruction, the library's own choice)")
+    parser.add_argument("--separate-shared", action="store_true",
+                        help="compute a shared expert as a dense MLP of its own (two more launches), as the reference does, instead "
+                             "of as group #E of the routed launches")
     parser.add_argument("--graph", choices=["auto", "on", "off"], default="auto",
                         help="replay the step as one captured HIP graph (auto: for the launch-bound configs c1 and c3)")
     args = parser.parse_args()

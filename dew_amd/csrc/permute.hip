@@ -27,11 +27,21 @@ struct PermuteParams {
   int32_t* rows;       // [slots]
   int32_t* counts;     // workspace [blocks][buckets]
   int32_t* bases;      // workspace [blocks][buckets]
-  int slots, experts, top_k, blocks, buckets;
+  // `slots` sorted positions: the `routed` = tokens * top_k slots of `ids`, then `slots - routed` rows that every token
+  // sends to one always-on (shared) expert, which sorts as group `experts`. `groups` = the groups written (experts, or
+  // experts + 1 with a shared one); bucket `groups` collects the dropped slots (an id outside [0, experts)), last.
+  int slots, routed, experts, groups, top_k, blocks, buckets;
 };
 
-__device__ __forceinline__ int bucket_of(int id, int experts) {
-  return (id < 0 || id >= experts) ? experts : id;
+__device__ __forceinline__ int bucket_of(const PermuteParams& p, int slot) {
+  if (slot >= p.routed) return p.experts;  // a shared expert's row
+  const int id = p.ids[slot];
+  return (id < 0 || id >= p.experts) ? p.groups : id;
+}
+
+// The row of the activations a slot reads: its token, or for a shared expert's row the token it is.
+__device__ __forceinline__ int row_of(const PermuteParams& p, int slot) {
+  return slot < p.routed ? slot / p.top_k : slot - p.routed;
 }
 
 __global__ __launch_bounds__(kPermuteThreads) void permute_count_kernel(PermuteParams p) {
@@ -41,7 +51,7 @@ __global__ __launch_bounds__(kPermuteThreads) void permute_count_kernel(PermuteP
   const int begin = blockIdx.x * kSlotsPerBlock;
   const int end = min(begin + kSlotsPerBlock, p.slots);
   for (int slot = begin + threadIdx.x; slot < end; slot += kPermuteThreads)
-    atomicAdd(&hist[bucket_of(p.ids[slot], p.experts)], 1);
+    atomicAdd(&hist[bucket_of(p, slot)], 1);
   __syncthreads();
   for (int b = threadIdx.x; b < p.buckets; b += kPermuteThreads)
     p.counts[static_cast<size_t>(blockIdx.x) * p.buckets + b] = hist[b];
@@ -68,11 +78,11 @@ __global__ __launch_bounds__(kPermuteThreads) void permute_scan_kernel(PermutePa
   __syncthreads();
   for (int b = threadIdx.x; b < p.buckets; b += kPermuteThreads) {
     const int start = totals[b];
-    if (b < p.experts) {
+    if (b < p.groups) {
       p.sizes[b] = totals[b + 1] - start;
       p.offsets[b] = start;
     } else {
-      p.offsets[p.experts] = start;  // slots routed to a real expert
+      p.offsets[p.groups] = start;  // slots routed to a real expert
     }
     int running = start;
     for (int blk = 0; blk < p.blocks; ++blk) {
@@ -96,7 +106,7 @@ __global__ __launch_bounds__(kPermuteThreads) void permute_scatter_kernel(Permut
   const int wave_begin = block_begin + wave * kSlotsPerWave;
   for (int round = 0; round < kSlotsPerWave / 64; ++round) {
     const int slot = wave_begin + round * 64 + lane;
-    if (slot < p.slots) atomicAdd(&mine[bucket_of(p.ids[slot], p.experts)], 1);
+    if (slot < p.slots) atomicAdd(&mine[bucket_of(p, slot)], 1);
   }
   __syncthreads();
   // turn the per-wave counts into each wave's first position: block base + earlier waves' counts
@@ -115,7 +125,7 @@ __global__ __launch_bounds__(kPermuteThreads) void permute_scatter_kernel(Permut
   for (int round = 0; round < kSlotsPerWave / 64; ++round) {
     const int slot = wave_begin + round * 64 + lane;
     const bool valid = slot < p.slots;
-    const int bucket = valid ? bucket_of(p.ids[slot], p.experts) : p.buckets;  // invalid lanes match nobody real
+    const int bucket = valid ? bucket_of(p, slot) : p.buckets;  // invalid lanes match nobody real
     unsigned long long same = __ballot(valid);
     for (int bit = 0; bit < bits; ++bit) {
       const bool set = (bucket >> bit) & 1;
@@ -132,7 +142,7 @@ __global__ __launch_bounds__(kPermuteThreads) void permute_scatter_kernel(Permut
     __syncthreads();
     if (valid) {
       p.order[position] = slot;
-      p.rows[position] = slot / p.top_k;
+      p.rows[position] = row_of(p, slot);
     }
   }
 }
@@ -154,7 +164,7 @@ __global__ __launch_bounds__(kPermuteThreads) void permute_small_kernel(PermuteP
   const int wave_begin = wave * segment;
   for (int round = 0; round < rounds; ++round) {
     const int slot = wave_begin + round * 64 + lane;
-    if (slot < p.slots) atomicAdd(&mine[bucket_of(p.ids[slot], p.experts)], 1);
+    if (slot < p.slots) atomicAdd(&mine[bucket_of(p, slot)], 1);
   }
   __syncthreads();
   for (int b = threadIdx.x; b < p.buckets; b += kPermuteThreads) {
@@ -182,11 +192,11 @@ __global__ __launch_bounds__(kPermuteThreads) void permute_small_kernel(PermuteP
   __syncthreads();
   for (int b = threadIdx.x; b < p.buckets; b += kPermuteThreads) {
     const int start = totals[b];
-    if (b < p.experts) {
+    if (b < p.groups) {
       p.sizes[b] = totals[b + 1] - start;
       p.offsets[b] = start;
     } else {
-      p.offsets[p.experts] = start;
+      p.offsets[p.groups] = start;
     }
     int next = start;
     for (int w = 0; w < kPermuteWaves; ++w) {
@@ -201,7 +211,7 @@ __global__ __launch_bounds__(kPermuteThreads) void permute_small_kernel(PermuteP
   for (int round = 0; round < rounds; ++round) {
     const int slot = wave_begin + round * 64 + lane;
     const bool valid = slot < p.slots;
-    const int bucket = valid ? bucket_of(p.ids[slot], p.experts) : p.buckets;
+    const int bucket = valid ? bucket_of(p, slot) : p.buckets;
     unsigned long long same = __ballot(valid);
     for (int bit = 0; bit < bits; ++bit) {
       const bool set = (bucket >> bit) & 1;
@@ -217,7 +227,7 @@ __global__ __launch_bounds__(kPermuteThreads) void permute_small_kernel(PermuteP
     __syncthreads();
     if (valid) {
       p.order[position] = slot;
-      p.rows[position] = slot / p.top_k;
+      p.rows[position] = row_of(p, slot);
     }
   }
 }
@@ -234,9 +244,9 @@ namespace dew {
 
 // The sort's launches, given where the per-block counts and bases live (the caller's workspace or the library's own
 // scratch array): `counts` holds 2 * blocks * buckets int32, 256-byte aligned.
-static int permute_launches(const int32_t* indices, int32_t tokens, int32_t top_k, int32_t experts, int32_t* sizes,
-                            int32_t* offsets, int32_t* order, int32_t* rows, int32_t* counts, hipStream_t s) {
-  const int slots = tokens * top_k;
+static int permute_launches(const int32_t* indices, int32_t tokens, int32_t top_k, int32_t experts, int32_t shared_rows,
+                            int32_t* sizes, int32_t* offsets, int32_t* order, int32_t* rows, int32_t* counts, hipStream_t s) {
+  const int slots = tokens * top_k + shared_rows;
   PermuteParams p;
   p.ids = indices;
   p.sizes = sizes;
@@ -244,9 +254,11 @@ static int permute_launches(const int32_t* indices, int32_t tokens, int32_t top_
   p.order = order;
   p.rows = rows;
   p.slots = slots;
+  p.routed = tokens * top_k;
   p.experts = experts;
+  p.groups = experts + (shared_rows > 0 ? 1 : 0);
   p.top_k = top_k;
-  p.buckets = experts + 1;
+  p.buckets = p.groups + 1;
   p.blocks = (slots + kSlotsPerBlock - 1) / kSlotsPerBlock;
   p.counts = counts;
   p.bases = p.counts + static_cast<size_t>(p.blocks) * p.buckets;
@@ -313,7 +325,25 @@ extern "C" int dew_moe_permute(const int32_t* indices, int32_t tokens, int32_t t
               "dew_moe_permute: workspace of %zu bytes, need %zu", workspace_bytes,
               dew_moe_permute_workspace_bytes(slots, experts));
   const uintptr_t base = (reinterpret_cast<uintptr_t>(workspace) + 255) & ~static_cast<uintptr_t>(255);
-  return permute_launches(indices, tokens, top_k, experts, sizes, offsets, order, rows, reinterpret_cast<int32_t*>(base),
+  return permute_launches(indices, tokens, top_k, experts, 0, sizes, offsets, order, rows, reinterpret_cast<int32_t*>(base),
+                          static_cast<hipStream_t>(stream));
+}
+
+extern "C" int dew_moe_permute_shared(const int32_t* indices, int32_t tokens, int32_t top_k, int32_t experts, int32_t shared_rows,
+                                      int32_t* sizes, int32_t* offsets, int32_t* order, int32_t* rows, void* workspace,
+                                      size_t workspace_bytes, void* stream) {
+  using namespace dew;
+  const char* who = "dew_moe_permute_shared";
+  if (int rc = permute_arguments(who, indices, tokens, top_k, experts, sizes, offsets, order, rows)) return rc;
+  DEW_REQUIRE(shared_rows >= 0 && static_cast<int64_t>(tokens) * top_k + shared_rows < (1ll << 30) && experts < kMaxExperts,
+              "%s: %d shared rows beside %d x %d slots, %d experts (a shared group needs one below %d)", who, shared_rows, tokens,
+              top_k, experts, kMaxExperts);
+  DEW_REQUIRE(shared_rows == 0 || (order && rows), "%s: order and rows must not be null", who);
+  const int slots = tokens * top_k + shared_rows;
+  const size_t need = dew_moe_permute_workspace_bytes(slots, experts + 1);
+  DEW_REQUIRE(workspace && workspace_bytes >= need, "%s: workspace of %zu bytes, need %zu", who, workspace_bytes, need);
+  const uintptr_t base = (reinterpret_cast<uintptr_t>(workspace) + 255) & ~static_cast<uintptr_t>(255);
+  return permute_launches(indices, tokens, top_k, experts, shared_rows, sizes, offsets, order, rows, reinterpret_cast<int32_t*>(base),
                           static_cast<hipStream_t>(stream));
 }
 
@@ -329,6 +359,6 @@ extern "C" int dew_moe_permute_static(const int32_t* indices, int32_t tokens, in
   void* base = nullptr;
   if (int rc = static_scratch(who, &base)) return rc;
   // every int32 of the counts and bases a call reads is written earlier in the same call: nothing to clear
-  return permute_launches(indices, tokens, top_k, experts, sizes, offsets, order, rows, static_cast<int32_t*>(base),
+  return permute_launches(indices, tokens, top_k, experts, 0, sizes, offsets, order, rows, static_cast<int32_t*>(base),
                           static_cast<hipStream_t>(stream));
 }

@@ -297,6 +297,26 @@ class MxFp8:
         return MxFp8(self.codes.to(device), self.scales.to(device))
 
 
+def stacked(banks):
+    """Banks of one format and one matrix shape as one bank along the expert axis (the routed experts and, behind
+    them, an always-on expert the same launches multiply as one more group), or None where they do not stack."""
+    first = banks[0]
+    if any(type(bank) is not type(first) or tuple(bank.shape[1:]) != tuple(first.shape[1:]) for bank in banks):
+        return None
+    if isinstance(first, (Fp8Blocks, Bf16)) and any(getattr(bank, "kmajor", False) != getattr(first, "kmajor", False)
+                                                   or getattr(bank, "transposed", False) != getattr(first, "transposed", False) for bank in banks):
+        return None
+    if not dataclasses.is_dataclass(first) or isinstance(first, Layered):
+        return None
+    joined = {}
+    for field in dataclasses.fields(first):
+        value = getattr(first, field.name)
+        if field.name == "form":
+            continue
+        joined[field.name] = torch.cat([getattr(bank, field.name) for bank in banks]) if torch.is_tensor(value) else value
+    return type(first)(**joined)
+
+
 @dataclasses.dataclass(frozen=True)
 class Layered:
     """An expert kernel read in place from a run's stack (src/dew/nn/moe.py:595-606): `stack` the bank of every

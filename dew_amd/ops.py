@@ -118,20 +118,29 @@ class Plan:
     offsets: torch.Tensor
 
 
-def sort_by_expert(indices: torch.Tensor, num_experts: int) -> Plan:
+def sort_by_expert(indices: torch.Tensor, num_experts: int, shared_rows: int = 0) -> Plan:
+    """The stable sort of the routed slots by expert. With `shared_rows` (the tokens, where every token also takes one
+    always-on expert) that expert is group `num_experts` of the plan: `shared_rows` more sorted positions behind the
+    routed ones, position i of them reading token i and writing row `slots + i`; `sizes` and `offsets` grow by one."""
     _device(indices, "indices", torch.int32)
     top_k = indices.shape[-1]
     tokens = indices.numel() // top_k
-    slots = tokens * top_k
+    slots = tokens * top_k + shared_rows
+    groups = num_experts + (1 if shared_rows else 0)
     device = indices.device
     lib = _lib.library()
-    workspace = torch.empty(lib.dew_moe_permute_workspace_bytes(slots, num_experts), dtype=torch.uint8, device=device)
-    sizes = torch.empty(num_experts, dtype=torch.int32, device=device)
-    offsets = torch.empty(num_experts + 1, dtype=torch.int32, device=device)
+    workspace = torch.empty(lib.dew_moe_permute_workspace_bytes(slots, groups), dtype=torch.uint8, device=device)
+    sizes = torch.empty(groups, dtype=torch.int32, device=device)
+    offsets = torch.empty(groups + 1, dtype=torch.int32, device=device)
     order = torch.empty(slots, dtype=torch.int32, device=device)
     rows = torch.empty(slots, dtype=torch.int32, device=device)
-    _lib.check(lib.dew_moe_permute(_ptr(indices), tokens, top_k, num_experts, _ptr(sizes), _ptr(offsets), _ptr(order),
-                                   _ptr(rows), _ptr(workspace), workspace.numel(), _stream()), "dew_moe_permute")
+    if shared_rows:
+        _lib.check(lib.dew_moe_permute_shared(_ptr(indices), tokens, top_k, num_experts, shared_rows, _ptr(sizes), _ptr(offsets),
+                                              _ptr(order), _ptr(rows), _ptr(workspace), workspace.numel(), _stream()),
+                   "dew_moe_permute_shared")
+    else:
+        _lib.check(lib.dew_moe_permute(_ptr(indices), tokens, top_k, num_experts, _ptr(sizes), _ptr(offsets), _ptr(order),
+                                       _ptr(rows), _ptr(workspace), workspace.numel(), _stream()), "dew_moe_permute")
     return Plan(order, rows, sizes, offsets)
 
 
@@ -220,7 +229,7 @@ def prepare(bank) -> PreparedBank:
     elif isinstance(bank, formats.Fp8Blocks):
         fmt, codes, scales, tensor = _lib.W_FP8_BLOCK, bank.codes, bank.scale_inv, None
         _device(codes, "Fp8Blocks.codes", torch.uint8), _device(scales, "Fp8Blocks.scale_inv", torch.float32)
-        blocks = (bank.shape[2] // 128, bank.shape[1] // 128) if bank.kmajor else (bank.shape[1] // 128, bank.shape[2] // 128)
+        blocks = tuple(-(-extent // 128) for extent in ((bank.shape[2], bank.shape[1]) if bank.kmajor else bank.shape[1:]))
         if tuple(scales.shape) != (bank.shape[0], *blocks):
             raise KernelError(f"Fp8Blocks.scale_inv is {tuple(scales.shape)}, the bank's blocks {(bank.shape[0], *blocks)}")
     elif isinstance(bank, formats.Mxfp4Blocks):

@@ -114,6 +114,16 @@ int dew_moe_permute(const int32_t* indices /* [T,k] */, int32_t tokens, int32_t 
                     int32_t* sizes, int32_t* offsets, int32_t* order, int32_t* rows, void* workspace,
                     size_t workspace_bytes, void* stream);
 
+/* dew_moe_permute with an always-on (shared) expert folded in as group E (src/dew/nn/moe.py:1497-1503 adds the shared
+ * expert's output to every token's; as one more group of the same grouped launches it costs no launch of its own):
+ * behind the R routed slots come `shared_rows` more sorted positions, one a token, that belong to group E and read row
+ * i of the activations: sizes[E + 1] (sizes[E] = shared_rows), offsets[E + 2], order[R + shared_rows] and
+ * rows[R + shared_rows], with order = R + i and rows = i for the shared group's position i; dropped slots (ids outside
+ * [0, E)) still sort last, behind the shared group. Workspace: dew_moe_permute_workspace_bytes(R + shared_rows, E + 1). */
+int dew_moe_permute_shared(const int32_t* indices /* [T,k] */, int32_t tokens, int32_t top_k, int32_t experts,
+                           int32_t shared_rows, int32_t* sizes, int32_t* offsets, int32_t* order, int32_t* rows,
+                           void* workspace, size_t workspace_bytes, void* stream);
+
 /* dew_moe_permute for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc) and so have no workspace to hand in; no counterpart in the reference, whose FFI
  * handler takes its workspace from XLA's ScratchAllocator. The sort's per-block counts live in an array of

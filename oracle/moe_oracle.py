@@ -11,7 +11,7 @@ What pins each function (tests/test_oracle_golden.py):
 * `route`: router_indices (exact) / router_weights (1e-6) of tests/fixtures/moe/{mixtral,deepseek,
   deepseek_v2,deepseek_v4}.npz.
 * `sparse_mlp` (fp32 mode): block_output / experts_output of the same files (2e-5).
-* `sorted_by_expert`: brute force on tiny inputs + invariants (a stable counting sort is a closed form).
+* `sorted_by_expert`, `sorted_with_shared`: brute force on tiny inputs + invariants (a stable counting sort is a closed form).
 * `dequantize_fp8_blocks`: tests/fixtures/codecs/deepseek_kernels.npz `v3/*/dequantized`, bit for bit.
 * `decode_mxfp4`: tests/fixtures/gpt_oss/mxfp4.npz `output`, bit for bit.
 * `nvfp4_words_to_codes` / `nvfp4_bank_decoded`: the 32 literal encoder masks and the 8-step decode form of
@@ -418,6 +418,24 @@ def sorted_by_expert(indices, num_experts):
     sizes = np.bincount(experts, minlength=num_experts)[:num_experts].astype(np.int32)
     offsets = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
     return {"order": order, "rows": (order // k).astype(np.int32), "sizes": sizes, "offsets": offsets}
+
+
+def sorted_with_shared(indices, num_experts, shared_rows):
+    """`sorted_by_expert` with an always-on expert as group `num_experts`: behind the routed slots come `shared_rows`
+    more slots of that group, slot `R + i` reading token i (src/dew/nn/moe.py:1497-1503 runs that expert as a dense MLP
+    over every token; as one more group of the sort its rows ride the routed experts' launches). Dropped slots (an id
+    outside [0, num_experts)) sort behind it. Returns dict(order, rows, sizes [E + 1], offsets [E + 2])."""
+    indices = np.asarray(indices)
+    k = indices.shape[-1]
+    routed = indices.size
+    ids = indices.reshape(-1).astype(np.int64)
+    ids = np.where((ids < 0) | (ids >= num_experts), num_experts + 1, ids)
+    buckets = np.concatenate([ids, np.full(shared_rows, num_experts, np.int64)])
+    order = np.argsort(buckets, kind="stable").astype(np.int32)
+    sizes = np.bincount(buckets, minlength=num_experts + 1)[:num_experts + 1].astype(np.int32)
+    offsets = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    rows = np.where(order < routed, order // k, order - routed).astype(np.int32)
+    return {"order": order, "rows": rows, "sizes": sizes, "offsets": offsets}
 
 
 # --------------------------------------------------------------------------------------------------

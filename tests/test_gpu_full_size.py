@@ -40,8 +40,16 @@ def test_full_size_configuration(name):
 
     # the stable sort by expert: a permutation, experts non-decreasing, slots ascending inside an expert
     flat = indices.reshape(-1)
+    shared_rows = tokens if stepper.fused_shared else 0
+    assert stepper.fused_shared == case.shared                      # c4's shared expert rides the routed launches as group #E
     order = plan.order.long()
-    assert torch.equal(torch.sort(order).values, torch.arange(routed, device=device))
+    assert torch.equal(torch.sort(order).values, torch.arange(routed + shared_rows, device=device))
+    if shared_rows:   # the shared group: behind the routed slots, one row a token in token order
+        assert torch.equal(order[routed:], torch.arange(routed, routed + tokens, device=device))
+        assert torch.equal(plan.rows[routed:].long(), torch.arange(tokens, device=device))
+        assert int(plan.sizes[experts]) == tokens and int(plan.offsets[experts + 1]) == routed + tokens
+        plan = type(plan)(plan.order[:routed], plan.rows[:routed], plan.sizes[:experts], plan.offsets[:experts + 1])
+        order = plan.order.long()
     sorted_experts = flat[order]
     assert bool((sorted_experts[1:] >= sorted_experts[:-1]).all())
     same = sorted_experts[1:] == sorted_experts[:-1]
@@ -51,21 +59,29 @@ def test_full_size_configuration(name):
     assert torch.equal(plan.rows.long(), order // k)
 
     # the busiest expert's first rows through all three projections against the oracle, and the combine from the slots
-    _, (sampled_slots, want_down) = bench.cpu_baseline(case, data, out, plan, budget_rows=48)
-    slots = stepper.project(plan)                                   # c2: on split rows, the library's rule for its groups
+    _, (sampled_slots, want_down) = bench.oracle_sample(case, data, plan, budget_rows=48)
+    _, whole_plan = stepper()
+    slots = stepper.project(whole_plan)                             # c2: on split rows, the library's rule for its groups
     assert stepper.on_split_rows() == (name == "c2")
     got_down = slots[torch.from_numpy(sampled_slots).to(device).long()].float().cpu().numpy()
     peak, elementwise = oracle.relative_errors(got_down, want_down)
     assert peak <= 2e-2 and elementwise <= 2e-2, (peak, elementwise)
     assert peak <= 6e-3
     total = torch.zeros((tokens, case.d_model), dtype=torch.float32, device=device)
-    view = slots.view(tokens, k, case.d_model)
+    view = slots[:routed].view(tokens, k, case.d_model)
     for j in range(k):
         total = total + view[:, j, :].float() * weights[:, j, None]
     want_out = total.to(torch.bfloat16)
     if case.shared:
-        dense = ops.gateup_swiglu(data["x"], stepper.shared[0], stepper.shared[1], stepper.dense_offsets)
-        want_out = (want_out.float() + ops.grouped_gemm(dense, stepper.shared[2], stepper.dense_offsets).float()).to(torch.bfloat16)
+        # the shared expert's rows (group #E of the same launches) against the oracle's dense SwiGLU MLP on a sample of tokens
+        from moe_cases import dequantized
+        sampled = np.arange(0, tokens, tokens // 24)[:24]
+        matrices = [dequantized(data["shared"][n].to("cpu"))[0][0] for n in ("gate", "up", "down")]
+        want_shared = oracle.gated_mlp(data["x"][torch.from_numpy(sampled).to(device)].float().cpu().numpy(), *matrices)
+        got_shared = slots[routed:][torch.from_numpy(sampled).to(device)].float().cpu().numpy()
+        peak, elementwise = oracle.relative_errors(got_shared, want_shared)
+        assert peak <= 6e-3 and elementwise <= 2e-2, (peak, elementwise)
+        want_out = (want_out.float() + slots[routed:].float()).to(torch.bfloat16)
     assert torch.equal(out, want_out)
 
 

@@ -111,6 +111,20 @@ def test_permute_is_the_stable_sort_by_expert(ops, tokens, k, experts):
         assert np.array_equal(getattr(got, field).cpu().numpy(), want[field]), field
 
 
+@pytest.mark.parametrize("tokens,k,experts", [(1, 1, 1), (7, 2, 4), (64, 8, 128), (300, 3, 5), (1025, 2, 8), (8192, 8, 256), (3000, 6, 511)])
+def test_permute_with_a_shared_expert_as_one_more_group(ops, tokens, k, experts):
+    rng = np.random.default_rng(tokens * 31 + experts)
+    indices = rng.integers(0, experts, size=(tokens, k)).astype(np.int32)
+    if experts > 2:
+        indices[indices == 1] = 2                          # an empty expert
+    if tokens > 5:
+        indices[3, 0] = experts                            # a dropped slot: it sorts behind the shared group
+    want = oracle.sorted_with_shared(indices, experts, tokens)
+    got = ops.sort_by_expert(torch.from_numpy(indices).cuda(), experts, shared_rows=tokens)
+    for field in ("sizes", "offsets", "order", "rows"):
+        assert np.array_equal(getattr(got, field).cpu().numpy(), want[field]), field
+
+
 def test_permute_sorts_dropped_slots_last_and_outside_every_group(ops):
     indices = np.array([[0, 3], [3, 1], [2, 3], [0, 0]], np.int32)      # id 3 = the sentinel of 3 experts
     got = ops.sort_by_expert(torch.from_numpy(indices).cuda(), 3)

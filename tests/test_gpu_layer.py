@@ -80,6 +80,20 @@ def test_layer_matches_the_oracle(name):
     import dataclasses
     unfused = dataclasses.replace(layer, fused=False).apply(variables, x, logits=logits).float().cpu().numpy()
     assert np.array_equal(unfused, got)
+    if case.shared:
+        # the shared expert as group #E of the routed launches (the default) is the reference's arrangement, a dense
+        # MLP of its own whose output the combine adds, bit for bit
+        from dew_amd import moe
+        calls = []
+        found = moe.with_shared_expert
+        moe.with_shared_expert = lambda *a: calls.append(1) or found(*a)
+        try:
+            assert np.array_equal(layer.apply(variables, x, logits=logits).float().cpu().numpy(), got) and calls == [1]
+            apart = dataclasses.replace(layer, fuse_shared=False).apply(variables, x, logits=logits).float().cpu().numpy()
+            assert calls == [1]
+        finally:
+            moe.with_shared_expert = found
+        assert np.array_equal(apart, got)
 
 
 def test_large_groups_on_mxfp4_banks_run_on_split_rows_and_agree_with_the_bf16_launches(monkeypatch):

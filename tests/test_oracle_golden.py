@@ -319,3 +319,15 @@ def test_a_nan_selection_competes_as_minus_infinity():
     bias[:] = np.nan
     _, indices = oracle.route(logits, 4, score_function="sigmoid", bias=bias)
     assert np.array_equal(indices, np.tile(np.arange(4, dtype=np.int32), (9, 1)))
+
+
+def test_the_sort_with_a_shared_expert_by_brute_force():
+    """Tiny case by hand: 3 tokens, top-2, 3 experts, one dropped slot; the shared expert's three rows form group 3."""
+    indices = np.array([[2, 0], [0, 3], [1, 0]], np.int32)            # id 3: a dropped slot
+    got = oracle.sorted_with_shared(indices, 3, 3)
+    assert got["sizes"].tolist() == [3, 1, 1, 3] and got["offsets"].tolist() == [0, 3, 4, 5, 8]
+    assert got["order"].tolist() == [1, 2, 5, 4, 0, 6, 7, 8, 3]       # experts 0, 1, 2, the shared rows, the dropped slot
+    assert got["rows"].tolist() == [0, 1, 2, 2, 0, 0, 1, 2, 1]
+    plain = oracle.sorted_by_expert(np.array([[2, 0], [0, 1], [1, 0]], np.int32), 3)
+    with_shared = oracle.sorted_with_shared(np.array([[2, 0], [0, 1], [1, 0]], np.int32), 3, 3)
+    assert with_shared["order"][:6].tolist() == plain["order"].tolist() and with_shared["sizes"][:3].tolist() == plain["sizes"].tolist()
