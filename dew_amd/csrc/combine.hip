@@ -50,17 +50,36 @@ __global__ __launch_bounds__(256) void combine_kernel(const bf16_t* __restrict__
   }
 }
 
+// `limit` > 0: the gate clamped from above and the up projection both ways before their product (`swiglu_clamped`,
+// src/dew/nn/activations.py:327-333); the limit enters as the bf16 the operands' dtype rounds it to.
 __global__ __launch_bounds__(256) void swiglu_kernel(const bf16_t* __restrict__ gate, const bf16_t* __restrict__ up,
-                                                     bf16_t* __restrict__ hidden, long long chunks) {
+                                                     bf16_t* __restrict__ hidden, long long chunks, float limit) {
   for (long long item = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; item < chunks;
        item += static_cast<long long>(gridDim.x) * blockDim.x) {
     const Bf16x8 g = reinterpret_cast<const Bf16x8*>(gate)[item];
     const Bf16x8 u = reinterpret_cast<const Bf16x8*>(up)[item];
     Bf16x8 h;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) h.v[i] = swiglu_rounded(bf16_to_f32(g.v[i]), bf16_to_f32(u.v[i]));
+    for (int i = 0; i < 8; ++i) {
+      float gi = bf16_to_f32(g.v[i]), ui = bf16_to_f32(u.v[i]);
+      if (limit > 0.0f) {
+        gi = fminf(gi, limit);
+        ui = fminf(fmaxf(ui, -limit), limit);
+      }
+      h.v[i] = swiglu_rounded(gi, ui);
+    }
     reinterpret_cast<Bf16x8*>(hidden)[item] = h;
   }
+}
+
+// Round to nearest even on the host (the device has the hardware conversion).
+static float bf16_round_host(float value) {
+  uint32_t bits;
+  __builtin_memcpy(&bits, &value, 4);
+  bits += 0x7FFFu + ((bits >> 16) & 1u);
+  bits &= 0xFFFF0000u;
+  __builtin_memcpy(&value, &bits, 4);
+  return value;
 }
 
 }  // namespace dew
@@ -83,7 +102,12 @@ extern "C" int dew_moe_combine(const void* slots, const float* weights, const vo
 }
 
 extern "C" int dew_moe_swiglu(const void* gate, const void* up, void* hidden, int64_t count, void* stream) {
+  return dew_moe_swiglu_clamped(gate, up, 0.0f, hidden, count, stream);
+}
+
+extern "C" int dew_moe_swiglu_clamped(const void* gate, const void* up, float limit, void* hidden, int64_t count, void* stream) {
   using namespace dew;
+  DEW_REQUIRE(limit >= 0.0f, "dew_moe_swiglu: the clamp limit %g must be positive (0: none)", static_cast<double>(limit));
   DEW_REQUIRE(count >= 0 && count % 8 == 0, "dew_moe_swiglu: count %lld is not a multiple of 8", static_cast<long long>(count));
   if (count == 0) return DEW_MOE_OK;
   DEW_REQUIRE(gate && up && hidden, "dew_moe_swiglu: gate, up and hidden must not be null");
@@ -92,6 +116,6 @@ extern "C" int dew_moe_swiglu(const void* gate, const void* up, void* hidden, in
   const int blocks = static_cast<int>(min((chunks + 255) / 256, 256ll * 64));
   hipLaunchKernelGGL(swiglu_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
                      static_cast<const bf16_t*>(gate), static_cast<const bf16_t*>(up), static_cast<bf16_t*>(hidden),
-                     chunks);
+                     chunks, bf16_round_host(limit));
   return launched("swiglu_kernel");
 }

@@ -242,6 +242,64 @@ extern "C" size_t dew_moe_permute_workspace_bytes(int32_t slots, int32_t experts
 
 namespace dew {
 
+// Capacity dropping (`capacity_positions`, src/dew/nn/moe.py:832-855, applied at :914-919): a block a sequence. Each of a
+// sequence's `slots` = length * top_k slots queues at its expert in slot order; a slot whose place in the queue is
+// `capacity` or later is dropped: its id becomes `experts`, the sentinel that sorts last and outside every group.
+// The place is the slot's rank among its sequence's slots of the same expert: the single block's counting sort above,
+// without the scatter.
+__global__ __launch_bounds__(kPermuteThreads) void capacity_admit_kernel(const int32_t* __restrict__ ids, int32_t* __restrict__ admitted,
+                                                                         int slots, int experts, int capacity) {
+  extern __shared__ int32_t running[];  // [kPermuteWaves][buckets]
+  const int buckets = experts + 1;
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const int32_t* mine_ids = ids + static_cast<size_t>(blockIdx.x) * slots;
+  int32_t* out = admitted + static_cast<size_t>(blockIdx.x) * slots;
+  for (int i = threadIdx.x; i < kPermuteWaves * buckets; i += kPermuteThreads) running[i] = 0;
+  __syncthreads();
+  int32_t* mine = running + wave * buckets;
+  const int segment = ((slots + kPermuteThreads - 1) / kPermuteThreads) * 64;  // contiguous slots per wavefront
+  const int rounds = segment / 64, wave_begin = wave * segment;
+  auto bucket_at = [&](int slot) {
+    const int id = mine_ids[slot];
+    return (id < 0 || id >= experts) ? experts : id;
+  };
+  for (int round = 0; round < rounds; ++round) {
+    const int slot = wave_begin + round * 64 + lane;
+    if (slot < slots) atomicAdd(&mine[bucket_at(slot)], 1);
+  }
+  __syncthreads();
+  for (int b = threadIdx.x; b < buckets; b += kPermuteThreads) {  // each wavefront's first place in every queue
+    int next = 0;
+    for (int w = 0; w < kPermuteWaves; ++w) {
+      const int count = running[w * buckets + b];
+      running[w * buckets + b] = next;
+      next += count;
+    }
+  }
+  __syncthreads();
+  int bits = 1;
+  while ((1 << bits) < buckets) ++bits;
+  for (int round = 0; round < rounds; ++round) {
+    const int slot = wave_begin + round * 64 + lane;
+    const bool valid = slot < slots;
+    const int bucket = valid ? bucket_at(slot) : buckets;
+    unsigned long long same = __ballot(valid);
+    for (int bit = 0; bit < bits; ++bit) {
+      const bool set = (bucket >> bit) & 1;
+      const unsigned long long vote = __ballot(set);
+      same &= set ? vote : ~vote;
+    }
+    const int rank = __popcll(same & ((1ull << lane) - 1ull));
+    const int count = __popcll(same);
+    int place = 0;
+    if (valid) place = mine[bucket] + rank;
+    __syncthreads();
+    if (valid && rank == count - 1) mine[bucket] = place + 1;
+    __syncthreads();
+    if (valid) out[slot] = (bucket < experts && place < capacity) ? bucket : experts;
+  }
+}
+
 // The sort's launches, given where the per-block counts and bases live (the caller's workspace or the library's own
 // scratch array): `counts` holds 2 * blocks * buckets int32, 256-byte aligned.
 static int permute_launches(const int32_t* indices, int32_t tokens, int32_t top_k, int32_t experts, int32_t shared_rows,
@@ -361,4 +419,19 @@ extern "C" int dew_moe_permute_static(const int32_t* indices, int32_t tokens, in
   // every int32 of the counts and bases a call reads is written earlier in the same call: nothing to clear
   return permute_launches(indices, tokens, top_k, experts, 0, sizes, offsets, order, rows, static_cast<int32_t*>(base),
                           static_cast<hipStream_t>(stream));
+}
+
+extern "C" int dew_moe_capacity_admit(const int32_t* indices, int32_t sequences, int32_t length, int32_t top_k, int32_t experts,
+                                      int32_t capacity, int32_t* admitted, void* stream) {
+  using namespace dew;
+  const char* who = "dew_moe_capacity_admit";
+  DEW_REQUIRE(sequences >= 0 && length >= 0 && top_k >= 1 && capacity >= 0, "%s: %d sequences of %d x %d slots, capacity %d", who,
+              sequences, length, top_k, capacity);
+  DEW_REQUIRE(experts >= 1 && experts <= kMaxExperts, "%s: experts %d (at most %d)", who, experts, kMaxExperts);
+  DEW_REQUIRE(static_cast<int64_t>(sequences) * length * top_k < (1ll << 30), "%s: the slots overflow int32", who);
+  if (sequences == 0 || length == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(indices && admitted, "%s: indices and admitted must not be null", who);
+  hipLaunchKernelGGL(capacity_admit_kernel, dim3(sequences), dim3(kPermuteThreads), sizeof(int32_t) * kPermuteWaves * (experts + 1),
+                     static_cast<hipStream_t>(stream), indices, admitted, length * top_k, experts, capacity);
+  return launched("capacity_admit_kernel");
 }

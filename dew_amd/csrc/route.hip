@@ -33,6 +33,18 @@ __device__ __forceinline__ float exp_f32(float x) {
   return (p * first) * second;
 }
 
+// DeepSeek V4's score sqrt(softplus(x)) (src/dew/nn/moe.py:303-313), formed in float64 (softplus as max(x, 0) +
+// log1p(exp(-|x|)), the square root IEEE) and rounded once to fp32: the CPU oracle's arithmetic for this score.
+__device__ __forceinline__ float sqrt_softplus_f32(float x) {
+  const double wide = static_cast<double>(x);
+  return static_cast<float>(sqrt(fmax(wide, 0.0) + log1p(exp(-fabs(wide)))));
+}
+
+// A score that is a function of its own logit alone (every score function but softmax).
+__device__ __forceinline__ float pointwise_score(int score_function, float logit) {
+  return score_function == DEW_MOE_SCORE_SQRTSOFTPLUS ? sqrt_softplus_f32(logit) : 1.0f / (1.0f + exp_f32(-logit));
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
   for (int offset = 32; offset >= 1; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, kWave));
@@ -78,6 +90,7 @@ struct RouteParams {
   float* weights;
   int32_t* indices;
   int tokens, experts, top_k, score_function, normalize, expert_groups, groups_per_token;
+  int group_by_max;  // a group's score is its best selection (`group_score='max'`), not the sum of its two best
   float scaling;
   float* scores;  // nullable [T, E]: the activated scores, as the router sows them for the balance statistics
   float* log_z;   // nullable [T]: logsumexp of the logits (the z-loss's log partition)
@@ -119,7 +132,7 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
     for (int i = 0; i < kPerLane; ++i) score[i] = score[i] / denom;
   } else {
 #pragma unroll
-    for (int i = 0; i < kPerLane; ++i) score[i] = 1.0f / (1.0f + exp_f32(-logit[i]));
+    for (int i = 0; i < kPerLane; ++i) score[i] = pointwise_score(p.score_function, logit[i]);
   }
 
   // What the router sows beside its choices (src/dew/nn/moe.py:474-479): the scores, and the log partition
@@ -178,7 +191,7 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
           second = v;
         }
       }
-      group_score = first + second;
+      group_score = p.group_by_max ? first : first + second;
     }
     unsigned long long kept = 0ull;
     bool taken = false;
@@ -233,7 +246,7 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
   } else {
     if (owner) {
       weight = p.score_function == DEW_MOE_SCORE_SOFTMAX ? exp_f32(chosen_logit - top) / denom
-                                                         : 1.0f / (1.0f + exp_f32(-chosen_logit));
+                                                         : pointwise_score(p.score_function, chosen_logit);
     }
     if (p.normalize) {
       float total = __shfl(weight, 0, kWave);
@@ -263,29 +276,41 @@ extern "C" int dew_moe_route_sown(const float* logits, const float* bias, int32_
                                   int32_t top_k, int32_t score_function, int32_t normalize, float scaling,
                                   int32_t expert_groups, int32_t groups_per_token, float* weights,
                                   int32_t* indices, float* scores, float* log_z, void* stream) {
+  const dew_moe_router router{experts, top_k, score_function, normalize, scaling, expert_groups, groups_per_token,
+                              DEW_MOE_GROUP_TOP2};
+  return dew_moe_route_with(&router, logits, bias, tokens, weights, indices, scores, log_z, stream);
+}
+
+extern "C" int dew_moe_route_with(const dew_moe_router* router, const float* logits, const float* bias, int32_t tokens,
+                                  float* weights, int32_t* indices, float* scores, float* log_z, void* stream) {
   using namespace dew;
+  DEW_REQUIRE(router, "dew_moe_route: the router's description must not be null");
+  const int experts = router->experts, top_k = router->top_k, score_function = router->score_function;
+  const int expert_groups = router->expert_groups, groups_per_token = router->groups_per_token;
   DEW_REQUIRE(tokens >= 0 && experts >= 1, "dew_moe_route: tokens %d experts %d", tokens, experts);
   DEW_REQUIRE(tokens == 0 || (logits && weights && indices), "dew_moe_route: logits, weights and indices must not be null");
   DEW_REQUIRE(experts <= kWave * kMaxPerLane, "dew_moe_route: at most %d experts, got %d", kWave * kMaxPerLane,
               experts);
   DEW_REQUIRE(top_k >= 1 && top_k <= experts && top_k <= kWave, "dew_moe_route: top_k %d of %d experts (at most %d)",
               top_k, experts, kWave);
-  DEW_REQUIRE(score_function == DEW_MOE_SCORE_SOFTMAX || score_function == DEW_MOE_SCORE_SIGMOID,
-              "dew_moe_route: score_function %d is neither softmax (0) nor sigmoid (1)", score_function);
+  DEW_REQUIRE(score_function == DEW_MOE_SCORE_SOFTMAX || score_function == DEW_MOE_SCORE_SIGMOID || score_function == DEW_MOE_SCORE_SQRTSOFTPLUS,
+              "dew_moe_route: score_function %d is none of softmax (0), sigmoid (1), sqrtsoftplus (2)", score_function);
+  DEW_REQUIRE(router->group_score == DEW_MOE_GROUP_TOP2 || router->group_score == DEW_MOE_GROUP_MAX,
+              "dew_moe_route: group_score %d is neither top2 (0) nor max (1)", router->group_score);
   DEW_REQUIRE(expert_groups >= 1 && expert_groups <= kWave && experts % expert_groups == 0,
               "dew_moe_route: %d experts do not split into %d groups (at most %d)", experts, expert_groups, kWave);
   if (expert_groups > 1) {
     DEW_REQUIRE(groups_per_token >= 1 && groups_per_token <= expert_groups,
                 "dew_moe_route: groups_per_token %d of %d groups", groups_per_token, expert_groups);
-    DEW_REQUIRE(experts / expert_groups >= 2, "dew_moe_route: a group's score sums its two best experts, got %d a group",
-                experts / expert_groups);
+    DEW_REQUIRE(experts / expert_groups >= 2 || router->group_score == DEW_MOE_GROUP_MAX,
+                "dew_moe_route: a group's score sums its two best experts, got %d a group", experts / expert_groups);
     DEW_REQUIRE(top_k <= groups_per_token * (experts / expert_groups),
                 "dew_moe_route: top_k %d exceeds the %d experts of the kept groups", top_k,
                 groups_per_token * (experts / expert_groups));
   }
   if (tokens == 0) return DEW_MOE_OK;
-  RouteParams p{logits, bias, weights, indices, tokens, experts, top_k, score_function, normalize ? 1 : 0,
-                expert_groups, groups_per_token, scaling, scores, log_z};
+  RouteParams p{logits, bias, weights, indices, tokens, experts, top_k, score_function, router->normalize ? 1 : 0,
+                expert_groups, groups_per_token, router->group_score == DEW_MOE_GROUP_MAX ? 1 : 0, router->scaling, scores, log_z};
   const int blocks = (tokens + kRouteWaves - 1) / kRouteWaves;
   const size_t shared = expert_groups > 1 ? sizeof(float) * kRouteWaves * experts : 0;
   const dim3 grid(blocks), block(kWave * kRouteWaves);

@@ -39,12 +39,15 @@ def device_check() -> None:
 
 def route(logits: torch.Tensor, top_k: int, *, score_function: str = "softmax", normalize_weights: bool = True,
           bias: torch.Tensor | None = None, routed_scaling_factor: float = 1.0, expert_groups: int = 1,
-          groups_per_token: int = 1, sown: bool = False):
+          groups_per_token: int = 1, group_score: str = "top2", sown: bool = False):
     """(weights fp32 `[..., k]`, indices int32 `[..., k]`) of router `logits [..., E]` (fp32); with `sown`, also what
     the router sows for the balance statistics: (weights, indices, scores fp32 `[..., E]`, log_z fp32 `[...]`)."""
-    scores = {"softmax": _lib.SCORE_SOFTMAX, "sigmoid": _lib.SCORE_SIGMOID}
+    scores = {"softmax": _lib.SCORE_SOFTMAX, "sigmoid": _lib.SCORE_SIGMOID, "sqrtsoftplus": _lib.SCORE_SQRTSOFTPLUS}
+    group_scores = {"top2": _lib.GROUP_TOP2, "max": _lib.GROUP_MAX}
     if score_function not in scores:
         raise KernelError(f"score_function must be one of {list(scores)}, got {score_function!r}")
+    if group_score not in group_scores:
+        raise KernelError(f"group_score must be one of {list(group_scores)}, got {group_score!r}")
     _device(logits, "logits", torch.float32)
     if bias is not None:
         _device(bias, "bias", torch.float32)
@@ -54,19 +57,30 @@ def route(logits: torch.Tensor, top_k: int, *, score_function: str = "softmax", 
     tokens = logits.numel() // experts
     weights = torch.empty((*logits.shape[:-1], top_k), dtype=torch.float32, device=logits.device)
     indices = torch.empty((*logits.shape[:-1], top_k), dtype=torch.int32, device=logits.device)
-    if sown:
-        activated = torch.empty_like(logits)
-        log_z = torch.empty(logits.shape[:-1], dtype=torch.float32, device=logits.device)
-        _lib.check(_lib.library().dew_moe_route_sown(
-            _ptr(logits), _ptr(bias), tokens, experts, top_k, scores[score_function], int(bool(normalize_weights)),
-            float(routed_scaling_factor), expert_groups, groups_per_token, _ptr(weights), _ptr(indices), _ptr(activated),
-            _ptr(log_z), _stream()), "dew_moe_route_sown")
-        return weights, indices, activated, log_z
-    _lib.check(_lib.library().dew_moe_route(
-        _ptr(logits), _ptr(bias), tokens, experts, top_k, scores[score_function], int(bool(normalize_weights)),
-        float(routed_scaling_factor), expert_groups, groups_per_token, _ptr(weights), _ptr(indices), _stream()),
-        "dew_moe_route")
-    return weights, indices
+    activated = torch.empty_like(logits) if sown else None
+    log_z = torch.empty(logits.shape[:-1], dtype=torch.float32, device=logits.device) if sown else None
+    router = _lib.Router(experts, top_k, scores[score_function], int(bool(normalize_weights)), float(routed_scaling_factor),
+                         expert_groups, groups_per_token, group_scores[group_score])
+    _lib.check(_lib.library().dew_moe_route_with(router, _ptr(logits), _ptr(bias), tokens, _ptr(weights), _ptr(indices),
+                                                 _ptr(activated), _ptr(log_z), _stream()), "dew_moe_route")
+    return (weights, indices, activated, log_z) if sown else (weights, indices)
+
+
+def capacity_admitted(indices: torch.Tensor, num_experts: int, capacity_factor: float) -> torch.Tensor:
+    """`indices [..., length, k]` with every slot past its expert's queue in its sequence replaced by the sentinel id
+    `num_experts` (the reference's `capacity_positions` and the drop it decides, src/dew/nn/moe.py:832-855, 914-919);
+    the capacity is `int(max(ceil(length * k / E) * capacity_factor, capacity_factor))`."""
+    import math
+
+    _device(indices, "indices", torch.int32)
+    if indices.dim() < 2:
+        raise KernelError("capacity dropping takes indices [..., length, top_k]")
+    *leading, length, top_k = indices.shape
+    capacity = int(max(math.ceil(length * top_k / num_experts) * capacity_factor, capacity_factor))
+    admitted = torch.empty_like(indices)
+    _lib.check(_lib.library().dew_moe_capacity_admit(_ptr(indices), math.prod(leading), length, top_k, num_experts, capacity,
+                                                     _ptr(admitted), _stream()), "dew_moe_capacity_admit")
+    return admitted
 
 
 def balance_bias(bias: torch.Tensor, counts: torch.Tensor, rate: float) -> torch.Tensor:
@@ -363,12 +377,15 @@ def gateup_swiglu(x: torch.Tensor, gate: PreparedBank, up: PreparedBank, offsets
     return hidden
 
 
-def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+def swiglu(gate: torch.Tensor, up: torch.Tensor, limit: float | None = None) -> torch.Tensor:
+    """`bf16(bf16(silu(gate)) * up)`; with `limit`, the gate first clamped from above and up both ways by it
+    (the reference's `swiglu_clamped`)."""
     _device(gate, "gate", torch.bfloat16), _device(up, "up", torch.bfloat16)
     if gate.shape != up.shape:
         raise KernelError(f"gate {tuple(gate.shape)} and up {tuple(up.shape)} differ")
     hidden = torch.empty_like(gate)
-    _lib.check(_lib.library().dew_moe_swiglu(_ptr(gate), _ptr(up), _ptr(hidden), gate.numel(), _stream()), "dew_moe_swiglu")
+    _lib.check(_lib.library().dew_moe_swiglu_clamped(_ptr(gate), _ptr(up), 0.0 if limit is None else float(limit), _ptr(hidden),
+                                                     gate.numel(), _stream()), "dew_moe_swiglu")
     return hidden
 
 

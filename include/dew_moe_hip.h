@@ -42,8 +42,8 @@ enum {
                              /* u8 e4m3 [E,N,K]; scales u8 e8m0 [E,N,K/32]. For dew_moe_grouped_gemm_   */
                              /* mxfp8_rows only.                                                        */
   DEW_MOE_W_BF16 = 6,        /* unquantized matrices as the reference holds them: codes bf16 [E,K,N]    */
-                             /* (`experts/*_proj/kernel`, src/dew/nn/moe.py:1231-1235); no scales. With */
-                             /* DEW_MOE_LAYOUT_REFERENCE_KMAJOR, codes bf16 [E,N,K]: the same memory    */
+                             /* (`experts/<name>_proj/kernel`, src/dew/nn/moe.py:1231-1235); no scales. */
+                             /* With DEW_MOE_LAYOUT_REFERENCE_KMAJOR, codes bf16 [E,N,K]: the same memory    */
                              /* read as the transposed matrices (an input gradient's: depth and width   */
                              /* are then the transposed product's).                                     */
   DEW_MOE_W_MXFP4_BLOCKS = 7 /* an MXFP4 checkpoint's own tensors, for dew_moe_prepare_bank only: codes =  */
@@ -66,7 +66,19 @@ typedef struct dew_moe_bank {
   const float* tensor_scale; /* NVFP4 only, else NULL                                                   */
 } dew_moe_bank;
 
-enum { DEW_MOE_SCORE_SOFTMAX = 0, DEW_MOE_SCORE_SIGMOID = 1 };
+enum { DEW_MOE_SCORE_SOFTMAX = 0, DEW_MOE_SCORE_SIGMOID = 1,
+       DEW_MOE_SCORE_SQRTSOFTPLUS = 2 /* DeepSeek V4's sqrt(softplus(logit)), src/dew/nn/moe.py:303-313, 539-540 */ };
+enum { DEW_MOE_GROUP_TOP2 = 0, DEW_MOE_GROUP_MAX = 1 };  /* a group's score: its two best selections' sum, or its best (src/dew/nn/moe.py:557-565) */
+
+/* A router's fixed description (the fields of `Router`, src/dew/nn/moe.py:316-465, that its arithmetic reads). */
+typedef struct dew_moe_router {
+  int32_t experts, top_k;
+  int32_t score_function;  /* DEW_MOE_SCORE_*                                              */
+  int32_t normalize;       /* normalize_weights                                            */
+  float scaling;           /* routed_scaling_factor                                        */
+  int32_t expert_groups, groups_per_token;
+  int32_t group_score;     /* DEW_MOE_GROUP_*                                              */
+} dew_moe_router;
 
 /* ---- introspection (kernels/cutlass/ffi.cu:133-176: dew_cutlass_kernels/kernel_fields/architecture) ---- */
 const char* dew_moe_last_error(void);   /* thread-local, valid until the thread's next failing call      */
@@ -92,6 +104,11 @@ int dew_moe_route_sown(const float* logits, const float* bias /* nullable */, in
                        int32_t top_k, int32_t score_function, int32_t normalize, float scaling,
                        int32_t expert_groups, int32_t groups_per_token, float* weights, int32_t* indices,
                        float* scores /* nullable [T,E] */, float* log_z /* nullable [T] */, void* stream);
+
+/* dew_moe_route_sown from a router's description, which also carries the switches the two entry points above fix
+ * (sqrtsoftplus scores, `group_score='max'`). scores and log_z may be null.                                       */
+int dew_moe_route_with(const dew_moe_router* router /* host */, const float* logits, const float* bias /* nullable */,
+                       int32_t tokens, float* weights, int32_t* indices, float* scores, float* log_z, void* stream);
 
 /* The aux-loss-free balancing step (`load_balance_update` src/dew/nn/moe.py:271-300, applied to the selection bias as
  * `_updated_bias` src/dew/objectives/routing.py:342-345): bias[e] += rate * direction, direction -1 where counts[e]
@@ -135,6 +152,14 @@ int dew_moe_permute_shared(const int32_t* indices /* [T,k] */, int32_t tokens, i
 #define DEW_MOE_PERMUTE_STATIC_BYTES ((size_t)1 << 20)
 int dew_moe_permute_static(const int32_t* indices /* [T,k] */, int32_t tokens, int32_t top_k, int32_t experts,
                            int32_t* sizes, int32_t* offsets, int32_t* order, int32_t* rows, void* stream);
+
+/* Capacity dropping (`capacity_positions` src/dew/nn/moe.py:832-855, applied at :914-919): indices [sequences, length,
+ * top_k]; within each sequence a slot's place in its expert's queue is its rank, in slot order, among the sequence's slots
+ * of that expert; admitted = the id where the place is below `capacity`, else `experts` (the dropped slot's sentinel,
+ * which dew_moe_permute sorts last and outside every group, and whose rows the products write as zeros). The host
+ * computes capacity = int(max(ceil(length * top_k / experts) * capacity_factor, capacity_factor)).               */
+int dew_moe_capacity_admit(const int32_t* indices, int32_t sequences, int32_t length, int32_t top_k, int32_t experts,
+                           int32_t capacity, int32_t* admitted /* [sequences, length, top_k] */, void* stream);
 
 /* offsets[E+1] = exclusive prefix of group sizes[E] (implicit in jax.lax.ragged_dot's group_sizes,
  * src/dew/nn/kernels/xla_products.py:86-115; explicit at src/dew/nn/moe.py:1172).                        */
@@ -331,6 +356,9 @@ int dew_moe_gateup_swiglu(const void* x, const int32_t* gather, const int32_t* o
 
 /* The unfused epilogue alone (src/dew/nn/activations.py:336-356 gated_product('swiglu')).               */
 int dew_moe_swiglu(const void* gate, const void* up, void* hidden, int64_t count, void* stream);
+/* The same with the gate clamped from above and the up projection both ways by `limit` before their product
+ * (`swiglu_clamped`, src/dew/nn/activations.py:327-333: DeepSeek V4's and GLM's experts); limit 0 = none.  */
+int dew_moe_swiglu_clamped(const void* gate, const void* up, float limit, void* hidden, int64_t count, void* stream);
 
 /* ---- Combine (src/dew/nn/moe.py:1328-1333 `_combine`, :1503 shared add) ----------------------------
  * out[t,:] = bf16( sum_j f32(slots[t,j,:]) * weights[t,j] ), fp32 sum in slot order; with `addend`

@@ -795,15 +795,46 @@ def combine(slots, weights, *, dtype="bfloat16"):
     return bf16_round(total) if dtype == "bfloat16" else total
 
 
+def capacity_admitted(indices, num_experts, capacity_factor):
+    """`capacity_positions` and the drop it decides (src/dew/nn/moe.py:832-855, 914-919): `indices [..., length, top_k]`,
+    each leading row one sequence; a slot's place is its rank, in slot order, among its sequence's slots of the same
+    expert; a queue keeps `int(max(ceil(length * top_k / E) * capacity_factor, capacity_factor))` places, and a slot
+    past them takes the sentinel id E. Written as the plain double loop (the definition), not as the reference's
+    argsort arithmetic. Returns (admitted ids, capacity)."""
+    import math
+
+    indices = np.asarray(indices)
+    *_, length, top_k = indices.shape
+    capacity = int(max(math.ceil(length * top_k / num_experts) * capacity_factor, capacity_factor))
+    flat = indices.reshape(-1, length * top_k)
+    admitted = flat.copy()
+    for sequence in range(flat.shape[0]):
+        queued = np.zeros(num_experts + 1, np.int64)
+        for slot in range(flat.shape[1]):
+            expert = flat[sequence, slot]
+            expert = num_experts if expert < 0 or expert >= num_experts else expert
+            if expert == num_experts or queued[expert] >= capacity:
+                admitted[sequence, slot] = num_experts
+            queued[expert] += 1
+    return admitted.reshape(indices.shape).astype(np.int32), capacity
+
+
 def expert_mlp(x, weights, indices, gate_w, up_w, down_w, *, dtype="bfloat16", factors=(None, None, None),
-               limit=None):
+               limit=None, capacity_factor=None):
     """`ExpertMLP.__call__` (src/dew/nn/moe.py:1335-1353) on one device: sort, gather, paired gate/up
     products, SwiGLU, down product scattered to slot order, combine. The matrices are the dequantized
-    `[E, depth, width]` values. Returns (out [T, D], trace dict of the intermediates)."""
+    `[E, depth, width]` values; `indices [T, k]`, or `[..., length, k]` with `capacity_factor` (each leading row a
+    sequence whose experts' queues drop their slots past the capacity: a dropped slot's row is zero). Returns
+    (out [T, D], trace dict of the intermediates)."""
     x = np.asarray(x, F32)
     experts = gate_w.shape[0]
+    if capacity_factor is not None:
+        indices, _ = capacity_admitted(indices, experts, capacity_factor)
+    indices = np.asarray(indices).reshape(-1, np.asarray(indices).shape[-1])
+    x = x.reshape(-1, x.shape[-1])
+    weights = np.asarray(weights).reshape(indices.shape)
     plan = sorted_by_expert(indices, experts)
-    rows = x[plan["rows"]]
+    rows = x[plan["rows"]]   # (rows past the groups, the dropped slots', are multiplied by no matrix: `grouped_matmul` leaves them zero)
     gate = grouped_matmul(rows, gate_w, plan["sizes"], dtype=dtype, factor=factors[0])
     up = grouped_matmul(rows, up_w, plan["sizes"], dtype=dtype, factor=factors[1])
     hidden = swiglu(gate, up, dtype=dtype, limit=limit)

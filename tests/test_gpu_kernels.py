@@ -31,6 +31,12 @@ def bf16_np(t):
 
 
 ROUTERS = [
+    ("sqrtsoftplus-64-top6", 64, 6, dict(score_function="sqrtsoftplus", normalize_weights=True, routed_scaling_factor=2.5), True, 301),
+    ("sqrtsoftplus-256-top8-raw", 256, 8, dict(score_function="sqrtsoftplus", normalize_weights=False), False, 77),
+    ("softmax-64-top4-groups-by-max", 64, 4, dict(score_function="softmax", normalize_weights=False, routed_scaling_factor=2.5,
+                                                  expert_groups=4, groups_per_token=2, group_score="max"), False, 500),
+    ("sigmoid-32-top2-single-expert-groups", 32, 2, dict(score_function="sigmoid", normalize_weights=True, expert_groups=32,
+                                                         groups_per_token=4, group_score="max"), True, 40),
     ("softmax-8-top2", 8, 2, dict(score_function="softmax", normalize_weights=True), False, 1000),
     ("softmax-128-top8", 128, 8, dict(score_function="softmax", normalize_weights=True), False, 777),
     ("softmax-128-top8-raw", 128, 8, dict(score_function="softmax", normalize_weights=False), False, 130),
@@ -82,11 +88,14 @@ def test_router_reproduces_the_reference_fixtures_on_the_device(ops):
     from conftest import golden
     for name, settings in (("mixtral", dict(score_function="softmax", normalize_weights=True)),
                            ("deepseek", dict(score_function="sigmoid", normalize_weights=True, routed_scaling_factor=2.5,
-                                             expert_groups=4, groups_per_token=2))):
+                                             expert_groups=4, groups_per_token=2)),
+                           ("deepseek_v2", dict(score_function="softmax", normalize_weights=False, routed_scaling_factor=2.5,
+                                                expert_groups=4, groups_per_token=2, group_score="max")),
+                           ("deepseek_v4", dict(score_function="sqrtsoftplus", normalize_weights=True, routed_scaling_factor=2.5))):
         held = golden(f"moe/{name}.npz")
         hidden = held["hidden"].reshape(-1, 16)
         logits = oracle.router_logits(hidden, held["mlp.gate.weight"].T)
-        bias = held.get("mlp.gate.e_score_correction_bias") if name == "deepseek" else None
+        bias = held.get("mlp.gate.e_score_correction_bias") if name in ("deepseek", "deepseek_v4") else None
         k = held["router_indices"].shape[-1]
         weights, indices = ops.route(torch.from_numpy(logits).cuda(), k,
                                      bias=None if bias is None else torch.from_numpy(bias).cuda(), **settings)
@@ -536,3 +545,35 @@ def test_group_sizes_in_place_of_their_prefix_give_the_same_products(ops, quant)
                 assert torch.equal(ops.gateup_swiglu(xd, pb, pu, None, sizes=sd, gather=gather, rows=padded), want)
         assert torch.equal(gemm.gemm(xd, pb, sd, gather=gather[:rows]), ops.grouped_gemm(xd, pb, od, gather=gather[:rows]))
         assert torch.equal(gemm.gemm(xd, pb, sd, paired=pu, epilogue="swiglu"), ops.gateup_swiglu(xd, pb, pu, od, rows=rows))
+
+
+
+def test_the_clamped_swiglu_kernel_matches_the_oracle(ops):
+    """`swiglu_clamped`: the gate from above and the up projection both ways, on every bf16 gate against a few ups, for
+    a limit that is a bf16 (1.0) and one that is not (0.3, which enters as the bf16 nearest it)."""
+    gate = oracle.bf16_from_bits(np.arange(65536, dtype=np.uint16))
+    gate = gate[np.isfinite(gate)]
+    gate = np.concatenate([gate, np.zeros(-gate.size % 8, np.float32)])
+    up = np.resize(np.array([1.0, -0.75, 3.140625, 1e-3, 100.0, 2 ** -20, -7.0, 0.5], np.float32), gate.shape)
+    for limit in (1.0, 0.3):
+        rounded = float(torch.tensor(limit).to(torch.bfloat16))
+        want = oracle.swiglu(gate, up, limit=rounded)
+        got = bf16_np(ops.swiglu(torch.from_numpy(gate).to(torch.bfloat16).cuda(), torch.from_numpy(up).to(torch.bfloat16).cuda(), limit))
+        mismatched = (got != want) & ~(np.isnan(got) & np.isnan(want))
+        assert mismatched.mean() < 2e-3                    # the hardware exponential against the library's: a last bf16 bit, rarely
+        assert np.abs(got - want)[mismatched].max(initial=0) <= 2 ** -7 * np.abs(want)[mismatched].max(initial=1)
+        assert np.abs(got).max() <= rounded * 100.0 + 1.0  # |silu(min(g, limit)) * clip(u)| is bounded by limit * max|u|
+
+
+@pytest.mark.parametrize("sequences,length,k,experts,factor", [(1, 64, 2, 8, 1.0), (3, 100, 4, 16, 0.5), (2, 700, 8, 64, 1.25),
+                                                               (5, 33, 2, 4, 2.0), (1, 3000, 6, 512, 1.0), (4, 1, 2, 8, 1.0)])
+def test_capacity_dropping_keeps_each_queues_first_places(ops, sequences, length, k, experts, factor):
+    rng = np.random.default_rng(sequences * 7 + length)
+    skew = rng.random(experts) ** 3
+    indices = np.stack([np.stack([rng.choice(experts, size=k, replace=False, p=skew / skew.sum()) for _ in range(length)])
+                        for _ in range(sequences)]).astype(np.int32)
+    want, capacity = oracle.capacity_admitted(indices, experts, factor)
+    got = ops.capacity_admitted(torch.from_numpy(indices).cuda(), experts, factor).cpu().numpy()
+    assert np.array_equal(got, want)
+    kept = got != experts
+    assert kept.any() and (factor > 1.0 or length == 1 or (~kept).any())   # at factors up to 1 the skewed routing overflows some queue

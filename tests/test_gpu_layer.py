@@ -272,3 +272,39 @@ def test_unquantized_bf16_experts_run_through_the_layer_as_plain_tensors():
     want = oracle.grouped_matmul(dy.float().cpu().numpy(), gate.float().cpu().numpy().transpose(0, 2, 1), sizes)
     assert np.abs(copied.float().cpu().numpy() - want).max() <= 2.0 ** -7 * np.abs(want).max()
 
+
+
+def test_the_clamped_experts_reproduce_the_references_deepseek_v4_output_and_capacity_drops_rows():
+    """DeepSeek V4's experts (`swiglu_limit` 1.0) on the reference's own fixture: its fp32 matrices held as bf16 banks,
+    the recorded routing, against the oracle in bf16 and (within bf16's grain) the recorded fp32 output. Then the same
+    experts with a capacity factor: the dropped slots' rows come back zero, as the oracle's."""
+    from conftest import golden
+
+    from dew_amd import formats, moe
+
+    tensors = golden("moe/deepseek_v4.npz")
+    hidden = torch.from_numpy(tensors["hidden"].reshape(-1, 16))
+    pad = lambda m: np.pad(m, [(0, 0), (0, 128 - m.shape[1]), (0, 128 - m.shape[2])])   # the kernels' least matrix is 128 x 128
+    mats = [pad(np.stack([tensors[f"mlp.experts.{e}.{p}.weight"].T for e in range(8)])) for p in ("gate_proj", "up_proj", "down_proj")]
+    banks = [formats.Bf16(torch.from_numpy(m).to(torch.bfloat16).cuda()) for m in mats]
+    decoded = [bank.weights.float().cpu().numpy() for bank in banks]
+    x = torch.nn.functional.pad(hidden, (0, 112)).to(torch.bfloat16)
+    weights, indices = torch.from_numpy(tensors["router_weights"]), torch.from_numpy(tensors["router_indices"]).to(torch.int32)
+    variables = {"params": {}, "quantization": {f"{n}_proj": {"kernel": bank} for n, bank in zip(("gate", "up", "down"), banks)}}
+    experts = moe.ExpertMLP(8, 128, 128, swiglu_limit=1.0)
+    got = experts.apply(variables, x.cuda(), weights.cuda(), indices.cuda()).float().cpu().numpy()
+    want, _ = oracle.expert_mlp(x.float().numpy(), weights.numpy(), indices.numpy(), *decoded, limit=1.0)
+    by_max, by_element = oracle.relative_errors(got, want)
+    assert by_max <= TOLERANCE and by_element <= TOLERANCE
+    recorded = tensors["experts_output"].reshape(-1, 16)
+    assert np.abs(got[:, :16] - recorded).max() <= 2e-2 * np.abs(recorded).max()       # bf16 operands against the fp32 record
+    unclamped = moe.ExpertMLP(8, 128, 128).apply(variables, x.cuda(), weights.cuda(), indices.cuda()).float().cpu().numpy()
+    assert np.abs(unclamped[:, :16] - recorded).max() > 1.0
+
+    dropping = moe.ExpertMLP(8, 128, 128, swiglu_limit=1.0, capacity_factor=0.5)
+    shaped = indices.reshape(1, *indices.shape)                                        # one sequence
+    got = dropping.apply(variables, x.cuda().reshape(1, *x.shape), weights.cuda().reshape(1, *weights.shape), shaped.cuda())
+    want, trace = oracle.expert_mlp(x.float().numpy(), weights.numpy(), shaped.numpy(), *decoded, limit=1.0, capacity_factor=0.5)
+    assert trace["sizes"].sum() < indices.numel()                                      # something was dropped
+    by_max, by_element = oracle.relative_errors(got.float().cpu().numpy().reshape(want.shape), want)
+    assert by_max <= TOLERANCE and by_element <= TOLERANCE

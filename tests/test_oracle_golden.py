@@ -331,3 +331,33 @@ def test_the_sort_with_a_shared_expert_by_brute_force():
     plain = oracle.sorted_by_expert(np.array([[2, 0], [0, 1], [1, 0]], np.int32), 3)
     with_shared = oracle.sorted_with_shared(np.array([[2, 0], [0, 1], [1, 0]], np.int32), 3, 3)
     assert with_shared["order"][:6].tolist() == plain["order"].tolist() and with_shared["sizes"][:3].tolist() == plain["sizes"].tolist()
+
+
+def test_capacity_dropping_is_the_references_argsort_arithmetic():
+    """`capacity_admitted` is written as the definition (a queue per sequence and expert, in slot order); the
+    reference computes the same places by a stable argsort, a bincount and a cumsum (src/dew/nn/moe.py:845-855).
+    Restated here with NumPy's own stable sort, the two agree on random routings, and a hand case pins both."""
+    import math
+
+    def by_argsort(indices, experts, factor):
+        *_, length, top_k = indices.shape
+        capacity = int(max(math.ceil(length * top_k / experts) * factor, factor))
+        flat = indices.reshape(-1, length * top_k)
+        order = np.argsort(flat, axis=-1, kind="stable")
+        queued = np.take_along_axis(flat, order, axis=-1)
+        counts = np.stack([np.bincount(row, minlength=experts)[:experts] for row in flat])
+        starts = np.cumsum(counts, axis=-1) - counts
+        places = np.arange(length * top_k) - np.take_along_axis(starts, queued, axis=-1)
+        positions = np.zeros_like(flat)
+        np.put_along_axis(positions, order, places, axis=-1)
+        return np.where(positions.reshape(indices.shape) < capacity, indices, experts), capacity
+
+    hand = np.array([[[0, 1], [0, 2], [0, 1], [1, 0]]], np.int32)       # expert 0 is asked for four times, capacity 2
+    admitted, capacity = oracle.capacity_admitted(hand, 4, 1.0)
+    assert capacity == 2 and admitted.tolist() == [[[0, 1], [0, 2], [4, 1], [4, 4]]]
+    rng = np.random.default_rng(8)
+    for sequences, length, k, experts, factor in ((2, 50, 2, 8, 1.0), (3, 17, 3, 5, 0.5), (1, 200, 4, 16, 1.5)):
+        indices = np.stack([np.stack([rng.choice(experts, size=k, replace=False) for _ in range(length)]) for _ in range(sequences)]).astype(np.int32)
+        ours, ours_capacity = oracle.capacity_admitted(indices, experts, factor)
+        theirs, theirs_capacity = by_argsort(indices, experts, factor)
+        assert ours_capacity == theirs_capacity and np.array_equal(ours, theirs)
