@@ -434,3 +434,34 @@ extern "C" int dew_moe_prepare_bank(const dew_moe_bank* ref, void* prepared, dew
   }
   return DEW_MOE_OK;
 }
+
+extern "C" int dew_moe_prepared_view(int32_t format, int32_t experts, int32_t depth, int32_t width, const void* prepared,
+                                     const void* external_scales, const float* tensor_scale, dew_moe_bank* out) {
+  using namespace dew;
+  const char* who = "dew_moe_prepared_view";
+  DEW_REQUIRE(prepared && out, "%s: the prepared buffer and out must not be null", who);
+  DEW_REQUIRE(experts >= 1 && depth >= 1 && width >= 1, "%s: bank [%d, %d, %d]", who, experts, depth, width);
+  const uint8_t* base = static_cast<const uint8_t*>(prepared);
+  *out = dew_moe_bank{format, DEW_MOE_LAYOUT_PREPARED, experts, depth, width, base, nullptr, nullptr};
+  switch (format) {
+    case DEW_MOE_W_FP8_BLOCK:
+    case DEW_MOE_W_MXFP8:
+      out->scales = base + codes_bytes(format, experts, depth, width);
+      break;
+    case DEW_MOE_W_NVFP4:
+    case DEW_MOE_W_MXFP4:
+      DEW_REQUIRE(tensor_scale, "%s: an FP4 bank needs its tensor scales", who);
+      out->scales = base + codes_bytes(DEW_MOE_W_NVFP4, experts, depth, width);
+      out->tensor_scale = tensor_scale;
+      break;
+    case DEW_MOE_W_FP8_CHANNEL:
+      DEW_REQUIRE(external_scales, "%s: a per-channel FP8 bank's scales [E, N] stay outside the prepared buffer", who);
+      out->scales = external_scales;
+      break;
+    case DEW_MOE_W_BF16:
+      break;
+    default:
+      return fail(DEW_MOE_EINVAL, "%s: %d is no format a prepared bank has", who, format);
+  }
+  return DEW_MOE_OK;
+}

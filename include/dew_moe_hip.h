@@ -180,6 +180,14 @@ size_t dew_moe_prepared_bytes(int32_t format, int32_t experts, int32_t depth, in
 int dew_moe_prepare_bank(const dew_moe_bank* reference, void* prepared, dew_moe_bank* out /* host */,
                          void* stream);
 
+/* The descriptor of a bank prepared earlier, from the buffer alone: for a binding that holds the prepared bytes as an
+ * opaque array (an XLA buffer) and the bank's format tag and extents as static attributes. `format` is the PREPARED
+ * bank's (out->format of dew_moe_prepare_bank); external_scales: a per-channel FP8 bank's f32 [E, N], else null;
+ * tensor_scale: an FP4 bank's f32 [E] (for a bank prepared from DEW_MOE_W_MXFP4_BLOCKS, the ones that call wrote:
+ * out->tensor_scale, which lies inside the prepared buffer), else null. Host only, no launch.                  */
+int dew_moe_prepared_view(int32_t format, int32_t experts, int32_t depth, int32_t width, const void* prepared,
+                          const void* external_scales, const float* tensor_scale, dew_moe_bank* out /* host */);
+
 /* Tuning and testing knob (no counterpart in the reference): every later grouped product launched by the CALLING
  * THREAD uses block tiles of `rows` rows (32, 64, 128 or 256; 256 with FP4 banks whose width is whole 256s); 0, the
  * default, chooses per launch from the rows, experts and width. The setting is thread-local: other threads' launches
