@@ -108,6 +108,7 @@ class Stepper:
         self.dense_offsets = torch.tensor([0, tokens], dtype=torch.int32, device=data["x"].device)
         self.events = []
         self.split = split
+        self.fp6 = gemm.SPLIT_SECOND_TERM == "e2m3"   # the library's setting for the split rows' second term
 
     def __call__(self, timed: bool = False):
         torch, ops, case, data = self.torch, self.ops, self.case, self.data
@@ -134,10 +135,10 @@ class Stepper:
         if self.on_split_rows():
             # MXFP4 banks and groups of hundreds of rows: the rows as two e4m3 terms and the scaled matrix instruction;
             # the gate/up launch writes its hidden rows already split, so the only extra pass is the split of x
-            pieces = ops.split_rows(data["x"])
+            pieces = ops.split_rows_fp6(data["x"]) if self.fp6 else ops.split_rows(data["x"])
             if events:
                 events[0].record()
-            hidden = ops.gateup_swiglu_split_out(*pieces, self.gate, self.up, plan.offsets, gather=plan.rows)
+            hidden = ops.gateup_swiglu_split_out(*pieces, self.gate, self.up, plan.offsets, gather=plan.rows, fp6=self.fp6)
             if events:
                 events[1].record()
                 self.events.append(events)
@@ -303,10 +304,11 @@ def measure(config, args, device, sustained, with_cpu_baseline):
         roofline = {"bound": "hbm", "achieved": round(gateup_gbs, 1), "peak": PEAKS["hbm_gbs"], "unit": "GB/s"}
     else:
         roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAKS["bf16_mfma"], "unit": "TFLOP/s",
-                    "peak_note": ("the kernel multiplies each bf16 activation as two e4m3 terms by the stored FP4 codes "
-                                  "(v_mfma_scale_f32_32x32x64_f8f6f4, which runs at the dense fp8 rate, 5.0 PFLOP/s published): "
-                                  "two instruction flops per algorithmic flop, so the algorithm's ceiling is 2.5 PFLOP/s, the "
-                                  "dense bf16 peak; achieved counts algorithmic flops only") if stepper.on_split_rows() else
+                    "peak_note": ("the kernel multiplies each bf16 activation as two terms by the stored FP4 codes "
+                                  "(v_mfma_scale_f32_32x32x64_f8f6f4: the e4m3 term at the dense fp8 rate, 5.0 PFLOP/s published, the "
+                                  "second term at that rate (e4m3) or at the fp6/fp4 rate, 10.1 (e2m3)): two instructions per "
+                                  "algorithmic product; priced against the dense bf16 peak, 2.5 PFLOP/s, the ceiling of two fp8-rate "
+                                  "instructions; achieved counts algorithmic flops only") if stepper.on_split_rows() else
                                  ("dense bf16 MFMA: the kernel multiplies bf16 activations by weights dequantized exactly to "
                                   "bf16 (v_mfma_f32_32x32x16_bf16)"),
                     "frac_of_fp8_peak": round(achieved / PEAKS["fp8_mfma"], 4), "frac_of_fp4_peak": round(achieved / PEAKS["fp4_mfma"], 4),
@@ -315,7 +317,10 @@ def measure(config, args, device, sustained, with_cpu_baseline):
     roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
     if not decode and stepper.on_split_rows():
         roofline["executed"] = {"tflops": round(2 * achieved, 1), "frac_of_fp8_peak": round(2 * achieved / PEAKS["fp8_mfma"], 4),
-                                "note": "instruction flops: both terms' products"}
+                                "note": "instruction flops: both terms' products",
+                                "issue_time_frac": round(achieved / (1.0 / (1.0 / PEAKS["fp8_mfma"] + 1.0 / (PEAKS["fp4_mfma"] if stepper.fp6 else PEAKS["fp8_mfma"]))), 4),
+                                "issue_time_note": "achieved over the rate at which the two instructions of a product issue back to back at "
+                                                   "their published peaks (fp8 + fp8: 2.5 PFLOP/s; fp8 + fp6: 3.34 PFLOP/s)"}
     roofline["traffic"] = measured_traffic(config)
     roofline["traffic_source"] = (f"stored: rocprofv3 --pmc FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 of this command's gate/up launch, "
                                   f"{COUNTED_FROM[config]}; not measured in this run") if config in COUNTED_KIB else None
@@ -325,7 +330,7 @@ def measure(config, args, device, sustained, with_cpu_baseline):
                              "note": "measured in this run by bench_aids' MFMA and copy probes: the rate the chip holds on "
                                      "random data at its power limit, below the published peak"}
     roofline["kernel"] = "grouped_gemm_kernel<paired gate/up + SwiGLU>" + (
-        " on split rows (v_mfma_scale_f32_32x32x64_f8f6f4, two e4m3 terms x FP4)" if stepper.on_split_rows() else "")
+        f" on split rows (v_mfma_scale_f32_32x32x64_f8f6f4, an e4m3 and an {'e2m3' if stepper.fp6 else 'e4m3'} term x FP4)" if stepper.on_split_rows() else "")
     roofline["kernel_ms"] = round(gateup_ms, 4)
 
     result = {
@@ -378,6 +383,8 @@ def main():
     parser.add_argument("--bf16-operands", action="store_true",
                         help="keep MXFP4 banks with groups of hundreds of rows on the bf16 matrix instruction too (the default "
                              "there: rows split into two e4m3 terms and the scaled instruction, the library's own choice)")
+    parser.add_argument("--second-term", choices=["e4m3", "e2m3"], default=None,
+                        help="the split rows' second term in the first product (default: the library's, gemm.SPLIT_SECOND_TERM)")
     parser.add_argument("--separate-shared", action="store_true",
                         help="compute a shared expert as a dense MLP of its own (two more launches), as the reference does, instead "
                              "of as group #E of the routed launches")
@@ -390,8 +397,10 @@ def main():
 
     import torch
 
-    from dew_amd import ops
+    from dew_amd import gemm, ops
 
+    if args.second_term is not None:
+        gemm.SPLIT_SECOND_TERM = args.second_term
     ops.device_check()
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
@@ -419,6 +428,15 @@ def main():
                 print(f"[bench] measuring {config}", file=sys.stderr, flush=True)
                 measured = measure(config, args, device, sustained, with_cpu_baseline=False)
             per_config[config] = measured
+        # the same c2 workload with the split rows' second term in FP6 (gemm.SPLIT_SECOND_TERM = 'e2m3'): the faster, less
+        # exact option, measured in the same run beside the default so that its price in parity stands next to its gain
+        if gemm.SPLIT_SECOND_TERM != "e2m3":
+            print("[bench] measuring c2 with an e2m3 second term", file=sys.stderr, flush=True)
+            held, gemm.SPLIT_SECOND_TERM = gemm.SPLIT_SECOND_TERM, "e2m3"
+            try:
+                per_config["c2_option_e2m3_second_term"] = measure("c2", args, device, sustained, with_cpu_baseline=False)
+            finally:
+                gemm.SPLIT_SECOND_TERM = held
         result["configs"] = per_config
     print(json.dumps(result))
 

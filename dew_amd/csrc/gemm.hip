@@ -62,6 +62,11 @@ constexpr int kFormatMxFp8Window = 20;
 // The kernel gradient of bf16 operands (the reference's `gemm_t`): lhs_t rows [depth, tokens] bf16 and the rhs_t as a
 // DEW_MOE_W_BF16 bank of one expert whose depth is all the tokens; windows in whole 64-token steps.
 constexpr int kFormatBf16Window = 21;
+// kFormatMxSplit with the second term in FP6: rows split by dew_moe_split_rows_fp6 into an e4m3 term and an e2m3 term
+// under one power-of-two scale every 32 depths (the scaled instruction's own granularity). The FP6 x FP4 instruction
+// takes half the cycles of the FP8 x FP4 one, so a product's two instructions take three quarters of the time; the
+// second term is exact only for elements within two binades of their 32-deep block's largest (see split.hip).
+constexpr int kFormatMxSplit6 = 22;
 
 constexpr int BK = 64;
 constexpr int kThreads = 256;
@@ -191,7 +196,7 @@ __device__ __forceinline__ void schedule_phase() {
 // four wavefronts sit WM x WN (1 x 4: side by side along the columns, so no two of them need the same weight
 // bytes); each owns (BM/WM) x (BN/WN) of every matrix as 32 x 32 MFMA tiles.
 template <int FORMAT, int MODE, int BM, int BN, int WM, int WN>
-__global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 && (MODE == kSwigluOfTwo ? 2 : 1) * BN == 256) ? 2 : 1) void grouped_gemm_kernel(GemmParams p) {
+__global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 && ((MODE == kSwigluOfTwo || MODE == kSwigluOfTwoSplit) ? 2 : 1) * BN == 256) ? 2 : 1) void grouped_gemm_kernel(GemmParams p) {
   constexpr bool PAIRED = MODE == kSwigluOfTwo || MODE == kSwigluOfTwoSplit;
   constexpr bool kSplitOut = MODE == kSwigluOfTwoSplit;
   constexpr bool kGated = MODE == kInterleavedGated;
@@ -201,7 +206,8 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   constexpr bool kWindow = FORMAT == kFormatMxFp8Window || FORMAT == kFormatBf16Window;  // a kernel gradient: the same rows for every group, its own depths
   constexpr bool kMxRows = FORMAT == kFormatMxFp8Rows || FORMAT == kFormatMxFp8Window;  // e4m3 rows and weights, one scale per row (column) and 32 depths
   constexpr bool kFp8A = kFp8Rows || kMxRows;           // both operands e4m3 codes: a step is 128 depths
-  constexpr bool kSplit = FORMAT == kFormatMxSplit || FORMAT == kFormatMxSplitBlocks || kFp8A;  // A arrives as 8-bit codes
+  constexpr bool kLo6 = FORMAT == kFormatMxSplit6;      // the second term of a row in FP6 (e2m3), its scale beside it
+  constexpr bool kSplit = FORMAT == kFormatMxSplit || FORMAT == kFormatMxSplitBlocks || kLo6 || kFp8A;  // A arrives as 8-bit codes
   constexpr bool kBlockScales = FORMAT == kFormatMxSplitBlocks || kFp8Rows;
   constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4 || (kSplit && !kFp8A);
   constexpr bool kPow2 = FORMAT == DEW_MOE_W_MXFP4 || (kSplit && !kFp8A);
@@ -223,7 +229,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   // Quantized rows on the full 256 x 256 tile: a step's weights are 64 registers a lane, of which two sets fit
   // beside the accumulators (a load then has most of a 2048-cycle step to land).
   // (bf16 matrices: a step's raw data is twice FP8's, three sets of it fit beside the 256-row tile's accumulators)
-  constexpr int kSets = (kFp8A && BN == 256) ? 2 : (kBf16 || (!kFp4 && BM == 128 && kMatrices * BN == 256)) ? 3 : 4;
+  constexpr int kSets = (kFp8A && BN == 256) ? 2 : (kSplit && !kFp8A && BM == 128) ? 2 : (kBf16 || (!kFp4 && BM == 128 && kMatrices * BN == 256)) ? 3 : 4;
 
   extern __shared__ u32x4_t lds[];  // a ring of three stages of A: BM rows of 128 bytes each
   __shared__ int wave_tiles[4], wave_rows[4];
@@ -383,12 +389,14 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   const int a_pitch = block_scale_pitch(p.depth);
   uint8_t* block_scales = reinterpret_cast<uint8_t*>(lds + kStages * kStageChunks);
   if constexpr (kBlockScales) {
-    static_assert(!kBlockScales || BM == kThreads, "one thread copies one row's scales");
-    const int sorted = row0 + min(tid, valid_rows - 1);
-    const int source = p.gather ? p.gather[sorted] : sorted;
-    const u32x4_t* from = reinterpret_cast<const u32x4_t*>(p.a_scale + static_cast<size_t>(source) * a_pitch);
-    u32x4_t* to = reinterpret_cast<u32x4_t*>(block_scales + tid * a_pitch);
-    for (int piece = 0; piece < a_pitch / 16; ++piece) to[piece] = from[piece];
+    static_assert(!kBlockScales || BM <= kThreads, "one thread copies one row's scales");
+    if (tid < BM) {
+      const int sorted = row0 + min(tid, valid_rows - 1);
+      const int source = p.gather ? p.gather[sorted] : sorted;
+      const u32x4_t* from = reinterpret_cast<const u32x4_t*>(p.a_scale + static_cast<size_t>(source) * a_pitch);
+      u32x4_t* to = reinterpret_cast<u32x4_t*>(block_scales + tid * a_pitch);
+      for (int piece = 0; piece < a_pitch / 16; ++piece) to[piece] = from[piece];
+    }
   }
   int a_block_word[2][kBlockScales ? TI : 1], a_block_byte[kBlockScales ? TI : 1];
   auto load_block_scales = [&](int block) __attribute__((always_inline)) {
@@ -497,6 +505,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   // ---- fragments: slice kk of a step is 16 depths; a lane's are the 8 its weight bytes cover ----
   bf16x8_t a_frag[2][TI], b_frag[2][kTiles];
   i32x8_t a_term[2][kSplit ? TI : 1];  // split activations: [0] the hi term of a step, [1] its lo term
+  int a_lo_scale[kLo6 ? TI : 1];       // an FP6 second term's e8m0 scale of the lane's 32 depths (it lies behind the codes)
   float fp4_scale[kTiles];
   // a term of a 32-depth block is 32 bytes: the lane's block lane / 32 of the step holds hi in its chunks 0-1, lo in 2-3
   // The lane's four chunks of its first row tile, as chunk indices into a stage: computed once, so that a phase's
@@ -514,9 +523,15 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
       for (int i = 0; i < TI; ++i) {
         const u32x4_t first = first_piece[32 * i * kChunksPerRow];  // the swizzle reads a row's low four bits only
         const u32x4_t second = second_piece[32 * i * kChunksPerRow];
-        a_term[term.value][i] = i32x8_t{static_cast<int>(first[0]), static_cast<int>(first[1]), static_cast<int>(first[2]),
-                                        static_cast<int>(first[3]), static_cast<int>(second[0]), static_cast<int>(second[1]),
-                                        static_cast<int>(second[2]), static_cast<int>(second[3])};
+        if constexpr (kLo6 && term.value == 1) {  // 24 bytes of e2m3 codes, then the scale's dword
+          a_term[1][i] = i32x8_t{static_cast<int>(first[0]), static_cast<int>(first[1]), static_cast<int>(first[2]),
+                                 static_cast<int>(first[3]), static_cast<int>(second[0]), static_cast<int>(second[1]), 0, 0};
+          a_lo_scale[i] = static_cast<int>(second[2]);
+        } else {
+          a_term[term.value][i] = i32x8_t{static_cast<int>(first[0]), static_cast<int>(first[1]), static_cast<int>(first[2]),
+                                          static_cast<int>(first[3]), static_cast<int>(second[0]), static_cast<int>(second[1]),
+                                          static_cast<int>(second[2]), static_cast<int>(second[3])};
+        }
       }
     }
   };
@@ -569,11 +584,11 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   // Split activations: one scaled instruction multiplies 64 depths of one term by the stored FP4 codes under
   // both operands' power-of-two scales; the block scale byte is the e4m3 of a normal power of two, 2^(field - 7).
   int unscalable = 0;  // quantized rows: mantissa bits met in a weight block scale (the instruction takes powers of two only)
-  auto multiply_term = [&](auto set, auto term, int step) __attribute__((always_inline)) {
+  auto multiply_term = [&](auto set, auto term, int step, auto buffer) __attribute__((always_inline)) {
     if constexpr (kSplit) {
-      // block scales: of the unrolled four steps, steps 0, 1 read set 0 and steps 2, 3 set 1 (a scale holds for two
-      // 64-deep steps); quantized rows' 128-deep steps alternate
-      constexpr int kBuffer = kFp8A ? set.value % 2 : (set.value / 2) % 2;
+      // block scales: of the unrolled four steps, steps 0, 1 read buffer 0 and steps 2, 3 buffer 1 (a scale holds for
+      // two 64-deep steps); quantized rows' 128-deep steps alternate
+      constexpr int kBuffer = buffer.value;
 #pragma unroll
       for (int m = 0; m < kMatrices; ++m)
 #pragma unroll
@@ -607,9 +622,13 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
             const int b_scale = static_cast<int>(((s_regs[set.value][m * TJ + j] >> 3) & 15u) + 120u);
 #pragma unroll
             for (int i = 0; i < TI; ++i) {
-              acc[m][i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_term[term.value][i], codes, acc[m][i][j], 0, 4, term.value,
-                                                                          kBlockScales ? a_block_word[kBuffer][i] : a_scale_word[i], 0,
-                                                                          b_scale);
+              if constexpr (kLo6 && term.value == 1) {  // FP6 (e2m3) x FP4 under the term's own scale
+                acc[m][i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_term[1][i], codes, acc[m][i][j], 2, 4, 0, a_lo_scale[i], 0, b_scale);
+              } else {
+                acc[m][i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_term[term.value][i], codes, acc[m][i][j], 0, 4, term.value,
+                                                                            kBlockScales ? a_block_word[kBuffer][i] : a_scale_word[i], 0,
+                                                                            b_scale);
+              }
             }
           }
         }
@@ -653,7 +672,10 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   constexpr int kWaitLanded = (kYounger & 0xF) | (7 << 4) | (0 << 8) | ((kYounger >> 4) << 14);
   constexpr int kWaitAll = (0 & 0xF) | (7 << 4) | (0 << 8) | (0 << 14);  // vmcnt(0) lgkmcnt(0)
   int stage_index = 0;  // s % 3
-  auto iterate = [&](auto set, int step, auto last_steps) __attribute__((always_inline)) {
+  // `quarter`: the step's place among four consecutive steps, which is what the block scales' two buffers go by (it is
+  // the register set where there are four of them).
+  auto iterate = [&](auto set, auto quarter, int step, auto last_steps) __attribute__((always_inline)) {
+    constexpr std::integral_constant<int, kFp8A ? set.value % 2 : (quarter.value / 2) % 2> scale_buffer{};
     constexpr std::integral_constant<int, (set.value + 1) % kSets> following{};
     constexpr std::integral_constant<int, (set.value + kSets - 1) % kSets> filling{};
     const int next_index = stage_index == kStages - 1 ? 0 : stage_index + 1;
@@ -678,7 +700,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
       // younger than the last A load of the step before: only this phase's loads are sure to be
       constexpr int kSplitWait = (kSplitLoads & 0xF) | (7 << 4) | (0 << 8) | ((kSplitLoads >> 4) << 14);
       fetch_term(current, c1);
-      multiply_term(set, c0, step);
+      multiply_term(set, c0, step, scale_buffer);
       load_a(fill, ahead_a, c0, ah);
       load_a_scales(fill_index, ahead_a);  // (MXFP8 rows: the step's scale dwords, with this phase's loads)
       load_b(filling, ahead_b, c0, bh);
@@ -697,11 +719,11 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
         load_block_scales(min(step + 1, steps - 1));
         form_block_words(std::integral_constant<int, 1 - set.value % 2>{});
       } else {
-        if constexpr (kBlockScales && set.value % 2 == 0) load_block_scales(min(step / 2 + 1, p.depth / 128 - 1));
-        if constexpr (kBlockScales && set.value % 2 == 1) form_block_words(std::integral_constant<int, 1 - (set.value / 2) % 2>{});
+        if constexpr (kBlockScales && quarter.value % 2 == 0) load_block_scales(min(step / 2 + 1, p.depth / 128 - 1));
+        if constexpr (kBlockScales && quarter.value % 2 == 1) form_block_words(std::integral_constant<int, 1 - (quarter.value / 2) % 2>{});
       }
       fetch_term(next, c0);
-      multiply_term(set, c1, step);
+      multiply_term(set, c1, step, scale_buffer);
       load_a(fill, ahead_a, ah, a4);
       load_b(filling, ahead_b, bh, b4);
       constexpr int kSecondLoads = kRowLoads - ah.value + (kTiles - bh.value) * kLoadsPerTile;
@@ -778,19 +800,17 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
     dequantize(c0, c0, c0, 0);
   }
   int step = 0;
-  for (; step + kSets <= steps; step += kSets) {
-    iterate(c0, step, std::false_type{});
-    iterate(c1, step + 1, std::false_type{});
-    if constexpr (kSets >= 3) iterate(c2, step + 2, std::false_type{});
-    if constexpr (kSets == 4) iterate(c3, step + 3, std::false_type{});
+  // unrolled so that the register sets, and the block scales' buffers (which turn every four steps), are constants
+  constexpr int kUnroll = (kBlockScales && !kFp8A && kSets < 4) ? 4 : kSets;
+  static_assert(kUnroll % kSets == 0, "whole rounds of the register sets");
+  for (; step + kUnroll <= steps; step += kUnroll) {
+    static_range<0>(std::make_integer_sequence<int, kUnroll>{}, [&](auto at) {
+      iterate(std::integral_constant<int, decltype(at)::value % kSets>{}, at, step + decltype(at)::value, std::false_type{});
+    });
   }
-  if (step < steps) iterate(c0, step++, std::true_type{});  // the last steps % kSets steps
-  if constexpr (kSets >= 3) {
-    if (step < steps) iterate(c1, step++, std::true_type{});
-  }
-  if constexpr (kSets == 4) {
-    if (step < steps) iterate(c2, step++, std::true_type{});
-  }
+  static_range<0>(std::make_integer_sequence<int, kUnroll - 1>{}, [&](auto at) {  // the last steps % kUnroll steps
+    if (step < steps) iterate(std::integral_constant<int, decltype(at)::value % kSets>{}, at, step++, std::true_type{});
+  });
   __builtin_amdgcn_s_waitcnt(kWaitAll);  // the clamped tail loads still target the LDS
 
   // ---- epilogue: acc[..][q] is row 8 (q / 4) + 4 (lane / 32) + q % 4, column lane % 32 of its 32 x 32 tile.
@@ -1194,6 +1214,7 @@ extern "C" int dew_moe_grouped_gemm_split_blocks(const void* x_split, const uint
   GemmParams p{};
   if (int rc = fill_single(who, p, x_split, gather, offsets, w, bias, scatter, out, rows)) return rc;
   p.a_scale = x_scales;
+  if (forced_tile_rows == 128) return launch_tile<kFormatMxSplitBlocks, kPlain, 128, 256, 2, 2>(who, p, static_cast<hipStream_t>(stream));
   return launch_tile<kFormatMxSplitBlocks, kPlain, 256, 256, 2, 2>(who, p, static_cast<hipStream_t>(stream));
 }
 
@@ -1347,7 +1368,48 @@ extern "C" int dew_moe_gateup_swiglu_split_out(const void* x_split, const uint8_
   p.depth = gate->depth;
   p.width = gate->width;
   p.rows = rows;
-  return launch_tile<kFormatMxSplit, kSwigluOfTwoSplit, 256, 128, 2, 2>(who, p, static_cast<hipStream_t>(stream));
+  // 128-row tiles at two blocks a CU (256 registers a lane, two weight register sets): one block's tile search, first
+  // loads and epilogue run under the other's main loop. Measured on 8 experts x 4096 rows of 4096 x 14336: 5.18 ms
+  // against 5.30 ms for 256-row tiles at one block a CU, the same bits. (The plain product below stays on 256-row
+  // tiles: 2.55 against 2.61 ms.)
+  if (forced_tile_rows == 256) return launch_tile<kFormatMxSplit, kSwigluOfTwoSplit, 256, 128, 2, 2>(who, p, static_cast<hipStream_t>(stream));
+  return launch_tile<kFormatMxSplit, kSwigluOfTwoSplit, 128, 128, 2, 2>(who, p, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int dew_moe_gateup_swiglu_split_fp6_out(const void* x_split, const uint8_t* x_scale, const int32_t* gather,
+                                                   const int32_t* offsets, const dew_moe_bank* gate, const dew_moe_bank* up,
+                                                   void* hidden_split, uint8_t* hidden_scales, int32_t rows, void* stream) {
+  using namespace dew;
+  const char* who = "dew_moe_gateup_swiglu_split_fp6_out";
+  if (int rc = check_bank(who, gate, "gate")) return rc;
+  if (int rc = check_bank(who, up, "up")) return rc;
+  DEW_REQUIRE(gate->format == DEW_MOE_W_MXFP4 && up->format == DEW_MOE_W_MXFP4,
+              "%s: split activations multiply MXFP4 banks (power-of-two block scales); these are formats %d and %d", who,
+              gate->format, up->format);
+  DEW_REQUIRE(gate->experts == up->experts && gate->depth == up->depth && gate->width == up->width,
+              "%s: gate [%d, %d, %d] and up [%d, %d, %d] differ", who, gate->experts, gate->depth, gate->width, up->experts,
+              up->depth, up->width);
+  DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
+  if (rows == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(x_split && x_scale && offsets && hidden_split && hidden_scales,
+              "%s: x_split, x_scale, offsets, hidden_split and hidden_scales must not be null", who);
+  DEW_REQUIRE(aligned16(x_split) && aligned16(hidden_split), "%s: x_split and hidden_split must be 16-byte aligned", who);
+  GemmParams p{};
+  p.x = static_cast<const bf16_t*>(x_split);
+  p.a_scale = x_scale;
+  p.gather = gather;
+  p.offsets = offsets;
+  p.w0 = BankView{static_cast<const uint8_t*>(gate->codes), gate->scales, gate->tensor_scale};
+  p.w1 = BankView{static_cast<const uint8_t*>(up->codes), up->scales, up->tensor_scale};
+  p.out = static_cast<bf16_t*>(hidden_split);
+  p.out_scale = hidden_scales;
+  p.experts = gate->experts;
+  p.depth = gate->depth;
+  p.width = gate->width;
+  p.rows = rows;
+  // (128-row tiles, two blocks a CU: see dew_moe_gateup_swiglu_split_out)
+  if (forced_tile_rows == 256) return launch_tile<kFormatMxSplit6, kSwigluOfTwoSplit, 256, 128, 2, 2>(who, p, static_cast<hipStream_t>(stream));
+  return launch_tile<kFormatMxSplit6, kSwigluOfTwoSplit, 128, 128, 2, 2>(who, p, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int dew_moe_gateup_interleaved(const void* x, const int32_t* gather, const int32_t* offsets,

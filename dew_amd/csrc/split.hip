@@ -71,7 +71,105 @@ __global__ __launch_bounds__(64 * kSplitWaves) void split_rows_kernel(const bf16
   }
 }
 
+// The same rows with the second term in FP6: x = s hi + t lo, hi = e4m3(x / s) under the row's scale s as above and
+// lo = e2m3((x - s hi) / t) under t, one power of two for every 32 depths: the least that brings the block's largest
+// remainder within e2m3's range (7.5). A remainder is a multiple of its element's bf16 spacing; e2m3 holds it exactly
+// where that spacing is at least t / 8, that is for the elements within two binades of their block's largest
+// magnitude, and to within t / 16 (2^-10 of the block's largest magnitude, or less) for the smaller ones. A lane
+// converts one block: v_cvt_scalef32_2xpk16_fp6_f32 packs its 32 remainders (the even depths in its first operand,
+// the odd ones in its second: it interleaves them). A row's 64 depths are 128 bytes, [group 0: 32 bytes of hi codes,
+// 24 of lo codes, the lo scale's e8m0 byte in a dword, 4 unused][group 1 alike]; the hi codes of lane group g are depths
+// 16 g .. 16 g + 15 and 32 + 16 g .. 47 + 16 g, its lo codes depths 32 g .. 32 g + 31 (the instruction's own orders).
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(6))) uint32_t u32x6_t;
+
+__global__ __launch_bounds__(64 * kSplitWaves) void split_rows_fp6_kernel(const bf16_t* __restrict__ x, uint8_t* __restrict__ split,
+                                                                         uint8_t* __restrict__ scale, int rows, int depth) {
+  const int lane = threadIdx.x % 64;
+  const int row = blockIdx.x * kSplitWaves + threadIdx.x / 64;
+  if (row >= rows) return;
+  const bf16_t* source = x + static_cast<size_t>(row) * depth;
+  uint32_t largest = 0;
+  for (int chunk = lane; chunk < depth / 8; chunk += 64) {
+    const u32x4_t words = *reinterpret_cast<const u32x4_t*>(source + chunk * 8);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      largest = max(largest, (words[i] >> 7) & 0xFFu);
+      largest = max(largest, (words[i] >> 23) & 0xFFu);
+    }
+  }
+#pragma unroll
+  for (int offset = 32; offset >= 1; offset >>= 1) largest = max(largest, static_cast<uint32_t>(__shfl_xor(static_cast<int>(largest), offset, 64)));
+  const int field = min(max(static_cast<int>(largest), 16), 254);
+  const int hi_byte = field - 7;
+  if (lane == 0) scale[row] = static_cast<uint8_t>(hi_byte);
+  const float inverse = __uint_as_float(static_cast<uint32_t>(254 - hi_byte) << 23);  // 1 / s
+  uint8_t* target = split + static_cast<size_t>(row) * depth * 2;
+  for (int block = lane; block < depth / 32; block += 64) {
+    float rest[32];
+    uint32_t hi[8];
+    float most = 0.0f;
+#pragma unroll
+    for (int piece = 0; piece < 4; ++piece) {  // 8 depths a piece
+      const u32x4_t words = *reinterpret_cast<const u32x4_t*>(source + block * 32 + piece * 8);
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(words[i] << 16) * inverse;
+        v[2 * i + 1] = __uint_as_float(words[i] & 0xFFFF0000u) * inverse;
+      }
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        uint32_t codes = __builtin_amdgcn_cvt_pk_fp8_f32(v[4 * w], v[4 * w + 1], 0, false);
+        codes = __builtin_amdgcn_cvt_pk_fp8_f32(v[4 * w + 2], v[4 * w + 3], codes, true);
+        hi[2 * piece + w] = codes;
+        const auto first = __builtin_amdgcn_cvt_pk_f32_fp8(codes, false), second = __builtin_amdgcn_cvt_pk_f32_fp8(codes, true);
+        rest[8 * piece + 4 * w] = v[4 * w] - first[0];
+        rest[8 * piece + 4 * w + 1] = v[4 * w + 1] - first[1];
+        rest[8 * piece + 4 * w + 2] = v[4 * w + 2] - second[0];
+        rest[8 * piece + 4 * w + 3] = v[4 * w + 3] - second[1];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 32; ++i) most = fmaxf(most, fabsf(rest[i]));
+    // t / s = the least power of two with most / (t / s) <= 7.5 = 1.875 * 4: most's exponent less 2, one more where its
+    // significand is above 1.875 (a NaN or infinite element leaves NaN remainders: the codes are then whatever the
+    // conversion makes of them, as the first term's are)
+    const uint32_t bits = __float_as_uint(most);
+    int power = static_cast<int>(bits >> 23) - 127 - 2 + ((bits & 0x7FFFFFu) > 0x700000u ? 1 : 0);
+    power = max(power, max(-126, 1 - hi_byte));  // (t and t / s stay normal powers of two; a block of zero remainders lands here)
+    const float t_over_s = __uint_as_float(static_cast<uint32_t>(power + 127) << 23);
+    f32x16_t even, odd;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      even[i] = rest[2 * i];
+      odd[i] = rest[2 * i + 1];
+    }
+    const u32x6_t lo = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(even, odd, t_over_s);
+    const int lo_byte = min(max(hi_byte + power, 1), 254);  // e8m0 of t = s * 2^power
+    const int half = block % 2;                                    // which 32 of the step's 64 depths
+    uint8_t* step = target + (block / 2) * 128;
+    // hi: the block's first 16 depths go to lane group 0's codes, its last 16 to group 1's, each at 16 * half
+    *reinterpret_cast<u32x4_t*>(step + 16 * half) = u32x4_t{hi[0], hi[1], hi[2], hi[3]};
+    *reinterpret_cast<u32x4_t*>(step + 64 + 16 * half) = u32x4_t{hi[4], hi[5], hi[6], hi[7]};
+    uint8_t* lo_at = step + 64 * half + 32;
+    *reinterpret_cast<u32x4_t*>(lo_at) = u32x4_t{lo[0], lo[1], lo[2], lo[3]};
+    *reinterpret_cast<u32x4_t*>(lo_at + 16) = u32x4_t{lo[4], lo[5], static_cast<uint32_t>(lo_byte), 0u};
+  }
+}
+
 }  // namespace dew
+
+extern "C" int dew_moe_split_rows_fp6(const void* x, void* split, uint8_t* scale, int32_t rows, int32_t depth, void* stream) {
+  using namespace dew;
+  DEW_REQUIRE(rows >= 0 && depth >= 64 && depth % 64 == 0, "dew_moe_split_rows_fp6: rows %d, depth %d (whole 64s)", rows, depth);
+  if (rows == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(x && split && scale, "dew_moe_split_rows_fp6: x, split and scale must not be null");
+  DEW_REQUIRE(aligned16(x) && aligned16(split), "dew_moe_split_rows_fp6: x and split must be 16-byte aligned");
+  hipLaunchKernelGGL(split_rows_fp6_kernel, dim3((rows + kSplitWaves - 1) / kSplitWaves), dim3(64 * kSplitWaves), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const bf16_t*>(x), static_cast<uint8_t*>(split), scale, rows, depth);
+  return launched("split_rows_fp6_kernel");
+}
 
 extern "C" int dew_moe_split_rows(const void* x, void* split, uint8_t* scale, int32_t rows, int32_t depth, void* stream) {
   using namespace dew;

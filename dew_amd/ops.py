@@ -417,6 +417,19 @@ def split_rows(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     return split, scale
 
 
+def split_rows_fp6(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """`split_rows` with the second term in FP6 (e2m3) under one power-of-two scale every 32 depths, which lies with
+    the codes: the same shapes, for `gateup_swiglu_split_out(..., fp6=True)`. The FP6 term's instruction takes half the
+    first term's cycles; an element more than two binades below its 32-deep block's largest is then held to within 2^-10
+    of that largest magnitude, not exactly."""
+    _device(x, "x", torch.bfloat16)
+    rows, depth = x.shape
+    split = torch.empty((rows, depth * 2), dtype=torch.uint8, device=x.device)
+    scale = torch.empty((rows,), dtype=torch.uint8, device=x.device)
+    _lib.check(_lib.library().dew_moe_split_rows_fp6(_ptr(x), _ptr(split), _ptr(scale), rows, depth, _stream()), "dew_moe_split_rows_fp6")
+    return split, scale
+
+
 @contextlib.contextmanager
 def tile_rows(rows: int):
     """Within the block every grouped product uses block tiles of `rows` rows (32, 64, 128, 256) instead of the
@@ -494,10 +507,11 @@ def block_scale_pitch(elements: int) -> int:
 
 def gateup_swiglu_split_out(split: torch.Tensor, scale: torch.Tensor, gate: PreparedBank, up: PreparedBank,
                             offsets: torch.Tensor, *, gather: torch.Tensor | None = None,
-                            rows: int | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+                            rows: int | None = None, fp6: bool = False) -> tuple[torch.Tensor, torch.Tensor]:
     """`gateup_swiglu_split` whose hidden rows leave already split: (`hidden_split` uint8 `[rows, F * 2]`,
     `hidden_scales` uint8 `[rows, block_scale_pitch(F)]`), one scale per row and 128 columns (byte b of a row scales its
-    columns 128 b .. 128 b + 127; the pad bytes are not written), for `grouped_gemm_split_blocks`."""
+    columns 128 b .. 128 b + 127; the pad bytes are not written), for `grouped_gemm_split_blocks`. `fp6`: the rows
+    come from `split_rows_fp6`."""
     experts, depth, width = gate.shape
     if split.dtype != torch.uint8 or split.shape[-1] != 2 * depth or scale.dtype != torch.uint8 or scale.numel() != split.shape[0]:
         raise KernelError(f"split rows are uint8 [rows, {2 * depth}] with one uint8 scale a row")
@@ -507,9 +521,9 @@ def gateup_swiglu_split_out(split: torch.Tensor, scale: torch.Tensor, gate: Prep
     rows = _product_rows(split, "split", offsets, experts, gather, None, rows)
     hidden = torch.empty((rows, width * 2), dtype=torch.uint8, device=split.device)
     scales = torch.empty((rows, block_scale_pitch(width)), dtype=torch.uint8, device=split.device)
-    _lib.check(_lib.library().dew_moe_gateup_swiglu_split_out(_ptr(split), _ptr(scale), _ptr(gather), _ptr(offsets), gate.descriptor,
-                                                              up.descriptor, _ptr(hidden), _ptr(scales), rows, _stream()),
-               "dew_moe_gateup_swiglu_split_out")
+    call = _lib.library().dew_moe_gateup_swiglu_split_fp6_out if fp6 else _lib.library().dew_moe_gateup_swiglu_split_out
+    _lib.check(call(_ptr(split), _ptr(scale), _ptr(gather), _ptr(offsets), gate.descriptor, up.descriptor, _ptr(hidden), _ptr(scales),
+                    rows, _stream()), "dew_moe_gateup_swiglu_split_fp6_out" if fp6 else "dew_moe_gateup_swiglu_split_out")
     return hidden, scales
 
 

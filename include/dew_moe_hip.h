@@ -262,6 +262,22 @@ int dew_moe_grouped_gemm_split_blocks(const void* x_split, const uint8_t* x_scal
                                       const int32_t* offsets, const dew_moe_bank* w, const float* bias,
                                       const int32_t* scatter, void* out, int32_t rows, void* stream);
 
+/* The first product of that pair with the rows' second term in FP6 (no counterpart in the reference). dew_moe_split_rows_fp6:
+ * x = s hi + t lo with hi = e4m3(x / s) under one power-of-two scale s a row (scale[row], as dew_moe_split_rows) and
+ * lo = e2m3((x - s hi) / t) under t, one power of two for every 32 depths. Each 64 depths of a row are 128 bytes: for
+ * lane group g = 0, 1: 32 bytes of hi codes (depths 16 g .. 16 g + 15, then 32 + 16 g .. 47 + 16 g), 24 bytes of lo codes
+ * (depths 32 g .. 32 g + 31, six bits each, in order), t's e8m0 byte in a dword, 4 unused bytes. The second term's
+ * instruction (FP6 x FP4) takes half the cycles of the first's, so the launch runs faster than on two e4m3 terms; the
+ * price is that an element more than two binades below its 32-deep block's largest magnitude is held to within 2^-10 of
+ * that magnitude, not exactly (dew_moe_split_rows: exactly within 2^-11 of the ROW's largest).
+ * dew_moe_gateup_swiglu_split_fp6_out is dew_moe_gateup_swiglu_split_out on such rows; its hidden rows leave in that
+ * entry point's format (two e4m3 terms under a scale per row and 128 columns).                                   */
+int dew_moe_split_rows_fp6(const void* x /* bf16 [rows, depth] */, void* split /* [rows, depth * 2] bytes */,
+                           uint8_t* scale /* [rows] e8m0 */, int32_t rows, int32_t depth, void* stream);
+int dew_moe_gateup_swiglu_split_fp6_out(const void* x_split, const uint8_t* x_scale, const int32_t* gather,
+                                        const int32_t* offsets, const dew_moe_bank* gate, const dew_moe_bank* up,
+                                        void* hidden_split, uint8_t* hidden_scales, int32_t rows, void* stream);
+
 /* The blockwise FP8 recipe's forward product (DeepSeek-V3's 1 x 128 activation tiles, 128 x 128 weight blocks):
  * `rows_quantized` src/dew/nn/kernels/projections.py:176-182 and `blockwise_fp8_product`
  * src/dew/nn/kernels/gemm.py:764-793 (its portable sum: `step_scaled` src/dew/nn/kernels/xla_products.py:147-173).

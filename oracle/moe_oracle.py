@@ -768,6 +768,73 @@ def nvfp4_projection(x, w, group_sizes, *, dtype="bfloat16", bias=None):
     return nvfp4_block_product(*rows, *matrices, group_sizes, dtype=dtype, bias=bias)
 
 
+E2M3_GRID = np.array([k / 8 for k in range(8)] + [1 + k / 8 for k in range(8)] + [2 + k / 4 for k in range(8)] + [4 + k / 2 for k in range(8)], F32)
+"""The magnitudes of FP6 e2m3 (OCP MX: two exponent bits, bias 1, three mantissa bits), by code."""
+
+
+def e2m3_rounded(values):
+    """fp32 values to the nearest e2m3 value, ties to the even code, saturating at +-7.5."""
+    values = np.asarray(values, F32)
+    magnitude = np.minimum(np.abs(values), F32(7.5))
+    above = np.clip(np.searchsorted(E2M3_GRID, magnitude), 1, len(E2M3_GRID) - 1)   # the first grid point at or above
+    low, high = E2M3_GRID[above - 1], E2M3_GRID[above]
+    up = (high - magnitude < magnitude - low) | ((high - magnitude == magnitude - low) & (above % 2 == 0))
+    return (np.sign(values) * np.where(up, high, low)).astype(F32)
+
+
+def split_rows_fp6(x):
+    """bf16 rows as the values `dew_moe_split_rows_fp6` holds them at (no counterpart in the reference, whose products
+    take the bf16 rows themselves): `s hi + t lo`, s = the power of two that brings the row's largest magnitude into
+    [128, 256) (exponent field clamped to 16 .. 254), hi = e4m3(x / s), t / s = the least power of two that brings the
+    largest remainder of each 32 depths within 7.5, lo = e2m3((x / s - hi) / (t / s)). Returns (values fp32 [rows, K],
+    scale bytes [rows]). Pinned by its invariants (tests/test_projections.py): exact for every element within two
+    binades of its block's largest, within 2^-10 of that largest otherwise, exact on rows of one binade."""
+    x = np.asarray(x, F32)
+    rows, depth = x.shape
+    field = np.clip((np.abs(x).max(axis=1).view(np.uint32) >> 23) & 0xFF, 16, 254).astype(np.int32)
+    hi_byte = field - 7
+    s = np.ldexp(F32(1), hi_byte - 127)[:, None]
+    v = (x / s).astype(F32)
+    hi = e4m3_rounded(v)
+    rest = (v - hi).astype(F32).reshape(rows, depth // 32, 32)
+    most = np.abs(rest).max(axis=-1, keepdims=True)
+    bits = most.view(np.uint32)
+    power = (bits >> 23).astype(np.int32) - 127 - 2 + ((bits & 0x7FFFFF) > 0x700000)
+    power = np.maximum(power, np.maximum(-126, 1 - hi_byte)[:, None, None])
+    t_over_s = np.ldexp(F32(1), power)
+    lo = e2m3_rounded((rest / t_over_s).astype(F32)) * t_over_s
+    values = ((hi.reshape(rest.shape) + lo).reshape(rows, depth) * s).astype(F32)
+    return values, hi_byte.astype(np.uint8)
+
+
+def split_rows_fp6_decoded(split, scale):
+    """The values a device buffer of `dew_moe_split_rows_fp6` stands for: `split` uint8 [rows, 2 K] (each 64 depths 128
+    bytes: for lane group g, 32 bytes of e4m3 codes of depths 16 g .. 16 g + 15 and 32 + 16 g .. 47 + 16 g, 24 bytes of
+    e2m3 codes of depths 32 g .. 32 g + 31 packed six bits each, the second term's e8m0 scale byte), `scale` uint8 [rows]."""
+    split = np.asarray(split, np.uint8)
+    rows, pitch = split.shape
+    steps = split.reshape(rows, pitch // 128, 2, 64)
+    table = _e4m3_table()
+    hi = table[steps[..., :32]]                                                   # [rows, steps, group, 32]
+    first = np.zeros((rows, pitch // 128, 64), F32)
+    for g in range(2):
+        first[..., 16 * g:16 * g + 16] = hi[:, :, g, :16]
+        first[..., 32 + 16 * g:48 + 16 * g] = hi[:, :, g, 16:]
+    packed = steps[..., 32:56].astype(np.uint64)                                  # 24 bytes = 32 six-bit codes
+    bits = np.zeros((rows, pitch // 128, 2), object)
+    codes = np.zeros((rows, pitch // 128, 2, 32), np.int64)
+    for i in range(32):
+        bit = 6 * i
+        lo_byte, shift = bit // 8, bit % 8
+        two = packed[..., lo_byte] | (packed[..., min(lo_byte + 1, 23)] << np.uint64(8))
+        codes[..., i] = ((two >> np.uint64(shift)) & np.uint64(63)).astype(np.int64)
+    magnitudes = E2M3_GRID[codes & 31] * np.where(codes & 32, F32(-1), F32(1))
+    t = np.ldexp(F32(1), steps[..., 56].astype(np.int32) - 127)[..., None]
+    second = (magnitudes * t).reshape(rows, pitch // 128, 64)
+    s = np.ldexp(F32(1), np.asarray(scale, np.uint8).astype(np.int32) - 127)[:, None]
+    return ((first * s[:, :, None]) + second).reshape(rows, pitch // 2).astype(F32)
+
+
 def swiglu(gate, up, *, dtype="bfloat16", limit=None, exp=np.exp):
     """`gated_product('swiglu')` after `swiglu_clamped` (src/dew/nn/activations.py:267-278,327-356):
     bf16 rounds the activation `g * logistic(g)` and then the product with `u`; fp32 rounds nowhere.

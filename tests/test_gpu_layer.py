@@ -108,18 +108,27 @@ def test_large_groups_on_mxfp4_banks_run_on_split_rows_and_agree_with_the_bf16_l
     calls = []
     split_out = ops.gateup_swiglu_split_out
     monkeypatch.setattr(ops, "gateup_swiglu_split_out", lambda *a, **k: calls.append(1) or split_out(*a, **k))
-    assert gemm.SPLIT_ROWS
-    got = layer.apply(variables, x, logits=logits).float().cpu().numpy()
+    assert gemm.SPLIT_ROWS and gemm.SPLIT_SECOND_TERM == "e4m3"
+    got = layer.apply(variables, x, logits=logits).float().cpu().numpy()            # two e4m3 terms: the rows' bf16 values exactly
     assert calls == [1]
+    monkeypatch.setattr(gemm, "SPLIT_SECOND_TERM", "e2m3")
+    with_fp6 = layer.apply(variables, x, logits=logits).float().cpu().numpy()       # the option: an e4m3 and an e2m3 term
+    assert calls == [1, 1]
     monkeypatch.setattr(gemm, "SPLIT_ROWS", False)
     plain = layer.apply(variables, x, logits=logits).float().cpu().numpy()
-    assert calls == [1]
+    assert calls == [1, 1]
     want, _ = oracle_output(case, data)
-    for name, value in (("split rows", got), ("bf16 operands", plain)):
+    for name, value in (("split rows, two e4m3", got), ("bf16 operands", plain)):
         by_max, by_element = oracle.relative_errors(value, want)
         print(f"\n{name}: max|d|/max|ref| = {by_max:.3e}, element-wise max rel = {by_element:.3e}, identical = {(value == want).mean():.4f}")
         assert by_max <= TOLERANCE and by_element <= TOLERANCE
     assert (got == plain).mean() > 0.9 and np.abs(got - plain).max() <= 2.0 ** -6 * np.abs(plain).max()
+    # the FP6 second term is an option, not the default, because of what it costs here: inside 1e-2 of the largest output
+    # (the reference's own measure), but element-wise it can pass the 2e-2 bar on an MLP this narrow (512 deep)
+    by_max, by_element = oracle.relative_errors(with_fp6, want)
+    print(f"\nsplit rows, e4m3 + e2m3 (option): max|d|/max|ref| = {by_max:.3e}, element-wise max rel = {by_element:.3e}, "
+          f"identical = {(with_fp6 == want).mean():.4f}")
+    assert by_max <= 1e-2 and by_element <= 4e-2
 
 
 def test_layer_multiplies_its_own_gate_kernel_when_no_logits_are_given():
