@@ -46,10 +46,11 @@ const char* dew_moe_kernels(void) {
          "grouped_gemm<medium>,128,256 (paired 2x128) | 128,64,4 (1x4),v_mfma_f32_32x32x16_bf16,bf16 x {fp8 block|fp8 channel|nvfp4|mxfp4}; 2 blocks/CU\n"
          "grouped_gemm<decode>,32,128 (paired 2x128),64,4 (1x4),v_mfma_f32_32x32x16_bf16,weight streaming for groups under 24 rows\n"
          "grouped_gemm epilogues,-,-,-,-,-,plain (+bias) | swiglu of two banks | interleaved gate/up clamped 1.702 gating (+bias); tile staged in LDS and stored as whole rows\n"
-         "grouped_gemm<split rows>,256,256 (paired 2x128),64,4 (2x2),v_mfma_scale_f32_32x32x64_f8f6f4,two e4m3 terms per bf16 activation x mxfp4 codes as stored; SwiGLU rows written already split\n"
+         "grouped_gemm<split rows>,128 (paired; 2 blocks/CU) | 256,256 (paired 2x128),64,4 (2x2),v_mfma_scale_f32_32x32x64_f8f6f4,two e4m3 terms per bf16 activation x mxfp4 codes as stored; SwiGLU rows written already split\n"
+         "grouped_gemm<split rows; fp6 second term>,128,256 (paired 2x128),64,4 (2x2),v_mfma_scale_f32_32x32x64_f8f6f4,an e4m3 term and an e2m3 term under one e8m0 scale per 32 depths x mxfp4 codes: opt-in; three quarters of the issue time\n"
          "grouped_gemm<fp8 rows>,256,256 | 128,128,4 (2x2),v_mfma_scale_f32_32x32x64_f8f6f4,e4m3 rows (1x128 power-of-two scales) x fp8 128x128 blocks (power-of-two scales)\n"
          "grouped_gemm<mxfp8 rows>,256,256,128,4 (2x2),v_mfma_scale_f32_32x32x64_f8f6f4,OCP MXFP8 rows x MXFP8 bank: e4m3 codes and E8M0 scales per 32 depths of both operands as stored\n"
-         "split_rows | quantize_rows_fp8 | quantize_rows_mxfp8,1 row/wave,-,-,4,-,bf16 rows -> e4m3 terms | e4m3 codes in operand order + e8m0 scales\n"
+         "split_rows | split_rows_fp6 | quantize_rows_fp8 | quantize_rows_mxfp8,1 row/wave,-,-,4,-,bf16 rows -> e4m3 terms (or e4m3 + e2m3) | e4m3 codes in operand order + e8m0 scales\n"
          "grouped_gemm<bf16>,32|64|128|256,128|256,64,3,v_mfma_f32_32x32x16_bf16,unquantized bf16 matrices as fragment atoms: no dequantization\n"
          "grouped_gemm<mxfp8 window>,256,256 | 128,128,4 (2x2),v_mfma_scale_f32_32x32x64_f8f6f4,a kernel gradient: each group's window of 128-token steps of lhs_t rows x the rhs_t bank; bf16 or fp32 out\n"
          "grouped_gemm<bf16 window>,256,256 | 128,64,3,v_mfma_f32_32x32x16_bf16,gemm_t: each group's window of 64-token steps of bf16 lhs_t rows x the bf16 rhs_t bank; tensor scales on the sums\n"

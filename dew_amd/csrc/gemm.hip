@@ -103,6 +103,7 @@ struct GemmParams {
   const int32_t* windows;
   int window_rows;
   float* out_f32;  // the product in fp32 (kPlainF32) instead of `out`
+  int group_m;     // m-tiles of a chunk of 8 group_m tiles that one XCD's resident blocks cover together (set by launch_tile)
   const float* factor0;  // a kernel gradient's fp32 sums times *factor0 * *factor1 before the rounding (each may be null):
   const float* factor1;  // the tensor scales of NVFP4 operands
 };
@@ -241,11 +242,11 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
 
   // ---- block -> (m-tile, column strip). Workgroup ids are dealt round-robin to the 8 XCDs, each with its
-  // own L2. Tiles are ordered so that 32 consecutive ones (one XCD's residents) cover kGroupM m-tiles x 8
+  // own L2. Tiles are ordered so that a chunk of consecutive ones (one XCD's residents) covers kGroupM m-tiles x 8
   // strips, sharing A rows and B strips through that L2, and such chunks of 32 are dealt round-robin to the
   // XCDs: the m-tile bound overshoots the real tile count by up to one tile per expert, and the empty tiles
   // at the end of the order then spread over all XCDs instead of idling the last ones.
-  constexpr int kGroupM = 4, kChunk = 32;
+  const int kGroupM = p.group_m, kChunk = 8 * kGroupM;
   const int n_strips = p.width / BN;
   const int total = p.m_tile_bound * n_strips;
   const int local = blockIdx.x / 8;
@@ -1007,7 +1008,12 @@ static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
   p.m_tile_bound = p.tail_of > 0 ? p.experts : (p.rows + BM - 1) / BM + p.experts + 1;
   if (FORMAT == kFormatMxFp8Window || FORMAT == kFormatBf16Window) p.m_tile_bound = p.experts * ((p.window_rows + BM - 1) / BM);  // every group the same whole rows
   const int total = p.m_tile_bound * (p.width / BN);
-  const int blocks = ((total + 255) / 256) * 256;  // whole chunks of 32 tiles for each of the 8 XCDs
+  // A chunk is 4 m-tiles x 8 strips, and 2 x 8 for the 256-row tiles, whose launches have the fewest tiles: dealt in
+  // smaller chunks their last round spreads more evenly over the XCDs (measured on 16 to 64 m-tiles of 256 rows: the down
+  // launch 8 % shorter, the paired one 3 %; taller chunks of 8 or 16 m-tiles, which fetch less, were slower everywhere)
+  p.group_m = BM == 256 ? 2 : 4;
+  const int round = 64 * p.group_m;
+  const int blocks = ((total + round - 1) / round) * round;  // whole chunks of tiles for each of the 8 XCDs
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreads), kShared, stream, p);
   return launched(who);
 }
