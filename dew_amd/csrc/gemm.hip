@@ -94,8 +94,8 @@ struct GemmParams {
   float limit;        // the interleaved gated epilogue's clamp
   int experts, depth, width, rows, m_tile_bound;
   // A launch normally multiplies every group in tiles of its BM rows, the last of a group partly empty. Where that
-  // waste matters two launches share the groups: the taller tiles' launch leaves (skip_tails) a last tile that would
-  // hold at most BM / 2 rows to a launch of tiles half as tall, which multiplies (tail_of = the taller tile's rows)
+  // waste matters two launches share the groups: the taller tiles' launch leaves a last tile that would hold at most
+  // skip_tails rows to a launch of tiles that many rows tall, which multiplies (tail_of = the taller tile's rows)
   // only those last rows, the ones past a group's whole tiles of tail_of rows where they are at most its own BM.
   int skip_tails, tail_of;
   // A kernel gradient (kFormatMxFp8Window): every group multiplies the same window_rows rows over its own window of
@@ -289,7 +289,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
         tiles = rest >= 1 && rest <= BM ? 1 : 0;
         start += size - rest;
       } else {
-        tiles = size / BM + (size % BM > (p.skip_tails ? BM / 2 : 0) ? 1 : 0);
+        tiles = size / BM + (size % BM > p.skip_tails ? 1 : 0);
       }
     }
     int inclusive = tiles;
@@ -1061,7 +1061,7 @@ static int launch_format(const char* who, const GemmParams& p, hipStream_t strea
       // 256 groups of 256 +- 16 rows, 2.5 tiles a group become 2 and a 64-row one.
       const bool shared = forced_tile_rows == 0 && static_cast<long long>(p.experts) * (p.width / 128) >= 256;
       GemmParams taller = p;
-      taller.skip_tails = shared ? 1 : 0;
+      taller.skip_tails = shared ? 64 : 0;
       int status;
       if (!kPaired && p.width % 256 == 0 && static_cast<long long>(p.rows / 128 + 1) * (p.width / 256) >= 512)
         status = launch_tile<FORMAT, MODE, 128, 256, 1, 4>(who, taller, stream);  // enough tiles to fill the chip twice over
