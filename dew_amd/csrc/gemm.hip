@@ -1048,10 +1048,10 @@ static int tile_rows(const GemmParams& p, bool fp4) {
 template <int FORMAT, int MODE>
 static int launch_format(const char* who, const GemmParams& p, hipStream_t stream) {
   // (256-row tiles: the banks whose weights cost the vector unit little or nothing to bring to bf16. General NVFP4
-  // scales cost it as much as FP8 does, and two 128-row blocks a CU then run a paired launch of 1024-row groups 7 to 15 %
-  // faster than one 256-row block, the unpaired one the same)
-  constexpr bool kFp4 = FORMAT == DEW_MOE_W_MXFP4 || FORMAT == DEW_MOE_W_BF16;
+  // scales cost it as much as FP8 does: two 128-row blocks a CU run a paired launch of 1024-row groups 7 to 15 % faster
+  // than one 256-row block; a one-bank launch the same there and 4 to 7 % slower on 4096-row groups, so it keeps the taller tile)
   constexpr bool kPaired = MODE == kSwigluOfTwo;
+  constexpr bool kFp4 = FORMAT == DEW_MOE_W_MXFP4 || FORMAT == DEW_MOE_W_BF16 || (FORMAT == DEW_MOE_W_NVFP4 && !kPaired);
   switch (tile_rows(p, kFp4)) {
     case 32:
       // one bank: 256 columns a block where that still leaves every CU several blocks, so that a launch is one round
