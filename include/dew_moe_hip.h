@@ -148,7 +148,9 @@ int dew_moe_permute_shared(const int32_t* indices /* [T,k] */, int32_t tokens, i
  * problem whose dew_moe_permute_workspace_bytes() is larger is refused (slots / 2048 blocks x (experts + 1) x 8 bytes:
  * 1 MiB covers e.g. 2^20 slots over 255 experts). Calls on one GPU share that array: calls that overlap on
  * different streams of one GPU race; calls in stream order need nothing cleared between them. The call allocates and
- * frees nothing; outputs are identical to dew_moe_permute's.                                                    */
+ * frees nothing; outputs are identical to dew_moe_permute's. The device the stream belongs to must be current: the
+ * first call on a device looks up that device's copy of the array (hipGetSymbolAddress, once), so make that call
+ * before a capture begins.                                                                                        */
 #define DEW_MOE_PERMUTE_STATIC_BYTES ((size_t)1 << 20)
 int dew_moe_permute_static(const int32_t* indices /* [T,k] */, int32_t tokens, int32_t top_k, int32_t experts,
                            int32_t* sizes, int32_t* offsets, int32_t* order, int32_t* rows, void* stream);
