@@ -353,7 +353,9 @@ def measure(config, args, device, sustained, with_cpu_baseline):
                                  "note": "least gap over the tokens between the k-th selection and the best one left out; 0 is an "
                                          "exact tie (the lower index wins everywhere)"}
     if with_cpu_baseline or not args.no_parity:
-        baseline, (slots, want) = oracle_sample(case, data, plan)
+        # the timed CPU baseline takes a larger sample (about ten seconds of host work, most of it the GEMMs, not the one
+        # expert's dequantization); the other configs' parity samples stay small so that the default run takes minutes
+        baseline, (slots, want) = oracle_sample(case, data, plan, budget_rows=4096 if with_cpu_baseline else 192)
         if with_cpu_baseline:
             result["cpu_baseline"] = baseline
         # parity on the sample at full size: the device's down-projection rows for those slots
