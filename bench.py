@@ -259,16 +259,18 @@ def measure(config, args, device, sustained, with_cpu_baseline):
         stepper()
     torch.cuda.synchronize()
     if graphed:
-        # The step makes seven short launches; captured once, it replays as one graph with no host work between
-        # kernels. The launches themselves are the same C-ABI calls on the capture stream.
+        # A step is a handful of short launches. The timed steps are captured back to back as one graph, the way a
+        # model's decode graph holds one such step for every MoE layer, and replayed once: no host work between
+        # kernels, and the replay's own start-up (about 17 us a replay on this stack, whatever the graph holds) is paid
+        # once, not once a step. The launches themselves are the same C-ABI calls on the capture stream.
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            out, plan = stepper()
+            for _ in range(args.steps):
+                out, plan = stepper()
         graph.replay()
         torch.cuda.synchronize()
         began = time.perf_counter()
-        for _ in range(args.steps):
-            graph.replay()
+        graph.replay()
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - began
         # The dominant kernel's duration: HIP events around its launch inside eager steps on the same inputs. A
@@ -339,7 +341,7 @@ def measure(config, args, device, sustained, with_cpu_baseline):
                                f"{case.quant} weights, {case.router['score_function']} router"
                                + (" + shared expert" if case.shared else ""),
                    "routed_rows": routed_rows, "experts_touched": touched,
-                   **({"shared_expert": "group #E of the routed launches" if stepper.fused_shared else "two launches of its own"} if case.shared else {}), "launch": "hip graph replay" if graphed else "eager",
+                   **({"shared_expert": "group #E of the routed launches" if stepper.fused_shared else "two launches of its own"} if case.shared else {}), "launch": "hip graph replay (the timed steps captured back to back as one graph)" if graphed else "eager",
                    "algorithmic_flops": flops},
         "roofline": roofline,
     }
