@@ -150,16 +150,22 @@ __global__ __launch_bounds__(kPermuteThreads) void permute_scatter_kernel(Permut
 // All of the above in one launch for at most kSmallSlots slots (a decode step, a small prefill): one block
 // counts, scans and scatters, each wavefront a contiguous run of the slots, with the LDS histogram as the only
 // intermediate.
-constexpr int kSmallSlots = 2048;  // beyond this three launches over many blocks are faster (measured at 4096)
-__global__ __launch_bounds__(kPermuteThreads) void permute_small_kernel(PermuteParams p) {
-  extern __shared__ int32_t running[];  // [kPermuteWaves][buckets] then [buckets + 1] totals
-  int32_t* totals = running + kPermuteWaves * p.buckets;
+// Measured under graph replay, sixteen wavefronts: 2048 slots 5.1 to 6.8 us (four wavefronts: 7.9 to 10.0), 4096 slots
+// 7.5 us against 11.4 us for the three launches, 8192 slots the same either way.
+constexpr int kSmallSlots = 4096;      // beyond this three launches over many blocks are as fast or faster
+constexpr int kSmallThreads = 1024;    // sixteen wavefronts, where their counters fit the LDS a launch may take unasked
+constexpr int kNarrowSmallSlots = 2048;  // the four-wavefront form's reach, for more buckets than that
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void permute_small_kernel(PermuteParams p) {
+  constexpr int kWaves = THREADS / 64;
+  extern __shared__ int32_t running[];  // [kWaves][buckets] then [buckets + 1] totals
+  int32_t* totals = running + kWaves * p.buckets;
   const int lane = threadIdx.x % 64;
   const int wave = threadIdx.x / 64;
-  for (int i = threadIdx.x; i < kPermuteWaves * p.buckets; i += kPermuteThreads) running[i] = 0;
+  for (int i = threadIdx.x; i < kWaves * p.buckets; i += THREADS) running[i] = 0;
   __syncthreads();
   int32_t* mine = running + wave * p.buckets;
-  const int segment = ((p.slots + kPermuteThreads - 1) / kPermuteThreads) * 64;  // contiguous slots per wavefront
+  const int segment = ((p.slots + THREADS - 1) / THREADS) * 64;  // contiguous slots per wavefront
   const int rounds = segment / 64;
   const int wave_begin = wave * segment;
   for (int round = 0; round < rounds; ++round) {
@@ -167,9 +173,9 @@ __global__ __launch_bounds__(kPermuteThreads) void permute_small_kernel(PermuteP
     if (slot < p.slots) atomicAdd(&mine[bucket_of(p, slot)], 1);
   }
   __syncthreads();
-  for (int b = threadIdx.x; b < p.buckets; b += kPermuteThreads) {
+  for (int b = threadIdx.x; b < p.buckets; b += THREADS) {
     int sum = 0;
-    for (int w = 0; w < kPermuteWaves; ++w) sum += running[w * p.buckets + b];
+    for (int w = 0; w < kWaves; ++w) sum += running[w * p.buckets + b];
     totals[b] = sum;
   }
   __syncthreads();
@@ -190,7 +196,7 @@ __global__ __launch_bounds__(kPermuteThreads) void permute_small_kernel(PermuteP
     if (lane == 0) totals[p.buckets] = carried;
   }
   __syncthreads();
-  for (int b = threadIdx.x; b < p.buckets; b += kPermuteThreads) {
+  for (int b = threadIdx.x; b < p.buckets; b += THREADS) {
     const int start = totals[b];
     if (b < p.groups) {
       p.sizes[b] = totals[b + 1] - start;
@@ -199,7 +205,7 @@ __global__ __launch_bounds__(kPermuteThreads) void permute_small_kernel(PermuteP
       p.offsets[p.groups] = start;
     }
     int next = start;
-    for (int w = 0; w < kPermuteWaves; ++w) {
+    for (int w = 0; w < kWaves; ++w) {
       const int count = running[w * p.buckets + b];
       running[w * p.buckets + b] = next;
       next += count;
@@ -320,8 +326,14 @@ static int permute_launches(const int32_t* indices, int32_t tokens, int32_t top_
   p.blocks = (slots + kSlotsPerBlock - 1) / kSlotsPerBlock;
   p.counts = counts;
   p.bases = p.counts + static_cast<size_t>(p.blocks) * p.buckets;
-  if (slots <= kSmallSlots) {  // one block does it all faster than three launches
-    hipLaunchKernelGGL(permute_small_kernel, dim3(1), dim3(kPermuteThreads),
+  // one block does it all faster than three launches
+  const size_t wide_lds = sizeof(int32_t) * ((kSmallThreads / 64 + 1) * static_cast<size_t>(p.buckets) + 1);
+  if (slots <= kSmallSlots && wide_lds <= 65536) {
+    hipLaunchKernelGGL(permute_small_kernel<kSmallThreads>, dim3(1), dim3(kSmallThreads), wide_lds, s, p);
+    return launched("permute_small_kernel");
+  }
+  if (slots <= kNarrowSmallSlots) {
+    hipLaunchKernelGGL(permute_small_kernel<kPermuteThreads>, dim3(1), dim3(kPermuteThreads),
                        sizeof(int32_t) * ((kPermuteWaves + 1) * p.buckets + 1), s, p);
     return launched("permute_small_kernel");
   }

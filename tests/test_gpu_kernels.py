@@ -108,7 +108,8 @@ def test_router_reproduces_the_reference_fixtures_on_the_device(ops):
 
 
 @pytest.mark.parametrize("tokens,k,experts", [(1, 1, 1), (7, 2, 4), (64, 8, 128), (300, 3, 5), (2048, 2, 8),
-                                               (1025, 2, 8), (16384, 2, 8), (8192, 8, 256), (3000, 6, 512), (1024, 8, 128), (1025, 8, 64)])
+                                               (1025, 2, 8), (16384, 2, 8), (8192, 8, 256), (3000, 6, 512), (1024, 8, 128), (1025, 8, 64),
+                                               (512, 8, 960), (100, 4, 1000), (700, 4, 1000), (2049, 2, 8)])
 def test_permute_is_the_stable_sort_by_expert(ops, tokens, k, experts):
     rng = np.random.default_rng(tokens * 31 + experts)
     indices = rng.integers(0, experts, size=(tokens, k)).astype(np.int32)
