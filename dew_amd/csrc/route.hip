@@ -2,6 +2,8 @@
 // Follows Router.__call__ from the logits on (reference src/dew/nn/moe.py:466-565). Every floating-point
 // step is a fixed sequence of IEEE fp32/fp64 operations with contraction off, the same sequence the CPU
 // oracle runs, so the chosen experts agree bit for bit.
+#include <type_traits>
+
 #include "common.h"
 
 #pragma clang fp contract(off)
@@ -45,10 +47,23 @@ __device__ __forceinline__ float pointwise_score(int score_function, float logit
   return score_function == DEW_MOE_SCORE_SQRTSOFTPLUS ? sqrt_softplus_f32(logit) : 1.0f / (1.0f + exp_f32(-logit));
 }
 
+// The wavefront's largest value, in every lane: maxima within quads, half rows and rows of 16 lanes by DPP moves (one
+// instruction each, no LDS crossbar), then lane 15 of each row into the next row and lane 31 into the upper half, so that
+// lane 63 holds the maximum of all 64, which a lane read hands to everyone. (A maximum does not depend on the order it
+// is taken in, so this is the butterfly's result; the sums below keep their fixed order.)
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int offset = 32; offset >= 1; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, kWave));
-  return v;
+  auto moved = [](float value, auto control, auto rows) {
+    const int bits = __builtin_bit_cast(int, value);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(bits, bits, decltype(control)::value, decltype(rows)::value, 0xF, false));
+  };
+  using std::integral_constant;
+  v = fmaxf(v, moved(v, integral_constant<int, 0xB1>{}, integral_constant<int, 0xF>{}));   // quad_perm [1,0,3,2]
+  v = fmaxf(v, moved(v, integral_constant<int, 0x4E>{}, integral_constant<int, 0xF>{}));   // quad_perm [2,3,0,1]
+  v = fmaxf(v, moved(v, integral_constant<int, 0x141>{}, integral_constant<int, 0xF>{}));  // row_half_mirror
+  v = fmaxf(v, moved(v, integral_constant<int, 0x140>{}, integral_constant<int, 0xF>{}));  // row_mirror
+  v = fmaxf(v, moved(v, integral_constant<int, 0x142>{}, integral_constant<int, 0xA>{}));  // row_bcast15 into rows 1, 3
+  v = fmaxf(v, moved(v, integral_constant<int, 0x143>{}, integral_constant<int, 0xC>{}));  // row_bcast31 into rows 2, 3
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
 // Sum rounded once: fp64 partials per lane, then a butterfly; every lane ends with the same value.
