@@ -57,7 +57,10 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const bf16_t* __restrict__ 
   for (long long item = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; item < chunks;
        item += static_cast<long long>(gridDim.x) * blockDim.x) {
     const Bf16x8 g = reinterpret_cast<const Bf16x8*>(gate)[item];
-    const Bf16x8 u = reinterpret_cast<const Bf16x8*>(up)[item];
+    Bf16x8 u;  // without an up projection (a plain SiLU) every up value is one: bf16(bf16(g * logistic(g)) * 1) is the SiLU's one rounding
+#pragma unroll
+    for (int i = 0; i < 8; ++i) u.v[i] = 0x3F80;
+    if (up != nullptr) u = reinterpret_cast<const Bf16x8*>(up)[item];
     Bf16x8 h;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -103,6 +106,18 @@ extern "C" int dew_moe_combine(const void* slots, const float* weights, const vo
 
 extern "C" int dew_moe_swiglu(const void* gate, const void* up, void* hidden, int64_t count, void* stream) {
   return dew_moe_swiglu_clamped(gate, up, 0.0f, hidden, count, stream);
+}
+
+extern "C" int dew_moe_silu(const void* x, void* out, int64_t count, void* stream) {
+  using namespace dew;
+  DEW_REQUIRE(count >= 0 && count % 8 == 0, "dew_moe_silu: count %lld is not a multiple of 8", static_cast<long long>(count));
+  if (count == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(x && out && aligned16(x) && aligned16(out), "dew_moe_silu: x and out must not be null and must be 16-byte aligned");
+  const long long chunks = count / 8;
+  const int blocks = static_cast<int>(min((chunks + 255) / 256, 256ll * 64));
+  hipLaunchKernelGGL(swiglu_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<const bf16_t*>(x),
+                     static_cast<const bf16_t*>(nullptr), static_cast<bf16_t*>(out), chunks, 0.0f);
+  return launched("swiglu_kernel");
 }
 
 extern "C" int dew_moe_swiglu_clamped(const void* gate, const void* up, float limit, void* hidden, int64_t count, void* stream) {

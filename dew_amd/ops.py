@@ -389,6 +389,14 @@ def swiglu(gate: torch.Tensor, up: torch.Tensor, limit: float | None = None) -> 
     return hidden
 
 
+def silu(x: torch.Tensor) -> torch.Tensor:
+    """`bf16(x * logistic(x))`, formed in fp32 and rounded once (the reference's `silu`)."""
+    _device(x, "x", torch.bfloat16)
+    out = torch.empty_like(x)
+    _lib.check(_lib.library().dew_moe_silu(_ptr(x), _ptr(out), x.numel(), _stream()), "dew_moe_silu")
+    return out
+
+
 def combine(slots: torch.Tensor, weights: torch.Tensor, addend: torch.Tensor | None = None) -> torch.Tensor:
     """`out[t] = bf16(sum_j f32(slots[t, j]) * weights[t, j])` (+ the shared expert's `addend`)."""
     _device(slots, "slots", torch.bfloat16), _device(weights, "weights", torch.float32)

@@ -385,6 +385,9 @@ int dew_moe_swiglu(const void* gate, const void* up, void* hidden, int64_t count
 /* The same with the gate clamped from above and the up projection both ways by `limit` before their product
  * (`swiglu_clamped`, src/dew/nn/activations.py:327-333: DeepSeek V4's and GLM's experts); limit 0 = none.  */
 int dew_moe_swiglu_clamped(const void* gate, const void* up, float limit, void* hidden, int64_t count, void* stream);
+/* The activation alone: out = bf16(x * logistic(x)), formed in fp32 and rounded once (`silu`, src/dew/nn/activations.py:100-106),
+ * which routed value experts pass each chosen projection through (src/dew/nn/value_experts.py:79-82).      */
+int dew_moe_silu(const void* x /* bf16 [count] */, void* out /* bf16 [count] */, int64_t count, void* stream);
 
 /* ---- Combine (src/dew/nn/moe.py:1328-1333 `_combine`, :1503 shared add) ----------------------------
  * out[t,:] = bf16( sum_j f32(slots[t,j,:]) * weights[t,j] ), fp32 sum in slot order; with `addend`

@@ -25,6 +25,12 @@ What pins each function (tests/test_oracle_golden.py):
 * `grouped_matmul`: tools/grouped_oracle.py:20-27 semantics (float64 per-group product) on integer inputs,
   where fp32 sums are exact.
 
+* `silu` / `routed_values` (routed value experts, src/dew/nn/value_experts.py): the reference holds no vectors for the
+  layer alone (its fixture is a whole model's logits); `silu` is `swiglu`'s activation with its one rounding, checked
+  against `swiglu(x, 1)`, a float64 `x / (1 + e^-x)` and on every bf16; `routed_values` against a token-by-token
+  float64 sum of the chosen experts' products on integer operands (where every fp32 sum is exact), which a wrong
+  gather, scatter, weight pairing or a missing activation fails.
+
 * `load_balance_update`: the known answer of tests/test_moe.py:326-336 (counts 3, 1, 0, 0 at rate 0.001).
 * `router_statistics`: closed forms (scores = exp(logits - log_z) for softmax; log_z(logits + c) = log_z + c; the
   z-loss's log partition against a float64 logsumexp).
@@ -849,6 +855,32 @@ def swiglu(gate, up, *, dtype="bfloat16", limit=None, exp=np.exp):
     sig = (F32(1) / (F32(1) + exp(-gate).astype(F32)).astype(F32)).astype(F32)
     activated = bf16_round((gate * sig).astype(F32))
     return bf16_round((activated * up).astype(F32))
+
+
+def silu(x, *, dtype="bfloat16", exp=np.exp):
+    """`silu` (src/dew/nn/activations.py:100-106): `x * logistic(x)` in fp32, rounded once to the array's dtype. The
+    first of `swiglu`'s two roundings; the same stand-in for the backend's exp."""
+    x = np.asarray(x, F32)
+    if dtype == "bfloat16":
+        x = bf16_round(x)
+    sig = (F32(1) / (F32(1) + exp(-x).astype(F32)).astype(F32)).astype(F32)
+    activated = (x * sig).astype(F32)
+    return bf16_round(activated) if dtype == "bfloat16" else activated
+
+
+def routed_values(x, weights, indices, kernel, *, dtype="bfloat16", factor=None):
+    """`RoutedValues.__call__` from the routing on (src/dew/nn/value_experts.py:79-98): each token's chosen projections
+    `x @ kernel[e]` (one rounding), each through `silu`, summed under the router's weights in fp32 and rounded once.
+    `kernel [E, in, features]` dequantized values. Returns (out [T, features], the slots [T, k, features])."""
+    x = np.asarray(x, F32).reshape(-1, np.asarray(x).shape[-1])
+    indices = np.asarray(indices).reshape(x.shape[0], -1)
+    plan = sorted_by_expert(indices, kernel.shape[0])
+    projected = grouped_matmul(x[plan["rows"]], kernel, plan["sizes"], dtype=dtype, factor=factor)
+    activated = silu(projected, dtype=dtype)
+    slots = np.zeros_like(activated)
+    slots[plan["order"]] = activated
+    slots = slots.reshape(indices.shape[0], indices.shape[1], -1)
+    return combine(slots, np.asarray(weights).reshape(indices.shape), dtype=dtype), slots
 
 
 def combine(slots, weights, *, dtype="bfloat16"):

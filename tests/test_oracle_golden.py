@@ -361,3 +361,44 @@ def test_capacity_dropping_is_the_references_argsort_arithmetic():
         ours, ours_capacity = oracle.capacity_admitted(indices, experts, factor)
         theirs, theirs_capacity = by_argsort(indices, experts, factor)
         assert ours_capacity == theirs_capacity and np.array_equal(ours, theirs)
+
+
+def test_silu_is_the_activation_of_swiglu_with_its_one_rounding():
+    """`silu` against the three things that fix it: `swiglu` with an up projection of one (the same activation, then
+    a product by 1 that changes nothing), a float64 `x / (1 + e^-x)` rounded once, on every finite bf16; and the fp32
+    mode, which rounds nowhere."""
+    every = oracle.bf16_from_bits(np.arange(65536, dtype=np.uint16))
+    every = every[np.isfinite(every)]
+    got = oracle.silu(every)
+    assert np.array_equal(got, oracle.swiglu(every, np.ones_like(every)))
+    # (below -87 fp32's e^-x overflows and the reference's 1 / (1 + e^-x) is zero there, src/dew/nn/precision.py:568-575)
+    inside = every > -87
+    wide = every[inside].astype(np.float64)
+    truth = wide / (1.0 + np.exp(-wide))
+    rounded = oracle.bf16_round(truth.astype(np.float32))
+    # one rounding of the fp32 product: at most one bf16 step from the float64 value's rounding, and equal almost everywhere
+    steps = np.abs(oracle.bf16_bits(got[inside]).astype(np.int64) - oracle.bf16_bits(rounded).astype(np.int64))
+    assert steps.max() <= 1 and (steps == 0).mean() > 0.999
+    assert np.all(np.abs(got[~inside]) < 1e-35) and np.all(got[every < -89] == 0)
+    assert oracle.silu(np.float32([1.0]), dtype="float32")[0] == np.float32(np.float32(0.7310586) * 1)
+    assert oracle.silu(np.float32([0.0, -0.0]))[0] == 0
+
+
+def test_routed_values_are_each_tokens_weighted_sum_of_its_chosen_experts_activated_projections():
+    """Integer operands small enough that every fp32 sum is exact: the layer against a token-by-token float64 sum,
+    with weights that are powers of two. A wrong gather, scatter, weight pairing or a missing activation fails it."""
+    rng = np.random.default_rng(11)
+    tokens, experts, k, depth, width = 13, 5, 2, 16, 8
+    x = rng.integers(-3, 4, size=(tokens, depth)).astype(np.float32)
+    kernel = rng.integers(-2, 3, size=(experts, depth, width)).astype(np.float32)
+    indices = np.stack([rng.permutation(experts)[:k] for _ in range(tokens)]).astype(np.int32)
+    weights = np.exp2(rng.integers(-2, 2, size=(tokens, k))).astype(np.float32)
+    out, slots = oracle.routed_values(x, weights, indices, kernel)
+    for t in range(tokens):
+        total = np.zeros(width, np.float64)
+        for j in range(k):
+            projected = x[t].astype(np.float64) @ kernel[indices[t, j]].astype(np.float64)       # small integers: exact in bf16
+            activated = oracle.silu(projected.astype(np.float32)).astype(np.float64)
+            assert np.array_equal(slots[t, j], activated.astype(np.float32))
+            total += activated * float(weights[t, j])
+        assert np.array_equal(out[t], oracle.bf16_round(total.astype(np.float32))), t
