@@ -1426,6 +1426,88 @@ extern "C" int dew_moe_gateup_swiglu_split_fp6_out(const void* x_split, const ui
   return launch_tile<kFormatMxSplit6, kSwigluOfTwoSplit, 128, 128, 2, 2>(who, p, static_cast<hipStream_t>(stream));
 }
 
+// ---- the SwiGLU expert MLP on split rows as one call -----------------------------------------------------------------
+
+extern "C" int dew_moe_prefers_split_rows(const dew_moe_bank* gate, const dew_moe_bank* up, const dew_moe_bank* down, int32_t rows) {
+  using namespace dew;
+  auto wants = [rows](const dew_moe_bank* bank) {
+    return bank && bank->layout == DEW_MOE_LAYOUT_PREPARED && bank->format == DEW_MOE_W_MXFP4 && bank->width % 256 == 0 &&
+           bank->experts >= 1 && rows / bank->experts >= DEW_MOE_SPLIT_ROWS_FROM;
+  };
+  return wants(gate) && wants(up) && wants(down) && gate->experts == up->experts && gate->depth == up->depth &&
+                 gate->width == up->width && down->experts == gate->experts && down->depth == gate->width &&
+                 down->depth <= kMaxBlockScaleDepth
+             ? 1
+             : 0;
+}
+
+namespace dew {
+
+struct SplitMlpWorkspace {
+  size_t offsets, x_split, x_scale, hidden_split, hidden_scales, bytes;
+};
+
+static SplitMlpWorkspace split_mlp_workspace(int64_t tokens, int64_t rows, int64_t depth, int64_t hidden_width, int64_t experts) {
+  auto rounded = [](size_t bytes) { return (bytes + 255) / 256 * 256; };
+  SplitMlpWorkspace w{};
+  size_t at = 0;
+  w.offsets = at, at += rounded(static_cast<size_t>(experts + 1) * sizeof(int32_t));
+  w.x_split = at, at += rounded(static_cast<size_t>(tokens) * depth * 2);
+  w.x_scale = at, at += rounded(static_cast<size_t>(tokens));
+  w.hidden_split = at, at += rounded(static_cast<size_t>(rows) * hidden_width * 2);
+  w.hidden_scales = at, at += rounded(static_cast<size_t>(rows) * block_scale_pitch(static_cast<int>(hidden_width)));
+  w.bytes = at + 256;  // room to align the caller's base
+  return w;
+}
+
+}  // namespace dew
+
+extern "C" size_t dew_moe_swiglu_mlp_split_workspace_bytes(int32_t tokens, int32_t rows, int32_t depth, int32_t hidden_width,
+                                                           int32_t experts) {
+  if (tokens < 0 || rows < 0 || depth < 0 || hidden_width < 0 || experts < 0) return 0;
+  return dew::split_mlp_workspace(tokens, rows, depth, hidden_width, experts).bytes;
+}
+
+extern "C" int dew_moe_swiglu_mlp_split(const void* x, int32_t tokens, const int32_t* gather, const int32_t* offsets,
+                                        const int32_t* group_sizes, const dew_moe_bank* gate, const dew_moe_bank* up,
+                                        const dew_moe_bank* down, const int32_t* scatter, void* out, int32_t rows,
+                                        int32_t second_term, void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace dew;
+  const char* who = "dew_moe_swiglu_mlp_split";
+  if (int rc = check_bank(who, gate, "gate")) return rc;
+  if (int rc = check_bank(who, up, "up")) return rc;
+  if (int rc = check_bank(who, down, "down")) return rc;
+  DEW_REQUIRE(tokens >= 0 && rows >= 0, "%s: tokens %d rows %d", who, tokens, rows);
+  DEW_REQUIRE(second_term == DEW_MOE_SECOND_TERM_E4M3 || second_term == DEW_MOE_SECOND_TERM_E2M3,
+              "%s: the rows' second term %d is neither e4m3 (0) nor e2m3 (1)", who, second_term);
+  DEW_REQUIRE(down->experts == gate->experts && down->depth == gate->width, "%s: down [%d, %d, %d] does not follow gate [%d, %d, %d]", who,
+              down->experts, down->depth, down->width, gate->experts, gate->depth, gate->width);
+  if (rows == 0 || tokens == 0) return DEW_MOE_OK;
+  DEW_REQUIRE((offsets != nullptr) != (group_sizes != nullptr), "%s: the groups come as offsets [E + 1] or as group_sizes [E], one of them", who);
+  DEW_REQUIRE(gather != nullptr || rows <= tokens, "%s: %d rows of %d tokens need a gather", who, rows, tokens);
+  const SplitMlpWorkspace w = split_mlp_workspace(tokens, rows, gate->depth, gate->width, gate->experts);
+  DEW_REQUIRE(workspace && workspace_bytes >= w.bytes, "%s: workspace of %zu bytes, need %zu (dew_moe_swiglu_mlp_split_workspace_bytes)", who,
+              workspace_bytes, w.bytes);
+  uint8_t* base = reinterpret_cast<uint8_t*>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~static_cast<uintptr_t>(255));
+  if (group_sizes != nullptr) {
+    int32_t* formed = reinterpret_cast<int32_t*>(base + w.offsets);
+    if (int rc = dew_moe_group_offsets(group_sizes, gate->experts, formed, stream)) return rc;
+    offsets = formed;
+  }
+  void* x_split = base + w.x_split;
+  uint8_t* x_scale = base + w.x_scale;
+  void* hidden_split = base + w.hidden_split;
+  uint8_t* hidden_scales = base + w.hidden_scales;
+  if (second_term == DEW_MOE_SECOND_TERM_E2M3) {
+    if (int rc = dew_moe_split_rows_fp6(x, x_split, x_scale, tokens, gate->depth, stream)) return rc;
+    if (int rc = dew_moe_gateup_swiglu_split_fp6_out(x_split, x_scale, gather, offsets, gate, up, hidden_split, hidden_scales, rows, stream)) return rc;
+  } else {
+    if (int rc = dew_moe_split_rows(x, x_split, x_scale, tokens, gate->depth, stream)) return rc;
+    if (int rc = dew_moe_gateup_swiglu_split_out(x_split, x_scale, gather, offsets, gate, up, hidden_split, hidden_scales, rows, stream)) return rc;
+  }
+  return dew_moe_grouped_gemm_split_blocks(hidden_split, hidden_scales, nullptr, offsets, down, nullptr, scatter, out, rows, stream);
+}
+
 extern "C" int dew_moe_gateup_interleaved(const void* x, const int32_t* gather, const int32_t* offsets,
                                           const dew_moe_bank* gate_up, const float* bias, float limit, void* hidden,
                                           int32_t rows, void* stream) {

@@ -183,6 +183,52 @@ ffi::Error GateUpSwiglu(hipStream_t stream, ffi::AnyBuffer x, ffi::AnyBuffer gat
   return ffi::Error::Success();
 }
 
+// ---- dew_moe_swiglu_mlp_ffi: the routed experts' whole SwiGLU MLP (`ExpertMLP._project`, src/dew/nn/moe.py:1305-1326):
+// x bf16[T, D], the gate's, up's and down's prepared banks, group_sizes s32[E], gather s32[rows] | s32[0],
+// scatter s32[rows] | s32[0] -> out bf16[rows, D_out]. Where the library's rule says so (dew_moe_prefers_split_rows:
+// MXFP4 banks, groups of hundreds of rows) the rows run as two e4m3 terms on the scaled matrix instruction
+// (dew_moe_swiglu_mlp_split, its intermediates in XLA's scratch); else the paired launch and the down launch on bf16
+// operands, the hidden rows in scratch. `second_term` = DEW_MOE_SECOND_TERM_* for the split form. ----
+ffi::Error SwigluMlp(hipStream_t stream, ffi::ScratchAllocator scratch, ffi::AnyBuffer x, ffi::AnyBuffer gate_prepared,
+                     ffi::AnyBuffer gate_scales, ffi::AnyBuffer gate_tensor_scale, ffi::AnyBuffer up_prepared, ffi::AnyBuffer up_scales,
+                     ffi::AnyBuffer up_tensor_scale, ffi::AnyBuffer down_prepared, ffi::AnyBuffer down_scales,
+                     ffi::AnyBuffer down_tensor_scale, ffi::Buffer<ffi::S32> group_sizes, ffi::AnyBuffer gather, ffi::AnyBuffer scatter,
+                     ffi::Result<ffi::AnyBuffer> out, int32_t format, int32_t experts, int32_t depth, int32_t hidden_width,
+                     int32_t width, int32_t second_term) {
+  constexpr const char* kTarget = "dew_moe_swiglu_mlp";
+  if (!is(x, ffi::BF16, 2) || !is(*out, ffi::BF16, 2) || group_sizes.dimensions().size() != 1 || group_sizes.dimensions()[0] != experts)
+    return misshaped(kTarget, "x bf16[T, D], group_sizes s32[E], out bf16[rows, D_out]");
+  const int64_t tokens = x.dimensions()[0], rows = out->dimensions()[0];
+  auto indices_fit = [rows](const ffi::AnyBuffer& index) {
+    return index.element_count() == 0 || (index.element_type() == ffi::S32 && static_cast<int64_t>(index.element_count()) >= rows);
+  };
+  if (x.dimensions()[1] != depth || out->dimensions()[1] != width || (gather.element_count() == 0 && rows > tokens) ||
+      !indices_fit(gather) || !indices_fit(scatter))
+    return misshaped(kTarget, "the extents of x, the banks, gather, scatter and out do not chain");
+  dew_moe_bank gate{}, up{}, down{};
+  if (ffi::Error error = bank_of(kTarget, format, experts, depth, hidden_width, gate_prepared, gate_scales, gate_tensor_scale, &gate); error.failure()) return error;
+  if (ffi::Error error = bank_of(kTarget, format, experts, depth, hidden_width, up_prepared, up_scales, up_tensor_scale, &up); error.failure()) return error;
+  if (ffi::Error error = bank_of(kTarget, format, experts, hidden_width, width, down_prepared, down_scales, down_tensor_scale, &down); error.failure()) return error;
+  if (dew_moe_prefers_split_rows(&gate, &up, &down, static_cast<int32_t>(rows))) {
+    const size_t bytes = dew_moe_swiglu_mlp_split_workspace_bytes(static_cast<int32_t>(tokens), static_cast<int32_t>(rows), depth, hidden_width, experts);
+    void* workspace = scratch_of(scratch, bytes);
+    if (workspace == nullptr) return misshaped(kTarget, "XLA's scratch allocator has no room for the split rows");
+    if (dew_moe_swiglu_mlp_split(x.untyped_data(), static_cast<int32_t>(tokens), present<const int32_t*>(gather), nullptr,
+                                 group_sizes.typed_data(), &gate, &up, &down, present<const int32_t*>(scatter), out->untyped_data(),
+                                 static_cast<int32_t>(rows), second_term, workspace, bytes, stream))
+      return refused(kTarget);
+    return ffi::Error::Success();
+  }
+  void* hidden = scratch_of(scratch, static_cast<size_t>(rows) * hidden_width * 2);
+  if (hidden == nullptr) return misshaped(kTarget, "XLA's scratch allocator has no room for the hidden rows");
+  if (dew_moe_gateup_swiglu_sizes(x.untyped_data(), present<const int32_t*>(gather), group_sizes.typed_data(), &gate, &up, hidden,
+                                  static_cast<int32_t>(rows), stream) ||
+      dew_moe_grouped_gemm_sizes(hidden, nullptr, group_sizes.typed_data(), &down, nullptr, present<const int32_t*>(scatter),
+                                 out->untyped_data(), static_cast<int32_t>(rows), stream))
+    return refused(kTarget);
+  return ffi::Error::Success();
+}
+
 // ---- dew_moe_combine_ffi: slots bf16[T, k, D], weights f32[T, k], addend bf16[T, D] | bf16[0] -> out bf16[T, D] ----
 ffi::Error Combine(hipStream_t stream, ffi::AnyBuffer slots, ffi::AnyBuffer weights, ffi::AnyBuffer addend, ffi::Result<ffi::AnyBuffer> out) {
   constexpr const char* kTarget = "dew_moe_combine";
@@ -275,6 +321,31 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(dew_moe_gateup_swiglu_ffi, GateUpSwiglu,
                                   .Attr<int32_t>("experts")
                                   .Attr<int32_t>("depth")
                                   .Attr<int32_t>("width"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(dew_moe_swiglu_mlp_ffi, SwigluMlp,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Ctx<ffi::ScratchAllocator>()
+                                  .Arg<ffi::AnyBuffer>()   // x
+                                  .Arg<ffi::AnyBuffer>()   // gate: prepared, scales, tensor_scale
+                                  .Arg<ffi::AnyBuffer>()
+                                  .Arg<ffi::AnyBuffer>()
+                                  .Arg<ffi::AnyBuffer>()   // up
+                                  .Arg<ffi::AnyBuffer>()
+                                  .Arg<ffi::AnyBuffer>()
+                                  .Arg<ffi::AnyBuffer>()   // down
+                                  .Arg<ffi::AnyBuffer>()
+                                  .Arg<ffi::AnyBuffer>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()   // group_sizes
+                                  .Arg<ffi::AnyBuffer>()   // gather
+                                  .Arg<ffi::AnyBuffer>()   // scatter
+                                  .Ret<ffi::AnyBuffer>()
+                                  .Attr<int32_t>("format")
+                                  .Attr<int32_t>("experts")
+                                  .Attr<int32_t>("depth")
+                                  .Attr<int32_t>("hidden_width")
+                                  .Attr<int32_t>("width")
+                                  .Attr<int32_t>("second_term"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(dew_moe_combine_ffi, Combine,
                               ffi::Ffi::Bind()

@@ -220,8 +220,6 @@ def swiglu_mlp_on_split_rows(lhs: torch.Tensor, gate, up, down, group_sizes, *, 
     rows = lhs.shape[0] if gather is None else gather.numel()
     if not ops.prefers_split_pair(first, second, third, rows):
         return None
-    groups = GroupSizes.of(group_sizes)
-    fp6 = SPLIT_SECOND_TERM == "e2m3"
-    pieces = ops.split_rows_fp6(lhs) if fp6 else ops.split_rows(lhs)
-    hidden = ops.gateup_swiglu_split_out(*pieces, first, second, groups.offsets, gather=gather, fp6=fp6)
-    return ops.grouped_gemm_split_blocks(*hidden, third, groups.offsets, scatter=scatter)
+    groups = GroupSizes.operands(group_sizes)   # a caller's plain group sizes go in as they are: the call forms their prefix
+    return ops.swiglu_mlp_split(lhs, first, second, third, groups["offsets"], sizes=groups.get("sizes"), gather=gather,
+                                scatter=scatter, fp6=SPLIT_SECOND_TERM == "e2m3")

@@ -469,9 +469,31 @@ MAX_BLOCK_SCALE_DEPTH = 24576
 def prefers_split_pair(gate: PreparedBank, up: PreparedBank, down: PreparedBank, rows: int) -> bool:
     """Whether a SwiGLU expert MLP of `rows` rows is better run as `gateup_swiglu_split_out` then
     `grouped_gemm_split_blocks`: all three banks as `prefers_split` wants them, the down bank's depth the gate's width
-    and within the LDS's room for its scales."""
-    return prefers_split(gate, rows) and prefers_split(up, rows) and prefers_split(down, rows) and \
-        gate.shape == up.shape and down.shape[1] == gate.shape[2] and down.shape[1] <= MAX_BLOCK_SCALE_DEPTH
+    and within the LDS's room for its scales. The library's own rule (`dew_moe_prefers_split_rows`), so that a caller
+    through the C ABI alone decides the same way."""
+    return bool(_lib.library().dew_moe_prefers_split_rows(gate.descriptor, up.descriptor, down.descriptor, rows))
+
+
+def swiglu_mlp_split(x: torch.Tensor, gate: PreparedBank, up: PreparedBank, down: PreparedBank, offsets: torch.Tensor | None, *,
+                     sizes: torch.Tensor | None = None, gather: torch.Tensor | None = None, scatter: torch.Tensor | None = None,
+                     rows: int | None = None, fp6: bool = False) -> torch.Tensor:
+    """The SwiGLU expert MLP on split rows as one call (`dew_moe_swiglu_mlp_split`): `split_rows`, `gateup_swiglu_split_out`
+    and `grouped_gemm_split_blocks` with their intermediates in one workspace. The groups as `offsets` or as `sizes`."""
+    _device(x, "x", torch.bfloat16)
+    experts, depth, width = gate.shape
+    if x.dim() != 2 or x.shape[1] != depth:
+        raise KernelError(f"x {tuple(x.shape)} does not match the gate bank's depth {depth}")
+    rows = _product_rows(x, "x", offsets, experts, gather, scatter, rows, sizes)
+    tokens = x.shape[0]
+    lib = _lib.library()
+    workspace = torch.empty(lib.dew_moe_swiglu_mlp_split_workspace_bytes(tokens, rows, depth, width, experts), dtype=torch.uint8, device=x.device)
+    out = torch.empty((rows, down.shape[2]), dtype=torch.bfloat16, device=x.device)
+    _lib.check(lib.dew_moe_swiglu_mlp_split(_ptr(x), tokens, _ptr(gather), _ptr(offsets), _ptr(None if offsets is not None else sizes),
+                                            gate.descriptor, up.descriptor,
+                                            down.descriptor, _ptr(scatter), _ptr(out), rows,
+                                            _lib.SECOND_TERM_E2M3 if fp6 else _lib.SECOND_TERM_E4M3, _ptr(workspace), workspace.numel(),
+                                            _stream()), "dew_moe_swiglu_mlp_split")
+    return out
 
 
 def grouped_gemm_split(split: torch.Tensor, scale: torch.Tensor, bank: PreparedBank, offsets: torch.Tensor, *,

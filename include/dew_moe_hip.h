@@ -264,6 +264,25 @@ int dew_moe_grouped_gemm_split_blocks(const void* x_split, const uint8_t* x_scal
                                       const int32_t* offsets, const dew_moe_bank* w, const float* bias,
                                       const int32_t* scatter, void* out, int32_t rows, void* stream);
 
+/* The SwiGLU expert MLP on split rows as one call (`ExpertMLP._project`, src/dew/nn/moe.py:1305-1326: paired gate/up
+ * products, `gated_product('swiglu')`, the down product): dew_moe_split_rows (or _fp6) of x[tokens, D], then
+ * dew_moe_gateup_swiglu_split_out and dew_moe_grouped_gemm_split_blocks, the split rows and the split hidden rows in
+ * `workspace` (dew_moe_swiglu_mlp_split_workspace_bytes; any alignment). The groups come as `offsets [E + 1]` or as
+ * `group_sizes [E]` (the reference FFI's operand, kernels/cutlass/ffi.cu:185-198), the other null. out is bf16 [rows, down
+ * width], row i at scatter[i] where scatter is given. dew_moe_prefers_split_rows is the rule by which the host mirror takes
+ * this form (1) or the bf16-operand launches (0): three prepared MXFP4 banks of whole 256-column strips that chain, the
+ * down bank's depth within the LDS's room for a tile's scales, and groups averaging DEW_MOE_SPLIT_ROWS_FROM rows or more
+ * (measured: 1.20 times the bf16 launches at 900 rows a group, 1.05 at 512 to 768, 1.08 at 384, 0.975 at 256).       */
+enum { DEW_MOE_SECOND_TERM_E4M3 = 0, DEW_MOE_SECOND_TERM_E2M3 = 1 };
+#define DEW_MOE_SPLIT_ROWS_FROM 384
+int dew_moe_prefers_split_rows(const dew_moe_bank* gate, const dew_moe_bank* up, const dew_moe_bank* down, int32_t rows);
+size_t dew_moe_swiglu_mlp_split_workspace_bytes(int32_t tokens, int32_t rows, int32_t depth, int32_t hidden_width, int32_t experts);
+int dew_moe_swiglu_mlp_split(const void* x /* bf16 [tokens, D] */, int32_t tokens, const int32_t* gather /* nullable [rows] */,
+                             const int32_t* offsets /* [E + 1] or null */, const int32_t* group_sizes /* [E] or null */,
+                             const dew_moe_bank* gate, const dew_moe_bank* up, const dew_moe_bank* down,
+                             const int32_t* scatter /* nullable [rows] */, void* out, int32_t rows,
+                             int32_t second_term /* DEW_MOE_SECOND_TERM_* */, void* workspace, size_t workspace_bytes, void* stream);
+
 /* The first product of that pair with the rows' second term in FP6 (no counterpart in the reference). dew_moe_split_rows_fp6:
  * x = s hi + t lo with hi = e4m3(x / s) under one power-of-two scale s a row (scale[row], as dew_moe_split_rows) and
  * lo = e2m3((x - s hi) / t) under t, one power of two for every 32 depths. Each 64 depths of a row are 128 bytes: for

@@ -433,6 +433,37 @@ def test_the_expert_mlp_stays_on_split_rows_without_a_pass_between_its_products(
     assert (out == plain).mean() > 0.9
 
 
+@pytest.mark.parametrize("fp6", [False, True])
+def test_the_expert_mlp_on_split_rows_as_one_call_is_its_three_launches(ops, fp6):
+    """`dew_moe_swiglu_mlp_split`: the split of the rows, the gate/up launch and the down launch with their intermediates
+    in one workspace, given the groups' offsets or their plain sizes: the bits of the three calls, rows past the groups
+    zero, the scatter honoured."""
+    sizes = [700, 0, 290, 5]
+    depth, width, out_width = 512, 768, 256
+    gate, x, offsets = grouped_case("mxfp4", len(sizes), depth, width, sizes, seed=31)
+    up, _, _ = grouped_case("mxfp4", len(sizes), depth, width, sizes, seed=32)
+    down, _, _ = grouped_case("mxfp4", len(sizes), width, out_width, sizes, seed=33)
+    rng = np.random.default_rng(7)
+    padded = x.shape[0] + 9
+    gather = torch.from_numpy(np.concatenate([rng.integers(0, x.shape[0], size=x.shape[0]), np.zeros(9)]).astype(np.int32)).cuda()
+    scatter = torch.from_numpy(rng.permutation(padded).astype(np.int32)).cuda()
+    xd, od, sd = x.cuda(), torch.from_numpy(offsets).cuda(), torch.tensor(sizes, dtype=torch.int32).cuda()
+    pg, pu, pd = (ops.prepare(bank.to("cuda")) for bank in (gate, up, down))
+    pieces = ops.split_rows_fp6(xd) if fp6 else ops.split_rows(xd)
+    hidden = ops.gateup_swiglu_split_out(*pieces, pg, pu, od, gather=gather, rows=padded, fp6=fp6)
+    apart = ops.grouped_gemm_split_blocks(*hidden, pd, od, scatter=scatter, rows=padded)
+    with_offsets = ops.swiglu_mlp_split(xd, pg, pu, pd, od, gather=gather, scatter=scatter, rows=padded, fp6=fp6)
+    with_sizes = ops.swiglu_mlp_split(xd, pg, pu, pd, None, sizes=sd, gather=gather, scatter=scatter, rows=padded, fp6=fp6)
+    assert with_offsets.shape == (padded, out_width)
+    assert torch.equal(with_offsets, apart) and torch.equal(with_sizes, apart)
+    assert not bool(apart[scatter[x.shape[0]:].long()].any())
+    # no gather: the rows as they lie
+    straight = ops.swiglu_mlp_split(xd, pg, pu, pd, od, fp6=fp6)
+    assert torch.equal(straight, ops.grouped_gemm_split_blocks(*ops.gateup_swiglu_split_out(*pieces, pg, pu, od, fp6=fp6), pd, od))
+    with pytest.raises(ops.KernelError, match="asked of x"):
+        ops.swiglu_mlp_split(xd, pg, pu, pd, od, rows=padded)
+
+
 @pytest.mark.parametrize("quant", ["fp8_block", "fp8_channel", "mxfp4", "nvfp4", "bf16"])
 def test_a_layer_of_a_stacked_bank_is_read_where_it_lies(ops, quant):
     """`Layered(stack, layer)`: the grouped product of one layer's experts out of a bank stacking three layers', from

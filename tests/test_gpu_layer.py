@@ -106,8 +106,8 @@ def test_large_groups_on_mxfp4_banks_run_on_split_rows_and_agree_with_the_bf16_l
     layer, variables = layer_and_variables(case, data)
     x, logits = data["x"].cuda(), data["logits"].cuda()
     calls = []
-    split_out = ops.gateup_swiglu_split_out
-    monkeypatch.setattr(ops, "gateup_swiglu_split_out", lambda *a, **k: calls.append(1) or split_out(*a, **k))
+    on_split_rows = ops.swiglu_mlp_split
+    monkeypatch.setattr(ops, "swiglu_mlp_split", lambda *a, **k: calls.append(1) or on_split_rows(*a, **k))
     assert gemm.SPLIT_ROWS and gemm.SPLIT_SECOND_TERM == "e4m3"
     got = layer.apply(variables, x, logits=logits).float().cpu().numpy()            # two e4m3 terms: the rows' bf16 values exactly
     assert calls == [1]
