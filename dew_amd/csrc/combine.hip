@@ -53,7 +53,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const bf16_t* __restrict__
 // `limit` > 0: the gate clamped from above and the up projection both ways before their product (`swiglu_clamped`,
 // src/dew/nn/activations.py:327-333); the limit enters as the bf16 the operands' dtype rounds it to.
 __global__ __launch_bounds__(256) void swiglu_kernel(const bf16_t* __restrict__ gate, const bf16_t* __restrict__ up,
-                                                     bf16_t* __restrict__ hidden, long long chunks, float limit) {
+                                                     bf16_t* __restrict__ hidden, long long chunks, float limit, int activation) {
   for (long long item = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; item < chunks;
        item += static_cast<long long>(gridDim.x) * blockDim.x) {
     const Bf16x8 g = reinterpret_cast<const Bf16x8*>(gate)[item];
@@ -69,7 +69,7 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const bf16_t* __restrict__ 
         gi = fminf(gi, limit);
         ui = fminf(fmaxf(ui, -limit), limit);
       }
-      h.v[i] = swiglu_rounded(gi, ui);
+      h.v[i] = activation == DEW_MOE_GATE_GELU_TANH ? geglu_rounded(gi, ui) : swiglu_rounded(gi, ui);
     }
     reinterpret_cast<Bf16x8*>(hidden)[item] = h;
   }
@@ -116,12 +116,19 @@ extern "C" int dew_moe_silu(const void* x, void* out, int64_t count, void* strea
   const long long chunks = count / 8;
   const int blocks = static_cast<int>(min((chunks + 255) / 256, 256ll * 64));
   hipLaunchKernelGGL(swiglu_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<const bf16_t*>(x),
-                     static_cast<const bf16_t*>(nullptr), static_cast<bf16_t*>(out), chunks, 0.0f);
+                     static_cast<const bf16_t*>(nullptr), static_cast<bf16_t*>(out), chunks, 0.0f, DEW_MOE_GATE_SILU);
   return launched("swiglu_kernel");
 }
 
 extern "C" int dew_moe_swiglu_clamped(const void* gate, const void* up, float limit, void* hidden, int64_t count, void* stream) {
+  return dew_moe_gated_product(gate, up, DEW_MOE_GATE_SILU, limit, hidden, count, stream);
+}
+
+extern "C" int dew_moe_gated_product(const void* gate, const void* up, int32_t activation, float limit, void* hidden, int64_t count,
+                                     void* stream) {
   using namespace dew;
+  DEW_REQUIRE(activation == DEW_MOE_GATE_SILU || activation == DEW_MOE_GATE_GELU_TANH,
+              "dew_moe_gated_product: the gate's activation %d is neither silu (0: swiglu) nor the tanh gelu (1: geglu)", activation);
   DEW_REQUIRE(limit >= 0.0f, "dew_moe_swiglu: the clamp limit %g must be positive (0: none)", static_cast<double>(limit));
   DEW_REQUIRE(count >= 0 && count % 8 == 0, "dew_moe_swiglu: count %lld is not a multiple of 8", static_cast<long long>(count));
   if (count == 0) return DEW_MOE_OK;
@@ -131,6 +138,6 @@ extern "C" int dew_moe_swiglu_clamped(const void* gate, const void* up, float li
   const int blocks = static_cast<int>(min((chunks + 255) / 256, 256ll * 64));
   hipLaunchKernelGGL(swiglu_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
                      static_cast<const bf16_t*>(gate), static_cast<const bf16_t*>(up), static_cast<bf16_t*>(hidden),
-                     chunks, bf16_round_host(limit));
+                     chunks, bf16_round_host(limit), activation);
   return launched("swiglu_kernel");
 }

@@ -46,6 +46,19 @@ __device__ __forceinline__ bf16_t swiglu_rounded(float gate_sum, float up_sum) {
   return f32_to_bf16(activated * u);
 }
 
+// GeGLU with the tanh GELU (`gated_product('geglu')` over `gelu_tanh`, src/dew/nn/activations.py:57-69, 267-278): the
+// activation g * logistic(sqrt(8 / pi) (g + 0.044715 g^3)) in fp32 in that order of operations, rounded to bf16, then the
+// product with the up projection rounded again. Compile with contraction off: the reference's fp32 steps each round.
+__device__ __forceinline__ bf16_t geglu_rounded(float gate_sum, float up_sum) {
+  const float g = bf16_round(gate_sum), u = bf16_round(up_sum);
+  const float cube = (g * g) * g;
+  const float inner = 1.5957691216057308f * (g + 0.044715f * cube);
+  const float e = __builtin_amdgcn_exp2f(inner * -1.44269504088896340736f);
+  const float sig = __builtin_amdgcn_rcpf(1.0f + e);
+  const float activated = bf16_round(g * sig);
+  return f32_to_bf16(activated * u);
+}
+
 // GPT-OSS's gating of one (gate, up) pair already rounded to bf16 (src/dew/nn/gpt_oss.py:120-121 over
 // src/dew/nn/activations.py:72-74,327-333): gate clamped from above and up both ways by `limit`, then
 // (up + 1) * gate * logistic(1.702 gate) with every operation rounded to bf16 as an array of that dtype

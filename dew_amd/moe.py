@@ -253,8 +253,8 @@ class ExpertMLP(_Module):
     product (the reference's arrangement); the results are bit-identical."""
 
     def __post_init__(self):
-        if self.activation != "swiglu":
-            raise ValueError(f"activation {self.activation!r}: the HIP experts are SwiGLU experts")
+        if self.activation not in ops.GATES:
+            raise ValueError(f"activation {self.activation!r}: the HIP experts gate by one of {list(ops.GATES)}")
         if self.dispatch not in ("auto", "global"):
             raise ValueError(f"dispatch {self.dispatch!r}: one device sorts its slots locally ('global')")
         if self.scale_inputs:
@@ -270,12 +270,13 @@ class ExpertMLP(_Module):
     def _project(self, tokens: Gathered, sizes: GroupSizes, kernels) -> torch.Tensor:
         """src/dew/nn/moe.py:1305-1326."""
         gate_w, up_w, down_w = kernels
-        if self.swiglu_limit is not None:
+        if self.swiglu_limit is not None or self.activation != "swiglu":
             # the clamp sits between the paired product and the gating (`swiglu_clamped`, src/dew/nn/activations.py:327-333):
-            # the reference's own unfused arrangement, with the clamp in the SwiGLU kernel
+            # the reference's own unfused arrangement, with the clamp in the gating kernel; so does a GeGLU gate (Gemma's
+            # experts), which the launches' fused epilogue does not compute
             gate, up = paired_projections(tokens, gate_w, up_w, sizes, self.dtype, self.implementation, self.precision)
-            return expert_projection(ops.swiglu(gate, up, self.swiglu_limit), down_w, sizes, self.dtype, self.implementation,
-                                     self.precision, scatter=tokens.slots)
+            return expert_projection(ops.gated_product(gate, up, self.activation, self.swiglu_limit), down_w, sizes, self.dtype,
+                                     self.implementation, self.precision, scatter=tokens.slots)
         if self.fused and self.dtype in (None, torch.bfloat16):
             # large groups on MXFP4 banks: both launches on the scaled matrix instruction, the hidden rows never in bf16
             out = gemm.swiglu_mlp_on_split_rows(tokens.tokens, gate_w, up_w, down_w, sizes, gather=tokens.rows,

@@ -377,16 +377,27 @@ def gateup_swiglu(x: torch.Tensor, gate: PreparedBank, up: PreparedBank, offsets
     return hidden
 
 
-def swiglu(gate: torch.Tensor, up: torch.Tensor, limit: float | None = None) -> torch.Tensor:
-    """`bf16(bf16(silu(gate)) * up)`; with `limit`, the gate first clamped from above and up both ways by it
-    (the reference's `swiglu_clamped`)."""
+GATES = {"swiglu": _lib.GATE_SILU, "geglu": _lib.GATE_GELU_TANH}
+"""The gated activations the kernels compute (the reference's `gated_product`; its erf form 'geglu_exact' is not one)."""
+
+
+def gated_product(gate: torch.Tensor, up: torch.Tensor, activation: str = "swiglu", limit: float | None = None) -> torch.Tensor:
+    """`bf16(bf16(act(gate)) * up)` for `activation` 'swiglu' (silu) or 'geglu' (the tanh GELU); with `limit`, the gate
+    first clamped from above and up both ways by it (the reference's `swiglu_clamped`)."""
+    if activation not in GATES:
+        raise KernelError(f"the gate's activation is one of {list(GATES)}, got {activation!r}")
     _device(gate, "gate", torch.bfloat16), _device(up, "up", torch.bfloat16)
     if gate.shape != up.shape:
         raise KernelError(f"gate {tuple(gate.shape)} and up {tuple(up.shape)} differ")
     hidden = torch.empty_like(gate)
-    _lib.check(_lib.library().dew_moe_swiglu_clamped(_ptr(gate), _ptr(up), 0.0 if limit is None else float(limit), _ptr(hidden),
-                                                     gate.numel(), _stream()), "dew_moe_swiglu")
+    _lib.check(_lib.library().dew_moe_gated_product(_ptr(gate), _ptr(up), GATES[activation], 0.0 if limit is None else float(limit),
+                                                    _ptr(hidden), gate.numel(), _stream()), "dew_moe_gated_product")
     return hidden
+
+
+def swiglu(gate: torch.Tensor, up: torch.Tensor, limit: float | None = None) -> torch.Tensor:
+    """`gated_product` of 'swiglu'."""
+    return gated_product(gate, up, "swiglu", limit)
 
 
 def silu(x: torch.Tensor) -> torch.Tensor:

@@ -404,6 +404,12 @@ int dew_moe_swiglu(const void* gate, const void* up, void* hidden, int64_t count
 /* The same with the gate clamped from above and the up projection both ways by `limit` before their product
  * (`swiglu_clamped`, src/dew/nn/activations.py:327-333: DeepSeek V4's and GLM's experts); limit 0 = none.  */
 int dew_moe_swiglu_clamped(const void* gate, const void* up, float limit, void* hidden, int64_t count, void* stream);
+/* `gated_product(activation)` for the gates the reference's gated MLPs name besides SwiGLU (src/dew/nn/activations.py:255-265,
+ * 336-356): DEW_MOE_GATE_SILU is dew_moe_swiglu_clamped; DEW_MOE_GATE_GELU_TANH is 'geglu', the tanh GELU in its logistic
+ * form g * logistic(sqrt(8 / pi) (g + 0.044715 g^3)) (`gelu_tanh`, :57-69: Gemma's experts, src/dew/nn/gemma4_moe.py:84),
+ * with the same two roundings and the same optional clamp.                                                           */
+enum { DEW_MOE_GATE_SILU = 0, DEW_MOE_GATE_GELU_TANH = 1 };
+int dew_moe_gated_product(const void* gate, const void* up, int32_t activation, float limit, void* hidden, int64_t count, void* stream);
 /* The activation alone: out = bf16(x * logistic(x)), formed in fp32 and rounded once (`silu`, src/dew/nn/activations.py:100-106),
  * which routed value experts pass each chosen projection through (src/dew/nn/value_experts.py:79-82).      */
 int dew_moe_silu(const void* x /* bf16 [count] */, void* out /* bf16 [count] */, int64_t count, void* stream);

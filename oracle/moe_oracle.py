@@ -25,6 +25,8 @@ What pins each function (tests/test_oracle_golden.py):
 * `grouped_matmul`: tools/grouped_oracle.py:20-27 semantics (float64 per-group product) on integer inputs,
   where fp32 sums are exact.
 
+* `geglu`: the reference's logistic form of the tanh GELU against the textbook `0.5 x (1 + tanh(sqrt(2 / pi) (x + 0.044715
+  x^3)))` in float64 on every bf16 (a wrong constant, sign or power fails it), and its two roundings on hand cases.
 * `silu` / `routed_values` (routed value experts, src/dew/nn/value_experts.py): the reference holds no vectors for the
   layer alone (its fixture is a whole model's logits); `silu` is `swiglu`'s activation with its one rounding, checked
   against `swiglu(x, 1)`, a float64 `x / (1 + e^-x)` and on every bf16; `routed_values` against a token-by-token
@@ -857,6 +859,30 @@ def swiglu(gate, up, *, dtype="bfloat16", limit=None, exp=np.exp):
     return bf16_round((activated * up).astype(F32))
 
 
+def geglu(gate, up, *, dtype="bfloat16", limit=None, exp=np.exp):
+    """`gated_product('geglu')` (src/dew/nn/activations.py:255-278 over `gelu_tanh`, :57-69): the tanh GELU in its logistic
+    form `g * logistic(sqrt(8 / pi) (g + 0.044715 g^3))`, every step an fp32 operation in that order, rounded to bf16,
+    then the product with `u` rounded again; fp32 rounds nowhere. The clamp as in `swiglu`."""
+    gate, up = np.asarray(gate, F32), np.asarray(up, F32)
+    if limit is not None:
+        gate, up = np.minimum(gate, F32(limit)), np.clip(up, F32(-limit), F32(limit))
+
+    def activated(g):
+        cube = ((g * g).astype(F32) * g).astype(F32)
+        inner = (F32(np.sqrt(8 / np.pi)) * (g + (F32(0.044715) * cube).astype(F32)).astype(F32)).astype(F32)
+        with np.errstate(over="ignore"):
+            sig = (F32(1) / (F32(1) + exp(-inner).astype(F32)).astype(F32)).astype(F32)
+        return (g * sig).astype(F32)
+
+    if dtype != "bfloat16":
+        return (activated(gate) * up).astype(F32)
+    gate, up = bf16_round(gate), bf16_round(up)
+    return bf16_round((bf16_round(activated(gate)) * up).astype(F32))
+
+
+GATED_PRODUCTS = {"swiglu": swiglu, "geglu": geglu}
+
+
 def silu(x, *, dtype="bfloat16", exp=np.exp):
     """`silu` (src/dew/nn/activations.py:100-106): `x * logistic(x)` in fp32, rounded once to the array's dtype. The
     first of `swiglu`'s two roundings; the same stand-in for the backend's exp."""
@@ -919,7 +945,7 @@ def capacity_admitted(indices, num_experts, capacity_factor):
 
 
 def expert_mlp(x, weights, indices, gate_w, up_w, down_w, *, dtype="bfloat16", factors=(None, None, None),
-               limit=None, capacity_factor=None):
+               limit=None, capacity_factor=None, activation="swiglu"):
     """`ExpertMLP.__call__` (src/dew/nn/moe.py:1335-1353) on one device: sort, gather, paired gate/up
     products, SwiGLU, down product scattered to slot order, combine. The matrices are the dequantized
     `[E, depth, width]` values; `indices [T, k]`, or `[..., length, k]` with `capacity_factor` (each leading row a
@@ -936,7 +962,7 @@ def expert_mlp(x, weights, indices, gate_w, up_w, down_w, *, dtype="bfloat16", f
     rows = x[plan["rows"]]   # (rows past the groups, the dropped slots', are multiplied by no matrix: `grouped_matmul` leaves them zero)
     gate = grouped_matmul(rows, gate_w, plan["sizes"], dtype=dtype, factor=factors[0])
     up = grouped_matmul(rows, up_w, plan["sizes"], dtype=dtype, factor=factors[1])
-    hidden = swiglu(gate, up, dtype=dtype, limit=limit)
+    hidden = GATED_PRODUCTS[activation](gate, up, dtype=dtype, limit=limit)
     projected = grouped_matmul(hidden, down_w, plan["sizes"], dtype=dtype, factor=factors[2])
     slots = np.zeros_like(projected)
     slots[plan["order"]] = projected

@@ -250,6 +250,22 @@ def test_swiglu_kernel_matches_the_oracle_on_every_bf16_gate(ops):
     assert np.abs(got - want)[mismatched].max(initial=0) <= 2 ** -7 * np.abs(want)[mismatched].max(initial=1)
 
 
+def test_geglu_kernel_matches_the_oracle_on_every_bf16_gate(ops):
+    gate = oracle.bf16_from_bits(np.arange(65536, dtype=np.uint16))
+    gate = gate[np.isfinite(gate) & (np.abs(gate) < 1e12)]     # (beyond, the gate's cube overflows fp32: inf - inf on both sides)
+    gate = np.concatenate([gate, np.zeros(-gate.size % 8, np.float32)])
+    up = np.resize(np.array([1.0, -0.75, 3.140625, 1e-3, 100.0, 2 ** -20, -7.0, 0.5], np.float32), gate.shape)
+    for limit in (None, 2.0):
+        want = oracle.geglu(gate, up, limit=limit)
+        got = bf16_np(ops.gated_product(torch.from_numpy(gate).to(torch.bfloat16).cuda(), torch.from_numpy(up).to(torch.bfloat16).cuda(),
+                                        "geglu", limit))
+        mismatched = (got != want) & ~(np.isnan(got) & np.isnan(want))
+        assert mismatched.mean() < 2e-3                    # the hardware exponential against the library's: a last bf16 bit, rarely
+        assert np.abs(got - want)[mismatched].max(initial=0) <= 2 ** -7 * np.abs(want)[mismatched].max(initial=1)
+    with pytest.raises(ops.KernelError, match="activation"):
+        ops.gated_product(torch.zeros(8, dtype=torch.bfloat16, device="cuda"), torch.zeros(8, dtype=torch.bfloat16, device="cuda"), "reglu")
+
+
 def test_combine_weighs_in_fp32_and_rounds_once(ops):
     slots = torch.tensor([[[1.0] * 8, [-1.0] * 8]], dtype=torch.bfloat16)     # tests/test_moe_precision.py:652-674
     weights = torch.tensor([[0.5 + 2 ** -11, 0.5 - 2 ** -11]], dtype=torch.float32)

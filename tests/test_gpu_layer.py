@@ -317,3 +317,32 @@ def test_the_clamped_experts_reproduce_the_references_deepseek_v4_output_and_cap
     assert trace["sizes"].sum() < indices.numel()                                      # something was dropped
     by_max, by_element = oracle.relative_errors(got.float().cpu().numpy().reshape(want.shape), want)
     assert by_max <= TOLERANCE and by_element <= TOLERANCE
+
+
+@pytest.mark.parametrize("quant", ["bf16", "fp8_block", "mxfp4"])
+def test_geglu_experts_run_through_the_layer(quant):
+    """Gemma's experts gate by the tanh GELU (`activation='geglu'`, src/dew/nn/gemma4_moe.py:84): the paired product, the
+    stand-alone gating kernel and the down product against the oracle's `expert_mlp(activation='geglu')`; a SwiGLU layer
+    on the same banks is far from it."""
+    from moe_cases import quantize
+
+    from dew_amd import moe, ops
+
+    rng = np.random.default_rng(17)
+    tokens, experts, top_k, width, hidden = 200, 8, 2, 256, 512
+    x = torch.from_numpy(rng.standard_normal((tokens, width)).astype(np.float32)).to(torch.bfloat16)
+    banks = {name: quantize(torch.from_numpy((rng.standard_normal((experts, d, w)) * 0.08).astype(np.float32)), quant)
+             for name, (d, w) in (("gate", (width, hidden)), ("up", (width, hidden)), ("down", (hidden, width)))}
+    logits = rng.standard_normal((tokens, experts)).astype(np.float32)
+    weights, indices = ops.route(torch.from_numpy(logits).cuda(), top_k)
+    variables = {"params": {}, "quantization": {f"{n}_proj": {"kernel": bank.to("cuda")} for n, bank in banks.items()}}
+    got = moe.ExpertMLP(experts, hidden, width, activation="geglu").apply(variables, x.cuda(), weights, indices).float().cpu().numpy()
+    mats, factors = zip(*(dequantized(banks[name]) for name in ("gate", "up", "down")), strict=True)
+    want, _ = oracle.expert_mlp(x.float().numpy(), weights.cpu().numpy(), indices.cpu().numpy(), *mats, factors=factors, activation="geglu")
+    by_max, by_element = oracle.relative_errors(got, want)
+    assert by_max <= 6e-3 and by_element <= TOLERANCE, (by_max, by_element)
+    assert (got == want).mean() > 0.97
+    swiglu = moe.ExpertMLP(experts, hidden, width).apply(variables, x.cuda(), weights, indices).float().cpu().numpy()
+    assert np.abs(swiglu - want).max() > 0.05 * np.abs(want).max()
+    with pytest.raises(ValueError, match="gate by one of"):
+        moe.ExpertMLP(experts, hidden, width, activation="geglu_exact")

@@ -402,3 +402,27 @@ def test_routed_values_are_each_tokens_weighted_sum_of_its_chosen_experts_activa
             assert np.array_equal(slots[t, j], activated.astype(np.float32))
             total += activated * float(weights[t, j])
         assert np.array_equal(out[t], oracle.bf16_round(total.astype(np.float32))), t
+
+
+def test_geglu_is_the_tanh_gelu_with_the_two_roundings():
+    """The logistic form the reference computes against the textbook tanh form in float64, on every finite bf16 gate;
+    then the product's second rounding, the fp32 mode and the clamp."""
+    every = oracle.bf16_from_bits(np.arange(65536, dtype=np.uint16))
+    every = every[np.isfinite(every) & (np.abs(every) < 1e12)]            # (beyond, x^3 overflows fp32: the reference's too)
+    got = oracle.geglu(every, np.ones_like(every))
+    wide = every.astype(np.float64)
+    z = np.sqrt(2.0 / np.pi) * (wide + 0.044715 * wide ** 3)
+    # the textbook form where float64's 1 + tanh keeps its digits (x > -4); below, the tail the tanh form cancels is held
+    # to the same function written x / (1 + e^(-2 z)) in float64, down to where fp32's e^(-2 z) overflows (x near -10)
+    with np.errstate(over="ignore"):
+        truth = np.where(wide > -4, 0.5 * wide * (1.0 + np.tanh(z)), wide / (1.0 + np.exp(-2.0 * z)))
+    inside = np.abs(truth) > 1e-30
+    rounded = oracle.bf16_round(truth.astype(np.float32))
+    steps = np.abs(oracle.bf16_bits(got[inside]).astype(np.int64) - oracle.bf16_bits(rounded[inside]).astype(np.int64))
+    assert steps.max() <= 1 and (steps == 0).mean() > 0.995
+    assert np.all(np.abs(got[~inside]) <= 1e-30)
+    # gelu(1) = 0.841192 -> bf16 0.83984375 (a bf16 step is 2^-8 there); times up = 3 -> 2.51953125 -> bf16 2.515625
+    assert oracle.geglu(np.float32([1.0]), np.float32([1.0]))[0] == np.float32(0.83984375)
+    assert oracle.geglu(np.float32([1.0]), np.float32([3.0]))[0] == np.float32(2.515625)
+    assert abs(oracle.geglu(np.float32([1.0]), np.float32([3.0]), dtype="float32")[0] - 3 * 0.8411919906082768) < 1e-6
+    assert oracle.geglu(np.float32([5.0]), np.float32([-9.0]), limit=2.0)[0] == oracle.geglu(np.float32([2.0]), np.float32([-2.0]))[0]
