@@ -497,8 +497,17 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
 #pragma unroll
     for (int t = begin.value; t < end.value; ++t) {
 #pragma unroll
-      for (int a = 0; a < kAtoms; ++a)
-        b_regs[set.value][t][a] = *reinterpret_cast<const u32x4_t*>(b_src[t] + (static_cast<size_t>(step) * kAtoms + a) * kAtomBytes);
+      for (int a = 0; a < kAtoms; ++a) {
+        const u32x4_t* from = reinterpret_cast<const u32x4_t*>(b_src[t] + (static_cast<size_t>(step) * kAtoms + a) * kAtomBytes);
+        // Decode-sized groups (the 32-row tiles) read every weight byte once: loaded as non-temporal the stream runs 3 to 6 %
+        // faster (a read-only stream of 16-byte loads measures 7.1 TB/s so hinted against 5.6 to 6.4 without). Taller
+        // tiles keep the plain load: their groups' tiles share weight strips through the L2 (128-row tiles: 2 to 4 % slower
+        // with the hint).
+        if constexpr (BM <= 32)
+          b_regs[set.value][t][a] = __builtin_nontemporal_load(from);
+        else
+          b_regs[set.value][t][a] = *from;
+      }
       if (kFp4 || kMxRows) __builtin_memcpy(&s_regs[set.value][t], b_scale_src[t] + static_cast<size_t>(step) * 128, sizeof(uint32_t));
     }
   };
