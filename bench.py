@@ -218,8 +218,9 @@ def measured_traffic(config):
 
 
 def sustained_rates(device):
-    """What the chip sustains in this run: bf16 MFMA on random operands (TFLOP/s) and a plain copy (GB/s of
-    bytes read plus bytes written), each timed with HIP events over several launches after a warm-up."""
+    """What the chip sustains in this run: bf16 MFMA on random operands (TFLOP/s), a plain copy (GB/s of bytes read
+    plus bytes written) and a read-only stream issued as the decode tiles issue their weight loads (GB/s), each timed
+    with HIP events over several launches after a warm-up."""
     import torch
 
     from bench_aids import probes
@@ -239,7 +240,13 @@ def sustained_rates(device):
     moved = sum(2 * probes.probe_copy(src, dst) for _ in range(5))
     stop.record()
     torch.cuda.synchronize()
-    return round(mfma, 1), round(moved / (start.elapsed_time(stop) * 1e-3) / 1e9, 1)
+    copied = moved / (start.elapsed_time(stop) * 1e-3) / 1e9
+    probes.probe_read(src)
+    start.record()
+    fetched = sum(probes.probe_read(src) for _ in range(5))
+    stop.record()
+    torch.cuda.synchronize()
+    return round(mfma, 1), round(copied, 1), round(fetched / (start.elapsed_time(stop) * 1e-3) / 1e9, 1)
 
 
 def measure(config, args, device, sustained, with_cpu_baseline):
@@ -301,7 +308,7 @@ def measure(config, args, device, sustained, with_cpu_baseline):
     # bandwidth view: the touched experts' gate and up codes read once + activations in, hidden out
     gateup_bytes = (touched + (1 if stepper.fused_shared else 0)) * 2 * case.d_model * case.d_ff * bytes_per_weight + case.tokens * case.d_model * 2 + gateup_rows * case.d_ff * 2
     gateup_gbs = gateup_bytes / (gateup_ms * 1e-3) / 1e9
-    sustained_mfma, sustained_copy = sustained
+    sustained_mfma, sustained_copy, sustained_read = sustained
     if decode:
         roofline = {"bound": "hbm", "achieved": round(gateup_gbs, 1), "peak": PEAKS["hbm_gbs"], "unit": "GB/s"}
     else:
@@ -328,9 +335,11 @@ def measure(config, args, device, sustained, with_cpu_baseline):
                                   f"{COUNTED_FROM[config]}; not measured in this run") if config in COUNTED_KIB else None
     roofline["algorithmic"] = {"per_launch": gateup_bytes if decode else gateup_flops, "unit": "bytes" if decode else "flop"}
     roofline["sustained"] = {"bf16_mfma_random_operands_tflops": sustained_mfma, "plain_copy_gbs": sustained_copy,
-                             "frac_of_sustained": round(roofline["achieved"] / (sustained_copy if decode else sustained_mfma), 4),
-                             "note": "measured in this run by bench_aids' MFMA and copy probes: the rate the chip holds on "
-                                     "random data at its power limit, below the published peak"}
+                             "read_stream_gbs": sustained_read,
+                             "frac_of_sustained": round(roofline["achieved"] / (sustained_read if decode else sustained_mfma), 4),
+                             "note": "measured in this run by bench_aids' probes: the MFMA rate the chip holds on random data at "
+                                     "its power limit, a plain copy, and a read-only stream of non-temporal loads issued as the "
+                                     "decode tiles issue theirs (the reference for an HBM-bound launch)"}
     roofline["kernel"] = "grouped_gemm_kernel<paired gate/up + SwiGLU>" + (
         f" on split rows (v_mfma_scale_f32_32x32x64_f8f6f4, an e4m3 and an {'e2m3' if stepper.fp6 else 'e4m3'} term x FP4)" if stepper.on_split_rows() else "")
     roofline["kernel_ms"] = round(gateup_ms, 4)

@@ -5,6 +5,8 @@
 //                       GEMM kernels can approach on real data.
 //   dew_bench_probe_copy a plain 16-byte-per-lane copy: the HBM rate a streaming kernel sustains, and the known
 //                       traffic the FETCH_SIZE / WRITE_SIZE counters are scaled by.
+//   dew_bench_probe_read a read-only stream issued as the decode tiles issue their weight loads: what HBM delivers to
+//                       that access pattern with no arithmetic behind it.
 //
 // Built into its own small library (libdew_bench_probes.so) beside the benchmarks that use it: it is no part of the
 // MoE kernels' C ABI.
@@ -48,9 +50,29 @@ __global__ __launch_bounds__(256) void probe_copy_kernel(const u32x4_t* __restri
     dst[i] = src[i];
 }
 
+// A read-only stream issued the way the decode tiles read their weights: every wavefront walks 64 KiB segments (a
+// 32-column strip's depth), 1 KiB a load, eight non-temporal loads in flight a lane.
+__global__ __launch_bounds__(256) void probe_read_kernel(const u32x4_t* __restrict__ src, size_t chunks, uint32_t* __restrict__ sink) {
+  const size_t waves = static_cast<size_t>(gridDim.x) * 4, wave = static_cast<size_t>(blockIdx.x) * 4 + threadIdx.x / 64;
+  const int lane = threadIdx.x % 64;
+  constexpr size_t kSegment = 65536 / 16;
+  u32x4_t seen = {0, 0, 0, 0};
+  for (size_t segment = wave; (segment + 1) * kSegment <= chunks; segment += waves) {
+    const u32x4_t* mine = src + segment * kSegment + lane;
+    for (int i = 0; i < static_cast<int>(kSegment / 64); i += 8) {
+      u32x4_t held[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) held[u] = __builtin_nontemporal_load(mine + (i + u) * 64);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) seen ^= held[u];
+    }
+  }
+  if ((seen.x ^ seen.y ^ seen.z ^ seen.w) == 0x9E3779B9u) sink[0] = 1;  // (keeps the loads; practically never true)
+}
+
 }  // namespace dew_bench
 
-// Both return 0, 1 for arguments that do not fit (null or misaligned pointers, sizes that are not whole 16 bytes), or 3
+// All return 0, 1 for arguments that do not fit (null or misaligned pointers, sizes that are not whole 16 bytes), or 3
 // for a failed launch.
 extern "C" int dew_bench_probe_mfma(const void* operands /* 32 KiB of bf16 */, int32_t iters, float* sink /* 1 MiB */,
                                     double* flops /* host, nullable */, void* stream) {
@@ -67,5 +89,13 @@ extern "C" int dew_bench_probe_copy(const void* src, void* dst, size_t bytes, vo
   if (!src || !dst || bytes % 16 != 0 || ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) != 0) return 1;
   hipLaunchKernelGGL(probe_copy_kernel, dim3(256 * 32), dim3(256), 0, static_cast<hipStream_t>(stream),
                      static_cast<const u32x4_t*>(src), static_cast<u32x4_t*>(dst), bytes / 16);
+  return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+extern "C" int dew_bench_probe_read(const void* src, size_t bytes /* whole 64 KiB segments are read */, void* sink /* 4 bytes */, void* stream) {
+  using namespace dew_bench;
+  if (!src || !sink || bytes % 65536 != 0 || (reinterpret_cast<uintptr_t>(src) & 15u) != 0) return 1;
+  hipLaunchKernelGGL(probe_read_kernel, dim3(256 * 8), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<const u32x4_t*>(src),
+                     bytes / 16, static_cast<uint32_t*>(sink));
   return hipGetLastError() == hipSuccess ? 0 : 3;
 }

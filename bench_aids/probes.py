@@ -19,6 +19,7 @@ def _library():
         c = ctypes
         lib.dew_bench_probe_mfma.restype, lib.dew_bench_probe_mfma.argtypes = c.c_int32, [c.c_void_p, c.c_int32, c.c_void_p, c.POINTER(c.c_double), c.c_void_p]
         lib.dew_bench_probe_copy.restype, lib.dew_bench_probe_copy.argtypes = c.c_int32, [c.c_void_p, c.c_void_p, c.c_size_t, c.c_void_p]
+        lib.dew_bench_probe_read.restype, lib.dew_bench_probe_read.argtypes = c.c_int32, [c.c_void_p, c.c_size_t, c.c_void_p, c.c_void_p]
         _handle = lib
     return _handle
 
@@ -44,4 +45,16 @@ def probe_copy(src: torch.Tensor, dst: torch.Tensor) -> int:
     code = _library().dew_bench_probe_copy(src.data_ptr(), dst.data_ptr(), size, torch.cuda.current_stream().cuda_stream)
     if code != 0:
         raise RuntimeError(f"dew_bench_probe_copy returned {code}")
+    return size
+
+
+def probe_read(src: torch.Tensor) -> int:
+    """Launch the read-only stream over `src` (a contiguous device buffer of whole 64 KiB); returns the bytes read."""
+    size = src.numel() * src.element_size()
+    if not (src.is_cuda and src.is_contiguous()) or size % 65536:
+        raise ValueError("the read probe takes a contiguous device buffer of whole 64 KiB segments")
+    sink = torch.zeros(1, dtype=torch.int32, device=src.device)
+    code = _library().dew_bench_probe_read(src.data_ptr(), size, sink.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    if code != 0:
+        raise RuntimeError(f"dew_bench_probe_read returned {code}")
     return size
