@@ -14,7 +14,7 @@ import dataclasses
 import torch
 
 from . import formats, ops, selection
-from .selection import INHERENT, Kernel, Op, Requirement
+from .selection import Kernel, Op, Requirement
 
 GROUPED_MATMUL = "grouped_matmul"
 """The selector's choice name (`generation.Choice.GROUPED_MATMUL` in the reference)."""

@@ -21,7 +21,7 @@ from typing import NamedTuple
 
 import torch
 
-from . import formats, gemm, ops, selection
+from . import formats, gemm, ops
 from .gemm import GroupSizes
 
 GROUPED_MATMULS = ("auto", "hip", "xla", "pallas")
