@@ -480,6 +480,27 @@ def test_the_expert_mlp_on_split_rows_as_one_call_is_its_three_launches(ops, fp6
         ops.swiglu_mlp_split(xd, pg, pu, pd, od, rows=padded)
 
 
+def test_rows_that_are_not_finite_stay_their_own_on_split_rows_as_on_bf16_operands(ops):
+    """A row holding an infinity, a NaN or a magnitude whose products overflow comes back NaN from the split-row MLP as
+    from the bf16-operand launches; zero rows and rows far below the formats' range come back zero; the rows beside
+    them are untouched."""
+    rng = np.random.default_rng(0)
+    experts, depth, width, out_width = 2, 256, 256, 256
+    banks = [ops.prepare(quantize(torch.from_numpy((rng.standard_normal((experts, d, w)) * 0.05).astype(np.float32)), "mxfp4").to("cuda"))
+             for d, w in ((depth, width), (depth, width), (width, out_width))]
+    x = torch.from_numpy(rng.standard_normal((7, depth)).astype(np.float32)).to(torch.bfloat16)
+    clean = x.clone()
+    x[1, 5], x[2, 7], x[4, 9] = float("inf"), float("nan"), 3e38
+    x[3, :], x[5, :] = 0, 1e-38
+    offsets = torch.tensor([0, 3, 7], dtype=torch.int32).cuda()
+    on_split = ops.swiglu_mlp_split(x.cuda(), *banks, offsets).float().cpu().numpy()
+    on_bf16 = ops.grouped_gemm(ops.gateup_swiglu(x.cuda(), banks[0], banks[1], offsets), banks[2], offsets).float().cpu().numpy()
+    untouched = ops.swiglu_mlp_split(clean.cuda(), *banks, offsets).float().cpu().numpy()
+    for got in (on_split, on_bf16):
+        assert np.isnan(got[[1, 2, 4]]).all() and not got[[3, 5]].any() and np.isfinite(got[[0, 6]]).all()
+    assert np.array_equal(on_split[[0, 6]], untouched[[0, 6]])
+
+
 @pytest.mark.parametrize("quant", ["fp8_block", "fp8_channel", "mxfp4", "nvfp4", "bf16"])
 def test_a_layer_of_a_stacked_bank_is_read_where_it_lies(ops, quant):
     """`Layered(stack, layer)`: the grouped product of one layer's experts out of a bank stacking three layers', from
