@@ -1033,22 +1033,25 @@ static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
   return launched(who);
 }
 
-// Tile choice from what the host knows (rows and experts; the routing itself stays on the device): 256-row
-// tiles when the average group fills them, 128-row tiles otherwise, and for decode-sized groups a 32-row tile
-// whose four wavefronts split the columns, so that thousands of wavefronts stream the weights at once.
 // Rows of the block tile, from what the host knows (rows and experts; the routing itself stays on the device).
-// Two rules, both measured over group sizes of 8 .. 1024 rows on four model shapes. Fill: the tile about as tall as
-// the average group (a 128-row tile over 32-row groups multiplies three empty rows for each real one, and takes 1.3
-// to 2 times as long as 32-row tiles). Occupancy: a launch of fewer tiles than CUs halves its tile until there are
-// enough (8 experts x 512 rows x 512 columns: 144 tiles of 128 rows take 16.5 us, 272 tiles of 64 rows 11.7 us).
-// 256-row tiles, which fill every accumulator register, are kept to MXFP4 and bf16 banks whose groups fill them.
+// Three rules, measured over ragged groups (sizes spread an eighth around their mean) of 8 .. 2048 rows on four model
+// shapes. Fill: a group's last tile is half empty on average, so the tile is about as tall as the average group while
+// what the shorter tile loses when full (it reads and converts the weights again for half the rows: 15 to 26 % on an
+// FP8 bank, 5 to 11 % on one whose codes cost the vector unit little) is less than what the taller one multiplies
+// of empty rows: 32-row tiles up to 26 rows a group (at 32, half the groups need a second, nearly empty one and
+// 64-row tiles are 15 to 25 % faster), 64-row tiles up to 72 rows on FP8 banks (and from 129 to 184, where three
+// of them cover what two 128-row tiles would, 5 to 10 % faster) and up to 384 on the cheap ones.
+// Occupancy: a launch of fewer tiles than CUs halves its tile until there are enough (8 experts x 512 rows x 512
+// columns: 144 tiles of 128 rows take 16.5 us, 272 tiles of 64 rows 11.7 us). 256-row tiles, which fill every
+// accumulator register, are kept to the cheap banks and to groups of 2048 rows or more. Decode-sized groups take the
+// 32-row tile, whose four wavefronts split the columns, so that thousands of wavefronts stream the weights at once.
 static thread_local int forced_tile_rows = 0;  // dew_moe_tile_rows, per calling thread: 0 leaves the choice to the rules below
 
-static int tile_rows(const GemmParams& p, bool fp4) {
+static int tile_rows(const GemmParams& p, bool cheap) {
   if (forced_tile_rows != 0) return forced_tile_rows;
   const int average = p.rows / p.experts;
-  if (fp4 && average >= 1024 && p.width % 256 == 0) return 256;  // below, the half tile a group wastes outweighs its gain
-  int rows = average <= 36 ? 32 : average <= 72 ? 64 : 128;
+  if (cheap && average >= 2048 && p.width % 256 == 0) return 256;  // below, two 128-row blocks a CU are 2 to 5 % faster
+  int rows = average <= 26 ? 32 : average <= (cheap ? 384 : 72) || (average > 128 && average <= 184) ? 64 : 128;
   const long long strips = p.width / 128;
   while (rows > 32 && (p.rows / rows + p.experts / 2) * strips < 256) rows /= 2;
   return rows;
@@ -1073,10 +1076,14 @@ static int launch_format(const char* who, const GemmParams& p, hipStream_t strea
       if (kPaired || p.width % 256 == 0) return launch_tile<FORMAT, MODE, 256, kPaired ? 128 : 256, 1, 4>(who, p, stream);
       [[fallthrough]];  // one bank whose width is not whole 256s: the 128-row tile
     default: {
-      // Groups of a few hundred rows end in a 128-row tile that is half empty on average. With enough groups and
-      // strips for a launch of their own (256 tiles), last tiles of at most 64 rows go to the 64-row tile: measured on
-      // 256 groups of 256 +- 16 rows, 2.5 tiles a group become 2 and a 64-row one.
-      const bool shared = forced_tile_rows == 0 && static_cast<long long>(p.experts) * (p.width / 128) >= 256;
+      // Last tiles of at most 64 rows can go to a second launch of 64-row tiles. That launch runs after the first, so
+      // it pays only where it fills the chip by itself and most groups have such a last tile: the average group just
+      // over a whole number of tiles (256 groups of 256 +- 16 rows: 2.5 tiles a group become 2 and a 64-row one, 1.5
+      // to 2.5 % faster; at 160 or 200 rows a group the same two launches are 5 to 15 % slower than one, a bank of 8
+      // experts, whose few last tiles run their whole depth alone, 20 to 35 % slower, and groups of 1024 rows 1 %).
+      const int average = p.rows / p.experts;
+      const bool shared = forced_tile_rows == 0 && average >= 128 && average < 512 && average % 128 <= 40 &&
+                          static_cast<long long>(p.experts) * (p.width / 128) >= 512;
       GemmParams taller = p;
       taller.skip_tails = shared ? 64 : 0;
       int status;
