@@ -397,7 +397,8 @@ class SparseMLP(_Module):
         experts = self.experts
         if self.shared is None:
             return experts(x, weights, indices)
-        if self.fuse_shared and self.shared == self.hidden_features:
+        same_gating = self.swiglu_limit is None and self.activation == "swiglu"   # the shared expert's own (`GatedMLP`: SwiGLU, no clamp)
+        if self.fuse_shared and self.shared == self.hidden_features and same_gating:
             shared_path = (*self.path, "shared_experts")
             stack = with_shared_expert(experts.kernels(), tuple(expert_matrix(self.variables, (*shared_path, name)) for name in EXPERT_AXES))
             if stack is not None:

@@ -346,3 +346,34 @@ def test_geglu_experts_run_through_the_layer(quant):
     assert np.abs(swiglu - want).max() > 0.05 * np.abs(want).max()
     with pytest.raises(ValueError, match="gate by one of"):
         moe.ExpertMLP(experts, hidden, width, activation="geglu_exact")
+
+
+@pytest.mark.parametrize("gating", [dict(swiglu_limit=0.5), dict(activation="geglu")])
+def test_a_shared_expert_keeps_its_own_gating_beside_clamped_or_geglu_experts(gating):
+    """The shared expert is a dense SwiGLU MLP of its own (src/dew/nn/moe.py:1497-1503, nn/mlp.py:139-144), whatever gates
+    the routed experts: beside a clamp or a GeGLU gate it does not ride the routed launches, whose gating it would take."""
+    import dataclasses
+
+    from dew_amd import moe
+
+    case = CASES["c4-reduced"].scaled(tokens=96)
+    data = inputs(case, seed=4)
+    layer, variables = layer_and_variables(case, data)
+    layer = dataclasses.replace(layer, **gating)
+    calls = []
+    found = moe.with_shared_expert
+    moe.with_shared_expert = lambda *a: calls.append(1) or found(*a)
+    try:
+        got = layer.apply(variables, data["x"].cuda(), logits=data["logits"].cuda()).float().cpu().numpy()
+    finally:
+        moe.with_shared_expert = found
+    assert calls == []
+    mats, factors = zip(*(dequantized(data["banks"][name]) for name in ("gate", "up", "down")), strict=True)
+    x = data["x"].float().numpy()
+    weights, indices = oracle.route(data["logits"].numpy(), case.top_k, bias=data["bias"].numpy(), **case.router)
+    routed, _ = oracle.expert_mlp(x, weights, indices, *mats, factors=factors, limit=gating.get("swiglu_limit"),
+                                  activation=gating.get("activation", "swiglu"))
+    shared = [dequantized(data["shared"][name])[0][0] for name in ("gate", "up", "down")]
+    want = oracle.bf16_round(routed + oracle.gated_mlp(x, *shared))
+    by_max, by_element = oracle.relative_errors(got, want)
+    assert by_max <= 6e-3 and by_element <= TOLERANCE, (by_max, by_element)
