@@ -60,21 +60,37 @@ __global__ __launch_bounds__(kPermuteThreads) void permute_count_kernel(PermuteP
 // One block: totals per bucket, exclusive scan over buckets, then each block's base per bucket.
 __global__ __launch_bounds__(kPermuteThreads) void permute_scan_kernel(PermuteParams p) {
   extern __shared__ int32_t totals[];  // [buckets + 1]
+  __shared__ int32_t wave_sums[kPermuteThreads / 64];
   for (int b = threadIdx.x; b < p.buckets; b += kPermuteThreads) {
     int sum = 0;
+#pragma unroll 8
     for (int blk = 0; blk < p.blocks; ++blk) sum += p.counts[static_cast<size_t>(blk) * p.buckets + b];
     totals[b] = sum;
   }
   __syncthreads();
-  if (threadIdx.x == 0) {  // buckets <= 1025: a serial scan is a few microseconds and exact
-    int running = 0;
-    for (int b = 0; b < p.buckets; ++b) {
-      const int size = totals[b];
-      totals[b] = running;
-      running += size;
-    }
-    totals[p.buckets] = running;
+  // Exclusive scan over the buckets (integer sums: any order is exact): each thread owns a run of consecutive buckets,
+  // the runs' sums are scanned across the wavefront by shuffles and across the wavefronts through LDS.
+  const int per = (p.buckets + kPermuteThreads - 1) / kPermuteThreads;
+  const int first = min(static_cast<int>(threadIdx.x) * per, p.buckets), last = min(first + per, p.buckets);
+  int mine = 0;
+  for (int b = first; b < last; ++b) mine += totals[b];
+  int through = mine;  // inclusive scan of the runs' sums within the wavefront
+  const int lane = threadIdx.x % 64;
+#pragma unroll
+  for (int offset = 1; offset < 64; offset <<= 1) {
+    const int below = __shfl_up(through, offset, 64);
+    if (lane >= offset) through += below;
   }
+  if (lane == 63) wave_sums[threadIdx.x / 64] = through;
+  __syncthreads();
+  int running = through - mine;
+  for (int w = 0; w < static_cast<int>(threadIdx.x) / 64; ++w) running += wave_sums[w];
+  for (int b = first; b < last; ++b) {
+    const int size = totals[b];
+    totals[b] = running;
+    running += size;
+  }
+  if (threadIdx.x == kPermuteThreads - 1) totals[p.buckets] = running;  // the last thread's run ends the buckets (or is empty behind them)
   __syncthreads();
   for (int b = threadIdx.x; b < p.buckets; b += kPermuteThreads) {
     const int start = totals[b];
@@ -84,12 +100,13 @@ __global__ __launch_bounds__(kPermuteThreads) void permute_scan_kernel(PermutePa
     } else {
       p.offsets[p.groups] = start;  // slots routed to a real expert
     }
-    int running = start;
+    int next = start;
+#pragma unroll 8
     for (int blk = 0; blk < p.blocks; ++blk) {
       const size_t at = static_cast<size_t>(blk) * p.buckets + b;
       const int count = p.counts[at];
-      p.bases[at] = running;
-      running += count;
+      p.bases[at] = next;
+      next += count;
     }
   }
 }
