@@ -106,16 +106,6 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const bf16_t* __restrict__ 
   }
 }
 
-// Round to nearest even on the host (the device has the hardware conversion).
-static float bf16_round_host(float value) {
-  uint32_t bits;
-  __builtin_memcpy(&bits, &value, 4);
-  bits += 0x7FFFu + ((bits >> 16) & 1u);
-  bits &= 0xFFFF0000u;
-  __builtin_memcpy(&value, &bits, 4);
-  return value;
-}
-
 }  // namespace dew
 
 extern "C" int dew_moe_combine(const void* slots, const float* weights, const void* addend, void* out,

@@ -33,6 +33,16 @@ __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
 
 __device__ __forceinline__ float bf16_round(float f) { return bf16_to_f32(f32_to_bf16(f)); }
 
+// Round to nearest even on the host (the device has the hardware conversion): a finite value as the bf16 it becomes.
+static inline float bf16_round_host(float value) {
+  uint32_t bits;
+  __builtin_memcpy(&bits, &value, 4);
+  bits += 0x7FFFu + ((bits >> 16) & 1u);
+  bits &= 0xFFFF0000u;
+  __builtin_memcpy(&value, &bits, 4);
+  return value;
+}
+
 // SwiGLU on the fp32 sums of the gate and up products with the reference's roundings
 // (src/dew/nn/activations.py:267-278): g = bf16(gate), u = bf16(up), a = bf16(g * logistic(g)), h = bf16(a * u).
 // logistic(g) = 1 / (1 + e^-g) uses the hardware exp2 and reciprocal (each within 1 ulp of fp32): the
@@ -57,6 +67,18 @@ __device__ __forceinline__ bf16_t geglu_rounded(float gate_sum, float up_sum) {
   const float sig = __builtin_amdgcn_rcpf(1.0f + e);
   const float activated = bf16_round(g * sig);
   return f32_to_bf16(activated * u);
+}
+
+// Either gate on the fp32 sums of a paired launch, with the clamp the stand-alone gating kernel applies (`swiglu_clamped`,
+// src/dew/nn/activations.py:327-333): both sums rounded to bf16 first, then the gate clamped from above and the up
+// projection both ways by `limit` (> 0, already the bf16 it is compared in; 0: no clamp), then the gated product.
+__device__ __forceinline__ bf16_t gated_rounded(float gate_sum, float up_sum, float limit, int activation) {
+  float g = bf16_round(gate_sum), u = bf16_round(up_sum);
+  if (limit > 0.0f) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+  }
+  return activation == DEW_MOE_GATE_GELU_TANH ? geglu_rounded(g, u) : swiglu_rounded(g, u);
 }
 
 // GPT-OSS's gating of one (gate, up) pair already rounded to bf16 (src/dew/nn/gpt_oss.py:120-121 over

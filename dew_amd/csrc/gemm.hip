@@ -91,7 +91,8 @@ struct GemmParams {
   const uint8_t* a_scale;  // split activations: each source row's e8m0 scale, or its row of block_scale_pitch(depth) of them
   uint8_t* out_scale;      // split output: each written row's block_scale_pitch(width) e8m0 scales, one for 128 columns
   const float* bias;  // [experts, width] values of the compute dtype held in fp32, or null
-  float limit;        // the interleaved gated epilogue's clamp
+  float limit;        // the interleaved gated epilogue's clamp; a paired launch's (0: none)
+  int gating;         // a paired launch's gate: DEW_MOE_GATE_SILU (SwiGLU) or DEW_MOE_GATE_GELU_TANH (GeGLU)
   int experts, depth, width, rows, m_tile_bound;
   // A launch normally multiplies every group in tiles of its BM rows, the last of a group partly empty. Where that
   // waste matters two launches share the groups: the taller tiles' launch leaves a last tile that would hold at most
@@ -881,6 +882,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   }
   // bytes of (neighbour's pair, own pair) that make the lane's staged pair: see the swap below
   const uint32_t swap_select = odd_lane ? 0x03020706u : 0x05040100u;
+  const bool plain_swiglu = p.limit <= 0.0f && p.gating == DEW_MOE_GATE_SILU;  // (kernel arguments: the same for the whole launch)
   __builtin_amdgcn_s_barrier();  // every wavefront has read its last A fragments: the ring is free
 #pragma unroll
   for (int pass = 0; pass < kPasses; ++pass) {
@@ -916,8 +918,13 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
             // the lane's rows q (low half) and q + 1 (high half) of its column, rounded
             uint32_t mine;
             if constexpr (PAIRED) {
-              mine = swiglu_rounded(acc[0][i][j][q] * factor0, acc[kMatrices - 1][i][j][q] * factor1) |
-                     (static_cast<uint32_t>(swiglu_rounded(acc[0][i][j][q + 1] * factor0, acc[kMatrices - 1][i][j][q + 1] * factor1)) << 16);
+              if (plain_swiglu) {
+                mine = swiglu_rounded(acc[0][i][j][q] * factor0, acc[kMatrices - 1][i][j][q] * factor1) |
+                       (static_cast<uint32_t>(swiglu_rounded(acc[0][i][j][q + 1] * factor0, acc[kMatrices - 1][i][j][q + 1] * factor1)) << 16);
+              } else {  // a clamp or the GeGLU gate (the same for every lane: a branch, not a select)
+                mine = gated_rounded(acc[0][i][j][q] * factor0, acc[kMatrices - 1][i][j][q] * factor1, p.limit, p.gating) |
+                       (static_cast<uint32_t>(gated_rounded(acc[0][i][j][q + 1] * factor0, acc[kMatrices - 1][i][j][q + 1] * factor1, p.limit, p.gating)) << 16);
+              }
             } else if constexpr (kFp4) {
               mine = pack_bf16(acc[0][i][j][q] * factor0 + bias[j], acc[0][i][j][q + 1] * factor0 + bias[j]);
             } else if constexpr (kWindow) {
@@ -1540,8 +1547,12 @@ extern "C" int dew_moe_gateup_interleaved(const void* x, const int32_t* gather, 
 }
 
 static int gateup_swiglu_of(const char* who, const void* x, const int32_t* gather, const int32_t* offsets, const int32_t* sizes,
-                            const dew_moe_bank* gate, const dew_moe_bank* up, void* hidden, int32_t rows, void* stream) {
+                            const dew_moe_bank* gate, const dew_moe_bank* up, void* hidden, int32_t rows, void* stream,
+                            int32_t activation = DEW_MOE_GATE_SILU, float limit = 0.0f) {
   using namespace dew;
+  DEW_REQUIRE(activation == DEW_MOE_GATE_SILU || activation == DEW_MOE_GATE_GELU_TANH,
+              "%s: the gate's activation %d is neither silu (0: swiglu) nor the tanh gelu (1: geglu)", who, activation);
+  DEW_REQUIRE(limit >= 0.0f, "%s: the clamp limit %g must be positive (0: none)", who, static_cast<double>(limit));
   if (int rc = check_bank(who, gate, "gate")) return rc;
   if (int rc = check_bank(who, up, "up")) return rc;
   DEW_REQUIRE(gate->format == up->format && gate->experts == up->experts && gate->depth == up->depth && gate->width == up->width,
@@ -1564,7 +1575,18 @@ static int gateup_swiglu_of(const char* who, const void* x, const int32_t* gathe
   p.depth = gate->depth;
   p.width = gate->width;
   p.rows = rows;
+  p.gating = activation;
+  p.limit = limit > 0.0f ? bf16_round_host(limit) : 0.0f;  // the clamp is compared in the operands' dtype
   return launch<kSwigluOfTwo>(who, p, gate->format, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int dew_moe_gateup_gated(const void* x, const int32_t* gather, const int32_t* offsets, const int32_t* group_sizes,
+                                    const dew_moe_bank* gate, const dew_moe_bank* up, int32_t activation, float limit,
+                                    void* hidden, int32_t rows, void* stream) {
+  using namespace dew;
+  DEW_REQUIRE(rows == 0 || (offsets != nullptr) != (group_sizes != nullptr),
+              "dew_moe_gateup_gated: the groups come as offsets [E + 1] or as group_sizes [E], one of them");
+  return gateup_swiglu_of("dew_moe_gateup_gated", x, gather, offsets, group_sizes, gate, up, hidden, rows, stream, activation, limit);
 }
 
 extern "C" int dew_moe_gateup_swiglu(const void* x, const int32_t* gather, const int32_t* offsets,

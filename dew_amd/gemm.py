@@ -76,9 +76,16 @@ def _bias_fits(case, bias) -> bool:
                             and tuple(bias.shape) == (_shape(case.rhs)[0], _shape(case.rhs)[2]))
 
 
+def _is_clamp(operands) -> bool:
+    return not operands or (len(operands) == 1 and (operands[0] is None or float(operands[0]) > 0))
+
+
 _EPILOGUES = {
     None: lambda c: not c.epilogue_operands,
-    "swiglu": lambda c: c.paired is not None and not c.epilogue_operands,
+    # the gated product of a paired launch (`gated_product`, src/dew/nn/activations.py:336-356); one operand, where
+    # given, is `swiglu_clamped`'s limit (:327-333), applied to both products before the gate
+    "swiglu": lambda c: c.paired is not None and _is_clamp(c.epilogue_operands),
+    "geglu": lambda c: c.paired is not None and _is_clamp(c.epilogue_operands),
     # the reference's `_plus_bias` (src/dew/nn/moe.py:729-747): each expert's bias on its rows' fp32 sums
     "plus_bias": lambda c: c.paired is None and len(c.epilogue_operands) == 1 and c.epilogue_operands[0] is not None
                            and _bias_fits(c, c.epilogue_operands[0]),
@@ -159,7 +166,8 @@ def gemm(lhs: torch.Tensor, rhs, group_sizes, *, paired=None, gather: torch.Tens
          out_dtype=torch.bfloat16, compute=torch.bfloat16, implementation: str | None = None):
     """Each group's rows of `lhs` (read at `gather` where given) times its matrix of the bank `rhs`, written
     at `scatter` where given. With `paired`, a second bank multiplied by the same rows in the same launch:
-    returns both products, or, with `epilogue='swiglu'`, their gated product alone. On one bank,
+    returns both products, or, with `epilogue='swiglu'` (or `'geglu'`; `epilogue_operands = (limit,)` clamps both
+    products first), their gated product alone. On one bank,
     `epilogue='plus_bias'` adds `epilogue_operands = (bias [E, N],)` to the fp32 sums before the rounding, and
     `epilogue='gpt_oss_gated'` with `(bias or None, limit)` returns GPT-OSS's gated `[rows, N / 2]`."""
     case = GroupedCase(lhs, rhs, paired, epilogue, out_dtype, compute, tuple(epilogue_operands))
@@ -179,8 +187,9 @@ def gemm(lhs: torch.Tensor, rhs, group_sizes, *, paired=None, gather: torch.Tens
     second = prepared(paired)
     if scatter is not None:
         raise selection.KernelRefused(GROUPED_MATMUL, "hip", selection.Refusal("pair-scatter", "a paired product writes sorted rows"), iter(()))
-    if epilogue == "swiglu":
-        return ops.gateup_swiglu(lhs, first, second, offsets, gather=gather, **groups)
+    if epilogue in ("swiglu", "geglu"):
+        limit = epilogue_operands[0] if epilogue_operands else None
+        return ops.gateup_swiglu(lhs, first, second, offsets, gather=gather, activation=epilogue, limit=limit, **groups)
     return (ops.grouped_gemm(lhs, first, offsets, gather=gather, **groups),
             ops.grouped_gemm(lhs, second, offsets, gather=gather, **groups))
 

@@ -88,13 +88,15 @@ def paired_projections(x, first, second, group_sizes, dtype=None, implementation
                      implementation=_implementation(implementation))
 
 
-def gated_projections(x, gate, up, group_sizes, dtype=None, implementation: str = "auto", precision=None) -> torch.Tensor:
-    """The paired product with the SwiGLU product as the launch's epilogue: `gated_product('swiglu')` of
-    `paired_projections`' outputs (src/dew/nn/moe.py:1319-1325) in one kernel, bit for bit the unfused
-    arithmetic (both sums round to bf16 first)."""
+def gated_projections(x, gate, up, group_sizes, dtype=None, implementation: str = "auto", precision=None, *,
+                      activation: str = "swiglu", limit: float | None = None) -> torch.Tensor:
+    """The paired product with the gated product as the launch's epilogue: `gated_product(activation)` of
+    `paired_projections`' outputs (src/dew/nn/moe.py:1319-1325), after `swiglu_clamped`'s clamp where `limit` is given,
+    in one kernel, bit for bit the unfused arithmetic (both sums round to bf16 first)."""
     tokens, rows = (x.tokens, x.rows) if isinstance(x, Gathered) else (x, None)
     compute = torch.bfloat16 if dtype is None else dtype
-    return gemm.gemm(tokens, gate, group_sizes, paired=up, gather=rows, epilogue="swiglu", compute=compute,
+    return gemm.gemm(tokens, gate, group_sizes, paired=up, gather=rows, epilogue=activation,
+                     epilogue_operands=() if limit is None else (limit,), compute=compute,
                      out_dtype=compute, implementation=_implementation(implementation))
 
 
@@ -270,24 +272,21 @@ class ExpertMLP(_Module):
     def _project(self, tokens: Gathered, sizes: GroupSizes, kernels) -> torch.Tensor:
         """src/dew/nn/moe.py:1305-1326."""
         gate_w, up_w, down_w = kernels
-        if self.swiglu_limit is not None or self.activation != "swiglu":
-            # the clamp sits between the paired product and the gating (`swiglu_clamped`, src/dew/nn/activations.py:327-333):
-            # the reference's own unfused arrangement, with the clamp in the gating kernel; so does a GeGLU gate (Gemma's
-            # experts), which the launches' fused epilogue does not compute
-            gate, up = paired_projections(tokens, gate_w, up_w, sizes, self.dtype, self.implementation, self.precision)
-            return expert_projection(ops.gated_product(gate, up, self.activation, self.swiglu_limit), down_w, sizes, self.dtype,
-                                     self.implementation, self.precision, scatter=tokens.slots)
-        if self.fused and self.dtype in (None, torch.bfloat16):
+        plain = self.swiglu_limit is None and self.activation == "swiglu"
+        if self.fused and plain and self.dtype in (None, torch.bfloat16):
             # large groups on MXFP4 banks: both launches on the scaled matrix instruction, the hidden rows never in bf16
             out = gemm.swiglu_mlp_on_split_rows(tokens.tokens, gate_w, up_w, down_w, sizes, gather=tokens.rows,
                                                 scatter=tokens.slots, implementation=_implementation(self.implementation))
             if out is not None:
                 return out
         if self.fused:
-            hidden = gated_projections(tokens, gate_w, up_w, sizes, self.dtype, self.implementation, self.precision)
+            # the clamp (`swiglu_clamped`, src/dew/nn/activations.py:327-333: between the paired product and the gating)
+            # and a GeGLU gate (Gemma's experts) are the bf16-operand launch's epilogue too
+            hidden = gated_projections(tokens, gate_w, up_w, sizes, self.dtype, self.implementation, self.precision,
+                                       activation=self.activation, limit=self.swiglu_limit)
         else:
             gate, up = paired_projections(tokens, gate_w, up_w, sizes, self.dtype, self.implementation, self.precision)
-            hidden = ops.swiglu(gate, up)
+            hidden = ops.gated_product(gate, up, self.activation, self.swiglu_limit)
         return expert_projection(hidden, down_w, sizes, self.dtype, self.implementation, self.precision,
                                  scatter=tokens.slots)
 

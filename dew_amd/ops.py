@@ -357,9 +357,16 @@ def gateup_interleaved(x: torch.Tensor, gate_up: PreparedBank, offsets: torch.Te
 
 
 def gateup_swiglu(x: torch.Tensor, gate: PreparedBank, up: PreparedBank, offsets: torch.Tensor | None, *,
-                  gather: torch.Tensor | None = None, rows: int | None = None, sizes: torch.Tensor | None = None) -> torch.Tensor:
+                  gather: torch.Tensor | None = None, rows: int | None = None, sizes: torch.Tensor | None = None,
+                  activation: str = "swiglu", limit: float | None = None) -> torch.Tensor:
     """`hidden[i] = swiglu(x[gather[i]] @ Wg[e], x[gather[i]] @ Wu[e])`, bf16 `[rows, F]`, one launch. The groups are
-    `offsets [E + 1]`, or, where that is None, `sizes [E]`."""
+    `offsets [E + 1]`, or, where that is None, `sizes [E]`. `activation` 'geglu' gates by the tanh GELU instead, and
+    `limit` clamps the gate from above and the up projection both ways first (`gated_product`'s arithmetic, as the
+    launch's epilogue)."""
+    if activation not in GATES:
+        raise KernelError(f"the gate's activation is one of {list(GATES)}, got {activation!r}")
+    if limit is not None and not limit > 0:
+        raise KernelError(f"the clamp limit {limit} must be positive")
     _device(x, "x", torch.bfloat16)
     experts, depth, width = gate.shape
     if x.shape[-1] != depth:
@@ -368,6 +375,11 @@ def gateup_swiglu(x: torch.Tensor, gate: PreparedBank, up: PreparedBank, offsets
         raise KernelError(f"gate {gate.shape} and up {up.shape} differ")
     rows = _product_rows(x, "x", offsets, experts, gather, None, rows, sizes)
     hidden = torch.empty((rows, width), dtype=torch.bfloat16, device=x.device)
+    if activation != "swiglu" or limit is not None:
+        _lib.check(_lib.library().dew_moe_gateup_gated(_ptr(x), _ptr(gather), _ptr(offsets), _ptr(None if offsets is not None else sizes),
+                                                       gate.descriptor, up.descriptor, GATES[activation], 0.0 if limit is None else float(limit),
+                                                       _ptr(hidden), rows, _stream()), "dew_moe_gateup_gated")
+        return hidden
     if offsets is None:
         _lib.check(_lib.library().dew_moe_gateup_swiglu_sizes(_ptr(x), _ptr(gather), _ptr(sizes), gate.descriptor, up.descriptor,
                                                               _ptr(hidden), rows, _stream()), "dew_moe_gateup_swiglu_sizes")

@@ -410,6 +410,14 @@ int dew_moe_swiglu_clamped(const void* gate, const void* up, float limit, void* 
  * with the same two roundings and the same optional clamp.                                                           */
 enum { DEW_MOE_GATE_SILU = 0, DEW_MOE_GATE_GELU_TANH = 1 };
 int dew_moe_gated_product(const void* gate, const void* up, int32_t activation, float limit, void* hidden, int64_t count, void* stream);
+/* dew_moe_gateup_swiglu with that gating as the paired launch's epilogue: hidden = gated_product(activation) of the two
+ * products, clamped by `limit` first where that is positive, bit for bit dew_moe_gated_product over the two products of
+ * `paired_projections` (src/dew/nn/moe.py:745-770, 1319-1325) without their rows' trip through memory. The groups come
+ * as `offsets [E + 1]` or as `group_sizes [E]` (the other NULL). DeepSeek V4's and GLM's clamped experts and Gemma's
+ * GeGLU experts take it on every bank format of the bf16-operand launches.                                       */
+int dew_moe_gateup_gated(const void* x, const int32_t* gather, const int32_t* offsets /* nullable */,
+                         const int32_t* group_sizes /* nullable */, const dew_moe_bank* gate, const dew_moe_bank* up,
+                         int32_t activation, float limit, void* hidden, int32_t rows, void* stream);
 /* The activation alone: out = bf16(x * logistic(x)), formed in fp32 and rounded once (`silu`, src/dew/nn/activations.py:100-106),
  * which routed value experts pass each chosen projection through (src/dew/nn/value_experts.py:79-82).      */
 int dew_moe_silu(const void* x /* bf16 [count] */, void* out /* bf16 [count] */, int64_t count, void* stream);

@@ -234,6 +234,48 @@ def test_gateup_swiglu_matches_the_two_products_and_the_rounded_epilogue(ops, qu
     assert (fused == want).mean() > 0.9
 
 
+@pytest.mark.parametrize("tile", [0, 32, 128])
+@pytest.mark.parametrize("activation,limit", [("swiglu", 0.25), ("geglu", None), ("geglu", 0.5)])
+@pytest.mark.parametrize("quant", ["fp8_channel", "fp8_block", "mxfp4", "nvfp4", "bf16"])
+def test_a_clamp_or_the_geglu_gate_as_the_paired_launchs_epilogue(ops, quant, activation, limit, tile):
+    """`dew_moe_gateup_gated`: the launch's epilogue clamps and gates as the stand-alone gating kernel does over the two
+    products, bit for bit, and agrees with the oracle's `swiglu_clamped` / `gated_product` of its own products; the
+    groups arrive as offsets or as sizes."""
+    sizes = [100, 0, 37, 200]
+    rng = np.random.default_rng(23)
+    gate, x, offsets = grouped_case(quant, 4, 512, 256, sizes, seed=5)
+    up, _, _ = grouped_case(quant, 4, 512, 256, sizes, seed=6)
+    gather = rng.integers(0, x.shape[0], size=x.shape[0]).astype(np.int32)
+    gate_values, gate_factor = dequantized(gate)
+    up_values, up_factor = dequantized(up)
+    rows = bf16_np(x)[gather]
+    want = oracle.GATED_PRODUCTS[activation](oracle.grouped_matmul(rows, gate_values, sizes, factor=gate_factor),
+                                             oracle.grouped_matmul(rows, up_values, sizes, factor=up_factor), dtype="bfloat16", limit=limit)
+    xd, od, gd = x.cuda(), torch.from_numpy(offsets).cuda(), torch.from_numpy(gather).cuda()
+    pg, pu = ops.prepare(gate.to("cuda")), ops.prepare(up.to("cuda"))
+    with ops.tile_rows(tile):
+        fused = bf16_np(ops.gateup_swiglu(xd, pg, pu, od, gather=gd, activation=activation, limit=limit))
+        by_sizes = bf16_np(ops.gateup_swiglu(xd, pg, pu, None, gather=gd, sizes=torch.tensor(sizes, dtype=torch.int32).cuda(),
+                                             activation=activation, limit=limit))
+        apart = ops.gated_product(ops.grouped_gemm(xd, pg, od, gather=gd), ops.grouped_gemm(xd, pu, od, gather=gd), activation, limit)
+        plain = bf16_np(ops.gateup_swiglu(xd, pg, pu, od, gather=gd))
+    assert np.array_equal(fused, bf16_np(apart)) and np.array_equal(by_sizes, fused)
+    assert not np.array_equal(plain, fused)                 # (the clamp bites and the gates differ on these inputs)
+    scale = np.abs(want).max()
+    assert np.abs(fused - want).max() <= 2 ** -6 * scale
+    assert (fused == want).mean() > 0.9
+
+
+def test_the_gated_launch_refuses_what_it_cannot_run(ops):
+    gate, x, offsets = grouped_case("bf16", 2, 128, 128, [8, 8], seed=1)
+    pg = ops.prepare(gate.to("cuda"))
+    xd, od = x.cuda(), torch.from_numpy(offsets).cuda()
+    with pytest.raises(ops.KernelError, match="one of"):
+        ops.gateup_swiglu(xd, pg, pg, od, activation="geglu_exact")
+    with pytest.raises(ops.KernelError, match="positive"):
+        ops.gateup_swiglu(xd, pg, pg, od, limit=0.0)
+
+
 def test_swiglu_kernel_matches_the_oracle_on_every_bf16_gate(ops):
     gate_bits = np.arange(65536, dtype=np.uint16)
     gate = oracle.bf16_from_bits(gate_bits)
