@@ -162,11 +162,13 @@ ffi::Error GroupedGemm(hipStream_t stream, ffi::AnyBuffer x, ffi::AnyBuffer prep
 }
 
 // ---- dew_moe_gateup_swiglu_ffi: x bf16[M, K], the gate's and the up projection's prepared banks, group_sizes s32[E],
-// gather s32[rows] | s32[0] -> hidden bf16[rows, F] (paired_projections + gated_product('swiglu') in one launch) ----
+// gather s32[rows] | s32[0] -> hidden bf16[rows, F] (paired_projections + gated_product in one launch; `activation` =
+// DEW_MOE_GATE_*, `limit` > 0 = swiglu_clamped's clamp before the gate, 0 = none) ----
 ffi::Error GateUpSwiglu(hipStream_t stream, ffi::AnyBuffer x, ffi::AnyBuffer gate_prepared, ffi::AnyBuffer gate_scales,
                         ffi::AnyBuffer gate_tensor_scale, ffi::AnyBuffer up_prepared, ffi::AnyBuffer up_scales,
                         ffi::AnyBuffer up_tensor_scale, ffi::Buffer<ffi::S32> group_sizes, ffi::AnyBuffer gather,
-                        ffi::Result<ffi::AnyBuffer> hidden, int32_t format, int32_t experts, int32_t depth, int32_t width) {
+                        ffi::Result<ffi::AnyBuffer> hidden, int32_t format, int32_t experts, int32_t depth, int32_t width,
+                        int32_t activation, float limit) {
   constexpr const char* kTarget = "dew_moe_gateup_swiglu";
   if (!is(x, ffi::BF16, 2) || !is(*hidden, ffi::BF16, 2) || group_sizes.dimensions().size() != 1 || group_sizes.dimensions()[0] != experts)
     return misshaped(kTarget, "x bf16[M, K], group_sizes s32[E], hidden bf16[rows, F]");
@@ -177,8 +179,8 @@ ffi::Error GateUpSwiglu(hipStream_t stream, ffi::AnyBuffer x, ffi::AnyBuffer gat
   dew_moe_bank gate{}, up{};
   if (ffi::Error error = bank_of(kTarget, format, experts, depth, width, gate_prepared, gate_scales, gate_tensor_scale, &gate); error.failure()) return error;
   if (ffi::Error error = bank_of(kTarget, format, experts, depth, width, up_prepared, up_scales, up_tensor_scale, &up); error.failure()) return error;
-  if (dew_moe_gateup_swiglu_sizes(x.untyped_data(), present<const int32_t*>(gather), group_sizes.typed_data(), &gate, &up,
-                                  hidden->untyped_data(), static_cast<int32_t>(rows), stream))
+  if (dew_moe_gateup_gated(x.untyped_data(), present<const int32_t*>(gather), nullptr, group_sizes.typed_data(), &gate, &up, activation,
+                           limit, hidden->untyped_data(), static_cast<int32_t>(rows), stream))
     return refused(kTarget);
   return ffi::Error::Success();
 }
@@ -320,7 +322,9 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(dew_moe_gateup_swiglu_ffi, GateUpSwiglu,
                                   .Attr<int32_t>("format")
                                   .Attr<int32_t>("experts")
                                   .Attr<int32_t>("depth")
-                                  .Attr<int32_t>("width"));
+                                  .Attr<int32_t>("width")
+                                  .Attr<int32_t>("activation")
+                                  .Attr<float>("limit"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(dew_moe_swiglu_mlp_ffi, SwigluMlp,
                               ffi::Ffi::Bind()
