@@ -1374,11 +1374,12 @@ extern "C" int dew_moe_kernel_gradient_bf16(const void* lhs_t, const dew_moe_ban
   return launch_tile<kFormatBf16Window, kPlain, 256, 128, 1, 4>(who, p, s);
 }
 
-extern "C" int dew_moe_gateup_swiglu_split_out(const void* x_split, const uint8_t* x_scale, const int32_t* gather,
-                                               const int32_t* offsets, const dew_moe_bank* gate, const dew_moe_bank* up,
-                                               void* hidden_split, uint8_t* hidden_scales, int32_t rows, void* stream) {
-  using namespace dew;
-  const char* who = "dew_moe_gateup_swiglu_split_out";
+namespace dew {
+
+// The paired launch on split rows whose gated rows leave split as well; `second_e2m3`: the rows' second term is FP6.
+static int gateup_split_out_of(const char* who, bool second_e2m3, const void* x_split, const uint8_t* x_scale, const int32_t* gather,
+                               const int32_t* offsets, const dew_moe_bank* gate, const dew_moe_bank* up, void* hidden_split,
+                               uint8_t* hidden_scales, int32_t rows, void* stream, int32_t activation, float limit) {
   if (int rc = check_bank(who, gate, "gate")) return rc;
   if (int rc = check_bank(who, up, "up")) return rc;
   DEW_REQUIRE(gate->format == DEW_MOE_W_MXFP4 && up->format == DEW_MOE_W_MXFP4,
@@ -1387,6 +1388,9 @@ extern "C" int dew_moe_gateup_swiglu_split_out(const void* x_split, const uint8_
   DEW_REQUIRE(gate->experts == up->experts && gate->depth == up->depth && gate->width == up->width,
               "%s: gate [%d, %d, %d] and up [%d, %d, %d] differ", who, gate->experts, gate->depth, gate->width, up->experts,
               up->depth, up->width);
+  DEW_REQUIRE(activation == DEW_MOE_GATE_SILU || activation == DEW_MOE_GATE_GELU_TANH,
+              "%s: the gate's activation %d is neither silu (0: swiglu) nor the tanh gelu (1: geglu)", who, activation);
+  DEW_REQUIRE(limit >= 0.0f, "%s: the clamp limit %g must be positive (0: none)", who, static_cast<double>(limit));
   DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
   if (rows == 0) return DEW_MOE_OK;
   DEW_REQUIRE(x_split && x_scale && offsets && hidden_split && hidden_scales,
@@ -1405,48 +1409,35 @@ extern "C" int dew_moe_gateup_swiglu_split_out(const void* x_split, const uint8_
   p.depth = gate->depth;
   p.width = gate->width;
   p.rows = rows;
+  p.gating = activation;
+  p.limit = limit > 0.0f ? bf16_round_host(limit) : 0.0f;
   // 128-row tiles at two blocks a CU (256 registers a lane, two weight register sets): one block's tile search, first
   // loads and epilogue run under the other's main loop. Measured on 8 experts x 4096 rows of 4096 x 14336: 5.18 ms
-  // against 5.30 ms for 256-row tiles at one block a CU, the same bits. (The plain product below stays on 256-row
+  // against 5.30 ms for 256-row tiles at one block a CU, the same bits. (The plain product stays on 256-row
   // tiles: 2.55 against 2.61 ms.)
-  if (forced_tile_rows == 256) return launch_tile<kFormatMxSplit, kSwigluOfTwoSplit, 256, 128, 2, 2>(who, p, static_cast<hipStream_t>(stream));
-  return launch_tile<kFormatMxSplit, kSwigluOfTwoSplit, 128, 128, 2, 2>(who, p, static_cast<hipStream_t>(stream));
+  const hipStream_t s = static_cast<hipStream_t>(stream);
+  if (second_e2m3) {
+    if (forced_tile_rows == 256) return launch_tile<kFormatMxSplit6, kSwigluOfTwoSplit, 256, 128, 2, 2>(who, p, s);
+    return launch_tile<kFormatMxSplit6, kSwigluOfTwoSplit, 128, 128, 2, 2>(who, p, s);
+  }
+  if (forced_tile_rows == 256) return launch_tile<kFormatMxSplit, kSwigluOfTwoSplit, 256, 128, 2, 2>(who, p, s);
+  return launch_tile<kFormatMxSplit, kSwigluOfTwoSplit, 128, 128, 2, 2>(who, p, s);
+}
+
+}  // namespace dew
+
+extern "C" int dew_moe_gateup_swiglu_split_out(const void* x_split, const uint8_t* x_scale, const int32_t* gather,
+                                               const int32_t* offsets, const dew_moe_bank* gate, const dew_moe_bank* up,
+                                               void* hidden_split, uint8_t* hidden_scales, int32_t rows, void* stream) {
+  return dew::gateup_split_out_of("dew_moe_gateup_swiglu_split_out", false, x_split, x_scale, gather, offsets, gate, up, hidden_split,
+                                  hidden_scales, rows, stream, DEW_MOE_GATE_SILU, 0.0f);
 }
 
 extern "C" int dew_moe_gateup_swiglu_split_fp6_out(const void* x_split, const uint8_t* x_scale, const int32_t* gather,
                                                    const int32_t* offsets, const dew_moe_bank* gate, const dew_moe_bank* up,
                                                    void* hidden_split, uint8_t* hidden_scales, int32_t rows, void* stream) {
-  using namespace dew;
-  const char* who = "dew_moe_gateup_swiglu_split_fp6_out";
-  if (int rc = check_bank(who, gate, "gate")) return rc;
-  if (int rc = check_bank(who, up, "up")) return rc;
-  DEW_REQUIRE(gate->format == DEW_MOE_W_MXFP4 && up->format == DEW_MOE_W_MXFP4,
-              "%s: split activations multiply MXFP4 banks (power-of-two block scales); these are formats %d and %d", who,
-              gate->format, up->format);
-  DEW_REQUIRE(gate->experts == up->experts && gate->depth == up->depth && gate->width == up->width,
-              "%s: gate [%d, %d, %d] and up [%d, %d, %d] differ", who, gate->experts, gate->depth, gate->width, up->experts,
-              up->depth, up->width);
-  DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
-  if (rows == 0) return DEW_MOE_OK;
-  DEW_REQUIRE(x_split && x_scale && offsets && hidden_split && hidden_scales,
-              "%s: x_split, x_scale, offsets, hidden_split and hidden_scales must not be null", who);
-  DEW_REQUIRE(aligned16(x_split) && aligned16(hidden_split), "%s: x_split and hidden_split must be 16-byte aligned", who);
-  GemmParams p{};
-  p.x = static_cast<const bf16_t*>(x_split);
-  p.a_scale = x_scale;
-  p.gather = gather;
-  p.offsets = offsets;
-  p.w0 = BankView{static_cast<const uint8_t*>(gate->codes), gate->scales, gate->tensor_scale};
-  p.w1 = BankView{static_cast<const uint8_t*>(up->codes), up->scales, up->tensor_scale};
-  p.out = static_cast<bf16_t*>(hidden_split);
-  p.out_scale = hidden_scales;
-  p.experts = gate->experts;
-  p.depth = gate->depth;
-  p.width = gate->width;
-  p.rows = rows;
-  // (128-row tiles, two blocks a CU: see dew_moe_gateup_swiglu_split_out)
-  if (forced_tile_rows == 256) return launch_tile<kFormatMxSplit6, kSwigluOfTwoSplit, 256, 128, 2, 2>(who, p, static_cast<hipStream_t>(stream));
-  return launch_tile<kFormatMxSplit6, kSwigluOfTwoSplit, 128, 128, 2, 2>(who, p, static_cast<hipStream_t>(stream));
+  return dew::gateup_split_out_of("dew_moe_gateup_swiglu_split_fp6_out", true, x_split, x_scale, gather, offsets, gate, up, hidden_split,
+                                  hidden_scales, rows, stream, DEW_MOE_GATE_SILU, 0.0f);
 }
 
 // ---- the SwiGLU expert MLP on split rows as one call -----------------------------------------------------------------
@@ -1495,8 +1486,16 @@ extern "C" int dew_moe_swiglu_mlp_split(const void* x, int32_t tokens, const int
                                         const int32_t* group_sizes, const dew_moe_bank* gate, const dew_moe_bank* up,
                                         const dew_moe_bank* down, const int32_t* scatter, void* out, int32_t rows,
                                         int32_t second_term, void* workspace, size_t workspace_bytes, void* stream) {
+  return dew_moe_gated_mlp_split(x, tokens, gather, offsets, group_sizes, gate, up, down, DEW_MOE_GATE_SILU, 0.0f, scatter, out, rows,
+                                 second_term, workspace, workspace_bytes, stream);
+}
+
+extern "C" int dew_moe_gated_mlp_split(const void* x, int32_t tokens, const int32_t* gather, const int32_t* offsets,
+                                       const int32_t* group_sizes, const dew_moe_bank* gate, const dew_moe_bank* up,
+                                       const dew_moe_bank* down, int32_t activation, float limit, const int32_t* scatter, void* out,
+                                       int32_t rows, int32_t second_term, void* workspace, size_t workspace_bytes, void* stream) {
   using namespace dew;
-  const char* who = "dew_moe_swiglu_mlp_split";
+  const char* who = "dew_moe_gated_mlp_split";
   if (int rc = check_bank(who, gate, "gate")) return rc;
   if (int rc = check_bank(who, up, "up")) return rc;
   if (int rc = check_bank(who, down, "down")) return rc;
@@ -1523,10 +1522,12 @@ extern "C" int dew_moe_swiglu_mlp_split(const void* x, int32_t tokens, const int
   uint8_t* hidden_scales = base + w.hidden_scales;
   if (second_term == DEW_MOE_SECOND_TERM_E2M3) {
     if (int rc = dew_moe_split_rows_fp6(x, x_split, x_scale, tokens, gate->depth, stream)) return rc;
-    if (int rc = dew_moe_gateup_swiglu_split_fp6_out(x_split, x_scale, gather, offsets, gate, up, hidden_split, hidden_scales, rows, stream)) return rc;
+    if (int rc = gateup_split_out_of(who, true, x_split, x_scale, gather, offsets, gate, up, hidden_split, hidden_scales, rows, stream,
+                                     activation, limit)) return rc;
   } else {
     if (int rc = dew_moe_split_rows(x, x_split, x_scale, tokens, gate->depth, stream)) return rc;
-    if (int rc = dew_moe_gateup_swiglu_split_out(x_split, x_scale, gather, offsets, gate, up, hidden_split, hidden_scales, rows, stream)) return rc;
+    if (int rc = gateup_split_out_of(who, false, x_split, x_scale, gather, offsets, gate, up, hidden_split, hidden_scales, rows, stream,
+                                     activation, limit)) return rc;
   }
   return dew_moe_grouped_gemm_split_blocks(hidden_split, hidden_scales, nullptr, offsets, down, nullptr, scatter, out, rows, stream);
 }

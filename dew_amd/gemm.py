@@ -213,22 +213,24 @@ def gemm_t(lhs: torch.Tensor, rhs: torch.Tensor, group_sizes, *, out_dtype=torch
 
 
 def swiglu_mlp_on_split_rows(lhs: torch.Tensor, gate, up, down, group_sizes, *, gather: torch.Tensor | None = None,
-                             scatter: torch.Tensor | None = None, implementation: str | None = None):
+                             scatter: torch.Tensor | None = None, implementation: str | None = None,
+                             activation: str = "swiglu", limit: float | None = None):
     """`gemm(gemm(lhs, gate, paired=up, epilogue='swiglu'), down, scatter=scatter)` as two launches on the scaled
     matrix instruction, where that is the faster form, else None (the caller then makes the two `gemm` calls).
     The rows are split into two e4m3 terms under one power-of-two scale a row (`ops.split_rows`); the gate/up
     launch writes its SwiGLU rows already split, one scale per row and 128 columns, and the down launch reads
-    them, so no bf16 hidden rows are written at all. The same selector decides the call."""
+    them, so no bf16 hidden rows are written at all. The same selector decides the call. `activation` ('swiglu' or
+    'geglu') and `limit` (the clamp before the gate) are the gate/up launch's epilogue, as `gemm`'s."""
     if not SPLIT_ROWS or not (torch.is_tensor(lhs) and lhs.is_cuda and lhs.dtype == torch.bfloat16):
         return None
     if any(torch.is_tensor(bank) or isinstance(bank, formats.Bf16) for bank in (gate, up, down)):
         return None  # unquantized matrices have no FP4 codes for the scaled instruction (and a plain tensor is not re-laid to find out)
     named = None if implementation in (None, "auto") else implementation
-    selection.select(GROUPED, GroupedCase(lhs, gate, up, "swiglu"), named)
+    selection.select(GROUPED, GroupedCase(lhs, gate, up, activation, epilogue_operands=() if limit is None else (limit,)), named)
     first, second, third = prepared(gate), prepared(up), prepared(down)
     rows = lhs.shape[0] if gather is None else gather.numel()
     if not ops.prefers_split_pair(first, second, third, rows):
         return None
     groups = GroupSizes.operands(group_sizes)   # a caller's plain group sizes go in as they are: the call forms their prefix
     return ops.swiglu_mlp_split(lhs, first, second, third, groups["offsets"], sizes=groups.get("sizes"), gather=gather,
-                                scatter=scatter, fp6=SPLIT_SECOND_TERM == "e2m3")
+                                scatter=scatter, fp6=SPLIT_SECOND_TERM == "e2m3", activation=activation, limit=limit)

@@ -272,16 +272,16 @@ class ExpertMLP(_Module):
     def _project(self, tokens: Gathered, sizes: GroupSizes, kernels) -> torch.Tensor:
         """src/dew/nn/moe.py:1305-1326."""
         gate_w, up_w, down_w = kernels
-        plain = self.swiglu_limit is None and self.activation == "swiglu"
-        if self.fused and plain and self.dtype in (None, torch.bfloat16):
+        # The clamp (`swiglu_clamped`, src/dew/nn/activations.py:327-333: between the paired product and the gating) and a
+        # GeGLU gate (Gemma's experts) are the paired launch's epilogue, like the plain SwiGLU product.
+        if self.fused and self.dtype in (None, torch.bfloat16):
             # large groups on MXFP4 banks: both launches on the scaled matrix instruction, the hidden rows never in bf16
             out = gemm.swiglu_mlp_on_split_rows(tokens.tokens, gate_w, up_w, down_w, sizes, gather=tokens.rows,
-                                                scatter=tokens.slots, implementation=_implementation(self.implementation))
+                                                scatter=tokens.slots, implementation=_implementation(self.implementation),
+                                                activation=self.activation, limit=self.swiglu_limit)
             if out is not None:
                 return out
         if self.fused:
-            # the clamp (`swiglu_clamped`, src/dew/nn/activations.py:327-333: between the paired product and the gating)
-            # and a GeGLU gate (Gemma's experts) are the bf16-operand launch's epilogue too
             hidden = gated_projections(tokens, gate_w, up_w, sizes, self.dtype, self.implementation, self.precision,
                                        activation=self.activation, limit=self.swiglu_limit)
         else:

@@ -499,9 +499,14 @@ def prefers_split_pair(gate: PreparedBank, up: PreparedBank, down: PreparedBank,
 
 def swiglu_mlp_split(x: torch.Tensor, gate: PreparedBank, up: PreparedBank, down: PreparedBank, offsets: torch.Tensor | None, *,
                      sizes: torch.Tensor | None = None, gather: torch.Tensor | None = None, scatter: torch.Tensor | None = None,
-                     rows: int | None = None, fp6: bool = False) -> torch.Tensor:
-    """The SwiGLU expert MLP on split rows as one call (`dew_moe_swiglu_mlp_split`): `split_rows`, `gateup_swiglu_split_out`
-    and `grouped_gemm_split_blocks` with their intermediates in one workspace. The groups as `offsets` or as `sizes`."""
+                     rows: int | None = None, fp6: bool = False, activation: str = "swiglu", limit: float | None = None) -> torch.Tensor:
+    """The gated expert MLP on split rows as one call (`dew_moe_gated_mlp_split`): `split_rows`, `gateup_swiglu_split_out`
+    and `grouped_gemm_split_blocks` with their intermediates in one workspace. The groups as `offsets` or as `sizes`;
+    `activation` and `limit` as `gateup_swiglu` takes them."""
+    if activation not in GATES:
+        raise KernelError(f"the gate's activation is one of {list(GATES)}, got {activation!r}")
+    if limit is not None and not limit > 0:
+        raise KernelError(f"the clamp limit {limit} must be positive")
     _device(x, "x", torch.bfloat16)
     experts, depth, width = gate.shape
     if x.dim() != 2 or x.shape[1] != depth:
@@ -511,11 +516,11 @@ def swiglu_mlp_split(x: torch.Tensor, gate: PreparedBank, up: PreparedBank, down
     lib = _lib.library()
     workspace = torch.empty(lib.dew_moe_swiglu_mlp_split_workspace_bytes(tokens, rows, depth, width, experts), dtype=torch.uint8, device=x.device)
     out = torch.empty((rows, down.shape[2]), dtype=torch.bfloat16, device=x.device)
-    _lib.check(lib.dew_moe_swiglu_mlp_split(_ptr(x), tokens, _ptr(gather), _ptr(offsets), _ptr(None if offsets is not None else sizes),
-                                            gate.descriptor, up.descriptor,
-                                            down.descriptor, _ptr(scatter), _ptr(out), rows,
-                                            _lib.SECOND_TERM_E2M3 if fp6 else _lib.SECOND_TERM_E4M3, _ptr(workspace), workspace.numel(),
-                                            _stream()), "dew_moe_swiglu_mlp_split")
+    _lib.check(lib.dew_moe_gated_mlp_split(_ptr(x), tokens, _ptr(gather), _ptr(offsets), _ptr(None if offsets is not None else sizes),
+                                           gate.descriptor, up.descriptor, down.descriptor, GATES[activation],
+                                           0.0 if limit is None else float(limit), _ptr(scatter), _ptr(out), rows,
+                                           _lib.SECOND_TERM_E2M3 if fp6 else _lib.SECOND_TERM_E4M3, _ptr(workspace), workspace.numel(),
+                                           _stream()), "dew_moe_gated_mlp_split")
     return out
 
 

@@ -282,6 +282,13 @@ int dew_moe_swiglu_mlp_split(const void* x /* bf16 [tokens, D] */, int32_t token
                              const dew_moe_bank* gate, const dew_moe_bank* up, const dew_moe_bank* down,
                              const int32_t* scatter /* nullable [rows] */, void* out, int32_t rows,
                              int32_t second_term /* DEW_MOE_SECOND_TERM_* */, void* workspace, size_t workspace_bytes, void* stream);
+/* The same with the gate the experts name (`activation` = DEW_MOE_GATE_*, below: SwiGLU or GeGLU) and, where `limit` is
+ * positive, `swiglu_clamped`'s clamp of both products before it (src/dew/nn/activations.py:327-356): clamped or GeGLU experts
+ * on MXFP4 banks stay on split rows; dew_moe_swiglu_mlp_split is this with SwiGLU and no clamp.                          */
+int dew_moe_gated_mlp_split(const void* x, int32_t tokens, const int32_t* gather, const int32_t* offsets, const int32_t* group_sizes,
+                            const dew_moe_bank* gate, const dew_moe_bank* up, const dew_moe_bank* down, int32_t activation,
+                            float limit, const int32_t* scatter, void* out, int32_t rows, int32_t second_term, void* workspace,
+                            size_t workspace_bytes, void* stream);
 
 /* The first product of that pair with the rows' second term in FP6 (no counterpart in the reference). dew_moe_split_rows_fp6:
  * x = s hi + t lo with hi = e4m3(x / s) under one power-of-two scale s a row (scale[row], as dew_moe_split_rows) and

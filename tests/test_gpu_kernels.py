@@ -522,6 +522,32 @@ def test_the_expert_mlp_on_split_rows_as_one_call_is_its_three_launches(ops, fp6
         ops.swiglu_mlp_split(xd, pg, pu, pd, od, rows=padded)
 
 
+@pytest.mark.parametrize("activation,limit", [("swiglu", 0.25), ("geglu", None), ("geglu", 0.5)])
+def test_clamped_and_geglu_experts_stay_on_split_rows(ops, activation, limit):
+    """`dew_moe_gated_mlp_split`: the clamp and the GeGLU gate in the split-row gate/up launch's epilogue, against the
+    oracle's MLP with that gating and against the bf16-operand launches with the same epilogue (nearly all outputs
+    identical: the gated rows are what the bf16 launch would write wherever two e4m3 terms hold them)."""
+    sizes = [700, 0, 290, 5]
+    depth, width, out_width = 512, 768, 256
+    gate, x, offsets = grouped_case("mxfp4", len(sizes), depth, width, sizes, seed=41)
+    up, _, _ = grouped_case("mxfp4", len(sizes), depth, width, sizes, seed=42)
+    down, _, _ = grouped_case("mxfp4", len(sizes), width, out_width, sizes, seed=43)
+    xd, od = x.cuda(), torch.from_numpy(offsets).cuda()
+    pg, pu, pd = (ops.prepare(bank.to("cuda")) for bank in (gate, up, down))
+    on_split = bf16_np(ops.swiglu_mlp_split(xd, pg, pu, pd, od, activation=activation, limit=limit))
+    on_bf16 = bf16_np(ops.grouped_gemm(ops.gateup_swiglu(xd, pg, pu, od, activation=activation, limit=limit), pd, od))
+    plain = bf16_np(ops.swiglu_mlp_split(xd, pg, pu, pd, od))
+    (gv, gf), (uv, uf), (dv, df) = (dequantized(bank) for bank in (gate, up, down))
+    rows = bf16_np(x)
+    hidden = oracle.GATED_PRODUCTS[activation](oracle.grouped_matmul(rows, gv, sizes, factor=gf),
+                                               oracle.grouped_matmul(rows, uv, sizes, factor=uf), dtype="bfloat16", limit=limit)
+    want = oracle.grouped_matmul(hidden, dv, sizes, factor=df)
+    scale = np.abs(want).max()
+    assert np.abs(on_split - want).max() <= 2 ** -6 * scale and np.abs(on_split - on_bf16).max() <= 2 ** -6 * scale
+    assert (on_split == on_bf16).mean() > 0.9 and (on_split == want).mean() > 0.9
+    assert np.abs(plain - want).max() > 2 ** -4 * scale      # (the gating matters on these inputs)
+
+
 def test_rows_that_are_not_finite_stay_their_own_on_split_rows_as_on_bf16_operands(ops):
     """A row holding an infinity, a NaN or a magnitude whose products overflow comes back NaN from the split-row MLP as
     from the bf16-operand launches; zero rows and rows far below the formats' range come back zero; the rows beside
