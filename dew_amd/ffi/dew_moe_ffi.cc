@@ -190,13 +190,14 @@ ffi::Error GateUpSwiglu(hipStream_t stream, ffi::AnyBuffer x, ffi::AnyBuffer gat
 // scatter s32[rows] | s32[0] -> out bf16[rows, D_out]. Where the library's rule says so (dew_moe_prefers_split_rows:
 // MXFP4 banks, groups of hundreds of rows) the rows run as two e4m3 terms on the scaled matrix instruction
 // (dew_moe_swiglu_mlp_split, its intermediates in XLA's scratch); else the paired launch and the down launch on bf16
-// operands, the hidden rows in scratch. `second_term` = DEW_MOE_SECOND_TERM_* for the split form. ----
+// operands, the hidden rows in scratch. `second_term` = DEW_MOE_SECOND_TERM_* for the split form; `activation` and `limit`
+// as the gate/up handler takes them. ----
 ffi::Error SwigluMlp(hipStream_t stream, ffi::ScratchAllocator scratch, ffi::AnyBuffer x, ffi::AnyBuffer gate_prepared,
                      ffi::AnyBuffer gate_scales, ffi::AnyBuffer gate_tensor_scale, ffi::AnyBuffer up_prepared, ffi::AnyBuffer up_scales,
                      ffi::AnyBuffer up_tensor_scale, ffi::AnyBuffer down_prepared, ffi::AnyBuffer down_scales,
                      ffi::AnyBuffer down_tensor_scale, ffi::Buffer<ffi::S32> group_sizes, ffi::AnyBuffer gather, ffi::AnyBuffer scatter,
                      ffi::Result<ffi::AnyBuffer> out, int32_t format, int32_t experts, int32_t depth, int32_t hidden_width,
-                     int32_t width, int32_t second_term) {
+                     int32_t width, int32_t second_term, int32_t activation, float limit) {
   constexpr const char* kTarget = "dew_moe_swiglu_mlp";
   if (!is(x, ffi::BF16, 2) || !is(*out, ffi::BF16, 2) || group_sizes.dimensions().size() != 1 || group_sizes.dimensions()[0] != experts)
     return misshaped(kTarget, "x bf16[T, D], group_sizes s32[E], out bf16[rows, D_out]");
@@ -215,16 +216,16 @@ ffi::Error SwigluMlp(hipStream_t stream, ffi::ScratchAllocator scratch, ffi::Any
     const size_t bytes = dew_moe_swiglu_mlp_split_workspace_bytes(static_cast<int32_t>(tokens), static_cast<int32_t>(rows), depth, hidden_width, experts);
     void* workspace = scratch_of(scratch, bytes);
     if (workspace == nullptr) return misshaped(kTarget, "XLA's scratch allocator has no room for the split rows");
-    if (dew_moe_swiglu_mlp_split(x.untyped_data(), static_cast<int32_t>(tokens), present<const int32_t*>(gather), nullptr,
-                                 group_sizes.typed_data(), &gate, &up, &down, present<const int32_t*>(scatter), out->untyped_data(),
-                                 static_cast<int32_t>(rows), second_term, workspace, bytes, stream))
+    if (dew_moe_gated_mlp_split(x.untyped_data(), static_cast<int32_t>(tokens), present<const int32_t*>(gather), nullptr,
+                                group_sizes.typed_data(), &gate, &up, &down, activation, limit, present<const int32_t*>(scatter),
+                                out->untyped_data(), static_cast<int32_t>(rows), second_term, workspace, bytes, stream))
       return refused(kTarget);
     return ffi::Error::Success();
   }
   void* hidden = scratch_of(scratch, static_cast<size_t>(rows) * hidden_width * 2);
   if (hidden == nullptr) return misshaped(kTarget, "XLA's scratch allocator has no room for the hidden rows");
-  if (dew_moe_gateup_swiglu_sizes(x.untyped_data(), present<const int32_t*>(gather), group_sizes.typed_data(), &gate, &up, hidden,
-                                  static_cast<int32_t>(rows), stream) ||
+  if (dew_moe_gateup_gated(x.untyped_data(), present<const int32_t*>(gather), nullptr, group_sizes.typed_data(), &gate, &up, activation,
+                           limit, hidden, static_cast<int32_t>(rows), stream) ||
       dew_moe_grouped_gemm_sizes(hidden, nullptr, group_sizes.typed_data(), &down, nullptr, present<const int32_t*>(scatter),
                                  out->untyped_data(), static_cast<int32_t>(rows), stream))
     return refused(kTarget);
@@ -349,7 +350,9 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(dew_moe_swiglu_mlp_ffi, SwigluMlp,
                                   .Attr<int32_t>("depth")
                                   .Attr<int32_t>("hidden_width")
                                   .Attr<int32_t>("width")
-                                  .Attr<int32_t>("second_term"));
+                                  .Attr<int32_t>("second_term")
+                                  .Attr<int32_t>("activation")
+                                  .Attr<float>("limit"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(dew_moe_combine_ffi, Combine,
                               ffi::Ffi::Bind()
