@@ -17,6 +17,10 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
 
 constexpr int kSplitWaves = 4;  // rows per 256-thread block
 
+// HELD = the 16-byte chunks a lane holds of its row (depth = 512 HELD, up to 4096): the row is then read once, with
+// loads that leave nothing in the caches (nothing reads it again), and converted from registers; 0 = any depth, the row
+// read twice (the second time from the cache).
+template <int HELD>
 __global__ __launch_bounds__(64 * kSplitWaves) void split_rows_kernel(const bf16_t* __restrict__ x, uint8_t* __restrict__ split,
                                                                      uint8_t* __restrict__ scale, int rows, int depth) {
   const int lane = threadIdx.x % 64;
@@ -25,12 +29,26 @@ __global__ __launch_bounds__(64 * kSplitWaves) void split_rows_kernel(const bf16
   const bf16_t* source = x + static_cast<size_t>(row) * depth;
   // the row's largest exponent field (the sign bit dropped; NaN and infinity count as the largest finite one)
   uint32_t largest = 0;
-  for (int chunk = lane; chunk < depth / 8; chunk += 64) {
-    const u32x4_t words = *reinterpret_cast<const u32x4_t*>(source + chunk * 8);
+  u32x4_t held[HELD > 0 ? HELD : 1];
+  if constexpr (HELD > 0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      largest = max(largest, (words[i] >> 7) & 0xFFu);
-      largest = max(largest, (words[i] >> 23) & 0xFFu);
+    for (int c = 0; c < HELD; ++c) held[c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(source + (lane + 64 * c) * 8));
+#pragma unroll
+    for (int c = 0; c < HELD; ++c) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        largest = max(largest, (held[c][i] >> 7) & 0xFFu);
+        largest = max(largest, (held[c][i] >> 23) & 0xFFu);
+      }
+    }
+  } else {
+    for (int chunk = lane; chunk < depth / 8; chunk += 64) {
+      const u32x4_t words = *reinterpret_cast<const u32x4_t*>(source + chunk * 8);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        largest = max(largest, (words[i] >> 7) & 0xFFu);
+        largest = max(largest, (words[i] >> 23) & 0xFFu);
+      }
     }
   }
 #pragma unroll
@@ -41,8 +59,7 @@ __global__ __launch_bounds__(64 * kSplitWaves) void split_rows_kernel(const bf16
   if (lane == 0) scale[row] = static_cast<uint8_t>(hi_byte);
   const float inverse = __uint_as_float(static_cast<uint32_t>(254 - hi_byte) << 23);  // 2^-(hi_byte - 127)
   uint8_t* target = split + static_cast<size_t>(row) * depth * 2;
-  for (int chunk = lane; chunk < depth / 8; chunk += 64) {
-    const u32x4_t words = *reinterpret_cast<const u32x4_t*>(source + chunk * 8);
+  auto convert = [&](int chunk, const u32x4_t words) __attribute__((always_inline)) {
     float v[8];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -68,6 +85,12 @@ __global__ __launch_bounds__(64 * kSplitWaves) void split_rows_kernel(const bf16
     uint8_t* block = target + (chunk / 8) * 128 + group * 64 + half * 16 + piece * 8;
     *reinterpret_cast<u32x2_t*>(block) = u32x2_t{hi[0], hi[1]};
     *reinterpret_cast<u32x2_t*>(block + 32) = u32x2_t{lo[0], lo[1]};
+  };
+  if constexpr (HELD > 0) {
+#pragma unroll
+    for (int c = 0; c < HELD; ++c) convert(lane + 64 * c, held[c]);
+  } else {
+    for (int chunk = lane; chunk < depth / 8; chunk += 64) convert(chunk, *reinterpret_cast<const u32x4_t*>(source + chunk * 8));
   }
 }
 
@@ -177,7 +200,15 @@ extern "C" int dew_moe_split_rows(const void* x, void* split, uint8_t* scale, in
   if (rows == 0) return DEW_MOE_OK;
   DEW_REQUIRE(x && split && scale, "dew_moe_split_rows: x, split and scale must not be null");
   DEW_REQUIRE(aligned16(x) && aligned16(split), "dew_moe_split_rows: x and split must be 16-byte aligned");
-  hipLaunchKernelGGL(split_rows_kernel, dim3((rows + kSplitWaves - 1) / kSplitWaves), dim3(64 * kSplitWaves), 0,
-                     static_cast<hipStream_t>(stream), static_cast<const bf16_t*>(x), static_cast<uint8_t*>(split), scale, rows, depth);
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3((rows + kSplitWaves - 1) / kSplitWaves), dim3(64 * kSplitWaves), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const bf16_t*>(x), static_cast<uint8_t*>(split), scale, rows, depth);
+  };
+  switch (depth) {
+    case 1024: launch(split_rows_kernel<2>); break;
+    case 2048: launch(split_rows_kernel<4>); break;
+    case 4096: launch(split_rows_kernel<8>); break;
+    default: launch(split_rows_kernel<0>); break;
+  }
   return launched("split_rows_kernel");
 }
