@@ -201,6 +201,9 @@ template <int FORMAT, int MODE, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 && ((MODE == kSwigluOfTwo || MODE == kSwigluOfTwoSplit) ? 2 : 1) * BN == 256) ? 2 : 1) void grouped_gemm_kernel(GemmParams p) {
   constexpr bool PAIRED = MODE == kSwigluOfTwo || MODE == kSwigluOfTwoSplit;
   constexpr bool kSplitOut = MODE == kSwigluOfTwoSplit;
+  // Unquantized banks take the extents the reference's own grouped kernel does (multiples of 8 in its contract; here a depth in
+  // whole 64-deep steps and a width in whole 32-column atoms): a strip past the width multiplies columns it does not store.
+  constexpr bool kRagged = FORMAT == DEW_MOE_W_BF16;
   constexpr bool kGated = MODE == kInterleavedGated;
   constexpr int kOutBN = kGated ? BN / 2 : BN;  // output columns of the tile
   static_assert(WM * WN == 4 && BM % (32 * WM) == 0 && BN % (32 * WN) == 0 && BM % 32 == 0, "tile shape");
@@ -248,7 +251,8 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   // XCDs: the m-tile bound overshoots the real tile count by up to one tile per expert, and the empty tiles
   // at the end of the order then spread over all XCDs instead of idling the last ones.
   const int kGroupM = p.group_m, kChunk = 8 * kGroupM;
-  const int n_strips = p.width / BN;
+  // (a bf16 bank's width need not be whole strips: its last strip then holds fewer columns than BN, see kRagged below)
+  const int n_strips = (p.width + BN - 1) / BN;
   const int total = p.m_tile_bound * n_strips;
   const int local = blockIdx.x / 8;
   const int order = ((local / kChunk) * 8 + blockIdx.x % 8) * kChunk + local % kChunk;
@@ -328,6 +332,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
     for (int item = tid; item < (tail_end - tail_begin) * (kOutBN / 8); item += kThreads) {
       const int sorted = tail_begin + item / (kOutBN / 8);
       const int row = p.scatter ? p.scatter[sorted] : sorted;
+      if (kRagged && out_n0 + (item % (kOutBN / 8)) * 8 >= out_width) continue;  // the last strip's columns past the width
       *reinterpret_cast<u32x4_t*>(p.out + static_cast<size_t>(row) * out_width + out_n0 + (item % (kOutBN / 8)) * 8) = u32x4_t{0, 0, 0, 0};
       if constexpr (kSplitOut) {  // zero terms under a unit scale
         if (item % (kOutBN / 8) == 0) p.out_scale[static_cast<size_t>(sorted) * block_scale_pitch(p.width) + n0 / 128] = 127;
@@ -463,7 +468,8 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   const uint32_t b_lane = lane * 16, b_scale_lane = lane * 2;
 #pragma unroll
   for (int t = 0; t < kTiles; ++t) {
-    const int matrix = t / TJ, column = n0 + wn0 + 32 * (t % TJ);
+    // (past a ragged width the tile reads the bank's last 32 columns again, inside the expert's matrix; its results are not stored)
+    const int matrix = t / TJ, column = kRagged ? min(n0 + wn0 + 32 * (t % TJ), p.width - 32) : n0 + wn0 + 32 * (t % TJ);
     const uint8_t* codes = matrix == 0 ? p.w0.codes : p.w1.codes;
     const void* scales = matrix == 0 ? p.w0.scales : p.w1.scales;
     // (a kernel gradient's one "expert" holds every group's tokens: the group's window starts first_step steps in)
@@ -873,7 +879,9 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   float bias[TJ];
 #pragma unroll
   for (int j = 0; j < TJ; ++j)
-    bias[j] = (!PAIRED && p.bias) ? p.bias[static_cast<size_t>(expert) * p.width + n0 + wn0 + 32 * j + lane % 32] : 0.0f;
+    bias[j] = (!PAIRED && p.bias) ? p.bias[static_cast<size_t>(expert) * p.width + (kRagged ? min(n0 + wn0 + 32 * j + lane % 32, p.width - 1)
+                                                                                               : n0 + wn0 + 32 * j + lane % 32)]
+                                  : 0.0f;
   // quantized rows: a weight block scale that is no normal power of two cannot enter the instruction; the tile is
   // then written as NaN (through the addend every sum meets) rather than as the product under another scale
   if (kFp8Rows && unscalable != 0) {
@@ -991,7 +999,8 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
             p.out_scale[static_cast<size_t>(row0 + pass * kPassRows + staged_row) * block_scale_pitch(p.width) + n0 / 128] = static_cast<uint8_t>(hi_byte);
         }
       } else {
-        if (valid) *reinterpret_cast<u32x4_t*>(p.out + static_cast<size_t>(out_rows[it]) * out_width + out_n0 + chunk * 8) = words;
+        if (valid && (!kRagged || out_n0 + chunk * 8 < out_width))
+          *reinterpret_cast<u32x4_t*>(p.out + static_cast<size_t>(out_rows[it]) * out_width + out_n0 + chunk * 8) = words;
       }
     }
   }
@@ -1004,9 +1013,14 @@ static int check_bank(const char* who, const dew_moe_bank* bank, const char* nam
                   bank->format == DEW_MOE_W_MXFP4 || bank->format == DEW_MOE_W_MXFP8 || bank->format == DEW_MOE_W_BF16,
               "%s: %s bank has unknown format %d", who, name, bank->format);
   DEW_REQUIRE(bank->experts >= 1 && bank->experts <= 4096, "%s: %s bank has %d experts", who, name, bank->experts);
-  DEW_REQUIRE(bank->depth >= 128 && bank->depth % 128 == 0, "%s: %s bank depth %d is not a multiple of 128", who, name, bank->depth);
+  if (bank->format == DEW_MOE_W_BF16) {  // unquantized matrices: whole 64-deep steps and 32-column atoms (GPT-OSS's 2880 is 45 steps, 90 atoms)
+    DEW_REQUIRE(bank->depth >= 128 && bank->depth % 64 == 0, "%s: %s bank depth %d is not a multiple of 64", who, name, bank->depth);
+    DEW_REQUIRE(bank->width >= 128 && bank->width % 32 == 0, "%s: %s bank width %d is not a multiple of 32", who, name, bank->width);
+  } else {
+    DEW_REQUIRE(bank->depth >= 128 && bank->depth % 128 == 0, "%s: %s bank depth %d is not a multiple of 128", who, name, bank->depth);
+    DEW_REQUIRE(bank->width % 128 == 0 && bank->width >= 128, "%s: %s bank width %d is not a multiple of 128", who, name, bank->width);
+  }
   DEW_REQUIRE(bank->depth <= 128 * kMaxDepthBlocks, "%s: %s bank depth %d is above %d", who, name, bank->depth, 128 * kMaxDepthBlocks);
-  DEW_REQUIRE(bank->width % 128 == 0 && bank->width >= 128, "%s: %s bank width %d is not a multiple of 128", who, name, bank->width);
   DEW_REQUIRE(bank->codes && (bank->scales || bank->format == DEW_MOE_W_BF16), "%s: %s bank codes and scales must not be null", who, name);
   DEW_REQUIRE((bank->format != DEW_MOE_W_NVFP4 && bank->format != DEW_MOE_W_MXFP4) || bank->tensor_scale, "%s: %s NVFP4 bank needs tensor scales", who, name);
   DEW_REQUIRE(aligned16(bank->codes), "%s: %s bank codes must be 16-byte aligned", who, name);
@@ -1029,7 +1043,7 @@ static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
   // every expert may end in a partial tile, and the zeroed tail may add one more
   p.m_tile_bound = p.tail_of > 0 ? p.experts : (p.rows + BM - 1) / BM + p.experts + 1;
   if (FORMAT == kFormatMxFp8Window || FORMAT == kFormatBf16Window) p.m_tile_bound = p.experts * ((p.window_rows + BM - 1) / BM);  // every group the same whole rows
-  const int total = p.m_tile_bound * (p.width / BN);
+  const int total = p.m_tile_bound * ((p.width + BN - 1) / BN);
   // A chunk is 4 m-tiles x 8 strips, and 2 x 8 for the 256-row tiles, whose launches have the fewest tiles: dealt in
   // smaller chunks their last round spreads more evenly over the XCDs (measured on 16 to 64 m-tiles of 256 rows: the down
   // launch 8 % shorter, the paired one 3 %; taller chunks of 8 or 16 m-tiles, which fetch less, were slower everywhere)

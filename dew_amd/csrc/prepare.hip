@@ -335,7 +335,9 @@ extern "C" int dew_moe_prepare_bank(const dew_moe_bank* ref, void* prepared, dew
   DEW_REQUIRE(ref->experts >= 1 && ref->depth >= 1 && ref->width >= 1, "dew_moe_prepare_bank: bank [%d, %d, %d]",
               ref->experts, ref->depth, ref->width);
   DEW_REQUIRE(ref->codes && (ref->scales || ref->format == DEW_MOE_W_BF16), "dew_moe_prepare_bank: codes and scales must not be null");
-  DEW_REQUIRE(ref->width % 128 == 0, "dew_moe_prepare_bank: width %d is not a multiple of 128", ref->width);
+  // unquantized matrices as the reference holds them take any width in whole 32-column atoms and any depth in whole 64-deep steps
+  const bool plain_bf16 = ref->format == DEW_MOE_W_BF16 && ref->layout == DEW_MOE_LAYOUT_REFERENCE;
+  DEW_REQUIRE(ref->width % (plain_bf16 ? 32 : 128) == 0, "dew_moe_prepare_bank: width %d is not a multiple of %d", ref->width, plain_bf16 ? 32 : 128);
   DEW_REQUIRE((reinterpret_cast<uintptr_t>(prepared) & 255u) == 0, "dew_moe_prepare_bank: prepared buffer must be 256-byte aligned");
   hipStream_t s = static_cast<hipStream_t>(stream);
   *out = *ref;
@@ -391,7 +393,7 @@ extern "C" int dew_moe_prepare_bank(const dew_moe_bank* ref, void* prepared, dew
     out->scales = scales_out;
     out->tensor_scale = tensor_scale;
   } else if (ref->format == DEW_MOE_W_BF16) {
-    DEW_REQUIRE(ref->depth % 128 == 0, "dew_moe_prepare_bank: a bf16 bank's depth is whole 128s, not %d", ref->depth);
+    DEW_REQUIRE(ref->depth % (plain_bf16 ? 64 : 128) == 0, "dew_moe_prepare_bank: a bf16 bank's depth is whole %ds, not %d", plain_bf16 ? 64 : 128, ref->depth);
     if (ref->layout == DEW_MOE_LAYOUT_REFERENCE_KMAJOR) {
       DEW_REQUIRE(aligned16(ref->codes), "dew_moe_prepare_bank: K-major bf16 matrices must be 16-byte aligned");
       hipLaunchKernelGGL(prepare_bf16_kmajor_kernel, dim3(grid), dim3(256), 0, s, static_cast<const uint16_t*>(ref->codes),

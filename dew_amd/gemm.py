@@ -76,6 +76,13 @@ def _bias_fits(case, bias) -> bool:
                             and tuple(bias.shape) == (_shape(case.rhs)[0], _shape(case.rhs)[2]))
 
 
+def _extent_units(bank) -> tuple[int, int]:
+    """(depth, width) granules of a bank: an unquantized one's steps and atoms, else the 128 of the block scales and tiles."""
+    plain = torch.is_tensor(bank) or (isinstance(bank, formats.Bf16) and not bank.transposed) or (
+        isinstance(bank, ops.PreparedBank) and bank.descriptor.format == ops._lib.W_BF16)
+    return (64, 32) if plain else (128, 128)
+
+
 def _is_clamp(operands) -> bool:
     return not operands or (len(operands) == 1 and (operands[0] is None or float(operands[0]) > 0))
 
@@ -91,7 +98,7 @@ _EPILOGUES = {
                            and _bias_fits(c, c.epilogue_operands[0]),
     # GPT-OSS's interleaved gate/up with its clamped gating (src/dew/nn/gpt_oss.py:111-121)
     "gpt_oss_gated": lambda c: c.paired is None and len(c.epilogue_operands) == 2 and _bias_fits(c, c.epilogue_operands[0])
-                               and float(c.epilogue_operands[1]) > 0 and _shape(c.rhs)[2] % 256 == 0,
+                               and float(c.epilogue_operands[1]) > 0 and _shape(c.rhs)[2] % (2 * _extent_units(c.rhs)[1]) == 0,
 }
 
 
@@ -103,11 +110,14 @@ HIP = Kernel("hip", (
     Requirement("bf16", lambda c: c.lhs.dtype == torch.bfloat16 and c.compute == torch.bfloat16 and c.out_dtype == torch.bfloat16,
                 lambda c: f"rows {c.lhs.dtype}, compute {c.compute}, out {c.out_dtype}; the kernels compute and write bfloat16",
                 row="fp32 outputs"),
-    Requirement("depth", lambda c: _shape(c.rhs)[1] % 128 == 0 and c.lhs.shape[-1] == _shape(c.rhs)[1],
-                lambda c: f"depth {_shape(c.rhs)[1]} against rows {c.lhs.shape[-1]} deep; depths are whole 128s",
+    # (unquantized matrices: whole 64-deep steps and 32-column atoms, so GPT-OSS's 2880-wide experts run as they are; the
+    # reference's own grouped kernel takes extents in whole 8s, `_Cutlass.in_contract`, src/dew/nn/kernels/grouped_matmul.py:1874-1887)
+    Requirement("depth", lambda c: _shape(c.rhs)[1] % _extent_units(c.rhs)[0] == 0 and _shape(c.rhs)[1] >= 128
+                                   and c.lhs.shape[-1] == _shape(c.rhs)[1],
+                lambda c: f"depth {_shape(c.rhs)[1]} against rows {c.lhs.shape[-1]} deep; depths are whole {_extent_units(c.rhs)[0]}s",
                 row="ragged depth"),
-    Requirement("width", lambda c: _shape(c.rhs)[2] % 128 == 0,
-                lambda c: f"width {_shape(c.rhs)[2]} is not a multiple of the 128-column tile", row="ragged width"),
+    Requirement("width", lambda c: _shape(c.rhs)[2] % _extent_units(c.rhs)[1] == 0 and _shape(c.rhs)[2] >= 128,
+                lambda c: f"width {_shape(c.rhs)[2]} is not a multiple of {_extent_units(c.rhs)[1]}", row="ragged width"),
     Requirement("pair", lambda c: c.paired is None or (_shape(c.paired) == _shape(c.rhs) and type(c.paired) is type(c.rhs)),
                 "a paired product's matrices share one shape and format"),
     Requirement("epilogue", lambda c: _EPILOGUES.get(c.epilogue, lambda c: False)(c),

@@ -135,3 +135,81 @@ def test_gpt_oss_requirements_are_refused_by_name(ops):
         gemm.gemm(x.cuda(), bank.to("cuda"), sizes, epilogue="gpt_oss_gated", epilogue_operands=(None, -1.0), implementation="hip")
     out = gemm.gemm(x.cuda(), bank.to("cuda"), sizes, epilogue="gpt_oss_gated", epilogue_operands=(None, 7.0))
     assert out.shape == (11, 128)
+
+
+@pytest.mark.parametrize("tile", [0, 32, 64, 128, 256])
+@pytest.mark.parametrize("depth,width", [(192, 160), (320, 352), (2880, 2880)])
+def test_unquantized_banks_take_depths_in_whole_steps_and_widths_in_whole_atoms(ops, depth, width, tile):
+    """GPT-OSS's experts are 2880 wide (45 steps of 64 depths, 90 atoms of 32 columns, no whole 128s) and the reference keeps
+    such banks unquantized (`packed_banks`, src/dew/interop/quantized_loads.py:130-131): the bf16 bank's launches take
+    those extents as they are, the last strip's columns past the width neither stored nor biased from out of bounds."""
+    sizes = [150, 0, 37, 70] if depth < 2000 else [40, 0, 9]
+    bank, x, bias, offsets = bank_case("bf16", len(sizes), depth, width, sizes, seed=depth + width)
+    rows = x.shape[0] + 5                                    # five sorted positions past the groups
+    rng = np.random.default_rng(3)
+    scatter = torch.from_numpy(rng.permutation(rows).astype(np.int32)).cuda()
+    gather = torch.from_numpy(np.concatenate([np.arange(x.shape[0]), np.zeros(5)]).astype(np.int32)).cuda()
+    values, _ = dequantized(bank)
+    held = bias.to(torch.bfloat16).float()
+    want = oracle._biased_matmul(bf16_np(x), values, sizes, bias.numpy(), dtype="bfloat16", factor=None)
+    prepared = ops.prepare(bank.to("cuda"))
+    with ops.tile_rows(tile):
+        got = ops.grouped_gemm(x.cuda(), prepared, torch.from_numpy(offsets).cuda(), bias=held.cuda(), gather=gather, scatter=scatter, rows=rows)
+    assert got.shape == (rows, width)
+    got = bf16_np(got)
+    order = scatter.cpu().numpy()
+    assert not got[order[x.shape[0]:]].any()
+    assert np.abs(got[order[:x.shape[0]]] - want).max() <= 2 ** -7 * np.abs(want).max()
+    assert (got[order[:x.shape[0]]] == want).mean() > 0.97
+
+
+@pytest.mark.parametrize("tile", [0, 64, 128])
+def test_ragged_unquantized_banks_through_the_paired_and_the_interleaved_launches(ops, tile):
+    sizes = [150, 0, 37, 70]
+    depth, width = 320, 224
+    gate, x, _, offsets = bank_case("bf16", len(sizes), depth, width, sizes, seed=5)
+    up, _, _, _ = bank_case("bf16", len(sizes), depth, width, sizes, seed=6)
+    xd, od = x.cuda(), torch.from_numpy(offsets).cuda()
+    pg, pu = ops.prepare(gate.to("cuda")), ops.prepare(up.to("cuda"))
+    with ops.tile_rows(tile):
+        fused = ops.gateup_swiglu(xd, pg, pu, od)
+        apart = ops.swiglu(ops.grouped_gemm(xd, pg, od), ops.grouped_gemm(xd, pu, od))
+    assert fused.shape == (x.shape[0], width) and torch.equal(fused, apart)
+    want = oracle.swiglu(oracle.grouped_matmul(bf16_np(x), dequantized(gate)[0], sizes), oracle.grouped_matmul(bf16_np(x), dequantized(up)[0], sizes))
+    assert np.abs(bf16_np(fused) - want).max() <= 2 ** -6 * np.abs(want).max()
+    # the interleaved bank: 2 x 224 columns, gate even and up odd, GPT-OSS's clamped gating, a bias on the sums
+    both, x, bias, offsets = bank_case("bf16", len(sizes), depth, 2 * width, sizes, seed=7, scale=0.05)
+    values, _ = dequantized(both)
+    projected = oracle._biased_matmul(bf16_np(x), values, sizes, bias.numpy(), dtype="bfloat16", factor=None)
+    want = oracle.gpt_oss_gating(projected, limit=7.0)
+    with ops.tile_rows(tile):
+        got = ops.gateup_interleaved(x.cuda(), ops.prepare(both.to("cuda")), torch.from_numpy(offsets).cuda(),
+                                     bias=bias.to(torch.bfloat16).float().cuda(), limit=7.0)
+    assert got.shape == (x.shape[0], width)
+    got = bf16_np(got)
+    assert np.abs(got - want).max() <= 2 ** -6 * np.abs(want).max() and (got == want).mean() > 0.9
+
+
+def test_a_gpt_oss_layer_of_the_models_own_width_runs_unquantized():
+    """hidden 2880, intermediate 2880 (gpt-oss-20b's config), banks the reference's load keeps dense: the layer through
+    the selector, against the oracle."""
+    from dew_amd import formats, gpt_oss
+
+    tokens, hidden, intermediate, experts, top_k = 48, 2880, 2880, 4, 2
+    rng = np.random.default_rng(13)
+    x = torch.from_numpy(rng.standard_normal((tokens, hidden)).astype(np.float32)).to(torch.bfloat16)
+    router_kernel = torch.from_numpy((rng.standard_normal((hidden, experts)) * hidden ** -0.5).astype(np.float32))
+    router_bias = torch.from_numpy((rng.standard_normal(experts) * 0.1).astype(np.float32))
+    gate_up = formats.Bf16(torch.from_numpy((rng.standard_normal((experts, hidden, 2 * intermediate)) * hidden ** -0.5).astype(np.float32)).to(torch.bfloat16))
+    down = formats.Bf16(torch.from_numpy((rng.standard_normal((experts, intermediate, hidden)) * intermediate ** -0.5).astype(np.float32)).to(torch.bfloat16))
+    gate_bias = torch.from_numpy(rng.standard_normal((experts, 2 * intermediate)).astype(np.float32))
+    down_bias = torch.from_numpy(rng.standard_normal((experts, hidden)).astype(np.float32))
+    want, _ = oracle.gpt_oss_mlp(bf16_np(x), router_kernel.numpy(), router_bias.numpy(), dequantized(gate_up)[0], gate_bias.numpy(),
+                                 dequantized(down)[0], down_bias.numpy(), top_k_count=top_k, factors=(None, None))
+    variables = {"params": {"router": {"kernel": router_kernel.cuda(), "bias": router_bias.cuda()},
+                            "experts": {"gate_up_proj_bias": gate_bias.cuda(), "down_proj_bias": down_bias.cuda()}},
+                 "quantization": {"experts": {"gate_up_proj": gate_up.to("cuda"), "down_proj": down.to("cuda")}}}
+    got = gpt_oss.GptOssMLP(hidden, intermediate, experts, top_k).apply(variables, x.cuda())
+    assert got.shape == x.shape
+    peak_error, elementwise = oracle.relative_errors(bf16_np(got).reshape(want.shape), want)
+    assert peak_error <= 8e-3 and elementwise <= 2e-2
