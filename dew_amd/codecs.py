@@ -104,6 +104,21 @@ def quantize_mxfp4(weight: torch.Tensor):
     return packed.contiguous(), exponents
 
 
+def dequantize_mxfp4(blocks: torch.Tensor, scales: torch.Tensor, dtype=torch.bfloat16) -> torch.Tensor:
+    """Packed `[expert, output, group, 16]` blocks and E8M0 scales `[expert, output, group]` to `[expert, input, output]`
+    in `dtype` (reference src/dew/interop/codecs.py:193-224, transformers' `convert_moe_packed_tensors`): the low nibble
+    precedes the high one, a group of 32 inputs under the scale `2^(byte - 127)`; every value is exact in bf16. What a
+    load does with a bank that stays dense (src/dew/interop/quantized_loads.py:126-136), wherever the tensors live."""
+    codes = blocks.view(torch.uint8)
+    experts, outputs, groups, packed = codes.shape
+    if packed * 2 != GROUP or tuple(scales.shape) != (experts, outputs, groups):
+        raise ValueError(f"MXFP4 blocks [E, N, K / 32, 16] with scales [E, N, K / 32], not {tuple(codes.shape)} with {tuple(scales.shape)}")
+    nibbles = torch.stack([codes & 0xF, codes >> 4], dim=-1).reshape(experts, outputs, groups, GROUP)
+    values = e2m1_values(codes.device)[nibbles.long()]
+    decoded = torch.ldexp(values, (scales.view(torch.uint8).to(torch.int32) - 127)[..., None])
+    return decoded.reshape(experts, outputs, groups * GROUP).transpose(1, 2).to(dtype).contiguous()
+
+
 def mxfp4_tensor_powers(blocks: torch.Tensor, scales: torch.Tensor):
     """Each expert's power `k` that takes its E8M0 group powers into E4M3's range
     (reference src/dew/interop/codecs.py:238-262): the largest power of a group holding a nonzero code,

@@ -84,6 +84,14 @@ def packed_banks(tensors: Mapping[str, torch.Tensor], config: Mapping, *, device
     return tensors, banks
 
 
+def dense_bank(blocks: torch.Tensor, scales: torch.Tensor) -> formats.Bf16:
+    """An MXFP4 expert bank that `packed_banks` left as the source states it (a depth in no whole NVFP4 stages:
+    gpt-oss's 2880; group powers past one tensor scale's reach), decoded as the reference's load decodes it
+    (`dequantize_mxfp4`, src/dew/interop/codecs.py:193-224) into the unquantized bank the grouped launches multiply:
+    bf16 `[E, in, out]`, every MXFP4 value exactly."""
+    return formats.Bf16(codecs.dequantize_mxfp4(blocks, scales, torch.bfloat16))
+
+
 def fp8_block_bank(weights, scale_invs, *, device_codec: bool | None = None) -> formats.Fp8Blocks:
     """One projection's experts, each stored `[out, in]` e4m3 with `[out/128, in/128]` fp32 inverse scales
     (DeepSeek-V3 / Qwen3-FP8 checkpoints), as the bank the kernels multiply, still quantized: `[E, in, out]` codes

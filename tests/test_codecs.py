@@ -42,6 +42,24 @@ def test_mxfp4_encoder_reproduces_the_released_bytes(name):
     assert np.array_equal(blocks.numpy(), held[f"{name}_blocks"])
 
 
+def test_mxfp4_decodes_to_the_references_dense_bank():
+    """`dequantize_mxfp4` (what a load does with a bank that stays dense: gpt-oss's 2880-deep experts) on the reference's
+    own vector (tests/fixtures/gpt_oss/mxfp4.npz: blocks, scales, decoded output), bit for bit, and on a seeded bank
+    against the oracle's decoder; every value survives the bf16 it is held in."""
+    held = golden("gpt_oss/mxfp4.npz")
+    blocks, scales = torch.from_numpy(held["blocks"]), torch.from_numpy(held["scales"])
+    assert np.array_equal(codecs.dequantize_mxfp4(blocks, scales, torch.float32).numpy(), held["output"])
+    assert np.array_equal(codecs.dequantize_mxfp4(blocks, scales).float().numpy(), held["output"])
+    rng = np.random.default_rng(5)
+    weight = torch.from_numpy((rng.standard_normal((2, 320, 96)) * 0.02).astype(np.float32))     # 320 deep: no whole 256-deep stage
+    blocks, scales = codecs.quantize_mxfp4(weight)
+    dense = codecs.dequantize_mxfp4(blocks, scales)
+    assert dense.shape == (2, 320, 96) and dense.dtype == torch.bfloat16 and dense.is_contiguous()
+    assert np.array_equal(dense.float().numpy(), oracle.decode_mxfp4(blocks.numpy(), scales.numpy()))
+    with pytest.raises(ValueError, match="MXFP4 blocks"):
+        codecs.dequantize_mxfp4(blocks, scales[:, :, :1])
+
+
 def test_mxfp4_bank_as_nvfp4_holds_every_value_exactly():
     rng = np.random.default_rng(1)
     weight = torch.from_numpy((rng.standard_normal((3, 256, 6)) * 0.02).astype(np.float32))

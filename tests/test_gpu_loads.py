@@ -9,6 +9,7 @@ import torch
 from conftest import golden
 
 from dew_amd import _lib, codecs, formats, loads
+from oracle import moe_oracle as oracle
 
 pytestmark = pytest.mark.gpu
 
@@ -115,6 +116,31 @@ def test_a_bank_the_reference_keeps_dense_is_refused_by_name(ops, caplog):
     with caplog.at_level("WARNING"):
         left, banks = loads.packed_banks(tensors, MXFP4)
     assert not banks and set(left) == {"w_blocks", "w_scales"} and "stays dense" in caplog.text
+
+
+def test_a_bank_that_stays_dense_decodes_on_the_device_and_multiplies_as_the_references_does(ops, caplog):
+    """gpt-oss's experts in small: 320 deep (no whole 256-deep NVFP4 stage) and 352 wide. `packed_banks` leaves the
+    bank as the source states it; `dense_bank` decodes it on the device as the reference's load does
+    (`dequantize_mxfp4`) and the unquantized bank's launch multiplies it, against the oracle's product over the
+    oracle's own decoding."""
+    from dew_amd import gemm
+
+    rng = np.random.default_rng(17)
+    experts, depth, width, sizes = 3, 320, 352, [60, 0, 41]
+    weight = torch.from_numpy((rng.standard_normal((experts, depth, width)) * 0.05).astype(np.float32))
+    blocks, scales = codecs.quantize_mxfp4(weight)
+    tensors = {"w_blocks": blocks.cuda(), "w_scales": scales.cuda()}
+    with caplog.at_level("WARNING"):
+        left, banks = loads.packed_banks(tensors, MXFP4)
+    assert not banks and "no whole 256-deep stages" in caplog.text
+    bank = loads.dense_bank(left["w_blocks"], left["w_scales"])
+    assert bank.shape == (experts, depth, width) and bank.weights.is_cuda
+    dense = oracle.decode_mxfp4(blocks.numpy(), scales.numpy())
+    assert np.array_equal(bank.weights.float().cpu().numpy(), dense)
+    x = torch.from_numpy(rng.standard_normal((int(np.sum(sizes)), depth)).astype(np.float32)).to(torch.bfloat16)
+    got = gemm.gemm(x.cuda(), bank, torch.tensor(sizes, dtype=torch.int32).cuda()).float().cpu().numpy()
+    want = oracle.grouped_matmul(x.float().numpy(), dense, sizes)
+    assert got.shape == want.shape and np.abs(got - want).max() <= 2 ** -7 * np.abs(want).max() and (got == want).mean() > 0.97
 
 
 def test_packed_banks_on_the_device_hands_over_the_checkpoints_own_tensors(ops):
