@@ -201,9 +201,10 @@ template <int FORMAT, int MODE, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 && ((MODE == kSwigluOfTwo || MODE == kSwigluOfTwoSplit) ? 2 : 1) * BN == 256) ? 2 : 1) void grouped_gemm_kernel(GemmParams p) {
   constexpr bool PAIRED = MODE == kSwigluOfTwo || MODE == kSwigluOfTwoSplit;
   constexpr bool kSplitOut = MODE == kSwigluOfTwoSplit;
-  // Unquantized banks take the extents the reference's own grouped kernel does (multiples of 8 in its contract; here a depth in
-  // whole 64-deep steps and a width in whole 32-column atoms): a strip past the width multiplies columns it does not store.
-  constexpr bool kRagged = FORMAT == DEW_MOE_W_BF16;
+  // Unquantized and FP4 banks (their atoms are 64 deep and 32 columns wide at most) take a depth in whole 64-deep steps and a
+  // width in whole 32-column atoms, close to the multiples of 8 of the reference's own grouped kernel: a strip past the width
+  // multiplies columns it does not store. (GPT-OSS's experts are 2880 wide: 45 steps, 90 atoms, no whole 128s.)
+  constexpr bool kRagged = FORMAT == DEW_MOE_W_BF16 || FORMAT == DEW_MOE_W_MXFP4 || FORMAT == DEW_MOE_W_NVFP4;
   constexpr bool kGated = MODE == kInterleavedGated;
   constexpr int kOutBN = kGated ? BN / 2 : BN;  // output columns of the tile
   static_assert(WM * WN == 4 && BM % (32 * WM) == 0 && BN % (32 * WN) == 0 && BM % 32 == 0, "tile shape");
@@ -1013,7 +1014,7 @@ static int check_bank(const char* who, const dew_moe_bank* bank, const char* nam
                   bank->format == DEW_MOE_W_MXFP4 || bank->format == DEW_MOE_W_MXFP8 || bank->format == DEW_MOE_W_BF16,
               "%s: %s bank has unknown format %d", who, name, bank->format);
   DEW_REQUIRE(bank->experts >= 1 && bank->experts <= 4096, "%s: %s bank has %d experts", who, name, bank->experts);
-  if (bank->format == DEW_MOE_W_BF16) {  // unquantized matrices: whole 64-deep steps and 32-column atoms (GPT-OSS's 2880 is 45 steps, 90 atoms)
+  if (bank->format == DEW_MOE_W_BF16 || bank->format == DEW_MOE_W_MXFP4 || bank->format == DEW_MOE_W_NVFP4) {  // whole 64-deep steps and 32-column atoms
     DEW_REQUIRE(bank->depth >= 128 && bank->depth % 64 == 0, "%s: %s bank depth %d is not a multiple of 64", who, name, bank->depth);
     DEW_REQUIRE(bank->width >= 128 && bank->width % 32 == 0, "%s: %s bank width %d is not a multiple of 32", who, name, bank->width);
   } else {
@@ -1024,6 +1025,13 @@ static int check_bank(const char* who, const dew_moe_bank* bank, const char* nam
   DEW_REQUIRE(bank->codes && (bank->scales || bank->format == DEW_MOE_W_BF16), "%s: %s bank codes and scales must not be null", who, name);
   DEW_REQUIRE((bank->format != DEW_MOE_W_NVFP4 && bank->format != DEW_MOE_W_MXFP4) || bank->tensor_scale, "%s: %s NVFP4 bank needs tensor scales", who, name);
   DEW_REQUIRE(aligned16(bank->codes), "%s: %s bank codes must be 16-byte aligned", who, name);
+  return DEW_MOE_OK;
+}
+
+// The split-row launches read their rows' scales and their weights in whole 128-deep blocks and write whole 128-column strips.
+static int check_split_extents(const char* who, const dew_moe_bank* bank, const char* name) {
+  DEW_REQUIRE(bank->depth % 128 == 0 && bank->width % 128 == 0, "%s: %s bank [%d, %d] on split rows: depth and width are whole 128s", who, name,
+              bank->depth, bank->width);
   return DEW_MOE_OK;
 }
 
@@ -1204,6 +1212,7 @@ extern "C" int dew_moe_grouped_gemm_split(const void* x_split, const uint8_t* x_
   using namespace dew;
   const char* who = "dew_moe_grouped_gemm_split";
   if (int rc = check_bank(who, w, "weight")) return rc;
+  if (int rc = check_split_extents(who, w, "weight")) return rc;
   DEW_REQUIRE(w->format == DEW_MOE_W_MXFP4 && w->width % 256 == 0,
               "%s: split activations multiply an MXFP4 bank (power-of-two block scales) whose width is whole 256s; this one is "
               "format %d, width %d", who, w->format, w->width);
@@ -1223,6 +1232,8 @@ extern "C" int dew_moe_gateup_swiglu_split(const void* x_split, const uint8_t* x
   const char* who = "dew_moe_gateup_swiglu_split";
   if (int rc = check_bank(who, gate, "gate")) return rc;
   if (int rc = check_bank(who, up, "up")) return rc;
+  if (int rc = check_split_extents(who, gate, "gate")) return rc;
+  if (int rc = check_split_extents(who, up, "up")) return rc;
   DEW_REQUIRE(gate->format == DEW_MOE_W_MXFP4 && up->format == DEW_MOE_W_MXFP4,
               "%s: split activations multiply MXFP4 banks (power-of-two block scales); these are formats %d and %d", who,
               gate->format, up->format);
@@ -1254,6 +1265,7 @@ extern "C" int dew_moe_grouped_gemm_split_blocks(const void* x_split, const uint
   using namespace dew;
   const char* who = "dew_moe_grouped_gemm_split_blocks";
   if (int rc = check_bank(who, w, "weight")) return rc;
+  if (int rc = check_split_extents(who, w, "weight")) return rc;
   DEW_REQUIRE(w->format == DEW_MOE_W_MXFP4 && w->width % 256 == 0,
               "%s: split activations multiply an MXFP4 bank (power-of-two block scales) whose width is whole 256s; this one is "
               "format %d, width %d", who, w->format, w->width);
@@ -1396,6 +1408,8 @@ static int gateup_split_out_of(const char* who, bool second_e2m3, const void* x_
                                uint8_t* hidden_scales, int32_t rows, void* stream, int32_t activation, float limit) {
   if (int rc = check_bank(who, gate, "gate")) return rc;
   if (int rc = check_bank(who, up, "up")) return rc;
+  if (int rc = check_split_extents(who, gate, "gate")) return rc;
+  if (int rc = check_split_extents(who, up, "up")) return rc;
   DEW_REQUIRE(gate->format == DEW_MOE_W_MXFP4 && up->format == DEW_MOE_W_MXFP4,
               "%s: split activations multiply MXFP4 banks (power-of-two block scales); these are formats %d and %d", who,
               gate->format, up->format);
@@ -1460,7 +1474,7 @@ extern "C" int dew_moe_prefers_split_rows(const dew_moe_bank* gate, const dew_mo
   using namespace dew;
   auto wants = [rows](const dew_moe_bank* bank) {
     return bank && bank->layout == DEW_MOE_LAYOUT_PREPARED && bank->format == DEW_MOE_W_MXFP4 && bank->width % 256 == 0 &&
-           bank->experts >= 1 && rows / bank->experts >= DEW_MOE_SPLIT_ROWS_FROM;
+           bank->depth % 128 == 0 && bank->experts >= 1 && rows / bank->experts >= DEW_MOE_SPLIT_ROWS_FROM;
   };
   return wants(gate) && wants(up) && wants(down) && gate->experts == up->experts && gate->depth == up->depth &&
                  gate->width == up->width && down->experts == gate->experts && down->depth == gate->width &&

@@ -336,8 +336,10 @@ extern "C" int dew_moe_prepare_bank(const dew_moe_bank* ref, void* prepared, dew
               ref->experts, ref->depth, ref->width);
   DEW_REQUIRE(ref->codes && (ref->scales || ref->format == DEW_MOE_W_BF16), "dew_moe_prepare_bank: codes and scales must not be null");
   // unquantized matrices as the reference holds them take any width in whole 32-column atoms and any depth in whole 64-deep steps
+  // (so does an MXFP4 checkpoint's bank, whose groups are 32 deep: its atoms are 64 deep and 32 columns wide)
   const bool plain_bf16 = ref->format == DEW_MOE_W_BF16 && ref->layout == DEW_MOE_LAYOUT_REFERENCE;
-  DEW_REQUIRE(ref->width % (plain_bf16 ? 32 : 128) == 0, "dew_moe_prepare_bank: width %d is not a multiple of %d", ref->width, plain_bf16 ? 32 : 128);
+  const bool in_atoms = plain_bf16 || ref->format == DEW_MOE_W_MXFP4_BLOCKS;
+  DEW_REQUIRE(ref->width % (in_atoms ? 32 : 128) == 0, "dew_moe_prepare_bank: width %d is not a multiple of %d", ref->width, in_atoms ? 32 : 128);
   DEW_REQUIRE((reinterpret_cast<uintptr_t>(prepared) & 255u) == 0, "dew_moe_prepare_bank: prepared buffer must be 256-byte aligned");
   hipStream_t s = static_cast<hipStream_t>(stream);
   *out = *ref;
@@ -365,7 +367,7 @@ extern "C" int dew_moe_prepare_bank(const dew_moe_bank* ref, void* prepared, dew
       return fail(DEW_MOE_ELAUNCH, "dew_moe_prepare_bank: reading the scale summary back failed: %s", hipGetErrorString(hipGetLastError()));
     if (!found) out->format = DEW_MOE_W_MXFP4;
   } else if (ref->format == DEW_MOE_W_MXFP4_BLOCKS) {
-    DEW_REQUIRE(ref->depth % 256 == 0, "dew_moe_prepare_bank: an FP4 bank's depth is whole 256s, not %d", ref->depth);
+    DEW_REQUIRE(ref->depth % 64 == 0 && ref->depth >= 128, "dew_moe_prepare_bank: an MXFP4 checkpoint bank's depth is whole 64s, not %d", ref->depth);
     DEW_REQUIRE(aligned16(ref->codes), "dew_moe_prepare_bank: blocks must be 16-byte aligned");
     uint8_t* codes_out = static_cast<uint8_t*>(prepared);
     uint8_t* scales_out = codes_out + codes_bytes(ref->format, ref->experts, ref->depth, ref->width);

@@ -77,10 +77,11 @@ def _bias_fits(case, bias) -> bool:
 
 
 def _extent_units(bank) -> tuple[int, int]:
-    """(depth, width) granules of a bank: an unquantized one's steps and atoms, else the 128 of the block scales and tiles."""
-    plain = torch.is_tensor(bank) or (isinstance(bank, formats.Bf16) and not bank.transposed) or (
-        isinstance(bank, ops.PreparedBank) and bank.descriptor.format == ops._lib.W_BF16)
-    return (64, 32) if plain else (128, 128)
+    """(depth, width) granules of a bank: the 64-deep steps and 32-column atoms of an unquantized bank or an MXFP4
+    checkpoint's, else the 128 of the block scales and tiles."""
+    in_atoms = torch.is_tensor(bank) or (isinstance(bank, formats.Bf16) and not bank.transposed) or isinstance(bank, formats.Mxfp4Blocks) or (
+        isinstance(bank, ops.PreparedBank) and bank.descriptor.format in (ops._lib.W_BF16, ops._lib.W_MXFP4, ops._lib.W_NVFP4))
+    return (64, 32) if in_atoms else (128, 128)
 
 
 def _is_clamp(operands) -> bool:

@@ -55,10 +55,13 @@ def packed_banks(tensors: Mapping[str, torch.Tensor], config: Mapping, *, device
         blocks, scales = (tensors[name + suffix] for suffix in MXFP4_SUFFIXES)
         on_device = blocks.is_cuda if device_codec is None else device_codec
         powers = None
+        depth = blocks.shape[2] * codecs.GROUP if blocks.ndim == 4 else 0
         if blocks.ndim != 4:
             reason = "it holds no experts"
-        elif blocks.shape[2] * codecs.GROUP % formats.NVFP4_STAGE:
-            reason = f"its depth {blocks.shape[2] * codecs.GROUP} is no whole {formats.NVFP4_STAGE}-deep stages"
+        elif depth % formats.NVFP4_STAGE and not (on_device and depth % 64 == 0 and depth >= 128 and blocks.shape[1] % 32 == 0):
+            # (the reference's rule: its NvFp4 words are staged 256 deep. The device re-layout takes the checkpoint's own
+            # tensors in atoms 64 deep and 32 wide, so there gpt-oss's 2880-deep banks stay packed)
+            reason = f"its depth {depth} is no whole {formats.NVFP4_STAGE}-deep stages"
         elif on_device:
             # the device re-layout itself finds an expert whose group powers spread too far, and refuses the bank by name
             from . import gemm, ops

@@ -477,8 +477,8 @@ def prefers_split(bank: PreparedBank, rows: int) -> bool:
     launches): an MXFP4 bank of whole 256-column strips whose groups average 384 rows or more. (Measured on ragged
     groups of 4096 x 14336 x 4096 MLPs against the bf16 launches with their own best tiles: 1.20 times faster at 900
     rows a group, 1.05 at 512 to 768, 1.08 at 384, 0.975 at 256, where the 256-row tiles are half empty.)"""
-    experts, _, width = bank.shape
-    return bank.descriptor.format == _lib.W_MXFP4 and width % 256 == 0 and rows // experts >= SPLIT_ROWS_FROM
+    experts, depth, width = bank.shape
+    return bank.descriptor.format == _lib.W_MXFP4 and depth % 128 == 0 and width % 256 == 0 and rows // experts >= SPLIT_ROWS_FROM
 
 
 SPLIT_ROWS_FROM = 384

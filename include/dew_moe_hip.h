@@ -47,7 +47,8 @@ enum {
                              /* read as the transposed matrices (an input gradient's: depth and width   */
                              /* are then the transposed product's). In the plain layout K is any whole  */
                              /* number of 64s and N of 32s (GPT-OSS's 2880: the reference's kernel takes */
-                             /* whole 8s, grouped_matmul.py:1874-1887); every other bank's are whole 128s. */
+                             /* whole 8s, grouped_matmul.py:1874-1887), and so are a DEW_MOE_W_MXFP4_BLOCKS */
+                             /* bank's; every other bank's are whole 128s (an NVFP4 bank's depth 256s).   */
   DEW_MOE_W_MXFP4_BLOCKS = 7 /* an MXFP4 checkpoint's own tensors, for dew_moe_prepare_bank only: codes =  */
                              /* `*_blocks` u8 [E,N,K/32,16] (low nibble the even element), scales =       */
                              /* `*_scales` E8M0 u8 [E,N,K/32] (src/dew/interop/codecs.py:193-224). The    */

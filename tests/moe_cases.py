@@ -93,4 +93,6 @@ def dequantized(bank):
         return oracle.dequantize_fp8_channels(bank.codes.cpu().numpy(), bank.scales.cpu().numpy()), None
     if isinstance(bank, formats.Bf16):
         return bank.weights.float().cpu().numpy(), None
+    if isinstance(bank, formats.Mxfp4Blocks):
+        return oracle.decode_mxfp4(bank.blocks.cpu().numpy(), bank.scales.cpu().numpy()), None
     raise TypeError(type(bank))

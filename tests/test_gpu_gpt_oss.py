@@ -190,18 +190,24 @@ def test_ragged_unquantized_banks_through_the_paired_and_the_interleaved_launche
     assert np.abs(got - want).max() <= 2 ** -6 * np.abs(want).max() and (got == want).mean() > 0.9
 
 
-def test_a_gpt_oss_layer_of_the_models_own_width_runs_unquantized():
-    """hidden 2880, intermediate 2880 (gpt-oss-20b's config), banks the reference's load keeps dense: the layer through
-    the selector, against the oracle."""
-    from dew_amd import formats, gpt_oss
+@pytest.mark.parametrize("held", ["dense", "packed"])
+def test_a_gpt_oss_layer_of_the_models_own_width(held):
+    """hidden 2880, intermediate 2880 (gpt-oss-20b's config): the banks as the reference's load keeps them (dense bf16)
+    and as the device re-layout keeps them (the checkpoint's MXFP4 blocks, still 4-bit): the layer through the
+    selector, against the oracle."""
+    from dew_amd import codecs, formats, gpt_oss
 
     tokens, hidden, intermediate, experts, top_k = 48, 2880, 2880, 4, 2
     rng = np.random.default_rng(13)
     x = torch.from_numpy(rng.standard_normal((tokens, hidden)).astype(np.float32)).to(torch.bfloat16)
     router_kernel = torch.from_numpy((rng.standard_normal((hidden, experts)) * hidden ** -0.5).astype(np.float32))
     router_bias = torch.from_numpy((rng.standard_normal(experts) * 0.1).astype(np.float32))
-    gate_up = formats.Bf16(torch.from_numpy((rng.standard_normal((experts, hidden, 2 * intermediate)) * hidden ** -0.5).astype(np.float32)).to(torch.bfloat16))
-    down = formats.Bf16(torch.from_numpy((rng.standard_normal((experts, intermediate, hidden)) * intermediate ** -0.5).astype(np.float32)).to(torch.bfloat16))
+    gate_up = torch.from_numpy((rng.standard_normal((experts, hidden, 2 * intermediate)) * hidden ** -0.5).astype(np.float32))
+    down = torch.from_numpy((rng.standard_normal((experts, intermediate, hidden)) * intermediate ** -0.5).astype(np.float32))
+    if held == "packed":
+        gate_up, down = (formats.Mxfp4Blocks(*codecs.quantize_mxfp4(weight)) for weight in (gate_up, down))
+    else:
+        gate_up, down = formats.Bf16(gate_up.to(torch.bfloat16)), formats.Bf16(down.to(torch.bfloat16))
     gate_bias = torch.from_numpy(rng.standard_normal((experts, 2 * intermediate)).astype(np.float32))
     down_bias = torch.from_numpy(rng.standard_normal((experts, hidden)).astype(np.float32))
     want, _ = oracle.gpt_oss_mlp(bf16_np(x), router_kernel.numpy(), router_bias.numpy(), dequantized(gate_up)[0], gate_bias.numpy(),
@@ -213,3 +219,40 @@ def test_a_gpt_oss_layer_of_the_models_own_width_runs_unquantized():
     assert got.shape == x.shape
     peak_error, elementwise = oracle.relative_errors(bf16_np(got).reshape(want.shape), want)
     assert peak_error <= 8e-3 and elementwise <= 2e-2
+
+
+@pytest.mark.parametrize("tile", [0, 32, 128])
+def test_an_mxfp4_checkpoint_bank_of_gpt_oss_extents_stays_packed_on_the_device(ops, tile):
+    """The reference keeps a 2880-deep MXFP4 bank dense because its NvFp4 words are staged 256 deep
+    (src/dew/interop/quantized_loads.py:130-131). The device re-layout takes the checkpoint's own blocks and scales in
+    atoms 64 deep and 32 columns wide, so here such a bank stays 4-bit: its products are those of the dense bank the
+    reference would hold (`dequantize_mxfp4`) in the plain and the gated launches, to the last bit in nearly every output."""
+    from dew_amd import codecs, formats, gemm, loads
+
+    rng = np.random.default_rng(19)
+    experts, depth, width, sizes = 3, 320, 352, [150, 0, 41]
+    weight = torch.from_numpy((rng.standard_normal((experts, depth, 2 * width)) * 0.05).astype(np.float32))
+    blocks, scales = codecs.quantize_mxfp4(weight)
+    tensors = {"mlp.experts.gate_up_proj_blocks": blocks.cuda(), "mlp.experts.gate_up_proj_scales": scales.cuda()}
+    left, banks = loads.packed_banks(tensors, {"quantization_config": {"quant_method": "mxfp4"}})
+    packed = banks["mlp.experts.gate_up_proj"]
+    assert isinstance(packed, formats.Mxfp4Blocks) and packed.shape == (experts, depth, 2 * width)
+    dense = loads.dense_bank(blocks.cuda(), scales.cuda())
+    x = torch.from_numpy(rng.standard_normal((int(np.sum(sizes)), depth)).astype(np.float32)).to(torch.bfloat16).cuda()
+    bias = torch.from_numpy(rng.standard_normal((experts, 2 * width)).astype(np.float32)).to(torch.bfloat16).float().cuda()
+    group_sizes = torch.tensor(sizes, dtype=torch.int32).cuda()
+    assert gemm.prepared(packed).descriptor.format == ops._lib.W_MXFP4
+    def alike(mine, theirs):   # the same exact products, summed in fp32 in the two banks' own depth orders
+        mine, theirs = bf16_np(mine), bf16_np(theirs)
+        return mine.shape == theirs.shape and (mine == theirs).mean() > 0.99 and np.abs(mine - theirs).max() <= 2 ** -7 * np.abs(theirs).max()
+
+    with ops.tile_rows(tile):
+        assert alike(gemm.gemm(x, packed, group_sizes, epilogue="plus_bias", epilogue_operands=(bias,)),
+                     gemm.gemm(x, dense, group_sizes, epilogue="plus_bias", epilogue_operands=(bias,)))
+        gated = gemm.gemm(x, packed, group_sizes, epilogue="gpt_oss_gated", epilogue_operands=(bias, 7.0))
+        assert gated.shape == (x.shape[0], width)
+        assert alike(gated, gemm.gemm(x, dense, group_sizes, epilogue="gpt_oss_gated", epilogue_operands=(bias, 7.0)))
+    values = oracle.decode_mxfp4(blocks.numpy(), scales.numpy())
+    want = oracle.gpt_oss_gating(oracle._biased_matmul(bf16_np(x), values, sizes, bias.cpu().numpy(), dtype="bfloat16", factor=None), limit=7.0)
+    got = bf16_np(gated)
+    assert np.abs(got - want).max() <= 2 ** -6 * np.abs(want).max() and (got == want).mean() > 0.9

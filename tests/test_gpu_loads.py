@@ -119,8 +119,8 @@ def test_a_bank_the_reference_keeps_dense_is_refused_by_name(ops, caplog):
 
 
 def test_a_bank_that_stays_dense_decodes_on_the_device_and_multiplies_as_the_references_does(ops, caplog):
-    """gpt-oss's experts in small: 320 deep (no whole 256-deep NVFP4 stage) and 352 wide. `packed_banks` leaves the
-    bank as the source states it; `dense_bank` decodes it on the device as the reference's load does
+    """gpt-oss's experts in small: 320 deep (no whole 256-deep NVFP4 stage) and 352 wide. By the reference's rule
+    `packed_banks` leaves the bank as the source states it; `dense_bank` decodes it on the device as the reference's load does
     (`dequantize_mxfp4`) and the unquantized bank's launch multiplies it, against the oracle's product over the
     oracle's own decoding."""
     from dew_amd import gemm
@@ -131,8 +131,10 @@ def test_a_bank_that_stays_dense_decodes_on_the_device_and_multiplies_as_the_ref
     blocks, scales = codecs.quantize_mxfp4(weight)
     tensors = {"w_blocks": blocks.cuda(), "w_scales": scales.cuda()}
     with caplog.at_level("WARNING"):
-        left, banks = loads.packed_banks(tensors, MXFP4)
+        left, banks = loads.packed_banks(tensors, MXFP4, device_codec=False)   # the reference's own chain: NvFp4 words, staged 256 deep
     assert not banks and "no whole 256-deep stages" in caplog.text
+    kept, _ = loads.packed_banks(tensors, MXFP4)                                # (the device re-layout keeps this bank packed)
+    assert isinstance(_["w"], formats.Mxfp4Blocks) and set(kept) == {"w"}
     bank = loads.dense_bank(left["w_blocks"], left["w_scales"])
     assert bank.shape == (experts, depth, width) and bank.weights.is_cuda
     dense = oracle.decode_mxfp4(blocks.numpy(), scales.numpy())
