@@ -234,6 +234,34 @@ def test_gateup_swiglu_matches_the_two_products_and_the_rounded_epilogue(ops, qu
     assert (fused == want).mean() > 0.9
 
 
+@pytest.mark.parametrize("tokens,depth,experts,biased", [(1, 64, 8, False), (37, 512, 16, True), (64, 2880, 32, True), (100, 2048, 128, False),
+                                                         (257, 1024, 160, True), (96, 7168, 256, False), (33, 768, 384, True),
+                                                         (8200, 256, 160, True), (3000, 128, 40, False), (50, 520, 60, True), (70, 72, 600, False)])
+def test_gate_logits_are_fp32_products_summed_in_fp32(ops, tokens, depth, experts, biased):
+    """`Router.logits` (src/dew/nn/moe.py:526-534): bf16 tokens widened to fp32 times the fp32 gate kernel, IEEE fp32.
+    Against the float64 product: within a few fp32 roundings of the summed magnitudes, on the matrix-instruction kernel
+    (depths in whole 16s, up to 512 experts) and the plain one (the last two shapes); tokens in no whole 32s, experts in
+    no whole 32s, a bias on the finished sums."""
+    rng = np.random.default_rng(tokens + depth + experts)
+    x = torch.from_numpy(rng.standard_normal((tokens, depth)).astype(np.float32)).to(torch.bfloat16)
+    kernel = torch.from_numpy((rng.standard_normal((depth, experts)) * depth ** -0.5).astype(np.float32))
+    bias = torch.from_numpy(rng.standard_normal(experts).astype(np.float32)) if biased else None
+    guard = torch.full((tokens + 1, experts), 7.0, dtype=torch.float32, device="cuda")
+    got = ops.router_logits(x.cuda(), kernel.cuda(), None if bias is None else bias.cuda())
+    assert got.shape == (tokens, experts) and got.dtype == torch.float32 and bool(guard.eq(7.0).all())
+    exact = x.double().numpy() @ kernel.double().numpy()
+    magnitudes = np.abs(x.double().numpy()) @ np.abs(kernel.double().numpy())
+    if biased:
+        exact = exact + bias.double().numpy()
+        magnitudes = magnitudes + np.abs(bias.double().numpy())
+    assert np.all(np.abs(got.cpu().numpy() - exact) <= 2.0 ** -19 * magnitudes + 1e-30)
+    want = oracle.router_logits(x.float().numpy(), kernel.numpy())
+    if biased:
+        want = want + bias.numpy()
+    assert np.abs(got.cpu().numpy() - want).max() <= 1e-5 * np.abs(want).max()
+    assert torch.equal(got, ops.router_logits(x.cuda(), kernel.cuda(), None if bias is None else bias.cuda()))   # the same bits every time
+
+
 @pytest.mark.parametrize("tile", [0, 32, 128])
 @pytest.mark.parametrize("activation,limit", [("swiglu", 0.25), ("geglu", None), ("geglu", 0.5)])
 @pytest.mark.parametrize("quant", ["fp8_channel", "fp8_block", "mxfp4", "nvfp4", "bf16"])
