@@ -90,7 +90,8 @@ struct GemmParams {
   bf16_t* out;
   const uint8_t* a_scale;  // split activations: each source row's e8m0 scale, or its row of block_scale_pitch(depth) of them
   uint8_t* out_scale;      // split output: each written row's block_scale_pitch(width) e8m0 scales, one for 128 columns
-  const float* bias;  // [experts, width] values of the compute dtype held in fp32, or null
+  const float* bias;  // [experts, width] fp32, or null
+  int round_bias;     // the bias is a parameter of a bf16 product: rounded to bf16 as it is read (a quantized-rows recipe's stays fp32)
   float limit;        // the interleaved gated epilogue's clamp; a paired launch's (0: none)
   int gating;         // a paired launch's gate: DEW_MOE_GATE_SILU (SwiGLU) or DEW_MOE_GATE_GELU_TANH (GeGLU)
   int experts, depth, width, rows, m_tile_bound;
@@ -883,6 +884,10 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
     bias[j] = (!PAIRED && p.bias) ? p.bias[static_cast<size_t>(expert) * p.width + (kRagged ? min(n0 + wn0 + 32 * j + lane % 32, p.width - 1)
                                                                                                : n0 + wn0 + 32 * j + lane % 32)]
                                   : 0.0f;
+  if (p.round_bias) {  // (a caller passes the parameter as it holds it)
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) bias[j] = bf16_round(bias[j]);
+  }
   // quantized rows: a weight block scale that is no normal power of two cannot enter the instruction; the tile is
   // then written as NaN (through the addend every sum meets) rather than as the product under another scale
   if (kFp8Rows && unscalable != 0) {
@@ -1178,13 +1183,15 @@ extern "C" int dew_moe_tile_rows(int32_t rows) {
 }
 
 static int grouped_gemm_of(const char* who, const void* x, const int32_t* gather, const int32_t* offsets, const int32_t* sizes,
-                           const dew_moe_bank* w, const float* bias, const int32_t* scatter, void* out, int32_t rows, void* stream) {
+                           const dew_moe_bank* w, const float* bias, const int32_t* scatter, void* out, int32_t rows, void* stream,
+                           bool round_bias = false) {
   using namespace dew;
   if (int rc = check_bank(who, w, "weight")) return rc;
   DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
   if (rows == 0) return DEW_MOE_OK;
   GemmParams p{};
   if (int rc = fill_single(who, p, x, gather, offsets, w, bias, scatter, out, rows, sizes)) return rc;
+  p.round_bias = round_bias ? 1 : 0;
   return launch<kPlain>(who, p, w->format, static_cast<hipStream_t>(stream));
 }
 
@@ -1192,6 +1199,15 @@ extern "C" int dew_moe_grouped_gemm_bias(const void* x, const int32_t* gather, c
                                          const dew_moe_bank* w, const float* bias, const int32_t* scatter, void* out,
                                          int32_t rows, void* stream) {
   return grouped_gemm_of("dew_moe_grouped_gemm", x, gather, offsets, nullptr, w, bias, scatter, out, rows, stream);
+}
+
+extern "C" int dew_moe_grouped_gemm_param_bias(const void* x, const int32_t* gather, const int32_t* offsets, const int32_t* group_sizes,
+                                               const dew_moe_bank* w, const float* bias, const int32_t* scatter, void* out,
+                                               int32_t rows, void* stream) {
+  using namespace dew;
+  DEW_REQUIRE(rows == 0 || (offsets != nullptr) != (group_sizes != nullptr),
+              "dew_moe_grouped_gemm_param_bias: the groups come as offsets [E + 1] or as group_sizes [E], one of them");
+  return grouped_gemm_of("dew_moe_grouped_gemm_param_bias", x, gather, offsets, group_sizes, w, bias, scatter, out, rows, stream, true);
 }
 
 extern "C" int dew_moe_grouped_gemm_sizes(const void* x, const int32_t* gather, const int32_t* group_sizes,
@@ -1571,6 +1587,7 @@ extern "C" int dew_moe_gateup_interleaved(const void* x, const int32_t* gather, 
   if (rows == 0) return DEW_MOE_OK;
   GemmParams p{};
   if (int rc = fill_single(who, p, x, gather, offsets, gate_up, bias, nullptr, hidden, rows)) return rc;
+  p.round_bias = 1;
   p.limit = limit;
   return launch<kInterleavedGated>(who, p, gate_up->format, static_cast<hipStream_t>(stream));
 }

@@ -193,8 +193,8 @@ def gemm(lhs: torch.Tensor, rhs, group_sizes, *, paired=None, gather: torch.Tens
     groups = GroupSizes.operands(group_sizes)    # no prefix launch where the caller holds sizes only
     offsets = groups.pop("offsets")
     if paired is None:
-        bias = epilogue_operands[0] if epilogue == "plus_bias" else None
-        return ops.grouped_gemm(lhs, first, offsets, gather=gather, scatter=scatter, bias=bias, **groups)
+        bias = epilogue_operands[0] if epilogue == "plus_bias" else None   # (`_plus_bias`'s operand: rounded to the compute dtype, in the launch)
+        return ops.grouped_gemm(lhs, first, offsets, gather=gather, scatter=scatter, bias=bias, round_bias=True, **groups)
     second = prepared(paired)
     if scatter is not None:
         raise selection.KernelRefused(GROUPED_MATMUL, "hip", selection.Refusal("pair-scatter", "a paired product writes sorted rows"), iter(()))

@@ -75,7 +75,10 @@ def _biased(bias, compute) -> dict:
 
 
 def rounded_operand(value: torch.Tensor, compute) -> torch.Tensor:
-    """`value` rounded to `compute` and held in fp32 (the reference's `rounded_operand(...).astype(work)`)."""
+    """`value` rounded to `compute` and held in fp32 (the reference's `rounded_operand(...).astype(work)`). The launches
+    round a bias to bfloat16 as they read it, so for that compute dtype the parameter goes in as it is held: no pass."""
+    if compute == torch.bfloat16:
+        return value.to(torch.float32).contiguous()
     return value.to(compute).to(torch.float32).contiguous()
 
 

@@ -318,9 +318,11 @@ def _product_rows(operand: torch.Tensor, name: str, offsets: torch.Tensor, exper
 
 def grouped_gemm(x: torch.Tensor, bank: PreparedBank, offsets: torch.Tensor | None, *, gather: torch.Tensor | None = None,
                  scatter: torch.Tensor | None = None, rows: int | None = None,
-                 bias: torch.Tensor | None = None, sizes: torch.Tensor | None = None) -> torch.Tensor:
+                 bias: torch.Tensor | None = None, sizes: torch.Tensor | None = None, round_bias: bool = False) -> torch.Tensor:
     """`out[scatter[i]] = x[gather[i]] @ W[expert of sorted position i] (+ bias[expert])`, bf16 `[rows, N]`. The groups
-    are `offsets [E + 1]`, or, where that is None, `sizes [E]` (the launch then forms the prefix on the device)."""
+    are `offsets [E + 1]`, or, where that is None, `sizes [E]` (the launch then forms the prefix on the device). The
+    bias meets the fp32 sums as it is given, or, with `round_bias` (an expert layer's parameter), rounded to bf16 as the
+    launch reads it."""
     _device(x, "x", torch.bfloat16)
     experts, depth, width = bank.shape
     if x.shape[-1] != depth:
@@ -328,6 +330,11 @@ def grouped_gemm(x: torch.Tensor, bank: PreparedBank, offsets: torch.Tensor | No
     rows = _product_rows(x, "x", offsets, experts, gather, scatter, rows, sizes)
     bias = _expert_bias(bias, experts, width)
     out = torch.empty((rows, width), dtype=torch.bfloat16, device=x.device)
+    if round_bias and bias is not None:
+        _lib.check(_lib.library().dew_moe_grouped_gemm_param_bias(_ptr(x), _ptr(gather), _ptr(offsets), _ptr(None if offsets is not None else sizes),
+                                                                  bank.descriptor, _ptr(bias), _ptr(scatter), _ptr(out), rows, _stream()),
+                   "dew_moe_grouped_gemm_param_bias")
+        return out
     if offsets is None:
         _lib.check(_lib.library().dew_moe_grouped_gemm_sizes(_ptr(x), _ptr(gather), _ptr(sizes), bank.descriptor, _ptr(bias),
                                                              _ptr(scatter), _ptr(out), rows, _stream()), "dew_moe_grouped_gemm_sizes")

@@ -218,6 +218,12 @@ int dew_moe_grouped_gemm_sizes(const void* x, const int32_t* gather, const int32
                                int32_t rows, void* stream);
 int dew_moe_gateup_swiglu_sizes(const void* x, const int32_t* gather, const int32_t* group_sizes /* [E] */,
                                 const dew_moe_bank* gate, const dew_moe_bank* up, void* hidden, int32_t rows, void* stream);
+/* dew_moe_grouped_gemm_bias (groups as offsets or sizes, the other NULL) taking the bias as the parameter holds it, fp32: the
+ * launch rounds it to the compute dtype as it reads it (`rounded_operand`, src/dew/nn/moe.py:729-742), so the caller
+ * makes no rounding pass of its own a call. dew_moe_gateup_interleaved reads its bias the same way.             */
+int dew_moe_grouped_gemm_param_bias(const void* x, const int32_t* gather, const int32_t* offsets /* nullable */,
+                                    const int32_t* group_sizes /* nullable */, const dew_moe_bank* w, const float* bias,
+                                    const int32_t* scatter, void* out, int32_t rows, void* stream);
 
 /* The same with each expert's bias[E,N] (values of the compute dtype held in fp32) added to its rows' fp32
  * sums before their one rounding (src/dew/nn/moe.py:729-742 _biased / _plus_bias; NULL = none).          */

@@ -45,6 +45,11 @@ def test_the_bias_meets_the_fp32_sums_before_their_one_rounding(ops, quant, labe
     scatter = torch.from_numpy(np.random.default_rng(5).permutation(x.shape[0]).astype(np.int32))
     prepared = ops.prepare(bank.to("cuda"))
     got = ops.grouped_gemm(x.cuda(), prepared, torch.from_numpy(offsets).cuda(), bias=held.cuda(), scatter=scatter.cuda())
+    # with `round_bias` the launch rounds the bias to the compute dtype as it reads it: the fp32 parameter itself gives the same bits
+    assert torch.equal(got, ops.grouped_gemm(x.cuda(), prepared, torch.from_numpy(offsets).cuda(), bias=bias.cuda(), scatter=scatter.cuda(),
+                                             round_bias=True))
+    assert torch.equal(got, ops.grouped_gemm(x.cuda(), prepared, None, sizes=torch.tensor(sizes, dtype=torch.int32).cuda(), bias=bias.cuda(),
+                                             scatter=scatter.cuda(), round_bias=True))
     got = bf16_np(got)[scatter.numpy()]
     assert np.abs(got - want).max() <= 2 ** -7 * np.abs(want).max()
     assert (got == want).mean() > 0.97
