@@ -3,7 +3,7 @@
 // Depths in whole 16s run on the fp32 matrix instruction (v_mfma_f32_32x32x2_f32: fp32 operands, exact products, fp32
 // sums): a block takes 32 (or 64) tokens and up to four 32-expert tiles, its wavefronts a share of the depth each; the
 // partial sums of a tile meet in LDS in wavefront order, so the result does not depend on timing. Measured: 64 tokens
-// of GPT-OSS's 2880 x 32 gate in about 10 us and 8192 tokens of a 7168 x 256 gate in 339 us (89 TFLOP/s), where the
+// of GPT-OSS's 2880 x 32 gate in about 10 us and 8192 tokens of a 7168 x 256 gate in 319 us (94 TFLOP/s), where the
 // plain kernel below (a 64-token x 64-expert tile, 16-deep LDS steps, fp32 FMA; depths in no whole 16s still take it)
 // needed 550 us and 1.3 ms.
 #include "common.h"
@@ -42,27 +42,47 @@ __global__ __launch_bounds__(64 * WAVES) void router_logits_mfma_kernel(const bf
     for (int c = 0; c < TILES; ++c)
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[r][c][i] = 0.0f;
-  for (int chunk = first; chunk < last; ++chunk) {
-    float a[ROWS][8];
+  // A chunk's operands are loaded while the chunk before it multiplies (a block may be alone on its CU: nothing else
+  // would hide the loads).
+  u32x4 a_words[2][ROWS];
+  float b[2][TILES][8];
+  auto load = [&](int buffer, int chunk) __attribute__((always_inline)) {
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-      const u32x4 words = *reinterpret_cast<const u32x4*>(a_src[r] + chunk * 16);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        a[r][2 * i] = __uint_as_float(words[i] << 16);
-        a[r][2 * i + 1] = __uint_as_float(words[i] & 0xFFFF0000u);
-      }
-    }
+    for (int r = 0; r < ROWS; ++r) a_words[buffer][r] = *reinterpret_cast<const u32x4*>(a_src[r] + chunk * 16);
     const float* b_src = kernel + static_cast<size_t>(chunk * 16 + 8 * (lane / 32)) * experts;
 #pragma unroll
-    for (int c = 0; c < TILES; ++c) {
-      float b[8];
+    for (int c = 0; c < TILES; ++c)
 #pragma unroll
-      for (int j = 0; j < 8; ++j) b[j] = b_src[static_cast<size_t>(j) * experts + column[c]];
+      for (int j = 0; j < 8; ++j) b[buffer][c][j] = b_src[static_cast<size_t>(j) * experts + column[c]];
+  };
+  auto multiply = [&](int buffer) __attribute__((always_inline)) {
+    float a[ROWS][8];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        a[r][2 * i] = __uint_as_float(a_words[buffer][r][i] << 16);
+        a[r][2 * i + 1] = __uint_as_float(a_words[buffer][r][i] & 0xFFFF0000u);
+      }
+#pragma unroll
+    for (int c = 0; c < TILES; ++c)
 #pragma unroll
       for (int r = 0; r < ROWS; ++r)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[r][j], b[j], acc[r][c], 0, 0, 0);
+        for (int j = 0; j < 8; ++j) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[r][j], b[buffer][c][j], acc[r][c], 0, 0, 0);
+  };
+  if constexpr (WAVES == 16) {  // a decode step's wavefronts walk a few chunks each: nothing to overlap
+    for (int chunk = first; chunk < last; ++chunk) {
+      load(0, chunk);
+      multiply(0);
+    }
+  } else {
+    if (first < last) load(0, first);
+    for (int chunk = first; chunk < last; chunk += 2) {
+      load(1, min(chunk + 1, last - 1));
+      multiply(0);
+      load(0, min(chunk + 2, last - 1));
+      if (chunk + 1 < last) multiply(1);
     }
   }
   // register i of lane l is the sum of token 8 (i / 4) + 4 (l / 32) + i % 4, expert column l % 32 of the tile. A tile's
