@@ -354,6 +354,20 @@ def measure(config, args, device, sustained, with_cpu_baseline):
                    "algorithmic_flops": flops},
         "roofline": roofline,
     }
+    # The router's own GEMM (x @ gate kernel in fp32): outside the step, whose logits are synthetic as the benchmark defines
+    # them; what a layer that multiplies its own gate kernel adds to the step.
+    gate_kernel = torch.randn((case.d_model, case.experts), device=device, dtype=torch.float32) * case.d_model ** -0.5
+    stepper.ops.router_logits(data["x"], gate_kernel)
+    first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    first.record()
+    for _ in range(5):
+        stepper.ops.router_logits(data["x"], gate_kernel)
+    last.record()
+    torch.cuda.synchronize()
+    gate_us = first.elapsed_time(last) / 5 * 1e3
+    result["router_logits"] = {"us": round(gate_us, 1), "tflops_fp32": round(2.0 * case.tokens * case.d_model * case.experts / gate_us / 1e6, 2),
+                               "note": "x @ gate kernel [D, E] in fp32 (dew_moe_router_logits), launched eagerly; not part of ms_per_step"}
+    del gate_kernel
     # the routing's least top-k margin: how close the last chosen selection comes to the best one left out
     router = {k: v for k, v in case.router.items() if k in ("score_function", "expert_groups", "groups_per_token")}
     _, selection = oracle.selection_scores(data["logits"].cpu().numpy(), bias=None if data["bias"] is None else data["bias"].cpu().numpy(),
@@ -429,7 +443,7 @@ def main():
         "ms_per_step": top["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic", "config": top["config"], "roofline": top["roofline"],
     }
-    for name in ("cpu_baseline", "sample_parity", "min_topk_margin"):
+    for name in ("cpu_baseline", "sample_parity", "min_topk_margin", "router_logits"):
         if name in top:
             result[name] = top[name]
     if not args.only:
