@@ -81,6 +81,25 @@ __global__ __launch_bounds__(256) void combine_kernel(const bf16_t* __restrict__
   }
 }
 
+// Llama 4's placement of the routing weight (src/dew/nn/moe.py:1124-1126): sorted position i holds token gather[i]'s
+// row times the weight of its slot, weights[slots[i]], both in bf16, the product rounded once.
+__global__ __launch_bounds__(256) void scale_rows_kernel(const bf16_t* __restrict__ x, const int32_t* __restrict__ gather,
+                                                         const int32_t* __restrict__ slots, const float* __restrict__ weights,
+                                                         bf16_t* __restrict__ out, int rows, int depth) {
+  const int chunks = depth / 8;
+  const long long total = static_cast<long long>(rows) * chunks;
+  for (long long item = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; item < total;
+       item += static_cast<long long>(gridDim.x) * blockDim.x) {
+    const int row = static_cast<int>(item / chunks), chunk = static_cast<int>(item % chunks);
+    const float w = bf16_round(weights[slots[row]]);
+    const Bf16x8 source = *reinterpret_cast<const Bf16x8*>(x + static_cast<size_t>(gather[row]) * depth + static_cast<size_t>(chunk) * 8);
+    Bf16x8 scaled;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) scaled.v[i] = f32_to_bf16(bf16_to_f32(source.v[i]) * w);
+    *reinterpret_cast<Bf16x8*>(out + static_cast<size_t>(row) * depth + static_cast<size_t>(chunk) * 8) = scaled;
+  }
+}
+
 // `limit` > 0: the gate clamped from above and the up projection both ways before their product (`swiglu_clamped`,
 // src/dew/nn/activations.py:327-333); the limit enters as the bf16 the operands' dtype rounds it to.
 __global__ __launch_bounds__(256) void swiglu_kernel(const bf16_t* __restrict__ gate, const bf16_t* __restrict__ up,
@@ -134,6 +153,20 @@ extern "C" int dew_moe_combine(const void* slots, const float* weights, const vo
     default: stream_slots ? launch(combine_kernel<0, true>) : launch(combine_kernel<0, false>); break;
   }
   return launched("combine_kernel");
+}
+
+extern "C" int dew_moe_scale_rows(const void* x, const int32_t* gather, const int32_t* slots, const float* weights, void* out,
+                                  int32_t rows, int32_t depth, void* stream) {
+  using namespace dew;
+  DEW_REQUIRE(rows >= 0 && depth >= 8 && depth % 8 == 0, "dew_moe_scale_rows: rows %d, depth %d (whole 8s)", rows, depth);
+  if (rows == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(x && gather && slots && weights && out, "dew_moe_scale_rows: x, gather, slots, weights and out must not be null");
+  DEW_REQUIRE(aligned16(x) && aligned16(out), "dew_moe_scale_rows: x and out must be 16-byte aligned");
+  const long long total = static_cast<long long>(rows) * (depth / 8);
+  const int blocks = static_cast<int>(min((total + 255) / 256, 256ll * 64));
+  hipLaunchKernelGGL(scale_rows_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<const bf16_t*>(x), gather,
+                     slots, weights, static_cast<bf16_t*>(out), rows, depth);
+  return launched("scale_rows_kernel");
 }
 
 extern "C" int dew_moe_swiglu(const void* gate, const void* up, void* hidden, int64_t count, void* stream) {

@@ -115,10 +115,10 @@ HIP = Kernel("hip", (
     # reference's own grouped kernel takes extents in whole 8s, `_Cutlass.in_contract`, src/dew/nn/kernels/grouped_matmul.py:1874-1887)
     Requirement("depth", lambda c: _shape(c.rhs)[1] % _extent_units(c.rhs)[0] == 0 and _shape(c.rhs)[1] >= 128
                                    and c.lhs.shape[-1] == _shape(c.rhs)[1],
-                lambda c: f"depth {_shape(c.rhs)[1]} against rows {c.lhs.shape[-1]} deep; depths are whole {_extent_units(c.rhs)[0]}s",
+                lambda c: f"depth {_shape(c.rhs)[1]} against rows {c.lhs.shape[-1]} deep; depths are whole {_extent_units(c.rhs)[0]}s, 128 at least",
                 row="ragged depth"),
     Requirement("width", lambda c: _shape(c.rhs)[2] % _extent_units(c.rhs)[1] == 0 and _shape(c.rhs)[2] >= 128,
-                lambda c: f"width {_shape(c.rhs)[2]} is not a multiple of {_extent_units(c.rhs)[1]}", row="ragged width"),
+                lambda c: f"width {_shape(c.rhs)[2]} is not a multiple of {_extent_units(c.rhs)[1]}, 128 at least", row="ragged width"),
     Requirement("pair", lambda c: c.paired is None or (_shape(c.paired) == _shape(c.rhs) and type(c.paired) is type(c.rhs)),
                 "a paired product's matrices share one shape and format"),
     Requirement("epilogue", lambda c: _EPILOGUES.get(c.epilogue, lambda c: False)(c),

@@ -414,6 +414,20 @@ def gated_product(gate: torch.Tensor, up: torch.Tensor, activation: str = "swigl
     return hidden
 
 
+def scale_rows(x: torch.Tensor, gather: torch.Tensor, slots: torch.Tensor, weights: torch.Tensor) -> torch.Tensor:
+    """The rows Llama 4's input-scaled experts multiply: sorted position i holds `bf16(x[gather[i]] * bf16(weights.ravel()[slots[i]]))`,
+    bf16 `[len(gather), D]` (`gather`, `slots` = the dispatch sort's `rows` and `order`)."""
+    _device(x, "x", torch.bfloat16), _device(weights, "weights", torch.float32)
+    for name, index in (("gather", gather), ("slots", slots)):
+        _device(index, name, torch.int32)
+    if x.dim() != 2 or gather.numel() != slots.numel() or slots.numel() > weights.numel():
+        raise KernelError(f"{gather.numel()} rows of x {tuple(x.shape)} under {slots.numel()} slots of {weights.numel()} weights")
+    out = torch.empty((gather.numel(), x.shape[1]), dtype=torch.bfloat16, device=x.device)
+    _lib.check(_lib.library().dew_moe_scale_rows(_ptr(x), _ptr(gather), _ptr(slots), _ptr(weights), _ptr(out), gather.numel(), x.shape[1],
+                                                 _stream()), "dew_moe_scale_rows")
+    return out
+
+
 def swiglu(gate: torch.Tensor, up: torch.Tensor, limit: float | None = None) -> torch.Tensor:
     """`gated_product` of 'swiglu'."""
     return gated_product(gate, up, "swiglu", limit)

@@ -434,6 +434,12 @@ int dew_moe_gated_product(const void* gate, const void* up, int32_t activation, 
 int dew_moe_gateup_gated(const void* x, const int32_t* gather, const int32_t* offsets /* nullable */,
                          const int32_t* group_sizes /* nullable */, const dew_moe_bank* gate, const dew_moe_bank* up,
                          int32_t activation, float limit, void* hidden, int32_t rows, void* stream);
+/* Llama 4's input-scaled experts (`scale_inputs`, src/dew/nn/moe.py:1124-1126, 1256-1259: `Llama4TextMoe.forward`): the
+ * rows the experts multiply, out[i] = bf16(x[gather[i]] * bf16(weights[slots[i]])) for the sorted positions i < rows
+ * (gather = the sort's rows, slots = its order, weights [T*k] the router's). The launches then read `out` without a
+ * gather and the combine sums the slots unweighted (weights of one).                                              */
+int dew_moe_scale_rows(const void* x /* bf16 [T,D] */, const int32_t* gather, const int32_t* slots, const float* weights,
+                       void* out /* bf16 [rows,D] */, int32_t rows, int32_t depth, void* stream);
 /* The activation alone: out = bf16(x * logistic(x)), formed in fp32 and rounded once (`silu`, src/dew/nn/activations.py:100-106),
  * which routed value experts pass each chosen projection through (src/dew/nn/value_experts.py:79-82).      */
 int dew_moe_silu(const void* x /* bf16 [count] */, void* out /* bf16 [count] */, int64_t count, void* stream);

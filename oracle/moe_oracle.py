@@ -18,6 +18,9 @@ What pins each function (tests/test_oracle_golden.py):
   src/dew/algebra/bits.py:696-705 checked against each other on every basis word and random words; staged
   order known answers of tests/test_gemm_nvfp4.py:37-38; form digest 7fb7f1b609cea47a.
 * `combine`: known answer of tests/test_moe_precision.py:652-674 (weights 1/2 +- 2^-11 give 2^-10).
+* `expert_mlp(scale_inputs=True)` / `sparse_mlp(scale_inputs=True)` (Llama 4's input-scaled experts, fp32 mode): `output`
+  of tests/fixtures/llama4/moe.npz (sigmoid of the top-2 logits on each token's input, the shared expert added) at the
+  reference's own tolerance 1e-5 (tests/test_llama4.py:162-191); weighting the outputs instead must miss it by > 1e-3.
 * `swiglu`: closed form, the two bf16 roundings checked on hand-computed cases.
 * `gpt_oss_mlp` (fp32 mode): `output` of tests/fixtures/gpt_oss/moe.npz at the reference's own tolerance (1.6e-4,
   tests/test_gpt_oss.py:45-66): biased router, top-k on the logits, softmax of the chosen, interleaved gate/up
@@ -945,7 +948,7 @@ def capacity_admitted(indices, num_experts, capacity_factor):
 
 
 def expert_mlp(x, weights, indices, gate_w, up_w, down_w, *, dtype="bfloat16", factors=(None, None, None),
-               limit=None, capacity_factor=None, activation="swiglu"):
+               limit=None, capacity_factor=None, activation="swiglu", scale_inputs=False):
     """`ExpertMLP.__call__` (src/dew/nn/moe.py:1335-1353) on one device: sort, gather, paired gate/up
     products, SwiGLU, down product scattered to slot order, combine. The matrices are the dequantized
     `[E, depth, width]` values; `indices [T, k]`, or `[..., length, k]` with `capacity_factor` (each leading row a
@@ -960,6 +963,11 @@ def expert_mlp(x, weights, indices, gate_w, up_w, down_w, *, dtype="bfloat16", f
     weights = np.asarray(weights).reshape(indices.shape)
     plan = sorted_by_expert(indices, experts)
     rows = x[plan["rows"]]   # (rows past the groups, the dropped slots', are multiplied by no matrix: `grouped_matmul` leaves them zero)
+    if scale_inputs:
+        # Llama 4's placement of the routing weight (src/dew/nn/moe.py:1124-1126, `Llama4TextMoe.forward`): each slot's
+        # row times its weight, both in the compute dtype, one rounding; the outputs are then summed unweighted (:1328-1330)
+        scale = weights.reshape(-1)[plan["order"]][:, None]
+        rows = bf16_round(bf16_round(rows) * bf16_round(scale)) if dtype == "bfloat16" else (rows * scale.astype(F32)).astype(F32)
     gate = grouped_matmul(rows, gate_w, plan["sizes"], dtype=dtype, factor=factors[0])
     up = grouped_matmul(rows, up_w, plan["sizes"], dtype=dtype, factor=factors[1])
     hidden = GATED_PRODUCTS[activation](gate, up, dtype=dtype, limit=limit)
@@ -968,7 +976,7 @@ def expert_mlp(x, weights, indices, gate_w, up_w, down_w, *, dtype="bfloat16", f
     slots[plan["order"]] = projected
     tokens, k = np.asarray(indices).shape
     slots = slots.reshape(tokens, k, -1)
-    out = combine(slots, weights, dtype=dtype)
+    out = combine(slots, np.ones_like(weights) if scale_inputs else weights, dtype=dtype)
     return out, {**plan, "gate": gate, "up": up, "hidden": hidden, "slots": slots}
 
 
@@ -1054,12 +1062,12 @@ def gated_mlp(x, gate_w, up_w, down_w, *, dtype="bfloat16"):
 
 
 def sparse_mlp(x, logits, gate_w, up_w, down_w, *, top_k_count, dtype="bfloat16", shared=None,
-               factors=(None, None, None), limit=None, **router):
+               factors=(None, None, None), limit=None, scale_inputs=False, **router):
     """`SparseMLP.__call__` (src/dew/nn/moe.py:1488-1503) from the router logits on: route, routed
     experts, plus the shared expert's output (`shared` = its three dense matrices)."""
     weights, indices = route(logits, top_k_count, **router)
     routed, trace = expert_mlp(x, weights, indices, gate_w, up_w, down_w, dtype=dtype, factors=factors,
-                               limit=limit)
+                               limit=limit, scale_inputs=scale_inputs)
     trace.update(weights=weights, indices=indices)
     if shared is not None:
         both = routed + gated_mlp(x, *shared, dtype=dtype)

@@ -377,3 +377,57 @@ def test_a_shared_expert_keeps_its_own_gating_beside_clamped_or_geglu_experts(ga
     want = oracle.bf16_round(routed + oracle.gated_mlp(x, *shared))
     by_max, by_element = oracle.relative_errors(got, want)
     assert by_max <= 6e-3 and by_element <= TOLERANCE, (by_max, by_element)
+
+
+def test_llama_4s_input_scaled_experts_on_the_references_fixture_and_a_seeded_layer():
+    """`scale_inputs` (src/dew/nn/moe.py:1124-1126, 1256-1259): the routing weight on each expert's input, the outputs
+    summed unweighted. The reference's own vector (tests/fixtures/llama4/moe.npz: 32-wide tokens, 48-wide experts) padded
+    with zeros to the launches' extents and held in bf16: the layer's output is the fixture's within bf16 arithmetic, and
+    weighting the outputs instead is far from it. Then a seeded layer of kernel-sized FP8 banks against the oracle."""
+    import dataclasses
+
+    from conftest import golden
+    from dew_amd import formats, moe
+
+    tensors = golden("llama4/moe.npz")
+    hidden = tensors["hidden"].reshape(-1, 32)
+    gate_up = tensors["feed_forward.experts.gate_up_proj"]
+    D, F = 128, 128
+
+    def padded(matrix, rows, cols):      # [..., r, c] -> [..., rows, cols], zeros around
+        out = np.zeros((*matrix.shape[:-2], rows, cols), np.float32)
+        out[..., :matrix.shape[-2], :matrix.shape[-1]] = matrix
+        return torch.from_numpy(out).to(torch.bfloat16)
+
+    def bank(matrix, rows, cols):
+        return {"kernel": formats.Bf16(padded(matrix, rows, cols)).to("cuda")}
+
+    experts = {"gate_proj": bank(gate_up[..., :48], D, F), "up_proj": bank(gate_up[..., 48:], D, F),
+               "down_proj": bank(tensors["feed_forward.experts.down_proj"], F, D)}
+    shared = {name: bank(tensors[f"feed_forward.shared_expert.{name}.weight"].T[None], *((D, F) if name != "down_proj" else (F, D)))
+              for name in ("gate_proj", "up_proj", "down_proj")}
+    variables = {"params": {"gate": {"kernel": padded(tensors["feed_forward.router.weight"].T, D, 4).float().cuda()}},
+                 "quantization": {"experts": experts, "shared_experts": shared}}
+    x = padded(hidden, hidden.shape[0], D).cuda()
+    layer = moe.SparseMLP(num_experts=4, top_k=2, hidden_features=F, out_features=D, score_function="sigmoid", normalize_weights=False,
+                          shared=F, scale_inputs=True)
+    got = layer.apply(variables, x).float().cpu().numpy()
+    want = tensors["output"]
+    assert not got[:, 32:].any()
+    scale = np.abs(want).max()
+    assert np.abs(got[:, :32] - want).max() <= 2e-2 * scale
+    other = dataclasses.replace(layer, scale_inputs=False).apply(variables, x).float().cpu().numpy()
+    assert np.abs(other[:, :32] - want).max() > 4 * np.abs(got[:, :32] - want).max()
+
+    # a seeded layer at kernel sizes against the oracle: the same routing, rows scaled in bf16, unweighted sum
+    case = CASES["c4-reduced"].scaled(tokens=200, shared=False)
+    data = inputs(case, seed=8)
+    layer, variables = layer_and_variables(case, data)
+    layer = dataclasses.replace(layer, scale_inputs=True)
+    got = layer.apply(variables, data["x"].cuda(), logits=data["logits"].cuda()).float().cpu().numpy()
+    mats, factors = zip(*(dequantized(data["banks"][name]) for name in ("gate", "up", "down")), strict=True)
+    want, _ = oracle.sparse_mlp(data["x"].float().numpy(), data["logits"].numpy(), *mats, top_k_count=case.top_k, factors=factors,
+                                bias=data["bias"].numpy(), scale_inputs=True, **case.router)
+    by_max, by_element = oracle.relative_errors(got, want)
+    assert by_max <= 6e-3 and by_element <= TOLERANCE, (by_max, by_element)
+    assert (got == want).mean() > 0.95

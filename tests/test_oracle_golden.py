@@ -81,6 +81,24 @@ def test_fp32_experts_reproduce_the_deepseek_v4_clamped_output():
     assert np.abs(unclamped - tensors["experts_output"]).max() > 1.0
 
 
+def test_fp32_block_reproduces_llama_4s_input_scaled_experts():
+    """`Llama4TextMoe` (tests/fixtures/llama4/moe.npz, the reference's own check tests/test_llama4.py:162-191): the
+    sigmoid of the top-2 logits scales each token's input to its experts, the outputs are summed unweighted, the shared
+    expert adds. Tolerance 1e-5 as there; weighting the outputs instead misses by more than 1e-3."""
+    tensors = golden("llama4/moe.npz")
+    hidden = tensors["hidden"].reshape(-1, tensors["hidden"].shape[-1])
+    gate_up = tensors["feed_forward.experts.gate_up_proj"]
+    width = gate_up.shape[-1] // 2
+    mats = [gate_up[..., :width], gate_up[..., width:], tensors["feed_forward.experts.down_proj"]]
+    shared = [tensors[f"feed_forward.shared_expert.{name}.weight"].T for name in ("gate_proj", "up_proj", "down_proj")]
+    logits = oracle.router_logits(hidden, tensors["feed_forward.router.weight"].T)
+    settings = dict(top_k_count=2, dtype="float32", shared=shared, score_function="sigmoid", normalize_weights=False)
+    out, _ = oracle.sparse_mlp(hidden, logits, *mats, scale_inputs=True, **settings)
+    assert np.abs(out - tensors["output"]).max() < 1e-5
+    other, _ = oracle.sparse_mlp(hidden, logits, *mats, scale_inputs=False, **settings)
+    assert np.abs(other - tensors["output"]).max() > 1e-3
+
+
 def test_top_k_takes_the_lower_index_on_ties_in_descending_order():
     values = np.array([[1.0, 3.0, 3.0, -np.inf, 2.0, 3.0]], np.float32)
     got_values, got = oracle.top_k(values, 4)
