@@ -119,7 +119,10 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const bf16_t* __restrict__ 
         gi = fminf(gi, limit);
         ui = fminf(fmaxf(ui, -limit), limit);
       }
-      h.v[i] = activation == DEW_MOE_GATE_GELU_TANH ? geglu_rounded(gi, ui) : swiglu_rounded(gi, ui);
+      if (activation == DEW_MOE_ACT_RELU2)
+        h.v[i] = f32_to_bf16(fmaxf(gi, 0.0f) * fmaxf(gi, 0.0f));  // (the square of a bf16 value, rounded once)
+      else
+        h.v[i] = activation == DEW_MOE_GATE_GELU_TANH ? geglu_rounded(gi, ui) : swiglu_rounded(gi, ui);
     }
     reinterpret_cast<Bf16x8*>(hidden)[item] = h;
   }
@@ -182,6 +185,18 @@ extern "C" int dew_moe_silu(const void* x, void* out, int64_t count, void* strea
   const int blocks = static_cast<int>(min((chunks + 255) / 256, 256ll * 64));
   hipLaunchKernelGGL(swiglu_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<const bf16_t*>(x),
                      static_cast<const bf16_t*>(nullptr), static_cast<bf16_t*>(out), chunks, 0.0f, DEW_MOE_GATE_SILU);
+  return launched("swiglu_kernel");
+}
+
+extern "C" int dew_moe_relu2(const void* x, void* out, int64_t count, void* stream) {
+  using namespace dew;
+  DEW_REQUIRE(count >= 0 && count % 8 == 0, "dew_moe_relu2: count %lld is not a multiple of 8", static_cast<long long>(count));
+  if (count == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(x && out && aligned16(x) && aligned16(out), "dew_moe_relu2: x and out must not be null and must be 16-byte aligned");
+  const long long chunks = count / 8;
+  const int blocks = static_cast<int>(min((chunks + 255) / 256, 256ll * 64));
+  hipLaunchKernelGGL(swiglu_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<const bf16_t*>(x),
+                     static_cast<const bf16_t*>(nullptr), static_cast<bf16_t*>(out), chunks, 0.0f, DEW_MOE_ACT_RELU2);
   return launched("swiglu_kernel");
 }
 

@@ -258,20 +258,27 @@ class ExpertMLP(_Module):
     product (the reference's arrangement); the results are bit-identical."""
 
     def __post_init__(self):
-        if self.activation not in ops.GATES:
-            raise ValueError(f"activation {self.activation!r}: the HIP experts gate by one of {list(ops.GATES)}")
+        if self.activation not in ops.GATES and self.activation != "relu2":
+            raise ValueError(f"activation {self.activation!r}: the HIP experts gate by one of {list(ops.GATES)}, or are ungated 'relu2' ones")
+        if self.activation == "relu2" and self.swiglu_limit is not None:
+            raise ValueError("swiglu_limit clamps a gate; relu2 experts have none")
         if self.dispatch not in ("auto", "global"):
             raise ValueError(f"dispatch {self.dispatch!r}: one device sorts its slots locally ('global')")
 
     def model_flops(self, rows: int) -> float:
-        """Three projections per dispatched row (src/dew/nn/moe.py:1275-1281)."""
-        return 3 * 2.0 * rows * self.out_features * self.hidden_features
+        """Three projections per dispatched row, two for the ungated relu2 experts (src/dew/nn/moe.py:1275-1281)."""
+        return (2 if self.activation == "relu2" else 3) * 2.0 * rows * self.out_features * self.hidden_features
 
     def kernels(self):
-        return tuple(expert_matrix(self.variables, (*self.path, name)) for name in EXPERT_AXES)
+        names = ("up_proj", "down_proj") if self.activation == "relu2" else EXPERT_AXES
+        return tuple(expert_matrix(self.variables, (*self.path, name)) for name in names)
 
     def _project(self, tokens: Gathered, sizes: GroupSizes, kernels) -> torch.Tensor:
         """src/dew/nn/moe.py:1305-1326."""
+        if self.activation == "relu2":  # Nemotron-H's ungated expert: up_proj, squared ReLU, down_proj (:1319-1322)
+            up_w, down_w = kernels
+            up = expert_projection(tokens, up_w, sizes, self.dtype, self.implementation, self.precision)
+            return expert_projection(ops.relu2(up), down_w, sizes, self.dtype, self.implementation, self.precision, scatter=tokens.slots)
         gate_w, up_w, down_w = kernels
         # The clamp (`swiglu_clamped`, src/dew/nn/activations.py:327-333: between the paired product and the gating) and a
         # GeGLU gate (Gemma's experts) are the paired launch's epilogue, like the plain SwiGLU product.

@@ -441,6 +441,14 @@ def silu(x: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def relu2(x: torch.Tensor) -> torch.Tensor:
+    """`bf16(max(x, 0)^2)`: the squared ReLU of Nemotron-H's ungated experts (the reference's `relu2`)."""
+    _device(x, "x", torch.bfloat16)
+    out = torch.empty_like(x)
+    _lib.check(_lib.library().dew_moe_relu2(_ptr(x), _ptr(out), x.numel(), _stream()), "dew_moe_relu2")
+    return out
+
+
 def combine(slots: torch.Tensor, weights: torch.Tensor, addend: torch.Tensor | None = None) -> torch.Tensor:
     """`out[t] = bf16(sum_j f32(slots[t, j]) * weights[t, j])` (+ the shared expert's `addend`)."""
     _device(slots, "slots", torch.bfloat16), _device(weights, "weights", torch.float32)

@@ -424,7 +424,7 @@ int dew_moe_swiglu_clamped(const void* gate, const void* up, float limit, void* 
  * 336-356): DEW_MOE_GATE_SILU is dew_moe_swiglu_clamped; DEW_MOE_GATE_GELU_TANH is 'geglu', the tanh GELU in its logistic
  * form g * logistic(sqrt(8 / pi) (g + 0.044715 g^3)) (`gelu_tanh`, :57-69: Gemma's experts, src/dew/nn/gemma4_moe.py:84),
  * with the same two roundings and the same optional clamp.                                                           */
-enum { DEW_MOE_GATE_SILU = 0, DEW_MOE_GATE_GELU_TANH = 1 };
+enum { DEW_MOE_GATE_SILU = 0, DEW_MOE_GATE_GELU_TANH = 1, DEW_MOE_ACT_RELU2 = 2 /* dew_moe_relu2's own: no gate */ };
 int dew_moe_gated_product(const void* gate, const void* up, int32_t activation, float limit, void* hidden, int64_t count, void* stream);
 /* dew_moe_gateup_swiglu with that gating as the paired launch's epilogue: hidden = gated_product(activation) of the two
  * products, clamped by `limit` first where that is positive, bit for bit dew_moe_gated_product over the two products of
@@ -440,6 +440,9 @@ int dew_moe_gateup_gated(const void* x, const int32_t* gather, const int32_t* of
  * gather and the combine sums the slots unweighted (weights of one).                                              */
 int dew_moe_scale_rows(const void* x /* bf16 [T,D] */, const int32_t* gather, const int32_t* slots, const float* weights,
                        void* out /* bf16 [rows,D] */, int32_t rows, int32_t depth, void* stream);
+/* Nemotron-H's ungated experts (`activation='relu2'`, src/dew/nn/moe.py:1250-1252, 1319-1322: up_proj, squared ReLU,
+ * down_proj): out = bf16(max(x, 0)^2) (`relu2`, src/dew/nn/activations.py:109-111), between two dew_moe_grouped_gemm launches. */
+int dew_moe_relu2(const void* x /* bf16 [count] */, void* out /* bf16 [count] */, int64_t count, void* stream);
 /* The activation alone: out = bf16(x * logistic(x)), formed in fp32 and rounded once (`silu`, src/dew/nn/activations.py:100-106),
  * which routed value experts pass each chosen projection through (src/dew/nn/value_experts.py:79-82).      */
 int dew_moe_silu(const void* x /* bf16 [count] */, void* out /* bf16 [count] */, int64_t count, void* stream);

@@ -18,6 +18,9 @@ What pins each function (tests/test_oracle_golden.py):
   src/dew/algebra/bits.py:696-705 checked against each other on every basis word and random words; staged
   order known answers of tests/test_gemm_nvfp4.py:37-38; form digest 7fb7f1b609cea47a.
 * `combine`: known answer of tests/test_moe_precision.py:652-674 (weights 1/2 +- 2^-11 give 2^-10).
+* `relu2` / `expert_mlp(activation='relu2')` (Nemotron-H's ungated experts): that same known answer is stated on a relu2
+  layer (up = 1, relu2(1) = 1, down = +-1), which the two-projection path reproduces; the activation itself is the closed
+  form max(x, 0)^2 with one rounding, checked on every bf16.
 * `expert_mlp(scale_inputs=True)` / `sparse_mlp(scale_inputs=True)` (Llama 4's input-scaled experts, fp32 mode): `output`
   of tests/fixtures/llama4/moe.npz (sigmoid of the top-2 logits on each token's input, the shared expert added) at the
   reference's own tolerance 1e-5 (tests/test_llama4.py:162-191); weighting the outputs instead must miss it by > 1e-3.
@@ -947,6 +950,13 @@ def capacity_admitted(indices, num_experts, capacity_factor):
     return admitted.reshape(indices.shape).astype(np.int32), capacity
 
 
+def relu2(x, *, dtype="bfloat16"):
+    """`relu2` (src/dew/nn/activations.py:109-111): the square of the ReLU, computed in the compute dtype: one rounding."""
+    x = np.asarray(x, F32)
+    squared = (np.maximum(x, F32(0)) ** 2).astype(F32)
+    return bf16_round(squared) if dtype == "bfloat16" else squared
+
+
 def expert_mlp(x, weights, indices, gate_w, up_w, down_w, *, dtype="bfloat16", factors=(None, None, None),
                limit=None, capacity_factor=None, activation="swiglu", scale_inputs=False):
     """`ExpertMLP.__call__` (src/dew/nn/moe.py:1335-1353) on one device: sort, gather, paired gate/up
@@ -955,7 +965,7 @@ def expert_mlp(x, weights, indices, gate_w, up_w, down_w, *, dtype="bfloat16", f
     sequence whose experts' queues drop their slots past the capacity: a dropped slot's row is zero). Returns
     (out [T, D], trace dict of the intermediates)."""
     x = np.asarray(x, F32)
-    experts = gate_w.shape[0]
+    experts = up_w.shape[0]
     if capacity_factor is not None:
         indices, _ = capacity_admitted(indices, experts, capacity_factor)
     indices = np.asarray(indices).reshape(-1, np.asarray(indices).shape[-1])
@@ -968,9 +978,12 @@ def expert_mlp(x, weights, indices, gate_w, up_w, down_w, *, dtype="bfloat16", f
         # row times its weight, both in the compute dtype, one rounding; the outputs are then summed unweighted (:1328-1330)
         scale = weights.reshape(-1)[plan["order"]][:, None]
         rows = bf16_round(bf16_round(rows) * bf16_round(scale)) if dtype == "bfloat16" else (rows * scale.astype(F32)).astype(F32)
-    gate = grouped_matmul(rows, gate_w, plan["sizes"], dtype=dtype, factor=factors[0])
     up = grouped_matmul(rows, up_w, plan["sizes"], dtype=dtype, factor=factors[1])
-    hidden = GATED_PRODUCTS[activation](gate, up, dtype=dtype, limit=limit)
+    if activation == "relu2":   # Nemotron-H's ungated experts: up_proj, squared ReLU, down_proj (src/dew/nn/moe.py:1319-1322); `gate_w` is None
+        gate, hidden = None, relu2(up, dtype=dtype)
+    else:
+        gate = grouped_matmul(rows, gate_w, plan["sizes"], dtype=dtype, factor=factors[0])
+        hidden = GATED_PRODUCTS[activation](gate, up, dtype=dtype, limit=limit)
     projected = grouped_matmul(hidden, down_w, plan["sizes"], dtype=dtype, factor=factors[2])
     slots = np.zeros_like(projected)
     slots[plan["order"]] = projected

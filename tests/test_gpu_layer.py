@@ -431,3 +431,50 @@ def test_llama_4s_input_scaled_experts_on_the_references_fixture_and_a_seeded_la
     by_max, by_element = oracle.relative_errors(got, want)
     assert by_max <= 6e-3 and by_element <= TOLERANCE, (by_max, by_element)
     assert (got == want).mean() > 0.95
+
+
+def test_nemotron_hs_ungated_relu2_experts():
+    """`activation='relu2'` (src/dew/nn/moe.py:1250-1252, 1319-1322): up_proj, squared ReLU, down_proj. The
+    reference's known answer (tests/test_moe_precision.py:652-674: experts answering 1 and -1 under weights 1/2 +- 2^-11
+    give 2^-10), padded with zeros to the launches' extents; the activation on every bf16; a seeded layer of FP8 banks
+    against the oracle."""
+    from dew_amd import formats, moe, ops
+
+    def one_hot(values):   # [E, 128, 128] bf16 banks whose [e, 0, 0] entries are `values`
+        bank = torch.zeros((len(values), 128, 128), dtype=torch.bfloat16)
+        bank[:, 0, 0] = torch.tensor(values, dtype=torch.bfloat16)
+        return {"kernel": formats.Bf16(bank).to("cuda")}
+
+    variables = {"params": {}, "quantization": {"up_proj": one_hot([1.0, 1.0]), "down_proj": one_hot([1.0, -1.0])}}
+    x = torch.zeros((1, 128), dtype=torch.bfloat16)
+    x[0, 0] = 1.0
+    weights = torch.tensor([[0.5 + 2.0 ** -11, 0.5 - 2.0 ** -11]], dtype=torch.float32).cuda()
+    indices = torch.tensor([[0, 1]], dtype=torch.int32).cuda()
+    out = moe.ExpertMLP(2, 128, 128, activation="relu2").apply(variables, x.cuda(), weights, indices)
+    assert out.dtype == torch.bfloat16 and float(out[0, 0]) == 2.0 ** -10 and not bool(out[0, 1:].any())
+
+    every = (torch.arange(1 << 16, dtype=torch.int32) << 16).view(torch.float32)
+    every = every[torch.isfinite(every)].to(torch.bfloat16)
+    every = every[: every.numel() // 8 * 8]
+    got = ops.relu2(every.cuda()).float().cpu().numpy()
+    want = oracle.relu2(every.float().numpy())
+    finite = np.isfinite(want)
+    assert np.array_equal(got[finite], want[finite]) and np.all(np.isinf(got[~finite]))
+
+    rng = np.random.default_rng(21)
+    tokens, experts, top_k, width, hidden = 300, 8, 2, 256, 512
+    from moe_cases import quantize
+    xs = torch.from_numpy(rng.standard_normal((tokens, width)).astype(np.float32)).to(torch.bfloat16)
+    banks = {name: quantize(torch.from_numpy((rng.standard_normal((experts, d, w)) * 0.08).astype(np.float32)), "fp8_block")
+             for name, (d, w) in (("up", (width, hidden)), ("down", (hidden, width)))}
+    logits = rng.standard_normal((tokens, experts)).astype(np.float32)
+    weights, indices = ops.route(torch.from_numpy(logits).cuda(), top_k)
+    variables = {"params": {}, "quantization": {f"{n}_proj": {"kernel": bank.to("cuda")} for n, bank in banks.items()}}
+    got = moe.ExpertMLP(experts, hidden, width, activation="relu2").apply(variables, xs.cuda(), weights, indices).float().cpu().numpy()
+    (up_values, _), (down_values, _) = dequantized(banks["up"]), dequantized(banks["down"])
+    want, _ = oracle.expert_mlp(xs.float().numpy(), weights.cpu().numpy(), indices.cpu().numpy(), None, up_values, down_values, activation="relu2")
+    by_max, by_element = oracle.relative_errors(got, want)
+    assert by_max <= 6e-3 and by_element <= TOLERANCE, (by_max, by_element)
+    assert (got == want).mean() > 0.97
+    with pytest.raises(ValueError, match="relu2 experts have none"):
+        moe.ExpertMLP(experts, hidden, width, activation="relu2", swiglu_limit=1.0)

@@ -99,6 +99,23 @@ def test_fp32_block_reproduces_llama_4s_input_scaled_experts():
     assert np.abs(other - tensors["output"]).max() > 1e-3
 
 
+def test_relu2_experts_reproduce_the_references_known_answer():
+    """tests/test_moe_precision.py:652-674 is stated on an ungated relu2 layer: two experts answer 1 and -1 (up = 1,
+    relu2(1) = 1, down = +-1), weighted 1/2 +- 2^-11: the bf16 output is 2^-10. And the activation on every bf16."""
+    x = np.ones((1, 1), np.float32)
+    weights = np.array([[0.5 + 2.0 ** -11, 0.5 - 2.0 ** -11]], np.float32)
+    indices = np.array([[0, 1]], np.int32)
+    up, down = np.ones((2, 1, 1), np.float32), np.array([[[1.0]], [[-1.0]]], np.float32)
+    out, _ = oracle.expert_mlp(x, weights, indices, None, up, down, activation="relu2")
+    assert out.shape == (1, 1) and out[0, 0] == 2.0 ** -10
+    every = (np.arange(1 << 16, dtype=np.uint32) << 16).view(np.float32)
+    every = every[np.isfinite(every)]
+    got = oracle.relu2(every)
+    truth = np.where(every > 0, every.astype(np.float64) ** 2, 0.0)
+    finite = truth < 3.3e38
+    assert np.array_equal(got[finite], oracle.bf16_round(truth[finite].astype(np.float32))) and not got[every < 0].any()
+
+
 def test_top_k_takes_the_lower_index_on_ties_in_descending_order():
     values = np.array([[1.0, 3.0, 3.0, -np.inf, 2.0, 3.0]], np.float32)
     got_values, got = oracle.top_k(values, 4)
