@@ -38,7 +38,9 @@ class Router(ctypes.Structure):
 
     _fields_ = [("experts", ctypes.c_int32), ("top_k", ctypes.c_int32), ("score_function", ctypes.c_int32),
                 ("normalize", ctypes.c_int32), ("scaling", ctypes.c_float), ("expert_groups", ctypes.c_int32),
-                ("groups_per_token", ctypes.c_int32), ("group_score", ctypes.c_int32)]
+                ("groups_per_token", ctypes.c_int32), ("group_score", ctypes.c_int32),
+                ("bias_in_weights", ctypes.c_int32), ("weight_sum_epsilon", ctypes.c_float), ("weight_sum_min", ctypes.c_float),
+                ("fill_excluded", ctypes.c_int32), ("excluded_group_score", ctypes.c_float), ("logit_softcap", ctypes.c_float)]
 
 
 class KernelError(RuntimeError):

@@ -109,7 +109,15 @@ struct RouteParams {
   float scaling;
   float* scores;  // nullable [T, E]: the activated scores, as the router sows them for the balance statistics
   float* log_z;   // nullable [T]: logsumexp of the logits (the z-loss's log partition)
+  int bias_in_weights;   // the weights are the chosen scores + bias
+  float sum_epsilon, sum_min;
+  int fill_excluded;     // an expert outside the kept groups competes at `excluded` rather than -inf
+  float excluded;
+  float softcap;         // above 0: every logit is read as softcap * tanh(logit / softcap)
 };
+
+// Laguna's capped gate logit (`capped_logits`, src/dew/nn/precision.py:2086-2092): cap * tanh(logit / cap) in fp32.
+__device__ __forceinline__ float capped(float logit, float cap) { return cap > 0.0f ? cap * tanhf(logit / cap) : logit; }
 
 template <int kPerLane>  // experts <= 64 * kPerLane
 __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p) {
@@ -126,7 +134,7 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
 #pragma unroll
   for (int i = 0; i < kPerLane; ++i) {
     const int e = lane + kWave * i;
-    logit[i] = e < p.experts ? row[e] : ninf;
+    logit[i] = e < p.experts ? capped(row[e], p.softcap) : ninf;
   }
 
   float top = ninf, denom = 1.0f;
@@ -225,7 +233,7 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
 #pragma unroll
     for (int i = 0; i < kPerLane; ++i) {
       const int e = lane + kWave * i;
-      if (e < p.experts && !((kept >> (e / per_group)) & 1ull)) select[i] = ninf;
+      if (e < p.experts && !((kept >> (e / per_group)) & 1ull)) select[i] = p.fill_excluded ? p.excluded : ninf;
     }
   }
 
@@ -251,9 +259,9 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
 
   // gate weights: lane j < k owns the j-th choice
   const bool owner = lane < p.top_k;
-  const float chosen_logit = owner ? row[my_choice] : ninf;
+  const float chosen_logit = owner ? capped(row[my_choice], p.softcap) : ninf;
   float weight = 0.0f;
-  if (p.score_function == DEW_MOE_SCORE_SOFTMAX && p.normalize) {
+  if (p.score_function == DEW_MOE_SCORE_SOFTMAX && p.normalize && !p.bias_in_weights && !(p.sum_min != 0.0f)) {
     const float m = wave_max(chosen_logit);
     const float shifted = owner ? exp_f32(chosen_logit - m) : 0.0f;
     const float total = wave_sum_once(static_cast<double>(shifted));
@@ -262,11 +270,13 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
     if (owner) {
       weight = p.score_function == DEW_MOE_SCORE_SOFTMAX ? exp_f32(chosen_logit - top) / denom
                                                          : pointwise_score(p.score_function, chosen_logit);
+      if (p.bias_in_weights) weight = weight + p.bias[my_choice];
     }
     if (p.normalize) {
       float total = __shfl(weight, 0, kWave);
       for (int j = 1; j < p.top_k; ++j) total = total + __shfl(weight, j, kWave);
-      total = total + 1e-20f;
+      total = total + p.sum_epsilon;
+      if (p.sum_min != 0.0f) total = fmaxf(total, p.sum_min);
       weight = weight / total;
     }
   }
@@ -292,7 +302,7 @@ extern "C" int dew_moe_route_sown(const float* logits, const float* bias, int32_
                                   int32_t expert_groups, int32_t groups_per_token, float* weights,
                                   int32_t* indices, float* scores, float* log_z, void* stream) {
   const dew_moe_router router{experts, top_k, score_function, normalize, scaling, expert_groups, groups_per_token,
-                              DEW_MOE_GROUP_TOP2};
+                              DEW_MOE_GROUP_TOP2, 0, DEW_MOE_WEIGHT_SUM_EPSILON, 0.0f, 0, 0.0f, 0.0f};
   return dew_moe_route_with(&router, logits, bias, tokens, weights, indices, scores, log_z, stream);
 }
 
@@ -323,9 +333,17 @@ extern "C" int dew_moe_route_with(const dew_moe_router* router, const float* log
                 "dew_moe_route: top_k %d exceeds the %d experts of the kept groups", top_k,
                 groups_per_token * (experts / expert_groups));
   }
+  DEW_REQUIRE(!router->bias_in_weights || bias, "dew_moe_route: bias_in_weights gates on the balancing bias, which is null");
+  DEW_REQUIRE(router->weight_sum_epsilon >= 0.0f && router->weight_sum_min >= 0.0f,
+              "dew_moe_route: weight_sum_epsilon %g and weight_sum_min %g bound a sum from below: neither is negative",
+              static_cast<double>(router->weight_sum_epsilon), static_cast<double>(router->weight_sum_min));
+  DEW_REQUIRE(router->logit_softcap >= 0.0f, "dew_moe_route: logit_softcap %g is a positive cap, or 0 for none",
+              static_cast<double>(router->logit_softcap));
   if (tokens == 0) return DEW_MOE_OK;
   RouteParams p{logits, bias, weights, indices, tokens, experts, top_k, score_function, router->normalize ? 1 : 0,
-                expert_groups, groups_per_token, router->group_score == DEW_MOE_GROUP_MAX ? 1 : 0, router->scaling, scores, log_z};
+                expert_groups, groups_per_token, router->group_score == DEW_MOE_GROUP_MAX ? 1 : 0, router->scaling, scores, log_z,
+                router->bias_in_weights ? 1 : 0, router->weight_sum_epsilon, router->weight_sum_min,
+                router->fill_excluded ? 1 : 0, router->excluded_group_score, router->logit_softcap};
   const int blocks = (tokens + kRouteWaves - 1) / kRouteWaves;
   const size_t shared = expert_groups > 1 ? sizeof(float) * kRouteWaves * experts : 0;
   const dim3 grid(blocks), block(kWave * kRouteWaves);

@@ -76,7 +76,8 @@ ffi::Error Route(hipStream_t stream, ffi::AnyBuffer logits, ffi::AnyBuffer bias,
       (bias.element_count() != 0 && static_cast<int64_t>(bias.element_count()) != experts))
     return misshaped(kTarget, "the extents of logits, bias, weights and indices do not agree");
   const dew_moe_router router{static_cast<int32_t>(experts), static_cast<int32_t>(top_k), score_function, normalize ? 1 : 0,
-                              scaling, expert_groups, groups_per_token, group_score};
+                              scaling, expert_groups, groups_per_token, group_score,
+                              /* the switches this target leaves at the router's defaults */ 0, DEW_MOE_WEIGHT_SUM_EPSILON, 0.0f, 0, 0.0f, 0.0f};
   if (dew_moe_route_with(&router, static_cast<const float*>(logits.untyped_data()), present<const float*>(bias),
                          static_cast<int32_t>(tokens), static_cast<float*>(weights->untyped_data()),
                          static_cast<int32_t*>(indices->untyped_data()), nullptr, nullptr, stream))

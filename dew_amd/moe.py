@@ -152,8 +152,22 @@ class Router(_Module):
     groups_per_token: int = 1
     group_score: str = "top2"
     expert_bias: bool = False
+    bias_in_weights: bool = False
+    """LLaDA-MoE's reading of the balancing bias: the biased scores are also the weights."""
+    weight_sum_epsilon: float = ops.WEIGHT_SUM_EPSILON
+    weight_sum_min: float = 0.0
+    """ERNIE 4.5's `moe_norm_min`: above 0, the chosen weights divide by `max(sum + weight_sum_epsilon, weight_sum_min)`,
+    a softmax's too."""
+    excluded_group_score: float | None = None
+    """What an expert outside a token's best groups is chosen by: None for never (DeepSeek V3's -inf), or A.X-K2's 0.0."""
+    logit_softcap: float | None = None
+    """Laguna's cap `c` on each gate logit, `c * tanh(logit / c)`, before the scores and the z-loss read it."""
 
     def __post_init__(self):
+        if self.bias_in_weights and not self.expert_bias:
+            raise ValueError("bias_in_weights gates on the balancing bias, which expert_bias holds")
+        if self.logit_softcap is not None and not self.logit_softcap > 0:
+            raise ValueError(f"logit_softcap is a positive cap on the gate logits, or None for none; got {self.logit_softcap}")
         if self.score_function not in ("softmax", "sigmoid", "sqrtsoftplus"):
             raise ValueError(f"score_function {self.score_function!r}: the router scores by 'softmax', 'sigmoid' or 'sqrtsoftplus'")
         if self.group_score not in ("top2", "max"):
@@ -177,7 +191,10 @@ class Router(_Module):
         found = ops.route(logits, self.top_k, score_function=self.score_function,
                           normalize_weights=self.normalize_weights, bias=bias,
                           routed_scaling_factor=self.routed_scaling_factor, expert_groups=self.expert_groups,
-                          groups_per_token=self.groups_per_token, group_score=self.group_score, sown=sown is not None)
+                          groups_per_token=self.groups_per_token, group_score=self.group_score, sown=sown is not None,
+                          bias_in_weights=self.bias_in_weights, weight_sum_epsilon=self.weight_sum_epsilon,
+                          weight_sum_min=self.weight_sum_min, excluded_group_score=self.excluded_group_score,
+                          logit_softcap=self.logit_softcap)
         if sown is not None:
             sown.update(indices=found[1], scores=found[2], log_z=found[3])
         return found[0], found[1]
@@ -385,12 +402,20 @@ class SparseMLP(_Module):
     scale_inputs: bool = False
     """Llama 4's placement of the routing weight on each expert's input, the outputs summed unweighted
     (src/dew/nn/moe.py:1256-1259, 1397)."""
+    bias_in_weights: bool = False
+    weight_sum_epsilon: float = ops.WEIGHT_SUM_EPSILON
+    weight_sum_min: float = 0.0
+    excluded_group_score: float | None = None
+    router_softcap: float | None = None
+    """The router's switches (`Router`'s fields of the same names; `router_softcap` is its `logit_softcap`,
+    src/dew/nn/moe.py:1440-1446)."""
 
     @property
     def gate(self) -> Router:
         return Router(self.num_experts, self.out_features, self.top_k, self.score_function, self.normalize_weights,
                       self.routed_scaling_factor, self.expert_groups, self.groups_per_token, self.group_score,
-                      self.expert_bias)._bound(self.variables, (*self.path, "gate"))
+                      self.expert_bias, self.bias_in_weights, self.weight_sum_epsilon, self.weight_sum_min,
+                      self.excluded_group_score, self.router_softcap)._bound(self.variables, (*self.path, "gate"))
 
     @property
     def experts(self) -> ExpertMLP:

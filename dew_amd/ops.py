@@ -37,11 +37,18 @@ def device_check() -> None:
 # ---- router -------------------------------------------------------------------------------------------
 
 
+WEIGHT_SUM_EPSILON = 1e-20
+"""What a renormalization adds to the chosen weights' sum (`WEIGHT_SUM_EPSILON`, src/dew/nn/moe.py:181)."""
+
+
 def route(logits: torch.Tensor, top_k: int, *, score_function: str = "softmax", normalize_weights: bool = True,
           bias: torch.Tensor | None = None, routed_scaling_factor: float = 1.0, expert_groups: int = 1,
-          groups_per_token: int = 1, group_score: str = "top2", sown: bool = False):
+          groups_per_token: int = 1, group_score: str = "top2", sown: bool = False, bias_in_weights: bool = False,
+          weight_sum_epsilon: float = WEIGHT_SUM_EPSILON, weight_sum_min: float = 0.0, excluded_group_score: float | None = None,
+          logit_softcap: float | None = None):
     """(weights fp32 `[..., k]`, indices int32 `[..., k]`) of router `logits [..., E]` (fp32); with `sown`, also what
-    the router sows for the balance statistics: (weights, indices, scores fp32 `[..., E]`, log_z fp32 `[...]`)."""
+    the router sows for the balance statistics: (weights, indices, scores fp32 `[..., E]`, log_z fp32 `[...]`). The last
+    five switches are `Router`'s of the same names (src/dew/nn/moe.py:361-384)."""
     scores = {"softmax": _lib.SCORE_SOFTMAX, "sigmoid": _lib.SCORE_SIGMOID, "sqrtsoftplus": _lib.SCORE_SQRTSOFTPLUS}
     group_scores = {"top2": _lib.GROUP_TOP2, "max": _lib.GROUP_MAX}
     if score_function not in scores:
@@ -60,7 +67,9 @@ def route(logits: torch.Tensor, top_k: int, *, score_function: str = "softmax", 
     activated = torch.empty_like(logits) if sown else None
     log_z = torch.empty(logits.shape[:-1], dtype=torch.float32, device=logits.device) if sown else None
     router = _lib.Router(experts, top_k, scores[score_function], int(bool(normalize_weights)), float(routed_scaling_factor),
-                         expert_groups, groups_per_token, group_scores[group_score])
+                         expert_groups, groups_per_token, group_scores[group_score], int(bool(bias_in_weights)),
+                         float(weight_sum_epsilon), float(weight_sum_min), int(excluded_group_score is not None),
+                         float(excluded_group_score or 0.0), float(logit_softcap or 0.0))
     _lib.check(_lib.library().dew_moe_route_with(router, _ptr(logits), _ptr(bias), tokens, _ptr(weights), _ptr(indices),
                                                  _ptr(activated), _ptr(log_z), _stream()), "dew_moe_route")
     return (weights, indices, activated, log_z) if sown else (weights, indices)

@@ -81,7 +81,17 @@ typedef struct dew_moe_router {
   float scaling;           /* routed_scaling_factor                                        */
   int32_t expert_groups, groups_per_token;
   int32_t group_score;     /* DEW_MOE_GROUP_*                                              */
+  /* The switches below follow `Router`'s fields of the same names (src/dew/nn/moe.py:361-384, read at :483-494 and
+   * :510-513). All zero but weight_sum_epsilon = DEW_MOE_WEIGHT_SUM_EPSILON is the router the fields above describe. */
+  int32_t bias_in_weights;      /* LLaDA-MoE: the weights are the chosen scores + bias, not the chosen scores        */
+  float weight_sum_epsilon;     /* added to the chosen weights' sum before a renormalization divides by it           */
+  float weight_sum_min;         /* ERNIE 4.5's moe_norm_min: above 0, the least that sum (+ epsilon) divides by; a
+                                 * softmax router then renormalizes its chosen scores this way too                   */
+  int32_t fill_excluded;        /* whether excluded_group_score is set (else an excluded expert is never chosen)     */
+  float excluded_group_score;   /* A.X-K2's 0.0: what an expert outside a token's best groups is chosen by           */
+  float logit_softcap;          /* Laguna: above 0, every logit is read as cap * tanh(logit / cap); 0 for none       */
 } dew_moe_router;
+#define DEW_MOE_WEIGHT_SUM_EPSILON 1e-20f   /* WEIGHT_SUM_EPSILON, src/dew/nn/moe.py:181 */
 
 /* ---- introspection (kernels/cutlass/ffi.cu:133-176: dew_cutlass_kernels/kernel_fields/architecture) ---- */
 const char* dew_moe_last_error(void);   /* thread-local, valid until the thread's next failing call      */

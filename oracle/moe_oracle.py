@@ -39,6 +39,12 @@ What pins each function (tests/test_oracle_golden.py):
   float64 sum of the chosen experts' products on integer operands (where every fp32 sum is exact), which a wrong
   gather, scatter, weight pairing or a missing activation fails.
 
+* `route`'s further switches (`bias_in_weights`, `weight_sum_epsilon`, `weight_sum_min`, `excluded_group_score`,
+  `logit_softcap`; src/dew/nn/moe.py:361-384): the reference holds no vectors for them. `excluded_group_score` is pinned
+  by the reference's own case restated (tests/test_moe.py:265-292: which experts are chosen, filled at 0.0 and at -inf);
+  the others by their definitions in float64 (the biased scores gathered; the sums floored, with the tokens below the
+  floor summing to sum / floor and the rest to one; `cap * tanh(x / cap)`, bounded, order-preserving), each of which a
+  dropped bias, a floor applied before the epsilon or a cap applied after the scores fails.
 * `load_balance_update`: the known answer of tests/test_moe.py:326-336 (counts 3, 1, 0, 0 at rate 0.001).
 * `router_statistics`: closed forms (scores = exp(logits - log_z) for softmax; log_z(logits + c) = log_z + c; the
   z-loss's log partition against a float64 logsumexp).
@@ -322,9 +328,21 @@ def top_k(values, k):
     return np.take_along_axis(values, order, axis=-1), order.astype(np.int32)
 
 
-def selection_scores(logits, *, score_function="softmax", bias=None, expert_groups=1, groups_per_token=1, group_score="top2"):
+def capped_logits(logits, softcap):
+    """`capped_logits` (src/dew/nn/precision.py:2086-2092) as the router applies it (src/dew/nn/moe.py:526-534):
+    `cap * tanh(logits / cap)` in fp32, the logits themselves where there is no cap."""
+    logits = np.asarray(logits, F32)
+    if softcap is None:
+        return logits
+    cap = F32(softcap)
+    return (cap * np.tanh((logits / cap).astype(F32)).astype(F32)).astype(F32)
+
+
+def selection_scores(logits, *, score_function="softmax", bias=None, expert_groups=1, groups_per_token=1, group_score="top2",
+                     excluded_group_score=None):
     """(scores, selection) of `Router.__call__` (src/dew/nn/moe.py:466-470, 516-524): the activated scores and what the
-    top-k runs over, the scores plus the bias with the experts outside a token's best groups at -inf (:496-565)."""
+    top-k runs over, the scores plus the bias with the experts outside a token's best groups at -inf, or at
+    `excluded_group_score` where the router fills one in (:496-565)."""
     logits = np.asarray(logits, F32)
     experts = logits.shape[-1]
     if score_function == "softmax":
@@ -350,7 +368,8 @@ def selection_scores(logits, *, score_function="softmax", bias=None, expert_grou
         _, groups = top_k(group_scores, groups_per_token)
         kept = np.zeros(group_scores.shape, bool)
         np.put_along_axis(kept, groups, True, axis=-1)
-        selection = np.where(np.repeat(kept, per_group, axis=-1), selection, F32(-np.inf))
+        fill = F32(-np.inf) if excluded_group_score is None else F32(excluded_group_score)
+        selection = np.where(np.repeat(kept, per_group, axis=-1), selection, fill)
     return scores, selection
 
 
@@ -371,22 +390,30 @@ def top_k_margin(selection, top_k_count):
 
 def route(logits, top_k_count, *, score_function="softmax", normalize_weights=True, bias=None,
           routed_scaling_factor=1.0, expert_groups=1, groups_per_token=1, group_score="top2",
-          weight_sum_epsilon=1e-20):
-    """`Router.__call__` from its logits on (src/dew/nn/moe.py:466-494): scores, selection (bias,
-    group-limited mask :496-565), top-k, weights. Returns (weights fp32 [T, k], indices int32 [T, k])."""
-    logits = np.asarray(logits, F32)
+          weight_sum_epsilon=1e-20, weight_sum_min=0.0, bias_in_weights=False, excluded_group_score=None,
+          logit_softcap=None):
+    """`Router.__call__` from its logits on (src/dew/nn/moe.py:466-494): the cap on the logits (:526-534), scores,
+    selection (bias, group-limited mask :496-565), top-k, weights (:483-494: a softmax router renormalizes the chosen
+    logits unless `bias_in_weights` or `weight_sum_min` say otherwise; else the chosen scores, plus the bias under
+    `bias_in_weights`, over `max(sum + weight_sum_epsilon, weight_sum_min)`). Returns (weights fp32 [T, k], indices
+    int32 [T, k])."""
+    logits = capped_logits(logits, logit_softcap)
     scores, selection = selection_scores(logits, score_function=score_function, bias=bias, expert_groups=expert_groups,
-                                         groups_per_token=groups_per_token, group_score=group_score)
+                                         groups_per_token=groups_per_token, group_score=group_score,
+                                         excluded_group_score=excluded_group_score)
     _, indices = top_k(selection, top_k_count)
-    if normalize_weights and score_function == "softmax":
+    if normalize_weights and score_function == "softmax" and not bias_in_weights and not weight_sum_min:
         weights = expert_softmax(np.take_along_axis(logits, indices, axis=-1))        # moe.py:194-199,485
     else:
-        weights = np.take_along_axis(scores, indices, axis=-1)
+        gating = (scores + np.asarray(bias, F32)).astype(F32) if bias_in_weights else scores
+        weights = np.take_along_axis(gating, indices, axis=-1)
         if normalize_weights:
             total = weights[..., 0].copy()
             for j in range(1, top_k_count):
                 total = (total + weights[..., j]).astype(F32)
             total = (total + F32(weight_sum_epsilon)).astype(F32)
+            if weight_sum_min:
+                total = np.maximum(total, F32(weight_sum_min))
             weights = (weights / total[..., None]).astype(F32)
     return (weights * F32(routed_scaling_factor)).astype(F32), indices
 

@@ -46,6 +46,13 @@ ROUTERS = [
     ("sigmoid-64-top6-raw", 64, 6, dict(score_function="sigmoid", normalize_weights=False, routed_scaling_factor=1.5), True, 65),
     ("softmax-320-top4-groups", 320, 4, dict(score_function="softmax", normalize_weights=True, expert_groups=5,
                                              groups_per_token=2), False, 33),
+    ("sigmoid-64-top6-bias-in-weights", 64, 6, dict(score_function="sigmoid", normalize_weights=True, bias_in_weights=True), True, 200),
+    ("softmax-32-top4-bias-in-weights-raw", 32, 4, dict(score_function="softmax", normalize_weights=False, bias_in_weights=True,
+                                                        routed_scaling_factor=2.0), True, 100),
+    ("sigmoid-128-top8-sum-floor", 128, 8, dict(score_function="sigmoid", normalize_weights=True, weight_sum_min=7.5), False, 300),
+    ("softmax-64-top4-sum-floor-and-epsilon", 64, 4, dict(score_function="softmax", normalize_weights=True, weight_sum_min=0.5,
+                                                          weight_sum_epsilon=1e-6), False, 150),
+    ("sigmoid-256-top8-wide-epsilon", 256, 8, dict(score_function="sigmoid", normalize_weights=True, weight_sum_epsilon=0.25), True, 90),
 ]
 
 
@@ -62,6 +69,59 @@ def test_router_matches_the_oracle_bit_for_bit(ops, name, experts, k, settings, 
                              **settings)
     assert np.array_equal(got_i.cpu().numpy(), want_i)
     assert np.array_equal(got_w.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
+
+
+@pytest.mark.parametrize("fill", [0.0, 0.3, None])
+@pytest.mark.parametrize("experts,groups,kept,k,group_score", [(64, 8, 2, 8, "top2"), (256, 8, 1, 8, "top2"), (32, 4, 2, 6, "max")])
+def test_an_excluded_groups_experts_compete_at_the_score_filled_in(ops, experts, groups, kept, k, group_score, fill):
+    """A.X-K2's fill for the experts outside a token's best groups (`excluded_group_score`): under a bias that puts most
+    of the selections below the fill, those experts outrank the kept groups' weaker ones."""
+    rng = np.random.default_rng(experts + groups)
+    logits = (rng.standard_normal((333, experts)) * 2).astype(np.float32)
+    bias = (rng.standard_normal(experts) * 0.1 - 0.8).astype(np.float32)
+    settings = dict(score_function="sigmoid", normalize_weights=True, routed_scaling_factor=2.5, expert_groups=groups,
+                    groups_per_token=kept, group_score=group_score, excluded_group_score=fill)
+    want_w, want_i = oracle.route(logits, k, bias=bias, **settings)
+    got_w, got_i = ops.route(torch.from_numpy(logits).cuda(), k, bias=torch.from_numpy(bias).cuda(), **settings)
+    assert np.array_equal(got_i.cpu().numpy(), want_i)
+    assert np.array_equal(got_w.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
+    if fill is not None:    # the case means something: some chosen experts sit outside their token's kept groups
+        _, limited = oracle.route(logits, k, bias=bias, **{**settings, "excluded_group_score": None})
+        assert not np.array_equal(np.sort(limited, -1), np.sort(want_i, -1))
+
+
+@pytest.mark.parametrize("score_function,experts,k,cap", [("softmax", 64, 4, 30.0), ("sigmoid", 256, 8, 5.0), ("softmax", 128, 8, 2.0)])
+def test_a_logit_softcap_caps_what_every_reader_of_the_logits_reads(ops, score_function, experts, k, cap):
+    """`logit_softcap`: scores, choices, weights and the sown log partition all read `cap * tanh(logit / cap)`. The
+    hyperbolic tangent is the device library's and the oracle's NumPy's (the reference's is XLA's: no one's bits are
+    pinned), so the weights are compared at the reference's router tolerance, 1e-6, and the choices exactly wherever the
+    oracle's own margin between the last expert chosen and the first left out exceeds a few fp32 spacings."""
+    rng = np.random.default_rng(int(cap * 10) + experts)
+    logits = (rng.standard_normal((400, experts)) * 4).astype(np.float32)
+    settings = dict(score_function=score_function, normalize_weights=True, logit_softcap=cap)
+    want_w, want_i = oracle.route(logits, k, **settings)
+    got = ops.route(torch.from_numpy(logits).cuda(), k, sown=True, **settings)
+    got_w, got_i = got[0].cpu().numpy(), got[1].cpu().numpy()
+    _, selection = oracle.selection_scores(oracle.capped_logits(logits, cap), score_function=score_function)
+    ranked = -np.sort(-selection, axis=-1)
+    clear = (ranked[:, :-1] - ranked[:, 1:])[:, :k].min(-1) > 8 * np.spacing(np.abs(ranked[:, 0]))   # no two of the first k + 1 within a few spacings
+    assert clear.mean() > 0.9
+    assert np.array_equal(got_i[clear], want_i[clear])
+    assert np.abs(got_w[clear] - want_w[clear]).max() <= 1e-6
+    want_scores, want_log_z = oracle.router_statistics(oracle.capped_logits(logits, cap), score_function=score_function)
+    assert np.abs(got[2].cpu().numpy() - want_scores).max() <= 1e-6
+    assert np.abs(got[3].cpu().numpy() - want_log_z).max() <= 1e-5
+    assert np.abs(got[3].cpu().numpy()).max() <= cap + np.log(experts) + 1e-3
+
+
+def test_router_refuses_bounds_that_bound_nothing(ops):
+    logits = torch.zeros(4, 8, device="cuda")
+    with pytest.raises(ops.KernelError, match="bias_in_weights"):
+        ops.route(logits, 2, bias_in_weights=True)
+    with pytest.raises(ops.KernelError, match="weight_sum"):
+        ops.route(logits, 2, weight_sum_min=-1.0)
+    with pytest.raises(ops.KernelError, match="logit_softcap"):
+        ops.route(logits, 2, logit_softcap=-3.0)
 
 
 def test_a_nan_selection_bias_is_never_chosen_and_every_choice_stays_in_range(ops):

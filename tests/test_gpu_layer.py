@@ -478,3 +478,41 @@ def test_nemotron_hs_ungated_relu2_experts():
     assert (got == want).mean() > 0.97
     with pytest.raises(ValueError, match="relu2 experts have none"):
         moe.ExpertMLP(experts, hidden, width, activation="relu2", swiglu_limit=1.0)
+
+
+@pytest.mark.parametrize("switches", [dict(weight_sum_min=7.5), dict(bias_in_weights=True), dict(excluded_group_score=0.9),
+                                      dict(weight_sum_epsilon=0.5)],
+                         ids=["ernie-sum-floor", "llada-bias-in-weights", "filled-groups", "wide-epsilon"])
+def test_the_layer_hands_the_routers_further_switches_to_its_router(switches):
+    """ERNIE 4.5's floor under the chosen weights' sum, LLaDA-MoE's biased weights, a fill for excluded groups (A.X-K2's switch)
+    and a sum epsilon of the caller's (`SparseMLP`'s fields of src/dew/nn/moe.py:1391-1396): the whole layer against
+    the oracle under the same switches, the routing bit for bit."""
+    import dataclasses
+
+    case = CASES["c4-reduced"].scaled(tokens=160, shared=False)
+    data = inputs(case, seed=12)
+    layer, variables = layer_and_variables(case, data)
+    layer = dataclasses.replace(layer, **switches)
+    sown = {}
+    weights, indices = layer._bound(variables, ()).gate.routed(data["logits"].cuda(), sown)
+    want_w, want_i = oracle.route(data["logits"].numpy(), case.top_k, bias=data["bias"].numpy(), **case.router, **switches)
+    assert np.array_equal(indices.cpu().numpy(), want_i)
+    assert np.array_equal(weights.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
+    plain_w, plain_i = oracle.route(data["logits"].numpy(), case.top_k, bias=data["bias"].numpy(), **case.router)
+    assert not (np.array_equal(plain_w, want_w) and np.array_equal(plain_i, want_i))      # the switch switches something
+    got = layer.apply(variables, data["x"].cuda(), logits=data["logits"].cuda()).float().cpu().numpy()
+    mats, factors = zip(*(dequantized(data["banks"][name]) for name in ("gate", "up", "down")), strict=True)
+    want, _ = oracle.sparse_mlp(data["x"].float().numpy(), data["logits"].numpy(), *mats, top_k_count=case.top_k, factors=factors,
+                                bias=data["bias"].numpy(), **case.router, **switches)
+    by_max, by_element = oracle.relative_errors(got, want)
+    assert by_max <= 6e-3 and by_element <= TOLERANCE, (by_max, by_element)
+
+
+def test_the_layers_router_softcap_is_its_routers_logit_softcap():
+    from dew_amd import moe
+    layer = moe.SparseMLP(num_experts=8, top_k=2, hidden_features=128, out_features=128, router_softcap=30.0)
+    assert layer._bound({}, ()).gate.logit_softcap == 30.0
+    with pytest.raises(ValueError, match="positive cap"):
+        moe.Router(8, 128, 2, logit_softcap=0.0)
+    with pytest.raises(ValueError, match="expert_bias holds"):
+        moe.Router(8, 128, 2, bias_in_weights=True)

@@ -461,3 +461,82 @@ def test_geglu_is_the_tanh_gelu_with_the_two_roundings():
     assert oracle.geglu(np.float32([1.0]), np.float32([3.0]))[0] == np.float32(2.515625)
     assert abs(oracle.geglu(np.float32([1.0]), np.float32([3.0]), dtype="float32")[0] - 3 * 0.8411919906082768) < 1e-6
     assert oracle.geglu(np.float32([5.0]), np.float32([-9.0]), limit=2.0)[0] == oracle.geglu(np.float32([2.0]), np.float32([-2.0]))[0]
+
+
+# ---- the router's further switches (src/dew/nn/moe.py:361-384): each pinned by what its definition fixes ----
+
+
+@pytest.mark.parametrize("fill", [0.0, None], ids=["axk2-zero", "deepseek-inf"])
+def test_an_expert_outside_the_best_groups_is_chosen_by_the_score_filled_in(fill):
+    """The reference's own case (tests/test_moe.py:265-292): eight experts in four groups, two groups a token's best,
+    every selection below zero (sigmoid scores under a bias of -5). Filled at 0.0 the four experts outside those groups
+    outrank the groups' own and are the choice; at -inf they never are."""
+    rng = np.random.default_rng(0x3080)
+    logits = rng.standard_normal((6, 8)).astype(np.float32)
+    bias = np.full(8, -5.0, np.float32)
+    _, indices = oracle.route(logits, 4, score_function="sigmoid", bias=bias, expert_groups=4, groups_per_token=2,
+                              excluded_group_score=fill)
+    scores = 1.0 / (1.0 + np.exp(-logits.astype(np.float64))) - 5.0
+    pairs = scores.reshape(6, 4, 2)
+    best_groups = np.argsort(-pairs.sum(-1), axis=-1, kind="stable")[:, :2]          # two experts a group: top2 is the sum
+    for token in range(6):
+        inside = sorted(int(g) * 2 + j for g in best_groups[token] for j in range(2))
+        outside = sorted(set(range(8)) - set(inside))
+        assert sorted(indices[token].tolist()) == (outside if fill is not None else inside)
+
+
+def test_a_weight_sum_floor_divides_small_sums_by_itself_and_moves_a_softmax_to_its_scores():
+    rng = np.random.default_rng(11)
+    logits = (rng.standard_normal((50, 16)) * 2 - 3).astype(np.float32)        # sigmoid scores mostly small
+    plain, chosen = oracle.route(logits, 2, score_function="sigmoid", normalize_weights=False)
+    sums = plain.astype(np.float64).sum(-1)
+    floor = float(np.median(sums))
+    weights, indices = oracle.route(logits, 2, score_function="sigmoid", weight_sum_min=floor)
+    assert np.array_equal(indices, chosen)
+    truth = plain.astype(np.float64) / np.maximum(sums + 1e-20, floor)[:, None]
+    assert np.abs(weights - truth).max() <= ROUTER_TOLERANCE
+    small = sums < floor
+    assert small.any() and (~small).any()
+    assert np.abs(weights[small].astype(np.float64).sum(-1) - sums[small] / floor).max() <= ROUTER_TOLERANCE   # they sum to less than one
+    assert np.abs(weights[~small].astype(np.float64).sum(-1) - 1.0).max() <= ROUTER_TOLERANCE
+    # a softmax router under a floor gathers its scores and divides them (:483-494); a floor below every sum changes
+    # nothing but the roundings on the way
+    renormalized, _ = oracle.route(logits, 2)
+    floored, _ = oracle.route(logits, 2, weight_sum_min=1e-12)
+    assert np.abs(floored - renormalized).max() <= ROUTER_TOLERANCE
+    wide, _ = oracle.route(logits, 2, weight_sum_epsilon=1.0, score_function="sigmoid")
+    assert np.abs(wide - plain.astype(np.float64) / (sums + 1.0)[:, None]).max() <= ROUTER_TOLERANCE
+
+
+def test_bias_in_weights_makes_the_biased_scores_the_weights():
+    rng = np.random.default_rng(12)
+    logits = rng.standard_normal((30, 12)).astype(np.float32)
+    bias = (rng.standard_normal(12) * 0.3).astype(np.float32)
+    for normalize in (False, True):
+        weights, indices = oracle.route(logits, 3, bias=bias, bias_in_weights=True, normalize_weights=normalize)
+        wide = logits.astype(np.float64)
+        softmax = np.exp(wide - wide.max(-1, keepdims=True))
+        biased = softmax / softmax.sum(-1, keepdims=True) + bias
+        assert np.array_equal(indices, np.argsort(-biased, axis=-1, kind="stable")[:, :3])
+        truth = np.take_along_axis(biased, indices, -1)
+        if normalize:
+            truth = truth / (truth.sum(-1, keepdims=True) + 1e-20)
+        assert np.abs(weights - truth).max() <= ROUTER_TOLERANCE
+    unbiased_weights, _ = oracle.route(logits, 3, bias=bias, normalize_weights=False)
+    assert np.abs(unbiased_weights - (np.take_along_axis(biased, indices, -1) - bias[indices])).max() <= ROUTER_TOLERANCE
+
+
+def test_a_logit_softcap_bounds_the_logits_and_keeps_their_order():
+    rng = np.random.default_rng(13)
+    logits = (rng.standard_normal((40, 16)) * 20).astype(np.float32)
+    capped = oracle.capped_logits(logits, 30.0)
+    assert np.abs(capped).max() < 30.0
+    assert np.abs(capped - 30.0 * np.tanh(logits.astype(np.float64) / 30.0)).max() <= 4e-6
+    assert oracle.capped_logits(logits, None) is not None and np.array_equal(oracle.capped_logits(logits, None), logits)
+    # tanh is increasing: a softmax router without a bias chooses the same experts, by weights that are the capped logits'
+    weights, indices = oracle.route(logits, 4, logit_softcap=30.0)
+    assert np.array_equal(indices, oracle.route(logits, 4)[1])
+    assert np.array_equal(weights, oracle.route(capped, 4)[0])
+    chosen = np.take_along_axis(capped.astype(np.float64), indices, -1)
+    truth = np.exp(chosen - chosen.max(-1, keepdims=True))
+    assert np.abs(weights - truth / truth.sum(-1, keepdims=True)).max() <= ROUTER_TOLERANCE
