@@ -24,7 +24,11 @@ What pins each function (tests/test_oracle_golden.py):
 * `expert_mlp(scale_inputs=True)` / `sparse_mlp(scale_inputs=True)` (Llama 4's input-scaled experts, fp32 mode): `output`
   of tests/fixtures/llama4/moe.npz (sigmoid of the top-2 logits on each token's input, the shared expert added) at the
   reference's own tolerance 1e-5 (tests/test_llama4.py:162-191); weighting the outputs instead must miss it by > 1e-3.
-* `swiglu`: closed form, the two bf16 roundings checked on hand-computed cases.
+* `swiglu`: closed form, the two bf16 roundings checked on hand-computed cases; and every one of the 2048 outputs Torch
+  recorded for bf16 `silu(gate) * up` in the reference's tests/fixtures/gated_product/bf16.npz (`swiglu/output`, the
+  arm tests/test_causal_transformer.py:1290-1340 holds the reference's product to), bit for bit. `geglu` on the same
+  file's `geglu/output`: bit for bit wherever Torch's tanh has not saturated to -1 (there Torch records 0 and the
+  reference's logistic form leaves a product below 1e-16).
 * `gpt_oss_mlp` (fp32 mode): `output` of tests/fixtures/gpt_oss/moe.npz at the reference's own tolerance (1.6e-4,
   tests/test_gpt_oss.py:45-66): biased router, top-k on the logits, softmax of the chosen, interleaved gate/up
   with both biases, clamp 7, (up + 1) * gate * logistic(1.702 gate). Dropping the down bias must move it by > 0.5.

@@ -396,6 +396,26 @@ def test_geglu_kernel_matches_the_oracle_on_every_bf16_gate(ops):
         ops.gated_product(torch.zeros(8, dtype=torch.bfloat16, device="cuda"), torch.zeros(8, dtype=torch.bfloat16, device="cuda"), "reglu")
 
 
+def test_the_gating_kernels_reproduce_torchs_recorded_bf16_products(ops):
+    """The reference's tests/fixtures/gated_product/bf16.npz (Torch's bf16 `silu(gate) * up` and tanh-GELU product on 2048
+    drawn pairs, the arm the reference's own product is held to): SwiGLU bit for bit; GeGLU bit for bit but where the
+    hardware exponential moves a last bf16 bit, and where Torch's tanh has saturated (its 0 against a product below 1e-16)."""
+    from conftest import golden
+    held = golden("gated_product/bf16.npz")
+
+    def on_device(name):
+        return torch.from_numpy(held[name]).to(torch.bfloat16).cuda()
+
+    got = bf16_np(ops.gated_product(on_device("swiglu/gate"), on_device("swiglu/up"), "swiglu"))
+    assert np.array_equal(got, held["swiglu/output"])
+    got = bf16_np(ops.gated_product(on_device("geglu/gate"), on_device("geglu/up"), "geglu"))
+    want = held["geglu/output"]
+    differs = got != want
+    saturated = differs & (want == 0)
+    assert np.abs(got[saturated]).max(initial=0) < 1e-16
+    assert (differs & ~saturated).sum() <= 4 and np.all(np.abs(got - want)[differs & ~saturated] <= 2 ** -7 * np.abs(want[differs & ~saturated]))
+
+
 def test_combine_weighs_in_fp32_and_rounds_once(ops):
     slots = torch.tensor([[[1.0] * 8, [-1.0] * 8]], dtype=torch.bfloat16)     # tests/test_moe_precision.py:652-674
     weights = torch.tensor([[0.5 + 2 ** -11, 0.5 - 2 ** -11]], dtype=torch.float32)

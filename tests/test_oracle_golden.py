@@ -540,3 +540,19 @@ def test_a_logit_softcap_bounds_the_logits_and_keeps_their_order():
     chosen = np.take_along_axis(capped.astype(np.float64), indices, -1)
     truth = np.exp(chosen - chosen.max(-1, keepdims=True))
     assert np.abs(weights - truth / truth.sum(-1, keepdims=True)).max() <= ROUTER_TOLERANCE
+
+
+def test_the_gated_products_are_torchs_recorded_bf16_outputs():
+    """tests/fixtures/gated_product/bf16.npz of the reference: Torch's bf16 `silu(gate) * up` and tanh-`gelu(gate) * up`
+    on 2048 drawn bf16 pairs, the arm the reference's own gated product is held to
+    (tests/test_causal_transformer.py:1290-1340). The rounding after the activation and the one after the product are
+    Torch's bf16 arithmetic; dropping either moves hundreds of these outputs."""
+    held = golden("gated_product/bf16.npz")
+    gate, up, output = held["swiglu/gate"], held["swiglu/up"], held["swiglu/output"]
+    assert np.array_equal(oracle.swiglu(gate, up), output)
+    once = oracle.bf16_round(gate.astype(np.float64) / (1.0 + np.exp(-gate.astype(np.float64))) * up)   # one rounding only
+    assert (once != output).sum() > 100
+    gate, up, output = held["geglu/gate"], held["geglu/up"], held["geglu/output"]
+    got = oracle.geglu(gate, up)
+    differs = got != output
+    assert differs.sum() < 40 and np.all(output[differs] == 0) and np.abs(got[differs]).max() < 1e-16   # Torch's tanh at -1
