@@ -1,7 +1,8 @@
 """A quantized checkpoint's expert banks taken to the kernels' formats at load time, without decoding a value:
 the host-side mirror of the reference's `packed_banks` / `with_banks` (src/dew/interop/quantized_loads.py:106-168)
 for MXFP4 sources (gpt-oss's `*_blocks` / `*_scales`), and the same service for FP8 128 x 128 block sources
-(`weight` / `weight_scale_inv`, which the reference decodes at load, src/dew/interop/codecs.py:638-648).
+(`weight` / `weight_scale_inv`, which the reference decodes at load, src/dew/interop/codecs.py:638-648) and for
+DeepSeek-V4's FP4 routed experts (`weight` nibbles / E8M0 `scale`, MXFP4's own storage).
 
 Tensors may live on the host or the device; every step is a torch index or bit operation, so a bank loaded to the
 GPU is re-laid there. The banks go into the `'quantization'` collection at the path their parameter had.
@@ -129,6 +130,41 @@ def fp8_expert_banks(tensors: Mapping[str, torch.Tensor], prefix: str, experts: 
                                            [tensors[name + FP8_SUFFIXES[1]] for name in names])
         for name in names:
             for suffix in FP8_SUFFIXES:
+                del tensors[name + suffix]
+    return tensors, banks
+
+
+FP4_SUFFIXES = (".weight", ".scale")
+"""The two tensors a DeepSeek-V4 FP4 routed expert is stored as (src/dew/interop/codecs.py `deepseek_v4(fp4_experts=True)`)."""
+
+
+def fp4_expert_bank(weights, scales) -> formats.Mxfp4Blocks:
+    """One projection's DeepSeek-V4 FP4 experts, each stored `[out, in / 2]` bytes of two E2M1 codes (the lower input in
+    the low nibble) with `[out, in / 32]` E8M0 scales, as the MXFP4 bank the kernels multiply, still packed. The storage
+    is MXFP4's own (an E2M1 code times `2 ** (scale - 127)` per 32 inputs), so the bytes are stacked and viewed as
+    `[E, out, in / 32, 16]` blocks, not decoded (the reference's load decodes them dense, src/dew/interop/codecs.py
+    `DeepseekV4.decode`); `codecs.dequantize_mxfp4` of the bank is the release's own reading of the expert in every value."""
+    weights, scales = list(weights), list(scales)
+    codes = torch.stack([weight.view(torch.uint8) for weight in weights]).contiguous()
+    powers = torch.stack([scale.view(torch.uint8) for scale in scales]).contiguous()
+    experts, width, half = codes.shape
+    if half % 16 or tuple(powers.shape) != (experts, width, half // 16):
+        raise ValueError(f"an FP4 expert is [out, in / 2] bytes in whole groups of 32 inputs with [out, in / 32] E8M0 scales, got "
+                         f"{tuple(codes.shape)} and {tuple(powers.shape)}")
+    return formats.Mxfp4Blocks(codes.reshape(experts, width, half // 16, 16), powers)
+
+
+def fp4_expert_banks(tensors: Mapping[str, torch.Tensor], prefix: str, experts: int,
+                     projections=("w1", "w3", "w2")) -> tuple[dict, dict]:
+    """`tensors` without `prefix.{e}.{projection}.weight` / `.scale` for e < experts, and the stacked packed banks by
+    projection name (the release's w1, w3, w2 are the gate, up and down projections)."""
+    tensors, banks = dict(tensors), {}
+    for projection in projections:
+        names = [f"{prefix}.{e}.{projection}" for e in range(experts)]
+        banks[projection] = fp4_expert_bank([tensors[name + FP4_SUFFIXES[0]] for name in names],
+                                            [tensors[name + FP4_SUFFIXES[1]] for name in names])
+        for name in names:
+            for suffix in FP4_SUFFIXES:
                 del tensors[name + suffix]
     return tensors, banks
 

@@ -143,3 +143,29 @@ def test_a_bank_packed_by_another_encoder_is_refused():
     with pytest.raises(ValueError, match="whole 256s"):
         formats.NvFp4.of(torch.zeros((1, 128, 4), dtype=torch.uint8), torch.zeros((1, 8, 4), dtype=torch.uint8),
                          torch.ones(1))
+
+
+@pytest.mark.parametrize("release", ["v4", "v4_1"])
+def test_a_deepseek_v4_fp4_expert_is_an_mxfp4_bank_as_stored(release):
+    """The FP4 routed expert of the reference's tests/fixtures/codecs/deepseek_v4_release.npz (each release's own
+    conversion over a tiny checkpoint, tests/test_codecs.py:219-237 there): stacked as it is stored
+    (`loads.fp4_expert_bank`, no value decoded), the bank's MXFP4 decoding is the release's dense reading of the expert in
+    every value, by the product's decoder and by the oracle's."""
+    from dew_amd import loads
+    held = golden("codecs/deepseek_v4_fp4_expert.npz")
+    weight, scale, dense = (held[f"{release}/{name}"] for name in ("weight", "scale", "dense"))
+    bank = loads.fp4_expert_bank([torch.from_numpy(weight.copy())] * 2, [torch.from_numpy(scale.copy())] * 2)
+    outputs, inputs = dense.shape
+    assert isinstance(bank, formats.Mxfp4Blocks) and bank.shape == (2, inputs, outputs)
+    assert np.array_equal(bank.blocks.numpy().reshape(2, outputs, inputs // 2), np.stack([weight.view(np.uint8)] * 2))   # the bytes themselves
+    decoded = codecs.dequantize_mxfp4(bank.blocks, bank.scales, torch.float32).numpy()
+    assert np.array_equal(decoded[0], dense.T) and np.array_equal(decoded[1], dense.T)
+    assert np.array_equal(oracle.decode_mxfp4(bank.blocks.numpy(), bank.scales.numpy())[0], dense.T)
+    tensors = {f"ffn.experts.{e}.{p}{suffix}": torch.from_numpy((weight if suffix == ".weight" else scale).copy())
+               for e in range(2) for p in ("w1", "w3", "w2") for suffix in loads.FP4_SUFFIXES}
+    tensors["ffn.gate.weight"] = torch.zeros(2, 4)
+    left, banks = loads.fp4_expert_banks(tensors, "ffn.experts", 2)
+    assert list(left) == ["ffn.gate.weight"] and sorted(banks) == ["w1", "w2", "w3"]
+    assert all(torch.equal(found.blocks, bank.blocks) and torch.equal(found.scales, bank.scales) for found in banks.values())
+    with pytest.raises(ValueError, match="whole groups of 32"):
+        loads.fp4_expert_bank([torch.from_numpy(weight[:, :24].copy())], [torch.from_numpy(scale.copy())])

@@ -177,3 +177,32 @@ def test_an_fp8_checkpoints_tensors_are_read_where_they_lie(ops):
     x = torch.from_numpy(rng.standard_normal((sum(sizes), depth)).astype(np.float32)).to(torch.bfloat16).cuda()
     assert torch.equal(ops.grouped_gemm(x, direct, offsets), ops.grouped_gemm(x, chain, offsets))
     assert torch.equal(ops.gateup_swiglu(x, direct, direct, offsets), ops.gateup_swiglu(x, chain, chain, offsets))
+
+
+@pytest.mark.parametrize("release", ["v4", "v4_1"])
+def test_a_deepseek_v4_fp4_expert_multiplies_packed_as_the_releases_dense_reading_does(ops, release):
+    """The FP4 routed expert the reference's tests hold (tests/fixtures/codecs/deepseek_v4_release.npz: the releases' own
+    conversion), stacked as stored (`loads.fp4_expert_bank`) and multiplied on the device without a dense copy, against
+    the oracle's product over the release's dense reading of that expert. V4.1's tiny expert is 96 deep and 64 wide,
+    below the launches' least extents, so its bytes are tiled to 192 x 128; its scale bytes were drawn over 21 binades,
+    past what one expert's packed bank spans (17), so the re-layout refuses it by name and it multiplies as the decoded
+    bank (`loads.dense_bank`), as such a bank of gpt-oss's would."""
+    from dew_amd import gemm
+
+    held = golden("codecs/deepseek_v4_fp4_expert.npz")
+    weight, scale, dense = (held[f"{release}/{name}"] for name in ("weight", "scale", "dense"))
+    if release == "v4_1":
+        weight, scale, dense = (np.tile(array, (2, 2)) for array in (weight, scale, dense))
+    sizes = [37, 0, 70]
+    bank = loads.fp4_expert_bank([torch.from_numpy(weight.copy()).cuda()] * 3, [torch.from_numpy(scale.copy()).cuda()] * 3)
+    outputs, inputs = dense.shape
+    assert bank.shape == (3, inputs, outputs) and bank.blocks.is_cuda
+    if release == "v4_1":
+        with pytest.raises(ops.KernelError, match="stays dense"):
+            gemm.prepared(bank)
+        bank = loads.dense_bank(bank.blocks, bank.scales)
+    rng = np.random.default_rng(inputs)
+    x = torch.from_numpy(rng.standard_normal((sum(sizes), inputs)).astype(np.float32)).to(torch.bfloat16)
+    got = gemm.gemm(x.cuda(), bank, torch.tensor(sizes, dtype=torch.int32).cuda()).float().cpu().numpy()
+    want = oracle.grouped_matmul(x.float().numpy(), np.stack([dense.T] * 3), sizes)
+    assert got.shape == want.shape and np.abs(got - want).max() <= 2 ** -7 * np.abs(want).max() and (got == want).mean() > 0.97
