@@ -114,6 +114,8 @@ struct RouteParams {
   int fill_excluded;     // an expert outside the kept groups competes at `excluded` rather than -inf
   float excluded;
   float softcap;         // above 0: every logit is read as softcap * tanh(logit / softcap)
+  const int32_t* given;    // nullable [T, k]: the experts to use in place of the router's own choice (a replayed record, a hash table's)
+  const uint8_t* covered;  // nullable [T]: with `given`, the tokens it covers; the others keep the router's choice
 };
 
 // Laguna's capped gate logit (`capped_logits`, src/dew/nn/precision.py:2086-2092): cap * tanh(logit / cap) in fp32.
@@ -237,10 +239,14 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
     }
   }
 
+  // A token whose experts are given takes them as they come (ids outside the experts are held to the nearest one, so
+  // every read below stays in range); the wavefront is one token, so the branch is uniform.
+  const bool replayed = p.given != nullptr && (p.covered == nullptr || p.covered[token] != 0);
   // top-k: k rounds of a wave-wide argmax, ties to the lower index
   unsigned taken_mask = 0u;
   int my_choice = 0;
-  for (int round = 0; round < p.top_k; ++round) {
+  if (replayed && lane < p.top_k) my_choice = min(max(p.given[static_cast<size_t>(token) * p.top_k + lane], 0), p.experts - 1);
+  for (int round = 0; round < (replayed ? 0 : p.top_k); ++round) {
     Best b;
     b.value = ninf;
     b.index = 0x7fffffff;
@@ -308,7 +314,14 @@ extern "C" int dew_moe_route_sown(const float* logits, const float* bias, int32_
 
 extern "C" int dew_moe_route_with(const dew_moe_router* router, const float* logits, const float* bias, int32_t tokens,
                                   float* weights, int32_t* indices, float* scores, float* log_z, void* stream) {
+  return dew_moe_route_replayed(router, logits, bias, nullptr, nullptr, tokens, weights, indices, scores, log_z, stream);
+}
+
+extern "C" int dew_moe_route_replayed(const dew_moe_router* router, const float* logits, const float* bias,
+                                      const int32_t* given, const uint8_t* covered, int32_t tokens, float* weights,
+                                      int32_t* indices, float* scores, float* log_z, void* stream) {
   using namespace dew;
+  DEW_REQUIRE(given || !covered, "dew_moe_route: a coverage without the experts it covers");
   DEW_REQUIRE(router, "dew_moe_route: the router's description must not be null");
   const int experts = router->experts, top_k = router->top_k, score_function = router->score_function;
   const int expert_groups = router->expert_groups, groups_per_token = router->groups_per_token;
@@ -343,7 +356,7 @@ extern "C" int dew_moe_route_with(const dew_moe_router* router, const float* log
   RouteParams p{logits, bias, weights, indices, tokens, experts, top_k, score_function, router->normalize ? 1 : 0,
                 expert_groups, groups_per_token, router->group_score == DEW_MOE_GROUP_MAX ? 1 : 0, router->scaling, scores, log_z,
                 router->bias_in_weights ? 1 : 0, router->weight_sum_epsilon, router->weight_sum_min,
-                router->fill_excluded ? 1 : 0, router->excluded_group_score, router->logit_softcap};
+                router->fill_excluded ? 1 : 0, router->excluded_group_score, router->logit_softcap, given, covered};
   const int blocks = (tokens + kRouteWaves - 1) / kRouteWaves;
   const size_t shared = expert_groups > 1 ? sizeof(float) * kRouteWaves * experts : 0;
   const dim3 grid(blocks), block(kWave * kRouteWaves);

@@ -162,12 +162,17 @@ class Router(_Module):
     """What an expert outside a token's best groups is chosen by: None for never (DeepSeek V3's -inf), or A.X-K2's 0.0."""
     logit_softcap: float | None = None
     """Laguna's cap `c` on each gate logit, `c * tanh(logit / c)`, before the scores and the z-loss read it."""
+    hash_vocab: int | None = None
+    """DeepSeek V4's hash router: the experts are the row of the `tid2eid [hash_vocab, top_k]` table (int32, at
+    `moe/<path>/tid2eid`) at the token id the caller passes, weighted by the learned gate."""
 
     def __post_init__(self):
         if self.bias_in_weights and not self.expert_bias:
             raise ValueError("bias_in_weights gates on the balancing bias, which expert_bias holds")
         if self.logit_softcap is not None and not self.logit_softcap > 0:
             raise ValueError(f"logit_softcap is a positive cap on the gate logits, or None for none; got {self.logit_softcap}")
+        if self.hash_vocab is not None and (self.expert_bias or self.expert_groups > 1):
+            raise ValueError("hash routing selects by the token table alone, so it has no balancing bias and no expert groups")
         if self.score_function not in ("softmax", "sigmoid", "sqrtsoftplus"):
             raise ValueError(f"score_function {self.score_function!r}: the router scores by 'softmax', 'sigmoid' or 'sqrtsoftplus'")
         if self.group_score not in ("top2", "max"):
@@ -180,11 +185,13 @@ class Router(_Module):
         kernel = _at(self.variables["params"], (*self.path, "kernel"))
         return ops.router_logits(x.reshape(-1, x.shape[-1]).contiguous(), kernel).reshape(*x.shape[:-1], self.num_experts)
 
-    def routed(self, logits: torch.Tensor, sown: dict | None = None):
+    def routed(self, logits: torch.Tensor, sown: dict | None = None, *, given: torch.Tensor | None = None,
+               covered: torch.Tensor | None = None):
         """(weights, indices) from the logits on (src/dew/nn/moe.py:466-494). A caller that opens the 'router'
         collection passes `sown`, a dict: it receives what the reference's router sows there (:474-479), the
         choices under 'indices', the activated scores under 'scores' and each position's log partition
-        `logsumexp(logits)` under 'log_z', written by the same launch."""
+        `logsumexp(logits)` under 'log_z', written by the same launch. `given` are experts to use in place of the
+        router's own choice for the tokens `covered` marks (all, where None): `chosen_experts` (:202-224)."""
         bias = _at(self.variables.get("moe"), (*self.path, "e_score_correction_bias")) if self.expert_bias else None
         if self.expert_bias and bias is None:
             raise KeyError(f"no moe/{'/'.join(self.path)}/e_score_correction_bias")
@@ -194,15 +201,45 @@ class Router(_Module):
                           groups_per_token=self.groups_per_token, group_score=self.group_score, sown=sown is not None,
                           bias_in_weights=self.bias_in_weights, weight_sum_epsilon=self.weight_sum_epsilon,
                           weight_sum_min=self.weight_sum_min, excluded_group_score=self.excluded_group_score,
-                          logit_softcap=self.logit_softcap)
+                          logit_softcap=self.logit_softcap, given=given, covered=covered)
         if sown is not None:
             sown.update(indices=found[1], scores=found[2], log_z=found[3])
         return found[0], found[1]
 
+    def given_experts(self, shape: tuple, tokens=None, routes=None):
+        """(given, covered) for `routed`: the hash table's rows at the token ids (`_selected`, src/dew/nn/moe.py:500-507),
+        over them a replayed record where it covers a token (`chosen_experts`, :202-224). (None, None) where the router
+        chooses on its own."""
+        given = covered = None
+        if self.hash_vocab is not None:
+            if tokens is None:
+                raise ValueError("hash routing selects by the token ids, which the caller passes")
+            table = _at(self.variables.get("moe"), (*self.path, "tid2eid"))
+            if table is None:
+                raise KeyError(f"no moe/{'/'.join(self.path)}/tid2eid")
+            given = table.to(torch.int32)[tokens.long()].contiguous()
+        elif tokens is not None:
+            raise ValueError("only a hash router reads the token ids")
+        if routes is not None:
+            replayed, covers = routes
+            if tuple(replayed.shape) != tuple(shape):
+                raise ValueError(f"replayed routing is {tuple(replayed.shape)} for {tuple(shape[:-1])} tokens choosing {shape[-1]} experts each")
+            if replayed.dtype.is_floating_point or replayed.dtype == torch.bool:
+                raise ValueError(f"replayed routing holds expert ids, got {replayed.dtype}")
+            replayed = replayed.to(torch.int32).contiguous()
+            if covers is not None and tuple(covers.shape) != tuple(shape[:-1]):
+                raise ValueError(f"replay coverage is {tuple(covers.shape)} for {tuple(shape[:-1])} tokens")
+            if given is None or covers is None:
+                given, covered = replayed, None if covers is None else covers.to(torch.bool).contiguous()
+            else:       # a hash router under a partial record: the table's rows where the record is silent
+                given = torch.where(covers.to(torch.bool)[..., None], replayed, given).contiguous()
+        return given, covered
+
     def __call__(self, x, tokens=None, media=None, routes=None, blocks=None):
-        if tokens is not None or media is not None or routes is not None or blocks is not None:
-            raise ValueError("hash, media, replayed and block routing are not part of the HIP router")
-        return self.routed(self.logits(x))
+        if media is not None or blocks is not None:
+            raise ValueError("media-bias and block routing are not part of the HIP router")
+        given, covered = self.given_experts((*x.shape[:-1], self.top_k), tokens, routes)
+        return self.routed(self.logits(x), given=given, covered=covered)
 
 
 def load_balance_update(counts: torch.Tensor, rate: float) -> torch.Tensor:
@@ -406,6 +443,7 @@ class SparseMLP(_Module):
     weight_sum_epsilon: float = ops.WEIGHT_SUM_EPSILON
     weight_sum_min: float = 0.0
     excluded_group_score: float | None = None
+    hash_vocab: int | None = None
     router_softcap: float | None = None
     """The router's switches (`Router`'s fields of the same names; `router_softcap` is its `logit_softcap`,
     src/dew/nn/moe.py:1440-1446)."""
@@ -415,7 +453,7 @@ class SparseMLP(_Module):
         return Router(self.num_experts, self.out_features, self.top_k, self.score_function, self.normalize_weights,
                       self.routed_scaling_factor, self.expert_groups, self.groups_per_token, self.group_score,
                       self.expert_bias, self.bias_in_weights, self.weight_sum_epsilon, self.weight_sum_min,
-                      self.excluded_group_score, self.router_softcap)._bound(self.variables, (*self.path, "gate"))
+                      self.excluded_group_score, self.router_softcap, self.hash_vocab)._bound(self.variables, (*self.path, "gate"))
 
     @property
     def experts(self) -> ExpertMLP:
@@ -435,7 +473,10 @@ class SparseMLP(_Module):
         if logits is None:
             weights, indices = gate(x, tokens, media, routes, blocks)
         else:
-            weights, indices = gate.routed(logits)
+            if media is not None or blocks is not None:
+                raise ValueError("media-bias and block routing are not part of the HIP router")
+            given, covered = gate.given_experts((*x.shape[:-1], self.top_k), tokens, routes)
+            weights, indices = gate.routed(logits, given=given, covered=covered)
         # routed + shared (src/dew/nn/moe.py:1497-1503): the bf16 add runs in the combine kernel's epilogue. A shared
         # expert of the routed experts' width and format is multiplied by the routed launches, as their group #E.
         experts = self.experts

@@ -49,6 +49,10 @@ What pins each function (tests/test_oracle_golden.py):
   the others by their definitions in float64 (the biased scores gathered; the sums floored, with the tokens below the
   floor summing to sum / floor and the rest to one; `cap * tanh(x / cap)`, bounded, order-preserving), each of which a
   dropped bias, a floor applied before the epsilon or a cap applied after the scores fails.
+* `route(given=, covered=)` (replayed routes and the hash router's table rows, `chosen_experts` src/dew/nn/moe.py:202-224):
+  no vectors in the reference; pinned by what the definition fixes: the router's own choice given back reproduces its
+  weights bit for bit, a permutation of it permutes them, uncovered tokens keep the router's own routing, and the weights
+  of arbitrary given experts are the float64 gather-and-normalize of their scores.
 * `load_balance_update`: the known answer of tests/test_moe.py:326-336 (counts 3, 1, 0, 0 at rate 0.001).
 * `router_statistics`: closed forms (scores = exp(logits - log_z) for softmax; log_z(logits + c) = log_z + c; the
   z-loss's log partition against a float64 logsumexp).
@@ -395,17 +399,20 @@ def top_k_margin(selection, top_k_count):
 def route(logits, top_k_count, *, score_function="softmax", normalize_weights=True, bias=None,
           routed_scaling_factor=1.0, expert_groups=1, groups_per_token=1, group_score="top2",
           weight_sum_epsilon=1e-20, weight_sum_min=0.0, bias_in_weights=False, excluded_group_score=None,
-          logit_softcap=None):
+          logit_softcap=None, given=None, covered=None):
     """`Router.__call__` from its logits on (src/dew/nn/moe.py:466-494): the cap on the logits (:526-534), scores,
     selection (bias, group-limited mask :496-565), top-k, weights (:483-494: a softmax router renormalizes the chosen
     logits unless `bias_in_weights` or `weight_sum_min` say otherwise; else the chosen scores, plus the bias under
-    `bias_in_weights`, over `max(sum + weight_sum_epsilon, weight_sum_min)`). Returns (weights fp32 [T, k], indices
-    int32 [T, k])."""
+    `bias_in_weights`, over `max(sum + weight_sum_epsilon, weight_sum_min)`). `given` [T, k] are experts used in place
+    of the top-k for the tokens `covered` [T] marks (all where None). Returns (weights fp32 [T, k], indices int32 [T, k])."""
     logits = capped_logits(logits, logit_softcap)
     scores, selection = selection_scores(logits, score_function=score_function, bias=bias, expert_groups=expert_groups,
                                          groups_per_token=groups_per_token, group_score=group_score,
                                          excluded_group_score=excluded_group_score)
     _, indices = top_k(selection, top_k_count)
+    if given is not None:      # `chosen_experts` (src/dew/nn/moe.py:202-224): a replayed record, or the hash table's rows (:500-507)
+        given = np.asarray(given).astype(np.int32)
+        indices = given if covered is None else np.where(np.asarray(covered, bool)[..., None], given, indices).astype(np.int32)
     if normalize_weights and score_function == "softmax" and not bias_in_weights and not weight_sum_min:
         weights = expert_softmax(np.take_along_axis(logits, indices, axis=-1))        # moe.py:194-199,485
     else:

@@ -114,6 +114,70 @@ def test_a_logit_softcap_caps_what_every_reader_of_the_logits_reads(ops, score_f
     assert np.abs(got[3].cpu().numpy()).max() <= cap + np.log(experts) + 1e-3
 
 
+@pytest.mark.parametrize("score_function,experts,k,extra", [("softmax", 64, 4, {}), ("sigmoid", 256, 8, dict(routed_scaling_factor=2.5)),
+                                                            ("sqrtsoftplus", 128, 6, {}), ("softmax", 32, 2, dict(normalize_weights=False)),
+                                                            ("sigmoid", 64, 8, dict(expert_groups=8, groups_per_token=3))])
+def test_given_experts_weigh_as_the_router_weighs_them(ops, score_function, experts, k, extra):
+    """A replayed record's or a hash table's experts (`dew_moe_route_replayed`): every token covered, and some; ids
+    outside the experts held to the nearest; the router's own choice given back is its own routing."""
+    rng = np.random.default_rng(experts * 7 + k)
+    tokens = 271
+    logits = (rng.standard_normal((tokens, experts)) * 2).astype(np.float32)
+    biased = score_function == "sigmoid"
+    bias = (rng.standard_normal(experts) * 0.1).astype(np.float32) if biased else None
+    settings = dict(score_function=score_function, **extra)
+    table = rng.integers(0, experts, size=(tokens, k)).astype(np.int32)
+    covered = rng.integers(0, 2, size=tokens).astype(bool)
+    on_device = dict(bias=None if bias is None else torch.from_numpy(bias).cuda())
+    for given, covers in ((table, None), (table, covered)):
+        want_w, want_i = oracle.route(logits, k, bias=bias, given=given, covered=covers, **settings)
+        got_w, got_i = ops.route(torch.from_numpy(logits).cuda(), k, given=torch.from_numpy(given).cuda(),
+                                 covered=None if covers is None else torch.from_numpy(covers).cuda(), **on_device, **settings)
+        assert np.array_equal(got_i.cpu().numpy(), want_i)
+        assert np.array_equal(got_w.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
+    own_w, own_i = ops.route(torch.from_numpy(logits).cuda(), k, **on_device, **settings)
+    again_w, again_i = ops.route(torch.from_numpy(logits).cuda(), k, given=own_i, **on_device, **settings)
+    assert torch.equal(again_i, own_i) and torch.equal(again_w, own_w)
+    wild = table.copy()
+    wild[::3, 0], wild[1::3, -1] = -5, experts + 9
+    got_w, got_i = ops.route(torch.from_numpy(logits).cuda(), k, given=torch.from_numpy(wild).cuda(), **on_device, **settings)
+    want_w, want_i = oracle.route(logits, k, bias=bias, given=np.clip(wild, 0, experts - 1), **settings)
+    assert np.array_equal(got_i.cpu().numpy(), want_i) and np.array_equal(got_w.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
+    with pytest.raises(ops.KernelError, match="replayed routing"):
+        ops.route(torch.from_numpy(logits).cuda(), k, given=torch.from_numpy(table[:, :1].copy()).cuda(), **settings)
+    with pytest.raises(ops.KernelError, match="coverage"):
+        ops.route(torch.from_numpy(logits).cuda(), k, covered=torch.from_numpy(covered).cuda(), **settings)
+
+
+def test_a_hash_router_takes_its_experts_from_the_token_table(ops):
+    """DeepSeek V4's hash router (`hash_vocab`, src/dew/nn/moe.py:337-341, 500-507): the experts are `tid2eid[token id]`,
+    weighted by the learned gate; a replayed record covers some tokens over it; only a hash router reads token ids."""
+    from dew_amd import moe
+    rng = np.random.default_rng(31)
+    vocab, experts, k, width = 50, 16, 3, 128
+    kernel = (rng.standard_normal((width, experts)) * 0.2).astype(np.float32)
+    table = rng.integers(0, experts, size=(vocab, k)).astype(np.int32)
+    x = torch.from_numpy(rng.standard_normal((2, 9, width)).astype(np.float32)).to(torch.bfloat16)
+    ids = rng.integers(0, vocab, size=(2, 9))
+    variables = {"params": {"kernel": torch.from_numpy(kernel).cuda()}, "moe": {"tid2eid": torch.from_numpy(table).cuda()}}
+    router = moe.Router(experts, width, k, score_function="sqrtsoftplus", routed_scaling_factor=1.5, hash_vocab=vocab)
+    weights, indices = router.apply(variables, x.cuda(), torch.from_numpy(ids).cuda())
+    logits = oracle.router_logits(x.float().numpy().reshape(-1, width), kernel)
+    want_w, want_i = oracle.route(logits, k, score_function="sqrtsoftplus", routed_scaling_factor=1.5, given=table[ids.reshape(-1)])
+    assert indices.shape == (2, 9, k) and np.array_equal(indices.cpu().numpy().reshape(-1, k), table[ids.reshape(-1)])
+    assert np.abs(weights.cpu().numpy().reshape(-1, k) - want_w).max() <= 1e-6
+    replayed = rng.integers(0, experts, size=(2, 9, k)).astype(np.uint8)          # engines ship the narrowest unsigned type
+    covers = rng.integers(0, 2, size=(2, 9)).astype(bool)
+    _, mixed = router.apply(variables, x.cuda(), torch.from_numpy(ids).cuda(), routes=(torch.from_numpy(replayed).cuda(), torch.from_numpy(covers).cuda()))
+    assert np.array_equal(mixed.cpu().numpy(), np.where(covers[..., None], replayed.astype(np.int32), table[ids]))
+    with pytest.raises(ValueError, match="token ids, which the caller passes"):
+        router.apply(variables, x.cuda())
+    with pytest.raises(ValueError, match="only a hash router"):
+        moe.Router(experts, width, k).apply(variables, x.cuda(), torch.from_numpy(ids).cuda())
+    with pytest.raises(ValueError, match="expert ids"):
+        moe.Router(experts, width, k).apply(variables, x.cuda(), routes=(torch.zeros(2, 9, k).cuda(), None))
+
+
 def test_router_refuses_bounds_that_bound_nothing(ops):
     logits = torch.zeros(4, 8, device="cuda")
     with pytest.raises(ops.KernelError, match="bias_in_weights"):

@@ -556,3 +556,36 @@ def test_the_gated_products_are_torchs_recorded_bf16_outputs():
     got = oracle.geglu(gate, up)
     differs = got != output
     assert differs.sum() < 40 and np.all(output[differs] == 0) and np.abs(got[differs]).max() < 1e-16   # Torch's tanh at -1
+
+
+def test_given_experts_take_the_routers_weights_for_them():
+    """Replayed routes and a hash table's rows (`chosen_experts`, src/dew/nn/moe.py:202-224, 500-507): the router's own
+    choice given back is its own routing; a reordering of it reorders the weights; a token the record does not cover
+    keeps the router's choice; arbitrary experts weigh by their scores, gathered and normalized."""
+    rng = np.random.default_rng(14)
+    logits = (rng.standard_normal((60, 16)) * 2).astype(np.float32)
+    for settings in (dict(score_function="softmax"), dict(score_function="sigmoid", routed_scaling_factor=2.5),
+                     dict(score_function="softmax", normalize_weights=False), dict(score_function="sqrtsoftplus")):
+        weights, indices = oracle.route(logits, 4, **settings)
+        again_w, again_i = oracle.route(logits, 4, given=indices, **settings)
+        assert np.array_equal(again_i, indices) and np.array_equal(again_w, weights)
+        flipped_w, flipped_i = oracle.route(logits, 4, given=indices[:, ::-1], **settings)
+        assert np.array_equal(flipped_i, indices[:, ::-1]) and np.abs(flipped_w - weights[:, ::-1]).max() <= ROUTER_TOLERANCE
+        table = rng.integers(0, 16, size=(60, 4)).astype(np.int32)
+        covered = rng.integers(0, 2, size=60).astype(bool)
+        mixed_w, mixed_i = oracle.route(logits, 4, given=table, covered=covered, **settings)
+        assert np.array_equal(mixed_i[covered], table[covered]) and np.array_equal(mixed_i[~covered], indices[~covered])
+        assert np.array_equal(mixed_w[~covered], weights[~covered])
+        wide = logits.astype(np.float64)
+        if settings["score_function"] == "softmax":
+            scores = np.exp(wide - wide.max(-1, keepdims=True))
+            scores /= scores.sum(-1, keepdims=True)
+        elif settings["score_function"] == "sigmoid":
+            scores = 1 / (1 + np.exp(-wide))
+        else:
+            scores = np.sqrt(np.logaddexp(0.0, wide))
+        truth = np.take_along_axis(scores, table.astype(np.int64), -1)
+        if settings.get("normalize_weights", True):
+            truth = truth / (truth.sum(-1, keepdims=True) + 1e-20)
+        truth = truth * settings.get("routed_scaling_factor", 1.0)
+        assert np.abs(mixed_w[covered] - truth[covered]).max() <= 2 * ROUTER_TOLERANCE
