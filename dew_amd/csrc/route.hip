@@ -116,6 +116,8 @@ struct RouteParams {
   float softcap;         // above 0: every logit is read as softcap * tanh(logit / softcap)
   const int32_t* given;    // nullable [T, k]: the experts to use in place of the router's own choice (a replayed record, a hash table's)
   const uint8_t* covered;  // nullable [T]: with `given`, the tokens it covers; the others keep the router's choice
+  const float* media_bias; // nullable [E]: the bias a media token's experts are chosen by, in place of `bias`
+  const uint8_t* media;    // nullable [T]: the media tokens
 };
 
 // Laguna's capped gate logit (`capped_logits`, src/dew/nn/precision.py:2086-2092): cap * tanh(logit / cap) in fp32.
@@ -184,11 +186,15 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
     if (active && lane == 0) p.log_z[token] = m + logf(total);
   }
 
+  const bool by_media = p.media != nullptr && p.media[token] != 0;  // DeepSeek-V4.1's image-span tokens (one token a wavefront)
 #pragma unroll
   for (int i = 0; i < kPerLane; ++i) {
     const int e = lane + kWave * i;
     float s = score[i];
-    if (p.bias != nullptr && e < p.experts) s = s + p.bias[e];
+    if (e < p.experts) {
+      if (by_media) s = s + p.media_bias[e];
+      else if (p.bias != nullptr) s = s + p.bias[e];
+    }
     // A NaN selection (a NaN in the bias or the logits) is never preferred: it competes as -inf, so every round still
     // finds an expert in range (no comparison with NaN holds, and a round without a candidate would name no expert).
     select[i] = (e < p.experts && s == s) ? s : ninf;
@@ -314,14 +320,16 @@ extern "C" int dew_moe_route_sown(const float* logits, const float* bias, int32_
 
 extern "C" int dew_moe_route_with(const dew_moe_router* router, const float* logits, const float* bias, int32_t tokens,
                                   float* weights, int32_t* indices, float* scores, float* log_z, void* stream) {
-  return dew_moe_route_replayed(router, logits, bias, nullptr, nullptr, tokens, weights, indices, scores, log_z, stream);
+  return dew_moe_route_call(router, logits, bias, nullptr, nullptr, nullptr, nullptr, tokens, weights, indices, scores, log_z, stream);
 }
 
-extern "C" int dew_moe_route_replayed(const dew_moe_router* router, const float* logits, const float* bias,
-                                      const int32_t* given, const uint8_t* covered, int32_t tokens, float* weights,
-                                      int32_t* indices, float* scores, float* log_z, void* stream) {
+extern "C" int dew_moe_route_call(const dew_moe_router* router, const float* logits, const float* bias,
+                                  const float* media_bias, const uint8_t* media, const int32_t* given,
+                                  const uint8_t* covered, int32_t tokens, float* weights, int32_t* indices, float* scores,
+                                  float* log_z, void* stream) {
   using namespace dew;
   DEW_REQUIRE(given || !covered, "dew_moe_route: a coverage without the experts it covers");
+  DEW_REQUIRE((media == nullptr) == (media_bias == nullptr), "dew_moe_route: the media tokens and the bias that chooses for them come together");
   DEW_REQUIRE(router, "dew_moe_route: the router's description must not be null");
   const int experts = router->experts, top_k = router->top_k, score_function = router->score_function;
   const int expert_groups = router->expert_groups, groups_per_token = router->groups_per_token;
@@ -356,7 +364,7 @@ extern "C" int dew_moe_route_replayed(const dew_moe_router* router, const float*
   RouteParams p{logits, bias, weights, indices, tokens, experts, top_k, score_function, router->normalize ? 1 : 0,
                 expert_groups, groups_per_token, router->group_score == DEW_MOE_GROUP_MAX ? 1 : 0, router->scaling, scores, log_z,
                 router->bias_in_weights ? 1 : 0, router->weight_sum_epsilon, router->weight_sum_min,
-                router->fill_excluded ? 1 : 0, router->excluded_group_score, router->logit_softcap, given, covered};
+                router->fill_excluded ? 1 : 0, router->excluded_group_score, router->logit_softcap, given, covered, media_bias, media};
   const int blocks = (tokens + kRouteWaves - 1) / kRouteWaves;
   const size_t shared = expert_groups > 1 ? sizeof(float) * kRouteWaves * experts : 0;
   const dim3 grid(blocks), block(kWave * kRouteWaves);

@@ -162,6 +162,9 @@ class Router(_Module):
     """What an expert outside a token's best groups is chosen by: None for never (DeepSeek V3's -inf), or A.X-K2's 0.0."""
     logit_softcap: float | None = None
     """Laguna's cap `c` on each gate logit, `c * tanh(logit / c)`, before the scores and the z-loss read it."""
+    media_bias: bool = False
+    """DeepSeek-V4.1's second bias (`moe/<path>/media_bias`), choosing for the image-span tokens the `media` mask marks in
+    place of `expert_bias`."""
     hash_vocab: int | None = None
     """DeepSeek V4's hash router: the experts are the row of the `tid2eid [hash_vocab, top_k]` table (int32, at
     `moe/<path>/tid2eid`) at the token id the caller passes, weighted by the learned gate."""
@@ -186,7 +189,7 @@ class Router(_Module):
         return ops.router_logits(x.reshape(-1, x.shape[-1]).contiguous(), kernel).reshape(*x.shape[:-1], self.num_experts)
 
     def routed(self, logits: torch.Tensor, sown: dict | None = None, *, given: torch.Tensor | None = None,
-               covered: torch.Tensor | None = None):
+               covered: torch.Tensor | None = None, media: torch.Tensor | None = None):
         """(weights, indices) from the logits on (src/dew/nn/moe.py:466-494). A caller that opens the 'router'
         collection passes `sown`, a dict: it receives what the reference's router sows there (:474-479), the
         choices under 'indices', the activated scores under 'scores' and each position's log partition
@@ -195,13 +198,21 @@ class Router(_Module):
         bias = _at(self.variables.get("moe"), (*self.path, "e_score_correction_bias")) if self.expert_bias else None
         if self.expert_bias and bias is None:
             raise KeyError(f"no moe/{'/'.join(self.path)}/e_score_correction_bias")
+        media_bias = None
+        if media is not None:       # `selection` (src/dew/nn/moe.py:516-524): a media token's own bias
+            if not self.media_bias:
+                raise ValueError("only a router with a media bias reads the media mask")
+            media_bias = _at(self.variables.get("moe"), (*self.path, "media_bias"))
+            if media_bias is None:
+                raise KeyError(f"no moe/{'/'.join(self.path)}/media_bias")
+            media = media.to(torch.bool).contiguous()
         found = ops.route(logits, self.top_k, score_function=self.score_function,
                           normalize_weights=self.normalize_weights, bias=bias,
                           routed_scaling_factor=self.routed_scaling_factor, expert_groups=self.expert_groups,
                           groups_per_token=self.groups_per_token, group_score=self.group_score, sown=sown is not None,
                           bias_in_weights=self.bias_in_weights, weight_sum_epsilon=self.weight_sum_epsilon,
                           weight_sum_min=self.weight_sum_min, excluded_group_score=self.excluded_group_score,
-                          logit_softcap=self.logit_softcap, given=given, covered=covered)
+                          logit_softcap=self.logit_softcap, given=given, covered=covered, media=media, media_bias=media_bias)
         if sown is not None:
             sown.update(indices=found[1], scores=found[2], log_z=found[3])
         return found[0], found[1]
@@ -236,10 +247,10 @@ class Router(_Module):
         return given, covered
 
     def __call__(self, x, tokens=None, media=None, routes=None, blocks=None):
-        if media is not None or blocks is not None:
-            raise ValueError("media-bias and block routing are not part of the HIP router")
+        if blocks is not None:
+            raise ValueError("block routing is not part of the HIP router")
         given, covered = self.given_experts((*x.shape[:-1], self.top_k), tokens, routes)
-        return self.routed(self.logits(x), given=given, covered=covered)
+        return self.routed(self.logits(x), given=given, covered=covered, media=media)
 
 
 def load_balance_update(counts: torch.Tensor, rate: float) -> torch.Tensor:
@@ -444,6 +455,7 @@ class SparseMLP(_Module):
     weight_sum_min: float = 0.0
     excluded_group_score: float | None = None
     hash_vocab: int | None = None
+    media_bias: bool = False
     router_softcap: float | None = None
     """The router's switches (`Router`'s fields of the same names; `router_softcap` is its `logit_softcap`,
     src/dew/nn/moe.py:1440-1446)."""
@@ -453,7 +465,7 @@ class SparseMLP(_Module):
         return Router(self.num_experts, self.out_features, self.top_k, self.score_function, self.normalize_weights,
                       self.routed_scaling_factor, self.expert_groups, self.groups_per_token, self.group_score,
                       self.expert_bias, self.bias_in_weights, self.weight_sum_epsilon, self.weight_sum_min,
-                      self.excluded_group_score, self.router_softcap, self.hash_vocab)._bound(self.variables, (*self.path, "gate"))
+                      self.excluded_group_score, self.router_softcap, self.media_bias, self.hash_vocab)._bound(self.variables, (*self.path, "gate"))
 
     @property
     def experts(self) -> ExpertMLP:
@@ -473,10 +485,10 @@ class SparseMLP(_Module):
         if logits is None:
             weights, indices = gate(x, tokens, media, routes, blocks)
         else:
-            if media is not None or blocks is not None:
-                raise ValueError("media-bias and block routing are not part of the HIP router")
+            if blocks is not None:
+                raise ValueError("block routing is not part of the HIP router")
             given, covered = gate.given_experts((*x.shape[:-1], self.top_k), tokens, routes)
-            weights, indices = gate.routed(logits, given=given, covered=covered)
+            weights, indices = gate.routed(logits, given=given, covered=covered, media=media)
         # routed + shared (src/dew/nn/moe.py:1497-1503): the bf16 add runs in the combine kernel's epilogue. A shared
         # expert of the routed experts' width and format is multiplied by the routed launches, as their group #E.
         experts = self.experts

@@ -45,12 +45,14 @@ def route(logits: torch.Tensor, top_k: int, *, score_function: str = "softmax", 
           bias: torch.Tensor | None = None, routed_scaling_factor: float = 1.0, expert_groups: int = 1,
           groups_per_token: int = 1, group_score: str = "top2", sown: bool = False, bias_in_weights: bool = False,
           weight_sum_epsilon: float = WEIGHT_SUM_EPSILON, weight_sum_min: float = 0.0, excluded_group_score: float | None = None,
-          logit_softcap: float | None = None, given: torch.Tensor | None = None, covered: torch.Tensor | None = None):
+          logit_softcap: float | None = None, given: torch.Tensor | None = None, covered: torch.Tensor | None = None,
+          media: torch.Tensor | None = None, media_bias: torch.Tensor | None = None):
     """(weights fp32 `[..., k]`, indices int32 `[..., k]`) of router `logits [..., E]` (fp32); with `sown`, also what
     the router sows for the balance statistics: (weights, indices, scores fp32 `[..., E]`, log_z fp32 `[...]`). The
     five switches after `sown` are `Router`'s of the same names (src/dew/nn/moe.py:361-384). `given` (int32 `[..., k]`) are
     experts to use in place of the router's own choice (a replayed record, a hash table's rows), for the tokens `covered`
-    (bool `[...]`) marks, all of them where it is None; the weights are the router's for those experts."""
+    (bool `[...]`) marks, all of them where it is None; the weights are the router's for those experts. `media` (bool
+    `[...]`) marks the tokens whose experts are chosen by `media_bias [E]` in place of `bias`."""
     scores = {"softmax": _lib.SCORE_SOFTMAX, "sigmoid": _lib.SCORE_SIGMOID, "sqrtsoftplus": _lib.SCORE_SQRTSOFTPLUS}
     group_scores = {"top2": _lib.GROUP_TOP2, "max": _lib.GROUP_MAX}
     if score_function not in scores:
@@ -74,6 +76,13 @@ def route(logits: torch.Tensor, top_k: int, *, score_function: str = "softmax", 
         _device(covered, "covered", torch.bool)
         if covered.shape != logits.shape[:-1]:
             raise KernelError(f"replay coverage is {tuple(covered.shape)} for {tuple(logits.shape[:-1])} tokens")
+    if (media is None) != (media_bias is None):
+        raise KernelError("the media tokens and the bias that chooses for them come together")
+    if media is not None:
+        _device(media, "media", torch.bool), _device(media_bias, "media_bias", torch.float32)
+        if media.shape != logits.shape[:-1] or media_bias.shape != logits.shape[-1:]:
+            raise KernelError(f"media {tuple(media.shape)} marks {tuple(logits.shape[:-1])} tokens and media_bias "
+                              f"{tuple(media_bias.shape)} biases {logits.shape[-1]} experts")
     weights = torch.empty((*logits.shape[:-1], top_k), dtype=torch.float32, device=logits.device)
     indices = torch.empty((*logits.shape[:-1], top_k), dtype=torch.int32, device=logits.device)
     activated = torch.empty_like(logits) if sown else None
@@ -82,8 +91,8 @@ def route(logits: torch.Tensor, top_k: int, *, score_function: str = "softmax", 
                          expert_groups, groups_per_token, group_scores[group_score], int(bool(bias_in_weights)),
                          float(weight_sum_epsilon), float(weight_sum_min), int(excluded_group_score is not None),
                          float(excluded_group_score or 0.0), float(logit_softcap or 0.0))
-    _lib.check(_lib.library().dew_moe_route_replayed(router, _ptr(logits), _ptr(bias), _ptr(given), _ptr(covered), tokens, _ptr(weights),
-                                                     _ptr(indices), _ptr(activated), _ptr(log_z), _stream()), "dew_moe_route")
+    _lib.check(_lib.library().dew_moe_route_call(router, _ptr(logits), _ptr(bias), _ptr(media_bias), _ptr(media), _ptr(given), _ptr(covered),
+                                                 tokens, _ptr(weights), _ptr(indices), _ptr(activated), _ptr(log_z), _stream()), "dew_moe_route")
     return (weights, indices, activated, log_z) if sown else (weights, indices)
 
 

@@ -123,13 +123,17 @@ int dew_moe_route_sown(const float* logits, const float* bias /* nullable */, in
 int dew_moe_route_with(const dew_moe_router* router /* host */, const float* logits, const float* bias /* nullable */,
                        int32_t tokens, float* weights, int32_t* indices, float* scores, float* log_z, void* stream);
 
-/* dew_moe_route_with over experts that are given (`chosen_experts`, src/dew/nn/moe.py:202-224: a replayed record of an
- * engine's routing; and the hash router's `tid2eid[token ids]`, :500-507): token t uses given[t, :] in that order in place
- * of its own top-k, where `covered` is null or covered[t] != 0; the weights are the router's for those experts
- * (:483-494). An id outside [0, experts) is held to the nearest expert. given null is dew_moe_route_with.          */
-int dew_moe_route_replayed(const dew_moe_router* router /* host */, const float* logits, const float* bias /* nullable */,
-                           const int32_t* given /* nullable [T,k] */, const uint8_t* covered /* nullable [T] */,
-                           int32_t tokens, float* weights, int32_t* indices, float* scores, float* log_z, void* stream);
+/* dew_moe_route_with with the per-token inputs of `Router.__call__(x, tokens, media, routes)` (src/dew/nn/moe.py:466-524):
+ *  - media [T] with media_bias [E] (both or neither): DeepSeek-V4.1's image-span tokens, whose experts are chosen by
+ *    scores + media_bias in place of scores + bias (`selection`, :516-524);
+ *  - given [T,k], covered [T] (`chosen_experts`, :202-224: a replayed record of an engine's routing; and the hash router's
+ *    `tid2eid[token ids]`, :500-507): token t uses given[t, :] in that order in place of its own top-k, where `covered` is
+ *    null or covered[t] != 0. An id outside [0, experts) is held to the nearest expert.
+ * The weights are the router's for the experts used (:483-494). All four null is dew_moe_route_with.                  */
+int dew_moe_route_call(const dew_moe_router* router /* host */, const float* logits, const float* bias /* nullable */,
+                       const float* media_bias /* nullable [E] */, const uint8_t* media /* nullable [T] */,
+                       const int32_t* given /* nullable [T,k] */, const uint8_t* covered /* nullable [T] */,
+                       int32_t tokens, float* weights, int32_t* indices, float* scores, float* log_z, void* stream);
 
 /* The aux-loss-free balancing step (`load_balance_update` src/dew/nn/moe.py:271-300, applied to the selection bias as
  * `_updated_bias` src/dew/objectives/routing.py:342-345): bias[e] += rate * direction, direction -1 where counts[e]

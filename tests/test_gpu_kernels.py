@@ -118,7 +118,7 @@ def test_a_logit_softcap_caps_what_every_reader_of_the_logits_reads(ops, score_f
                                                             ("sqrtsoftplus", 128, 6, {}), ("softmax", 32, 2, dict(normalize_weights=False)),
                                                             ("sigmoid", 64, 8, dict(expert_groups=8, groups_per_token=3))])
 def test_given_experts_weigh_as_the_router_weighs_them(ops, score_function, experts, k, extra):
-    """A replayed record's or a hash table's experts (`dew_moe_route_replayed`): every token covered, and some; ids
+    """A replayed record's or a hash table's experts (`dew_moe_route_call`): every token covered, and some; ids
     outside the experts held to the nearest; the router's own choice given back is its own routing."""
     rng = np.random.default_rng(experts * 7 + k)
     tokens = 271
@@ -147,6 +147,34 @@ def test_given_experts_weigh_as_the_router_weighs_them(ops, score_function, expe
         ops.route(torch.from_numpy(logits).cuda(), k, given=torch.from_numpy(table[:, :1].copy()).cuda(), **settings)
     with pytest.raises(ops.KernelError, match="coverage"):
         ops.route(torch.from_numpy(logits).cuda(), k, covered=torch.from_numpy(covered).cuda(), **settings)
+
+
+@pytest.mark.parametrize("experts,k,groups,kept,biased", [(256, 8, 8, 4, True), (64, 6, 1, 1, True), (32, 2, 4, 2, False)])
+def test_media_tokens_are_chosen_for_by_the_media_bias(ops, experts, k, groups, kept, biased):
+    """DeepSeek-V4.1's image-span bias (`media_bias`, src/dew/nn/moe.py:342-344, 516-524) in the route kernel, against the
+    oracle bit for bit, through the kernel's wrapper and through the `Router` mirror's `media` argument."""
+    from dew_amd import moe
+    rng = np.random.default_rng(experts + k)
+    tokens = 300
+    logits = (rng.standard_normal((tokens, experts)) * 1.5).astype(np.float32)
+    bias = (rng.standard_normal(experts) * 0.3).astype(np.float32) if biased else None
+    media_bias = (rng.standard_normal(experts) * 0.3).astype(np.float32)
+    media = rng.integers(0, 2, size=tokens).astype(bool)
+    settings = dict(score_function="sigmoid", routed_scaling_factor=2.5, expert_groups=groups, groups_per_token=kept)
+    want_w, want_i = oracle.route(logits, k, bias=bias, media=media, media_bias=media_bias, **settings)
+    got_w, got_i = ops.route(torch.from_numpy(logits).cuda(), k, bias=None if bias is None else torch.from_numpy(bias).cuda(),
+                             media=torch.from_numpy(media).cuda(), media_bias=torch.from_numpy(media_bias).cuda(), **settings)
+    assert np.array_equal(got_i.cpu().numpy(), want_i) and np.array_equal(got_w.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
+    variables = {"params": {}, "moe": {"media_bias": torch.from_numpy(media_bias).cuda()}}
+    if biased:
+        variables["moe"]["e_score_correction_bias"] = torch.from_numpy(bias).cuda()
+    router = moe.Router(experts, 128, k, expert_bias=biased, media_bias=True, **settings)._bound(variables, ())
+    mirror_w, mirror_i = router.routed(torch.from_numpy(logits).cuda(), media=torch.from_numpy(media).cuda())
+    assert torch.equal(mirror_i, got_i) and torch.equal(mirror_w, got_w)
+    with pytest.raises(ValueError, match="only a router with a media bias"):
+        moe.Router(experts, 128, k, **settings)._bound(variables, ()).routed(torch.from_numpy(logits).cuda(), media=torch.from_numpy(media).cuda())
+    with pytest.raises(ops.KernelError, match="come together"):
+        ops.route(torch.from_numpy(logits).cuda(), k, media=torch.from_numpy(media).cuda(), **settings)
 
 
 def test_a_hash_router_takes_its_experts_from_the_token_table(ops):

@@ -589,3 +589,22 @@ def test_given_experts_take_the_routers_weights_for_them():
             truth = truth / (truth.sum(-1, keepdims=True) + 1e-20)
         truth = truth * settings.get("routed_scaling_factor", 1.0)
         assert np.abs(mixed_w[covered] - truth[covered]).max() <= 2 * ROUTER_TOLERANCE
+
+
+def test_media_tokens_are_routed_by_their_own_bias():
+    """`selection` (src/dew/nn/moe.py:516-524): a media token's experts are chosen by scores + media_bias, the others' by
+    scores + bias; the weights stay the unbiased scores'."""
+    rng = np.random.default_rng(15)
+    logits = rng.standard_normal((40, 32)).astype(np.float32)
+    bias, media_bias = (rng.standard_normal(32) * 0.5).astype(np.float32), (rng.standard_normal(32) * 0.5).astype(np.float32)
+    media = rng.integers(0, 2, size=40).astype(bool)
+    settings = dict(score_function="sigmoid", expert_groups=4, groups_per_token=2, routed_scaling_factor=2.5)
+    weights, indices = oracle.route(logits, 4, bias=bias, media=media, media_bias=media_bias, **settings)
+    text_w, text_i = oracle.route(logits, 4, bias=bias, **settings)
+    image_w, image_i = oracle.route(logits, 4, bias=media_bias, **settings)
+    assert np.array_equal(indices, np.where(media[:, None], image_i, text_i))
+    assert np.array_equal(weights, np.where(media[:, None], image_w, text_w))
+    assert not np.array_equal(indices, text_i) and not np.array_equal(indices, image_i)
+    unbiased_w, unbiased_i = oracle.route(logits, 4, media=media, media_bias=media_bias, **settings)      # a router with the media bias alone
+    plain_w, plain_i = oracle.route(logits, 4, **settings)
+    assert np.array_equal(unbiased_i, np.where(media[:, None], image_i, plain_i))
