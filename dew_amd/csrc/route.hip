@@ -2,6 +2,7 @@
 // Follows Router.__call__ from the logits on (reference src/dew/nn/moe.py:466-565). Every floating-point
 // step is a fixed sequence of IEEE fp32/fp64 operations with contraction off, the same sequence the CPU
 // oracle runs, so the chosen experts agree bit for bit.
+#include <algorithm>
 #include <type_traits>
 
 #include "common.h"
@@ -118,7 +119,31 @@ struct RouteParams {
   const uint8_t* covered;  // nullable [T]: with `given`, the tokens it covers; the others keep the router's choice
   const float* media_bias; // nullable [E]: the bias a media token's experts are chosen by, in place of `bias`
   const uint8_t* media;    // nullable [T]: the media tokens
+  // Block routing (`Router.block_mask`, src/dew/nn/moe.py:566-585): tokens are `rows` x `length`, each in the block of its
+  // row that `blocks` numbers (negative: padding, a block of its own); a token chooses among its block's shortlist.
+  const int32_t* blocks;   // nullable [T]
+  int length;              // tokens a row
+  uint32_t* block_keys;    // [rows x (length + 1), E]: a block's best selection for every expert, as ordered keys (0: none yet)
+  const uint8_t* allowed;  // [rows x (length + 1), 64]: bit i of byte `lane` set where expert lane + 64 i is on the block's shortlist
+  int gather_blocks;       // this launch only gathers the blocks' best selections into block_keys
 };
+
+// A float as an unsigned key of the same order (-inf lowest of the non-NaN), never 0.
+__device__ __forceinline__ uint32_t ordered_key(float v) {
+  const uint32_t bits = __float_as_uint(v);
+  return (bits & 0x80000000u) ? ~bits : bits | 0x80000000u;
+}
+
+__device__ __forceinline__ float from_ordered_key(uint32_t key) {
+  if (key == 0u) return -__builtin_inff();  // no token wrote here
+  return __uint_as_float((key & 0x80000000u) ? key & 0x7fffffffu : ~key);
+}
+
+// The block a token routes with: its row's blocks are numbered from 0, padding (or an id past the row) is block `length`.
+__device__ __forceinline__ size_t block_of(const RouteParams& p, int token) {
+  const int id = p.blocks[token];
+  return static_cast<size_t>(token / p.length) * (p.length + 1) + ((id < 0 || id > p.length) ? p.length : id);
+}
 
 // Laguna's capped gate logit (`capped_logits`, src/dew/nn/precision.py:2086-2092): cap * tanh(logit / cap) in fp32.
 __device__ __forceinline__ float capped(float logit, float cap) { return cap > 0.0f ? cap * tanhf(logit / cap) : logit; }
@@ -198,6 +223,24 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
     // A NaN selection (a NaN in the bias or the logits) is never preferred: it competes as -inf, so every round still
     // finds an expert in range (no comparison with NaN holds, and a round without a candidate would name no expert).
     select[i] = (e < p.experts && s == s) ? s : ninf;
+  }
+
+  if (p.blocks != nullptr) {  // (a block router has no expert groups: no barrier lies ahead of the early return)
+    const size_t block = block_of(p, token);
+    if (p.gather_blocks) {
+      if (active) {
+#pragma unroll
+        for (int i = 0; i < kPerLane; ++i) {
+          const int e = lane + kWave * i;
+          if (e < p.experts) atomicMax(p.block_keys + block * p.experts + e, ordered_key(select[i]));
+        }
+      }
+      return;
+    }
+    const unsigned shortlist = p.allowed[block * kWave + lane];
+#pragma unroll
+    for (int i = 0; i < kPerLane; ++i)
+      if (!((shortlist >> i) & 1u)) select[i] = ninf;
   }
 
   if (p.expert_groups > 1) {
@@ -299,6 +342,41 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
   }
 }
 
+// Each block's shortlist: the `count` best of its best selections (ties to the lower index), one wavefront a block.
+__global__ __launch_bounds__(kWave* kRouteWaves) void block_shortlist_kernel(const uint32_t* __restrict__ keys, uint8_t* __restrict__ allowed,
+                                                                             int blocks, int experts, int count) {
+  const int lane = threadIdx.x % kWave;
+  const int block = blockIdx.x * kRouteWaves + threadIdx.x / kWave;
+  if (block >= blocks) return;
+  float best[kMaxPerLane];
+#pragma unroll
+  for (int i = 0; i < kMaxPerLane; ++i) {
+    const int e = lane + kWave * i;
+    best[i] = e < experts ? from_ordered_key(keys[static_cast<size_t>(block) * experts + e]) : -__builtin_inff();
+  }
+  unsigned taken = 0u;
+  for (int round = 0; round < count; ++round) {
+    Best b;
+    b.value = -__builtin_inff();
+    b.index = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) {
+      const int e = lane + kWave * i;
+      if (e < experts && !((taken >> i) & 1u) && better(best[i], e, b)) {
+        b.value = best[i];
+        b.index = e;
+      }
+    }
+    b = wave_best(b);
+    if ((b.index % kWave) == lane) taken |= 1u << (b.index / kWave);
+  }
+  allowed[static_cast<size_t>(block) * kWave + lane] = static_cast<uint8_t>(taken);
+}
+
+__global__ __launch_bounds__(256) void clear_words_kernel(uint32_t* __restrict__ words, size_t count) {
+  for (size_t i = blockIdx.x * 256ull + threadIdx.x; i < count; i += static_cast<size_t>(gridDim.x) * 256) words[i] = 0u;
+}
+
 }  // namespace dew
 
 extern "C" int dew_moe_route(const float* logits, const float* bias, int32_t tokens, int32_t experts,
@@ -323,11 +401,30 @@ extern "C" int dew_moe_route_with(const dew_moe_router* router, const float* log
   return dew_moe_route_call(router, logits, bias, nullptr, nullptr, nullptr, nullptr, tokens, weights, indices, scores, log_z, stream);
 }
 
+namespace dew {
+struct BlockRouting {
+  const int32_t* blocks = nullptr;
+  int length = 0;
+  uint32_t* keys = nullptr;
+  const uint8_t* allowed = nullptr;
+  int gather = 0;
+};
+static int route_launch(const dew_moe_router* router, const float* logits, const float* bias, const float* media_bias,
+                        const uint8_t* media, const int32_t* given, const uint8_t* covered, const BlockRouting& by_block,
+                        int32_t tokens, float* weights, int32_t* indices, float* scores, float* log_z, void* stream);
+}  // namespace dew
+
 extern "C" int dew_moe_route_call(const dew_moe_router* router, const float* logits, const float* bias,
                                   const float* media_bias, const uint8_t* media, const int32_t* given,
                                   const uint8_t* covered, int32_t tokens, float* weights, int32_t* indices, float* scores,
                                   float* log_z, void* stream) {
-  using namespace dew;
+  return dew::route_launch(router, logits, bias, media_bias, media, given, covered, dew::BlockRouting{}, tokens, weights, indices,
+                           scores, log_z, stream);
+}
+
+int dew::route_launch(const dew_moe_router* router, const float* logits, const float* bias, const float* media_bias,
+                             const uint8_t* media, const int32_t* given, const uint8_t* covered, const BlockRouting& by_block,
+                             int32_t tokens, float* weights, int32_t* indices, float* scores, float* log_z, void* stream) {
   DEW_REQUIRE(given || !covered, "dew_moe_route: a coverage without the experts it covers");
   DEW_REQUIRE((media == nullptr) == (media_bias == nullptr), "dew_moe_route: the media tokens and the bias that chooses for them come together");
   DEW_REQUIRE(router, "dew_moe_route: the router's description must not be null");
@@ -364,7 +461,8 @@ extern "C" int dew_moe_route_call(const dew_moe_router* router, const float* log
   RouteParams p{logits, bias, weights, indices, tokens, experts, top_k, score_function, router->normalize ? 1 : 0,
                 expert_groups, groups_per_token, router->group_score == DEW_MOE_GROUP_MAX ? 1 : 0, router->scaling, scores, log_z,
                 router->bias_in_weights ? 1 : 0, router->weight_sum_epsilon, router->weight_sum_min,
-                router->fill_excluded ? 1 : 0, router->excluded_group_score, router->logit_softcap, given, covered, media_bias, media};
+                router->fill_excluded ? 1 : 0, router->excluded_group_score, router->logit_softcap, given, covered, media_bias, media,
+                by_block.blocks, by_block.length, by_block.keys, by_block.allowed, by_block.gather};
   const int blocks = (tokens + kRouteWaves - 1) / kRouteWaves;
   const size_t shared = expert_groups > 1 ? sizeof(float) * kRouteWaves * experts : 0;
   const dim3 grid(blocks), block(kWave * kRouteWaves);
@@ -379,6 +477,48 @@ extern "C" int dew_moe_route_call(const dew_moe_router* router, const float* log
     hipLaunchKernelGGL(route_kernel<kMaxPerLane>, grid, block, shared, s, p);
   }
   return launched("route_kernel");
+}
+
+extern "C" size_t dew_moe_route_blocks_workspace_bytes(int32_t rows, int32_t length, int32_t experts) {
+  if (rows <= 0 || length <= 0 || experts <= 0) return 0;
+  const size_t blocks = static_cast<size_t>(rows) * (static_cast<size_t>(length) + 1);
+  return blocks * experts * sizeof(uint32_t) + blocks * dew::kWave;
+}
+
+extern "C" int dew_moe_route_blocks(const dew_moe_router* router, const float* logits, const float* bias,
+                                    const int32_t* blocks, int32_t rows, int32_t length, int32_t block_experts,
+                                    void* workspace, size_t workspace_bytes, float* weights, int32_t* indices, float* scores,
+                                    float* log_z, void* stream) {
+  using namespace dew;
+  DEW_REQUIRE(router, "dew_moe_route_blocks: the router's description must not be null");
+  DEW_REQUIRE(rows >= 0 && length >= 1 && static_cast<long long>(rows) * length <= 0x7fffffffLL,
+              "dew_moe_route_blocks: %d rows of %d tokens", rows, length);
+  DEW_REQUIRE(router->expert_groups == 1, "dew_moe_route_blocks: block routing limits a token to its block's experts, so it has no expert groups");
+  DEW_REQUIRE(block_experts >= router->top_k && block_experts <= router->experts,
+              "dew_moe_route_blocks: block_experts %d must hold the top_k of %d and at most the %d experts", block_experts,
+              router->top_k, router->experts);
+  if (rows == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(blocks, "dew_moe_route_blocks: the tokens' blocks must not be null");
+  const size_t needed = dew_moe_route_blocks_workspace_bytes(rows, length, router->experts);
+  DEW_REQUIRE(workspace && workspace_bytes >= needed && reinterpret_cast<uintptr_t>(workspace) % 4 == 0,
+              "dew_moe_route_blocks: the workspace holds %zu bytes of the %zu needed (dew_moe_route_blocks_workspace_bytes), 4-byte aligned",
+              workspace ? workspace_bytes : size_t{0}, needed);
+  const int tokens = rows * length;
+  const size_t segments = static_cast<size_t>(rows) * (static_cast<size_t>(length) + 1);
+  const size_t words = segments * router->experts;
+  uint32_t* keys = static_cast<uint32_t*>(workspace);
+  uint8_t* allowed = reinterpret_cast<uint8_t*>(keys + words);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // (a kernel, not a memset: a caller may capture these launches in a graph)
+  hipLaunchKernelGGL(clear_words_kernel, dim3(static_cast<unsigned>(std::min<size_t>((words + 255) / 256, 4096))), dim3(256), 0, s, keys, words);
+  BlockRouting by_block;
+  by_block.blocks = blocks, by_block.length = length, by_block.keys = keys, by_block.allowed = allowed, by_block.gather = 1;
+  int status = route_launch(router, logits, bias, nullptr, nullptr, nullptr, nullptr, by_block, tokens, weights, indices, nullptr, nullptr, stream);
+  if (status != DEW_MOE_OK) return status;
+  hipLaunchKernelGGL(block_shortlist_kernel, dim3(static_cast<unsigned>((segments + kRouteWaves - 1) / kRouteWaves)), dim3(kWave * kRouteWaves),
+                     0, s, keys, allowed, static_cast<int>(segments), router->experts, block_experts);
+  by_block.gather = 0;
+  return route_launch(router, logits, bias, nullptr, nullptr, nullptr, nullptr, by_block, tokens, weights, indices, scores, log_z, stream);
 }
 
 namespace dew {

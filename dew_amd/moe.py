@@ -162,6 +162,10 @@ class Router(_Module):
     """What an expert outside a token's best groups is chosen by: None for never (DeepSeek V3's -inf), or A.X-K2's 0.0."""
     logit_softcap: float | None = None
     """Laguna's cap `c` on each gate logit, `c * tanh(logit / c)`, before the scores and the z-loss read it."""
+    routing_block: int | None = None
+    block_experts: int | None = None
+    """LLaDA2.2's block routing: the caller numbers each token's block of `routing_block` places (`blocks`), and a token
+    chooses among the `block_experts` experts its block scores best, a block's score its best token's."""
     media_bias: bool = False
     """DeepSeek-V4.1's second bias (`moe/<path>/media_bias`), choosing for the image-span tokens the `media` mask marks in
     place of `expert_bias`."""
@@ -174,8 +178,18 @@ class Router(_Module):
             raise ValueError("bias_in_weights gates on the balancing bias, which expert_bias holds")
         if self.logit_softcap is not None and not self.logit_softcap > 0:
             raise ValueError(f"logit_softcap is a positive cap on the gate logits, or None for none; got {self.logit_softcap}")
-        if self.hash_vocab is not None and (self.expert_bias or self.expert_groups > 1):
-            raise ValueError("hash routing selects by the token table alone, so it has no balancing bias and no expert groups")
+        if self.hash_vocab is not None and (self.expert_bias or self.expert_groups > 1 or self.routing_block is not None):
+            raise ValueError("hash routing selects by the token table alone, so it has no balancing bias, no expert groups and no routing blocks")
+        if (self.routing_block is None) != (self.block_experts is None):
+            raise ValueError("block routing names its block of tokens and the experts a block may use, "
+                             f"got routing_block={self.routing_block} and block_experts={self.block_experts}")
+        if self.routing_block is not None:
+            if self.routing_block < 1:
+                raise ValueError(f"routing_block counts a block's tokens, got {self.routing_block}")
+            if not self.top_k <= self.block_experts <= self.num_experts:
+                raise ValueError(f"block_experts must hold the top_k of {self.top_k} and at most the {self.num_experts} experts, got {self.block_experts}")
+            if self.expert_groups > 1:
+                raise ValueError("block routing limits a token to its block's experts, so it has no expert groups")
         if self.score_function not in ("softmax", "sigmoid", "sqrtsoftplus"):
             raise ValueError(f"score_function {self.score_function!r}: the router scores by 'softmax', 'sigmoid' or 'sqrtsoftplus'")
         if self.group_score not in ("top2", "max"):
@@ -246,11 +260,37 @@ class Router(_Module):
                 given = torch.where(covers.to(torch.bool)[..., None], replayed, given).contiguous()
         return given, covered
 
-    def __call__(self, x, tokens=None, media=None, routes=None, blocks=None):
+    def routed_by_blocks(self, logits: torch.Tensor, blocks: torch.Tensor, sown: dict | None = None):
+        """`routed` of a block router (`routing_block`): `logits [rows, length, E]`, `blocks [rows, length]`."""
+        bias = _at(self.variables.get("moe"), (*self.path, "e_score_correction_bias")) if self.expert_bias else None
+        if self.expert_bias and bias is None:
+            raise KeyError(f"no moe/{'/'.join(self.path)}/e_score_correction_bias")
+        if logits.dim() == 2:
+            logits = logits[None]
+        found = ops.route_blocks(logits.contiguous(), self.top_k, torch.broadcast_to(blocks.to(torch.int32), logits.shape[:-1]).contiguous(),
+                                 self.block_experts, score_function=self.score_function, normalize_weights=self.normalize_weights,
+                                 bias=bias, routed_scaling_factor=self.routed_scaling_factor, sown=sown is not None,
+                                 bias_in_weights=self.bias_in_weights, weight_sum_epsilon=self.weight_sum_epsilon,
+                                 weight_sum_min=self.weight_sum_min, logit_softcap=self.logit_softcap)
+        if sown is not None:
+            sown.update(indices=found[1], scores=found[2], log_z=found[3])
+        return found[0], found[1]
+
+    def chosen(self, logits: torch.Tensor, tokens=None, media=None, routes=None, blocks=None):
+        """(weights, indices) of `logits [..., E]` under the per-token inputs of `__call__` (src/dew/nn/moe.py:466-524)."""
+        if (blocks is None) != (self.routing_block is None):
+            raise ValueError("a block router chooses each block's experts together, from the blocks its caller numbers, "
+                             "and only a block router reads them")
         if blocks is not None:
-            raise ValueError("block routing is not part of the HIP router")
-        given, covered = self.given_experts((*x.shape[:-1], self.top_k), tokens, routes)
-        return self.routed(self.logits(x), given=given, covered=covered, media=media)
+            if media is not None or routes is not None:
+                raise ValueError("a replayed record or a media mask over block routing is not part of the HIP router")
+            weights, indices = self.routed_by_blocks(logits.reshape(-1, *logits.shape[-2:]), blocks.reshape(-1, blocks.shape[-1]))
+            return weights.reshape(*logits.shape[:-1], self.top_k), indices.reshape(*logits.shape[:-1], self.top_k)
+        given, covered = self.given_experts((*logits.shape[:-1], self.top_k), tokens, routes)
+        return self.routed(logits, given=given, covered=covered, media=media)
+
+    def __call__(self, x, tokens=None, media=None, routes=None, blocks=None):
+        return self.chosen(self.logits(x), tokens, media, routes, blocks)
 
 
 def load_balance_update(counts: torch.Tensor, rate: float) -> torch.Tensor:
@@ -456,6 +496,8 @@ class SparseMLP(_Module):
     excluded_group_score: float | None = None
     hash_vocab: int | None = None
     media_bias: bool = False
+    routing_block: int | None = None
+    block_experts: int | None = None
     router_softcap: float | None = None
     """The router's switches (`Router`'s fields of the same names; `router_softcap` is its `logit_softcap`,
     src/dew/nn/moe.py:1440-1446)."""
@@ -465,7 +507,7 @@ class SparseMLP(_Module):
         return Router(self.num_experts, self.out_features, self.top_k, self.score_function, self.normalize_weights,
                       self.routed_scaling_factor, self.expert_groups, self.groups_per_token, self.group_score,
                       self.expert_bias, self.bias_in_weights, self.weight_sum_epsilon, self.weight_sum_min,
-                      self.excluded_group_score, self.router_softcap, self.media_bias, self.hash_vocab)._bound(self.variables, (*self.path, "gate"))
+                      self.excluded_group_score, self.router_softcap, self.routing_block, self.block_experts, self.media_bias, self.hash_vocab)._bound(self.variables, (*self.path, "gate"))
 
     @property
     def experts(self) -> ExpertMLP:
@@ -485,10 +527,7 @@ class SparseMLP(_Module):
         if logits is None:
             weights, indices = gate(x, tokens, media, routes, blocks)
         else:
-            if blocks is not None:
-                raise ValueError("block routing is not part of the HIP router")
-            given, covered = gate.given_experts((*x.shape[:-1], self.top_k), tokens, routes)
-            weights, indices = gate.routed(logits, given=given, covered=covered, media=media)
+            weights, indices = gate.chosen(logits, tokens, media, routes, blocks)
         # routed + shared (src/dew/nn/moe.py:1497-1503): the bf16 add runs in the combine kernel's epilogue. A shared
         # expert of the routed experts' width and format is multiplied by the routed launches, as their group #E.
         experts = self.experts

@@ -96,6 +96,39 @@ def route(logits: torch.Tensor, top_k: int, *, score_function: str = "softmax", 
     return (weights, indices, activated, log_z) if sown else (weights, indices)
 
 
+def route_blocks(logits: torch.Tensor, top_k: int, blocks: torch.Tensor, block_experts: int, *, score_function: str = "softmax",
+                 normalize_weights: bool = True, bias: torch.Tensor | None = None, routed_scaling_factor: float = 1.0,
+                 sown: bool = False, bias_in_weights: bool = False, weight_sum_epsilon: float = WEIGHT_SUM_EPSILON,
+                 weight_sum_min: float = 0.0, logit_softcap: float | None = None):
+    """`route` under LLaDA2.2's block routing: `logits [rows, length, E]`, `blocks [rows, length]` int32 numbering each
+    token's block within its row from 0 (negative: padding); a token chooses among the `block_experts` experts its block
+    scores best, a block's score for an expert being its best token's selection (the reference's `Router.block_mask`)."""
+    scores = {"softmax": _lib.SCORE_SOFTMAX, "sigmoid": _lib.SCORE_SIGMOID, "sqrtsoftplus": _lib.SCORE_SQRTSOFTPLUS}
+    if score_function not in scores:
+        raise KernelError(f"score_function must be one of {list(scores)}, got {score_function!r}")
+    _device(logits, "logits", torch.float32), _device(blocks, "blocks", torch.int32)
+    if logits.dim() != 3 or blocks.shape != logits.shape[:2]:
+        raise KernelError(f"block routing takes logits [rows, length, E] and blocks [rows, length], got {tuple(logits.shape)} and {tuple(blocks.shape)}")
+    if bias is not None:
+        _device(bias, "bias", torch.float32)
+        if bias.shape != logits.shape[-1:]:
+            raise KernelError(f"bias {tuple(bias.shape)} does not match {logits.shape[-1]} experts")
+    rows, length, experts = logits.shape
+    weights = torch.empty((rows, length, top_k), dtype=torch.float32, device=logits.device)
+    indices = torch.empty((rows, length, top_k), dtype=torch.int32, device=logits.device)
+    activated = torch.empty_like(logits) if sown else None
+    log_z = torch.empty((rows, length), dtype=torch.float32, device=logits.device) if sown else None
+    router = _lib.Router(experts, top_k, scores[score_function], int(bool(normalize_weights)), float(routed_scaling_factor), 1, 1,
+                         _lib.GROUP_TOP2, int(bool(bias_in_weights)), float(weight_sum_epsilon), float(weight_sum_min), 0, 0.0,
+                         float(logit_softcap or 0.0))
+    library = _lib.library()
+    workspace = torch.empty(max(library.dew_moe_route_blocks_workspace_bytes(rows, length, experts), 4) // 4 + 1, dtype=torch.int32, device=logits.device)
+    _lib.check(library.dew_moe_route_blocks(router, _ptr(logits), _ptr(bias), _ptr(blocks), rows, length, block_experts, _ptr(workspace),
+                                            workspace.numel() * 4, _ptr(weights), _ptr(indices), _ptr(activated), _ptr(log_z), _stream()),
+               "dew_moe_route_blocks")
+    return (weights, indices, activated, log_z) if sown else (weights, indices)
+
+
 def capacity_admitted(indices: torch.Tensor, num_experts: int, capacity_factor: float) -> torch.Tensor:
     """`indices [..., length, k]` with every slot past its expert's queue in its sequence replaced by the sentinel id
     `num_experts` (the reference's `capacity_positions` and the drop it decides, src/dew/nn/moe.py:832-855, 914-919);

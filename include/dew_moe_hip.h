@@ -135,6 +135,19 @@ int dew_moe_route_call(const dew_moe_router* router /* host */, const float* log
                        const int32_t* given /* nullable [T,k] */, const uint8_t* covered /* nullable [T] */,
                        int32_t tokens, float* weights, int32_t* indices, float* scores, float* log_z, void* stream);
 
+/* LLaDA2.2's block routing (`routing_block` / `block_experts`, `Router.block_mask` src/dew/nn/moe.py:566-585, applied in
+ * `selection` :516-524): the tokens are `rows` x `length`; blocks[t] numbers token t's block within its row from 0 (the
+ * reference's `numbered_blocks`, src/dew/nn/inputs.py:462-476), negative for padding, which is a block of its own. A block's
+ * score for an expert is its best token's selection (scores + bias); a token chooses its top_k among the `block_experts`
+ * best of its block (ties to the lower index). Three launches and a clearing one on `stream`; the workspace
+ * (dew_moe_route_blocks_workspace_bytes: a key per block and expert, a shortlist per block) is the caller's, no allocation
+ * here. The router has no expert groups.                                                                                  */
+size_t dew_moe_route_blocks_workspace_bytes(int32_t rows, int32_t length, int32_t experts);
+int dew_moe_route_blocks(const dew_moe_router* router /* host */, const float* logits /* [rows * length, E] */,
+                         const float* bias /* nullable */, const int32_t* blocks /* [rows * length] */, int32_t rows,
+                         int32_t length, int32_t block_experts, void* workspace, size_t workspace_bytes, float* weights,
+                         int32_t* indices, float* scores /* nullable */, float* log_z /* nullable */, void* stream);
+
 /* The aux-loss-free balancing step (`load_balance_update` src/dew/nn/moe.py:271-300, applied to the selection bias as
  * `_updated_bias` src/dew/objectives/routing.py:342-345): bias[e] += rate * direction, direction -1 where counts[e]
  * is above floor(sum / E), +1 where below it or equal with a remainder, else 0. counts = dew_moe_permute's sizes. */

@@ -49,6 +49,10 @@ What pins each function (tests/test_oracle_golden.py):
   the others by their definitions in float64 (the biased scores gathered; the sums floored, with the tokens below the
   floor summing to sum / floor and the rest to one; `cap * tanh(x / cap)`, bounded, order-preserving), each of which a
   dropped bias, a floor applied before the epsilon or a cap applied after the scores fails.
+* `block_mask` / `route(blocks=, block_experts=)` (LLaDA2.2's block routing): no vectors in the reference; the function is
+  the definition's own loops (a block's best selection per expert, its `block_experts` best), checked against a hand case,
+  against blocks of one token (where the mask is each token's own top `block_experts`), against one block a row with
+  `block_experts = E` (no limit) and against a relabelling of the blocks (which changes nothing).
 * `route(media=, media_bias=)` (DeepSeek-V4.1's image-span bias): by the definition: the media tokens route as a router
   whose bias is `media_bias` routes them, the others as one whose bias is `bias`, row for row.
 * `route(given=, covered=)` (replayed routes and the hash router's table rows, `chosen_experts` src/dew/nn/moe.py:202-224):
@@ -348,8 +352,24 @@ def capped_logits(logits, softcap):
     return (cap * np.tanh((logits / cap).astype(F32)).astype(F32)).astype(F32)
 
 
+def block_mask(selection, blocks, experts):
+    """`Router.block_mask` (src/dew/nn/moe.py:566-585): True where an expert is one of the `experts` best of its token's
+    block, a block's score for an expert its best token's selection; `selection [rows, length, E]`, `blocks [rows, length]`
+    numbering each row's blocks from 0, a negative id (padding) a block of its own. Written as the definition's loops."""
+    selection, blocks = np.asarray(selection, F32), np.asarray(blocks)
+    kept = np.zeros(selection.shape, bool)
+    for row in range(selection.shape[0]):
+        ids = np.where(blocks[row] < 0, -1, blocks[row])
+        for block in np.unique(ids):
+            members = np.flatnonzero(ids == block)
+            best = selection[row, members].max(axis=0)
+            _, allowed = top_k(best, experts)
+            kept[np.ix_([row], members, allowed)] = True
+    return kept
+
+
 def selection_scores(logits, *, score_function="softmax", bias=None, expert_groups=1, groups_per_token=1, group_score="top2",
-                     excluded_group_score=None, media=None, media_bias=None):
+                     excluded_group_score=None, media=None, media_bias=None, blocks=None, block_experts=None):
     """(scores, selection) of `Router.__call__` (src/dew/nn/moe.py:466-470, 516-524): the activated scores and what the
     top-k runs over, the scores plus the bias with the experts outside a token's best groups at -inf, or at
     `excluded_group_score` where the router fills one in (:496-565)."""
@@ -366,6 +386,8 @@ def selection_scores(logits, *, score_function="softmax", bias=None, expert_grou
     selection = scores if bias is None else (scores + np.asarray(bias, F32)).astype(F32)
     if media is not None:      # a media token's own bias (`selection`, src/dew/nn/moe.py:516-524)
         selection = np.where(np.asarray(media, bool)[..., None], (scores + np.asarray(media_bias, F32)).astype(F32), selection)
+    if blocks is not None:     # outside each block's shortlist -inf (`selection`, src/dew/nn/moe.py:522-523)
+        selection = np.where(block_mask(np.where(np.isnan(selection), F32(-np.inf), selection), blocks, block_experts), selection, F32(-np.inf))
     # A NaN selection competes as -inf (the HIP router's rule): none of the reference's tests feeds its `lax.top_k` a
     # NaN, so this is a choice of this restatement, made so that every choice stays an expert in range.
     selection = np.where(np.isnan(selection), F32(-np.inf), selection)
@@ -403,7 +425,7 @@ def top_k_margin(selection, top_k_count):
 def route(logits, top_k_count, *, score_function="softmax", normalize_weights=True, bias=None,
           routed_scaling_factor=1.0, expert_groups=1, groups_per_token=1, group_score="top2",
           weight_sum_epsilon=1e-20, weight_sum_min=0.0, bias_in_weights=False, excluded_group_score=None,
-          logit_softcap=None, given=None, covered=None, media=None, media_bias=None):
+          logit_softcap=None, given=None, covered=None, media=None, media_bias=None, blocks=None, block_experts=None):
     """`Router.__call__` from its logits on (src/dew/nn/moe.py:466-494): the cap on the logits (:526-534), scores,
     selection (bias, group-limited mask :496-565), top-k, weights (:483-494: a softmax router renormalizes the chosen
     logits unless `bias_in_weights` or `weight_sum_min` say otherwise; else the chosen scores, plus the bias under
@@ -412,7 +434,8 @@ def route(logits, top_k_count, *, score_function="softmax", normalize_weights=Tr
     logits = capped_logits(logits, logit_softcap)
     scores, selection = selection_scores(logits, score_function=score_function, bias=bias, expert_groups=expert_groups,
                                          groups_per_token=groups_per_token, group_score=group_score,
-                                         excluded_group_score=excluded_group_score, media=media, media_bias=media_bias)
+                                         excluded_group_score=excluded_group_score, media=media, media_bias=media_bias,
+                                         blocks=blocks, block_experts=block_experts)
     _, indices = top_k(selection, top_k_count)
     if given is not None:      # `chosen_experts` (src/dew/nn/moe.py:202-224): a replayed record, or the hash table's rows (:500-507)
         given = np.asarray(given).astype(np.int32)

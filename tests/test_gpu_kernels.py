@@ -177,6 +177,42 @@ def test_media_tokens_are_chosen_for_by_the_media_bias(ops, experts, k, groups, 
         ops.route(torch.from_numpy(logits).cuda(), k, media=torch.from_numpy(media).cuda(), **settings)
 
 
+@pytest.mark.parametrize("score_function,experts,k,allowed,rows,length,block,biased",
+                         [("sigmoid", 64, 4, 8, 3, 50, 8, True), ("softmax", 256, 8, 16, 2, 129, 32, False),
+                          ("sigmoid", 128, 6, 6, 5, 17, 4, True), ("sqrtsoftplus", 32, 2, 32, 1, 64, 16, False),
+                          ("softmax", 8, 2, 3, 4, 9, 1, True), ("sigmoid", 512, 8, 24, 1, 40, 8, False)])
+def test_block_routing_chooses_within_each_blocks_shortlist(ops, score_function, experts, k, allowed, rows, length, block, biased):
+    """LLaDA2.2's block routing (`dew_moe_route_blocks`) against the oracle's `block_mask`, bit for bit: whole and partial
+    blocks, padding inside and behind a row (a block of its own), a shortlist as short as the top-k and as long as the
+    experts, and the `Router` mirror's `blocks` argument."""
+    from dew_amd import moe
+    rng = np.random.default_rng(experts + length)
+    logits = (rng.standard_normal((rows, length, experts)) * 1.5).astype(np.float32)
+    bias = (rng.standard_normal(experts) * 0.2).astype(np.float32) if biased else None
+    blocks = np.tile(np.arange(length) // block, (rows, 1)).astype(np.int32)
+    blocks[0, length - 3:] = -1                       # padding behind the row
+    if rows > 1:
+        blocks[1, 2] = -1                             # ... and inside one
+    settings = dict(score_function=score_function, routed_scaling_factor=1.5)
+    want_w, want_i = oracle.route(logits, k, bias=bias, blocks=blocks, block_experts=allowed, **settings)
+    got_w, got_i = ops.route_blocks(torch.from_numpy(logits).cuda(), k, torch.from_numpy(blocks).cuda(), allowed,
+                                    bias=None if bias is None else torch.from_numpy(bias).cuda(), **settings)
+    assert np.array_equal(got_i.cpu().numpy(), want_i)
+    assert np.array_equal(got_w.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
+    if allowed < experts:
+        assert not np.array_equal(want_i, oracle.route(logits, k, bias=bias, **settings)[1])
+    variables = {"params": {}, "moe": {} if bias is None else {"e_score_correction_bias": torch.from_numpy(bias).cuda()}}
+    router = moe.Router(experts, 128, k, expert_bias=biased, routing_block=block, block_experts=allowed, **settings)._bound(variables, ())
+    mirror_w, mirror_i = router.chosen(torch.from_numpy(logits).cuda(), blocks=torch.from_numpy(blocks).cuda())
+    assert torch.equal(mirror_i, got_i) and torch.equal(mirror_w, got_w)
+    with pytest.raises(ValueError, match="only a block router reads them"):
+        moe.Router(experts, 128, k, **settings)._bound(variables, ()).chosen(torch.from_numpy(logits).cuda(), blocks=torch.from_numpy(blocks).cuda())
+    with pytest.raises(ValueError, match="from the blocks its caller numbers"):
+        router.chosen(torch.from_numpy(logits).cuda())
+    with pytest.raises(ops.KernelError, match="block_experts"):
+        ops.route_blocks(torch.from_numpy(logits).cuda(), k, torch.from_numpy(blocks).cuda(), k - 1, **settings)
+
+
 def test_a_hash_router_takes_its_experts_from_the_token_table(ops):
     """DeepSeek V4's hash router (`hash_vocab`, src/dew/nn/moe.py:337-341, 500-507): the experts are `tid2eid[token id]`,
     weighted by the learned gate; a replayed record covers some tokens over it; only a hash router reads token ids."""

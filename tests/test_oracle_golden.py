@@ -608,3 +608,34 @@ def test_media_tokens_are_routed_by_their_own_bias():
     unbiased_w, unbiased_i = oracle.route(logits, 4, media=media, media_bias=media_bias, **settings)      # a router with the media bias alone
     plain_w, plain_i = oracle.route(logits, 4, **settings)
     assert np.array_equal(unbiased_i, np.where(media[:, None], image_i, plain_i))
+
+
+def test_block_routing_limits_a_token_to_its_blocks_best_experts():
+    """`Router.block_mask` (src/dew/nn/moe.py:566-585): a hand case; blocks of one token (each token's own best); one
+    block a row with every expert allowed (no limit); a relabelling of the blocks; padding as a block of its own."""
+    selection = np.array([[[0.9, 0.1, 0.5, 0.2],       # block 0: best per expert over its two tokens = [0.9, 0.8, 0.5, 0.2]
+                           [0.3, 0.8, 0.4, 0.1],
+                           [0.1, 0.2, 0.3, 0.4],       # block 1 alone: best two are experts 3, 2
+                           [0.7, 0.6, 0.1, 0.0]]], np.float32)   # padding: a block of its own, best two 0, 1
+    mask = oracle.block_mask(selection, np.array([[0, 0, 1, -1]]), 2)
+    assert np.array_equal(mask[0], np.array([[1, 1, 0, 0], [1, 1, 0, 0], [0, 0, 1, 1], [1, 1, 0, 0]], bool))
+    rng = np.random.default_rng(16)
+    logits = rng.standard_normal((3, 24, 16)).astype(np.float32)
+    alone = np.tile(np.arange(24), (3, 1))
+    _, selection = oracle.selection_scores(logits, score_function="sigmoid")
+    mask = oracle.block_mask(selection, alone, 5)
+    assert np.array_equal(mask, selection >= -np.sort(-selection, axis=-1)[..., 4:5])
+    for settings in (dict(score_function="sigmoid"), dict(score_function="softmax", normalize_weights=False)):
+        free_w, free_i = oracle.route(logits, 3, **settings)
+        whole_w, whole_i = oracle.route(logits, 3, blocks=np.zeros((3, 24), np.int64), block_experts=16, **settings)
+        assert np.array_equal(whole_i, free_i) and np.array_equal(whole_w, free_w)
+        blocks = np.tile(np.arange(24) // 4, (3, 1))
+        blocks[1, 20:] = -1
+        weights, indices = oracle.route(logits, 3, blocks=blocks, block_experts=4, **settings)
+        assert not np.array_equal(indices, free_i)
+        relabelled = np.where(blocks < 0, -1, 5 - blocks)
+        again_w, again_i = oracle.route(logits, 3, blocks=relabelled, block_experts=4, **settings)
+        assert np.array_equal(again_i, indices) and np.array_equal(again_w, weights)
+        for row in range(3):                       # every block uses at most block_experts experts, and the same shortlist
+            for block in np.unique(blocks[row]):
+                assert np.unique(indices[row, blocks[row] == block]).size <= 4
