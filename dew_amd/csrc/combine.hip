@@ -100,6 +100,36 @@ __global__ __launch_bounds__(256) void scale_rows_kernel(const bf16_t* __restric
   }
 }
 
+// Qwen2-MoE's gate on the shared expert (`shared_gate`, src/dew/nn/moe.py:1497-1503: `shared * logistic(Dense(1)(x))` in
+// the compute dtype): one wavefront a token forms the gate's logit, the fp32 sum of the token times the gate's kernel
+// (each rounded to bf16, as the layer's promotion casts it), rounded to bf16; its logistic, rounded to bf16; and the
+// token's row of the shared expert's output times it, each product rounded once.
+__global__ __launch_bounds__(256) void gate_rows_kernel(const bf16_t* __restrict__ x, const float* __restrict__ kernel,
+                                                        const bf16_t* rows_in, bf16_t* out /* may be rows_in */, int tokens,
+                                                        int depth, int width) {
+  const int lane = threadIdx.x % 64;
+  const int token = blockIdx.x * 4 + threadIdx.x / 64;
+  if (token >= tokens) return;
+  float sum = 0.0f;
+  for (int chunk = lane; chunk < depth / 8; chunk += 64) {
+    const Bf16x8 values = *reinterpret_cast<const Bf16x8*>(x + static_cast<size_t>(token) * depth + static_cast<size_t>(chunk) * 8);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sum += bf16_to_f32(values.v[i]) * bf16_round(kernel[chunk * 8 + i]);
+  }
+#pragma unroll
+  for (int offset = 32; offset >= 1; offset >>= 1) sum += __shfl_xor(sum, offset, 64);
+  const float logit = bf16_round(sum);
+  const float gate = bf16_round(1.0f / (1.0f + expf(-logit)));
+  for (int chunk = lane; chunk < width / 8; chunk += 64) {
+    const size_t at = static_cast<size_t>(token) * width + static_cast<size_t>(chunk) * 8;
+    const Bf16x8 values = *reinterpret_cast<const Bf16x8*>(rows_in + at);
+    Bf16x8 gated;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) gated.v[i] = f32_to_bf16(bf16_to_f32(values.v[i]) * gate);
+    *reinterpret_cast<Bf16x8*>(out + at) = gated;
+  }
+}
+
 // `limit` > 0: the gate clamped from above and the up projection both ways before their product (`swiglu_clamped`,
 // src/dew/nn/activations.py:327-333); the limit enters as the bf16 the operands' dtype rounds it to.
 __global__ __launch_bounds__(256) void swiglu_kernel(const bf16_t* __restrict__ gate, const bf16_t* __restrict__ up,
@@ -170,6 +200,19 @@ extern "C" int dew_moe_scale_rows(const void* x, const int32_t* gather, const in
   hipLaunchKernelGGL(scale_rows_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<const bf16_t*>(x), gather,
                      slots, weights, static_cast<bf16_t*>(out), rows, depth);
   return launched("scale_rows_kernel");
+}
+
+extern "C" int dew_moe_gate_rows(const void* x, const float* kernel, const void* rows_in, void* out, int32_t tokens, int32_t depth,
+                                 int32_t width, void* stream) {
+  using namespace dew;
+  DEW_REQUIRE(tokens >= 0 && depth > 0 && depth % 8 == 0 && width > 0 && width % 8 == 0,
+              "dew_moe_gate_rows: tokens %d, depth %d and width %d (whole 8s)", tokens, depth, width);
+  if (tokens == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(x && kernel && rows_in && out, "dew_moe_gate_rows: x, kernel, rows and out must not be null");
+  DEW_REQUIRE(aligned16(x) && aligned16(rows_in) && aligned16(out), "dew_moe_gate_rows: x, rows and out must be 16-byte aligned");
+  hipLaunchKernelGGL(gate_rows_kernel, dim3((tokens + 3) / 4), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<const bf16_t*>(x),
+                     kernel, static_cast<const bf16_t*>(rows_in), static_cast<bf16_t*>(out), tokens, depth, width);
+  return launched("gate_rows_kernel");
 }
 
 extern "C" int dew_moe_swiglu(const void* gate, const void* up, void* hidden, int64_t count, void* stream) {

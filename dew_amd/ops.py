@@ -504,6 +504,20 @@ def silu(x: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def gate_rows(x: torch.Tensor, kernel: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+    """`rows [T, W]` (bf16) with each token's row times its gate, `bf16(logistic(bf16(x[t] . bf16(kernel))))`: the
+    reference's `shared_gate` on a shared expert's output under a bf16 compute dtype. `kernel` is the gate's fp32 `[D]`
+    (or `[D, 1]`) parameter."""
+    _device(x, "x", torch.bfloat16), _device(kernel, "kernel", torch.float32), _device(rows, "rows", torch.bfloat16)
+    if x.dim() != 2 or rows.dim() != 2 or rows.shape[0] != x.shape[0] or kernel.numel() != x.shape[1]:
+        raise KernelError(f"gate_rows takes x [T, D], a kernel of D values and rows [T, W], got {tuple(x.shape)}, {tuple(kernel.shape)} "
+                          f"and {tuple(rows.shape)}")
+    out = torch.empty_like(rows)
+    _lib.check(_lib.library().dew_moe_gate_rows(_ptr(x), _ptr(kernel), _ptr(rows), _ptr(out), x.shape[0], x.shape[1], rows.shape[1],
+                                                _stream()), "dew_moe_gate_rows")
+    return out
+
+
 def relu2(x: torch.Tensor) -> torch.Tensor:
     """`bf16(max(x, 0)^2)`: the squared ReLU of Nemotron-H's ungated experts (the reference's `relu2`)."""
     _device(x, "x", torch.bfloat16)

@@ -475,6 +475,12 @@ int dew_moe_gateup_gated(const void* x, const int32_t* gather, const int32_t* of
  * gather and the combine sums the slots unweighted (weights of one).                                              */
 int dew_moe_scale_rows(const void* x /* bf16 [T,D] */, const int32_t* gather, const int32_t* slots, const float* weights,
                        void* out /* bf16 [rows,D] */, int32_t rows, int32_t depth, void* stream);
+/* Qwen2-MoE's gate on the shared expert (`shared_gate`, src/dew/nn/moe.py:1469-1475, 1497-1503, under a bf16 compute
+ * dtype): out[t, :] = bf16(rows[t, :] * g[t]), g[t] = bf16(logistic(bf16(sum_d x[t, d] * bf16(kernel[d])))), the sum in
+ * fp32. rows and out may be the same buffer.                                                                          */
+int dew_moe_gate_rows(const void* x /* bf16 [T,D] */, const float* kernel /* [D] */, const void* rows /* bf16 [T,W] */,
+                      void* out /* bf16 [T,W] */, int32_t tokens, int32_t depth, int32_t width, void* stream);
+
 /* Nemotron-H's ungated experts (`activation='relu2'`, src/dew/nn/moe.py:1250-1252, 1319-1322: up_proj, squared ReLU,
  * down_proj): out = bf16(max(x, 0)^2) (`relu2`, src/dew/nn/activations.py:109-111), between two dew_moe_grouped_gemm launches. */
 int dew_moe_relu2(const void* x /* bf16 [count] */, void* out /* bf16 [count] */, int64_t count, void* stream);

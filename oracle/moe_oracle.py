@@ -53,6 +53,9 @@ What pins each function (tests/test_oracle_golden.py):
   the definition's own loops (a block's best selection per expert, its `block_experts` best), checked against a hand case,
   against blocks of one token (where the mask is each token's own top `block_experts`), against one block a row with
   `block_experts = E` (no limit) and against a relabelling of the blocks (which changes nothing).
+* `gated_rows` (`shared_gate`, Qwen2-MoE's scalar gate on the shared expert): no vectors in the reference. The dtype flow
+  is read from the reference's sources (the gate's Dense under `dtype=bf16`; `logistic`'s one rounding); the arithmetic
+  is pinned by a hand case whose three roundings each move the result, and by float64 `sigmoid(x . w) * rows` within bf16.
 * `route(media=, media_bias=)` (DeepSeek-V4.1's image-span bias): by the definition: the media tokens route as a router
   whose bias is `media_bias` routes them, the others as one whose bias is `bias`, row for row.
 * `route(given=, covered=)` (replayed routes and the hash router's table rows, `chosen_experts` src/dew/nn/moe.py:202-224):
@@ -1139,8 +1142,20 @@ def gated_mlp(x, gate_w, up_w, down_w, *, dtype="bfloat16"):
     return grouped_matmul(swiglu(gate, up, dtype=dtype), np.asarray(down_w)[None], sizes, dtype=dtype)
 
 
+def gated_rows(x, kernel, rows):
+    """`shared * logistic(shared_expert_gate(x))` (src/dew/nn/moe.py:1469-1475, 1499-1502) under a bf16 compute dtype: the
+    gate's `Dense(1)` promotes its fp32 kernel to bf16 (flax's `promote_dtype` under `dtype`), multiplies bf16 operands
+    with an fp32 sum and returns bf16; the logistic is formed in fp32 and rounded once to bf16
+    (src/dew/nn/activations.py:85-98); the bf16 product with the shared expert's output is rounded once."""
+    x = np.asarray(x, F32)
+    kernel = bf16_round(np.asarray(kernel, F32).reshape(-1))
+    logit = bf16_round((x.astype(np.float64) @ kernel.astype(np.float64)).astype(F32))
+    gate = bf16_round((1.0 / (1.0 + np.exp(-logit.astype(np.float64)))).astype(F32))
+    return bf16_round((np.asarray(rows, F32) * gate[:, None]).astype(F32))
+
+
 def sparse_mlp(x, logits, gate_w, up_w, down_w, *, top_k_count, dtype="bfloat16", shared=None,
-               factors=(None, None, None), limit=None, scale_inputs=False, **router):
+               factors=(None, None, None), limit=None, scale_inputs=False, shared_gate=None, **router):
     """`SparseMLP.__call__` (src/dew/nn/moe.py:1488-1503) from the router logits on: route, routed
     experts, plus the shared expert's output (`shared` = its three dense matrices)."""
     weights, indices = route(logits, top_k_count, **router)
@@ -1148,7 +1163,10 @@ def sparse_mlp(x, logits, gate_w, up_w, down_w, *, top_k_count, dtype="bfloat16"
                                limit=limit, scale_inputs=scale_inputs)
     trace.update(weights=weights, indices=indices)
     if shared is not None:
-        both = routed + gated_mlp(x, *shared, dtype=dtype)
+        apart = gated_mlp(x, *shared, dtype=dtype)
+        if shared_gate is not None:      # Qwen2-MoE's scalar gate on the shared expert (bf16 compute dtype)
+            apart = gated_rows(x, shared_gate, apart)
+        both = routed + apart
         routed = bf16_round(both) if dtype == "bfloat16" else both.astype(F32)
     return routed, trace
 

@@ -516,3 +516,46 @@ def test_the_layers_router_softcap_is_its_routers_logit_softcap():
         moe.Router(8, 128, 2, logit_softcap=0.0)
     with pytest.raises(ValueError, match="expert_bias holds"):
         moe.Router(8, 128, 2, bias_in_weights=True)
+
+
+@pytest.mark.parametrize("fuse_shared", [True, False])
+def test_qwen2_moes_gate_on_the_shared_expert(fuse_shared):
+    """`shared_gate` (src/dew/nn/moe.py:1469-1475, 1499-1502) under the bf16 compute dtype: the kernel alone against the
+    oracle (the logit's fp32 sum runs in another order, so a gate may sit one bf16 ulp away: at most 2^-7 of a row's
+    values, rarely), the oracle's hand case on the device, and the whole layer with the shared expert inside the routed
+    launches and beside them."""
+    import dataclasses
+
+    from dew_amd import ops
+    rng = np.random.default_rng(41)
+    x = torch.from_numpy(rng.standard_normal((333, 512)).astype(np.float32)).to(torch.bfloat16)
+    kernel = (rng.standard_normal(512) * 0.05).astype(np.float32)
+    rows = torch.from_numpy(rng.standard_normal((333, 256)).astype(np.float32)).to(torch.bfloat16)
+    got = ops.gate_rows(x.cuda(), torch.from_numpy(kernel).cuda(), rows.cuda()).float().cpu().numpy()
+    want = oracle.gated_rows(x.float().numpy(), kernel, rows.float().numpy())
+    assert (got == want).mean() > 0.98 and np.abs(got - want).max() <= 2.0 ** -7 * np.abs(want).max()
+    hand_x = torch.zeros((1, 8), dtype=torch.bfloat16)
+    hand_x[0, 0] = 1.0
+    hand = ops.gate_rows(hand_x.cuda(), torch.full((8,), 0.3).cuda(), torch.tensor([[3.0, -1.0, 0, 0, 0, 0, 0, 0]], dtype=torch.bfloat16).cuda())
+    assert hand[0, :2].float().cpu().tolist() == [1.71875, -0.57421875]
+
+    case = CASES["c4-reduced"].scaled(tokens=200)
+    data = inputs(case, seed=13)
+    layer, variables = layer_and_variables(case, data)
+    gate = (rng.standard_normal(case.d_model) * 0.05).astype(np.float32)
+    variables["params"]["shared_expert_gate"] = {"kernel": torch.from_numpy(gate).reshape(-1, 1).cuda()}
+    layer = dataclasses.replace(layer, shared_gate=True, fuse_shared=fuse_shared, dtype=torch.bfloat16)
+    got = layer.apply(variables, data["x"].cuda(), logits=data["logits"].cuda()).float().cpu().numpy()
+    mats, factors = zip(*(dequantized(data["banks"][name]) for name in ("gate", "up", "down")), strict=True)
+    shared = [dequantized(data["shared"][name])[0][0] for name in ("gate", "up", "down")]
+    want, _ = oracle.sparse_mlp(data["x"].float().numpy(), data["logits"].numpy(), *mats, top_k_count=case.top_k, factors=factors,
+                                bias=data["bias"].numpy(), shared=shared, shared_gate=gate, **case.router)
+    ungated, _ = oracle.sparse_mlp(data["x"].float().numpy(), data["logits"].numpy(), *mats, top_k_count=case.top_k, factors=factors,
+                                   bias=data["bias"].numpy(), shared=shared, **case.router)
+    by_max, by_element = oracle.relative_errors(got, want)
+    assert by_max <= 6e-3 and by_element <= TOLERANCE, (by_max, by_element)
+    assert oracle.relative_errors(got, ungated)[0] > 10 * by_max                 # the gate gates
+    with pytest.raises(ValueError, match="compute dtype"):
+        dataclasses.replace(layer, dtype=None).apply(variables, data["x"].cuda(), logits=data["logits"].cuda())
+    with pytest.raises(ValueError, match="requires a shared expert"):
+        dataclasses.replace(layer, shared=None).apply(variables, data["x"].cuda(), logits=data["logits"].cuda())

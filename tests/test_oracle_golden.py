@@ -639,3 +639,32 @@ def test_block_routing_limits_a_token_to_its_blocks_best_experts():
         for row in range(3):                       # every block uses at most block_experts experts, and the same shortlist
             for block in np.unique(blocks[row]):
                 assert np.unique(indices[row, blocks[row] == block]).size <= 4
+
+
+def test_the_shared_experts_gate_rounds_its_logit_its_logistic_and_its_product():
+    """`gated_rows` (`shared_gate` under a bf16 compute dtype). By hand: x = (1, 0, ...), kernel = (0.3, ...): the kernel
+    rounds to bf16 0.30078125, which is the logit; logistic(0.30078125) = 0.574633..., bf16 0.57421875 (the neighbours
+    are 0.57421875 and 0.578125); a row value of 3.0 gives 1.72265625, which lies between the bf16 neighbours 1.71875
+    and 1.7265625, nearer the former. Unrounded, 3 * sigmoid(0.3) = 1.7233... would round to 1.7265625."""
+    x = np.zeros((1, 8), np.float32)
+    x[0, 0] = 1.0
+    kernel = np.full(8, 0.3, np.float32)
+    assert oracle.gated_rows(x, kernel, np.array([[3.0, -1.0]], np.float32)).tolist() == [[1.71875, -0.57421875]]
+    assert oracle.bf16_round(np.float32(3.0 / (1.0 + np.exp(-0.3)))) == np.float32(1.7265625)
+    rng = np.random.default_rng(17)
+    x = oracle.bf16_round(rng.standard_normal((50, 64)).astype(np.float32))
+    kernel = (rng.standard_normal(64) * 0.2).astype(np.float32)
+    rows = oracle.bf16_round(rng.standard_normal((50, 24)).astype(np.float32))
+    truth = rows.astype(np.float64) / (1.0 + np.exp(-(x.astype(np.float64) @ kernel.astype(np.float64))))[:, None]
+    got = oracle.gated_rows(x, kernel, rows)
+    assert np.abs(got - truth).max() <= 3 * 2.0 ** -8 * np.abs(truth).max()          # three bf16 roundings and the kernel's own
+    assert np.abs(got - truth).max() > 0
+    # the layer: the shared expert's output gated, then added
+    logits = rng.standard_normal((50, 4)).astype(np.float32)
+    banks = [oracle.bf16_round((rng.standard_normal(shape) * 0.1).astype(np.float32)) for shape in ((4, 64, 32), (4, 64, 32), (4, 32, 64))]
+    shared = [bank[0] for bank in banks]
+    gate = (rng.standard_normal(64) * 0.2).astype(np.float32)
+    gated, _ = oracle.sparse_mlp(x, logits, *banks, top_k_count=2, shared=shared, shared_gate=gate)
+    routed, _ = oracle.sparse_mlp(x, logits, *banks, top_k_count=2)
+    apart = oracle.gated_rows(x, gate, oracle.gated_mlp(x, *shared))
+    assert np.array_equal(gated, oracle.bf16_round(routed + apart))
