@@ -2,8 +2,9 @@
 // (reference src/dew/nn/moe.py:526-534: tokens widened to fp32, Precision.HIGHEST), and group offsets.
 // Depths in whole 16s run on the fp32 matrix instruction (v_mfma_f32_32x32x2_f32: fp32 operands, exact products, fp32
 // sums): a block takes 32 (or 64) tokens and up to four 32-expert tiles, its wavefronts a share of the depth each; the
-// partial sums of a tile meet in LDS in wavefront order, so the result does not depend on timing. Measured: 64 tokens
-// of GPT-OSS's 2880 x 32 gate in about 10 us and 8192 tokens of a 7168 x 256 gate in 319 us (94 TFLOP/s), where the
+// partial sums of a tile meet in LDS in wavefront order, so the result does not depend on timing. A decode step's few
+// tokens take 16 x 16 tiles (v_mfma_f32_16x16x4_f32), four times the blocks. Measured: 64 tokens of GPT-OSS's 2880 x 32
+// gate in about 5 us of kernel and 8192 tokens of a 7168 x 256 gate in 319 us (94 TFLOP/s), where the
 // plain kernel below (a 64-token x 64-expert tile, 16-deep LDS steps, fp32 FMA; depths in no whole 16s still take it)
 // needed 550 us and 1.3 ms.
 #include "common.h"
@@ -71,7 +72,7 @@ __global__ __launch_bounds__(64 * WAVES) void router_logits_mfma_kernel(const bf
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[r][j], b[buffer][c][j], acc[r][c], 0, 0, 0);
   };
-  if constexpr (WAVES == 16) {  // a decode step's wavefronts walk a few chunks each: nothing to overlap
+  if constexpr (WAVES == 16) {  // a decode step's wavefronts walk a few chunks each (loads kept further ahead changed nothing: the matrix pipe is the limit)
     for (int chunk = first; chunk < last; ++chunk) {
       load(0, chunk);
       multiply(0);
@@ -108,6 +109,71 @@ __global__ __launch_bounds__(64 * WAVES) void router_logits_mfma_kernel(const bf
         if (t < tokens && e < experts) logits[static_cast<size_t>(t) * experts + e] = bias ? sum + bias[e] : sum;
       }
     }
+  }
+}
+
+// The few tokens of a decode step on finer tiles: 16 tokens x 16 experts a block (v_mfma_f32_16x16x4_f32, the same
+// rate a CU as the 32 x 32 form), sixteen wavefronts a share of the depth each. A 32 x 32 tile's block keeps its whole
+// product on one CU's four matrix pipes (64 tokens of a 2880 x 32 gate: two blocks, 20 us); four times the blocks
+// finish in a quarter of that. Lane l multiplies token l % 16 and expert l % 16 over the depths 4 (l / 16) .. + 3 of a
+// 16-deep chunk, one depth an instruction; its four sums are tokens 4 (l / 16) + i of expert column l % 16.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+__global__ __launch_bounds__(1024) void router_logits_fine_kernel(const bf16_t* __restrict__ x, const float* __restrict__ kernel,
+                                                                  const float* __restrict__ bias, float* __restrict__ logits,
+                                                                  int tokens, int depth, int experts) {
+  constexpr int kWaves = 16;
+  __shared__ float partial[kWaves][4][64];
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const int t0 = blockIdx.x * 16, e0 = blockIdx.y * 16;
+  const int chunks = depth / 16;
+  const int first = static_cast<int>(static_cast<long long>(chunks) * wave / kWaves);
+  const int last = static_cast<int>(static_cast<long long>(chunks) * (wave + 1) / kWaves);
+  const bf16_t* a_src = x + static_cast<size_t>(min(t0 + lane % 16, tokens - 1)) * depth + 4 * (lane / 16);
+  const float* b_src = kernel + static_cast<size_t>(4 * (lane / 16)) * experts + min(e0 + lane % 16, experts - 1);
+  f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+  // four chunks' loads are in flight while the four before them multiply (a wavefront's walk is a chain of round trips
+  // otherwise: 28 chunks of a 7168-deep gate)
+  constexpr int kAhead = 4;
+  u32x2 words[2][kAhead];
+  float b[2][kAhead][4];
+  auto load = [&](int set, int chunk) __attribute__((always_inline)) {
+#pragma unroll
+    for (int ahead = 0; ahead < kAhead; ++ahead) {
+      const int at = min(chunk + ahead, last - 1);  // (past the share: the last chunk again, which multiplies nothing)
+      words[set][ahead] = *reinterpret_cast<const u32x2*>(a_src + at * 16);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[set][ahead][j] = b_src[static_cast<size_t>(at * 16 + j) * experts];
+    }
+  };
+  auto multiply = [&](int set, int chunk) __attribute__((always_inline)) {
+#pragma unroll
+    for (int ahead = 0; ahead < kAhead; ++ahead) {
+      if (chunk + ahead >= last) continue;
+      const u32x2 w = words[set][ahead];
+      const float a[4] = {__uint_as_float(w[0] << 16), __uint_as_float(w[0] & 0xFFFF0000u), __uint_as_float(w[1] << 16),
+                          __uint_as_float(w[1] & 0xFFFF0000u)};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j], b[set][ahead][j], acc, 0, 0, 0);
+    }
+  };
+  if (first < last) load(0, first);
+  for (int chunk = first; chunk < last; chunk += 2 * kAhead) {
+    if (chunk + kAhead < last) load(1, chunk + kAhead);
+    multiply(0, chunk);
+    if (chunk + 2 * kAhead < last) load(0, chunk + 2 * kAhead);
+    if (chunk + kAhead < last) multiply(1, chunk + kAhead);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) partial[wave][i][lane] = acc[i];
+  __syncthreads();
+  if (wave < 4) {  // wavefront i finishes register i of every lane, adding the wavefronts' partial sums in wavefront order
+    float sum = partial[0][wave][lane];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) sum += partial[w][wave][lane];
+    const int t = t0 + 4 * (lane / 16) + wave, e = e0 + lane % 16;
+    if (t < tokens && e < experts) logits[static_cast<size_t>(t) * experts + e] = bias ? sum + bias[e] : sum;
   }
 }
 
@@ -182,6 +248,11 @@ extern "C" int dew_moe_router_logits(const void* x, const float* kernel, const f
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int tiles = (experts + 31) / 32;
   if (depth % 16 == 0 && depth >= 64 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0) {
+    if (static_cast<long long>((tokens + 31) / 32) * tiles < 64) {  // a decode step: finer tiles, four times the blocks
+      hipLaunchKernelGGL(router_logits_fine_kernel, dim3((tokens + 15) / 16, (experts + 15) / 16), dim3(1024), 0, s,
+                         static_cast<const bf16_t*>(x), kernel, bias, logits, tokens, depth, experts);
+      return launched("router_logits_fine_kernel");
+    }
     if (tokens <= 2048) {  // at most 64 token blocks: a block takes one tile, its sixteen wavefronts share the depth
       hipLaunchKernelGGL((router_logits_mfma_kernel<1, 16>), dim3((tokens + 31) / 32, tiles), dim3(1024), 0, s, static_cast<const bf16_t*>(x),
                          kernel, bias, logits, tokens, depth, experts);
