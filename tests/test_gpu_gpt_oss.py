@@ -261,3 +261,34 @@ def test_an_mxfp4_checkpoint_bank_of_gpt_oss_extents_stays_packed_on_the_device(
     want = oracle.gpt_oss_gating(oracle._biased_matmul(bf16_np(x), values, sizes, bias.cpu().numpy(), dtype="bfloat16", factor=None), limit=7.0)
     got = bf16_np(gated)
     assert np.abs(got - want).max() <= 2 ** -6 * np.abs(want).max() and (got == want).mean() > 0.9
+
+
+@pytest.mark.parametrize("quant", ["mxfp4", "nvfp4"])
+def test_a_decode_step_on_many_fp4_experts_of_a_ragged_width(ops, quant):
+    """Enough experts and columns that a decode step's one-bank launches take their 256-column blocks (experts x strips of
+    256 >= 640) on a width that is no whole 256s (2688 = 10 strips and 128 columns): the plain product with its bias and
+    GPT-OSS's gated one, a few rows an expert and several experts empty, against the oracle."""
+    from dew_amd import codecs, formats, gemm
+    from moe_cases import dequantized, quantize
+
+    rng = np.random.default_rng(23)
+    experts, depth, width = 64, 256, 2688
+    sizes = rng.integers(0, 9, size=experts)
+    sizes[rng.integers(0, experts, size=6)] = 0
+    weight = torch.from_numpy((rng.standard_normal((experts, depth, width)) * 0.05).astype(np.float32))
+    bank = formats.Mxfp4Blocks(*codecs.quantize_mxfp4(weight)) if quant == "mxfp4" else quantize(weight, "nvfp4")
+    values, factor = dequantized(bank)
+    x = torch.from_numpy(rng.standard_normal((int(sizes.sum()) + 5, depth)).astype(np.float32)).to(torch.bfloat16)
+    bias = torch.from_numpy(rng.standard_normal((experts, width)).astype(np.float32)).to(torch.bfloat16).float()
+    group_sizes = torch.tensor(sizes, dtype=torch.int32).cuda()
+    got = bf16_np(gemm.gemm(x.cuda(), bank.to("cuda"), group_sizes, epilogue="plus_bias", epilogue_operands=(bias.cuda(),)))
+    want = oracle._biased_matmul(bf16_np(x), values, sizes.tolist(), bias.numpy(), dtype="bfloat16", factor=factor)
+    assert got.shape == want.shape and not got[int(sizes.sum()):].any()
+    assert np.abs(got - want).max() <= 2 ** -7 * np.abs(want).max() and (got == want).mean() > 0.97
+    if quant == "nvfp4":      # (the interleaved gated launch is GPT-OSS's: MXFP4 and unquantized banks)
+        return
+    gated = bf16_np(gemm.gemm(x.cuda(), bank.to("cuda"), group_sizes, epilogue="gpt_oss_gated", epilogue_operands=(bias.cuda(), 7.0)))
+    sums = oracle._biased_matmul(bf16_np(x), values, sizes.tolist(), bias.numpy(), dtype="bfloat16", factor=factor)
+    want = oracle.gpt_oss_gating(sums, limit=7.0)
+    assert gated.shape == (x.shape[0], width // 2)
+    assert np.abs(gated - want).max() <= 2 ** -6 * np.abs(want).max() and (gated == want).mean() > 0.9
