@@ -185,10 +185,17 @@ __global__ __launch_bounds__(THREADS) void permute_small_kernel(PermuteParams p)
   const int segment = ((p.slots + THREADS - 1) / THREADS) * 64;  // contiguous slots per wavefront
   const int rounds = segment / 64;
   const int wave_begin = wave * segment;
-  for (int round = 0; round < rounds; ++round) {
+  // a lane's buckets stay in registers between the count and the scatter (one round trip to the indices, not two)
+  constexpr int kMaxRounds = (THREADS == kSmallThreads ? kSmallSlots : kNarrowSmallSlots) / THREADS;
+  int kept[kMaxRounds];
+#pragma unroll
+  for (int round = 0; round < kMaxRounds; ++round) {
     const int slot = wave_begin + round * 64 + lane;
-    if (slot < p.slots) atomicAdd(&mine[bucket_of(p, slot)], 1);
+    kept[round] = (round < rounds && slot < p.slots) ? bucket_of(p, slot) : p.buckets;
   }
+#pragma unroll
+  for (int round = 0; round < kMaxRounds; ++round)
+    if (kept[round] < p.buckets) atomicAdd(&mine[kept[round]], 1);
   __syncthreads();
   for (int b = threadIdx.x; b < p.buckets; b += THREADS) {
     int sum = 0;
@@ -231,10 +238,12 @@ __global__ __launch_bounds__(THREADS) void permute_small_kernel(PermuteParams p)
   __syncthreads();
   int bits = 1;
   while ((1 << bits) < p.buckets) ++bits;
-  for (int round = 0; round < rounds; ++round) {
+#pragma unroll
+  for (int round = 0; round < kMaxRounds; ++round) {
+    if (round >= rounds) continue;  // (the same for the whole block)
     const int slot = wave_begin + round * 64 + lane;
-    const bool valid = slot < p.slots;
-    const int bucket = valid ? bucket_of(p, slot) : p.buckets;
+    const int bucket = kept[round];
+    const bool valid = bucket < p.buckets;
     unsigned long long same = __ballot(valid);
     for (int bit = 0; bit < bits; ++bit) {
       const bool set = (bucket >> bit) & 1;
@@ -245,9 +254,11 @@ __global__ __launch_bounds__(THREADS) void permute_small_kernel(PermuteParams p)
     const int count = __popcll(same);
     int position = 0;
     if (valid) position = mine[bucket] + rank;
-    __syncthreads();
+    // (the running positions are the wavefront's own: its reads above are done before the write below is issued, and
+    // the next round's reads come after it in the same queue; no other wavefront touches them)
+    __builtin_amdgcn_wave_barrier();
     if (valid && rank == count - 1) mine[bucket] = position + 1;
-    __syncthreads();
+    __builtin_amdgcn_wave_barrier();
     if (valid) {
       p.order[position] = slot;
       p.rows[position] = row_of(p, slot);
