@@ -163,7 +163,12 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
 #pragma unroll
   for (int i = 0; i < kPerLane; ++i) {
     const int e = lane + kWave * i;
-    logit[i] = e < p.experts ? capped(row[e], p.softcap) : ninf;
+    logit[i] = e < p.experts ? row[e] : ninf;
+  }
+  if (p.softcap > 0.0f) {  // (a branch of its own: the cap's hyperbolic tangent stays out of the routers that have none)
+#pragma unroll
+    for (int i = 0; i < kPerLane; ++i)
+      if (lane + kWave * i < p.experts) logit[i] = capped(logit[i], p.softcap);
   }
 
   float top = ninf, denom = 1.0f;
@@ -314,7 +319,8 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
 
   // gate weights: lane j < k owns the j-th choice
   const bool owner = lane < p.top_k;
-  const float chosen_logit = owner ? capped(row[my_choice], p.softcap) : ninf;
+  float chosen_logit = owner ? row[my_choice] : ninf;
+  if (p.softcap > 0.0f && owner) chosen_logit = capped(chosen_logit, p.softcap);
   float weight = 0.0f;
   if (p.score_function == DEW_MOE_SCORE_SOFTMAX && p.normalize && !p.bias_in_weights && !(p.sum_min != 0.0f)) {
     const float m = wave_max(chosen_logit);
