@@ -559,3 +559,46 @@ def test_qwen2_moes_gate_on_the_shared_expert(fuse_shared):
         dataclasses.replace(layer, dtype=None).apply(variables, data["x"].cuda(), logits=data["logits"].cuda())
     with pytest.raises(ValueError, match="requires a shared expert"):
         dataclasses.replace(layer, shared=None).apply(variables, data["x"].cuda(), logits=data["logits"].cuda())
+
+
+def test_a_captured_layer_replays_to_the_eager_result():
+    """The whole layer (gate GEMM, router, sort, the grouped launches, combine, the shared expert's gate) and a block
+    router's four launches recorded into one HIP graph: every replay, on new inputs and with eager work and
+    synchronizations between the replays, returns the eager call's bits. (Nothing in these paths clears memory with a
+    memset node: the counters and keys that start at zero are cleared by kernels.)"""
+    import dataclasses
+
+    from dew_amd import moe, ops
+    case = CASES["c4-reduced"].scaled(tokens=48)
+    data = inputs(case, seed=21)
+    layer, variables = layer_and_variables(case, data)
+    rng = np.random.default_rng(5)
+    variables["params"]["gate"] = {"kernel": torch.from_numpy((rng.standard_normal((case.d_model, case.experts)) * 0.05).astype(np.float32)).cuda()}
+    variables["params"]["shared_expert_gate"] = {"kernel": torch.from_numpy((rng.standard_normal((case.d_model, 1)) * 0.05).astype(np.float32)).cuda()}
+    layer = dataclasses.replace(layer, shared_gate=True, dtype=torch.bfloat16)
+    block_router = moe.Router(case.experts, case.d_model, case.top_k, score_function="sigmoid", routing_block=8, block_experts=24)._bound(variables, ("gate",))
+    blocks = (torch.arange(48, dtype=torch.int32) // 8).reshape(1, 48).cuda()
+    xs = [torch.from_numpy(rng.standard_normal((48, case.d_model)).astype(np.float32)).to(torch.bfloat16).cuda() for _ in range(3)]
+
+    def step(x):
+        out = layer.apply(variables, x)
+        weights, indices = block_router.chosen(block_router.logits(x)[None], blocks=blocks)
+        return out, weights, indices
+
+    eager = [tuple(t.clone() for t in step(x)) for x in xs]
+    held = xs[0].clone()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        step(held)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            recorded = step(held)
+    torch.cuda.synchronize()
+    for turn in (0, 1, 2, 1, 0):
+        held.copy_(xs[turn])
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(recorded, eager[turn], strict=True):
+            assert torch.equal(got, want), turn
+        step(xs[(turn + 1) % 3])                     # the program's own eager work between the replays
+        torch.cuda.synchronize()
