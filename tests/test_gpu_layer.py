@@ -602,3 +602,31 @@ def test_a_captured_layer_replays_to_the_eager_result():
             assert torch.equal(got, want), turn
         step(xs[(turn + 1) % 3])                     # the program's own eager work between the replays
         torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("name,tokens", [("c2-reduced", 2048), ("c5-reduced", 300), ("c1-full", 256)])
+def test_captured_layers_of_the_other_formats_replay_to_the_eager_result(name, tokens):
+    """The MXFP4 layer on split rows (its workspace comes from the caller's allocator, here the graph's pool), the NVFP4
+    and the per-channel FP8 layers: recorded once, replayed on new inputs between eager calls, the eager bits each time."""
+    case = CASES[name].scaled(tokens=tokens)
+    data = inputs(case, seed=22)
+    layer, variables = layer_and_variables(case, data)
+    rng = np.random.default_rng(6)
+    xs = [torch.from_numpy(rng.standard_normal((tokens, case.d_model)).astype(np.float32)).to(torch.bfloat16).cuda() for _ in range(2)]
+    logits = [torch.from_numpy(rng.standard_normal((tokens, case.experts)).astype(np.float32)).cuda() for _ in range(2)]
+    eager = [layer.apply(variables, x, logits=l).clone() for x, l in zip(xs, logits, strict=True)]
+    held_x, held_l = xs[0].clone(), logits[0].clone()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        layer.apply(variables, held_x, logits=held_l)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            recorded = layer.apply(variables, held_x, logits=held_l)
+    torch.cuda.synchronize()
+    for turn in (0, 1, 1, 0):
+        held_x.copy_(xs[turn]), held_l.copy_(logits[turn])
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(recorded, eager[turn]), turn
+        layer.apply(variables, xs[1 - turn], logits=logits[1 - turn])
+        torch.cuda.synchronize()
