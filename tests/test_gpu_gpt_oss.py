@@ -126,6 +126,25 @@ def test_gpt_oss_layer_matches_the_oracle(quant):
     peak_error, elementwise = oracle.relative_errors(bf16_np(got).reshape(want.shape), want)
     assert peak_error <= 2e-2 and elementwise <= 2e-2          # max|got - want| / max|want| and element-wise with an rms floor
     assert peak_error <= 8e-3
+    # recorded into a HIP graph (its gate GEMM, biased router, sort, both biased launches, its own combine), the layer
+    # replays to the eager bits on new tokens
+    others = [torch.from_numpy(rng.standard_normal(x.shape).astype(np.float32)).to(torch.bfloat16).cuda() for _ in range(2)]
+    eager = [layer.apply(variables, other).clone() for other in others]
+    held = others[0].clone()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        layer.apply(variables, held)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            recorded = layer.apply(variables, held)
+    torch.cuda.synchronize()
+    for turn in (1, 0, 1):
+        held.copy_(others[turn])
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(recorded, eager[turn])
+        layer.apply(variables, others[1 - turn])
+        torch.cuda.synchronize()
 
 
 def test_gpt_oss_requirements_are_refused_by_name(ops):
