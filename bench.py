@@ -202,11 +202,11 @@ def oracle_sample(case, data, plan, budget_rows=192):
 # written). The counters cannot be read from inside this process, so the figures sit here, taken from the summaries under
 # profiles/ named in COUNTED_FROM; `roofline.traffic_source` says so in the line. A workload without an entry reports null.
 COUNTER_SCALE = {"FETCH_SIZE": 2.0, "WRITE_SIZE": 1.0}
-COUNTED_KIB = {"c1": {"FETCH_SIZE": 8971.0, "WRITE_SIZE": 8192.0},
-               "c2": {"FETCH_SIZE": 4171500.1, "WRITE_SIZE": 931923.7},
-               "c3": {"FETCH_SIZE": 199656.6, "WRITE_SIZE": 768.0},
-               "c4": {"FETCH_SIZE": 5254499.9 + 1961016.3, "WRITE_SIZE": 277320.0 + 17592.0},   # the 128-row tiles' launch + the last tiles' 64-row launch (shared expert's rows among them)
-               "c5": {"FETCH_SIZE": 1229873.8, "WRITE_SIZE": 229376.0}}
+COUNTED_KIB = {"c1": {"FETCH_SIZE": 12975.7, "WRITE_SIZE": 8192.0},
+               "c2": {"FETCH_SIZE": 4169892.2, "WRITE_SIZE": 931938.8},
+               "c3": {"FETCH_SIZE": 199655.3, "WRITE_SIZE": 768.0},
+               "c4": {"FETCH_SIZE": 5254501.5 + 1961660.6, "WRITE_SIZE": 277320.0 + 17592.0},   # the 128-row tiles' launch + the last tiles' 64-row launch (shared expert's rows among them)
+               "c5": {"FETCH_SIZE": 1229803.8, "WRITE_SIZE": 229376.0}}
 COUNTED_FROM = {"c1": "profiles/grouped_gemm_c1_small_fp8_channel.txt", "c2": "profiles/grouped_gemm_c2_prefill_mxfp4.txt",
                 "c3": "profiles/grouped_gemm_c3_decode_fp8.txt", "c4": "profiles/grouped_gemm_c4_prefill_fp8_blocks.txt",
                 "c5": "profiles/grouped_gemm_c5_prefill_nvfp4.txt"}
