@@ -26,7 +26,6 @@ from pathlib import Path
 
 ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
-sys.path.insert(0, str(ROOT / "tests"))
 
 PEAKS = {"bf16_mfma": 2500.0, "fp8_mfma": 5000.0, "fp4_mfma": 10100.0, "hbm_gbs": 8000.0}
 """MI355X published dense peaks, TFLOP/s and GB/s."""
@@ -42,7 +41,7 @@ def build_workload(case, device, seed=0):
     """Synthetic tensors of `case` on the device: bf16 activations ~N(0,1), fp32 router logits ~N(0,1) (+ a
     per-expert bias), banks ~N(0,0.02) quantized on the device one expert matrix at a time."""
     import torch
-    from moe_cases import quantize
+    from bench_aids.workloads import quantize
 
     from dew_amd import formats, gemm
 
@@ -153,68 +152,159 @@ class Stepper:
         return sum(start.elapsed_time(stop) for start, stop in self.events) / max(1, len(self.events))
 
 
-def oracle_sample(case, data, plan, budget_rows=192):
-    """The CPU oracle (dequantize -> bf16-exact fp32 GEMMs -> SwiGLU -> down) on a bounded sample of the workload: the
-    busiest expert's first `budget_rows` sorted rows, all three projections at full width. Returns the timing as the
-    `cpu_baseline` object and (the slots of those rows, the oracle's down-projection rows for them)."""
+def sampled_groups(sizes, budget_rows, first_budget=None):
+    """Which sorted rows the CPU oracle follows: of the busiest expert, the one of median size and the least non-empty one
+    (as many of them as differ), each group's first and last rows, `budget_rows` a group in all (`first_budget` for the
+    busiest: the timed baseline's larger sample). A group's last rows are the ones a launch's partial last tile, or a
+    second launch of shorter tiles, multiplies. Returns [(expert, positions within the group)]."""
+    import numpy as np
+
+    filled = np.flatnonzero(sizes > 0)
+    by_size = filled[np.argsort(sizes[filled], kind="stable")]
+    chosen = []
+    for expert in (int(by_size[-1]), int(by_size[len(by_size) // 2]), int(by_size[0])):
+        if expert not in chosen:
+            chosen.append(expert)
+    groups = []
+    for place, expert in enumerate(chosen):
+        size, budget = int(sizes[expert]), int(first_budget if place == 0 and first_budget else budget_rows)
+        if size <= budget:
+            positions = np.arange(size)
+        else:
+            positions = np.concatenate([np.arange(budget - budget // 2), np.arange(size - budget // 2, size)])
+        groups.append((expert, positions))
+    return groups
+
+
+def oracle_sample(case, data, plan, budget_rows=64, first_budget=None):
+    """The CPU oracle (dequantize -> bf16-exact fp32 GEMMs -> SwiGLU -> down) on a bounded sample of the workload: first
+    and last sorted rows of up to three experts (`sampled_groups`), all three projections at full width. Returns the
+    timing as the `cpu_baseline` object and (the slots of those rows, the oracle's down-projection rows for them, the
+    experts sampled)."""
+    import numpy as np
     import torch
-    from moe_cases import dequantized
 
     from dew_amd import formats
     from oracle import moe_oracle as oracle
+    from oracle.banks import dequantized
 
     sizes = plan.sizes.cpu().numpy()[:case.experts]      # (a fused shared expert is group #E of the plan: not sampled here)
     offsets = plan.offsets.cpu().numpy()
-    expert = int(sizes.argmax())
-    rows = int(min(budget_rows, sizes[expert]))
-    sorted_rows = plan.rows.cpu().numpy()[offsets[expert]:offsets[expert] + rows]
-    slots = plan.order.cpu().numpy()[offsets[expert]:offsets[expert] + rows]
+    sorted_rows_all, order_all = plan.rows.cpu().numpy(), plan.order.cpu().numpy()
 
-    def one(bank):
+    def one(bank, expert):
         if isinstance(bank, formats.NvFp4):
             return formats.NvFp4(bank.words[expert:expert + 1].cpu(), bank.scales[expert:expert + 1].cpu(), bank.scale[expert:expert + 1].cpu())
         if isinstance(bank, formats.Fp8Blocks):
             return formats.Fp8Blocks(bank.codes[expert:expert + 1].cpu(), bank.scale_inv[expert:expert + 1].cpu())
         return formats.Fp8Channels(bank.codes[expert:expert + 1].cpu(), bank.scales[expert:expert + 1].cpu())
 
-    held = [one(data["banks"][n]) for n in ("gate", "up", "down")]
-    x = data["x"][torch.from_numpy(sorted_rows).to(data["x"].device).long()].float().cpu().numpy()
     threads = os.cpu_count() or 1
+    dequant_s = gemm_s = 0.0
+    all_slots, all_down, described, total_rows = [], [], [], 0
+    for expert, positions in sampled_groups(sizes, budget_rows, first_budget):
+        at = offsets[expert] + positions
+        x = data["x"][torch.from_numpy(sorted_rows_all[at]).to(data["x"].device).long()].float().cpu().numpy()
+        held = [one(data["banks"][n], expert) for n in ("gate", "up", "down")]
+        began = time.perf_counter()
+        mats, factors = zip(*(dequantized(bank) for bank in held), strict=True)
+        dequant_s += time.perf_counter() - began
+        began = time.perf_counter()
+        rows = len(positions)
+        gate = oracle.grouped_matmul(x, mats[0], [rows], factor=factors[0])
+        up = oracle.grouped_matmul(x, mats[1], [rows], factor=factors[1])
+        hidden = oracle.swiglu(gate, up)
+        all_down.append(oracle.grouped_matmul(hidden, mats[2], [rows], factor=factors[2]))
+        gemm_s += time.perf_counter() - began
+        all_slots.append(order_all[at])
+        described.append(f"{rows} of expert {expert}'s {int(sizes[expert])}")
+        total_rows += rows
+        del mats
+    flops = 6.0 * total_rows * case.d_model * case.d_ff
+    baseline = {"value": round(flops / (dequant_s + gemm_s) / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                "sample": f"first and last sorted rows of the busiest, the median and the least non-empty expert ({', '.join(described)}), "
+                          f"3 projections at full width: dequantize {dequant_s:.2f} s + fp32 GEMMs/SwiGLU {gemm_s:.2f} s "
+                          "(NumPy/OpenBLAS on bf16-exact fp32 operands)",
+                "gemm_only_tflops": round(flops / gemm_s / 1e12, 5)}
+    return baseline, (np.concatenate(all_slots), np.concatenate(all_down), [expert for expert, _ in sampled_groups(sizes, budget_rows, first_budget)])
+
+
+WHOLE_ON_CPU = ("c1", "c3")
+"""The workloads small enough for the CPU oracle to run whole (seconds): their baseline is no sample and no extrapolation,
+and their parity is every element of the layer's output."""
+
+
+def oracle_whole(case, data):
+    """The CPU oracle on the whole workload (router, sort, three projections of every expert, combine), timed; returns the
+    `cpu_baseline` object and (the oracle's layer output, its routing trace)."""
+    from oracle import moe_oracle as oracle
+    from oracle.banks import dequantized
+
+    threads = os.cpu_count() or 1
+    x, logits = data["x"].float().cpu().numpy(), data["logits"].cpu().numpy()
     began = time.perf_counter()
-    mats, factors = zip(*(dequantized(bank) for bank in held), strict=True)
+    mats, factors = zip(*(dequantized(data["banks"][n].to("cpu")) for n in ("gate", "up", "down")), strict=True)
     dequant_s = time.perf_counter() - began
     began = time.perf_counter()
-    gate = oracle.grouped_matmul(x, mats[0], [rows], factor=factors[0])
-    up = oracle.grouped_matmul(x, mats[1], [rows], factor=factors[1])
-    hidden = oracle.swiglu(gate, up)
-    down = oracle.grouped_matmul(hidden, mats[2], [rows], factor=factors[2])
-    gemm_s = time.perf_counter() - began
-    flops = 6.0 * rows * case.d_model * case.d_ff
-    return {"value": round(flops / (dequant_s + gemm_s) / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": f"{rows} sorted rows of expert {expert} (the busiest), 3 projections at full width: dequantize "
-                      f"{dequant_s:.2f} s + fp32 GEMMs/SwiGLU {gemm_s:.2f} s (NumPy/OpenBLAS on bf16-exact fp32 operands)",
-            "gemm_only_tflops": round(flops / gemm_s / 1e12, 5)}, (slots, down)
+    want, trace = oracle.sparse_mlp(x, logits, *mats, top_k_count=case.top_k, factors=factors,
+                                    bias=None if data["bias"] is None else data["bias"].cpu().numpy(), **case.router)
+    layer_s = time.perf_counter() - began
+    flops = 6.0 * case.tokens * case.top_k * case.d_model * case.d_ff
+    return {"value": round(flops / (dequant_s + layer_s) / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"the whole workload, no extrapolation: dequantize every expert {dequant_s:.2f} s + route, sort, 3 grouped "
+                      f"projections, SwiGLU, combine {layer_s:.2f} s (NumPy/OpenBLAS on bf16-exact fp32 operands)"}, (want, trace)
 
 
 # HBM bytes one launch of the dominant (gate/up) kernel moved, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (KiB per
 # dispatch, two runs of `bench.py --config cN --only` per workload), each scaled by what the same counter reads for the plain
-# copy probe of known size (--calibrate-copy: FETCH_SIZE reads half of the bytes fetched, WRITE_SIZE all of the bytes
-# written). The counters cannot be read from inside this process, so the figures sit here, taken from the summaries under
-# profiles/ named in COUNTED_FROM; `roofline.traffic_source` says so in the line. A workload without an entry reports null.
-COUNTER_SCALE = {"FETCH_SIZE": 2.0, "WRITE_SIZE": 1.0}
-COUNTED_KIB = {"c1": {"FETCH_SIZE": 12975.7, "WRITE_SIZE": 8192.0},
-               "c2": {"FETCH_SIZE": 4169892.2, "WRITE_SIZE": 931938.8},
-               "c3": {"FETCH_SIZE": 199655.3, "WRITE_SIZE": 768.0},
-               "c4": {"FETCH_SIZE": 5254501.5 + 1961660.6, "WRITE_SIZE": 277320.0 + 17592.0},   # the 128-row tiles' launch + the last tiles' 64-row launch (shared expert's rows among them)
-               "c5": {"FETCH_SIZE": 1229803.8, "WRITE_SIZE": 229376.0}}
+# copy probe of known size (--calibrate-copy). The counters cannot be read from inside this process: the figures are parsed,
+# at every run, from the rocprofv3 summaries committed under profiles/ (the files named here), so the line cannot drift from
+# them; `roofline.traffic_source` names the file. A workload whose summary is missing or has no such row reports null.
 COUNTED_FROM = {"c1": "profiles/grouped_gemm_c1_small_fp8_channel.txt", "c2": "profiles/grouped_gemm_c2_prefill_mxfp4.txt",
                 "c3": "profiles/grouped_gemm_c3_decode_fp8.txt", "c4": "profiles/grouped_gemm_c4_prefill_fp8_blocks.txt",
                 "c5": "profiles/grouped_gemm_c5_prefill_nvfp4.txt"}
+CALIBRATION = "profiles/probe_copy_counter_calibration.txt"
+PAIRED_MODES = (1, 3)
+"""Second template argument of grouped_gemm_kernel<FORMAT, MODE, ...> for the paired gate/up launches: SwiGLU of two banks,
+and the same leaving its rows split."""
+
+
+def counter_scales():
+    """{counter: factor} of the copy calibration: known bytes over what the counter read."""
+    import re
+
+    text = (ROOT / CALIBRATION).read_text()
+    return {name: float(factor) for name, factor in re.findall(r"^\s*(FETCH_SIZE|WRITE_SIZE)\s.*scale factor ([0-9.]+)\s*$", text, re.M)}
+
+
+def counted_kib(config):
+    """{counter: KiB per step} summed over the paired gate/up launches of a step (a workload whose groups' last rows go to a
+    second launch of shorter tiles has two), read from section 2 of the workload's committed summary; None without one."""
+    import re
+
+    path = ROOT / COUNTED_FROM.get(config, "")
+    if not path.is_file():
+        return None
+    section = path.read_text().split("2. HBM traffic", 1)
+    if len(section) < 2:
+        return None
+    totals = {"FETCH_SIZE": 0.0, "WRITE_SIZE": 0.0}
+    found = False
+    for line in section[1].splitlines():
+        row = re.match(r"^dew::grouped_gemm_kernel<\d+, (\d+), [^>]*>(?: grid \d+)?\s+\d+\s+([0-9.]+)\s+([0-9.]+)\s", line)
+        if row and int(row.group(1)) in PAIRED_MODES:
+            totals["FETCH_SIZE"] += float(row.group(2))
+            totals["WRITE_SIZE"] += float(row.group(3))
+            found = True
+    return totals if found else None
 
 
 def measured_traffic(config):
-    counted = COUNTED_KIB.get(config)
-    return None if counted is None else round(sum(counted[name] * COUNTER_SCALE[name] for name in counted) * 1024.0)
+    counted = counted_kib(config)
+    if counted is None:
+        return None
+    scales = counter_scales()
+    return round(sum(counted[name] * scales[name] for name in counted) * 1024.0)
 
 
 def sustained_rates(device):
@@ -253,7 +343,7 @@ def measure(config, args, device, sustained, with_cpu_baseline):
     """One workload, measured: its part of the line (ms_per_step, value, config, roofline, sample_parity,
     min_topk_margin and, where asked, cpu_baseline)."""
     import torch
-    from moe_cases import CONFIGS
+    from bench_aids.workloads import CONFIGS
 
     from bench_aids import probes
     from oracle import moe_oracle as oracle
@@ -331,8 +421,9 @@ def measure(config, args, device, sustained, with_cpu_baseline):
                                 "issue_time_note": "achieved over the rate at which the two instructions of a product issue back to back at "
                                                    "their published peaks (fp8 + fp8: 2.5 PFLOP/s; fp8 + fp6: 3.34 PFLOP/s)"}
     roofline["traffic"] = measured_traffic(config)
-    roofline["traffic_source"] = (f"stored: rocprofv3 --pmc FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 of this command's gate/up launch, "
-                                  f"{COUNTED_FROM[config]}; not measured in this run") if config in COUNTED_KIB else None
+    roofline["traffic_source"] = (f"parsed from {COUNTED_FROM[config]}: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE of this command's "
+                                  f"gate/up launch(es), scaled by {CALIBRATION}; counters of an earlier run of the same command, "
+                                  "not of this one") if roofline["traffic"] is not None else None
     roofline["algorithmic"] = {"per_launch": gateup_bytes if decode else gateup_flops, "unit": "bytes" if decode else "flop"}
     roofline["sustained"] = {"bf16_mfma_random_operands_tflops": sustained_mfma, "plain_copy_gbs": sustained_copy,
                              "read_stream_gbs": sustained_read,
@@ -377,10 +468,29 @@ def measure(config, args, device, sustained, with_cpu_baseline):
     result["min_topk_margin"] = {"value": gap if finite else None, "fp32_spacings": round(spacings, 1) if finite else None, "token": token,
                                  "note": "least gap over the tokens between the k-th selection and the best one left out; 0 is an "
                                          "exact tie (the lower index wins everywhere)"}
-    if with_cpu_baseline or not args.no_parity:
-        # the timed CPU baseline takes a larger sample (about ten seconds of host work, most of it the GEMMs, not the one
-        # expert's dequantization); the other configs' parity samples stay small so that the default run takes minutes
-        baseline, (slots, want) = oracle_sample(case, data, plan, budget_rows=4096 if with_cpu_baseline else 192)
+    if config in WHOLE_ON_CPU and not args.no_parity:
+        # small enough for the CPU oracle to follow whole: the baseline is the whole workload, and parity is every routed
+        # row's down projection, the routing itself and the layer's output
+        import numpy as np
+
+        baseline, (want, trace) = oracle_whole(case, data)
+        result["cpu_baseline"] = baseline
+        weights, indices = stepper.ops.route(data["logits"], case.top_k, bias=data["bias"], **case.router)
+        routing_identical = bool(np.array_equal(indices.cpu().numpy(), trace["indices"]) and np.array_equal(weights.cpu().numpy(), trace["weights"]))
+        got = stepper.project(plan).float().cpu().numpy()[:routed_rows]
+        want_slots = trace["slots"].reshape(routed_rows, case.d_model)
+        by_max, by_element = oracle.relative_errors(got, want_slots)
+        out_max, out_element = oracle.relative_errors(out.float().cpu().numpy(), want)
+        result["sample_parity"] = {"max_abs_over_max_ref": round(float(by_max), 6), "elementwise": round(float(by_element), 6),
+                                   "identical_frac": round(float((got == want_slots).mean()), 5), "rows": int(routed_rows),
+                                   "experts": f"all {touched} touched experts, every routed row", "routing_identical": routing_identical,
+                                   "layer_output": {"max_abs_over_max_ref": round(float(out_max), 6), "elementwise": round(float(out_element), 6),
+                                                    "identical_frac": round(float((out.float().cpu().numpy() == want).mean()), 5)},
+                                   "bar": 2e-2}
+    elif with_cpu_baseline or not args.no_parity:
+        # the timed CPU baseline takes a larger sample of the busiest expert (about ten seconds of host work, most of it the
+        # GEMMs, not the dequantization); the other configs' parity samples stay small so that the default run takes minutes
+        baseline, (slots, want, experts) = oracle_sample(case, data, plan, budget_rows=64, first_budget=4096 if with_cpu_baseline else None)
         if with_cpu_baseline:
             result["cpu_baseline"] = baseline
         # parity on the sample at full size: the device's down-projection rows for those slots
@@ -388,6 +498,8 @@ def measure(config, args, device, sustained, with_cpu_baseline):
         by_max, by_element = oracle.relative_errors(got, want)
         result["sample_parity"] = {"max_abs_over_max_ref": round(float(by_max), 6), "elementwise": round(float(by_element), 6),
                                    "identical_frac": round(float((got == want).mean()), 5), "rows": int(len(slots)),
+                                   "experts": [int(e) for e in experts],
+                                   "rows_note": "first and last sorted rows of the busiest, the median and the least non-empty expert",
                                    "bar": 2e-2}
     del stepper, data, out, plan
     gc.collect()
@@ -450,7 +562,7 @@ def main():
         per_config = {}
         for config in ALL_CONFIGS:
             if config == args.config:
-                measured = {k: v for k, v in top.items() if k != "cpu_baseline"}
+                measured = {k: v for k, v in top.items() if k != "cpu_baseline" or config in WHOLE_ON_CPU}
             else:
                 print(f"[bench] measuring {config}", file=sys.stderr, flush=True)
                 measured = measure(config, args, device, sustained, with_cpu_baseline=False)

@@ -1,4 +1,7 @@
-"""Seeded inputs of the five benchmark configurations, at full or reduced size, for the parity tests."""
+"""The five benchmark workloads: their shapes, router settings and seeded synthetic inputs, at full or reduced size.
+
+Read by bench.py (what it measures), by the parity tests (the same cases, mostly reduced) and by the smoke run.
+"""
 
 import dataclasses
 
@@ -77,22 +80,3 @@ def inputs(case: Case, seed: int = 0):
         shared = dict(gate=bank(case.d_model, case.d_ff, 1), up=bank(case.d_model, case.d_ff, 1),
                       down=bank(case.d_ff, case.d_model, 1))
     return dict(x=x, logits=torch.from_numpy(logits), bias=bias, banks=banks, shared=shared)
-
-
-def dequantized(bank):
-    """(values `[E, K, N]` fp32 as the reference's load decodes them, per-expert accumulator factor or None),
-    by the oracle's decoders."""
-    from oracle import moe_oracle as oracle
-
-    if isinstance(bank, formats.NvFp4):
-        words = bank.words.cpu().numpy().view(np.uint32)
-        return oracle.nvfp4_bank_decoded(words, bank.scales.cpu().numpy()), oracle.nvfp4_bank_factor(bank.scale.cpu().numpy())
-    if isinstance(bank, formats.Fp8Blocks):
-        return oracle.dequantize_fp8_blocks(bank.codes.cpu().numpy(), bank.scale_inv.cpu().numpy()), None
-    if isinstance(bank, formats.Fp8Channels):
-        return oracle.dequantize_fp8_channels(bank.codes.cpu().numpy(), bank.scales.cpu().numpy()), None
-    if isinstance(bank, formats.Bf16):
-        return bank.weights.float().cpu().numpy(), None
-    if isinstance(bank, formats.Mxfp4Blocks):
-        return oracle.decode_mxfp4(bank.blocks.cpu().numpy(), bank.scales.cpu().numpy()), None
-    raise TypeError(type(bank))

@@ -110,16 +110,19 @@ __global__ __launch_bounds__(256) void gate_rows_kernel(const bf16_t* __restrict
   const int lane = threadIdx.x % 64;
   const int token = blockIdx.x * 4 + threadIdx.x / 64;
   if (token >= tokens) return;
-  float sum = 0.0f;
+  // The logit's sum in float64 (each product of two bf16 values is exact there, and their sum is exact to 2^-53 of its
+  // terms whatever the order), rounded to fp32 and then to bf16, which is what the CPU oracle's float64 dot product gives;
+  // the logistic by the library's fixed-sequence exponential and an IEEE division, the oracle's own steps.
+  double sum = 0.0;
   for (int chunk = lane; chunk < depth / 8; chunk += 64) {
     const Bf16x8 values = *reinterpret_cast<const Bf16x8*>(x + static_cast<size_t>(token) * depth + static_cast<size_t>(chunk) * 8);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) sum += bf16_to_f32(values.v[i]) * bf16_round(kernel[chunk * 8 + i]);
+    for (int i = 0; i < 8; ++i) sum += static_cast<double>(bf16_to_f32(values.v[i])) * static_cast<double>(bf16_round(kernel[chunk * 8 + i]));
   }
 #pragma unroll
   for (int offset = 32; offset >= 1; offset >>= 1) sum += __shfl_xor(sum, offset, 64);
-  const float logit = bf16_round(sum);
-  const float gate = bf16_round(1.0f / (1.0f + expf(-logit)));
+  const float logit = bf16_round(static_cast<float>(sum));
+  const float gate = bf16_round(1.0f / (1.0f + exp_f32(-logit)));
   for (int chunk = lane; chunk < width / 8; chunk += 64) {
     const size_t at = static_cast<size_t>(token) * width + static_cast<size_t>(chunk) * 8;
     const Bf16x8 values = *reinterpret_cast<const Bf16x8*>(rows_in + at);

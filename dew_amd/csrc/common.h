@@ -94,6 +94,28 @@ __device__ __forceinline__ bf16_t gated_pair_rounded(float gate, float up, float
   return f32_to_bf16(u1 * q);
 }
 
+// e^x by Cody-Waite reduction and a degree-7 Taylor sum in Horner form, times 2^n in two exact steps
+// (the reference's portable exp, src/dew/nn/precision.py:470-488). The CPU oracle runs the same sequence, so a file that uses
+// it is compiled with contraction off (-ffp-contract=off): a fused multiply-add would round differently.
+__device__ __forceinline__ float exp_f32(float x) {
+  x = fminf(fmaxf(x, -104.0f), 90.0f);
+  const float n = rintf(x * 0x1.715476p+0f);
+  const float r = (x - n * 0x1.62e4p-1f) - n * 0x1.7f7d1cp-20f;
+  float p = 0x1.a01a02p-13f;               // 1/5040 ... 1/6 rounded to fp32
+  p = p * r + 0x1.6c16c2p-10f;
+  p = p * r + 0x1.111112p-7f;
+  p = p * r + 0x1.555556p-5f;
+  p = p * r + 0x1.555556p-3f;
+  p = p * r + 0.5f;
+  p = p * r + 1.0f;
+  p = p * r + 1.0f;
+  const int ni = static_cast<int>(n);
+  const int half = ni >> 1;  // floor(n / 2)
+  const float first = __uint_as_float(static_cast<uint32_t>(half + 127) << 23);
+  const float second = __uint_as_float(static_cast<uint32_t>(ni - half + 127) << 23);
+  return (p * first) * second;
+}
+
 // ---- prepared bank geometry (fragment-native atoms) ----
 // FP8 atom: 32 n x 32 k bytes = 1 KiB; lane l = (g = l / 32, n = l % 32) holds k = 16 g .. 16 g + 15.
 // FP4 atom: 32 n x 64 k nibbles = 1 KiB; lane l holds k = 32 g .. 32 g + 31 (byte j: low nibble k = 32 g + 2 j).

@@ -254,11 +254,17 @@ __global__ __launch_bounds__(THREADS) void permute_small_kernel(PermuteParams p)
     const int count = __popcll(same);
     int position = 0;
     if (valid) position = mine[bucket] + rank;
-    // (the running positions are the wavefront's own: its reads above are done before the write below is issued, and
-    // the next round's reads come after it in the same queue; no other wavefront touches them)
+    // The running positions are the wavefront's own (no other wavefront touches them), so no block barrier is needed,
+    // only an order between this wavefront's lanes: every lane's read above before the one lane's write below, and that
+    // write before the next round's reads. The wavefront-scope fences state that order to the compiler and the memory
+    // model (they cost no instruction: a wavefront's LDS operations are issued and served in order).
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     if (valid && rank == count - 1) mine[bucket] = position + 1;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     if (valid) {
       p.order[position] = slot;
       p.rows[position] = row_of(p, slot);

@@ -15,27 +15,6 @@ constexpr int kWave = 64;
 constexpr int kMaxPerLane = 8;   // experts <= 512
 constexpr int kRouteWaves = 4;   // tokens per 256-thread block
 
-// e^x by Cody-Waite reduction and a degree-7 Taylor sum in Horner form, times 2^n in two exact steps
-// (the reference's portable exp, src/dew/nn/precision.py:470-488).
-__device__ __forceinline__ float exp_f32(float x) {
-  x = fminf(fmaxf(x, -104.0f), 90.0f);
-  const float n = rintf(x * 0x1.715476p+0f);
-  const float r = (x - n * 0x1.62e4p-1f) - n * 0x1.7f7d1cp-20f;
-  float p = 0x1.a01a02p-13f;               // 1/5040 ... 1/6 rounded to fp32
-  p = p * r + 0x1.6c16c2p-10f;
-  p = p * r + 0x1.111112p-7f;
-  p = p * r + 0x1.555556p-5f;
-  p = p * r + 0x1.555556p-3f;
-  p = p * r + 0.5f;
-  p = p * r + 1.0f;
-  p = p * r + 1.0f;
-  const int ni = static_cast<int>(n);
-  const int half = ni >> 1;  // floor(n / 2)
-  const float first = __uint_as_float(static_cast<uint32_t>(half + 127) << 23);
-  const float second = __uint_as_float(static_cast<uint32_t>(ni - half + 127) << 23);
-  return (p * first) * second;
-}
-
 // DeepSeek V4's score sqrt(softplus(x)) (src/dew/nn/moe.py:303-313), formed in float64 (softplus as max(x, 0) +
 // log1p(exp(-|x|)), the square root IEEE) and rounded once to fp32: the CPU oracle's arithmetic for this score.
 __device__ __forceinline__ float sqrt_softplus_f32(float x) {
@@ -293,13 +272,20 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
     }
   }
 
-  // A token whose experts are given takes them as they come (ids outside the experts are held to the nearest one, so
-  // every read below stays in range); the wavefront is one token, so the branch is uniform.
+  // A token whose experts are given takes them as they come; the wavefront is one token, so the branch is uniform. A given
+  // id outside [0, experts) (a dropped slot's sentinel in a replayed record) is written back as it came, with weight zero
+  // and no part in the other slots' normalization: the reference passes such ids through (`chosen_experts`,
+  // src/dew/nn/moe.py:202-224) and its sort drops the slot. Its reads below go to the nearest expert, to stay in range.
   const bool replayed = p.given != nullptr && (p.covered == nullptr || p.covered[token] != 0);
   // top-k: k rounds of a wave-wide argmax, ties to the lower index
   unsigned taken_mask = 0u;
-  int my_choice = 0;
-  if (replayed && lane < p.top_k) my_choice = min(max(p.given[static_cast<size_t>(token) * p.top_k + lane], 0), p.experts - 1);
+  int my_choice = 0, given_id = 0;
+  bool in_range = true;
+  if (replayed && lane < p.top_k) {
+    given_id = p.given[static_cast<size_t>(token) * p.top_k + lane];
+    in_range = given_id >= 0 && given_id < p.experts;
+    my_choice = min(max(given_id, 0), p.experts - 1);
+  }
   for (int round = 0; round < (replayed ? 0 : p.top_k); ++round) {
     Best b;
     b.value = ninf;
@@ -318,7 +304,7 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
   }
 
   // gate weights: lane j < k owns the j-th choice
-  const bool owner = lane < p.top_k;
+  const bool owner = lane < p.top_k && in_range;
   float chosen_logit = owner ? row[my_choice] : ninf;
   if (p.softcap > 0.0f && owner) chosen_logit = capped(chosen_logit, p.softcap);
   float weight = 0.0f;
@@ -342,9 +328,9 @@ __global__ __launch_bounds__(kWave* kRouteWaves) void route_kernel(RouteParams p
     }
   }
   weight = weight * p.scaling;
-  if (active && owner) {
-    p.weights[static_cast<size_t>(token) * p.top_k + lane] = weight;
-    p.indices[static_cast<size_t>(token) * p.top_k + lane] = my_choice;
+  if (active && lane < p.top_k) {
+    p.weights[static_cast<size_t>(token) * p.top_k + lane] = in_range ? weight : 0.0f;
+    p.indices[static_cast<size_t>(token) * p.top_k + lane] = replayed ? given_id : my_choice;
   }
 }
 

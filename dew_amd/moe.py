@@ -318,26 +318,28 @@ def _sorted_locally(indices: torch.Tensor, num_experts: int, shared_rows: int = 
     return plan, GroupSizes(plan.sizes, plan.offsets)
 
 
-_STACKED = {}
-"""Routed banks with the shared expert's behind them (`with_shared_expert`), by the identities of the banks stacked."""
-
-
 def with_shared_expert(routed, shared):
-    """The routed experts' three banks with the always-on expert's matrices stacked behind them as expert #E, so that
-    the routed launches multiply the shared expert too (src/dew/nn/moe.py:1497-1503 computes it as a dense MLP of its
-    own: two more launches). None where the formats or shapes do not stack. The stack is formed once per pair of banks."""
+    """The routed experts' three banks with the always-on expert's matrices behind them as expert #E, each as ONE prepared
+    bank, so that the routed launches multiply the shared expert too (src/dew/nn/moe.py:1497-1503 computes it as a dense MLP
+    of its own: two more launches). None where the formats or shapes do not stack.
+
+    Memory: the two banks are joined in the reference's layout only for the length of the re-layout; what stays is the
+    prepared stack alone, held on the routed bank object (as its own `_prepared` form would be) and released with it, so a
+    layer that fuses its shared expert holds the caller's banks and one prepared copy of E + 1 experts, the same bytes as the
+    unfused arrangement's two prepared banks. At load the transient joined copy adds one more bank's bytes (DeepSeek-V3's
+    256 x 7168 x 2048 FP8 banks: 3.8 GB each) until the re-layout has run."""
     found = []
     for mine, theirs in zip(routed, shared, strict=True):
         if isinstance(mine, (formats.Layered, ops.PreparedBank)) or torch.is_tensor(mine) or torch.is_tensor(theirs):
             return None
-        key = (id(mine), id(theirs))
-        held = _STACKED.get(key)
-        if held is None or held[0] is not mine or held[1] is not theirs:
+        held = getattr(mine, "_with_shared", None)
+        if held is None or held[0] is not theirs:
             joined = formats.stacked([mine, theirs])
             if joined is None:
                 return None
-            held = _STACKED[key] = (mine, theirs, joined)
-        found.append(held[2])
+            held = (theirs, ops.prepare(joined))      # `joined` itself is dropped here: only its prepared form is kept
+            object.__setattr__(mine, "_with_shared", held)
+        found.append(held[1])
     return tuple(found)
 
 

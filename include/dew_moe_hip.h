@@ -128,7 +128,9 @@ int dew_moe_route_with(const dew_moe_router* router /* host */, const float* log
  *    scores + media_bias in place of scores + bias (`selection`, :516-524);
  *  - given [T,k], covered [T] (`chosen_experts`, :202-224: a replayed record of an engine's routing; and the hash router's
  *    `tid2eid[token ids]`, :500-507): token t uses given[t, :] in that order in place of its own top-k, where `covered` is
- *    null or covered[t] != 0. An id outside [0, experts) is held to the nearest expert.
+ *    null or covered[t] != 0. An id outside [0, experts) (a dropped slot's sentinel in a record) is written to `indices` as
+ *    it came, with weight 0 and no part in the token's other weights; dew_moe_permute puts such a slot in no group, so the
+ *    products write its row as zeros, as the reference's sort drops it (`_sorted_locally`, :1101-1128).
  * The weights are the router's for the experts used (:483-494). All four null is dew_moe_route_with.                  */
 int dew_moe_route_call(const dew_moe_router* router /* host */, const float* logits, const float* bias /* nullable */,
                        const float* media_bias /* nullable [E] */, const uint8_t* media /* nullable [T] */,

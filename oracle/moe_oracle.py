@@ -440,14 +440,29 @@ def route(logits, top_k_count, *, score_function="softmax", normalize_weights=Tr
                                          excluded_group_score=excluded_group_score, media=media, media_bias=media_bias,
                                          blocks=blocks, block_experts=block_experts)
     _, indices = top_k(selection, top_k_count)
+    valid = None
     if given is not None:      # `chosen_experts` (src/dew/nn/moe.py:202-224): a replayed record, or the hash table's rows (:500-507)
         given = np.asarray(given).astype(np.int32)
         indices = given if covered is None else np.where(np.asarray(covered, bool)[..., None], given, indices).astype(np.int32)
+        # ids outside the experts (a dropped slot's sentinel) pass through as they are; such a slot weighs nothing and takes
+        # no part in the other slots' normalization (the sort drops it, src/dew/nn/moe.py:1101-1128)
+        valid = (indices >= 0) & (indices < logits.shape[-1])
+        if valid.all():
+            valid = None
+    safe = indices if valid is None else np.clip(indices, 0, logits.shape[-1] - 1)
     if normalize_weights and score_function == "softmax" and not bias_in_weights and not weight_sum_min:
-        weights = expert_softmax(np.take_along_axis(logits, indices, axis=-1))        # moe.py:194-199,485
+        if valid is None:
+            weights = expert_softmax(np.take_along_axis(logits, safe, axis=-1))        # moe.py:194-199,485
+        else:
+            chosen = np.where(valid, np.take_along_axis(logits, safe, axis=-1), F32(-np.inf)).astype(F32)
+            with np.errstate(invalid="ignore", divide="ignore"):
+                shifted = np.where(valid, exp_f32(np.where(valid, chosen - chosen.max(axis=-1, keepdims=True), F32(0))), F32(0)).astype(F32)
+                weights = (shifted / _sum_rounded_once(shifted)[..., None]).astype(F32)
     else:
         gating = (scores + np.asarray(bias, F32)).astype(F32) if bias_in_weights else scores
-        weights = np.take_along_axis(gating, indices, axis=-1)
+        weights = np.take_along_axis(gating, safe, axis=-1)
+        if valid is not None:
+            weights = np.where(valid, weights, F32(0)).astype(F32)
         if normalize_weights:
             total = weights[..., 0].copy()
             for j in range(1, top_k_count):
@@ -456,6 +471,8 @@ def route(logits, top_k_count, *, score_function="softmax", normalize_weights=Tr
             if weight_sum_min:
                 total = np.maximum(total, F32(weight_sum_min))
             weights = (weights / total[..., None]).astype(F32)
+    if valid is not None:
+        weights = np.where(valid, weights, F32(0)).astype(F32)
     return (weights * F32(routed_scaling_factor)).astype(F32), indices
 
 
@@ -1150,7 +1167,7 @@ def gated_rows(x, kernel, rows):
     x = np.asarray(x, F32)
     kernel = bf16_round(np.asarray(kernel, F32).reshape(-1))
     logit = bf16_round((x.astype(np.float64) @ kernel.astype(np.float64)).astype(F32))
-    gate = bf16_round((1.0 / (1.0 + np.exp(-logit.astype(np.float64)))).astype(F32))
+    gate = bf16_round(logistic(logit))   # (fp32, the fixed-sequence exponential: the device kernel's own steps, so the gates agree bit for bit)
     return bf16_round((np.asarray(rows, F32) * gate[:, None]).astype(F32))
 
 

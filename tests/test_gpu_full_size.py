@@ -1,12 +1,12 @@
 """The benchmark configurations at their full sizes, where the CPU oracle cannot follow the whole layer: checked
 through properties that do not depend on size (the sort's invariants, the router on a sample of tokens, the combine
-recomputed from the slots, bit-identical repeats) and against the oracle on a bounded sample of rows of the busiest
-expert at full width. Inputs are generated on the device exactly as the benchmark generates them."""
+recomputed from the slots, bit-identical repeats) and against the oracle on a bounded sample of rows at full width:
+the first and last rows of three experts (the busiest, the median, the least non-empty one), and c3 whole. Inputs are generated on the device exactly as the benchmark generates them."""
 
 import numpy as np
 import pytest
 import torch
-from moe_cases import CONFIGS
+from bench_aids.workloads import CONFIGS
 
 import bench
 from oracle import moe_oracle as oracle
@@ -58,12 +58,24 @@ def test_full_size_configuration(name):
     assert torch.equal(plan.offsets.long(), torch.cat([torch.zeros(1, dtype=torch.long, device=device), torch.cumsum(plan.sizes.long(), 0)]))
     assert torch.equal(plan.rows.long(), order // k)
 
-    # the busiest expert's first rows through all three projections against the oracle, and the combine from the slots
-    _, (sampled_slots, want_down) = bench.oracle_sample(case, data, plan, budget_rows=48)
+    # first and last rows of the busiest, the median and the least non-empty expert through all three projections against the
+    # oracle (a group's last rows are the ones a partial last tile, or c4's second launch of 64-row tiles, multiplies); c3,
+    # whose experts hold 1 to 10 rows, is followed whole: every routed row, the routing and the layer's output
     _, whole_plan = stepper()
     slots = stepper.project(whole_plan)                             # c2: on split rows, the library's rule for its groups
     assert stepper.on_split_rows() == (name == "c2")
-    got_down = slots[torch.from_numpy(sampled_slots).to(device).long()].float().cpu().numpy()
+    if name in bench.WHOLE_ON_CPU:
+        _, (want_out_oracle, trace) = bench.oracle_whole(case, data)
+        assert np.array_equal(indices.cpu().numpy(), trace["indices"]) and np.array_equal(weights.cpu().numpy(), trace["weights"])
+        got_down, want_down = slots[:routed].float().cpu().numpy(), trace["slots"].reshape(routed, case.d_model)
+        sampled_experts = list(range(experts))
+        peak, elementwise = oracle.relative_errors(out.float().cpu().numpy(), want_out_oracle)
+        assert peak <= 6e-3 and elementwise <= 2e-2, (peak, elementwise)
+    else:
+        _, (sampled_slots, want_down, sampled_experts) = bench.oracle_sample(case, data, plan, budget_rows=64)
+        got_down = slots[torch.from_numpy(sampled_slots).to(device).long()].float().cpu().numpy()
+        assert len(sampled_experts) == 3
+    assert len(want_down) >= 64
     peak, elementwise = oracle.relative_errors(got_down, want_down)
     assert peak <= 2e-2 and elementwise <= 2e-2, (peak, elementwise)
     assert peak <= 6e-3
@@ -74,7 +86,7 @@ def test_full_size_configuration(name):
     want_out = total.to(torch.bfloat16)
     if case.shared:
         # the shared expert's rows (group #E of the same launches) against the oracle's dense SwiGLU MLP on a sample of tokens
-        from moe_cases import dequantized
+        from oracle.banks import dequantized
         sampled = np.arange(0, tokens, tokens // 24)[:24]
         matrices = [dequantized(data["shared"][n].to("cpu"))[0][0] for n in ("gate", "up", "down")]
         want_shared = oracle.gated_mlp(data["x"][torch.from_numpy(sampled).to(device)].float().cpu().numpy(), *matrices)

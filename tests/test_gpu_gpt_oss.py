@@ -5,7 +5,8 @@ import numpy as np
 import pytest
 import torch
 
-from moe_cases import dequantized, quantize
+from bench_aids.workloads import quantize
+from oracle.banks import dequantized
 from oracle import moe_oracle as oracle
 
 pytestmark = pytest.mark.gpu
@@ -288,7 +289,8 @@ def test_a_decode_step_on_many_fp4_experts_of_a_ragged_width(ops, quant):
     256 >= 640) on a width that is no whole 256s (2688 = 10 strips and 128 columns): the plain product with its bias and
     GPT-OSS's gated one, a few rows an expert and several experts empty, against the oracle."""
     from dew_amd import codecs, formats, gemm
-    from moe_cases import dequantized, quantize
+    from bench_aids.workloads import quantize
+    from oracle.banks import dequantized
 
     rng = np.random.default_rng(23)
     experts, depth, width = 64, 256, 2688

@@ -7,7 +7,8 @@ import dataclasses
 import numpy as np
 import pytest
 import torch
-from moe_cases import CONFIGS, dequantized, inputs, quantize
+from bench_aids.workloads import CONFIGS, inputs, quantize
+from oracle.banks import dequantized
 
 from oracle import moe_oracle as oracle
 
@@ -119,7 +120,8 @@ def test_a_logit_softcap_caps_what_every_reader_of_the_logits_reads(ops, score_f
                                                             ("sigmoid", 64, 8, dict(expert_groups=8, groups_per_token=3))])
 def test_given_experts_weigh_as_the_router_weighs_them(ops, score_function, experts, k, extra):
     """A replayed record's or a hash table's experts (`dew_moe_route_call`): every token covered, and some; ids
-    outside the experts held to the nearest; the router's own choice given back is its own routing."""
+    outside the experts (a dropped slot's sentinel) come back as given with weight zero and the sort drops their slots; the
+    router's own choice given back is its own routing."""
     rng = np.random.default_rng(experts * 7 + k)
     tokens = 271
     logits = (rng.standard_normal((tokens, experts)) * 2).astype(np.float32)
@@ -139,10 +141,15 @@ def test_given_experts_weigh_as_the_router_weighs_them(ops, score_function, expe
     again_w, again_i = ops.route(torch.from_numpy(logits).cuda(), k, given=own_i, **on_device, **settings)
     assert torch.equal(again_i, own_i) and torch.equal(again_w, own_w)
     wild = table.copy()
-    wild[::3, 0], wild[1::3, -1] = -5, experts + 9
+    wild[::3, 0], wild[1::3, -1], wild[5] = experts, experts + 9, -5       # the sentinel itself, a corrupt id, a token with no expert at all
     got_w, got_i = ops.route(torch.from_numpy(logits).cuda(), k, given=torch.from_numpy(wild).cuda(), **on_device, **settings)
-    want_w, want_i = oracle.route(logits, k, bias=bias, given=np.clip(wild, 0, experts - 1), **settings)
-    assert np.array_equal(got_i.cpu().numpy(), want_i) and np.array_equal(got_w.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
+    want_w, want_i = oracle.route(logits, k, bias=bias, given=wild, **settings)
+    assert np.array_equal(want_i, wild) and np.array_equal(got_i.cpu().numpy(), want_i)
+    assert np.array_equal(got_w.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
+    outside = (wild < 0) | (wild >= experts)
+    assert not got_w.cpu().numpy()[outside].any() and not got_w.cpu().numpy()[5].any()
+    plan = ops.sort_by_expert(got_i, experts)                                # the sort drops those slots: they belong to no group
+    assert int(plan.sizes.sum()) == int((~outside).sum()) and int(plan.offsets[-1]) == int((~outside).sum())
     with pytest.raises(ops.KernelError, match="replayed routing"):
         ops.route(torch.from_numpy(logits).cuda(), k, given=torch.from_numpy(table[:, :1].copy()).cuda(), **settings)
     with pytest.raises(ops.KernelError, match="coverage"):

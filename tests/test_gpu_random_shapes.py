@@ -4,7 +4,8 @@ one-row groups included), gathers, scatters, biases and every tile height, each 
 import numpy as np
 import pytest
 import torch
-from moe_cases import dequantized, quantize
+from bench_aids.workloads import quantize
+from oracle.banks import dequantized
 
 from oracle import moe_oracle as oracle
 

@@ -5,7 +5,8 @@ output within the bars of the expert MLP's tests."""
 import numpy as np
 import pytest
 import torch
-from moe_cases import dequantized, quantize
+from bench_aids.workloads import quantize
+from oracle.banks import dequantized
 
 from oracle import moe_oracle as oracle
 

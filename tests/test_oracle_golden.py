@@ -589,6 +589,17 @@ def test_given_experts_take_the_routers_weights_for_them():
             truth = truth / (truth.sum(-1, keepdims=True) + 1e-20)
         truth = truth * settings.get("routed_scaling_factor", 1.0)
         assert np.abs(mixed_w[covered] - truth[covered]).max() <= 2 * ROUTER_TOLERANCE
+        # an id outside the experts (a dropped slot's sentinel, src/dew/nn/moe.py:1101-1128) passes through with weight zero,
+        # and the token's other slots weigh as if the record had held them alone
+        dropped = table.copy()
+        dropped[::2, 1], dropped[1::4, 3] = 16, -1
+        dropped_w, dropped_i = oracle.route(logits, 4, given=dropped, **settings)
+        outside = (dropped < 0) | (dropped >= 16)
+        assert np.array_equal(dropped_i, dropped) and not dropped_w[outside].any()
+        kept = np.where(outside, 0.0, np.take_along_axis(scores, np.clip(dropped, 0, 15).astype(np.int64), -1))
+        if settings.get("normalize_weights", True):
+            kept = kept / (kept.sum(-1, keepdims=True) + 1e-20)
+        assert np.abs(dropped_w - kept * settings.get("routed_scaling_factor", 1.0)).max() <= 2 * ROUTER_TOLERANCE
 
 
 def test_media_tokens_are_routed_by_their_own_bias():
