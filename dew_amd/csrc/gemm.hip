@@ -38,6 +38,8 @@ typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;  // a 16-byte register quad (native vector: stays in VGPRs)
 typedef __attribute__((ext_vector_type(8))) int i32x8_t;       // an operand of the scaled matrix instruction
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
 
 // Kernel-side format of an MXFP4 bank multiplied by activation rows already split into two e4m3 terms
 // (dew_moe_split_rows): v_mfma_scale_f32_32x32x64_f8f6f4 takes the FP4 codes and their power-of-two block scales
@@ -67,6 +69,13 @@ constexpr int kFormatBf16Window = 21;
 // takes half the cycles of the FP8 x FP4 one, so a product's two instructions take three quarters of the time; the
 // second term is exact only for elements within two binades of their 32-deep block's largest (see split.hip).
 constexpr int kFormatMxSplit6 = 22;
+// Kernel-side format of a general NVFP4 bank (e4m3 block scales with mantissas) multiplied by activation rows brought to
+// f16 under one power-of-two scale a row (dew_moe_rows_f16), on v_mfma_f32_32x32x16_f16. A code times its block scale has
+// at most six significant bits and lies in 2^-10 .. 2688: exact in f16, formed by one packed conversion and one packed f16
+// multiply for two codes (the bf16 form needs the multiply in fp32 and a packed rounding: twice the vector instructions).
+// Every product is the bf16 path's product times a power of two and the sums are fp32 either way, so the launch returns
+// the bf16-operand launch's bits.
+constexpr int kFormatNvF16 = 23;
 
 constexpr int BK = 64;
 constexpr int kThreads = 256;
@@ -159,6 +168,16 @@ __device__ __forceinline__ bf16x8_t fragment_fp4_pow2(uint32_t word, float scale
       __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 3))});
 }
 
+// The same eight codes as f16 values times the block scale itself (an e4m3 value is exact in f16, and so is its product
+// with an E2M1 code): one packed conversion and one packed multiply for two codes.
+__device__ __forceinline__ bf16x8_t fragment_fp4_f16(uint32_t word, _Float16 scale) {
+  const f16x2_t both = {scale, scale};
+  const f16x2_t a = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, 1.0f, 0) * both, b = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, 1.0f, 1) * both;
+  const f16x2_t c = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, 1.0f, 2) * both, d = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, 1.0f, 3) * both;
+  return __builtin_bit_cast(bf16x8_t, u32x4_t{__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b),
+                                              __builtin_bit_cast(uint32_t, c), __builtin_bit_cast(uint32_t, d)});
+}
+
 // Bytes of one row's block scales (one e8m0 byte for 128 elements), padded to whole 16-byte loads.
 __host__ __device__ constexpr int block_scale_pitch(int elements) { return (elements / 128 + 15) / 16 * 16; }
 
@@ -205,7 +224,9 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   // Unquantized and FP4 banks (their atoms are 64 deep and 32 columns wide at most) take a depth in whole 64-deep steps and a
   // width in whole 32-column atoms, close to the multiples of 8 of the reference's own grouped kernel: a strip past the width
   // multiplies columns it does not store. (GPT-OSS's experts are 2880 wide: 45 steps, 90 atoms, no whole 128s.)
-  constexpr bool kRagged = FORMAT == DEW_MOE_W_BF16 || FORMAT == DEW_MOE_W_MXFP4 || FORMAT == DEW_MOE_W_NVFP4;
+  constexpr bool kNvF16 = FORMAT == kFormatNvF16;  // f16 rows under a scale a row, a general NVFP4 bank decoded to f16
+  static_assert(!kNvF16 || MODE == kSwigluOfTwo, "f16 rows: the paired launch");
+  constexpr bool kRagged = FORMAT == DEW_MOE_W_BF16 || FORMAT == DEW_MOE_W_MXFP4 || FORMAT == DEW_MOE_W_NVFP4 || kNvF16;
   constexpr bool kGated = MODE == kInterleavedGated;
   constexpr int kOutBN = kGated ? BN / 2 : BN;  // output columns of the tile
   static_assert(WM * WN == 4 && BM % (32 * WM) == 0 && BN % (32 * WN) == 0 && BM % 32 == 0, "tile shape");
@@ -216,7 +237,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   constexpr bool kLo6 = FORMAT == kFormatMxSplit6;      // the second term of a row in FP6 (e2m3), its scale beside it
   constexpr bool kSplit = FORMAT == kFormatMxSplit || FORMAT == kFormatMxSplitBlocks || kLo6 || kFp8A;  // A arrives as 8-bit codes
   constexpr bool kBlockScales = FORMAT == kFormatMxSplitBlocks || kFp8Rows;
-  constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4 || (kSplit && !kFp8A);
+  constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4 || kNvF16 || (kSplit && !kFp8A);
   constexpr bool kPow2 = FORMAT == DEW_MOE_W_MXFP4 || (kSplit && !kFp8A);
   constexpr bool kBlockBank = FORMAT == DEW_MOE_W_FP8_BLOCK || kFp8Rows;  // one fp32 scale per 128 x 128 weights
   constexpr int kMatrices = PAIRED ? 2 : 1;
@@ -244,6 +265,8 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   // FP8 128 x 128 blocks: the scales of the block's column blocks down the whole depth, read once
   constexpr int kScaleColumns = kBlockBank ? kMatrices * (BN / 128) : 1;
   __shared__ float depth_scales[kScaleColumns][kBlockBank ? kMaxDepthBlocks : 1];
+
+  __shared__ float row_factor[kNvF16 ? BM : 1];  // f16 rows: 2^s of each of the tile's rows, which its sums are owed
 
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
 
@@ -359,6 +382,13 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
     return;
   }
   const int wm0 = (wave / WN) * (BM / WM), wn0 = (wave % WN) * (BN / WN);
+  if constexpr (kNvF16) {
+    static_assert(!kNvF16 || BM <= kThreads, "one thread fetches one row's scale");
+    if (tid < BM) {  // (read in the epilogue, behind the loop's barriers)
+      const int sorted = row0 + min(tid, valid_rows - 1);
+      row_factor[tid] = __uint_as_float(static_cast<uint32_t>(p.a_scale[p.gather ? p.gather[sorted] : sorted]) << 23);
+    }
+  }
 
   // ---- A loader. One global_load_lds_dwordx4 of a wavefront fills 1 KiB of LDS, lane l landing at byte 16 l:
   // 8 rows of a stage, lane l = row l / 8, stored chunk l % 8. The lane therefore fetches the logical chunk
@@ -526,6 +556,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   i32x8_t a_term[2][kSplit ? TI : 1];  // split activations: [0] the hi term of a step, [1] its lo term
   int a_lo_scale[kLo6 ? TI : 1];       // an FP6 second term's e8m0 scale of the lane's 32 depths (it lies behind the codes)
   float fp4_scale[kTiles];
+  _Float16 fp4_half[kNvF16 ? kTiles : 1];  // f16 rows: the block scale as f16
   // a term of a 32-depth block is 32 bytes: the lane's block lane / 32 of the step holds hi in its chunks 0-1, lo in 2-3
   // The lane's four chunks of its first row tile, as chunk indices into a stage: computed once, so that a phase's
   // reads are the stage's base plus one of these plus 32 rows (a constant) a row tile further.
@@ -563,7 +594,12 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   auto dequantize = [&](auto set, auto kk, auto into, int step) __attribute__((always_inline)) {
 #pragma unroll
     for (int t = 0; t < kTiles; ++t) {
-      if constexpr (kFp4) {
+      if constexpr (kNvF16) {
+        if constexpr (kk.value % 2 == 0)  // slices 0, 1 lie in the lane's first 16-deep block, 2, 3 in its second
+          fp4_half[t] = static_cast<_Float16>(kk.value == 0 ? __builtin_amdgcn_cvt_f32_fp8(s_regs[set.value][t], 0)
+                                                            : __builtin_amdgcn_cvt_f32_fp8(s_regs[set.value][t], 1));
+        b_frag[into.value][t] = fragment_fp4_f16(b_regs[set.value][t][0][kk.value], fp4_half[t]);
+      } else if constexpr (kFp4) {
         if constexpr (kk.value % 2 == 0)  // slices 0, 1 lie in the lane's first 16-deep block, 2, 3 in its second
           fp4_scale[t] = (kk.value == 0 ? __builtin_amdgcn_cvt_f32_fp8(s_regs[set.value][t], 0)
                                         : __builtin_amdgcn_cvt_f32_fp8(s_regs[set.value][t], 1)) * 0.00390625f;
@@ -596,8 +632,13 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
 #pragma unroll
       for (int i = 0; i < TI; ++i)
 #pragma unroll
-        for (int j = 0; j < TJ; ++j)
-          acc[m][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_frag[from.value][i], b_frag[from.value][m * TJ + j], acc[m][i][j], 0, 0, 0);
+        for (int j = 0; j < TJ; ++j) {
+          if constexpr (kNvF16)
+            acc[m][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a_frag[from.value][i]),
+                                                                  __builtin_bit_cast(f16x8_t, b_frag[from.value][m * TJ + j]), acc[m][i][j], 0, 0, 0);
+          else
+            acc[m][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_frag[from.value][i], b_frag[from.value][m * TJ + j], acc[m][i][j], 0, 0, 0);
+        }
   };
 
   // Split activations: one scaled instruction multiplies 64 depths of one term by the stored FP4 codes under
@@ -678,7 +719,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   constexpr std::integral_constant<int, kTiles> b4{};
   constexpr std::integral_constant<int, kTiles> all_tiles{};
   constexpr int kMfmas = kMatrices * TI * TJ;
-  constexpr int kDequantOps = kBf16 ? 0 : kTiles * (kPow2 ? 5 : 17);  // vector instructions to dequantize one slice
+  constexpr int kDequantOps = kBf16 ? 0 : kTiles * (kPow2 ? 5 : kNvF16 ? 10 : 17);  // vector instructions to dequantize one slice
   constexpr int kLoadsPerTile = kAtoms + (kFp4 || kMxRows ? 1 : 0);
   constexpr int kLoadsPerPhase = (kRowLoads + 3) / 4 + ((kTiles + 3) / 4) * kLoadsPerTile;
   // s_waitcnt vmcnt(kYounger) lgkmcnt(0): everything but the kYounger youngest vector-memory operations is done.
@@ -847,8 +888,9 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   float factor0 = 1.0f, factor1 = 1.0f;
   if (kFp4) {  // the 2^8 the decode owes times the expert's tensor scale (src/dew/nn/kernels/gemm.py:660-662)
     // (the scaled instruction applies the block scales themselves, not their 2^-8)
-    factor0 = (kSplit ? 1.0f : 256.0f) * p.w0.tensor_scale[expert];
-    if (PAIRED) factor1 = (kSplit ? 1.0f : 256.0f) * p.w1.tensor_scale[expert];
+    // (f16 rows: the codes times their block scales as they are, no 2^-8; each row's own 2^s joins below)
+    factor0 = (kSplit || kNvF16 ? 1.0f : 256.0f) * p.w0.tensor_scale[expert];
+    if (PAIRED) factor1 = (kSplit || kNvF16 ? 1.0f : 256.0f) * p.w1.tensor_scale[expert];
   }
   float window_factor = 1.0f;
   if constexpr (kWindow) window_factor = (p.factor0 ? *p.factor0 : 1.0f) * (p.factor1 ? *p.factor1 : 1.0f);
@@ -932,12 +974,16 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
             // the lane's rows q (low half) and q + 1 (high half) of its column, rounded
             uint32_t mine;
             if constexpr (PAIRED) {
+              // (f16 rows: a row's sums times its own 2^s as well, an exact factor of the expert's)
+              const int lane_row = kNvF16 ? wm0 + 32 * i + 8 * (q / 4) + 4 * (lane / 32) + q % 4 : 0;
+              const float first0 = kNvF16 ? factor0 * row_factor[lane_row] : factor0, first1 = kNvF16 ? factor1 * row_factor[lane_row] : factor1;
+              const float second0 = kNvF16 ? factor0 * row_factor[lane_row + 1] : factor0, second1 = kNvF16 ? factor1 * row_factor[lane_row + 1] : factor1;
               if (plain_swiglu) {
-                mine = swiglu_rounded(acc[0][i][j][q] * factor0, acc[kMatrices - 1][i][j][q] * factor1) |
-                       (static_cast<uint32_t>(swiglu_rounded(acc[0][i][j][q + 1] * factor0, acc[kMatrices - 1][i][j][q + 1] * factor1)) << 16);
+                mine = swiglu_rounded(acc[0][i][j][q] * first0, acc[kMatrices - 1][i][j][q] * first1) |
+                       (static_cast<uint32_t>(swiglu_rounded(acc[0][i][j][q + 1] * second0, acc[kMatrices - 1][i][j][q + 1] * second1)) << 16);
               } else {  // a clamp or the GeGLU gate (the same for every lane: a branch, not a select)
-                mine = gated_rounded(acc[0][i][j][q] * factor0, acc[kMatrices - 1][i][j][q] * factor1, p.limit, p.gating) |
-                       (static_cast<uint32_t>(gated_rounded(acc[0][i][j][q + 1] * factor0, acc[kMatrices - 1][i][j][q + 1] * factor1, p.limit, p.gating)) << 16);
+                mine = gated_rounded(acc[0][i][j][q] * first0, acc[kMatrices - 1][i][j][q] * first1, p.limit, p.gating) |
+                       (static_cast<uint32_t>(gated_rounded(acc[0][i][j][q + 1] * second0, acc[kMatrices - 1][i][j][q + 1] * second1, p.limit, p.gating)) << 16);
               }
             } else if constexpr (kFp4) {
               mine = pack_bf16(acc[0][i][j][q] * factor0 + bias[j], acc[0][i][j][q + 1] * factor0 + bias[j]);
@@ -1631,6 +1677,45 @@ static int gateup_swiglu_of(const char* who, const void* x, const int32_t* gathe
   p.gating = activation;
   p.limit = limit > 0.0f ? bf16_round_host(limit) : 0.0f;  // the clamp is compared in the operands' dtype
   return launch<kSwigluOfTwo>(who, p, gate->format, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int dew_moe_gateup_gated_f16(const void* x_f16, const uint8_t* x_scale, const int32_t* gather, const int32_t* offsets,
+                                        const int32_t* group_sizes, const dew_moe_bank* gate, const dew_moe_bank* up, int32_t activation,
+                                        float limit, void* hidden, int32_t rows, void* stream) {
+  using namespace dew;
+  const char* who = "dew_moe_gateup_gated_f16";
+  DEW_REQUIRE(activation == DEW_MOE_GATE_SILU || activation == DEW_MOE_GATE_GELU_TANH,
+              "%s: the gate's activation %d is neither silu (0: swiglu) nor the tanh gelu (1: geglu)", who, activation);
+  DEW_REQUIRE(limit >= 0.0f, "%s: the clamp limit %g must be positive (0: none)", who, static_cast<double>(limit));
+  if (int rc = check_bank(who, gate, "gate")) return rc;
+  if (int rc = check_bank(who, up, "up")) return rc;
+  DEW_REQUIRE(gate->format == DEW_MOE_W_NVFP4 && up->format == DEW_MOE_W_NVFP4,
+              "%s: f16 rows multiply NVFP4 banks whose block scales carry mantissas (an MXFP4 bank's power-of-two scales cost "
+              "nothing on bf16 rows: dew_moe_gateup_gated); these are formats %d and %d", who, gate->format, up->format);
+  DEW_REQUIRE(gate->experts == up->experts && gate->depth == up->depth && gate->width == up->width,
+              "%s: gate [%d, %d, %d] and up [%d, %d, %d] differ", who, gate->experts, gate->depth, gate->width, up->experts, up->depth,
+              up->width);
+  DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
+  if (rows == 0) return DEW_MOE_OK;
+  DEW_REQUIRE((offsets != nullptr) != (group_sizes != nullptr), "%s: the groups come as offsets [E + 1] or as group_sizes [E], one of them", who);
+  DEW_REQUIRE(x_f16 && x_scale && hidden, "%s: x_f16, x_scale and hidden must not be null", who);
+  DEW_REQUIRE(aligned16(x_f16) && aligned16(hidden), "%s: x_f16 and hidden must be 16-byte aligned", who);
+  GemmParams p{};
+  p.x = static_cast<const bf16_t*>(x_f16);
+  p.a_scale = x_scale;
+  p.gather = gather;
+  p.offsets = offsets;
+  p.sizes = group_sizes;
+  p.w0 = BankView{static_cast<const uint8_t*>(gate->codes), gate->scales, gate->tensor_scale};
+  p.w1 = BankView{static_cast<const uint8_t*>(up->codes), up->scales, up->tensor_scale};
+  p.out = static_cast<bf16_t*>(hidden);
+  p.experts = gate->experts;
+  p.depth = gate->depth;
+  p.width = gate->width;
+  p.rows = rows;
+  p.gating = activation;
+  p.limit = limit > 0.0f ? bf16_round_host(limit) : 0.0f;
+  return launch_format<kFormatNvF16, kSwigluOfTwo>(who, p, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int dew_moe_gateup_gated(const void* x, const int32_t* gather, const int32_t* offsets, const int32_t* group_sizes,

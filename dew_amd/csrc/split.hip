@@ -181,6 +181,51 @@ __global__ __launch_bounds__(64 * kSplitWaves) void split_rows_fp6_kernel(const 
   }
 }
 
+// Activation rows as f16 for the f16 matrix instruction (general NVFP4 banks, whose code x e4m3-scale products are exact in
+// f16 and cost the vector unit half of what their bf16 form costs): x = 2^s f, one power of two per row chosen so that the
+// row's largest magnitude lands in [2^15, 2^16), under f16's largest finite value. A bf16 value has 8 significant bits and
+// f16 holds 11, so f is exact for every element within 2^-29 of its row's largest magnitude (f16's normal range) and loses
+// bits only below that, at most 2^-40 of the largest magnitude. The row's scale is stored as the e8m0 byte of 2^s. Same
+// two bytes an element and the same row pitch as the bf16 source.
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+
+__global__ __launch_bounds__(64 * kSplitWaves) void rows_f16_kernel(const bf16_t* __restrict__ x, uint16_t* __restrict__ halves,
+                                                                   uint8_t* __restrict__ scale, int rows, int depth) {
+  const int lane = threadIdx.x % 64;
+  const int row = blockIdx.x * kSplitWaves + threadIdx.x / 64;
+  if (row >= rows) return;
+  const bf16_t* source = x + static_cast<size_t>(row) * depth;
+  uint32_t largest = 0;
+  for (int chunk = lane; chunk < depth / 8; chunk += 64) {
+    const u32x4_t words = *reinterpret_cast<const u32x4_t*>(source + chunk * 8);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      largest = max(largest, (words[i] >> 7) & 0xFFu);
+      largest = max(largest, (words[i] >> 23) & 0xFFu);
+    }
+  }
+#pragma unroll
+  for (int offset = 32; offset >= 1; offset >>= 1) largest = max(largest, static_cast<uint32_t>(__shfl_xor(static_cast<int>(largest), offset, 64)));
+  // largest magnitude in [2^(field - 127), 2^(field - 126)): times 2^(142 - field) it lies in [2^15, 2^16). The byte
+  // (field - 15: the e8m0 of 2^s) and its inverse stay normal powers of two; NaN and infinity count as the largest finite.
+  const int field = min(max(static_cast<int>(largest), 16), 254);
+  const int byte = field - 15;
+  if (lane == 0) scale[row] = static_cast<uint8_t>(byte);
+  const float inverse = __uint_as_float(static_cast<uint32_t>(254 - byte) << 23);  // 2^-s
+  uint16_t* target = halves + static_cast<size_t>(row) * depth;
+  for (int chunk = lane; chunk < depth / 8; chunk += 64) {
+    const u32x4_t words = *reinterpret_cast<const u32x4_t*>(source + chunk * 8);
+    u32x4_t packed;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const f16x2_t pair = {static_cast<_Float16>(__uint_as_float(words[i] << 16) * inverse),
+                            static_cast<_Float16>(__uint_as_float(words[i] & 0xFFFF0000u) * inverse)};
+      packed[i] = __builtin_bit_cast(uint32_t, pair);
+    }
+    *reinterpret_cast<u32x4_t*>(target + chunk * 8) = packed;
+  }
+}
+
 }  // namespace dew
 
 extern "C" int dew_moe_split_rows_fp6(const void* x, void* split, uint8_t* scale, int32_t rows, int32_t depth, void* stream) {
@@ -211,4 +256,15 @@ extern "C" int dew_moe_split_rows(const void* x, void* split, uint8_t* scale, in
     default: launch(split_rows_kernel<0>); break;
   }
   return launched("split_rows_kernel");
+}
+
+extern "C" int dew_moe_rows_f16(const void* x, void* halves, uint8_t* scale, int32_t rows, int32_t depth, void* stream) {
+  using namespace dew;
+  DEW_REQUIRE(rows >= 0 && depth >= 64 && depth % 64 == 0, "dew_moe_rows_f16: rows %d, depth %d (whole 64s)", rows, depth);
+  if (rows == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(x && halves && scale, "dew_moe_rows_f16: x, halves and scale must not be null");
+  DEW_REQUIRE(aligned16(x) && aligned16(halves), "dew_moe_rows_f16: x and halves must be 16-byte aligned");
+  hipLaunchKernelGGL(rows_f16_kernel, dim3((rows + kSplitWaves - 1) / kSplitWaves), dim3(64 * kSplitWaves), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const bf16_t*>(x), static_cast<uint16_t*>(halves), scale, rows, depth);
+  return launched("rows_f16_kernel");
 }

@@ -445,6 +445,15 @@ def gateup_swiglu(x: torch.Tensor, gate: PreparedBank, up: PreparedBank, offsets
         raise KernelError(f"gate {gate.shape} and up {up.shape} differ")
     rows = _product_rows(x, "x", offsets, experts, gather, None, rows, sizes)
     hidden = torch.empty((rows, width), dtype=torch.bfloat16, device=x.device)
+    if prefers_f16_rows(gate, up, rows):
+        # general NVFP4 banks, groups tall enough to be bound by the matrix cores: the rows as f16 under a scale a row and
+        # the f16 matrix instruction, which halves the vector work of decoding the banks; the same bits
+        halves, scales = rows_f16(x)
+        _lib.check(_lib.library().dew_moe_gateup_gated_f16(_ptr(halves), _ptr(scales), _ptr(gather), _ptr(offsets),
+                                                           _ptr(None if offsets is not None else sizes), gate.descriptor, up.descriptor,
+                                                           GATES[activation], 0.0 if limit is None else float(limit), _ptr(hidden), rows,
+                                                           _stream()), "dew_moe_gateup_gated_f16")
+        return hidden
     if activation != "swiglu" or limit is not None:
         _lib.check(_lib.library().dew_moe_gateup_gated(_ptr(x), _ptr(gather), _ptr(offsets), _ptr(None if offsets is not None else sizes),
                                                        gate.descriptor, up.descriptor, GATES[activation], 0.0 if limit is None else float(limit),
@@ -457,6 +466,30 @@ def gateup_swiglu(x: torch.Tensor, gate: PreparedBank, up: PreparedBank, offsets
     _lib.check(_lib.library().dew_moe_gateup_swiglu(_ptr(x), _ptr(gather), _ptr(offsets), gate.descriptor, up.descriptor,
                                                     _ptr(hidden), rows, _stream()), "dew_moe_gateup_swiglu")
     return hidden
+
+
+F16_ROWS = True
+"""Whether a paired launch on general NVFP4 banks (block scales with mantissas) whose groups average F16_ROWS_FROM rows or
+more runs on f16 rows and the f16 matrix instruction (`prefers_f16_rows`). Bit-identical to the bf16-operand launch either
+way: every product is the same exact one times a power of two. False keeps the bf16 instruction."""
+F16_ROWS_FROM = 64
+
+
+def prefers_f16_rows(gate: PreparedBank, up: PreparedBank, rows: int) -> bool:
+    return (F16_ROWS and gate.descriptor.format == _lib.W_NVFP4 and up.descriptor.format == _lib.W_NVFP4
+            and rows >= F16_ROWS_FROM * gate.experts)
+
+
+def rows_f16(x: torch.Tensor):
+    """(`halves [rows, depth]` float16, `scale [rows]` e8m0 bytes): each bf16 row as f16 values times one power of two, chosen
+    so that the row's largest magnitude lies in [2^15, 2^16) (`dew_moe_rows_f16`)."""
+    _device(x, "x", torch.bfloat16)
+    if x.dim() != 2 or x.shape[1] % 64:
+        raise KernelError(f"x is {tuple(x.shape)}: rows of whole 64s")
+    halves = torch.empty(x.shape, dtype=torch.float16, device=x.device)
+    scale = torch.empty((x.shape[0],), dtype=torch.uint8, device=x.device)
+    _lib.check(_lib.library().dew_moe_rows_f16(_ptr(x), _ptr(halves), _ptr(scale), x.shape[0], x.shape[1], _stream()), "dew_moe_rows_f16")
+    return halves, scale
 
 
 GATES = {"swiglu": _lib.GATE_SILU, "geglu": _lib.GATE_GELU_TANH}

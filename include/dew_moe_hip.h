@@ -471,6 +471,19 @@ int dew_moe_gated_product(const void* gate, const void* up, int32_t activation, 
 int dew_moe_gateup_gated(const void* x, const int32_t* gather, const int32_t* offsets /* nullable */,
                          const int32_t* group_sizes /* nullable */, const dew_moe_bank* gate, const dew_moe_bank* up,
                          int32_t activation, float limit, void* hidden, int32_t rows, void* stream);
+/* The same paired launch for general NVFP4 banks (DEW_MOE_W_NVFP4: e4m3 block scales with mantissas, `NvFp4`,
+ * src/dew/nn/kernels/formats.py:27-137) on f16 operands: `nvfp4_product`'s decode (src/dew/nn/kernels/gemm.py:609-662,
+ * formats.py:108-113: code x block scale, exact in bf16) is as exact in f16, where it costs the vector unit one packed
+ * conversion and one packed multiply for two codes, half of the bf16 form. dew_moe_rows_f16 brings the rows to f16 under one
+ * power-of-two scale a row (halves [rows, depth] f16, scale [rows] e8m0 bytes: x = 2^(scale - 127) halves, the row's largest
+ * magnitude in [2^15, 2^16); exact for every element within 2^-29 of it); dew_moe_gateup_gated_f16 is dew_moe_gateup_gated on
+ * those rows (gather indexes them and their scales). Each product is the bf16 launch's times a power of two and the sums
+ * are fp32, so `hidden` is bit for bit dew_moe_gateup_gated's. No counterpart in the reference, whose decode is XLA's.   */
+int dew_moe_rows_f16(const void* x /* bf16 [rows, depth] */, void* halves /* f16 [rows, depth] */, uint8_t* scale /* [rows] */,
+                     int32_t rows, int32_t depth, void* stream);
+int dew_moe_gateup_gated_f16(const void* x_f16, const uint8_t* x_scale, const int32_t* gather, const int32_t* offsets /* nullable */,
+                             const int32_t* group_sizes /* nullable */, const dew_moe_bank* gate, const dew_moe_bank* up,
+                             int32_t activation, float limit, void* hidden, int32_t rows, void* stream);
 /* Llama 4's input-scaled experts (`scale_inputs`, src/dew/nn/moe.py:1124-1126, 1256-1259: `Llama4TextMoe.forward`): the
  * rows the experts multiply, out[i] = bf16(x[gather[i]] * bf16(weights[slots[i]])) for the sorted positions i < rows
  * (gather = the sort's rows, slots = its order, weights [T*k] the router's). The launches then read `out` without a
