@@ -31,6 +31,9 @@ PEAKS = {"bf16_mfma": 2500.0, "fp8_mfma": 5000.0, "fp4_mfma": 10100.0, "hbm_gbs"
 """MI355X published dense peaks, TFLOP/s and GB/s."""
 
 ALL_CONFIGS = ("c1", "c2", "c3", "c4", "c5")
+TERM_RATES = {"e4m3": ("e4m3", "e4m3"), "e2m3": ("e4m3", "e2m3"), "e2m3x2": ("e2m3", "e2m3")}
+"""The two terms a split row is held as, by the library's setting (an e4m3 term's instruction runs at the fp8 rate, an
+e2m3 term's at the fp6/fp4 rate)."""
 GRAPHED = ("c1", "c3")
 """The launch-bound workloads: their step is replayed as one captured HIP graph."""
 DECODE = ("c3",)
@@ -107,7 +110,7 @@ class Stepper:
         self.dense_offsets = torch.tensor([0, tokens], dtype=torch.int32, device=data["x"].device)
         self.events = []
         self.split = split
-        self.fp6 = gemm.SPLIT_SECOND_TERM == "e2m3"   # the library's setting for the split rows' second term
+        self.terms = gemm.SPLIT_SECOND_TERM           # the library's setting for how split rows are held ('e4m3': two e4m3 terms)
 
     def __call__(self, timed: bool = False):
         torch, ops, case, data = self.torch, self.ops, self.case, self.data
@@ -134,10 +137,10 @@ class Stepper:
         if self.on_split_rows():
             # MXFP4 banks and groups of hundreds of rows: the rows as two e4m3 terms and the scaled matrix instruction;
             # the gate/up launch writes its hidden rows already split, so the only extra pass is the split of x
-            pieces = ops.split_rows_fp6(data["x"]) if self.fp6 else ops.split_rows(data["x"])
+            pieces = ops.split_rows_as(data["x"], self.terms)
             if events:
                 events[0].record()
-            hidden = ops.gateup_swiglu_split_out(*pieces, self.gate, self.up, plan.offsets, gather=plan.rows, fp6=self.fp6)
+            hidden = ops.gateup_swiglu_split_out(*pieces, self.gate, self.up, plan.offsets, gather=plan.rows, terms=self.terms)
             if events:
                 events[1].record()
                 self.events.append(events)
@@ -417,9 +420,10 @@ def measure(config, args, device, sustained, with_cpu_baseline):
     if not decode and stepper.on_split_rows():
         roofline["executed"] = {"tflops": round(2 * achieved, 1), "frac_of_fp8_peak": round(2 * achieved / PEAKS["fp8_mfma"], 4),
                                 "note": "instruction flops: both terms' products",
-                                "issue_time_frac": round(achieved / (1.0 / (1.0 / PEAKS["fp8_mfma"] + 1.0 / (PEAKS["fp4_mfma"] if stepper.fp6 else PEAKS["fp8_mfma"]))), 4),
+                                "issue_time_frac": round(achieved / (1.0 / sum(1.0 / PEAKS["fp8_mfma" if term == "e4m3" else "fp4_mfma"]
+                                                                               for term in TERM_RATES[stepper.terms])), 4),
                                 "issue_time_note": "achieved over the rate at which the two instructions of a product issue back to back at "
-                                                   "their published peaks (fp8 + fp8: 2.5 PFLOP/s; fp8 + fp6: 3.34 PFLOP/s)"}
+                                                   "their published peaks (fp8 + fp8: 2.5 PFLOP/s; fp8 + fp6: 3.34; fp6 + fp6: 5.05)"}
     roofline["traffic"] = measured_traffic(config)
     roofline["traffic_source"] = (f"parsed from {COUNTED_FROM[config]}: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE of this command's "
                                   f"gate/up launch(es), scaled by {CALIBRATION}; counters of an earlier run of the same command, "
@@ -432,7 +436,7 @@ def measure(config, args, device, sustained, with_cpu_baseline):
                                      "its power limit, a plain copy, and a read-only stream of non-temporal loads issued as the "
                                      "decode tiles issue theirs (the reference for an HBM-bound launch)"}
     roofline["kernel"] = "grouped_gemm_kernel<paired gate/up + SwiGLU>" + (
-        f" on split rows (v_mfma_scale_f32_32x32x64_f8f6f4, an e4m3 and an {'e2m3' if stepper.fp6 else 'e4m3'} term x FP4)" if stepper.on_split_rows() else "")
+        f" on split rows (v_mfma_scale_f32_32x32x64_f8f6f4, {' + '.join(TERM_RATES[stepper.terms])} terms x FP4)" if stepper.on_split_rows() else "")
     roofline["kernel_ms"] = round(gateup_ms, 4)
 
     result = {
@@ -522,8 +526,9 @@ def main():
     parser.add_argument("--bf16-operands", action="store_true",
                         help="keep MXFP4 banks with groups of hundreds of rows on the bf16 matrix instruction too (the default "
                              "there: rows split into two e4m3 terms and the scaled instruction, the library's own choice)")
-    parser.add_argument("--second-term", choices=["e4m3", "e2m3"], default=None,
-                        help="the split rows' second term in the first product (default: the library's, gemm.SPLIT_SECOND_TERM)")
+    parser.add_argument("--second-term", choices=["e4m3", "e2m3", "e2m3x2"], default=None,
+                        help="how the split rows of the first product are held: two e4m3 terms, an e4m3 and an e2m3 term, or two "
+                             "e2m3 terms (default: the library's, gemm.SPLIT_SECOND_TERM)")
     parser.add_argument("--separate-shared", action="store_true",
                         help="compute a shared expert as a dense MLP of its own (two more launches), as the reference does, instead "
                              "of as group #E of the routed launches")
@@ -567,15 +572,17 @@ def main():
                 print(f"[bench] measuring {config}", file=sys.stderr, flush=True)
                 measured = measure(config, args, device, sustained, with_cpu_baseline=False)
             per_config[config] = measured
-        # the same c2 workload with the split rows' second term in FP6 (gemm.SPLIT_SECOND_TERM = 'e2m3'): the faster, less
-        # exact option, measured in the same run beside the default so that its price in parity stands next to its gain
-        if gemm.SPLIT_SECOND_TERM != "e2m3":
-            print("[bench] measuring c2 with an e2m3 second term", file=sys.stderr, flush=True)
-            held, gemm.SPLIT_SECOND_TERM = gemm.SPLIT_SECOND_TERM, "e2m3"
-            try:
-                per_config["c2_option_e2m3_second_term"] = measure("c2", args, device, sustained, with_cpu_baseline=False)
-            finally:
-                gemm.SPLIT_SECOND_TERM = held
+        # the same c2 workload with the split rows' terms in FP6 (gemm.SPLIT_SECOND_TERM = 'e2m3': the second; 'e2m3x2': both):
+        # the faster, less exact options, measured in the same run beside the default so that their price in parity stands
+        # next to their gain
+        for option, label in (("e2m3", "c2_option_e2m3_second_term"), ("e2m3x2", "c2_option_two_e2m3_terms")):
+            if gemm.SPLIT_SECOND_TERM != option:
+                print(f"[bench] measuring c2 with {label}", file=sys.stderr, flush=True)
+                held, gemm.SPLIT_SECOND_TERM = gemm.SPLIT_SECOND_TERM, option
+                try:
+                    per_config[label] = measure("c2", args, device, sustained, with_cpu_baseline=False)
+                finally:
+                    gemm.SPLIT_SECOND_TERM = held
         result["configs"] = per_config
     print(json.dumps(result))
 

@@ -69,6 +69,9 @@ constexpr int kFormatBf16Window = 21;
 // takes half the cycles of the FP8 x FP4 one, so a product's two instructions take three quarters of the time; the
 // second term is exact only for elements within two binades of their 32-deep block's largest (see split.hip).
 constexpr int kFormatMxSplit6 = 22;
+// kFormatMxSplit with both terms in FP6 (dew_moe_split_rows_e2m3_pair: each term's power-of-two scale every 32 depths lies
+// with its codes, no scale a row): two FP6 x FP4 instructions a product, the time of one FP8 x FP4 instruction.
+constexpr int kFormatMxSplit66 = 24;
 // Kernel-side format of a general NVFP4 bank (e4m3 block scales with mantissas) multiplied by activation rows brought to
 // f16 under one power-of-two scale a row (dew_moe_rows_f16), on v_mfma_f32_32x32x16_f16. A code times its block scale has
 // at most six significant bits and lies in 2^-10 .. 2688: exact in f16, formed by one packed conversion and one packed f16
@@ -234,7 +237,8 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   constexpr bool kWindow = FORMAT == kFormatMxFp8Window || FORMAT == kFormatBf16Window;  // a kernel gradient: the same rows for every group, its own depths
   constexpr bool kMxRows = FORMAT == kFormatMxFp8Rows || FORMAT == kFormatMxFp8Window;  // e4m3 rows and weights, one scale per row (column) and 32 depths
   constexpr bool kFp8A = kFp8Rows || kMxRows;           // both operands e4m3 codes: a step is 128 depths
-  constexpr bool kLo6 = FORMAT == kFormatMxSplit6;      // the second term of a row in FP6 (e2m3), its scale beside it
+  constexpr bool kHi6 = FORMAT == kFormatMxSplit66;     // both terms of a row in FP6 (e2m3), each with its scale beside it
+  constexpr bool kLo6 = FORMAT == kFormatMxSplit6 || kHi6;  // the second term of a row in FP6 (e2m3), its scale beside it
   constexpr bool kSplit = FORMAT == kFormatMxSplit || FORMAT == kFormatMxSplitBlocks || kLo6 || kFp8A;  // A arrives as 8-bit codes
   constexpr bool kBlockScales = FORMAT == kFormatMxSplitBlocks || kFp8Rows;
   constexpr bool kFp4 = FORMAT == DEW_MOE_W_NVFP4 || FORMAT == DEW_MOE_W_MXFP4 || kNvF16 || (kSplit && !kFp8A);
@@ -413,7 +417,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
     if constexpr (kSplit) {
       const int sorted = row0 + min(wm0 + 32 * i + lane % 32, valid_rows - 1);
       const int source = p.gather ? p.gather[sorted] : sorted;
-      if constexpr (!kBlockScales) {
+      if constexpr (!kBlockScales && !kHi6) {  // (two FP6 terms carry their scales with their codes)
         const int byte = p.a_scale[source];
         a_scale_word[i] = byte | ((byte - 4) << 8);
       }
@@ -554,7 +558,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   // ---- fragments: slice kk of a step is 16 depths; a lane's are the 8 its weight bytes cover ----
   bf16x8_t a_frag[2][TI], b_frag[2][kTiles];
   i32x8_t a_term[2][kSplit ? TI : 1];  // split activations: [0] the hi term of a step, [1] its lo term
-  int a_lo_scale[kLo6 ? TI : 1];       // an FP6 second term's e8m0 scale of the lane's 32 depths (it lies behind the codes)
+  int a_fp6_scale[2][kLo6 ? TI : 1];   // an FP6 term's e8m0 scale of the lane's 32 depths (it lies behind the codes)
   float fp4_scale[kTiles];
   _Float16 fp4_half[kNvF16 ? kTiles : 1];  // f16 rows: the block scale as f16
   // a term of a 32-depth block is 32 bytes: the lane's block lane / 32 of the step holds hi in its chunks 0-1, lo in 2-3
@@ -573,10 +577,10 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
       for (int i = 0; i < TI; ++i) {
         const u32x4_t first = first_piece[32 * i * kChunksPerRow];  // the swizzle reads a row's low four bits only
         const u32x4_t second = second_piece[32 * i * kChunksPerRow];
-        if constexpr (kLo6 && term.value == 1) {  // 24 bytes of e2m3 codes, then the scale's dword
-          a_term[1][i] = i32x8_t{static_cast<int>(first[0]), static_cast<int>(first[1]), static_cast<int>(first[2]),
-                                 static_cast<int>(first[3]), static_cast<int>(second[0]), static_cast<int>(second[1]), 0, 0};
-          a_lo_scale[i] = static_cast<int>(second[2]);
+        if constexpr ((kLo6 && term.value == 1) || kHi6) {  // 24 bytes of e2m3 codes, then the scale's dword
+          a_term[term.value][i] = i32x8_t{static_cast<int>(first[0]), static_cast<int>(first[1]), static_cast<int>(first[2]),
+                                          static_cast<int>(first[3]), static_cast<int>(second[0]), static_cast<int>(second[1]), 0, 0};
+          a_fp6_scale[term.value][i] = static_cast<int>(second[2]);
         } else {
           a_term[term.value][i] = i32x8_t{static_cast<int>(first[0]), static_cast<int>(first[1]), static_cast<int>(first[2]),
                                           static_cast<int>(first[3]), static_cast<int>(second[0]), static_cast<int>(second[1]),
@@ -682,8 +686,9 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
             const int b_scale = static_cast<int>(((s_regs[set.value][m * TJ + j] >> 3) & 15u) + 120u);
 #pragma unroll
             for (int i = 0; i < TI; ++i) {
-              if constexpr (kLo6 && term.value == 1) {  // FP6 (e2m3) x FP4 under the term's own scale
-                acc[m][i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_term[1][i], codes, acc[m][i][j], 2, 4, 0, a_lo_scale[i], 0, b_scale);
+              if constexpr ((kLo6 && term.value == 1) || kHi6) {  // FP6 (e2m3) x FP4 under the term's own scale
+                acc[m][i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_term[term.value][i], codes, acc[m][i][j], 2, 4, 0,
+                                                                            a_fp6_scale[term.value][i], 0, b_scale);
               } else {
                 acc[m][i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_term[term.value][i], codes, acc[m][i][j], 0, 4, term.value,
                                                                             kBlockScales ? a_block_word[kBuffer][i] : a_scale_word[i], 0,
@@ -1471,8 +1476,8 @@ extern "C" int dew_moe_kernel_gradient_bf16(const void* lhs_t, const dew_moe_ban
 
 namespace dew {
 
-// The paired launch on split rows whose gated rows leave split as well; `second_e2m3`: the rows' second term is FP6.
-static int gateup_split_out_of(const char* who, bool second_e2m3, const void* x_split, const uint8_t* x_scale, const int32_t* gather,
+// The paired launch on split rows whose gated rows leave split as well; `terms`: the rows' terms (DEW_MOE_SECOND_TERM_*).
+static int gateup_split_out_of(const char* who, int terms, const void* x_split, const uint8_t* x_scale, const int32_t* gather,
                                const int32_t* offsets, const dew_moe_bank* gate, const dew_moe_bank* up, void* hidden_split,
                                uint8_t* hidden_scales, int32_t rows, void* stream, int32_t activation, float limit) {
   if (int rc = check_bank(who, gate, "gate")) return rc;
@@ -1490,7 +1495,7 @@ static int gateup_split_out_of(const char* who, bool second_e2m3, const void* x_
   DEW_REQUIRE(limit >= 0.0f, "%s: the clamp limit %g must be positive (0: none)", who, static_cast<double>(limit));
   DEW_REQUIRE(rows >= 0, "%s: rows %d", who, rows);
   if (rows == 0) return DEW_MOE_OK;
-  DEW_REQUIRE(x_split && x_scale && offsets && hidden_split && hidden_scales,
+  DEW_REQUIRE(x_split && (x_scale || terms == DEW_MOE_TERMS_E2M3_PAIR) && offsets && hidden_split && hidden_scales,
               "%s: x_split, x_scale, offsets, hidden_split and hidden_scales must not be null", who);
   DEW_REQUIRE(aligned16(x_split) && aligned16(hidden_split), "%s: x_split and hidden_split must be 16-byte aligned", who);
   GemmParams p{};
@@ -1513,7 +1518,11 @@ static int gateup_split_out_of(const char* who, bool second_e2m3, const void* x_
   // against 5.30 ms for 256-row tiles at one block a CU, the same bits. (The plain product stays on 256-row
   // tiles: 2.55 against 2.61 ms.)
   const hipStream_t s = static_cast<hipStream_t>(stream);
-  if (second_e2m3) {
+  if (terms == DEW_MOE_TERMS_E2M3_PAIR) {
+    if (forced_tile_rows == 256) return launch_tile<kFormatMxSplit66, kSwigluOfTwoSplit, 256, 128, 2, 2>(who, p, s);
+    return launch_tile<kFormatMxSplit66, kSwigluOfTwoSplit, 128, 128, 2, 2>(who, p, s);
+  }
+  if (terms == DEW_MOE_SECOND_TERM_E2M3) {
     if (forced_tile_rows == 256) return launch_tile<kFormatMxSplit6, kSwigluOfTwoSplit, 256, 128, 2, 2>(who, p, s);
     return launch_tile<kFormatMxSplit6, kSwigluOfTwoSplit, 128, 128, 2, 2>(who, p, s);
   }
@@ -1526,15 +1535,22 @@ static int gateup_split_out_of(const char* who, bool second_e2m3, const void* x_
 extern "C" int dew_moe_gateup_swiglu_split_out(const void* x_split, const uint8_t* x_scale, const int32_t* gather,
                                                const int32_t* offsets, const dew_moe_bank* gate, const dew_moe_bank* up,
                                                void* hidden_split, uint8_t* hidden_scales, int32_t rows, void* stream) {
-  return dew::gateup_split_out_of("dew_moe_gateup_swiglu_split_out", false, x_split, x_scale, gather, offsets, gate, up, hidden_split,
+  return dew::gateup_split_out_of("dew_moe_gateup_swiglu_split_out", DEW_MOE_SECOND_TERM_E4M3, x_split, x_scale, gather, offsets, gate, up, hidden_split,
                                   hidden_scales, rows, stream, DEW_MOE_GATE_SILU, 0.0f);
 }
 
 extern "C" int dew_moe_gateup_swiglu_split_fp6_out(const void* x_split, const uint8_t* x_scale, const int32_t* gather,
                                                    const int32_t* offsets, const dew_moe_bank* gate, const dew_moe_bank* up,
                                                    void* hidden_split, uint8_t* hidden_scales, int32_t rows, void* stream) {
-  return dew::gateup_split_out_of("dew_moe_gateup_swiglu_split_fp6_out", true, x_split, x_scale, gather, offsets, gate, up, hidden_split,
-                                  hidden_scales, rows, stream, DEW_MOE_GATE_SILU, 0.0f);
+  return dew::gateup_split_out_of("dew_moe_gateup_swiglu_split_fp6_out", DEW_MOE_SECOND_TERM_E2M3, x_split, x_scale, gather, offsets, gate, up,
+                                  hidden_split, hidden_scales, rows, stream, DEW_MOE_GATE_SILU, 0.0f);
+}
+
+extern "C" int dew_moe_gateup_swiglu_split_e2m3_pair_out(const void* x_split, const int32_t* gather, const int32_t* offsets,
+                                                         const dew_moe_bank* gate, const dew_moe_bank* up, void* hidden_split,
+                                                         uint8_t* hidden_scales, int32_t rows, void* stream) {
+  return dew::gateup_split_out_of("dew_moe_gateup_swiglu_split_e2m3_pair_out", DEW_MOE_TERMS_E2M3_PAIR, x_split, nullptr, gather, offsets, gate,
+                                  up, hidden_split, hidden_scales, rows, stream, DEW_MOE_GATE_SILU, 0.0f);
 }
 
 // ---- the SwiGLU expert MLP on split rows as one call -----------------------------------------------------------------
@@ -1597,8 +1613,8 @@ extern "C" int dew_moe_gated_mlp_split(const void* x, int32_t tokens, const int3
   if (int rc = check_bank(who, up, "up")) return rc;
   if (int rc = check_bank(who, down, "down")) return rc;
   DEW_REQUIRE(tokens >= 0 && rows >= 0, "%s: tokens %d rows %d", who, tokens, rows);
-  DEW_REQUIRE(second_term == DEW_MOE_SECOND_TERM_E4M3 || second_term == DEW_MOE_SECOND_TERM_E2M3,
-              "%s: the rows' second term %d is neither e4m3 (0) nor e2m3 (1)", who, second_term);
+  DEW_REQUIRE(second_term == DEW_MOE_SECOND_TERM_E4M3 || second_term == DEW_MOE_SECOND_TERM_E2M3 || second_term == DEW_MOE_TERMS_E2M3_PAIR,
+              "%s: the rows' terms %d are neither two e4m3 (0), e4m3 and e2m3 (1) nor two e2m3 (2)", who, second_term);
   DEW_REQUIRE(down->experts == gate->experts && down->depth == gate->width, "%s: down [%d, %d, %d] does not follow gate [%d, %d, %d]", who,
               down->experts, down->depth, down->width, gate->experts, gate->depth, gate->width);
   if (rows == 0 || tokens == 0) return DEW_MOE_OK;
@@ -1617,15 +1633,15 @@ extern "C" int dew_moe_gated_mlp_split(const void* x, int32_t tokens, const int3
   uint8_t* x_scale = base + w.x_scale;
   void* hidden_split = base + w.hidden_split;
   uint8_t* hidden_scales = base + w.hidden_scales;
-  if (second_term == DEW_MOE_SECOND_TERM_E2M3) {
+  if (second_term == DEW_MOE_TERMS_E2M3_PAIR) {
+    if (int rc = dew_moe_split_rows_e2m3_pair(x, x_split, tokens, gate->depth, stream)) return rc;
+  } else if (second_term == DEW_MOE_SECOND_TERM_E2M3) {
     if (int rc = dew_moe_split_rows_fp6(x, x_split, x_scale, tokens, gate->depth, stream)) return rc;
-    if (int rc = gateup_split_out_of(who, true, x_split, x_scale, gather, offsets, gate, up, hidden_split, hidden_scales, rows, stream,
-                                     activation, limit)) return rc;
   } else {
     if (int rc = dew_moe_split_rows(x, x_split, x_scale, tokens, gate->depth, stream)) return rc;
-    if (int rc = gateup_split_out_of(who, false, x_split, x_scale, gather, offsets, gate, up, hidden_split, hidden_scales, rows, stream,
-                                     activation, limit)) return rc;
   }
+  if (int rc = gateup_split_out_of(who, second_term, x_split, x_scale, gather, offsets, gate, up, hidden_split, hidden_scales, rows, stream,
+                                   activation, limit)) return rc;
   return dew_moe_grouped_gemm_split_blocks(hidden_split, hidden_scales, nullptr, offsets, down, nullptr, scatter, out, rows, stream);
 }
 

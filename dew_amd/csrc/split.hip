@@ -181,6 +181,68 @@ __global__ __launch_bounds__(64 * kSplitWaves) void split_rows_fp6_kernel(const 
   }
 }
 
+// Both terms in FP6: x = s hi + t lo with hi = e2m3(x / s) and lo = e2m3((x - s hi) / t), s and t each one power of two for
+// every 32 depths: the least that brings the block's largest magnitude (s), then its largest remainder (t), within
+// e2m3's range (7.5). Two FP6 x FP4 instructions take the time of one FP8 x FP4 instruction, half of what the two e4m3
+// terms take. e2m3 holds four significant bits in its upper three binades and steps of an eighth of its scale below, so
+// an element within two binades of its block's largest is held exactly (four bits in each term) and any other to within
+// 2^-10 of that largest magnitude. There is no scale a row: both terms' scales lie with their codes. A row's 64 depths are
+// 128 bytes, [group 0: 24 bytes of hi codes, hi's e8m0 byte in a dword, 4 unused, 24 bytes of lo codes, lo's, 4 unused]
+// [group 1 alike], lane group g holding depths 32 g .. 32 g + 31 (the 6-bit operand's own order).
+typedef __attribute__((ext_vector_type(32))) float f32x32_t;
+
+__device__ __forceinline__ float e2m3_block_scale(float most) {
+  // the least power of two t with most / t <= 7.5 = 1.875 * 4: most's exponent less 2, one more where its significand is
+  // above 1.875; kept a normal power of two whose e8m0 byte is 1 .. 254 (a block of zeros lands on the least)
+  const uint32_t bits = __float_as_uint(most);
+  int power = static_cast<int>(bits >> 23) - 127 - 2 + ((bits & 0x7FFFFFu) > 0x700000u ? 1 : 0);
+  power = min(max(power, -126), 127);
+  return __uint_as_float(static_cast<uint32_t>(power + 127) << 23);
+}
+
+__global__ __launch_bounds__(64 * kSplitWaves) void split_rows_e2m3_pair_kernel(const bf16_t* __restrict__ x, uint8_t* __restrict__ split,
+                                                                               int rows, int depth) {
+  const int lane = threadIdx.x % 64;
+  const int row = blockIdx.x * kSplitWaves + threadIdx.x / 64;
+  if (row >= rows) return;
+  const bf16_t* source = x + static_cast<size_t>(row) * depth;
+  uint8_t* target = split + static_cast<size_t>(row) * depth * 2;
+  for (int block = lane; block < depth / 32; block += 64) {
+    float rest[32];
+#pragma unroll
+    for (int piece = 0; piece < 4; ++piece) {  // 8 depths a piece
+      const u32x4_t words = *reinterpret_cast<const u32x4_t*>(source + block * 32 + piece * 8);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        rest[8 * piece + 2 * i] = __uint_as_float(words[i] << 16);
+        rest[8 * piece + 2 * i + 1] = __uint_as_float(words[i] & 0xFFFF0000u);
+      }
+    }
+    uint8_t* at = target + (block / 2) * 128 + (block % 2) * 64;  // the step's 128 bytes, the lane group's 64 of them
+#pragma unroll
+    for (int term = 0; term < 2; ++term) {
+      float most = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 32; ++i) most = fmaxf(most, fabsf(rest[i]));
+      const float scale = e2m3_block_scale(most);
+      f32x16_t even, odd;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        even[i] = rest[2 * i];
+        odd[i] = rest[2 * i + 1];
+      }
+      const u32x6_t codes = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(even, odd, scale);
+      if (term == 0) {  // what the first term holds, as the matrix instruction will read it, leaves the remainder
+        const f32x32_t held = __builtin_amdgcn_cvt_scalef32_pk32_f32_fp6(codes, scale);
+#pragma unroll
+        for (int i = 0; i < 32; ++i) rest[i] -= held[i];
+      }
+      *reinterpret_cast<u32x4_t*>(at + 32 * term) = u32x4_t{codes[0], codes[1], codes[2], codes[3]};
+      *reinterpret_cast<u32x4_t*>(at + 32 * term + 16) = u32x4_t{codes[4], codes[5], __float_as_uint(scale) >> 23, 0u};
+    }
+  }
+}
+
 // Activation rows as f16 for the f16 matrix instruction (general NVFP4 banks, whose code x e4m3-scale products are exact in
 // f16 and cost the vector unit half of what their bf16 form costs): x = 2^s f, one power of two per row chosen so that the
 // row's largest magnitude lands in [2^15, 2^16), under f16's largest finite value. A bf16 value has 8 significant bits and
@@ -267,4 +329,15 @@ extern "C" int dew_moe_rows_f16(const void* x, void* halves, uint8_t* scale, int
   hipLaunchKernelGGL(rows_f16_kernel, dim3((rows + kSplitWaves - 1) / kSplitWaves), dim3(64 * kSplitWaves), 0,
                      static_cast<hipStream_t>(stream), static_cast<const bf16_t*>(x), static_cast<uint16_t*>(halves), scale, rows, depth);
   return launched("rows_f16_kernel");
+}
+
+extern "C" int dew_moe_split_rows_e2m3_pair(const void* x, void* split, int32_t rows, int32_t depth, void* stream) {
+  using namespace dew;
+  DEW_REQUIRE(rows >= 0 && depth >= 64 && depth % 64 == 0, "dew_moe_split_rows_e2m3_pair: rows %d, depth %d (whole 64s)", rows, depth);
+  if (rows == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(x && split, "dew_moe_split_rows_e2m3_pair: x and split must not be null");
+  DEW_REQUIRE(aligned16(x) && aligned16(split), "dew_moe_split_rows_e2m3_pair: x and split must be 16-byte aligned");
+  hipLaunchKernelGGL(split_rows_e2m3_pair_kernel, dim3((rows + kSplitWaves - 1) / kSplitWaves), dim3(64 * kSplitWaves), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const bf16_t*>(x), static_cast<uint8_t*>(split), rows, depth);
+  return launched("split_rows_e2m3_pair_kernel");
 }

@@ -244,4 +244,4 @@ def swiglu_mlp_on_split_rows(lhs: torch.Tensor, gate, up, down, group_sizes, *, 
         return None
     groups = GroupSizes.operands(group_sizes)   # a caller's plain group sizes go in as they are: the call forms their prefix
     return ops.swiglu_mlp_split(lhs, first, second, third, groups["offsets"], sizes=groups.get("sizes"), gather=gather,
-                                scatter=scatter, fp6=SPLIT_SECOND_TERM == "e2m3", activation=activation, limit=limit)
+                                scatter=scatter, terms=SPLIT_SECOND_TERM, activation=activation, limit=limit)

@@ -600,6 +600,29 @@ def split_rows_fp6(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     return split, scale
 
 
+def split_rows_e2m3_pair(x: torch.Tensor) -> tuple[torch.Tensor, None]:
+    """`split_rows` with both terms in FP6 (e2m3), each under one power-of-two scale every 32 depths that lies with its
+    codes: (`split` uint8 `[rows, depth * 2]`, None: there is no scale a row), for `gateup_swiglu_split_out(..., terms=
+    'e2m3x2')`. The two instructions of a product take the time of one FP8-rate instruction; the rows are held as exactly
+    as `split_rows_fp6` holds them (exactly within two binades of a 32-deep block's largest magnitude, to 2^-10 of it below)."""
+    _device(x, "x", torch.bfloat16)
+    rows, depth = x.shape
+    split = torch.empty((rows, depth * 2), dtype=torch.uint8, device=x.device)
+    _lib.check(_lib.library().dew_moe_split_rows_e2m3_pair(_ptr(x), _ptr(split), rows, depth, _stream()), "dew_moe_split_rows_e2m3_pair")
+    return split, None
+
+
+SPLIT_TERMS = {"e4m3": _lib.SECOND_TERM_E4M3, "e2m3": _lib.SECOND_TERM_E2M3, "e2m3x2": _lib.TERMS_E2M3_PAIR}
+"""How split rows are held: two e4m3 terms (exact; the default), an e4m3 and an e2m3 term, or two e2m3 terms."""
+
+
+def split_rows_as(x: torch.Tensor, terms: str = "e4m3"):
+    """`x` split as `terms` names (SPLIT_TERMS): the (split, scale) pair `gateup_swiglu_split_out(..., terms=terms)` reads."""
+    if terms not in SPLIT_TERMS:
+        raise KernelError(f"split rows are held as one of {list(SPLIT_TERMS)}, got {terms!r}")
+    return {"e4m3": split_rows, "e2m3": split_rows_fp6, "e2m3x2": split_rows_e2m3_pair}[terms](x)
+
+
 @contextlib.contextmanager
 def tile_rows(rows: int):
     """Within the block every grouped product uses block tiles of `rows` rows (32, 64, 128, 256) instead of the
@@ -638,10 +661,14 @@ def prefers_split_pair(gate: PreparedBank, up: PreparedBank, down: PreparedBank,
 
 def swiglu_mlp_split(x: torch.Tensor, gate: PreparedBank, up: PreparedBank, down: PreparedBank, offsets: torch.Tensor | None, *,
                      sizes: torch.Tensor | None = None, gather: torch.Tensor | None = None, scatter: torch.Tensor | None = None,
-                     rows: int | None = None, fp6: bool = False, activation: str = "swiglu", limit: float | None = None) -> torch.Tensor:
+                     rows: int | None = None, fp6: bool = False, activation: str = "swiglu", limit: float | None = None,
+                     terms: str | None = None) -> torch.Tensor:
     """The gated expert MLP on split rows as one call (`dew_moe_gated_mlp_split`): `split_rows`, `gateup_swiglu_split_out`
     and `grouped_gemm_split_blocks` with their intermediates in one workspace. The groups as `offsets` or as `sizes`;
-    `activation` and `limit` as `gateup_swiglu` takes them."""
+    `activation` and `limit` as `gateup_swiglu` takes them; `terms` (SPLIT_TERMS; `fp6=True` is 'e2m3') how x is split."""
+    terms = ("e2m3" if fp6 else "e4m3") if terms is None else terms
+    if terms not in SPLIT_TERMS:
+        raise KernelError(f"split rows are held as one of {list(SPLIT_TERMS)}, got {terms!r}")
     if activation not in GATES:
         raise KernelError(f"the gate's activation is one of {list(GATES)}, got {activation!r}")
     if limit is not None and not limit > 0:
@@ -658,7 +685,7 @@ def swiglu_mlp_split(x: torch.Tensor, gate: PreparedBank, up: PreparedBank, down
     _lib.check(lib.dew_moe_gated_mlp_split(_ptr(x), tokens, _ptr(gather), _ptr(offsets), _ptr(None if offsets is not None else sizes),
                                            gate.descriptor, up.descriptor, down.descriptor, GATES[activation],
                                            0.0 if limit is None else float(limit), _ptr(scatter), _ptr(out), rows,
-                                           _lib.SECOND_TERM_E2M3 if fp6 else _lib.SECOND_TERM_E4M3, _ptr(workspace), workspace.numel(),
+                                           SPLIT_TERMS[terms], _ptr(workspace), workspace.numel(),
                                            _stream()), "dew_moe_gated_mlp_split")
     return out
 
@@ -704,23 +731,34 @@ def block_scale_pitch(elements: int) -> int:
 
 def gateup_swiglu_split_out(split: torch.Tensor, scale: torch.Tensor, gate: PreparedBank, up: PreparedBank,
                             offsets: torch.Tensor, *, gather: torch.Tensor | None = None,
-                            rows: int | None = None, fp6: bool = False) -> tuple[torch.Tensor, torch.Tensor]:
+                            rows: int | None = None, fp6: bool = False, terms: str | None = None) -> tuple[torch.Tensor, torch.Tensor]:
     """`gateup_swiglu_split` whose hidden rows leave already split: (`hidden_split` uint8 `[rows, F * 2]`,
     `hidden_scales` uint8 `[rows, block_scale_pitch(F)]`), one scale per row and 128 columns (byte b of a row scales its
-    columns 128 b .. 128 b + 127; the pad bytes are not written), for `grouped_gemm_split_blocks`. `fp6`: the rows
-    come from `split_rows_fp6`."""
+    columns 128 b .. 128 b + 127; the pad bytes are not written), for `grouped_gemm_split_blocks`. `terms` (SPLIT_TERMS;
+    `fp6=True` is 'e2m3'): how the rows were split (`split_rows_as`); two e2m3 terms come without a scale a row."""
+    terms = ("e2m3" if fp6 else "e4m3") if terms is None else terms
+    if terms not in SPLIT_TERMS:
+        raise KernelError(f"split rows are held as one of {list(SPLIT_TERMS)}, got {terms!r}")
     experts, depth, width = gate.shape
-    if split.dtype != torch.uint8 or split.shape[-1] != 2 * depth or scale.dtype != torch.uint8 or scale.numel() != split.shape[0]:
-        raise KernelError(f"split rows are uint8 [rows, {2 * depth}] with one uint8 scale a row")
-    _device(scale, "scale", torch.uint8)
+    if split.dtype != torch.uint8 or split.shape[-1] != 2 * depth:
+        raise KernelError(f"split rows are uint8 [rows, {2 * depth}]")
+    if terms != "e2m3x2":
+        if scale is None or scale.dtype != torch.uint8 or scale.numel() != split.shape[0]:
+            raise KernelError("split rows of an e4m3 first term come with one uint8 scale a row")
+        _device(scale, "scale", torch.uint8)
     if up.shape != gate.shape:
         raise KernelError(f"gate {gate.shape} and up {up.shape} differ")
     rows = _product_rows(split, "split", offsets, experts, gather, None, rows)
     hidden = torch.empty((rows, width * 2), dtype=torch.uint8, device=split.device)
     scales = torch.empty((rows, block_scale_pitch(width)), dtype=torch.uint8, device=split.device)
-    call = _lib.library().dew_moe_gateup_swiglu_split_fp6_out if fp6 else _lib.library().dew_moe_gateup_swiglu_split_out
-    _lib.check(call(_ptr(split), _ptr(scale), _ptr(gather), _ptr(offsets), gate.descriptor, up.descriptor, _ptr(hidden), _ptr(scales),
-                    rows, _stream()), "dew_moe_gateup_swiglu_split_fp6_out" if fp6 else "dew_moe_gateup_swiglu_split_out")
+    if terms == "e2m3x2":
+        _lib.check(_lib.library().dew_moe_gateup_swiglu_split_e2m3_pair_out(_ptr(split), _ptr(gather), _ptr(offsets), gate.descriptor, up.descriptor,
+                                                                            _ptr(hidden), _ptr(scales), rows, _stream()),
+                   "dew_moe_gateup_swiglu_split_e2m3_pair_out")
+        return hidden, scales
+    name = "dew_moe_gateup_swiglu_split_fp6_out" if terms == "e2m3" else "dew_moe_gateup_swiglu_split_out"
+    _lib.check(getattr(_lib.library(), name)(_ptr(split), _ptr(scale), _ptr(gather), _ptr(offsets), gate.descriptor, up.descriptor, _ptr(hidden),
+                                             _ptr(scales), rows, _stream()), name)
     return hidden, scales
 
 

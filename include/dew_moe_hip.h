@@ -319,7 +319,7 @@ int dew_moe_grouped_gemm_split_blocks(const void* x_split, const uint8_t* x_scal
  * this form (1) or the bf16-operand launches (0): three prepared MXFP4 banks of whole 256-column strips that chain, the
  * down bank's depth within the LDS's room for a tile's scales, and groups averaging DEW_MOE_SPLIT_ROWS_FROM rows or more
  * (measured: 1.20 times the bf16 launches at 900 rows a group, 1.05 at 512 to 768, 1.08 at 384, 0.975 at 256).       */
-enum { DEW_MOE_SECOND_TERM_E4M3 = 0, DEW_MOE_SECOND_TERM_E2M3 = 1 };
+enum { DEW_MOE_SECOND_TERM_E4M3 = 0, DEW_MOE_SECOND_TERM_E2M3 = 1, DEW_MOE_TERMS_E2M3_PAIR = 2 /* both terms e2m3, below */ };
 #define DEW_MOE_SPLIT_ROWS_FROM 384
 int dew_moe_prefers_split_rows(const dew_moe_bank* gate, const dew_moe_bank* up, const dew_moe_bank* down, int32_t rows);
 size_t dew_moe_swiglu_mlp_split_workspace_bytes(int32_t tokens, int32_t rows, int32_t depth, int32_t hidden_width, int32_t experts);
@@ -351,6 +351,22 @@ int dew_moe_split_rows_fp6(const void* x /* bf16 [rows, depth] */, void* split /
 int dew_moe_gateup_swiglu_split_fp6_out(const void* x_split, const uint8_t* x_scale, const int32_t* gather,
                                         const int32_t* offsets, const dew_moe_bank* gate, const dew_moe_bank* up,
                                         void* hidden_split, uint8_t* hidden_scales, int32_t rows, void* stream);
+
+/* The same first product with BOTH terms in FP6 (no counterpart in the reference; an option, not the default, for the same
+ * reason as the FP6 second term: it is not exact). dew_moe_split_rows_e2m3_pair: x = s hi + t lo, hi = e2m3(x / s),
+ * lo = e2m3((x - s hi) / t), s and t each one power of two for every 32 depths (the least that brings the block's largest
+ * magnitude, then its largest remainder, within 7.5); no scale a row. Each 64 depths of a row are 128 bytes: for lane group
+ * g = 0, 1 (depths 32 g .. 32 g + 31): 24 bytes of hi codes (six bits each, in order), s's e8m0 byte in a dword, 4 unused
+ * bytes, then the same for lo and t. An element within two binades of its block's largest magnitude is held exactly, any
+ * other to within 2^-10 of that magnitude: the bound of dew_moe_split_rows_fp6, whose launch this one replaces at two
+ * thirds of its matrix-instruction time (two FP6 x FP4 instructions: the time of ONE FP8 x FP4 instruction).
+ * dew_moe_gateup_swiglu_split_e2m3_pair_out is dew_moe_gateup_swiglu_split_out on such rows (no x_scale); its hidden rows
+ * leave as two e4m3 terms under a scale per row and 128 columns, as that entry point's do.                          */
+int dew_moe_split_rows_e2m3_pair(const void* x /* bf16 [rows, depth] */, void* split /* [rows, depth * 2] bytes */, int32_t rows,
+                                 int32_t depth, void* stream);
+int dew_moe_gateup_swiglu_split_e2m3_pair_out(const void* x_split, const int32_t* gather, const int32_t* offsets,
+                                              const dew_moe_bank* gate, const dew_moe_bank* up, void* hidden_split,
+                                              uint8_t* hidden_scales, int32_t rows, void* stream);
 
 /* The blockwise FP8 recipe's forward product (DeepSeek-V3's 1 x 128 activation tiles, 128 x 128 weight blocks):
  * `rows_quantized` src/dew/nn/kernels/projections.py:176-182 and `blockwise_fp8_product`

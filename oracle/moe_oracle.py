@@ -934,6 +934,61 @@ def split_rows_fp6_decoded(split, scale):
     return ((first * s[:, :, None]) + second).reshape(rows, pitch // 2).astype(F32)
 
 
+def _e2m3_block_scale(most):
+    """The least power of two t with most / t <= 7.5 (e2m3's largest magnitude), kept a normal power of two with an e8m0
+    byte of 1 .. 254 (a block of zeros takes the least one)."""
+    bits = np.asarray(most, F32).view(np.uint32)
+    power = (bits >> 23).astype(np.int32) - 127 - 2 + ((bits & 0x7FFFFF) > 0x700000)
+    return np.clip(power, -126, 127)
+
+
+def split_rows_e2m3_pair(x):
+    """bf16 rows as the values `dew_moe_split_rows_e2m3_pair` holds them at (no counterpart in the reference): for every 32
+    depths `s hi + t lo`, s = the least power of two with the block's largest magnitude within 7.5 s, hi = e2m3(x / s),
+    t the same for the remainders x - s hi, lo = e2m3((x - s hi) / t). Returns (values fp32 [rows, K], the two scales' e8m0
+    bytes [rows, K / 32, 2]). Pinned by its invariants (tests/test_projections.py): exact for every element within two
+    binades of its block's largest magnitude, within 2^-10 of that magnitude otherwise, exact on blocks of three binades."""
+    x = np.asarray(x, F32)
+    rows, depth = x.shape
+    rest = x.reshape(rows, depth // 32, 32).copy()
+    total = np.zeros_like(rest)
+    scales = []
+    for _ in range(2):
+        power = _e2m3_block_scale(np.abs(rest).max(axis=-1, keepdims=True))
+        scale = np.ldexp(F32(1), power)
+        held = (e2m3_rounded((rest / scale).astype(F32)) * scale).astype(F32)
+        total = (total + held).astype(F32)
+        rest = (rest - held).astype(F32)
+        scales.append((power[..., 0] + 127).astype(np.uint8))
+    return total.reshape(rows, depth), np.stack(scales, axis=-1)
+
+
+def _six_bit_codes(packed):
+    """`[..., 24]` bytes as the 32 six-bit codes they pack, in order (code i at bits 6 i .. 6 i + 5, little-endian)."""
+    packed = np.asarray(packed, np.uint8).astype(np.uint64)
+    codes = np.zeros((*packed.shape[:-1], 32), np.int64)
+    for i in range(32):
+        low, shift = (6 * i) // 8, (6 * i) % 8
+        two = packed[..., low] | (packed[..., min(low + 1, 23)] << np.uint64(8))
+        codes[..., i] = ((two >> np.uint64(shift)) & np.uint64(63)).astype(np.int64)
+    return codes
+
+
+def split_rows_e2m3_pair_decoded(split):
+    """The values a device buffer of `dew_moe_split_rows_e2m3_pair` stands for, and its scale bytes: `split` uint8
+    [rows, 2 K], each 64 depths 128 bytes: for lane group g (depths 32 g .. 32 g + 31) and term t, 24 bytes of e2m3 codes,
+    the term's e8m0 byte, 7 unused bytes. Returns (values fp32 [rows, K], scale bytes [rows, K / 32, 2])."""
+    split = np.asarray(split, np.uint8)
+    rows, pitch = split.shape
+    pieces = split.reshape(rows, pitch // 128, 2, 2, 32)               # [rows, steps, group, term, 32 bytes]
+    codes = _six_bit_codes(pieces[..., :24])
+    magnitudes = E2M3_GRID[codes & 31] * np.where(codes & 32, F32(-1), F32(1))
+    scales = pieces[..., 24]
+    values = (magnitudes * np.ldexp(F32(1), scales.astype(np.int32) - 127)[..., None]).astype(F32)
+    total = (values[:, :, :, 0] + values[:, :, :, 1]).astype(F32)       # [rows, steps, group, 32]
+    return total.reshape(rows, pitch // 2), scales.reshape(rows, pitch // 64, 2)
+
+
 def swiglu(gate, up, *, dtype="bfloat16", limit=None, exp=np.exp):
     """`gated_product('swiglu')` after `swiglu_clamped` (src/dew/nn/activations.py:267-278,327-356):
     bf16 rounds the activation `g * logistic(g)` and then the product with `u`; fp32 rounds nowhere.

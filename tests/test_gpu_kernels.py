@@ -1040,3 +1040,87 @@ def test_the_gateup_launch_on_an_fp6_second_term_multiplies_the_values_the_rows_
     six = ops.gateup_swiglu_split_out(*ops.split_rows_fp6(xn), pg, pu, od, gather=gd, fp6=True)
     eight = ops.gateup_swiglu_split_out(*ops.split_rows(xn), pg, pu, od, gather=gd)
     assert torch.equal(six[0], eight[0]) and torch.equal(six[1][:, :width // 128], eight[1][:, :width // 128])
+
+
+def test_split_rows_as_two_e2m3_terms_hold_what_the_oracle_says(ops):
+    """`split_rows_e2m3_pair`: the device's bytes decoded on the host are the oracle's values and scale bytes, bit for bit,
+    on rows of many shapes; an element within two binades of its 32-deep block's largest magnitude is held exactly, any
+    other within 2^-10 of that magnitude; blocks of three binades are held exactly."""
+    rng = np.random.default_rng(18)
+    rows, depth = 64, 512
+    x = rng.standard_normal((rows, depth)).astype(np.float32)
+    x[8:16] *= 10.0 ** rng.uniform(-4, 4, size=(8, depth)).astype(np.float32)
+    x[16] = 0.0
+    x[17, 5] = 3.0e4
+    x[18] *= 1e-30
+    x[19] = np.exp2(rng.integers(0, 3, size=depth)) * rng.choice([-1.0, 1.0], size=depth) * (1 + rng.integers(0, 128, size=depth) / 128)  # three binades
+    x[20] *= 1e30
+    xb = torch.from_numpy(x).to(torch.bfloat16)
+    split, none = ops.split_rows_e2m3_pair(xb.cuda())
+    assert none is None and split.shape == (rows, 2 * depth)
+    want_values, want_scales = oracle.split_rows_e2m3_pair(bf16_np(xb))
+    got, got_scales = oracle.split_rows_e2m3_pair_decoded(split.cpu().numpy())
+    assert np.array_equal(got_scales, want_scales) and np.array_equal(got, want_values)
+    exact = bf16_np(xb)
+    blocks = np.abs(exact).reshape(rows, depth // 32, 32)
+    largest = blocks.max(axis=-1, keepdims=True)
+    binade = np.where(largest > 0, np.exp2(np.floor(np.log2(np.maximum(largest, 1e-45)))), 0.0)
+    near = (blocks >= binade / 4).reshape(rows, depth)
+    assert near.mean() > 0.5 and np.array_equal(got[near], exact[near])
+    assert (np.abs(got - exact).reshape(rows, depth // 32, 32) <= largest * 2.0 ** -10).all()
+    assert np.array_equal(got[19], exact[19]) and not got[16].any()
+    assert ops.split_rows_as(xb.cuda(), "e2m3x2")[1] is None and torch.equal(ops.split_rows_as(xb.cuda(), "e2m3x2")[0], split)
+
+
+@pytest.mark.parametrize("depth", [256, 1280])
+def test_the_gateup_launch_on_two_e2m3_terms_multiplies_the_values_the_rows_hold(ops, depth):
+    """Two FP6 terms change the rows' values (to the oracle's `split_rows_e2m3_pair`), not the product's arithmetic: against
+    the float64 sums of those values through the decoded banks the hidden rows agree as the two-e4m3 launch's do with the
+    bf16 rows', at both tile heights; and rows both forms hold exactly (three binades a row) give the two-e4m3 launch's
+    hidden rows bit for bit."""
+    sizes = [700, 0, 290, 5]
+    width = 256
+    gate, x, offsets = grouped_case("mxfp4", len(sizes), depth, width, sizes, seed=depth + 31)
+    up, _, _ = grouped_case("mxfp4", len(sizes), depth, width, sizes, seed=depth + 32)
+    (gate_values, gate_factor), (up_values, up_factor) = dequantized(gate), dequantized(up)
+    rng = np.random.default_rng(depth + 1)
+    rows = x.shape[0]
+    gather = rng.integers(0, rows, size=rows).astype(np.int32)
+    od, gd = torch.from_numpy(offsets).cuda(), torch.from_numpy(gather).cuda()
+    pg, pu = ops.prepare(gate.to("cuda")), ops.prepare(up.to("cuda"))
+
+    def hidden_rows(split, scales):     # the split hidden rows rebuilt on the host
+        pieces = split.cpu().numpy().reshape(rows, width // 64, 2, 2, 2, 16)
+        terms = oracle._e4m3_table()[pieces].astype(np.float64)
+        values = (terms[:, :, :, 0] + terms[:, :, :, 1] / 16).transpose(0, 1, 3, 2, 4).reshape(rows, width // 128, 128)
+        s = np.ldexp(np.float64(1), scales.cpu().numpy()[:, :width // 128].astype(np.int64) - 127)[:, :, None]
+        return (values * s).reshape(rows, width)
+
+    held, _ = oracle.split_rows_e2m3_pair(bf16_np(x))
+    bounds = np.concatenate([[0], np.cumsum(sizes)])
+    want = np.zeros((rows, width))
+    for e in range(len(sizes)):
+        span = slice(bounds[e], bounds[e + 1])
+        operand = held[gather[span]].astype(np.float64)
+        g = oracle.bf16_round((operand @ gate_values[e].astype(np.float64) * (1.0 if gate_factor is None else gate_factor[e])).astype(np.float32))
+        u = oracle.bf16_round((operand @ up_values[e].astype(np.float64) * (1.0 if up_factor is None else up_factor[e])).astype(np.float32))
+        want[span] = oracle.swiglu(g, u)
+    pieces = ops.split_rows_e2m3_pair(x.cuda())
+    for tile in (0, 256):
+        with ops.tile_rows(tile):
+            got = hidden_rows(*ops.gateup_swiglu_split_out(*pieces, pg, pu, od, gather=gd, terms="e2m3x2"))
+        assert np.abs(got - want).max() <= 2 ** -6 * np.abs(want).max() and (got == want).mean() > 0.9, tile
+    exact = oracle.swiglu(oracle.grouped_matmul(bf16_np(x)[gather], gate_values, sizes, factor=gate_factor),
+                          oracle.grouped_matmul(bf16_np(x)[gather], up_values, sizes, factor=up_factor))
+    assert np.abs(got - exact).max() <= 1e-2 * np.abs(exact).max()
+    narrow = np.exp2(rng.integers(-1, 2, size=x.shape)) * rng.choice([-1.0, 1.0], size=x.shape) * (1 + rng.integers(0, 128, size=x.shape) / 128)
+    xn = torch.from_numpy(narrow.astype(np.float32)).to(torch.bfloat16).cuda()
+    six = ops.gateup_swiglu_split_out(*ops.split_rows_e2m3_pair(xn), pg, pu, od, gather=gd, terms="e2m3x2")
+    eight = ops.gateup_swiglu_split_out(*ops.split_rows(xn), pg, pu, od, gather=gd)
+    assert torch.equal(six[0], eight[0]) and torch.equal(six[1][:, :width // 128], eight[1][:, :width // 128])
+    # the whole MLP as one call on the same rows' terms
+    down, _, _ = grouped_case("mxfp4", len(sizes), width, 256, sizes, seed=depth + 33)
+    pd = ops.prepare(down.to("cuda"))
+    whole = ops.swiglu_mlp_split(x.cuda(), pg, pu, pd, od, gather=gd, terms="e2m3x2")
+    apart = ops.grouped_gemm_split_blocks(*ops.gateup_swiglu_split_out(*pieces, pg, pu, od, gather=gd, terms="e2m3x2"), pd, od)
+    assert torch.equal(whole, apart)

@@ -167,3 +167,26 @@ def test_the_nvfp4_operand_follows_the_bank_quantizers_closed_form():
     decoded = values * np.repeat(scales, 16, axis=1) * tensor
     assert (np.abs(decoded - x) <= 0.5 * np.repeat(scales, 16, axis=1) * tensor * 2.0 + 1e-30).all()   # the widest step is 2
     assert oracle.nvfp4_quantized(np.zeros((2, 32), np.float32))[2] == 1.0
+
+
+def test_rows_as_two_e2m3_terms_keep_what_their_bound_says():
+    """`split_rows_e2m3_pair` (the oracle of `dew_moe_split_rows_e2m3_pair`; no counterpart in the reference) by what its
+    definition fixes: every element within two binades of its 32-deep block's largest magnitude is held exactly (four
+    significant bits in each term), any other within 2^-10 of that magnitude; each term lies within e2m3's range under its
+    scale; a block of three binades is exact; a zero block holds zeros under the least scale."""
+    from oracle import moe_oracle as oracle
+
+    rng = np.random.default_rng(2)
+    x = oracle.bf16_round(rng.standard_normal((40, 256)).astype(np.float32) * 10.0 ** rng.uniform(-3, 3, size=(40, 1)).astype(np.float32))
+    x[3] = 0.0
+    x[4] = oracle.bf16_round((np.exp2(rng.integers(0, 3, size=256)) * (1 + rng.integers(0, 128, size=256) / 128)).astype(np.float32))
+    held, scales = oracle.split_rows_e2m3_pair(x)
+    blocks, kept = np.abs(x).reshape(40, 8, 32), held.reshape(40, 8, 32)
+    largest = blocks.max(axis=-1, keepdims=True)
+    binade = np.where(largest > 0, np.exp2(np.floor(np.log2(np.maximum(largest, 1e-45)))), 0.0)
+    near = blocks >= binade / 4
+    assert near.mean() > 0.6 and np.array_equal(kept[near], x.reshape(40, 8, 32)[near])
+    assert (np.abs(kept - x.reshape(40, 8, 32)) <= largest * 2.0 ** -10).all()
+    assert np.array_equal(held[4], x[4]) and not held[3].any() and (scales[3] == 1).all()
+    first = np.ldexp(np.float32(1), scales[..., 0].astype(np.int32) - 127)[..., None]
+    assert (largest <= 7.5 * first).all() and (largest[largest > 0] > 3.75 * first[largest > 0]).all()   # the least such power of two
