@@ -982,7 +982,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
               // (f16 rows: a row's sums times its own 2^s as well, an exact factor of the expert's)
               const int lane_row = kNvF16 ? wm0 + 32 * i + 8 * (q / 4) + 4 * (lane / 32) + q % 4 : 0;
               const float first0 = kNvF16 ? factor0 * row_factor[lane_row] : factor0, first1 = kNvF16 ? factor1 * row_factor[lane_row] : factor1;
-              const float second0 = kNvF16 ? factor0 * row_factor[lane_row + 1] : factor0, second1 = kNvF16 ? factor1 * row_factor[lane_row + 1] : factor1;
+              const float second0 = kNvF16 ? factor0 * row_factor[kNvF16 ? lane_row + 1 : 0] : factor0, second1 = kNvF16 ? factor1 * row_factor[kNvF16 ? lane_row + 1 : 0] : factor1;
               if (plain_swiglu) {
                 mine = swiglu_rounded(acc[0][i][j][q] * first0, acc[kMatrices - 1][i][j][q] * first1) |
                        (static_cast<uint32_t>(swiglu_rounded(acc[0][i][j][q + 1] * second0, acc[kMatrices - 1][i][j][q + 1] * second1)) << 16);
