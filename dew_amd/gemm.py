@@ -143,16 +143,16 @@ operands, the whole step 8.35 against 8.70 ms. False keeps every product on the 
 
 
 SPLIT_SECOND_TERM = "e4m3"
-"""The second term of rows split for the scaled matrix instruction in the expert MLP's first product (two thirds of the
-MLP's work): 'e4m3' (both terms FP8: every element's bf16 value exactly, within 2^-11 of its row's largest; the
-default) or 'e2m3' (FP6 under one power-of-two scale every 32 depths: its instruction takes half the first term's
-cycles; an element more than two binades below its 32-deep block's largest magnitude is held to within 2^-10 of that
-largest, the others exactly). Measured on 16384 tokens of 4096 -> 14336 over 8 experts in one run: the gate/up launch
-4.68 ms ('e2m3') against 5.23 ms ('e4m3'), the step 7.48 against 8.00 ms; on a 192-row sample against the CPU oracle
-both are within 5.3e-3 of the largest output, but 56 % against 91 % of the outputs are bit-identical to the oracle's and
-the element-wise figure is 1.3e-2 against 7.8e-3; on a narrower MLP (512 -> 768) the element-wise figure reaches 2.1e-2,
-past the 2e-2 bar. So 'e2m3' is an option for a caller that accepts that, not the default. The second product (hidden
-rows, whose 128-column blocks span more binades) keeps two e4m3 terms either way."""
+"""How the rows of the expert MLP's first product (two thirds of the MLP's work) are held on the scaled matrix instruction:
+'e4m3' (two FP8 terms: every element's bf16 value exactly, within 2^-11 of its row's largest; the default), or one of two
+EXPERIMENTAL options that are not exact: 'e2m3' (the second term in FP6 under one power-of-two scale every 32 depths: its
+instruction takes half the first term's cycles) and 'e2m3x2' (both terms in FP6, each under its own scale every 32 depths: two
+instructions in the time of one FP8-rate instruction). Either option holds an element exactly within two binades of its
+32-deep block's largest magnitude and to 2^-10 of that magnitude below. Measured on 16384 tokens of 4096 -> 14336 over 8 experts
+in one run: the gate/up launch 5.07 ms ('e4m3'), 4.54 ('e2m3'), 4.32 ('e2m3x2'); against the CPU oracle all three are within
+4.3e-3 of the largest output, but 91 % / 56 % / 55.5 % of the outputs are bit-identical to the oracle's and the element-wise figure
+is 7.8e-3 / 1.3e-2 / 1.3e-2; on a narrower MLP (512 -> 768) the options' element-wise figure reaches 2.1e-2, past the 2e-2 bar. The
+second product (hidden rows, whose blocks span more binades) keeps two e4m3 terms whichever is chosen."""
 
 
 def prepared(bank) -> ops.PreparedBank:

@@ -336,7 +336,9 @@ int dew_moe_gated_mlp_split(const void* x, int32_t tokens, const int32_t* gather
                             float limit, const int32_t* scatter, void* out, int32_t rows, int32_t second_term, void* workspace,
                             size_t workspace_bytes, void* stream);
 
-/* The first product of that pair with the rows' second term in FP6 (no counterpart in the reference). dew_moe_split_rows_fp6:
+/* EXPERIMENTAL options (this one and the next): not exact, outside the 2e-2 element-wise bar the default launches hold
+ * (a 512-deep MLP has read 2.1e-2; the reference's own metric max|d| / max|ref| stays under 1e-2), off by default everywhere.
+ * The first product of that pair with the rows' second term in FP6 (no counterpart in the reference). dew_moe_split_rows_fp6:
  * x = s hi + t lo with hi = e4m3(x / s) under one power-of-two scale s a row (scale[row], as dew_moe_split_rows) and
  * lo = e2m3((x - s hi) / t) under t, one power of two for every 32 depths. Each 64 depths of a row are 128 bytes: for
  * lane group g = 0, 1: 32 bytes of hi codes (depths 16 g .. 16 g + 15, then 32 + 16 g .. 47 + 16 g), 24 bytes of lo codes

@@ -16,6 +16,9 @@ from oracle import moe_oracle as oracle
 pytestmark = pytest.mark.gpu
 
 TOLERANCE = 2e-2
+ELEMENTWISE_ON_FP6_OPTIONS = 4e-2
+"""The element-wise bar of the two experimental FP6 forms of split rows (`gemm.SPLIT_SECOND_TERM` 'e2m3', 'e2m3x2'): twice the
+default paths' 2e-2. They are not exact and are off by default; the reference's own metric is held to 1e-2 on them."""
 
 CASES = {
     "c1-full": CONFIGS["c1"],
@@ -113,23 +116,27 @@ def test_large_groups_on_mxfp4_banks_run_on_split_rows_and_agree_with_the_bf16_l
     got = layer.apply(variables, x, logits=logits).float().cpu().numpy()            # two e4m3 terms: the rows' bf16 values exactly
     assert calls == [1]
     monkeypatch.setattr(gemm, "SPLIT_SECOND_TERM", "e2m3")
-    with_fp6 = layer.apply(variables, x, logits=logits).float().cpu().numpy()       # the option: an e4m3 and an e2m3 term
-    assert calls == [1, 1]
+    with_fp6 = layer.apply(variables, x, logits=logits).float().cpu().numpy()       # an experimental option: an e4m3 and an e2m3 term
+    monkeypatch.setattr(gemm, "SPLIT_SECOND_TERM", "e2m3x2")
+    with_two_fp6 = layer.apply(variables, x, logits=logits).float().cpu().numpy()   # the other: two e2m3 terms
+    assert calls == [1, 1, 1]
     monkeypatch.setattr(gemm, "SPLIT_ROWS", False)
     plain = layer.apply(variables, x, logits=logits).float().cpu().numpy()
-    assert calls == [1, 1]
+    assert calls == [1, 1, 1]
     want, _ = oracle_output(case, data)
     for name, value in (("split rows, two e4m3", got), ("bf16 operands", plain)):
         by_max, by_element = oracle.relative_errors(value, want)
         print(f"\n{name}: max|d|/max|ref| = {by_max:.3e}, element-wise max rel = {by_element:.3e}, identical = {(value == want).mean():.4f}")
         assert by_max <= TOLERANCE and by_element <= TOLERANCE
     assert (got == plain).mean() > 0.9 and np.abs(got - plain).max() <= 2.0 ** -6 * np.abs(plain).max()
-    # the FP6 second term is an option, not the default, because of what it costs here: inside 1e-2 of the largest output
-    # (the reference's own measure), but element-wise it can pass the 2e-2 bar on an MLP this narrow (512 deep)
-    by_max, by_element = oracle.relative_errors(with_fp6, want)
-    print(f"\nsplit rows, e4m3 + e2m3 (option): max|d|/max|ref| = {by_max:.3e}, element-wise max rel = {by_element:.3e}, "
-          f"identical = {(with_fp6 == want).mean():.4f}")
-    assert by_max <= 1e-2 and by_element <= 4e-2
+    # The FP6 terms are experimental options, not the default, because of what they cost here: inside 1e-2 of the largest
+    # output (the reference's own measure, which every path holds to 2e-2), but element-wise they pass this repository's
+    # 2e-2 bar on an MLP this narrow (512 deep), so they are held to a bar of their own, stated as such in the header.
+    for name, value in (("e4m3 + e2m3", with_fp6), ("e2m3 + e2m3", with_two_fp6)):
+        by_max, by_element = oracle.relative_errors(value, want)
+        print(f"\nsplit rows, {name} (experimental option): max|d|/max|ref| = {by_max:.3e}, element-wise max rel = {by_element:.3e}, "
+              f"identical = {(value == want).mean():.4f}")
+        assert by_max <= 1e-2 and by_element <= ELEMENTWISE_ON_FP6_OPTIONS
 
 
 def test_layer_multiplies_its_own_gate_kernel_when_no_logits_are_given():
