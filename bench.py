@@ -417,6 +417,8 @@ def measure(config, args, device, sustained, with_cpu_baseline):
                     "hbm_view": {"algorithmic_bytes": gateup_bytes, "gbs": round(gateup_gbs, 1),
                                  "frac_of_hbm_peak": round(gateup_gbs / PEAKS["hbm_gbs"], 4)}}
     roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
+    if not decode:   # the fractions of the narrower formats' published peaks right beside it
+        roofline["frac_of_fp8_peak"], roofline["frac_of_fp4_peak"] = roofline.pop("frac_of_fp8_peak"), roofline.pop("frac_of_fp4_peak")
     if not decode and stepper.on_split_rows():
         roofline["executed"] = {"tflops": round(2 * achieved, 1), "frac_of_fp8_peak": round(2 * achieved / PEAKS["fp8_mfma"], 4),
                                 "note": "instruction flops: both terms' products",
