@@ -551,7 +551,13 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
         else
           b_regs[set.value][t][a] = *from;
       }
-      if (kFp4 || kMxRows) __builtin_memcpy(&s_regs[set.value][t], b_scale_src[t] + static_cast<size_t>(step) * 128, sizeof(uint32_t));
+      if constexpr (kMxRows) {  // a dword a lane: its column's four scale bytes of the step
+        __builtin_memcpy(&s_regs[set.value][t], b_scale_src[t] + static_cast<size_t>(step) * 128, sizeof(uint32_t));
+      } else if constexpr (kFp4) {
+        // the lane's two e4m3 bytes as the aligned 16-bit load they are (a dword load at 2 lane is misaligned in every
+        // other lane and reads two bytes past the lane's own: 2.4 % of the split-row paired launch)
+        s_regs[set.value][t] = *reinterpret_cast<const uint16_t*>(b_scale_src[t] + static_cast<size_t>(step) * 128);
+      }
     }
   };
 
