@@ -386,12 +386,115 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
     return;
   }
   const int wm0 = (wave / WN) * (BM / WM), wn0 = (wave % WN) * (BN / WN);
+
+  // ---- B loader: tile t = (matrix, 32-column tile j of the wavefront); the lane's piece of each atom ----
+  const uint8_t* b_src[kTiles];
+  const uint8_t* b_scale_src[kTiles];  // FP4: the lane's two e4m3 block scales of each atom
+  float channel_scale[kTiles];         // FP8 channel: the lane's column scale
+  const int n_atoms = p.width / 32, k_atoms = p.depth / kAtomK;
+  const uint32_t b_lane = lane * 16, b_scale_lane = lane * 2;
+#pragma unroll
+  for (int t = 0; t < kTiles; ++t) {
+    // (past a ragged width the tile reads the bank's last 32 columns again, inside the expert's matrix; its results are not stored)
+    const int matrix = t / TJ, column = kRagged ? min(n0 + wn0 + 32 * (t % TJ), p.width - 32) : n0 + wn0 + 32 * (t % TJ);
+    const uint8_t* codes = matrix == 0 ? p.w0.codes : p.w1.codes;
+    const void* scales = matrix == 0 ? p.w0.scales : p.w1.scales;
+    // (a kernel gradient's one "expert" holds every group's tokens: the group's window starts first_step steps in)
+    const size_t first_atom = (static_cast<size_t>(kWindow ? 0 : expert) * n_atoms + column / 32) * k_atoms + first_step * kAtoms;
+    b_src[t] = codes + first_atom * kAtomBytes + b_lane;
+    b_scale_src[t] = nullptr;
+    channel_scale[t] = 1.0f;
+    if (kFp4) {
+      b_scale_src[t] = static_cast<const uint8_t*>(scales) + first_atom * 128 + b_scale_lane;
+    } else if (kMxRows) {  // [E][N / 32][K / 128][32 columns][4 bytes]: the lane's column's dword of each step
+      b_scale_src[t] = static_cast<const uint8_t*>(scales) +
+                       ((static_cast<size_t>(kWindow ? 0 : expert) * n_atoms + column / 32) * (p.depth / 128) + first_step) * 128 + (lane % 32) * 4;
+    } else if (FORMAT == DEW_MOE_W_FP8_CHANNEL) {
+      channel_scale[t] = static_cast<const float*>(scales)[static_cast<size_t>(expert) * p.width + column + lane % 32];
+    }
+  }
+  // FP8 128 x 128 blocks: this thread's first block scale goes into a register now, ahead of the weight loads, and into
+  // the LDS table further down, once the loads behind it are out (a launch of at most 256 scale entries a tile, every
+  // one but the deepest, has no other; the rest are copied there in a loop).
+  float early_scale = 0.0f;
+  if constexpr (kBlockBank) {
+    const int depth_blocks = p.depth / 128, width_blocks = p.width / 128;
+    if (tid < kScaleColumns * depth_blocks) {
+      const int which = tid / depth_blocks, block = tid % depth_blocks;
+      const float* scales = static_cast<const float*>(which / (BN / 128) == 0 ? p.w0.scales : p.w1.scales);
+      early_scale = scales[(static_cast<size_t>(expert) * depth_blocks + block) * width_blocks + n0 / 128 + which % (BN / 128)];
+    }
+  }
+
+  // Raw weight data in flight: kSets register sets (steps s .. s + kSets - 1), so a load has kSets - 2 to
+  // kSets - 1 steps to land.
+  u32x4_t b_regs[kSets][kTiles][kAtoms];
+  uint32_t s_regs[kSets][kTiles];  // FP4: two e4m3 scale bytes in the low half
+  auto load_b = [&](auto set, int step, auto begin, auto end) __attribute__((always_inline)) {
+#pragma unroll
+    for (int t = begin.value; t < end.value; ++t) {
+#pragma unroll
+      for (int a = 0; a < kAtoms; ++a) {
+        const u32x4_t* from = reinterpret_cast<const u32x4_t*>(b_src[t] + (static_cast<size_t>(step) * kAtoms + a) * kAtomBytes);
+        // Decode-sized groups (the 32-row tiles) read every weight byte once: loaded as non-temporal the stream runs 3 to 6 %
+        // faster (a read-only stream of 16-byte loads measures 7.1 TB/s so hinted against 5.6 to 6.4 without). Taller
+        // tiles keep the plain load: their groups' tiles share weight strips through the L2 (128-row tiles: 2 to 4 % slower
+        // with the hint).
+        if constexpr (BM <= 32)
+          b_regs[set.value][t][a] = __builtin_nontemporal_load(from);
+        else
+          b_regs[set.value][t][a] = *from;
+      }
+      if constexpr (kMxRows) {  // a dword a lane: its column's four scale bytes of the step
+        __builtin_memcpy(&s_regs[set.value][t], b_scale_src[t] + static_cast<size_t>(step) * 128, sizeof(uint32_t));
+      } else if constexpr (kFp4) {
+        // the lane's two e4m3 bytes as the aligned 16-bit load they are (a dword load at 2 lane is misaligned in every
+        // other lane and reads two bytes past the lane's own: 2.4 % of the split-row paired launch)
+        s_regs[set.value][t] = *reinterpret_cast<const uint16_t*>(b_scale_src[t] + static_cast<size_t>(step) * 128);
+      }
+    }
+  };
+
+  // A tile's start is a chain of dependent loads: the groups' offsets, then the rows' gather indices, then the rows and
+  // their scales. The weights depend on the first link alone. So the gather indices are asked for first and the first
+  // weight loads right behind them, before anything waits: loads return in order, the indices are back after one round
+  // trip with the weights still in flight, and the rows' loads follow them. (Issued behind the other set-up, as they
+  // were, the weights started two round trips later: about 1.5 us of a decode launch's 35 to 70.)
+  int a_source[kRowLoads];  // the source row of each of this lane's row loads
+#pragma unroll
+  for (int i = 0; i < kRowLoads; ++i) {
+    const int sorted = row0 + min((wave * kRowLoads + i) * 8 + lane / 8, valid_rows - 1);
+    a_source[i] = kWindow ? sorted - expert * p.window_rows : p.gather ? p.gather[sorted] : sorted;
+  }
+  int tile_source[kSplit ? TI : 1];  // split rows: the lane's row of each row tile
+  if constexpr (kSplit) {
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {
+      const int sorted = row0 + min(wm0 + 32 * i + lane % 32, valid_rows - 1);
+      tile_source[i] = p.gather ? p.gather[sorted] : sorted;
+    }
+  }
+  int thread_source = 0;  // row tid of the tile, where one thread fetches one row's scales
+  if constexpr (kNvF16 || kBlockScales || kMxRows) {
+    if (tid < BM) {
+      const int sorted = row0 + min(tid, valid_rows - 1);
+      thread_source = kWindow ? sorted - expert * p.window_rows : p.gather ? p.gather[sorted] : sorted;
+    }
+  }
+  {
+    constexpr std::integral_constant<int, 0> set0{};
+    constexpr std::integral_constant<int, 1> set1{};
+    constexpr std::integral_constant<int, 2> set2{};
+    constexpr std::integral_constant<int, kTiles> every_tile{};
+    load_b(set0, 0, set0, every_tile);
+    if constexpr (kSets >= 3) load_b(set1, min(1, steps - 1), set0, every_tile);
+    if constexpr (kSets == 4) load_b(set2, min(2, steps - 1), set0, every_tile);
+  }
+
   if constexpr (kNvF16) {
     static_assert(!kNvF16 || BM <= kThreads, "one thread fetches one row's scale");
-    if (tid < BM) {  // (read in the epilogue, behind the loop's barriers)
-      const int sorted = row0 + min(tid, valid_rows - 1);
-      row_factor[tid] = __uint_as_float(static_cast<uint32_t>(p.a_scale[p.gather ? p.gather[sorted] : sorted]) << 23);
-    }
+    if (tid < BM)  // (read in the epilogue, behind the loop's barriers)
+      row_factor[tid] = __uint_as_float(static_cast<uint32_t>(p.a_scale[thread_source]) << 23);
   }
 
   // ---- A loader. One global_load_lds_dwordx4 of a wavefront fills 1 KiB of LDS, lane l landing at byte 16 l:
@@ -402,10 +505,8 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   for (int i = 0; i < kRowLoads; ++i) {
     const int row = (wave * kRowLoads + i) * 8 + lane / 8;
     const int chunk = (lane % 8) ^ (((row >> 1) & 7) ^ ((row & 1) << 2));
-    const int sorted = row0 + min(row, valid_rows - 1);
-    const int source = kWindow ? sorted - expert * p.window_rows : p.gather ? p.gather[sorted] : sorted;
     // (a row of e4m3 codes is depth bytes.) Less the load's immediate offset, which the instruction adds back: see load_a
-    a_src[i] = p.x + static_cast<size_t>(source) * (kFp8A ? p.depth / 2 : p.depth) + first_step * (kFp8A ? kStepDepth / 2 : kStepDepth) + chunk * 8 - (i % 4) * 512;
+    a_src[i] = p.x + static_cast<size_t>(a_source[i]) * (kFp8A ? p.depth / 2 : p.depth) + first_step * (kFp8A ? kStepDepth / 2 : kStepDepth) + chunk * 8 - (i % 4) * 512;
     asm volatile("" : "+v"(a_src[i]));  // kept as computed: the compiler otherwise re-adds the bias at every load
   }
   // Split activations: the lane's row of each row tile carries one e8m0 scale; the hi term multiplies under it
@@ -415,10 +516,8 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   for (int i = 0; i < TI; ++i) {
     a_scale_word[i] = 0;
     if constexpr (kSplit) {
-      const int sorted = row0 + min(wm0 + 32 * i + lane % 32, valid_rows - 1);
-      const int source = p.gather ? p.gather[sorted] : sorted;
       if constexpr (!kBlockScales && !kHi6) {  // (two FP6 terms carry their scales with their codes)
-        const int byte = p.a_scale[source];
+        const int byte = p.a_scale[tile_source[i]];
         a_scale_word[i] = byte | ((byte - 4) << 8);
       }
     }
@@ -434,9 +533,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   if constexpr (kBlockScales) {
     static_assert(!kBlockScales || BM <= kThreads, "one thread copies one row's scales");
     if (tid < BM) {
-      const int sorted = row0 + min(tid, valid_rows - 1);
-      const int source = p.gather ? p.gather[sorted] : sorted;
-      const u32x4_t* from = reinterpret_cast<const u32x4_t*>(p.a_scale + static_cast<size_t>(source) * a_pitch);
+      const u32x4_t* from = reinterpret_cast<const u32x4_t*>(p.a_scale + static_cast<size_t>(thread_source) * a_pitch);
       u32x4_t* to = reinterpret_cast<u32x4_t*>(block_scales + tid * a_pitch);
       for (int piece = 0; piece < a_pitch / 16; ++piece) to[piece] = from[piece];
     }
@@ -476,9 +573,7 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   (void)a_mx_src;  // (the host pass compiles no load)
   if constexpr (kMxRows) {
     static_assert(!kMxRows || BM == kThreads, "one thread fetches one row's scales");
-    const int sorted = row0 + min(tid, valid_rows - 1);
-    const int source = kWindow ? sorted - expert * p.window_rows : p.gather ? p.gather[sorted] : sorted;
-    a_mx_src = p.a_scale + static_cast<size_t>(source) * (p.depth / 32) + first_step * 4;
+    a_mx_src = p.a_scale + static_cast<size_t>(thread_source) * (p.depth / 32) + first_step * 4;
   }
   auto load_a_scales = [&](int stage_number, int step) __attribute__((always_inline)) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -496,70 +591,16 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
     }
   };
 
-  // ---- B loader: tile t = (matrix, 32-column tile j of the wavefront); the lane's piece of each atom ----
-  const uint8_t* b_src[kTiles];
-  const uint8_t* b_scale_src[kTiles];  // FP4: the lane's two e4m3 block scales of each atom
-  float channel_scale[kTiles];         // FP8 channel: the lane's column scale
-  const int n_atoms = p.width / 32, k_atoms = p.depth / kAtomK;
-  const uint32_t b_lane = lane * 16, b_scale_lane = lane * 2;
-#pragma unroll
-  for (int t = 0; t < kTiles; ++t) {
-    // (past a ragged width the tile reads the bank's last 32 columns again, inside the expert's matrix; its results are not stored)
-    const int matrix = t / TJ, column = kRagged ? min(n0 + wn0 + 32 * (t % TJ), p.width - 32) : n0 + wn0 + 32 * (t % TJ);
-    const uint8_t* codes = matrix == 0 ? p.w0.codes : p.w1.codes;
-    const void* scales = matrix == 0 ? p.w0.scales : p.w1.scales;
-    // (a kernel gradient's one "expert" holds every group's tokens: the group's window starts first_step steps in)
-    const size_t first_atom = (static_cast<size_t>(kWindow ? 0 : expert) * n_atoms + column / 32) * k_atoms + first_step * kAtoms;
-    b_src[t] = codes + first_atom * kAtomBytes + b_lane;
-    b_scale_src[t] = nullptr;
-    channel_scale[t] = 1.0f;
-    if (kFp4) {
-      b_scale_src[t] = static_cast<const uint8_t*>(scales) + first_atom * 128 + b_scale_lane;
-    } else if (kMxRows) {  // [E][N / 32][K / 128][32 columns][4 bytes]: the lane's column's dword of each step
-      b_scale_src[t] = static_cast<const uint8_t*>(scales) +
-                       ((static_cast<size_t>(kWindow ? 0 : expert) * n_atoms + column / 32) * (p.depth / 128) + first_step) * 128 + (lane % 32) * 4;
-    } else if (FORMAT == DEW_MOE_W_FP8_CHANNEL) {
-      channel_scale[t] = static_cast<const float*>(scales)[static_cast<size_t>(expert) * p.width + column + lane % 32];
-    }
-  }
   if constexpr (kBlockBank) {
     const int depth_blocks = p.depth / 128, width_blocks = p.width / 128;
-    for (int item = tid; item < kScaleColumns * depth_blocks; item += kThreads) {
+    if (tid < kScaleColumns * depth_blocks) depth_scales[tid / depth_blocks][tid % depth_blocks] = early_scale;
+    for (int item = tid + kThreads; item < kScaleColumns * depth_blocks; item += kThreads) {
       const int which = item / depth_blocks, block = item % depth_blocks;
       const float* scales = static_cast<const float*>(which / (BN / 128) == 0 ? p.w0.scales : p.w1.scales);
       depth_scales[which][block] =
           scales[(static_cast<size_t>(expert) * depth_blocks + block) * width_blocks + n0 / 128 + which % (BN / 128)];
     }
   }
-
-  // Raw weight data in flight: kSets register sets (steps s .. s + kSets - 1), so a load has kSets - 2 to
-  // kSets - 1 steps to land.
-  u32x4_t b_regs[kSets][kTiles][kAtoms];
-  uint32_t s_regs[kSets][kTiles];  // FP4: two e4m3 scale bytes in the low half
-  auto load_b = [&](auto set, int step, auto begin, auto end) __attribute__((always_inline)) {
-#pragma unroll
-    for (int t = begin.value; t < end.value; ++t) {
-#pragma unroll
-      for (int a = 0; a < kAtoms; ++a) {
-        const u32x4_t* from = reinterpret_cast<const u32x4_t*>(b_src[t] + (static_cast<size_t>(step) * kAtoms + a) * kAtomBytes);
-        // Decode-sized groups (the 32-row tiles) read every weight byte once: loaded as non-temporal the stream runs 3 to 6 %
-        // faster (a read-only stream of 16-byte loads measures 7.1 TB/s so hinted against 5.6 to 6.4 without). Taller
-        // tiles keep the plain load: their groups' tiles share weight strips through the L2 (128-row tiles: 2 to 4 % slower
-        // with the hint).
-        if constexpr (BM <= 32)
-          b_regs[set.value][t][a] = __builtin_nontemporal_load(from);
-        else
-          b_regs[set.value][t][a] = *from;
-      }
-      if constexpr (kMxRows) {  // a dword a lane: its column's four scale bytes of the step
-        __builtin_memcpy(&s_regs[set.value][t], b_scale_src[t] + static_cast<size_t>(step) * 128, sizeof(uint32_t));
-      } else if constexpr (kFp4) {
-        // the lane's two e4m3 bytes as the aligned 16-bit load they are (a dword load at 2 lane is misaligned in every
-        // other lane and reads two bytes past the lane's own: 2.4 % of the split-row paired launch)
-        s_regs[set.value][t] = *reinterpret_cast<const uint16_t*>(b_scale_src[t] + static_cast<size_t>(step) * 128);
-      }
-    }
-  };
 
   // ---- fragments: slice kk of a step is 16 depths; a lane's are the 8 its weight bytes cover ----
   bf16x8_t a_frag[2][TI], b_frag[2][kTiles];
@@ -728,7 +769,6 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   constexpr std::integral_constant<int, 2 * kTiles / 4> b2{};
   constexpr std::integral_constant<int, 3 * kTiles / 4> b3{};
   constexpr std::integral_constant<int, kTiles> b4{};
-  constexpr std::integral_constant<int, kTiles> all_tiles{};
   constexpr int kMfmas = kMatrices * TI * TJ;
   constexpr int kDequantOps = kBf16 ? 0 : kTiles * (kPow2 ? 5 : kNvF16 ? 10 : 17);  // vector instructions to dequantize one slice
   constexpr int kLoadsPerTile = kAtoms + (kFp4 || kMxRows ? 1 : 0);
@@ -860,9 +900,6 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
     __builtin_amdgcn_sched_barrier(0);
     stage_index = next_index;
   };
-  load_b(c0, 0, c0, all_tiles);
-  if constexpr (kSets >= 3) load_b(c1, min(1, steps - 1), c0, all_tiles);
-  if constexpr (kSets == 4) load_b(c2, min(2, steps - 1), c0, all_tiles);
   load_a(lds, 0, c0, a4);
   load_a(lds + kStageChunks, min(1, steps - 1), c0, a4);
   load_a_scales(0, 0);
