@@ -1008,56 +1008,70 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
       const int sorted = row0 + min(pass * kPassRows + (tid + it * kThreads) / kRowChunks, valid_rows - 1);
       out_rows[it] = p.scatter ? p.scatter[sorted] : sorted;
     }
+    // The tile's rounded outputs into the LDS. `plain` (SwiGLU, no clamp) is the same for the whole launch; the choice is made
+    // once, around the whole nest, and each side holds cross-lane moves and LDS stores: written as a condition around the
+    // arithmetic alone, the compiler evaluated both gates for every output and selected (two exponentials and reciprocals
+    // an output; the arithmetic of a 32-row tile's outputs took 6 300 cycles, a tenth of a decode tile's life).
+    auto stage_tiles = [&](auto plain) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < TI; ++i) {
-      const int block_tile = wm0 / 32 + i;  // this wavefront's row tile i among the block's
-      if (block_tile / kPassTiles != pass) continue;
-      const int ii = block_tile % kPassTiles;
+      for (int i = 0; i < TI; ++i) {
+        const int block_tile = wm0 / 32 + i;  // this wavefront's row tile i among the block's
+        if (block_tile / kPassTiles != pass) continue;
+        const int ii = block_tile % kPassTiles;
 #pragma unroll
-      for (int q = 0; q < 16; q += 2) {
-        const int row = 32 * ii + 8 * (q / 4) + 4 * (lane / 32) + q % 4 + (odd_lane ? 1 : 0);  // within the pass
+        for (int q = 0; q < 16; q += 2) {
+          const int row = 32 * ii + 8 * (q / 4) + 4 * (lane / 32) + q % 4 + (odd_lane ? 1 : 0);  // within the pass
 #pragma unroll
-        for (int j = 0; j < TJ; ++j) {
-          if constexpr (kGated) {
-            // The even lane holds a gate column and the odd lane the up column beside it, rows q and q + 1 each:
-            // the even lane takes the pair of row q, the odd lane the pair of row q + 1, and each writes one value.
-            float mine[2];
+          for (int j = 0; j < TJ; ++j) {
+            if constexpr (kGated) {
+              // The even lane holds a gate column and the odd lane the up column beside it, rows q and q + 1 each:
+              // the even lane takes the pair of row q, the odd lane the pair of row q + 1, and each writes one value.
+              float mine[2];
 #pragma unroll
-            for (int r = 0; r < 2; ++r) mine[r] = bf16_round(acc[0][i][j][q + r] * factor0 + bias[j]);
-            const float sent = odd_lane ? mine[0] : mine[1];
-            const float got = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(uint32_t, sent), 0xB1, 0xF, 0xF, true));
-            const bf16_t value = odd_lane ? gated_pair_rounded(got, mine[1], p.limit) : gated_pair_rounded(mine[0], got, p.limit);
-            reinterpret_cast<bf16_t*>(staged)[row * (2 * kRowDwords) + (wn0 + 32 * j + lane % 32) / 2] = value;
-          } else {
-            // the lane's rows q (low half) and q + 1 (high half) of its column, rounded
-            uint32_t mine;
-            if constexpr (PAIRED) {
-              // (f16 rows: a row's sums times its own 2^s as well, an exact factor of the expert's)
-              const int lane_row = kNvF16 ? wm0 + 32 * i + 8 * (q / 4) + 4 * (lane / 32) + q % 4 : 0;
-              const float first0 = kNvF16 ? factor0 * row_factor[lane_row] : factor0, first1 = kNvF16 ? factor1 * row_factor[lane_row] : factor1;
-              const float second0 = kNvF16 ? factor0 * row_factor[kNvF16 ? lane_row + 1 : 0] : factor0, second1 = kNvF16 ? factor1 * row_factor[kNvF16 ? lane_row + 1 : 0] : factor1;
-              if (plain_swiglu) {
-                mine = swiglu_rounded(acc[0][i][j][q] * first0, acc[kMatrices - 1][i][j][q] * first1) |
-                       (static_cast<uint32_t>(swiglu_rounded(acc[0][i][j][q + 1] * second0, acc[kMatrices - 1][i][j][q + 1] * second1)) << 16);
-              } else {  // a clamp or the GeGLU gate (the same for every lane: a branch, not a select)
-                mine = gated_rounded(acc[0][i][j][q] * first0, acc[kMatrices - 1][i][j][q] * first1, p.limit, p.gating) |
-                       (static_cast<uint32_t>(gated_rounded(acc[0][i][j][q + 1] * second0, acc[kMatrices - 1][i][j][q + 1] * second1, p.limit, p.gating)) << 16);
-              }
-            } else if constexpr (kFp4) {
-              mine = pack_bf16(acc[0][i][j][q] * factor0 + bias[j], acc[0][i][j][q + 1] * factor0 + bias[j]);
-            } else if constexpr (kWindow) {
-              mine = pack_bf16(acc[0][i][j][q] * window_factor, acc[0][i][j][q + 1] * window_factor);
+              for (int r = 0; r < 2; ++r) mine[r] = bf16_round(acc[0][i][j][q + r] * factor0 + bias[j]);
+              const float sent = odd_lane ? mine[0] : mine[1];
+              const float got = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(uint32_t, sent), 0xB1, 0xF, 0xF, true));
+              const bf16_t value = odd_lane ? gated_pair_rounded(got, mine[1], p.limit) : gated_pair_rounded(mine[0], got, p.limit);
+              reinterpret_cast<bf16_t*>(staged)[row * (2 * kRowDwords) + (wn0 + 32 * j + lane % 32) / 2] = value;
             } else {
-              mine = pack_bf16(acc[0][i][j][q] + bias[j], acc[0][i][j][q + 1] + bias[j]);
+              // the lane's rows q (low half) and q + 1 (high half) of its column, rounded
+              uint32_t mine;
+              if constexpr (PAIRED) {
+                // (f16 rows: a row's sums times its own 2^s as well, an exact factor of the expert's)
+                const int lane_row = kNvF16 ? wm0 + 32 * i + 8 * (q / 4) + 4 * (lane / 32) + q % 4 : 0;
+                const float first0 = kNvF16 ? factor0 * row_factor[lane_row] : factor0, first1 = kNvF16 ? factor1 * row_factor[lane_row] : factor1;
+                const float second0 = kNvF16 ? factor0 * row_factor[kNvF16 ? lane_row + 1 : 0] : factor0, second1 = kNvF16 ? factor1 * row_factor[kNvF16 ? lane_row + 1 : 0] : factor1;
+                if constexpr (decltype(plain)::value) {
+                  mine = swiglu_rounded(acc[0][i][j][q] * first0, acc[kMatrices - 1][i][j][q] * first1) |
+                         (static_cast<uint32_t>(swiglu_rounded(acc[0][i][j][q + 1] * second0, acc[kMatrices - 1][i][j][q + 1] * second1)) << 16);
+                } else {  // a clamp or the GeGLU gate
+                  mine = gated_rounded(acc[0][i][j][q] * first0, acc[kMatrices - 1][i][j][q] * first1, p.limit, p.gating) |
+                         (static_cast<uint32_t>(gated_rounded(acc[0][i][j][q + 1] * second0, acc[kMatrices - 1][i][j][q + 1] * second1, p.limit, p.gating)) << 16);
+                }
+              } else if constexpr (kFp4) {
+                mine = pack_bf16(acc[0][i][j][q] * factor0 + bias[j], acc[0][i][j][q + 1] * factor0 + bias[j]);
+              } else if constexpr (kWindow) {
+                mine = pack_bf16(acc[0][i][j][q] * window_factor, acc[0][i][j][q + 1] * window_factor);
+              } else {
+                mine = pack_bf16(acc[0][i][j][q] + bias[j], acc[0][i][j][q + 1] + bias[j]);
+              }
+              // the even lane keeps row q of both columns and the odd lane row q + 1: each takes the neighbour's pair
+              // (quad_perm [1,0,3,2]) and picks its four bytes out of the two pairs with one byte permute
+              const uint32_t other = __builtin_amdgcn_mov_dpp(mine, 0xB1, 0xF, 0xF, true);
+              const uint32_t packed = __builtin_amdgcn_perm(other, mine, swap_select);
+              staged[row * kRowDwords + (wn0 + 32 * j + (lane % 32 & ~1)) / 2] = packed;
             }
-            // the even lane keeps row q of both columns and the odd lane row q + 1: each takes the neighbour's pair
-            // (quad_perm [1,0,3,2]) and picks its four bytes out of the two pairs with one byte permute
-            const uint32_t other = __builtin_amdgcn_mov_dpp(mine, 0xB1, 0xF, 0xF, true);
-            const uint32_t packed = __builtin_amdgcn_perm(other, mine, swap_select);
-            staged[row * kRowDwords + (wn0 + 32 * j + (lane % 32 & ~1)) / 2] = packed;
           }
         }
       }
+    };
+    if constexpr (PAIRED) {
+      if (plain_swiglu)
+        stage_tiles(std::true_type{});
+      else
+        stage_tiles(std::false_type{});
+    } else {
+      stage_tiles(std::true_type{});
     }
     __syncthreads();
 #pragma unroll
