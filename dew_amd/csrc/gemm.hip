@@ -184,12 +184,12 @@ __device__ __forceinline__ bf16x8_t fragment_fp4_f16(uint32_t word, _Float16 sca
 // Bytes of one row's block scales (one e8m0 byte for 128 elements), padded to whole 16-byte loads.
 __host__ __device__ constexpr int block_scale_pitch(int elements) { return (elements / 128 + 15) / 16 * 16; }
 
-// Dynamic LDS of a block: the three-stage ring of A rows, or the staged output tile where that is larger
-// (the 32-row tile of 256 columns).
+// Dynamic LDS of a block: the three-stage ring of A rows, or the staged output tile (the 32-row tile of 256 columns) with
+// the table of its rows' destinations behind it, where that is larger.
 template <int BM, int BN, int MODE>
 constexpr size_t shared_bytes() {
   constexpr size_t ring = 3 * static_cast<size_t>(BM) * BK * 2;
-  constexpr size_t staged = static_cast<size_t>(BM / ((BN == 256 && BM > 32) ? 2 : 1)) * ((MODE == 2 ? BN / 2 : BN) / 2 + 4) * 4;
+  constexpr size_t staged = static_cast<size_t>(BM / ((BN == 256 && BM > 32) ? 2 : 1)) * ((MODE == 2 ? BN / 2 : BN) / 2 + 4) * 4 + BM * 4;
   return ring > staged ? ring : staged;
 }
 
@@ -424,6 +424,14 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
       const float* scales = static_cast<const float*>(which / (BN / 128) == 0 ? p.w0.scales : p.w1.scales);
       early_scale = scales[(static_cast<size_t>(expert) * depth_blocks + block) * width_blocks + n0 / 128 + which % (BN / 128)];
     }
+  }
+
+  // FP4 banks: the expert's tensor scales, which the epilogue multiplies by, are asked for here as well (fetched there, the
+  // epilogue's arithmetic began with a memory round trip)
+  float tensor_scale0 = 1.0f, tensor_scale1 = 1.0f;
+  if constexpr (kFp4) {
+    tensor_scale0 = p.w0.tensor_scale[expert];
+    if constexpr (PAIRED) tensor_scale1 = p.w1.tensor_scale[expert];
   }
 
   // Raw weight data in flight: kSets register sets (steps s .. s + kSets - 1), so a load has kSets - 2 to
@@ -908,6 +916,10 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   __builtin_amdgcn_s_waitcnt(kWaitAll);
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
+  if constexpr (kFp4) {  // (the same for every lane: kept in scalar registers through the loop)
+    tensor_scale0 = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, tensor_scale0)));
+    tensor_scale1 = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, tensor_scale1)));
+  }
   if constexpr (kSplit) {
     load_block_scales(0);
     form_block_words(c0);
@@ -943,13 +955,11 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   // A ring no longer needs, row-major, and the block then writes whole output rows, 16 bytes a lane, so that
   // the tile leaves as full cache lines (direct 4-byte stores of 64-byte row pieces took a quarter of the
   // kernel's time). Tiles of 256 columns are staged in two passes of BM / 2 rows.
-  float factor0 = 1.0f, factor1 = 1.0f;
-  if (kFp4) {  // the 2^8 the decode owes times the expert's tensor scale (src/dew/nn/kernels/gemm.py:660-662)
-    // (the scaled instruction applies the block scales themselves, not their 2^-8)
-    // (f16 rows: the codes times their block scales as they are, no 2^-8; each row's own 2^s joins below)
-    factor0 = (kSplit || kNvF16 ? 1.0f : 256.0f) * p.w0.tensor_scale[expert];
-    if (PAIRED) factor1 = (kSplit || kNvF16 ? 1.0f : 256.0f) * p.w1.tensor_scale[expert];
-  }
+  // the 2^8 the decode owes times the expert's tensor scale (src/dew/nn/kernels/gemm.py:660-662)
+  // (the scaled instruction applies the block scales themselves, not their 2^-8)
+  // (f16 rows: the codes times their block scales as they are, no 2^-8; each row's own 2^s joins below)
+  const float factor0 = kFp4 ? (kSplit || kNvF16 ? 1.0f : 256.0f) * tensor_scale0 : 1.0f;
+  const float factor1 = kFp4 && PAIRED ? (kSplit || kNvF16 ? 1.0f : 256.0f) * tensor_scale1 : 1.0f;
   float window_factor = 1.0f;
   if constexpr (kWindow) window_factor = (p.factor0 ? *p.factor0 : 1.0f) * (p.factor1 ? *p.factor1 : 1.0f);
   if constexpr (MODE == kPlainF32) {
@@ -973,8 +983,10 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   constexpr int kRowChunks = kOutBN / 8;      // 16-byte pieces of an output row
   constexpr int kStoreIters = kPassRows * kRowChunks / kThreads;
   static_assert(kPassRows * kRowChunks % kThreads == 0, "whole store rounds");
-  static_assert((BM / 32) % kPasses == 0 && kPassRows * kRowDwords * 4 <= shared_bytes<BM, BN, MODE>(), "staged tile fits the LDS");
+  static_assert((BM / 32) % kPasses == 0 && kPassRows * kRowDwords * 4 + BM * 4 <= shared_bytes<BM, BN, MODE>(), "staged tile fits the LDS");
+  static_assert(BM <= kThreads, "one thread fetches one row's destination");
   uint32_t* staged = reinterpret_cast<uint32_t*>(lds);
+  int* out_row_of = reinterpret_cast<int*>(staged + kPassRows * kRowDwords);  // where each of the tile's rows goes, behind the staged tile
   const bool odd_lane = lane & 1;
   const int out_width = kGated ? p.width / 2 : p.width, out_n0 = kGated ? n0 / 2 : n0;
   // Each expert's bias meets its rows' fp32 sums before their one rounding (src/dew/nn/moe.py:729-742).
@@ -998,16 +1010,24 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   const uint32_t swap_select = odd_lane ? 0x03020706u : 0x05040100u;
   const bool plain_swiglu = p.limit <= 0.0f && p.gating == DEW_MOE_GATE_SILU;  // (kernel arguments: the same for the whole launch)
   __builtin_amdgcn_s_barrier();  // every wavefront has read its last A fragments: the ring is free
+  if constexpr (!PAIRED) {
+    // (the bias has landed: stated here, so that the arithmetic below waits for no load, and the scatter indices, which
+    // are fetched next, stay in flight under it)
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) asm volatile("" : "+v"(bias[j]));
+  }
+  // Where the tile's rows go: thread t fetches row t's scatter index now, ahead of the arithmetic, and leaves it in a table in
+  // the LDS behind the first pass's arithmetic; the store rounds read their rows' entries from there. (Fetched by every
+  // thread for each of its store rounds they were up to 16 loads a thread, held in registers through the arithmetic, and
+  // where registers were short the compiler moved them aside at once, which waited for them before the arithmetic.)
+  int out_row = 0;
+  if (tid < BM) {
+    const int sorted = row0 + min(tid, valid_rows - 1);
+    out_row = p.scatter ? p.scatter[sorted] : sorted;
+  }
 #pragma unroll
   for (int pass = 0; pass < kPasses; ++pass) {
     if (pass > 0) __syncthreads();  // the previous pass has left the LDS
-    // where this thread's rows of the pass go: the scatter indices are fetched before the arithmetic below
-    int out_rows[kStoreIters];
-#pragma unroll
-    for (int it = 0; it < kStoreIters; ++it) {
-      const int sorted = row0 + min(pass * kPassRows + (tid + it * kThreads) / kRowChunks, valid_rows - 1);
-      out_rows[it] = p.scatter ? p.scatter[sorted] : sorted;
-    }
     // The tile's rounded outputs into the LDS. `plain` (SwiGLU, no clamp) is the same for the whole launch; the choice is made
     // once, around the whole nest, and each side holds cross-lane moves and LDS stores: written as a condition around the
     // arithmetic alone, the compiler evaluated both gates for every output and selected (two exponentials and reciprocals
@@ -1073,13 +1093,27 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
     } else {
       stage_tiles(std::true_type{});
     }
+    if (pass == 0 && tid < BM) out_row_of[tid] = out_row;
     __syncthreads();
+    // The thread's pieces of the staged rows and their rows' destinations are all read first, so that no store's address
+    // hangs on a load from global memory: each store below stands under its own condition, and with the scatter indices
+    // fetched by the storing thread the compiler put a full wait in front of each address, which on this chip waits for the
+    // stores before it as well: a pass's eight stores went out one write round trip after another (14 000 cycles of a
+    // 128 x 256 tile's 91 000).
+    u32x4_t staged_words[kStoreIters];
+    int out_rows[kStoreIters];
+#pragma unroll
+    for (int it = 0; it < kStoreIters; ++it) {
+      const int item = tid + it * kThreads;
+      staged_words[it] = *reinterpret_cast<const u32x4_t*>(staged + (item / kRowChunks) * kRowDwords + (item % kRowChunks) * 4);
+      out_rows[it] = out_row_of[pass * kPassRows + item / kRowChunks];
+    }
 #pragma unroll
     for (int it = 0; it < kStoreIters; ++it) {
       const int item = tid + it * kThreads;
       const int staged_row = item / kRowChunks, chunk = item % kRowChunks;
       const bool valid = pass * kPassRows + staged_row < valid_rows;
-      const u32x4_t words = *reinterpret_cast<const u32x4_t*>(staged + staged_row * kRowDwords + chunk * 4);
+      const u32x4_t words = staged_words[it];
       if constexpr (kSplitOut) {
         // The row's 128 columns of this tile as two e4m3 terms under one scale (dew_moe_split_rows' arithmetic on a
         // 128-column block): the 16 lanes that hold the row's chunks agree on its largest exponent field, each
