@@ -1038,6 +1038,13 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
         const int block_tile = wm0 / 32 + i;  // this wavefront's row tile i among the block's
         if (block_tile / kPassTiles != pass) continue;
         const int ii = block_tile % kPassTiles;
+        // f16 rows: the 2^s of the lane's 16 rows of this row tile, read ahead of the tile's arithmetic (read where they
+        // are used, each read stood behind the staging stores before it and was waited for on its own)
+        float row_scale[kNvF16 ? 16 : 1];
+        if constexpr (kNvF16) {
+#pragma unroll
+          for (int q = 0; q < 16; ++q) row_scale[q] = row_factor[wm0 + 32 * i + 8 * (q / 4) + 4 * (lane / 32) + q % 4];
+        }
 #pragma unroll
         for (int q = 0; q < 16; q += 2) {
           const int row = 32 * ii + 8 * (q / 4) + 4 * (lane / 32) + q % 4 + (odd_lane ? 1 : 0);  // within the pass
@@ -1058,9 +1065,8 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
               uint32_t mine;
               if constexpr (PAIRED) {
                 // (f16 rows: a row's sums times its own 2^s as well, an exact factor of the expert's)
-                const int lane_row = kNvF16 ? wm0 + 32 * i + 8 * (q / 4) + 4 * (lane / 32) + q % 4 : 0;
-                const float first0 = kNvF16 ? factor0 * row_factor[lane_row] : factor0, first1 = kNvF16 ? factor1 * row_factor[lane_row] : factor1;
-                const float second0 = kNvF16 ? factor0 * row_factor[kNvF16 ? lane_row + 1 : 0] : factor0, second1 = kNvF16 ? factor1 * row_factor[kNvF16 ? lane_row + 1 : 0] : factor1;
+                const float first0 = kNvF16 ? factor0 * row_scale[kNvF16 ? q : 0] : factor0, first1 = kNvF16 ? factor1 * row_scale[kNvF16 ? q : 0] : factor1;
+                const float second0 = kNvF16 ? factor0 * row_scale[kNvF16 ? q + 1 : 0] : factor0, second1 = kNvF16 ? factor1 * row_scale[kNvF16 ? q + 1 : 0] : factor1;
                 if constexpr (decltype(plain)::value) {
                   mine = swiglu_rounded(acc[0][i][j][q] * first0, acc[kMatrices - 1][i][j][q] * first1) |
                          (static_cast<uint32_t>(swiglu_rounded(acc[0][i][j][q + 1] * second0, acc[kMatrices - 1][i][j][q + 1] * second1)) << 16);
