@@ -1219,6 +1219,9 @@ static int launch_tile(const char* who, GemmParams p, hipStream_t stream) {
   // smaller chunks their last round spreads more evenly over the XCDs (measured on 16 to 64 m-tiles of 256 rows: the down
   // launch 8 % shorter, the paired one 3 %; taller chunks of 8 or 16 m-tiles, which fetch less, were slower everywhere)
   p.group_m = BM == 256 ? 2 : 4;
+  // (a one-bank launch of few tiles likewise: C5's down launch, 1 168 tiles of 128 rows, runs its step 1 % shorter dealt in
+  // chunks of 16; the paired launches are best at 4 x 8 down to the decode sizes)
+  if (MODE != kSwigluOfTwo && MODE != kSwigluOfTwoSplit && total < 2048) p.group_m = 2;
   const int round = 64 * p.group_m;
   const int blocks = ((total + round - 1) / round) * round;  // whole chunks of tiles for each of the 8 XCDs
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreads), kShared, stream, p);
