@@ -20,7 +20,7 @@ EXPORTS = (
     "dew_moe_last_error", "dew_moe_architecture", "dew_moe_kernels", "dew_moe_kernel_fields",
     "dew_moe_device_check", "dew_moe_route", "dew_moe_router_logits", "dew_moe_group_offsets", "dew_moe_permute_workspace_bytes", "dew_moe_permute", "dew_moe_permute_static", "dew_moe_permute_shared",
     "dew_moe_prepared_bytes", "dew_moe_prepare_bank", "dew_moe_prepared_view", "dew_moe_tile_rows", "dew_moe_grouped_gemm", "dew_moe_grouped_gemm_bias", "dew_moe_grouped_gemm_sizes", "dew_moe_grouped_gemm_param_bias", "dew_moe_gateup_swiglu_sizes",
-    "dew_moe_gateup_interleaved", "dew_moe_split_rows", "dew_moe_grouped_gemm_split", "dew_moe_gateup_swiglu_split", "dew_moe_gateup_swiglu_split_out", "dew_moe_split_rows_fp6", "dew_moe_gateup_swiglu_split_fp6_out", "dew_moe_grouped_gemm_split_blocks", "dew_moe_route_sown", "dew_moe_balance_bias", "dew_moe_quantize_rows_nvfp4", "dew_moe_quantize_columns_fp8", "dew_moe_quantize_columns_mxfp8", "dew_moe_kernel_gradient_mxfp8", "dew_moe_transpose_columns", "dew_moe_transpose_groups", "dew_moe_quantize_columns_nvfp4", "dew_moe_kernel_gradient_bf16", "dew_moe_quantize_rows_mxfp8", "dew_moe_grouped_gemm_mxfp8_rows", "dew_moe_quantize_rows_fp8", "dew_moe_grouped_gemm_fp8_rows", "dew_moe_gateup_swiglu", "dew_moe_swiglu", "dew_moe_swiglu_clamped", "dew_moe_gated_product", "dew_moe_scale_rows", "dew_moe_gate_rows", "dew_moe_gateup_gated", "dew_moe_silu", "dew_moe_relu2", "dew_moe_prefers_split_rows", "dew_moe_swiglu_mlp_split_workspace_bytes", "dew_moe_swiglu_mlp_split", "dew_moe_gated_mlp_split", "dew_moe_capacity_admit", "dew_moe_route_with", "dew_moe_route_call", "dew_moe_route_blocks_workspace_bytes", "dew_moe_route_blocks", "dew_moe_combine",
+    "dew_moe_gateup_interleaved", "dew_moe_split_rows", "dew_moe_grouped_gemm_split", "dew_moe_gateup_swiglu_split", "dew_moe_gateup_swiglu_split_out", "dew_moe_split_rows_fp6", "dew_moe_gateup_swiglu_split_fp6_out", "dew_moe_grouped_gemm_split_blocks", "dew_moe_route_sown", "dew_moe_balance_bias", "dew_moe_quantize_rows_nvfp4", "dew_moe_quantize_columns_fp8", "dew_moe_quantize_columns_mxfp8", "dew_moe_kernel_gradient_mxfp8", "dew_moe_transpose_columns", "dew_moe_transpose_groups", "dew_moe_quantize_columns_nvfp4", "dew_moe_kernel_gradient_bf16", "dew_moe_quantize_rows_mxfp8", "dew_moe_grouped_gemm_mxfp8_rows", "dew_moe_quantize_rows_fp8", "dew_moe_grouped_gemm_fp8_rows", "dew_moe_gateup_swiglu", "dew_moe_swiglu", "dew_moe_swiglu_clamped", "dew_moe_gated_product", "dew_moe_scale_rows", "dew_moe_gate_rows", "dew_moe_gate_rows_add_f32", "dew_moe_gateup_gated", "dew_moe_silu", "dew_moe_relu2", "dew_moe_prefers_split_rows", "dew_moe_swiglu_mlp_split_workspace_bytes", "dew_moe_swiglu_mlp_split", "dew_moe_gated_mlp_split", "dew_moe_capacity_admit", "dew_moe_route_with", "dew_moe_route_call", "dew_moe_route_blocks_workspace_bytes", "dew_moe_route_blocks", "dew_moe_combine",
     "dew_moe_rows_f16", "dew_moe_gateup_gated_f16", "dew_moe_split_rows_e2m3_pair", "dew_moe_gateup_swiglu_split_e2m3_pair_out",
 )
 """Every symbol include/dew_moe_hip.h declares."""
@@ -115,6 +115,7 @@ def library() -> ctypes.CDLL:
         "dew_moe_silu": (i32, [ptr, ptr, i64, ptr]),
         "dew_moe_relu2": (i32, [ptr, ptr, i64, ptr]),
         "dew_moe_gate_rows": (i32, [ptr, ptr, ptr, ptr, i32, i32, i32, ptr]),
+        "dew_moe_gate_rows_add_f32": (i32, [ptr, ptr, ptr, ptr, ptr, i32, i32, i32, ptr]),
         "dew_moe_gated_product": (i32, [ptr, ptr, i32, f32, ptr, i64, ptr]),
         "dew_moe_scale_rows": (i32, [ptr, ptr, ptr, ptr, ptr, i32, i32, ptr]),
         "dew_moe_gateup_gated": (i32, [ptr, ptr, ptr, ptr, bank, bank, i32, f32, ptr, i32, ptr]),

@@ -133,6 +133,41 @@ __global__ __launch_bounds__(256) void gate_rows_kernel(const bf16_t* __restrict
   }
 }
 
+// The same gate where the layer states no compute dtype (src/dew/nn/moe.py:1469-1475, 1497-1503): the gate's `Dense(1)` then
+// promotes the bf16 token to its fp32 kernel, so the logit, its logistic and the product with the shared expert's bf16 row
+// are fp32, and so is the layer's output, routed + shared: out[t, :] = f32(routed[t, :]) + f32(shared[t, :]) * g[t], each
+// operation rounded once in fp32. One wavefront a token.
+__global__ __launch_bounds__(256) void gate_rows_add_f32_kernel(const bf16_t* __restrict__ x, const float* __restrict__ kernel,
+                                                                const bf16_t* __restrict__ shared, const bf16_t* __restrict__ routed,
+                                                                float* __restrict__ out, int tokens, int depth, int width) {
+  const int lane = threadIdx.x % 64;
+  const int token = blockIdx.x * 4 + threadIdx.x / 64;
+  if (token >= tokens) return;
+  // (the logit's sum in float64, rounded once to fp32: every product of a bf16 and an fp32 value is exact there)
+  double sum = 0.0;
+  for (int chunk = lane; chunk < depth / 8; chunk += 64) {
+    const Bf16x8 values = *reinterpret_cast<const Bf16x8*>(x + static_cast<size_t>(token) * depth + static_cast<size_t>(chunk) * 8);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sum += static_cast<double>(bf16_to_f32(values.v[i])) * static_cast<double>(kernel[chunk * 8 + i]);
+  }
+#pragma unroll
+  for (int offset = 32; offset >= 1; offset >>= 1) sum += __shfl_xor(sum, offset, 64);
+  const float gate = 1.0f / (1.0f + exp_f32(-static_cast<float>(sum)));
+  for (int chunk = lane; chunk < width / 8; chunk += 64) {
+    const size_t at = static_cast<size_t>(token) * width + static_cast<size_t>(chunk) * 8;
+    const Bf16x8 mine = *reinterpret_cast<const Bf16x8*>(shared + at), theirs = *reinterpret_cast<const Bf16x8*>(routed + at);
+    float sums[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float gated = bf16_to_f32(mine.v[i]) * gate;
+      sums[i] = bf16_to_f32(theirs.v[i]) + gated;
+    }
+    float4* to = reinterpret_cast<float4*>(out + at);
+    to[0] = float4{sums[0], sums[1], sums[2], sums[3]};
+    to[1] = float4{sums[4], sums[5], sums[6], sums[7]};
+  }
+}
+
 // `limit` > 0: the gate clamped from above and the up projection both ways before their product (`swiglu_clamped`,
 // src/dew/nn/activations.py:327-333); the limit enters as the bf16 the operands' dtype rounds it to.
 __global__ __launch_bounds__(256) void swiglu_kernel(const bf16_t* __restrict__ gate, const bf16_t* __restrict__ up,
@@ -216,6 +251,21 @@ extern "C" int dew_moe_gate_rows(const void* x, const float* kernel, const void*
   hipLaunchKernelGGL(gate_rows_kernel, dim3((tokens + 3) / 4), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<const bf16_t*>(x),
                      kernel, static_cast<const bf16_t*>(rows_in), static_cast<bf16_t*>(out), tokens, depth, width);
   return launched("gate_rows_kernel");
+}
+
+extern "C" int dew_moe_gate_rows_add_f32(const void* x, const float* kernel, const void* shared, const void* routed, float* out,
+                                         int32_t tokens, int32_t depth, int32_t width, void* stream) {
+  using namespace dew;
+  DEW_REQUIRE(tokens >= 0 && depth > 0 && depth % 8 == 0 && width > 0 && width % 8 == 0,
+              "dew_moe_gate_rows_add_f32: tokens %d, depth %d and width %d (whole 8s)", tokens, depth, width);
+  if (tokens == 0) return DEW_MOE_OK;
+  DEW_REQUIRE(x && kernel && shared && routed && out, "dew_moe_gate_rows_add_f32: x, kernel, both row buffers and out must not be null");
+  DEW_REQUIRE(aligned16(x) && aligned16(shared) && aligned16(routed) && aligned16(out),
+              "dew_moe_gate_rows_add_f32: x, both row buffers and out must be 16-byte aligned");
+  hipLaunchKernelGGL(gate_rows_add_f32_kernel, dim3((tokens + 3) / 4), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const bf16_t*>(x), kernel, static_cast<const bf16_t*>(shared), static_cast<const bf16_t*>(routed), out, tokens,
+                     depth, width);
+  return launched("gate_rows_add_f32_kernel");
 }
 
 extern "C" int dew_moe_swiglu(const void* gate, const void* up, void* hidden, int64_t count, void* stream) {

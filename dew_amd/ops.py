@@ -551,6 +551,21 @@ def gate_rows(x: torch.Tensor, kernel: torch.Tensor, rows: torch.Tensor) -> torc
     return out
 
 
+def gate_rows_add_f32(x: torch.Tensor, kernel: torch.Tensor, shared: torch.Tensor, routed: torch.Tensor) -> torch.Tensor:
+    """`routed + shared * logistic(x @ kernel)` in fp32, `[T, W]`: the reference's `shared_gate` where the layer states no
+    compute dtype (its gate then runs in the fp32 of its kernel and widens the layer's output). `kernel` is the gate's
+    fp32 `[D]` (or `[D, 1]`) parameter; `shared` and `routed` are the bf16 rows of the shared and the routed experts."""
+    _device(x, "x", torch.bfloat16), _device(kernel, "kernel", torch.float32)
+    _device(shared, "shared", torch.bfloat16), _device(routed, "routed", torch.bfloat16)
+    if x.dim() != 2 or shared.dim() != 2 or shared.shape != routed.shape or shared.shape[0] != x.shape[0] or kernel.numel() != x.shape[1]:
+        raise KernelError(f"gate_rows_add_f32 takes x [T, D], a kernel of D values and two [T, W] row buffers, got {tuple(x.shape)}, "
+                          f"{tuple(kernel.shape)}, {tuple(shared.shape)} and {tuple(routed.shape)}")
+    out = torch.empty(shared.shape, dtype=torch.float32, device=x.device)
+    _lib.check(_lib.library().dew_moe_gate_rows_add_f32(_ptr(x), _ptr(kernel), _ptr(shared), _ptr(routed), _ptr(out), x.shape[0], x.shape[1],
+                                                        shared.shape[1], _stream()), "dew_moe_gate_rows_add_f32")
+    return out
+
+
 def relu2(x: torch.Tensor) -> torch.Tensor:
     """`bf16(max(x, 0)^2)`: the squared ReLU of Nemotron-H's ungated experts (the reference's `relu2`)."""
     _device(x, "x", torch.bfloat16)

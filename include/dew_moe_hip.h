@@ -513,6 +513,12 @@ int dew_moe_scale_rows(const void* x /* bf16 [T,D] */, const int32_t* gather, co
  * fp32. rows and out may be the same buffer.                                                                          */
 int dew_moe_gate_rows(const void* x /* bf16 [T,D] */, const float* kernel /* [D] */, const void* rows /* bf16 [T,W] */,
                       void* out /* bf16 [T,W] */, int32_t tokens, int32_t depth, int32_t width, void* stream);
+/* The same gate where the layer states no compute dtype (src/dew/nn/moe.py:1469-1475, 1497-1503): the gate's Dense(1) then
+ * runs in the fp32 of its kernel and the layer's output widens to fp32:
+ * out[t, :] = f32(routed[t, :]) + f32(shared[t, :]) * logistic(sum_d x[t, d] * kernel[d]), every operation in fp32.          */
+int dew_moe_gate_rows_add_f32(const void* x /* bf16 [T,D] */, const float* kernel /* [D] */, const void* shared /* bf16 [T,W] */,
+                              const void* routed /* bf16 [T,W] */, float* out /* [T,W] */, int32_t tokens, int32_t depth,
+                              int32_t width, void* stream);
 
 /* Nemotron-H's ungated experts (`activation='relu2'`, src/dew/nn/moe.py:1250-1252, 1319-1322: up_proj, squared ReLU,
  * down_proj): out = bf16(max(x, 0)^2) (`relu2`, src/dew/nn/activations.py:109-111), between two dew_moe_grouped_gemm launches. */

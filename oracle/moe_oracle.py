@@ -56,6 +56,8 @@ What pins each function (tests/test_oracle_golden.py):
 * `gated_rows` (`shared_gate`, Qwen2-MoE's scalar gate on the shared expert): no vectors in the reference. The dtype flow
   is read from the reference's sources (the gate's Dense under `dtype=bf16`; `logistic`'s one rounding); the arithmetic
   is pinned by a hand case whose three roundings each move the result, and by float64 `sigmoid(x . w) * rows` within bf16.
+  `gated_rows_added_f32` (the same gate where the layer states no compute dtype: fp32 throughout, added to the routed rows):
+  likewise, by float64 `routed + sigmoid(x . w) * shared` within two fp32 roundings.
 * `route(media=, media_bias=)` (DeepSeek-V4.1's image-span bias): by the definition: the media tokens route as a router
   whose bias is `media_bias` routes them, the others as one whose bias is `bias`, row for row.
 * `route(given=, covered=)` (replayed routes and the hash router's table rows, `chosen_experts` src/dew/nn/moe.py:202-224):
@@ -1224,6 +1226,19 @@ def gated_rows(x, kernel, rows):
     logit = bf16_round((x.astype(np.float64) @ kernel.astype(np.float64)).astype(F32))
     gate = bf16_round(logistic(logit))   # (fp32, the fixed-sequence exponential: the device kernel's own steps, so the gates agree bit for bit)
     return bf16_round((np.asarray(rows, F32) * gate[:, None]).astype(F32))
+
+
+def gated_rows_added_f32(x, kernel, shared, routed):
+    """`routed + shared * logistic(shared_expert_gate(x))` (src/dew/nn/moe.py:1469-1475, 1497-1503) where the layer states no
+    compute dtype: the gate's `Dense(1)` promotes the bf16 token to its fp32 kernel (flax's `promote_dtype` without a
+    `dtype`), so the logit, its logistic, the product with the shared expert's bf16 rows and the sum with the routed
+    experts' bf16 rows are float32, each operation rounded once. (The logit's sum in float64, rounded once: the device
+    kernel's own steps. Like the bf16 gate's, these rounding points are read from the sources and pinned by no fixture.)"""
+    x = np.asarray(x, F32)
+    kernel = np.asarray(kernel, F32).reshape(-1)
+    logit = (x.astype(np.float64) @ kernel.astype(np.float64)).astype(F32)
+    gated = (np.asarray(shared, F32) * logistic(logit)[:, None]).astype(F32)
+    return (np.asarray(routed, F32) + gated).astype(F32)
 
 
 def sparse_mlp(x, logits, gate_w, up_w, down_w, *, top_k_count, dtype="bfloat16", shared=None,

@@ -5,6 +5,8 @@ Bars: routing indices, group sizes/offsets and the permutation bit-exact; router
 within max relative error 2e-2 (measured both as max|d| / max|ref| and element-wise as |d| / max(|ref|,
 rms(ref))). The bf16-exact kernels land near 2^-8, far inside the bar; the observed figures are printed."""
 
+from dataclasses import replace as dataclasses_replace
+
 import numpy as np
 import pytest
 import torch
@@ -563,10 +565,102 @@ def test_qwen2_moes_gate_on_the_shared_expert(fuse_shared):
     by_max, by_element = oracle.relative_errors(got, want)
     assert by_max <= 6e-3 and by_element <= TOLERANCE, (by_max, by_element)
     assert oracle.relative_errors(got, ungated)[0] > 10 * by_max                 # the gate gates
-    with pytest.raises(ValueError, match="compute dtype"):
-        dataclasses.replace(layer, dtype=None).apply(variables, data["x"].cuda(), logits=data["logits"].cuda())
+    widened = dataclasses.replace(layer, dtype=None).apply(variables, data["x"].cuda(), logits=data["logits"].cuda())
+    assert widened.dtype == torch.float32                                        # (no compute dtype: the gate's fp32, see the next test)
     with pytest.raises(ValueError, match="requires a shared expert"):
         dataclasses.replace(layer, shared=None).apply(variables, data["x"].cuda(), logits=data["logits"].cuda())
+
+
+def test_qwen2_moes_gate_in_float32_widens_the_layers_output():
+    """`shared_gate` where the layer states no compute dtype (src/dew/nn/moe.py:1469-1475, 1497-1503): the gate's `Dense(1)`
+    runs in the fp32 of its kernel, and routed + shared * gate comes back fp32. The kernel alone against the oracle, bit for
+    bit (the logit's sum in float64 on both sides, then the same fp32 steps) and against float64 within two fp32 roundings;
+    then the whole layer, whose routed and shared rows are the bf16 layer's."""
+    import dataclasses
+
+    from dew_amd import ops
+    rng = np.random.default_rng(43)
+    x = torch.from_numpy(rng.standard_normal((1777, 512)).astype(np.float32)).to(torch.bfloat16)
+    kernel = (rng.standard_normal(512) * 0.05).astype(np.float32)
+    shared, routed = (torch.from_numpy(rng.standard_normal((1777, 256)).astype(np.float32)).to(torch.bfloat16) for _ in range(2))
+    got = ops.gate_rows_add_f32(x.cuda(), torch.from_numpy(kernel).cuda(), shared.cuda(), routed.cuda())
+    assert got.dtype == torch.float32
+    got = got.cpu().numpy()
+    want = oracle.gated_rows_added_f32(x.float().numpy(), kernel, shared.float().numpy(), routed.float().numpy())
+    assert np.array_equal(got, want)
+    exact = routed.double().numpy() + shared.double().numpy() / (1.0 + np.exp(-(x.double().numpy() @ kernel.astype(np.float64))))[:, None]
+    assert np.abs(got - exact).max() <= 4e-7 * np.abs(exact).max()
+
+    case = CASES["c4-reduced"].scaled(tokens=200)
+    data = inputs(case, seed=14)
+    layer, variables = layer_and_variables(case, data)
+    gate = (rng.standard_normal(case.d_model) * 0.05).astype(np.float32)
+    variables["params"]["shared_expert_gate"] = {"kernel": torch.from_numpy(gate).reshape(-1, 1).cuda()}
+    layer = dataclasses.replace(layer, shared_gate=True)        # no dtype
+    out = layer.apply(variables, data["x"].cuda(), logits=data["logits"].cuda())
+    assert out.dtype == torch.float32 and out.shape == data["x"].shape
+    mats, factors = zip(*(dequantized(data["banks"][name]) for name in ("gate", "up", "down")), strict=True)
+    apart = oracle.gated_mlp(data["x"].float().numpy(), *(dequantized(data["shared"][name])[0][0] for name in ("gate", "up", "down")))
+    alone, _ = oracle.sparse_mlp(data["x"].float().numpy(), data["logits"].numpy(), *mats, top_k_count=case.top_k, factors=factors,
+                                 bias=data["bias"].numpy(), **case.router)
+    want = oracle.gated_rows_added_f32(data["x"].float().numpy(), gate, apart, alone)
+    by_max, by_element = oracle.relative_errors(out.cpu().numpy(), want)
+    assert by_max <= 6e-3 and by_element <= TOLERANCE, (by_max, by_element)
+    with pytest.raises(ValueError, match="runs in bfloat16"):
+        dataclasses.replace(layer, dtype=torch.float16).apply(variables, data["x"].cuda(), logits=data["logits"].cuda())
+
+
+@pytest.mark.parametrize("with_norm,shared_gate", [(False, False), (True, False), (True, True)])
+def test_kimis_latent_experts(with_norm, shared_gate):
+    """`latent_features` (src/dew/nn/moe.py:1379-1385, 1458-1467, 1491-1496): the router reads the full width, a dense down
+    projection narrows the tokens to the experts' width, their combined rows go through the norm and a dense up projection,
+    and the shared expert, which reads the full width, is added behind it. Against the oracle's pieces in that order."""
+    from dew_amd import moe
+    full_width = 1536
+    narrow = CASES["c4-reduced"].scaled(tokens=200)                        # the experts: latent width 1024
+    data = inputs(narrow, seed=15)
+    full = inputs(narrow.scaled(d_model=full_width), seed=16)              # the tokens and the shared expert at the full width
+    rng = np.random.default_rng(44)
+    down = torch.from_numpy((rng.standard_normal((full_width, narrow.d_model)) * 0.03).astype(np.float32)).to(torch.bfloat16)
+    up = torch.from_numpy((rng.standard_normal((narrow.d_model, full_width)) * 0.03).astype(np.float32)).to(torch.bfloat16)
+    scale = torch.from_numpy(rng.uniform(0.5, 2.0, narrow.d_model).astype(np.float32))
+    norm = (lambda params, rows: (rows.float() * params["scale"]).to(torch.bfloat16)) if with_norm else None
+    layer = moe.SparseMLP(num_experts=narrow.experts, top_k=narrow.top_k, hidden_features=narrow.d_ff, out_features=full_width,
+                          expert_bias=True, shared=narrow.d_ff, latent_features=narrow.d_model, latent_norm=norm, shared_gate=shared_gate,
+                          dtype=torch.bfloat16, **narrow.router)
+    variables = {"params": {"routed_expert_down_proj": {"kernel": down.cuda()}, "routed_expert_up_proj": {"kernel": up.cuda()},
+                            "routed_expert_norm": {"scale": scale.cuda()}},
+                 "quantization": {"experts": {f"{n}_proj": {"kernel": b.to("cuda")} for n, b in data["banks"].items()},
+                                  "shared_experts": {f"{n}_proj": {"kernel": b.to("cuda")} for n, b in full["shared"].items()}},
+                 "moe": {"gate": {"e_score_correction_bias": data["bias"].cuda()}}}
+    gate = (rng.standard_normal(full_width) * 0.05).astype(np.float32)
+    if shared_gate:
+        variables["params"]["shared_expert_gate"] = {"kernel": torch.from_numpy(gate).reshape(-1, 1).cuda()}
+    got = layer.apply(variables, full["x"].cuda(), logits=data["logits"].cuda())
+    assert got.dtype == torch.bfloat16 and got.shape == full["x"].shape
+    assert layer._bound(variables, ()).experts.out_features == narrow.d_model
+
+    x = full["x"].float().numpy()
+    everyone = [x.shape[0]]
+    narrowed = oracle.grouped_matmul(x, down.float().numpy()[None], everyone)
+    mats, factors = zip(*(dequantized(data["banks"][name]) for name in ("gate", "up", "down")), strict=True)
+    weights, indices = oracle.route(data["logits"].numpy(), narrow.top_k, bias=data["bias"].numpy(), **narrow.router)
+    routed, _ = oracle.expert_mlp(narrowed, weights, indices, *mats, factors=factors)
+    if with_norm:
+        routed = oracle.bf16_round(routed * scale.numpy())
+    widened = oracle.grouped_matmul(routed, up.float().numpy()[None], everyone)
+    apart = oracle.gated_mlp(x, *(dequantized(full["shared"][name])[0][0] for name in ("gate", "up", "down")))
+    if shared_gate:
+        apart = oracle.gated_rows(x, gate, apart)
+    want = oracle.bf16_round(widened + apart)
+    by_max, by_element = oracle.relative_errors(got.float().cpu().numpy(), want)
+    # (five chained roundings: one bf16 ulp of the largest output is up to 7.8e-3 of it)
+    assert by_max <= 8e-3 and by_element <= TOLERANCE, (by_max, by_element)
+    without = dataclasses_replace(layer, shared=None, shared_gate=False).apply(variables, full["x"].cuda(), logits=data["logits"].cuda())
+    assert oracle.relative_errors(without.float().cpu().numpy(), widened)[1] <= TOLERANCE
+    with pytest.raises(ValueError, match="states no compute dtype"):
+        float_kernels = {**variables, "params": {**variables["params"], "routed_expert_down_proj": {"kernel": down.float().cuda()}}}
+        dataclasses_replace(layer, dtype=None).apply(float_kernels, full["x"].cuda(), logits=data["logits"].cuda())
 
 
 def test_a_captured_layer_replays_to_the_eager_result():
