@@ -79,3 +79,22 @@ def test_defective_index_tensors_are_refused_on_the_device_side_too(name):
     if name in SCATTERED:   # (the paired and gated products write sorted rows: they take no scatter)
         with pytest.raises(KernelError, match="scatter must be torch.int32"):
             call(scatter=torch.zeros(6, dtype=torch.int64, device=device))
+
+
+def test_the_float32_gate_and_a_latent_layers_projections_refuse_on_the_host():
+    """`gate_rows_add_f32` takes device tensors only; a latent layer's dense projection refuses a kernel of another shape,
+    and a float32 kernel where the layer states no compute dtype (the reference would then run the projection in float32)."""
+    from dew_amd import moe
+
+    x, rows = torch.zeros((4, 64), dtype=torch.bfloat16), torch.zeros((4, 32), dtype=torch.bfloat16)
+    with pytest.raises(KernelError, match="must be on the GPU"):
+        ops.gate_rows_add_f32(x, torch.zeros(64), rows, rows)
+    layer = moe.SparseMLP(num_experts=4, top_k=2, hidden_features=64, out_features=64, latent_features=32)
+    assert layer._bound({}, ()).experts.out_features == 32
+    variables = {"params": {"routed_expert_down_proj": {"kernel": torch.zeros((64, 32))}}}
+    with pytest.raises(ValueError, match="states no compute dtype"):
+        layer._bound(variables, ())._dense(x, "routed_expert_down_proj", 64, 32)
+    with pytest.raises(ValueError, match=r"the layer's is \(64, 16\)"):
+        layer._bound(variables, ())._dense(x, "routed_expert_down_proj", 64, 16)
+    with pytest.raises(KeyError, match="routed_expert_up_proj"):
+        layer._bound(variables, ())._dense(x, "routed_expert_up_proj", 32, 64)
