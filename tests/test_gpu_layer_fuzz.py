@@ -8,7 +8,13 @@ element-wise figure `|d| / max(|ref|, rms(ref))` is this repository's own, stric
 2e-2 on it; the split-row launches hold ELEMENTWISE_ON_SPLIT_ROWS = 3e-2, because their sums come from another matrix
 instruction (one bf16 ulp apart from the bf16 instruction's in about 1 % of outputs) and their hidden rows carry one
 scale per 128 columns, and where a routed and a shared output nearly cancel two such ulps have been seen to add up to
-2.05e-2 .. 2.45e-2 of the difference. `gemm.SPLIT_ROWS = False` keeps such a layer on the bf16 instruction and its 2e-2."""
+2.05e-2 .. 2.45e-2 of the difference. `gemm.SPLIT_ROWS = False` keeps such a layer on the bf16 instruction and its 2e-2.
+
+What the element-wise figure cannot promise, on any path: it divides by the output's rms, and one bf16 ulp of a slot (an expert's
+output row, before the combine weighs it) is 2^-8 of that slot, so a single flipped rounding on a slot five times the output's
+rms is 2e-2 of it. Of 1 900 further seeds of this generator two did that (ONE_ULP_SEEDS: 2.2e-2 and 2.05e-2, each one ulp of
+one slot of 0.17 .. 0.25 under an output rms of 0.03 .. 0.05, 99.94 % of the outputs bit-identical, the reference's metric at
+3.8e-3); they are kept here under the bar that names the case, ONE_ULP_OF_A_LARGE_SLOT."""
 
 import numpy as np
 import pytest
@@ -22,6 +28,9 @@ pytestmark = pytest.mark.gpu
 
 BAR = 2e-2
 ELEMENTWISE_ON_SPLIT_ROWS = 3e-2
+
+ONE_ULP_OF_A_LARGE_SLOT = 2.5e-2
+ONE_ULP_SEEDS = (30955, 30992)
 
 SEEDS = tuple(range(7000, 7036)) + (5051, 5085, 5086, 5127)
 """Thirty-six consecutive seeds and four that earlier, longer runs of the same generator singled out (5086: a capacity-dropped
@@ -98,6 +107,16 @@ def test_a_seeded_layer_matches_the_oracle(seed):
     by_max, by_element, on_split_rows = layer_against_the_oracle(case, settings, seed)
     assert by_max <= BAR, (by_max, by_element)
     assert by_element <= (ELEMENTWISE_ON_SPLIT_ROWS if on_split_rows else BAR), (by_max, by_element, on_split_rows)
+
+
+@pytest.mark.parametrize("seed", ONE_ULP_SEEDS)
+def test_one_ulp_of_a_large_slot_is_all_that_differs(seed):
+    """The two seeds whose element-wise figure passes 2e-2 on the bf16 instruction: the reference's metric holds with a wide
+    margin, and the figure stays under the bar one flipped bf16 rounding of a slot several times the output's rms explains."""
+    case, settings = drawn(seed)
+    by_max, by_element, on_split_rows = layer_against_the_oracle(case, settings, seed)
+    assert not on_split_rows
+    assert by_max <= 5e-3 and by_element <= ONE_ULP_OF_A_LARGE_SLOT, (by_max, by_element)
 
 
 SPLIT_ROW_LAYERS = [
