@@ -12,9 +12,10 @@ scale per 128 columns, and where a routed and a shared output nearly cancel two 
 
 What the element-wise figure cannot promise, on any path: it divides by the output's rms, and one bf16 ulp of a slot (an expert's
 output row, before the combine weighs it) is 2^-8 of that slot, so a single flipped rounding on a slot five times the output's
-rms is 2e-2 of it. Of 1 900 further seeds of this generator two did that (ONE_ULP_SEEDS: 2.2e-2 and 2.05e-2, each one ulp of
-one slot of 0.17 .. 0.25 under an output rms of 0.03 .. 0.05, 99.94 % of the outputs bit-identical, the reference's metric at
-3.8e-3); they are kept here under the bar that names the case, ONE_ULP_OF_A_LARGE_SLOT."""
+rms is 2e-2 of it. Of 4 700 further seeds of this generator five did that (2.00e-2 .. 2.2e-2; the split-row layers among them
+stayed under their 3e-2, at 2.87e-2 at most; the reference's metric never passed 5.3e-3). The two largest are kept here
+(ONE_ULP_SEEDS: 2.2e-2 and 2.05e-2, each one ulp of one slot of 0.17 .. 0.25 under an output rms of 0.03 .. 0.05, 99.94 % of the
+outputs bit-identical) under the bar that names the case, ONE_ULP_OF_A_LARGE_SLOT."""
 
 import numpy as np
 import pytest
