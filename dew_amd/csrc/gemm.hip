@@ -296,10 +296,17 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
   // gave group sizes instead of their prefix, of the sizes themselves: an expert's first row) ----
   if (tid == 0) found[0] = -1;
   int carried = 0, carried_rows = 0;
+  // (a round's sizes and first rows are asked for one round ahead: past 256 experts the rounds' loads then overlap, instead
+  // of one memory round trip a round in front of every tile)
+  auto size_of = [&](int e) { return e >= p.experts ? 0 : kWindow ? p.window_rows : p.sizes ? max(p.sizes[e], 0) : p.offsets[e + 1] - p.offsets[e]; };
+  auto first_row_of = [&](int e) { return e >= p.experts || (p.sizes && !kWindow) ? 0 : kWindow ? e * p.window_rows : p.offsets[e]; };
+  int next_size = size_of(tid), next_first_row = first_row_of(tid);
   for (int base = 0; base < p.experts; base += kThreads) {
     const int e = base + tid;
-    int start = 0, tiles = 0, size = 0;
-    if (e < p.experts) size = kWindow ? p.window_rows : p.sizes ? max(p.sizes[e], 0) : p.offsets[e + 1] - p.offsets[e];
+    int start = 0, tiles = 0;
+    const int size = next_size, first_row = next_first_row;
+    next_size = size_of(e + kThreads);
+    next_first_row = first_row_of(e + kThreads);
     if (p.sizes && !kWindow) {  // (uniform) exclusive prefix of the sizes
       int inclusive_rows = size;
 #pragma unroll
@@ -313,8 +320,8 @@ __global__ __launch_bounds__(kThreads, (FORMAT != DEW_MOE_W_BF16 && BM == 128 &&
       start = carried_rows + inclusive_rows - size;
       for (int w = 0; w < wave; ++w) start += wave_rows[w];
       carried_rows += wave_rows[0] + wave_rows[1] + wave_rows[2] + wave_rows[3];
-    } else if (e < p.experts) {
-      start = kWindow ? e * p.window_rows : p.offsets[e];
+    } else {
+      start = first_row;
     }
     const int group_end = start + size;
     if (e < p.experts) {
